@@ -1,0 +1,178 @@
+/*
+ * sg_math.h -- fp32 primitives with a FIXED operation order.
+ *
+ * Every function here is built only from IEEE-754 correctly rounded
+ * operations (+, -, *, /, sqrt, fma, round-to-nearest-even) and integer bit
+ * manipulation, so a gfx950 wavefront lane and an x86-64 host core return
+ * the same bits for the same input.  That is what lets the device kernels be
+ * compared bit-for-bit (sort permutations, PEER expert indices) with a CPU
+ * restatement of the same algorithm.
+ *
+ * Build rules that the property depends on (both compilers):
+ *   -ffp-contract=off      nothing is fused unless written as sg_fma()
+ *   no -ffast-math         no reassociation, IEEE division and sqrt
+ *   fp32 denormals kept    (the hipcc and gcc defaults)
+ *
+ * The transcendental approximations follow the classic Cephes single
+ * precision kernels (Cody-Waite range reduction + minimax polynomial); each
+ * is accurate to about 1e-7 relative on the range the optimizer uses.
+ *
+ * What the functions stand in for in the reference (file:line are relative
+ * to the reference tree):
+ *   sg_exp       expf       csrc/supergrok2_mamba_peer_kernels.cu:194,221,263,970
+ *   sg_log       logf       csrc/supergrok2_mamba_peer_kernels.cu:221
+ *   sg_softplus  stable softplus with the ">20 passes through" guard, :221
+ *   sg_sincos    __sincosf  csrc/supergrok2_mamba_peer_kernels.cu:240,434,652
+ *   sg_tanh      tanhf      csrc/supergrok2_mamba_peer_kernels.cu:989
+ *   sg_sigmoid   1/(1+expf(-x))   :970-971
+ *   sg_silu      z/(1+expf(-z))   :263,559,777
+ *   sg_abar_pair trapezoidal A_bar for the even/odd member of a RoPE pair, :228,431-432
+ */
+#ifndef SG_MATH_H_
+#define SG_MATH_H_
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define SG_HD __host__ __device__ __forceinline__
+#else
+#define SG_HD static inline __attribute__((always_inline))
+#endif
+
+SG_HD float sg_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+SG_HD float sg_rint(float x) { return __builtin_rintf(x); }
+
+SG_HD int32_t sg_f2i(float x) {
+    int32_t i;
+    __builtin_memcpy(&i, &x, 4);
+    return i;
+}
+SG_HD float sg_i2f(int32_t i) {
+    float x;
+    __builtin_memcpy(&x, &i, 4);
+    return x;
+}
+SG_HD float sg_abs(float x) { return sg_i2f(sg_f2i(x) & 0x7fffffff); }
+SG_HD float sg_min(float a, float b) { return a < b ? a : b; }
+SG_HD float sg_max(float a, float b) { return a > b ? a : b; }
+
+/* finite test on the bit pattern (no dependence on -ffinite-math settings) */
+SG_HD int sg_isfinite(float x) { return (sg_f2i(x) & 0x7f800000) != 0x7f800000; }
+
+/* exp(x), x clamped to [-86, 88] so the result is always a normal float. */
+SG_HD float sg_exp(float x) {
+    x = sg_min(sg_max(x, -86.0f), 88.0f);
+    const float k = sg_rint(x * 1.44269504088896341f);
+    float r = sg_fma(k, -0.693359375f, x);
+    r = sg_fma(k, 2.12194440e-4f, r);
+    float p = 1.9875691500e-4f;
+    p = sg_fma(p, r, 1.3981999507e-3f);
+    p = sg_fma(p, r, 8.3334519073e-3f);
+    p = sg_fma(p, r, 4.1665795894e-2f);
+    p = sg_fma(p, r, 1.6666665459e-1f);
+    p = sg_fma(p, r, 5.0000001201e-1f);
+    const float r2 = r * r;
+    p = sg_fma(p, r2, r) + 1.0f;
+    return sg_i2f((int32_t)((uint32_t)sg_f2i(p) + ((uint32_t)(int32_t)k << 23)));
+}
+
+/* log(u) for normal positive u. */
+SG_HD float sg_log(float u) {
+    const int32_t ix = sg_f2i(u);
+    const int32_t e = (ix - 0x3f3504f3) >> 23;          /* mantissa -> [sqrt(.5), sqrt(2)) */
+    const float f = sg_i2f((int32_t)((uint32_t)ix - ((uint32_t)e << 23))) - 1.0f;
+    const float fe = (float)e;
+    const float z = f * f;
+    float p = 7.0376836292e-2f;
+    p = sg_fma(p, f, -1.1514610310e-1f);
+    p = sg_fma(p, f, 1.1676998740e-1f);
+    p = sg_fma(p, f, -1.2420140846e-1f);
+    p = sg_fma(p, f, 1.4249322787e-1f);
+    p = sg_fma(p, f, -1.6668057665e-1f);
+    p = sg_fma(p, f, 2.0000714765e-1f);
+    p = sg_fma(p, f, -2.4999993993e-1f);
+    p = sg_fma(p, f, 3.3333331174e-1f);
+    float y = (p * f) * z;
+    y = sg_fma(fe, -2.12194440e-4f, y);
+    y = sg_fma(z, -0.5f, y);
+    return sg_fma(fe, 0.693359375f, f + y);
+}
+
+/* softplus with the reference's guard: raw > 20 passes through. */
+SG_HD float sg_softplus(float x) {
+    return (x > 20.0f) ? x : sg_log(1.0f + sg_exp(x));
+}
+
+SG_HD float sg_sigmoid(float x) { return 1.0f / (1.0f + sg_exp(-x)); }
+SG_HD float sg_silu(float z) { return z / (1.0f + sg_exp(-z)); }
+
+/* sin and cos of theta; two-constant Cody-Waite reduction by pi/2 (good to
+ * ~1e-7 absolute for |theta| < ~1e3, degrading gracefully beyond). */
+SG_HD void sg_sincos(float th, float* s_out, float* c_out) {
+    const float k = sg_rint(th * 0.636619772367581343f);
+    float r = sg_fma(k, -1.57079637050628662f, th);
+    r = sg_fma(k, 4.37113900018624283e-8f, r);
+    const float z = r * r;
+    float sp = -1.9515295891e-4f;
+    sp = sg_fma(sp, z, 8.3321608736e-3f);
+    sp = sg_fma(sp, z, -1.6666654611e-1f);
+    sp = sg_fma(sp * z, r, r);
+    float cp = 2.443315711809948e-5f;
+    cp = sg_fma(cp, z, -1.388731625493765e-3f);
+    cp = sg_fma(cp, z, 4.166664568298827e-2f);
+    cp = sg_fma(cp * z, z, sg_fma(z, -0.5f, 1.0f));
+    const int32_t q = (int32_t)k;
+    const int swap = q & 1;
+    const float s0 = swap ? cp : sp;
+    const float c0 = swap ? sp : cp;
+    *s_out = sg_i2f((int32_t)((uint32_t)sg_f2i(s0) ^ (((uint32_t)q & 2u) << 30)));
+    *c_out = sg_i2f((int32_t)((uint32_t)sg_f2i(c0) ^ ((((uint32_t)q + 1u) & 2u) << 30)));
+}
+
+/* 1/d for normal positive d: bit-trick seed + three Newton steps (~5e-8 rel). */
+SG_HD float sg_rcp_pos(float d) {
+    float r = sg_i2f(0x7EF311C7 - sg_f2i(d));
+    float e = sg_fma(-d, r, 1.0f);
+    r = sg_fma(r, e, r);
+    e = sg_fma(-d, r, 1.0f);
+    r = sg_fma(r, e, r);
+    e = sg_fma(-d, r, 1.0f);
+    r = sg_fma(r, e, r);
+    return r;
+}
+
+/* Trapezoidal discretisation for the two states of one RoPE pair:
+ *   A_bar = (1 + dt*A/2) / (1 - dt*A/2 + 1e-8)
+ * hA_e and hA_o are A/2 (exact halving).  A < 0 and dt >= 0, so the
+ * denominator is >= 1 and the "+1e-8f" of the reference is below half an ulp
+ * of it: adding it never changes an fp32 value >= 1, so it is dropped.  One shared reciprocal
+ * serves both members of the pair. */
+SG_HD void sg_abar_pair(float dt, float hA_e, float hA_o, float* ab_e, float* ab_o) {
+    const float n_e = sg_fma(dt, hA_e, 1.0f);
+    const float d_e = sg_fma(-dt, hA_e, 1.0f);
+    const float n_o = sg_fma(dt, hA_o, 1.0f);
+    const float d_o = sg_fma(-dt, hA_o, 1.0f);
+    const float r = sg_rcp_pos(d_e * d_o);
+    *ab_e = (n_e * d_o) * r;
+    *ab_o = (n_o * d_e) * r;
+}
+
+SG_HD float sg_tanh(float x) {
+    const float ax = sg_abs(x);
+    float y;
+    if (ax < 0.625f) {
+        const float z = x * x;
+        float p = -5.70498872745e-3f;
+        p = sg_fma(p, z, 2.06390887954e-2f);
+        p = sg_fma(p, z, -5.37397155531e-2f);
+        p = sg_fma(p, z, 1.33314422036e-1f);
+        p = sg_fma(p, z, -3.33332819422e-1f);
+        y = sg_fma(p * z, x, x);
+    } else {
+        const float t = 1.0f - 2.0f / (sg_exp(ax + ax) + 1.0f);
+        y = sg_i2f(sg_f2i(t) | (sg_f2i(x) & (int32_t)0x80000000));
+    }
+    return y;
+}
+
+#endif /* SG_MATH_H_ */

@@ -1,0 +1,523 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement of the SuperGrok v2 per-tensor
+ * optimizer step (magnitude sort -> bidirectional Mamba-3 scan -> per-element
+ * GRU -> 4-head PEER routing -> expert MLP -> mu/Adam/weight decay).
+ * Nothing in the shipped package links, imports or executes this file; it is
+ * the checker used by tests/, by the smoke check and by the cpu_baseline leg
+ * of bench.py.
+ *
+ * Two arithmetic policies share one algorithm template:
+ *   F32  fp32 with the fixed-order primitives of include/sg_math.h -- the
+ *        device kernels use the same primitives and the same operation
+ *        order, so integer results (sort permutation, expert indices,
+ *        expert_counts) must match bit for bit and float results to ~1 ulp.
+ *   F64  double precision, the reference's formulas written literally with
+ *        libm -- the "what the mathematics says" answer the F32 result is
+ *        pinned against (tests/test_oracle_*.py) and the source of the
+ *        top-1/top-2 routing margins.
+ *
+ * Reference lines followed (paths relative to the reference tree):
+ *   input projection, non-finite guard, |g| keys
+ *       csrc/supergrok2_mamba_peer_kernels.cu:92-117
+ *       grokking_optimizers/mamba3_peer_metanet.py:296-307
+ *   ascending stable sort of |g|
+ *       csrc/supergrok2_mamba_peer_kernels.cu:1538-1543,1860-1879 (radix sort => stable)
+ *   per-timestep projections xb,z,dt,B,C
+ *       csrc/supergrok2_mamba_peer_kernels.cu:289-346
+ *       grokking_optimizers/mamba3_peer_metanet.py:100-111
+ *   recurrence (trapezoidal A_bar, paired RoPE, B_bar*x, y = h.C, gate, D skip)
+ *       csrc/supergrok2_mamba_peer_kernels.cu:201-268
+ *       grokking_optimizers/mamba3_peer_metanet.py:122-153
+ *   chunked evaluation of the same recurrence through 2x2 affine summaries
+ *       csrc/supergrok2_mamba_peer_kernels.cu:59-80,444-551,662-769
+ *   reverse direction walks t = N-1..0 and writes at t
+ *       csrc/supergrok2_mamba_peer_kernels.cu:202,673
+ *       grokking_optimizers/mamba3_peer_metanet.py:311-312
+ *   out_proj, unsort, GRU, PEER argmax routing, expert MLP, skip, mu, Adam, WD
+ *       csrc/supergrok2_mamba_peer_kernels.cu:917-1088
+ *       grokking_optimizers/mamba3_peer_metanet.py:158,186-192,334-367
+ *       grokking_optimizers/supergrok2.py:451-464
+ *
+ * chunk_len semantics: the sequence (in scan order) is cut into chunks of
+ * chunk_len steps.  For every chunk but the last, the 2x2 affine summary
+ * (M,b) of each (column j, RoPE pair p) is accumulated from the identity;
+ * chunk start states follow by applying the summaries in order to the
+ * carried state; each chunk is then replayed directly from its start state.
+ * chunk_len <= 0 (or >= N) is the plain sequential recurrence of
+ * csrc/supergrok2_mamba_peer_kernels.cu:138-272.  The reference's own
+ * chunking (ceil(N/512) steps per thread, Blelloch tree over 512 summaries)
+ * is one more member of this family: all of them differ from the sequential
+ * result only by re-association of the affine products.
+ *
+ * Parity status: the reference's tests hold no golden vectors for this path
+ * (tests/test_supergrok2.py checks finiteness and run-to-run determinism
+ * only) and its CUDA kernels cannot run here, so every function below is
+ * pinned by the independent checks in tests/test_oracle_*.py (numpy/torch
+ * restatements, closed forms, library routines), not by reference outputs.
+ */
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "../include/sg_math.h"
+
+namespace {
+
+struct Dims {
+    int d_model, d_state, d_inner, gru_hidden, num_heads, pk_dim, expert_hidden, num_experts;
+};
+
+/* pointer order = argument order of supergrok2_mamba_peer_batched_step
+ * (csrc/ops.h:548-581) from input_proj_W to expert_b2 */
+enum {
+    W_IN_W = 0, W_IN_B,
+    W_F_INPROJ, W_F_DTW, W_F_DTB, W_F_B, W_F_C, W_F_ALOG, W_F_D, W_F_ROPE, W_F_OUT,
+    W_B_INPROJ, W_B_DTW, W_B_DTB, W_B_B, W_B_C, W_B_ALOG, W_B_D, W_B_ROPE, W_B_OUT,
+    W_GRU_WZ, W_GRU_BZ, W_GRU_WR, W_GRU_BR, W_GRU_WH, W_GRU_BH,
+    W_PEER_Q, W_KEYS_A, W_KEYS_B,
+    W_EXP_W1, W_EXP_B1, W_EXP_W2, W_EXP_B2,
+    W_COUNT
+};
+
+enum { S_ALPHA = 0, S_LAMB, S_BETA1, S_BC1, S_BC2, S_RESCALE, S_BETA2, S_LR, S_WD, S_EPS, S_COUNT };
+
+/* ---------------- 16-bit float conversions (round to nearest even) -------- */
+inline float bf16_to_f(uint16_t h) {
+    uint32_t u = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+inline uint16_t f_to_bf16(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+inline float f16_to_f(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1f, man = h & 0x3ffu, u;
+    if (exp == 0) {
+        if (man == 0) u = sign;
+        else {
+            int e = -1;
+            do { e++; man <<= 1; } while ((man & 0x400u) == 0);
+            u = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) u = sign | 0x7f800000u | (man << 13);
+    else u = sign | ((exp + 112) << 23) | (man << 13);
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+inline uint16_t f_to_f16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7fffffffu;
+    if (x >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | (x > 0x7f800000u ? 0x200u : 0));
+    if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);          /* overflow -> inf */
+    if (x < 0x33000001u) return (uint16_t)sign;                       /* underflow -> 0 */
+    int e = (int)(x >> 23);
+    uint32_t m = (x & 0x7fffffu) | 0x800000u;
+    int shift;
+    uint32_t base;
+    if (e < 113) { shift = 126 - e; base = 0; }        /* subnormal half */
+    else { shift = 13; base = (uint32_t)(e - 112) << 10; m &= 0x7fffffu; }
+    uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    uint32_t r = base + q;
+    if (rem > half || (rem == half && (r & 1u))) r++;
+    return (uint16_t)(sign | r);
+}
+inline float load_as_f(const void* p, int dtype, int64_t i) {
+    if (dtype == 0) return ((const float*)p)[i];
+    if (dtype == 1) return f16_to_f(((const uint16_t*)p)[i]);
+    return bf16_to_f(((const uint16_t*)p)[i]);
+}
+inline void store_from_f(void* p, int dtype, int64_t i, float v) {
+    if (dtype == 0) ((float*)p)[i] = v;
+    else if (dtype == 1) ((uint16_t*)p)[i] = f_to_f16(v);
+    else ((uint16_t*)p)[i] = f_to_bf16(v);
+}
+
+/* ---------------- arithmetic policies ------------------------------------ */
+struct F32 {
+    typedef float R;
+    static R fma(R a, R b, R c) { return sg_fma(a, b, c); }
+    static R exp(R x) { return sg_exp(x); }
+    static R softplus(R x) { return sg_softplus(x); }
+    static R sigmoid(R x) { return sg_sigmoid(x); }
+    static R silu(R x) { return sg_silu(x); }
+    static R tanh(R x) { return sg_tanh(x); }
+    static R sqrt(R x) { return __builtin_sqrtf(x); }
+    static void sincos(R t, R* s, R* c) { sg_sincos(t, s, c); }
+    /* A is the (negative) continuous-time pole; the primitive wants A/2 */
+    static void abar_pair(R dt, R A_e, R A_o, R* e, R* o) { sg_abar_pair(dt, 0.5f * A_e, 0.5f * A_o, e, o); }
+};
+struct F64 {
+    typedef double R;
+    static R fma(R a, R b, R c) { return a * b + c; }
+    static R exp(R x) { return std::exp(x); }
+    static R softplus(R x) { return (x > 20.0) ? x : std::log(1.0 + std::exp(x)); }
+    static R sigmoid(R x) { return 1.0 / (1.0 + std::exp(-x)); }
+    static R silu(R x) { return x / (1.0 + std::exp(-x)); }
+    static R tanh(R x) { return std::tanh(x); }
+    static R sqrt(R x) { return std::sqrt(x); }
+    static void sincos(R t, R* s, R* c) { *s = std::sin(t); *c = std::cos(t); }
+    static void abar_pair(R dt, R A_e, R A_o, R* e, R* o) {
+        *e = (1.0 + dt * A_e / 2.0) / (1.0 - dt * A_e / 2.0 + 1e-8);
+        *o = (1.0 + dt * A_o / 2.0) / (1.0 - dt * A_o / 2.0 + 1e-8);
+    }
+};
+
+/* ---------------- stable ascending sort of |g| ---------------------------- */
+void sort_perm(const float* g, int64_t N, int32_t* perm) {
+    std::vector<uint32_t> key(N);
+    for (int64_t i = 0; i < N; i++) {
+        float v = sg_isfinite(g[i]) ? g[i] : 0.0f;
+        key[i] = (uint32_t)sg_f2i(sg_abs(v));      /* non-negative floats order like their bits */
+        perm[i] = (int32_t)i;
+    }
+    std::stable_sort(perm, perm + N, [&](int32_t a, int32_t b) { return key[a] < key[b]; });
+}
+
+/* ---------------- one scan direction -------------------------------------- */
+template <class O>
+struct DirW {
+    const float *in_proj, *dt_W, *dt_b, *Bp, *Cp, *A_log, *D, *rope, *out_proj;
+};
+
+template <class O>
+struct StepProj {           /* per-timestep projections */
+    typename O::R xb[32], z[32], dt[32], B[32], C[32];
+};
+
+template <class O>
+void project(const Dims& d, const DirW<O>& w, const typename O::R* x, bool need_zc, StepProj<O>& o) {
+    typedef typename O::R R;
+    const int dm = d.d_model, di = d.d_inner, ds = d.d_state;
+    for (int j = 0; j < di; j++) {
+        R a = 0, b = 0;
+        for (int k = 0; k < dm; k++) a = O::fma((R)w.in_proj[j * dm + k], x[k], a);
+        if (need_zc)
+            for (int k = 0; k < dm; k++) b = O::fma((R)w.in_proj[(j + di) * dm + k], x[k], b);
+        o.xb[j] = a;
+        o.z[j] = b;
+    }
+    for (int j = 0; j < di; j++) {
+        R a = (R)w.dt_b[j];
+        for (int k = 0; k < di; k++) a = O::fma((R)w.dt_W[j * di + k], o.xb[k], a);
+        o.dt[j] = O::softplus(a);
+    }
+    for (int s = 0; s < ds; s++) {
+        R a = 0, b = 0;
+        for (int k = 0; k < di; k++) a = O::fma((R)w.Bp[s * di + k], o.xb[k], a);
+        if (need_zc)
+            for (int k = 0; k < di; k++) b = O::fma((R)w.Cp[s * di + k], o.xb[k], b);
+        o.B[s] = a;
+        o.C[s] = b;
+    }
+}
+
+/* x: [N][d_model] in sorted order.  h: [d_inner][d_state] carried state,
+ * updated in place.  ctx: [N][d_model], written at sorted position t. */
+template <class O>
+void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, int64_t N, bool reverse,
+              int64_t chunk_len, typename O::R* h, typename O::R* ctx) {
+    typedef typename O::R R;
+    const int dm = d.d_model, di = d.d_inner, ds = d.d_state, hp = ds / 2;
+    if (N <= 0) return;
+    if (chunk_len <= 0 || chunk_len > N) chunk_len = N;
+    const int64_t nchunks = (N + chunk_len - 1) / chunk_len;
+
+    std::vector<R> A(di * ds);
+    for (int i = 0; i < di * ds; i++) A[i] = -O::exp((R)w.A_log[i]);
+
+    std::vector<R> hstart((size_t)nchunks * di * ds);
+    std::copy(h, h + di * ds, hstart.begin());
+    StepProj<O> sp;
+
+    /* pass 1 + 2: summaries of chunks 0..nchunks-2, start states of 1..nchunks-1 */
+    std::vector<R> sm(di * hp * 6);
+    for (int64_t c = 0; c + 1 < nchunks; c++) {
+        for (int i = 0; i < di * hp; i++) {
+            R* m = &sm[i * 6];
+            m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 1; m[4] = 0; m[5] = 0;   /* col0=(m0,m1) col1=(m2,m3) b=(m4,m5) */
+        }
+        for (int64_t u = c * chunk_len; u < (c + 1) * chunk_len; u++) {
+            const int64_t t = reverse ? (N - 1 - u) : u;
+            project<O>(d, w, x + t * dm, false, sp);
+            for (int j = 0; j < di; j++) {
+                const R dt = sp.dt[j], xb = sp.xb[j];
+                for (int p = 0; p < hp; p++) {
+                    R ae, ao, sn, cs;
+                    O::abar_pair(dt, A[j * ds + 2 * p], A[j * ds + 2 * p + 1], &ae, &ao);
+                    O::sincos(dt * (R)w.rope[j * hp + p], &sn, &cs);
+                    const R be = (dt * sp.B[2 * p]) * xb, bo = (dt * sp.B[2 * p + 1]) * xb;
+                    R* m = &sm[(j * hp + p) * 6];
+                    for (int v = 0; v < 3; v++) {
+                        const R ve = m[2 * v], vo = m[2 * v + 1];
+                        const R re = O::fma(ve, cs, -(vo * sn));
+                        const R ro = O::fma(vo, cs, ve * sn);
+                        if (v < 2) { m[2 * v] = ae * re; m[2 * v + 1] = ao * ro; }
+                        else { m[4] = O::fma(ae, re, be); m[5] = O::fma(ao, ro, bo); }
+                    }
+                }
+            }
+        }
+        const R* h0 = &hstart[(size_t)c * di * ds];
+        R* h1 = &hstart[(size_t)(c + 1) * di * ds];
+        for (int j = 0; j < di; j++)
+            for (int p = 0; p < hp; p++) {
+                const R* m = &sm[(j * hp + p) * 6];
+                const R he = h0[j * ds + 2 * p], ho = h0[j * ds + 2 * p + 1];
+                h1[j * ds + 2 * p] = O::fma(m[0], he, O::fma(m[2], ho, m[4]));
+                h1[j * ds + 2 * p + 1] = O::fma(m[1], he, O::fma(m[3], ho, m[5]));
+            }
+    }
+
+    /* pass 3: replay every chunk from its start state */
+    std::vector<R> hc(di * ds), yp(hp), out(di);
+    for (int64_t c = 0; c < nchunks; c++) {
+        std::copy(&hstart[(size_t)c * di * ds], &hstart[(size_t)c * di * ds] + di * ds, hc.begin());
+        const int64_t u_end = std::min<int64_t>((c + 1) * chunk_len, N);
+        for (int64_t u = c * chunk_len; u < u_end; u++) {
+            const int64_t t = reverse ? (N - 1 - u) : u;
+            project<O>(d, w, x + t * dm, true, sp);
+            for (int j = 0; j < di; j++) {
+                const R dt = sp.dt[j], xb = sp.xb[j];
+                for (int p = 0; p < hp; p++) {
+                    R ae, ao, sn, cs;
+                    O::abar_pair(dt, A[j * ds + 2 * p], A[j * ds + 2 * p + 1], &ae, &ao);
+                    O::sincos(dt * (R)w.rope[j * hp + p], &sn, &cs);
+                    const R be = (dt * sp.B[2 * p]) * xb, bo = (dt * sp.B[2 * p + 1]) * xb;
+                    const R he = hc[j * ds + 2 * p], ho = hc[j * ds + 2 * p + 1];
+                    const R re = O::fma(he, cs, -(ho * sn));
+                    const R ro = O::fma(ho, cs, he * sn);
+                    const R ne = O::fma(ae, re, be), no = O::fma(ao, ro, bo);
+                    hc[j * ds + 2 * p] = ne;
+                    hc[j * ds + 2 * p + 1] = no;
+                    yp[p] = O::fma(no, sp.C[2 * p + 1], ne * sp.C[2 * p]);
+                }
+                /* balanced pairwise sum over the RoPE pairs (stride 1, 2, 4, ...) */
+                for (int st = 1; st < hp; st *= 2)
+                    for (int p = 0; p + st < hp; p += 2 * st) yp[p] = yp[p] + yp[p + st];
+                out[j] = O::fma(yp[0], O::silu(sp.z[j]), (R)w.D[j] * xb);
+            }
+            for (int dd = 0; dd < dm; dd++) {
+                R a = 0;
+                for (int j = 0; j < di; j++) a = O::fma((R)w.out_proj[dd * di + j], out[j], a);
+                ctx[t * dm + dd] = a;
+            }
+        }
+    }
+    std::copy(hc.begin(), hc.end(), h);
+}
+
+/* ---------------- full step for one tensor -------------------------------- */
+template <class O>
+int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int dtype, void* param,
+                const void* grad, const void* sharp, float* ea_io, float* easq_io, float* mu_io,
+                float* gru_io, float* mfwd_io, float* mbwd_io, int64_t N, const float* sc,
+                int32_t* expert_counts, int32_t* perm_out, int32_t* eidx_out, float* ctx_out,
+                float* margin_out, float* smart_out) {
+    typedef typename O::R R;
+    const int dm = d.d_model, di = d.d_inner, ds = d.d_state, gh = d.gru_hidden, H = d.num_heads;
+    const int pk = d.pk_dim, eh = d.expert_hidden, E = d.num_experts, hd = dm / 2;
+    if (N <= 0) return 0;
+    if (ds % 2 || ds > 32 || dm > 16 || gh > 8 || di > 32 || di % 4) return 1;
+
+    std::vector<float> g(N), s(N);
+    for (int64_t i = 0; i < N; i++) {
+        float gv = load_as_f(grad, dtype, i), sv = load_as_f(sharp, dtype, i);
+        g[i] = sg_isfinite(gv) ? gv : 0.0f;
+        s[i] = sg_isfinite(sv) ? sv : 0.0f;
+    }
+    std::vector<int32_t> perm(N);
+    sort_perm(g.data(), N, perm.data());
+    if (perm_out) std::copy(perm.begin(), perm.end(), perm_out);
+
+    /* input projection, gathered into sorted order */
+    std::vector<R> x((size_t)N * dm);
+    for (int64_t t = 0; t < N; t++) {
+        const R gv = g[perm[t]], sv = s[perm[t]];
+        for (int k = 0; k < dm; k++)
+            x[t * dm + k] = O::fma((R)W[W_IN_W][2 * k + 1], sv, (R)W[W_IN_W][2 * k] * gv) + (R)W[W_IN_B][k];
+    }
+
+    std::vector<R> ctx_sorted[2];
+    std::vector<R> hst[2];
+    for (int dir = 0; dir < 2; dir++) {
+        const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8]};
+        float* st = dir ? mbwd_io : mfwd_io;
+        hst[dir].assign(st, st + di * ds);
+        ctx_sorted[dir].resize((size_t)N * dm);
+        scan_dir<O>(d, w, x.data(), N, dir == 1, chunk_len, hst[dir].data(), ctx_sorted[dir].data());
+        for (int i = 0; i < di * ds; i++) st[i] = (float)hst[dir][i];
+    }
+    /* unsort: element perm[t] takes the context computed at sorted position t */
+    std::vector<R> cf((size_t)N * dm), cb((size_t)N * dm);
+    for (int64_t t = 0; t < N; t++)
+        for (int k = 0; k < dm; k++) {
+            cf[(size_t)perm[t] * dm + k] = ctx_sorted[0][t * dm + k];
+            cb[(size_t)perm[t] * dm + k] = ctx_sorted[1][t * dm + k];
+        }
+    if (ctx_out)
+        for (int64_t i = 0; i < N * dm; i++) {
+            ctx_out[i] = (float)cf[i];
+            ctx_out[(size_t)N * dm + i] = (float)cb[i];
+        }
+
+    const R alpha = sc[S_ALPHA], lamb = sc[S_LAMB], beta1 = sc[S_BETA1], beta2 = sc[S_BETA2];
+    const R rescale = sc[S_RESCALE], eps = sc[S_EPS];
+    R step_size, decay, bc2;
+    if (sizeof(R) == 4) {     /* fp32 host scalars exactly as the device entry point derives them */
+        step_size = sc[S_LR] / sc[S_BC1];
+        decay = 1.0f - sc[S_LR] * sc[S_WD];
+        bc2 = sc[S_BC2];
+    } else {
+        step_size = (R)sc[S_LR] / (R)sc[S_BC1];
+        decay = 1.0 - (R)sc[S_LR] * (R)sc[S_WD];
+        bc2 = sc[S_BC2];
+    }
+    const int grl = 2 + 2 * dm + gh, pin = gh + 2 * dm + 2;
+    const float *Wz = W[W_GRU_WZ], *bz = W[W_GRU_BZ], *Wr = W[W_GRU_WR], *br = W[W_GRU_BR];
+    const float *Wh = W[W_GRU_WH], *bh = W[W_GRU_BH];
+
+    for (int64_t i = 0; i < N; i++) {
+        const R gv = g[i], sv = s[i];
+        const R* f = &cf[(size_t)i * dm];
+        const R* b = &cb[(size_t)i * dm];
+        R hold[8], zg[8], rg[8], hnew[8];
+        for (int k = 0; k < gh; k++) hold[k] = gru_io[i * gh + k];
+        /* GRU gates: chain = bias, g, s, fwd ctx, bwd ctx, h */
+        for (int j = 0; j < gh; j++) {
+            const float *wz = Wz + j * grl, *wr = Wr + j * grl;
+            R vz = bz[j], vr = br[j];
+            vz = O::fma((R)wz[0], gv, vz); vz = O::fma((R)wz[1], sv, vz);
+            vr = O::fma((R)wr[0], gv, vr); vr = O::fma((R)wr[1], sv, vr);
+            for (int k = 0; k < dm; k++) { vz = O::fma((R)wz[2 + k], f[k], vz); vr = O::fma((R)wr[2 + k], f[k], vr); }
+            for (int k = 0; k < dm; k++) { vz = O::fma((R)wz[2 + dm + k], b[k], vz); vr = O::fma((R)wr[2 + dm + k], b[k], vr); }
+            for (int k = 0; k < gh; k++) { vz = O::fma((R)wz[2 + 2 * dm + k], hold[k], vz); vr = O::fma((R)wr[2 + 2 * dm + k], hold[k], vr); }
+            zg[j] = O::sigmoid(vz);
+            rg[j] = O::sigmoid(vr);
+        }
+        for (int j = 0; j < gh; j++) {
+            const float* wh = Wh + j * grl;
+            R v = bh[j];
+            v = O::fma((R)wh[0], gv, v); v = O::fma((R)wh[1], sv, v);
+            for (int k = 0; k < dm; k++) v = O::fma((R)wh[2 + k], f[k], v);
+            for (int k = 0; k < dm; k++) v = O::fma((R)wh[2 + dm + k], b[k], v);
+            for (int k = 0; k < gh; k++) v = O::fma((R)wh[2 + 2 * dm + k], rg[k] * hold[k], v);
+            const R ht = O::tanh(v);
+            hnew[j] = O::fma(zg[j], ht, ((R)1 - zg[j]) * hold[j]);
+        }
+        for (int k = 0; k < gh; k++) gru_io[i * gh + k] = (float)hnew[k];
+
+        /* PEER: per head query -> two sub-key argmaxes -> expert MLP */
+        R total = 0;
+        for (int hh = 0; hh < H; hh++) {
+            const float* q = W[W_PEER_Q] + (size_t)hh * dm * pin;
+            R query[16];
+            for (int dd = 0; dd < dm; dd++) {
+                const float* qr = q + dd * pin;
+                R v = 0;
+                for (int k = 0; k < gh; k++) v = O::fma((R)qr[k], hnew[k], v);
+                for (int k = 0; k < dm; k++) v = O::fma((R)qr[gh + k], f[k], v);
+                for (int k = 0; k < dm; k++) v = O::fma((R)qr[gh + dm + k], b[k], v);
+                v = O::fma((R)qr[gh + 2 * dm], gv, v);
+                v = O::fma((R)qr[gh + 2 * dm + 1], sv, v);
+                query[dd] = v;
+            }
+            int best[2];
+            for (int half = 0; half < 2; half++) {
+                const float* keys = W[half ? W_KEYS_B : W_KEYS_A] + (size_t)hh * pk * hd;
+                int bi = 0;
+                R bs = (R)-1e30f, second = (R)-1e30f;
+                for (int k = 0; k < pk; k++) {
+                    R dot = 0;
+                    for (int dd = 0; dd < hd; dd++) dot = O::fma(query[half * hd + dd], (R)keys[k * hd + dd], dot);
+                    if (dot > bs) { second = bs; bs = dot; bi = k; }
+                    else if (dot > second) second = dot;
+                }
+                best[half] = bi;
+                if (margin_out) margin_out[((size_t)i * H + hh) * 2 + half] = (float)(bs - second);
+            }
+            int e = best[0] * pk + best[1];
+            if (e >= E) e = E - 1;
+            if (expert_counts) expert_counts[e] += 1;
+            if (eidx_out) eidx_out[(size_t)i * H + hh] = e;
+            R ho = W[W_EXP_B2][e];
+            for (int k = 0; k < eh; k++) {
+                R zv = O::fma((R)W[W_EXP_W1][e * eh + k], gv, (R)W[W_EXP_B1][e * eh + k]);
+                zv = zv > 0 ? zv : (R)0;
+                ho = O::fma((R)W[W_EXP_W2][e * eh + k], zv, ho);
+            }
+            total = total + ho;
+        }
+        const R smart = gv + (rescale * total) / (R)H;
+        if (smart_out) smart_out[i] = (float)smart;
+
+        R mu = mu_io[i];
+        mu = O::fma(alpha, mu, ((R)1 - alpha) * gv);
+        mu_io[i] = (float)mu;
+        const R fg = O::fma(lamb, mu, smart);
+        R ea = ea_io[i], easq = easq_io[i];
+        ea = O::fma(beta1, ea, ((R)1 - beta1) * fg);
+        easq = O::fma(beta2, easq, (((R)1 - beta2) * fg) * fg);
+        ea_io[i] = (float)ea;
+        easq_io[i] = (float)easq;
+        const R denom = O::sqrt(easq / bc2) + eps;
+        R p = load_as_f(param, dtype, i);
+        p = O::fma(p, decay, -((step_size * ea) / denom));
+        store_from_f(param, dtype, i, (float)p);
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+/* stable ascending argsort of |g| with non-finite entries treated as 0 */
+void orc_sort_perm(const float* g, int64_t N, int32_t* perm) { sort_perm(g, N, perm); }
+
+/* One tensor, one optimizer step.  precision: 32 or 64.  dims[8] and
+ * scalars[10] in the enum orders above; W = 33 weight pointers.  Optional
+ * outputs may be NULL: perm [N], expert_idx [N][H], ctx [2][N][d_model]
+ * (forward then backward context in original element order), margin
+ * [N][H][2] (top-1 minus top-2 score per sub-key), smart [N]. */
+int orc_sg2_step(int precision, int64_t chunk_len, const float* const* W, const int32_t* dims,
+                 int dtype, void* param, const void* grad, const void* sharp, float* ea, float* easq,
+                 float* mu, float* gru, float* mfwd, float* mbwd, int64_t N, const float* scalars,
+                 int32_t* expert_counts, int32_t* perm, int32_t* expert_idx, float* ctx, float* margin,
+                 float* smart) {
+    Dims d = {dims[0], dims[1], dims[2], dims[3], dims[4], dims[5], dims[6], dims[7]};
+    if (precision == 32)
+        return step_tensor<F32>(d, W, chunk_len, dtype, param, grad, sharp, ea, easq, mu, gru, mfwd, mbwd,
+                                N, scalars, expert_counts, perm, expert_idx, ctx, margin, smart);
+    return step_tensor<F64>(d, W, chunk_len, dtype, param, grad, sharp, ea, easq, mu, gru, mfwd, mbwd, N,
+                            scalars, expert_counts, perm, expert_idx, ctx, margin, smart);
+}
+
+/* primitives exported one by one so tests can pin them against libm */
+float orc_exp(float x) { return sg_exp(x); }
+float orc_log(float x) { return sg_log(x); }
+float orc_softplus(float x) { return sg_softplus(x); }
+float orc_sigmoid(float x) { return sg_sigmoid(x); }
+float orc_silu(float x) { return sg_silu(x); }
+float orc_tanh(float x) { return sg_tanh(x); }
+float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }
+float orc_cos(float x) { float s, c; sg_sincos(x, &s, &c); return c; }
+float orc_rcp_pos(float x) { return sg_rcp_pos(x); }
+float orc_abar(float dt, float A) { float e, o; sg_abar_pair(dt, 0.5f * A, 0.5f * A, &e, &o); return e; }
+uint16_t orc_f_to_f16(float f) { return f_to_f16(f); }
+float orc_f16_to_f(uint16_t h) { return f16_to_f(h); }
+uint16_t orc_f_to_bf16(float f) { return f_to_bf16(f); }
+float orc_bf16_to_f(uint16_t h) { return bf16_to_f(h); }
+
+}  // extern "C"

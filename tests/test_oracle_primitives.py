@@ -1,0 +1,104 @@
+"""Pins the fixed-order fp32 primitives (include/sg_math.h, exported by the
+CPU checker) against libm in double precision."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import oracle as orc
+
+L = orc.lib()
+RNG = np.random.RandomState(123)
+
+
+def _maxrel(fn, ref, xs, floor=1e-30):
+    worst = 0.0
+    for x in xs:
+        x = float(np.float32(x))
+        r = ref(x)
+        worst = max(worst, abs(fn(x) - r) / max(abs(r), floor))
+    return worst
+
+
+def test_exp():
+    xs = np.concatenate([RNG.uniform(-80, 80, 20000), [0.0, -0.0, 1e-8, -86.0, 88.0, 20.0, -20.0]])
+    assert _maxrel(L.orc_exp, math.exp, xs) < 2e-7
+    # clamp: stays finite and monotone at the ends
+    assert L.orc_exp(200.0) == L.orc_exp(88.0) and L.orc_exp(-200.0) == L.orc_exp(-86.0)
+    assert L.orc_exp(0.0) == 1.0
+
+
+def test_log():
+    xs = np.exp(RNG.uniform(-30, 30, 20000))
+    assert _maxrel(L.orc_log, math.log, xs, floor=1e-3) < 2e-7
+    assert L.orc_log(1.0) == 0.0
+
+
+def test_softplus_is_the_literal_fp32_formula():
+    # log(1+exp(x)) with 1+exp(x) rounded to fp32 first, as the reference writes it
+    def ref(x):
+        if x > 20.0:
+            return x
+        return math.log(float(np.float32(1.0) + np.float32(math.exp(x))))
+    xs = RNG.uniform(-30, 30, 20000)
+    worst = 0.0
+    for x in xs:
+        x = float(np.float32(x))
+        worst = max(worst, abs(L.orc_softplus(x) - ref(x)))
+    assert worst < 3e-7 * 21
+    assert L.orc_softplus(25.0) == 25.0
+    assert L.orc_softplus(-30.0) == 0.0      # 1+e^-30 rounds to 1 in fp32
+
+
+def test_sigmoid_silu_tanh():
+    xs = RNG.uniform(-30, 30, 20000)
+    assert _maxrel(L.orc_sigmoid, lambda x: 1 / (1 + math.exp(-x)), xs) < 3e-7
+    assert _maxrel(L.orc_silu, lambda x: x / (1 + math.exp(-x)), xs) < 3e-7
+    xs = np.concatenate([RNG.uniform(-9, 9, 20000), RNG.uniform(-0.7, 0.7, 5000), [0.0, 0.625, -0.625, 1e-6]])
+    assert _maxrel(L.orc_tanh, math.tanh, xs) < 4e-7
+    assert L.orc_tanh(0.0) == 0.0 and L.orc_tanh(30.0) == 1.0 and L.orc_tanh(-30.0) == -1.0
+
+
+def test_sincos():
+    xs = np.concatenate([RNG.uniform(-100, 100, 30000), RNG.uniform(-1, 1, 5000),
+                         [0.0, math.pi / 4, -math.pi / 4, math.pi / 2, math.pi, 3 * math.pi / 2]])
+    ws, wc = 0.0, 0.0
+    for x in xs:
+        x = float(np.float32(x))
+        ws = max(ws, abs(L.orc_sin(x) - math.sin(x)))
+        wc = max(wc, abs(L.orc_cos(x) - math.cos(x)))
+    assert ws < 2.5e-7 and wc < 2.5e-7
+    assert L.orc_sin(0.0) == 0.0 and L.orc_cos(0.0) == 1.0
+
+
+def test_rcp_and_abar():
+    ds = np.exp(RNG.uniform(0, 60, 20000))
+    assert _maxrel(L.orc_rcp_pos, lambda d: 1.0 / d, ds) < 1.5e-7
+    worst = 0.0
+    for _ in range(20000):
+        dt = float(np.float32(RNG.uniform(0, 25)))
+        A = float(np.float32(-math.exp(RNG.uniform(-6, 4))))
+        ref = (1.0 + dt * A / 2.0) / (1.0 - dt * A / 2.0 + 1e-8)
+        worst = max(worst, abs(L.orc_abar(dt, A) - ref) / max(abs(ref), 1e-2))
+    assert worst < 6e-7
+    # the dropped "+1e-8f": for every denominator >= 1 it is an fp32 no-op
+    dens = np.float32(1.0) + np.abs(RNG.randn(100000).astype(np.float32)) * np.float32(10)
+    dens = np.concatenate([dens, np.float32([1.0, np.nextafter(np.float32(1), np.float32(2))])])
+    assert np.array_equal(dens + np.float32(1e-8), dens)
+    assert L.orc_abar(0.0, -1.0) == 1.0
+
+
+def test_half_conversions_match_numpy():
+    xs = np.concatenate([RNG.randn(20000).astype(np.float32) * np.float32(10.0 ** RNG.randint(-9, 6)),
+                         np.float32([0, -0.0, 65504, 65520, 1e-8, 6e-8, 6.1e-5, np.inf, -np.inf])])
+    for x in xs:
+        h = np.float32(x).astype(np.float16)
+        assert L.orc_f_to_f16(float(x)) == int(h.view(np.uint16)), x
+        assert L.orc_f16_to_f(int(h.view(np.uint16))) == float(h) or np.isnan(float(h))
+    import torch
+    t = torch.from_numpy(xs[np.isfinite(xs)])
+    b = t.to(torch.bfloat16)
+    bits = b.view(torch.int16).numpy().view(np.uint16)
+    for x, hb, back in zip(t.numpy(), bits, b.float().numpy()):
+        assert L.orc_f_to_bf16(float(x)) == int(hb)
+        assert L.orc_bf16_to_f(int(hb)) == float(back)
