@@ -1,0 +1,105 @@
+/*
+ * sg_abi.h -- C ABI of libsg_hip.so: hand-written gfx950 kernels for the
+ * fused per-parameter optimizer steps.  Plain pointers and sizes only; no
+ * torch types.  Every entry point
+ *   - returns 0 on success, non-zero on error (sg_last_error() has the text;
+ *     no exception crosses the boundary),
+ *   - enqueues its work on the hipStream_t passed as `stream` (void* so the
+ *     header needs no HIP include) and returns without synchronising,
+ *   - performs no device allocation: scratch memory comes in as `workspace`.
+ *
+ * The torch extension `_ops` (csrc/ops_shim.cpp in the package) keeps the
+ * reference's pybind signatures and forwards here.  Each declaration names
+ * the reference interface it stands behind (paths relative to the reference
+ * tree).
+ */
+#ifndef SG_ABI_H_
+#define SG_ABI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type of param / grad / sharpness tensors */
+enum { SG_F32 = 0, SG_F16 = 1, SG_BF16 = 2 };
+
+/* meta-net dimensions, the trailing ints of
+ * launch_mamba3_peer_batched_step (csrc/ops.h:342-370) */
+typedef struct SgDims {
+    int32_t d_model, d_state, d_inner, gru_hidden, num_heads, pk_dim, expert_hidden, num_experts;
+} SgDims;
+
+/* The 33 fp32 meta-net weight tensors (device pointers) in the argument
+ * order of supergrok2_mamba_peer_batched_step (csrc/ops.h:548-581):
+ * input_proj_W, input_proj_b, 9 forward-Mamba, 9 backward-Mamba
+ * (in_proj, dt_W, dt_b, B_proj, C_proj, A_log, D, rope, out_proj),
+ * gru_Wz,bz,Wr,br,Wh,bh, peer_query_Ws, prod_keys_A, prod_keys_B,
+ * expert_W1, expert_b1, expert_W2, expert_b2.
+ * Shapes: csrc/supergrok2_mamba_peer_kernels.cu:1453-1487. */
+#define SG2_NUM_WEIGHTS 33
+typedef struct Sg2Weights {
+    const float* w[SG2_NUM_WEIGHTS];
+} Sg2Weights;
+
+/* One parameter tensor of the batched step: the i-th entries of the
+ * std::vector arguments of supergrok2_mamba_peer_batched_step
+ * (csrc/ops.h:548-556,575-576).  All pointers are device pointers to
+ * contiguous storage; the tensor is treated as flat (numel elements).
+ * param, grad and sharpness share `dtype`; every state tensor is fp32. */
+typedef struct Sg2Tensor {
+    void* param;              /* [numel]            updated in place        */
+    const void* grad;         /* [numel]            read only               */
+    const void* sharpness;    /* [numel]            read only               */
+    float* exp_avg;           /* [numel]            updated                 */
+    float* exp_avg_sq;        /* [numel]            updated                 */
+    float* mu;                /* [numel]            updated                 */
+    float* gru_state;         /* [numel,gru_hidden] updated                 */
+    float* mamba_fwd_state;   /* [d_inner,d_state]  updated (scan carry)    */
+    float* mamba_bwd_state;   /* [d_inner,d_state]  updated (scan carry)    */
+    int64_t numel;
+    int32_t dtype;            /* SG_F32 / SG_F16 / SG_BF16                  */
+    float alpha_mu, lamb_eff, beta1, bc1, bc2;
+} Sg2Tensor;
+
+/* shared scalars of the batched step (csrc/ops.h:577) */
+typedef struct Sg2Scalars {
+    float rescale, beta2, lr, wd_eff, eps;
+} Sg2Scalars;
+
+/* Optional inspection outputs for parity tests (device pointers, any may be
+ * NULL).  Element order is the concatenation of the tensors in call order. */
+typedef struct Sg2Debug {
+    int32_t* perm;          /* [total]     sorted position -> element index within its tensor */
+    int32_t* expert_idx;    /* [total][num_heads]                                             */
+    float* ctx;             /* [2][total][d_model] forward / backward context, element order  */
+} Sg2Debug;
+
+/* text of the last error raised on the calling thread */
+const char* sg_last_error(void);
+
+/* Length (timesteps) of the scan chunks a tensor's sorted sequence is cut
+ * into; a multiple of 64.  0 restores the default (1024).  Affects results
+ * only by re-association of the chunk products. */
+int sg2_set_chunk_len(int chunk_len);
+int sg2_get_chunk_len(void);
+
+/* Bytes of scratch the batched step needs for these tensor sizes. */
+size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
+
+/* SuperGrok v2 full step over all tensors: replaces
+ * launch_mamba3_peer_batched_step (csrc/ops.h:342-370,
+ * csrc/supergrok2_mamba_peer_kernels.cu:1754-2117) behind
+ * supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877).
+ * `tensors` is a host array; tensors with numel == 0 are skipped.
+ * expert_counts: device int32[num_experts], incremented. */
+int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors,
+                     const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
+                     void* workspace, size_t workspace_bytes, const Sg2Debug* debug, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SG_ABI_H_ */

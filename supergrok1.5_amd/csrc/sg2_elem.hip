@@ -1,0 +1,206 @@
+// Per-element tail of the SuperGrok v2 step: GRU -> 4-head PEER product-key
+// routing -> expert MLP -> skip connection -> mu EMA -> Adam + weight decay.
+//
+// Replaces fused_elem_step_kernel
+// (csrc/supergrok2_mamba_peer_kernels.cu:793-1089 of the reference); the
+// out_proj contraction that kernel starts with is done by the scan kernel,
+// which hands over the two 8-float contexts per element in element order.
+//
+// One launch covers every tensor: a persistent grid walks tiles of 1024
+// elements; the tile index is mapped to (tensor, offset) by a binary search
+// over a P+1 entry prefix table.  The 144 expert MLPs live in LDS (records of
+// 48 floats padded to 52 so that random per-lane experts spread over the
+// banks); GRU / query / key weights are wave-uniform and come in through
+// scalar loads.  expert_counts is accumulated in an LDS histogram and flushed
+// once per workgroup (the reference issues one global atomic per element and
+// head).
+#include "sg2_internal.hpp"
+
+namespace sg2 {
+namespace {
+
+constexpr int ELEM_THREADS = 256;
+constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[16] W2[16] + pad
+
+template <bool DBG>
+__global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
+                                                       int32_t* __restrict__ dbg_eidx) {
+    __shared__ float s_exp[NE * EXP_STRIDE];
+    __shared__ float s_b2[NE];
+    __shared__ int s_cnt[NE];
+
+    {
+        const float* __restrict__ W1 = pl.W.w[W_EXP_W1];
+        const float* __restrict__ B1 = pl.W.w[W_EXP_B1];
+        const float* __restrict__ W2 = pl.W.w[W_EXP_W2];
+        for (int i = threadIdx.x; i < NE * EH; i += ELEM_THREADS) {
+            const int e = i / EH, k = i % EH;
+            s_exp[e * EXP_STRIDE + k] = W1[i];
+            s_exp[e * EXP_STRIDE + EH + k] = B1[i];
+            s_exp[e * EXP_STRIDE + 2 * EH + k] = W2[i];
+        }
+        for (int i = threadIdx.x; i < NE; i += ELEM_THREADS) {
+            s_b2[i] = pl.W.w[W_EXP_B2][i];
+            s_cnt[i] = 0;
+        }
+    }
+    __syncthreads();
+
+    const float* __restrict__ Wz = pl.W.w[W_GRU_WZ];
+    const float* __restrict__ bz = pl.W.w[W_GRU_BZ];
+    const float* __restrict__ Wr = pl.W.w[W_GRU_WR];
+    const float* __restrict__ br = pl.W.w[W_GRU_BR];
+    const float* __restrict__ Wh = pl.W.w[W_GRU_WH];
+    const float* __restrict__ bh = pl.W.w[W_GRU_BH];
+    const float* __restrict__ Wq = pl.W.w[W_PEER_Q];
+    const float* __restrict__ KA = pl.W.w[W_KEYS_A];
+    const float* __restrict__ KB = pl.W.w[W_KEYS_B];
+
+    for (int tile = blockIdx.x; tile < pl.elem_tiles; tile += gridDim.x) {
+        const int ti = sg::upper_seg(pl.elem_tile_prefix, pl.P, tile);
+        const TensorDev& T = pl.tensors[ti];
+        const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
+        const int cnt = min(ELEM_TILE, T.numel - start);
+        const int dtype = T.dtype;
+        const float alpha = T.alpha, lamb = T.lamb, beta1 = T.beta1, bc2 = T.bc2, step_size = T.step_size;
+        const float beta2 = pl.beta2, eps = pl.eps, rescale = pl.rescale, decay = pl.decay;
+
+        for (int k = threadIdx.x; k < cnt; k += ELEM_THREADS) {
+            const int i = start + k;
+            const float g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, i));
+            const float s = sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i));
+            float cf[DM], cb[DM], hold[GH];
+            {
+                const float4* pf = reinterpret_cast<const float4*>(pl.ctx + ((size_t)T.off + i) * DM);
+                const float4* pb = reinterpret_cast<const float4*>(pl.ctx + ((size_t)pl.total + T.off + i) * DM);
+                const float4 a0 = pf[0], a1 = pf[1], b0 = pb[0], b1 = pb[1];
+                cf[0] = a0.x; cf[1] = a0.y; cf[2] = a0.z; cf[3] = a0.w; cf[4] = a1.x; cf[5] = a1.y; cf[6] = a1.z; cf[7] = a1.w;
+                cb[0] = b0.x; cb[1] = b0.y; cb[2] = b0.z; cb[3] = b0.w; cb[4] = b1.x; cb[5] = b1.y; cb[6] = b1.z; cb[7] = b1.w;
+                const float4 h4 = reinterpret_cast<const float4*>(T.gru)[i];
+                hold[0] = h4.x; hold[1] = h4.y; hold[2] = h4.z; hold[3] = h4.w;
+            }
+
+            // ---- GRU: chain order = bias, g, s, fwd ctx, bwd ctx, h
+            float zg[GH], rg[GH], hnew[GH];
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const float* wz = Wz + j * GRL;
+                const float* wr = Wr + j * GRL;
+                float vz = bz[j], vr = br[j];
+                vz = sg_fma(wz[0], g, vz); vz = sg_fma(wz[1], s, vz);
+                vr = sg_fma(wr[0], g, vr); vr = sg_fma(wr[1], s, vr);
+#pragma unroll
+                for (int q = 0; q < DM; q++) { vz = sg_fma(wz[2 + q], cf[q], vz); vr = sg_fma(wr[2 + q], cf[q], vr); }
+#pragma unroll
+                for (int q = 0; q < DM; q++) { vz = sg_fma(wz[2 + DM + q], cb[q], vz); vr = sg_fma(wr[2 + DM + q], cb[q], vr); }
+#pragma unroll
+                for (int q = 0; q < GH; q++) { vz = sg_fma(wz[2 + 2 * DM + q], hold[q], vz); vr = sg_fma(wr[2 + 2 * DM + q], hold[q], vr); }
+                zg[j] = sg_sigmoid(vz);
+                rg[j] = sg_sigmoid(vr);
+            }
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const float* wh = Wh + j * GRL;
+                float v = bh[j];
+                v = sg_fma(wh[0], g, v); v = sg_fma(wh[1], s, v);
+#pragma unroll
+                for (int q = 0; q < DM; q++) v = sg_fma(wh[2 + q], cf[q], v);
+#pragma unroll
+                for (int q = 0; q < DM; q++) v = sg_fma(wh[2 + DM + q], cb[q], v);
+#pragma unroll
+                for (int q = 0; q < GH; q++) v = sg_fma(wh[2 + 2 * DM + q], rg[q] * hold[q], v);
+                const float ht = sg_tanh(v);
+                hnew[j] = sg_fma(zg[j], ht, (1.0f - zg[j]) * hold[j]);
+            }
+            reinterpret_cast<float4*>(T.gru)[i] = make_float4(hnew[0], hnew[1], hnew[2], hnew[3]);
+
+            // ---- PEER routing + expert MLP
+            float total = 0.0f;
+#pragma unroll
+            for (int hh = 0; hh < NH; hh++) {
+                float query[DM];
+#pragma unroll
+                for (int dd = 0; dd < DM; dd++) {
+                    const float* qr = Wq + (hh * DM + dd) * PIN;
+                    float v = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < GH; q++) v = sg_fma(qr[q], hnew[q], v);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + q], cf[q], v);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + DM + q], cb[q], v);
+                    v = sg_fma(qr[GH + 2 * DM], g, v);
+                    v = sg_fma(qr[GH + 2 * DM + 1], s, v);
+                    query[dd] = v;
+                }
+                int best[2];
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    const float* keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    int bi = 0;
+                    float bs = -1e30f;
+#pragma unroll
+                    for (int q = 0; q < PK; q++) {
+                        float dot = 0.0f;
+#pragma unroll
+                        for (int dd = 0; dd < DM / 2; dd++) dot = sg_fma(query[hf * (DM / 2) + dd], keys[q * (DM / 2) + dd], dot);
+                        if (dot > bs) { bs = dot; bi = q; }
+                    }
+                    best[hf] = bi;
+                }
+                int e = best[0] * PK + best[1];
+                if (e >= NE) e = NE - 1;
+                atomicAdd(&s_cnt[e], 1);
+                if (DBG) dbg_eidx[((size_t)T.off + i) * NH + hh] = e;
+
+                const float4* rec = reinterpret_cast<const float4*>(s_exp + e * EXP_STRIDE);
+                float ho = s_b2[e];
+#pragma unroll
+                for (int q4 = 0; q4 < EH / 4; q4++) {
+                    const float4 w1 = rec[q4], b1 = rec[EH / 4 + q4], w2 = rec[2 * (EH / 4) + q4];
+                    float z;
+                    z = sg_max(sg_fma(w1.x, g, b1.x), 0.0f); ho = sg_fma(w2.x, z, ho);
+                    z = sg_max(sg_fma(w1.y, g, b1.y), 0.0f); ho = sg_fma(w2.y, z, ho);
+                    z = sg_max(sg_fma(w1.z, g, b1.z), 0.0f); ho = sg_fma(w2.z, z, ho);
+                    z = sg_max(sg_fma(w1.w, g, b1.w), 0.0f); ho = sg_fma(w2.w, z, ho);
+                }
+                total = total + ho;
+            }
+            const float smart = g + (rescale * total) / (float)NH;
+
+            // ---- mu EMA, Adam moments, decoupled weight decay
+            float mu = T.mu[i];
+            mu = sg_fma(alpha, mu, (1.0f - alpha) * g);
+            T.mu[i] = mu;
+            const float fg = sg_fma(lamb, mu, smart);
+            float ea = T.ea[i], easq = T.easq[i];
+            ea = sg_fma(beta1, ea, (1.0f - beta1) * fg);
+            easq = sg_fma(beta2, easq, ((1.0f - beta2) * fg) * fg);
+            T.ea[i] = ea;
+            T.easq[i] = easq;
+            const float denom = __builtin_sqrtf(easq / bc2) + eps;
+            float pv = sg::load_elem(T.param, dtype, i);
+            pv = sg_fma(pv, decay, -((step_size * ea) / denom));
+            sg::store_elem(T.param, dtype, i, pv);
+        }
+    }
+    __syncthreads();
+    if (expert_counts != nullptr)
+        for (int i = threadIdx.x; i < NE; i += ELEM_THREADS)
+            if (s_cnt[i] != 0) atomicAdd(&expert_counts[i], s_cnt[i]);
+}
+
+}  // namespace
+
+int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st) {
+    if (pl.total == 0) return 0;
+    const int grid = pl.elem_tiles < 2048 ? pl.elem_tiles : 2048;
+    if (dbg_expert_idx)
+        hipLaunchKernelGGL(k_elem<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+    else
+        hipLaunchKernelGGL(k_elem<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+    SG_LAUNCH_CHECK("k_elem");
+    return 0;
+}
+
+}  // namespace sg2

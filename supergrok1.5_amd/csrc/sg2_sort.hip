@@ -1,0 +1,229 @@
+// Segmented, stable, ascending LSD radix sort of (|grad| bits, element index)
+// for all parameter tensors at once.  One segment per tensor.
+//
+// Stands in for the reference's input_proj_sort_kernel key generation
+// (csrc/supergrok2_mamba_peer_kernels.cu:92-117) and its
+// cub::DeviceSegmentedRadixSort::SortPairs call (:1860-1879).  Non-negative
+// floats order like their bit patterns, so the keys are sorted as uint32.
+//
+// Four passes of 8 bits.  Per pass:
+//   hist     per-tile digit counts -> spine[segment][digit][tile]
+//   scan     exclusive prefix over the whole spine (3 small kernels).  Because
+//            the spine is laid out segment-major, the global prefix of entry
+//            (seg, d, tile) is exactly: keys in earlier segments + keys of this
+//            segment with a smaller digit + keys with digit d in earlier tiles
+//            = destination of the first such key of this tile.
+//   scatter  stable rank inside the tile (each wave owns a contiguous quarter
+//            of the tile; match-any ballots give the rank among equal digits)
+//            and write to destination.
+#include "sg2_internal.hpp"
+
+namespace sg2 {
+namespace {
+
+constexpr int SORT_THREADS = 256;
+constexpr int ITEMS = SORT_TILE / SORT_THREADS;      // 16 rounds per wave
+constexpr int WAVES = SORT_THREADS / 64;
+constexpr int WAVE_ITEMS = SORT_TILE / WAVES;        // 1024 contiguous keys per wave
+
+// ---- key generation ----------------------------------------------------------
+__global__ __launch_bounds__(256) void k_keys(Plan pl) {
+    const int tile = blockIdx.x;
+    const int ti = sg::upper_seg(pl.elem_tile_prefix, pl.P, tile);
+    const TensorDev& T = pl.tensors[ti];
+    const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
+    const int cnt = min(ELEM_TILE, T.numel - start);
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int i = start + k;
+        const float g = sg::finite_or_zero(sg::load_elem(T.grad, T.dtype, i));
+        pl.keys[0][T.off + i] = (uint32_t)sg_f2i(sg_abs(g));
+        pl.vals[0][T.off + i] = i;
+    }
+}
+
+struct TileRef {
+    int base;        // index of the tile's first key in the packed arrays
+    int cnt;         // keys in the tile
+    int spine0;      // index of spine entry (digit 0) for this tile
+    int stride;      // spine stride between digits (= tiles of the segment)
+};
+__device__ __forceinline__ TileRef tile_ref(const Plan& pl, int tile) {
+    const int seg = sg::upper_seg(pl.sort_tile_prefix, pl.P, tile);
+    const int t0 = pl.sort_tile_prefix[seg];
+    const int nt = pl.sort_tile_prefix[seg + 1] - t0;
+    const TensorDev& T = pl.tensors[seg];
+    TileRef r;
+    r.base = T.off + (tile - t0) * SORT_TILE;
+    r.cnt = min(SORT_TILE, T.numel - (tile - t0) * SORT_TILE);
+    r.spine0 = 256 * t0 + (tile - t0);
+    r.stride = nt;
+    return r;
+}
+
+// ---- per-tile histogram ---------------------------------------------------------
+__global__ __launch_bounds__(SORT_THREADS) void k_hist(Plan pl, int src, int shift) {
+    __shared__ uint32_t h[256];
+    const TileRef tr = tile_ref(pl, blockIdx.x);
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const uint32_t* __restrict__ keys = pl.keys[src] + tr.base;
+    for (int k = threadIdx.x; k < tr.cnt; k += SORT_THREADS) atomicAdd(&h[(keys[k] >> shift) & 255u], 1u);
+    __syncthreads();
+    pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
+}
+
+// ---- exclusive scan of the spine -------------------------------------------------
+__device__ __forceinline__ uint32_t wave_incl_scan(uint32_t v) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(v, d, 64);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+// exclusive scan over the 256 threads of a block; *total receives the block sum
+__device__ __forceinline__ uint32_t block_excl_scan(uint32_t v, uint32_t* smem /*[4]*/, uint32_t* total) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const uint32_t inc = wave_incl_scan(v);
+    if (lane == 63) smem[w] = inc;
+    __syncthreads();
+    uint32_t base = 0, tot = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const uint32_t s = smem[k];
+        if (k < w) base += s;
+        tot += s;
+    }
+    __syncthreads();
+    *total = tot;
+    return base + inc - v;
+}
+
+__global__ __launch_bounds__(256) void k_spine_reduce(const uint32_t* __restrict__ spine, uint32_t* blocksums, int n) {
+    __shared__ uint32_t sm[4];
+    const int base = blockIdx.x * SCAN_BLOCK_ITEMS;
+    uint32_t s = 0;
+    for (int k = threadIdx.x; k < SCAN_BLOCK_ITEMS; k += 256)
+        if (base + k < n) s += spine[base + k];
+    uint32_t tot;
+    block_excl_scan(s, sm, &tot);
+    if (threadIdx.x == 0) blocksums[blockIdx.x] = tot;
+}
+__global__ __launch_bounds__(256) void k_spine_top(uint32_t* blocksums, int nb) {
+    __shared__ uint32_t sm[4];
+    uint32_t carry = 0;
+    for (int base = 0; base < nb; base += 256) {
+        const int i = base + threadIdx.x;
+        const uint32_t v = (i < nb) ? blocksums[i] : 0u;
+        uint32_t tot;
+        const uint32_t ex = block_excl_scan(v, sm, &tot);
+        if (i < nb) blocksums[i] = carry + ex;
+        carry += tot;
+    }
+}
+__global__ __launch_bounds__(256) void k_spine_down(uint32_t* spine, const uint32_t* __restrict__ blocksums, int n) {
+    __shared__ uint32_t sm[4];
+    constexpr int PER = SCAN_BLOCK_ITEMS / 256;
+    const int base = blockIdx.x * SCAN_BLOCK_ITEMS + threadIdx.x * PER;
+    uint32_t v[PER], s = 0;
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+        v[k] = (base + k < n) ? spine[base + k] : 0u;
+        s += v[k];
+    }
+    uint32_t tot;
+    uint32_t run = blocksums[blockIdx.x] + block_excl_scan(s, sm, &tot);
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+        if (base + k < n) spine[base + k] = run;
+        run += v[k];
+    }
+}
+
+// ---- stable scatter ---------------------------------------------------------------
+__global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int shift) {
+    __shared__ uint32_t cnt[WAVES][256];     // running digit counts of each wave; later: destinations
+    const TileRef tr = tile_ref(pl, blockIdx.x);
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int k = threadIdx.x; k < WAVES * 256; k += SORT_THREADS) (&cnt[0][0])[k] = 0;
+    __syncthreads();
+
+    const uint32_t* __restrict__ keys = pl.keys[src] + tr.base;
+    const int32_t* __restrict__ vals = pl.vals[src] + tr.base;
+    const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+
+    uint32_t key[ITEMS], rank[ITEMS];
+    int32_t val[ITEMS];
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int i = w * WAVE_ITEMS + r * 64 + lane;
+        const bool ok = i < tr.cnt;
+        key[r] = ok ? keys[i] : 0u;
+        val[r] = ok ? vals[i] : 0;
+    }
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int i = w * WAVE_ITEMS + r * 64 + lane;
+        const bool ok = i < tr.cnt;
+        const uint32_t d = (key[r] >> shift) & 255u;
+        uint64_t m = __ballot(ok);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t bal = __ballot(ok && bit);
+            m &= bit ? bal : ~bal;
+        }
+        if (ok) {
+            const uint32_t before = __popcll(m & lt);
+            const uint32_t prev = cnt[w][d];
+            rank[r] = prev + before;
+            if (before == 0) cnt[w][d] = prev + (uint32_t)__popcll(m);
+        }
+    }
+    __syncthreads();
+    {   // digit d = threadIdx.x: turn per-wave counts into per-wave destinations
+        const int d = threadIdx.x;
+        uint32_t run = pl.spine[tr.spine0 + d * tr.stride];
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) {
+            const uint32_t c = cnt[k][d];
+            cnt[k][d] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    uint32_t* __restrict__ kout = pl.keys[src ^ 1];
+    int32_t* __restrict__ vout = pl.vals[src ^ 1];
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int i = w * WAVE_ITEMS + r * 64 + lane;
+        if (i < tr.cnt) {
+            const uint32_t dst = cnt[w][(key[r] >> shift) & 255u] + rank[r];
+            kout[dst] = key[r];
+            vout[dst] = val[r];
+        }
+    }
+}
+
+}  // namespace
+
+int launch_sort(const Plan& pl, hipStream_t st) {
+    if (pl.total == 0) return 0;
+    hipLaunchKernelGGL(k_keys, dim3(pl.elem_tiles), dim3(256), 0, st, pl);
+    SG_LAUNCH_CHECK("k_keys");
+    const int n = 256 * pl.sort_tiles;
+    const int nb = (n + SCAN_BLOCK_ITEMS - 1) / SCAN_BLOCK_ITEMS;
+    for (int pass = 0; pass < 4; pass++) {
+        const int src = pass & 1, shift = 8 * pass;
+        hipLaunchKernelGGL(k_hist, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
+        hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
+        hipLaunchKernelGGL(k_spine_top, dim3(1), dim3(256), 0, st, pl.blocksums, nb);
+        hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
+        hipLaunchKernelGGL(k_scatter, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
+        SG_LAUNCH_CHECK("radix pass");
+    }
+    return 0;   // result is back in keys[0] / vals[0]
+}
+
+}  // namespace sg2

@@ -1,0 +1,186 @@
+// C-ABI entry points of the SuperGrok v2 batched step: validation, workspace
+// carving, the small per-call table upload and the launch sequence
+//   keys -> 4 radix passes -> chunk summaries -> chunk prefix -> scan output
+//   -> per-element GRU/PEER/expert/Adam.
+// Stands behind supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877 of
+// the reference) in place of launch_mamba3_peer_batched_step
+// (csrc/supergrok2_mamba_peer_kernels.cu:1754-2117).
+#include <vector>
+
+#include "sg2_internal.hpp"
+
+namespace sg2 {
+namespace {
+
+int g_chunk_len = 1024;
+
+struct Layout {
+    int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
+    size_t off_tables, off_keys[2], off_vals[2], off_spine, off_blocksums, off_summ, off_hstart, off_ctx, bytes;
+    size_t tables_bytes;
+};
+
+int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
+    int64_t total = 0, et = 0, stl = 0, ch = 0, wch = 0;
+    for (int i = 0; i < P; i++) {
+        const int64_t n = numels[i];
+        if (n < 0) return sg::fail("tensor %d: negative numel", i);
+        if (n > 0x7fffffff) return sg::fail("tensor %d: numel %lld exceeds 2^31-1", i, (long long)n);
+        total += n;
+        et += (n + ELEM_TILE - 1) / ELEM_TILE;
+        stl += (n + SORT_TILE - 1) / SORT_TILE;
+        const int64_t nc = (n + chunk_len - 1) / chunk_len;
+        ch += nc;
+        wch += nc > 0 ? nc - 1 : 0;
+    }
+    if (total > 0x7ffffff0) return sg::fail("total element count %lld exceeds the 2^31 indexing limit", (long long)total);
+    L->P = P; L->total = (int)total; L->elem_tiles = (int)et; L->sort_tiles = (int)stl;
+    L->chunks = (int)ch; L->wchunks = (int)wch;
+    L->nb = (int)((256 * stl + SCAN_BLOCK_ITEMS - 1) / SCAN_BLOCK_ITEMS);
+    size_t o = 0;
+    auto take = [&](size_t bytes) { size_t r = o; o = sg::align_up(o + bytes, 256); return r; };
+    L->tables_bytes = sizeof(TensorDev) * (size_t)P + 4 * sizeof(int) * (size_t)(P + 1);
+    L->off_tables = take(L->tables_bytes);
+    for (int k = 0; k < 2; k++) L->off_keys[k] = take(4 * (size_t)total);
+    for (int k = 0; k < 2; k++) L->off_vals[k] = take(4 * (size_t)total);
+    L->off_spine = take(4 * 256 * (size_t)stl);
+    L->off_blocksums = take(4 * (size_t)(L->nb + 1));
+    L->off_summ = take(4 * 2 * (size_t)wch * 6 * SCAN_THREADS);
+    L->off_hstart = take(4 * 2 * (size_t)ch * 2 * SCAN_THREADS);
+    L->off_ctx = take(4 * 2 * (size_t)total * DM);
+    L->bytes = o;
+    return 0;
+}
+
+int check_dims(const SgDims* d) {
+    if (!d) return sg::fail("dims is NULL");
+    // the limits the reference enforces (csrc/supergrok2_mamba_peer_kernels.cu:1796-1801)
+    if (d->d_state % 2) return sg::fail("d_state must be even for paired RoPE (got %d)", d->d_state);
+    if (d->d_state > 32) return sg::fail("d_state exceeds MAX_D_STATE (%d > 32)", d->d_state);
+    if (d->d_model > 16) return sg::fail("d_model exceeds MAX_D_MODEL (%d > 16)", d->d_model);
+    if (d->gru_hidden > 8) return sg::fail("gru_hidden exceeds MAX_GRU_HIDDEN (%d > 8)", d->gru_hidden);
+    if (d->d_inner > 32) return sg::fail("d_inner exceeds MAX_D_INNER (%d > 32)", d->d_inner);
+    if (d->d_inner % 4) return sg::fail("d_inner must be a multiple of 4 (got %d)", d->d_inner);
+    // the specialisation these kernels are compiled for
+    if (d->d_model != DM || d->d_state != DS || d->d_inner != DI || d->gru_hidden != GH || d->num_heads != NH ||
+        d->pk_dim != PK || d->expert_hidden != EH || d->num_experts != NE)
+        return sg::fail("unsupported meta-net dims: kernels are built for d_model=%d d_state=%d d_inner=%d "
+                        "gru_hidden=%d heads=%d pk_dim=%d expert_hidden=%d experts=%d",
+                        DM, DS, DI, GH, NH, PK, EH, NE);
+    return 0;
+}
+
+}  // namespace
+}  // namespace sg2
+
+extern "C" {
+
+const char* sg_last_error(void) { return sg::last_error().c_str(); }
+
+int sg2_set_chunk_len(int chunk_len) {
+    if (chunk_len == 0) chunk_len = 1024;
+    if (chunk_len < sg2::SCAN_TT || chunk_len % sg2::SCAN_TT) return sg::fail("chunk_len must be a positive multiple of %d", sg2::SCAN_TT);
+    sg2::g_chunk_len = chunk_len;
+    return 0;
+}
+int sg2_get_chunk_len(void) { return sg2::g_chunk_len; }
+
+size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
+    if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
+    sg2::Layout L;
+    if (sg2::make_layout(num_tensors, numels, sg2::g_chunk_len, &L)) return 0;
+    return L.bytes;
+}
+
+int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                     const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
+                     const Sg2Debug* debug, void* stream) {
+    using namespace sg2;
+    if (check_dims(dims)) return 1;
+    if (num_tensors == 0) return 0;
+    if (num_tensors < 0 || !tensors || !weights || !scalars) return sg::fail("NULL argument");
+    for (int k = 0; k < SG2_NUM_WEIGHTS; k++)
+        if (!weights->w[k]) return sg::fail("weight pointer %d is NULL", k);
+    hipStream_t st = (hipStream_t)stream;
+    const int P = num_tensors;
+
+    std::vector<int64_t> numels(P);
+    for (int i = 0; i < P; i++) {
+        const Sg2Tensor& t = tensors[i];
+        numels[i] = t.numel;
+        if (t.numel > 0) {
+            if (!t.param || !t.grad || !t.sharpness || !t.exp_avg || !t.exp_avg_sq || !t.mu || !t.gru_state ||
+                !t.mamba_fwd_state || !t.mamba_bwd_state)
+                return sg::fail("tensor %d: NULL pointer", i);
+            if (t.dtype != SG_F32 && t.dtype != SG_F16 && t.dtype != SG_BF16) return sg::fail("tensor %d: bad dtype %d", i, t.dtype);
+            if (((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
+        }
+    }
+    Layout L;
+    if (make_layout(P, numels.data(), g_chunk_len, &L)) return 1;
+    if (L.total == 0) return 0;
+    if (!workspace || workspace_bytes < L.bytes)
+        return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
+    if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
+
+    // ---- host tables -> one blob -> device
+    std::vector<unsigned char> blob(L.tables_bytes);
+    TensorDev* td = reinterpret_cast<TensorDev*>(blob.data());
+    int* pre = reinterpret_cast<int*>(blob.data() + sizeof(TensorDev) * (size_t)P);
+    int *p_et = pre, *p_st = pre + (P + 1), *p_ch = pre + 2 * (P + 1), *p_wc = pre + 3 * (P + 1);
+    p_et[0] = p_st[0] = p_ch[0] = p_wc[0] = 0;
+    int off = 0;
+    for (int i = 0; i < P; i++) {
+        const Sg2Tensor& t = tensors[i];
+        const int n = (int)t.numel;
+        const int nc = (n + g_chunk_len - 1) / g_chunk_len;
+        TensorDev& d = td[i];
+        d.param = t.param; d.grad = t.grad; d.sharp = t.sharpness;
+        d.ea = t.exp_avg; d.easq = t.exp_avg_sq; d.mu = t.mu; d.gru = t.gru_state;
+        d.mfwd = t.mamba_fwd_state; d.mbwd = t.mamba_bwd_state;
+        d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
+        d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
+        d.step_size = scalars->lr / t.bc1;
+        for (int k = 0; k < 5; k++) d.pad_[k] = 0;
+        off += n;
+        p_et[i + 1] = p_et[i] + (n + ELEM_TILE - 1) / ELEM_TILE;
+        p_st[i + 1] = p_st[i] + (n + SORT_TILE - 1) / SORT_TILE;
+        p_ch[i + 1] = p_ch[i] + nc;
+        p_wc[i + 1] = p_wc[i] + (nc > 0 ? nc - 1 : 0);
+    }
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_tables, blob.data(), L.tables_bytes, hipMemcpyHostToDevice, st));
+
+    Plan pl;
+    pl.tensors = reinterpret_cast<const TensorDev*>(ws + L.off_tables);
+    const int* dpre = reinterpret_cast<const int*>(ws + L.off_tables + sizeof(TensorDev) * (size_t)P);
+    pl.elem_tile_prefix = dpre;
+    pl.sort_tile_prefix = dpre + (P + 1);
+    pl.chunk_prefix = dpre + 2 * (P + 1);
+    pl.wchunk_prefix = dpre + 3 * (P + 1);
+    pl.P = P; pl.total = L.total; pl.elem_tiles = L.elem_tiles; pl.sort_tiles = L.sort_tiles;
+    pl.chunks = L.chunks; pl.wchunks = L.wchunks; pl.chunk_len = g_chunk_len;
+    for (int k = 0; k < 2; k++) {
+        pl.keys[k] = reinterpret_cast<uint32_t*>(ws + L.off_keys[k]);
+        pl.vals[k] = reinterpret_cast<int32_t*>(ws + L.off_vals[k]);
+    }
+    pl.spine = reinterpret_cast<uint32_t*>(ws + L.off_spine);
+    pl.blocksums = reinterpret_cast<uint32_t*>(ws + L.off_blocksums);
+    pl.summaries = reinterpret_cast<float*>(ws + L.off_summ);
+    pl.hstart = reinterpret_cast<float*>(ws + L.off_hstart);
+    pl.ctx = reinterpret_cast<float*>(ws + L.off_ctx);
+    pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
+    pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
+    pl.W = *weights;
+
+    if (launch_sort(pl, st)) return 1;
+    if (debug && debug->perm)
+        SG_HIP_CHECK(hipMemcpyAsync(debug->perm, pl.vals[0], 4 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
+    if (launch_scan(pl, st)) return 1;
+    if (debug && debug->ctx)
+        SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * DM, hipMemcpyDeviceToDevice, st));
+    if (launch_elem(pl, expert_counts, debug ? debug->expert_idx : nullptr, st)) return 1;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,74 @@
+// Shared host/device helpers for the gfx950 kernels of libsg_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <string>
+
+#include "../../include/sg_abi.h"
+#include "../../include/sg_math.h"
+
+namespace sg {
+
+// ---- error text of the calling thread -------------------------------------
+inline std::string& last_error() {
+    static thread_local std::string e;
+    return e;
+}
+inline int fail(const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return 1;
+}
+#define SG_HIP_CHECK(expr)                                                              \
+    do {                                                                                \
+        hipError_t e_ = (expr);                                                         \
+        if (e_ != hipSuccess) return sg::fail("%s: %s", #expr, hipGetErrorString(e_));  \
+    } while (0)
+#define SG_LAUNCH_CHECK(name)                                                           \
+    do {                                                                                \
+        hipError_t e_ = hipGetLastError();                                              \
+        if (e_ != hipSuccess) return sg::fail("launch %s: %s", name, hipGetErrorString(e_)); \
+    } while (0)
+
+// ---- element load/store with the tensor's storage type ---------------------
+__device__ __forceinline__ float bf16_bits_to_f(uint16_t h) { return sg_i2f((int32_t)((uint32_t)h << 16)); }
+__device__ __forceinline__ uint16_t f_to_bf16_bits(float f) {
+    uint32_t u = (uint32_t)sg_f2i(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float load_elem(const void* p, int dtype, int64_t i) {
+    if (dtype == SG_F32) return ((const float*)p)[i];
+    if (dtype == SG_F16) return __half2float(((const __half*)p)[i]);
+    return bf16_bits_to_f(((const uint16_t*)p)[i]);
+}
+__device__ __forceinline__ void store_elem(void* p, int dtype, int64_t i, float v) {
+    if (dtype == SG_F32) ((float*)p)[i] = v;
+    else if (dtype == SG_F16) ((__half*)p)[i] = __float2half_rn(v);
+    else ((uint16_t*)p)[i] = f_to_bf16_bits(v);
+}
+__device__ __forceinline__ float finite_or_zero(float v) { return sg_isfinite(v) ? v : 0.0f; }
+
+// largest i in [0, n) with prefix[i] <= x   (prefix is non-decreasing, prefix[0] == 0)
+__device__ __forceinline__ int upper_seg(const int* __restrict__ prefix, int n, int x) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (prefix[mid] <= x) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace sg

@@ -1,0 +1,139 @@
+"""ctypes view of libsg_hip.so (the C ABI declared in include/sg_abi.h).
+
+The torch extension `_ops` is the production caller of the library; this
+module binds the same entry points directly so that the parity tests and the
+benchmark can drive the C ABI with device pointers taken from torch tensors,
+and read the inspection outputs (sort permutation, expert indices, contexts).
+There is no fallback: if the library is missing, loading raises.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libsg_hip.so")
+
+SG_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+DIM_NAMES = ("d_model", "d_state", "d_inner", "gru_hidden", "num_heads", "pk_dim", "expert_hidden",
+             "num_experts")
+DEFAULT_DIMS = dict(d_model=8, d_state=16, d_inner=16, gru_hidden=4, num_heads=4, pk_dim=12,
+                    expert_hidden=16, num_experts=144)
+
+
+class SgDims(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in DIM_NAMES]
+
+
+class Sg2Weights(C.Structure):
+    _fields_ = [("w", C.c_void_p * 33)]
+
+
+class Sg2Tensor(C.Structure):
+    _fields_ = [("param", C.c_void_p), ("grad", C.c_void_p), ("sharpness", C.c_void_p),
+                ("exp_avg", C.c_void_p), ("exp_avg_sq", C.c_void_p), ("mu", C.c_void_p),
+                ("gru_state", C.c_void_p), ("mamba_fwd_state", C.c_void_p), ("mamba_bwd_state", C.c_void_p),
+                ("numel", C.c_int64), ("dtype", C.c_int32),
+                ("alpha_mu", C.c_float), ("lamb_eff", C.c_float), ("beta1", C.c_float),
+                ("bc1", C.c_float), ("bc2", C.c_float)]
+
+
+class Sg2Scalars(C.Structure):
+    _fields_ = [("rescale", C.c_float), ("beta2", C.c_float), ("lr", C.c_float), ("wd_eff", C.c_float),
+                ("eps", C.c_float)]
+
+
+class Sg2Debug(C.Structure):
+    _fields_ = [("perm", C.c_void_p), ("expert_idx", C.c_void_p), ("ctx", C.c_void_p)]
+
+
+EXPORTS = ("sg_last_error", "sg2_set_chunk_len", "sg2_get_chunk_len", "sg2_workspace_bytes", "sg2_batched_step")
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libsg_hip.so is not built (%s); run __graft_entry__.build()" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        L.sg_last_error.restype = C.c_char_p
+        L.sg2_set_chunk_len.argtypes = [C.c_int]
+        L.sg2_workspace_bytes.restype = C.c_size_t
+        L.sg2_workspace_bytes.argtypes = [C.POINTER(SgDims), C.c_int, C.POINTER(C.c_int64)]
+        L.sg2_batched_step.restype = C.c_int
+        L.sg2_batched_step.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
+                                       C.POINTER(Sg2Scalars), C.c_void_p, C.c_void_p, C.c_size_t,
+                                       C.POINTER(Sg2Debug), C.c_void_p]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().sg_last_error().decode()
+
+
+def make_dims(dims=None):
+    d = dict(DEFAULT_DIMS if dims is None else dims)
+    return SgDims(*[d[n] for n in DIM_NAMES])
+
+
+def workspace_bytes(numels, dims=None):
+    arr = (C.c_int64 * len(numels))(*numels)
+    d = make_dims(dims)
+    n = lib().sg2_workspace_bytes(C.byref(d), len(numels), arr)
+    if n == 0 and sum(numels) > 0:
+        raise RuntimeError(last_error())
+    return n
+
+
+class Sg2Step:
+    """Reusable call plan for sg2_batched_step on a fixed list of tensors."""
+
+    def __init__(self, weights, params, exp_avgs, exp_avg_sqs, mus, gru_states, mamba_fwd, mamba_bwd,
+                 expert_counts, dims=None, debug=False):
+        self.dims = make_dims(dims)
+        self.weights = [w.contiguous() for w in weights]
+        assert len(self.weights) == 33 and all(w.dtype == torch.float32 and w.is_cuda for w in self.weights)
+        self.W = Sg2Weights()
+        for k, w in enumerate(self.weights):
+            self.W.w[k] = w.data_ptr()
+        self.state = (params, exp_avgs, exp_avg_sqs, mus, gru_states, mamba_fwd, mamba_bwd)
+        self.P = len(params)
+        self.numels = [p.numel() for p in params]
+        self.total = sum(self.numels)
+        self.expert_counts = expert_counts
+        self.ws_bytes = workspace_bytes(self.numels, dims)
+        dev = params[0].device
+        self.workspace = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
+        self.tensors = (Sg2Tensor * self.P)()
+        self.debug = None
+        if debug:
+            H, dm = self.dims.num_heads, self.dims.d_model
+            self.perm = torch.empty(self.total, dtype=torch.int32, device=dev)
+            self.expert_idx = torch.empty(self.total, H, dtype=torch.int32, device=dev)
+            self.ctx = torch.empty(2, self.total, dm, dtype=torch.float32, device=dev)
+            self.debug = Sg2Debug(self.perm.data_ptr(), self.expert_idx.data_ptr(), self.ctx.data_ptr())
+
+    def __call__(self, grads, sharps, per_tensor, shared):
+        """per_tensor: list of dicts(alpha, lamb_eff, beta1, bc1, bc2); shared: dict(rescale, beta2, lr, wd_eff, eps)."""
+        params, eas, easqs, mus, grus, mf, mb = self.state
+        for i in range(self.P):
+            t = self.tensors[i]
+            p, g, s = params[i], grads[i], sharps[i]
+            assert g.dtype == p.dtype and s.dtype == p.dtype and g.is_contiguous() and s.is_contiguous()
+            t.param, t.grad, t.sharpness = p.data_ptr(), g.data_ptr(), s.data_ptr()
+            t.exp_avg, t.exp_avg_sq, t.mu = eas[i].data_ptr(), easqs[i].data_ptr(), mus[i].data_ptr()
+            t.gru_state, t.mamba_fwd_state, t.mamba_bwd_state = grus[i].data_ptr(), mf[i].data_ptr(), mb[i].data_ptr()
+            t.numel, t.dtype = p.numel(), SG_DTYPE[p.dtype]
+            sc = per_tensor[i]
+            t.alpha_mu, t.lamb_eff, t.beta1, t.bc1, t.bc2 = sc["alpha"], sc["lamb_eff"], sc["beta1"], sc["bc1"], sc["bc2"]
+        S = Sg2Scalars(shared["rescale"], shared["beta2"], shared["lr"], shared["wd_eff"], shared["eps"])
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = lib().sg2_batched_step(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, C.byref(S),
+                                    self.expert_counts.data_ptr() if self.expert_counts is not None else None,
+                                    self.workspace.data_ptr(), self.workspace.numel(),
+                                    C.byref(self.debug) if self.debug is not None else None, stream)
+        if rc != 0:
+            raise RuntimeError("sg2_batched_step: " + last_error())

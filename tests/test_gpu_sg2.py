@@ -1,0 +1,122 @@
+"""Parity of the SuperGrok v2 batched step (HIP, through the C ABI of
+libsg_hip.so) with the CPU checker on identical seeded inputs.
+
+Gates: sort permutation, PEER expert indices and expert_counts bit-exact;
+param / exp_avg / exp_avg_sq / mu / gru_state / Mamba carries within
+|a-b| <= 1e-4*max(|a|,|b|) + 1e-7 after every step (fp32)."""
+import numpy as np
+import pytest
+import torch
+
+import workloads as wl
+from helpers import DIMS
+from sg2_harness import Sg2Case, per_tensor_scalars, shared_scalars
+
+pytestmark = pytest.mark.gpu
+
+REL, FLOOR = 1e-4, 1e-7
+
+
+@pytest.fixture(autouse=True)
+def _default_chunk():
+    from grokking_optimizers import _cabi
+    _cabi.lib().sg2_set_chunk_len(0)
+    yield
+    _cabi.lib().sg2_set_chunk_len(0)
+
+
+def _run_steps(case, steps, chunk_len, grad_seed0=1, lamb_eff=0.0, wd_eff=1.0, grad_std=1e-3, sharp=False,
+               tail_frac=0.0):
+    worst = {}
+    for t in range(1, steps + 1):
+        grads = wl.make_grads(case.shapes, seed=grad_seed0 + t, std=grad_std, tail_frac=tail_frac, tail="student3")
+        sharps = ([g.abs() * 0.5 for g in wl.make_grads(case.shapes, seed=500 + t)] if sharp
+                  else [torch.zeros_like(g) for g in grads])
+        pt, sh = per_tensor_scalars(case.P, t, lamb_eff), shared_scalars(wd_eff)
+        print("step", t, "shapes", len(case.shapes), "chunk", chunk_len, flush=True)
+        case.gpu_step(grads, sharps, pt, sh)
+        dbg = case.oracle_step(grads, sharps, pt, sh, chunk_len)
+        w = case.compare(dbg, REL, FLOOR)
+        for k, v in w.items():
+            worst[k] = max(worst.get(k, 0.0), v)
+    return worst
+
+
+def test_small_tensors_single_chunk():
+    """All tensors below 256 elements (the reference's sequential-scan regime), 3 steps."""
+    case = Sg2Case(wl.small8_shapes(), seed=3)
+    w = _run_steps(case, 3, chunk_len=1024, sharp=True, lamb_eff=2.0, wd_eff=4.5)
+    print("worst tolerance ratios", w)
+
+
+def test_multi_chunk_small_chunks():
+    """Chunk length 64/256 on mid-size tensors exercises summaries + chunk prefix."""
+    from grokking_optimizers import _cabi
+    shapes = [(1000,), (64, 65), (257,), (3, 4096), (64,), (5000,)]
+    for cl in (64, 256):
+        assert _cabi.lib().sg2_set_chunk_len(cl) == 0
+        case = Sg2Case(shapes, seed=cl, random_state=True)
+        w = _run_steps(case, 3, chunk_len=cl, sharp=True, lamb_eff=2.0, wd_eff=4.5)
+        print("chunk", cl, "worst tolerance ratios", w)
+
+
+def test_shared14_one_step_default_chunk():
+    """The 14-tensor, 420 195-element transformer parameter set, default chunk length."""
+    case = Sg2Case(wl.shared14_shapes(), seed=0)
+    w = _run_steps(case, 2, chunk_len=1024)
+    print("worst tolerance ratios", w)
+    assert int(case.counts_gpu.sum()) == 2 * 4 * 420195
+
+
+def test_edge_cases():
+    """Empty tensor, N=1, all-zero grads, huge grads, NaN/Inf grads, fp16 and bf16 parameters."""
+    shapes = [(0,), (1,), (300,), (300,), (300,), (1500,), (1500,)]
+    dtypes = [torch.float32] * 5 + [torch.float16, torch.bfloat16]
+    case = Sg2Case(shapes, dtypes=dtypes, seed=5, random_state=True)
+    for t in range(1, 3):
+        grads = wl.make_grads(shapes, seed=40 + t)
+        grads[2].zero_()
+        grads[3].fill_(1e6)
+        grads[4][::17] = float("nan")
+        grads[4][5::31] = float("inf")
+        grads[4][7::29] = float("-inf")
+        sharps = [g.abs() for g in wl.make_grads(shapes, seed=60 + t)]
+        pt, sh = per_tensor_scalars(case.P, t, 2.0), shared_scalars(4.5)
+        print("edge step", t, flush=True)
+        case.gpu_step(grads, sharps, pt, sh)
+        dbg = case.oracle_step(grads, sharps, pt, sh, 1024)
+        case.compare(dbg, REL, FLOOR)
+    for st in case.gpu:
+        for k, v in st.items():
+            assert torch.isfinite(v.float()).all(), k
+
+
+def test_heavy_ties_sort_is_stable():
+    """Quantised gradients: thousands of exact ties; permutation must equal the stable argsort."""
+    shapes = [(20000,), (9000,)]
+    case = Sg2Case(shapes, seed=9)
+    grads = [torch.round(g * 2e4) / 2e4 for g in wl.make_grads(shapes, seed=77, std=1e-3)]
+    sharps = [torch.zeros_like(g) for g in grads]
+    pt, sh = per_tensor_scalars(case.P, 1), shared_scalars()
+    case.gpu_step(grads, sharps, pt, sh)
+    perm = case.step_fn.perm.cpu().numpy()
+    for i, g in enumerate(grads):
+        a, b = int(case.offsets[i]), int(case.offsets[i + 1])
+        want = np.argsort(np.abs(g.numpy()), kind="stable").astype(np.int32)
+        assert np.array_equal(perm[a:b], want)
+
+
+def test_rejects_unsupported_dims_and_small_workspace():
+    from grokking_optimizers import _cabi
+    import ctypes as C
+    d = dict(DIMS, d_state=15)
+    with pytest.raises(RuntimeError, match="d_state must be even"):
+        _cabi.workspace_bytes([10], d)
+    d = dict(DIMS, d_model=4)
+    with pytest.raises(RuntimeError, match="unsupported meta-net dims"):
+        _cabi.workspace_bytes([10], d)
+    case = Sg2Case([(100,)], seed=1)
+    case.step_fn.workspace = torch.empty(256, dtype=torch.uint8, device="cuda")
+    g = [torch.zeros(100)]
+    with pytest.raises(RuntimeError, match="workspace too small"):
+        case.gpu_step(g, g, per_tensor_scalars(1, 1), shared_scalars())
