@@ -99,6 +99,19 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
                      const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
                      void* workspace, size_t workspace_bytes, const Sg2Debug* debug, void* stream);
 
+/* Per-stage device timing of sg2_batched_step with HIP events recorded on the
+ * step's own stream (no counterpart in the reference, which has no profiling
+ * hooks).  Stages: 0 key generation + radix sort, 1 scan chunk summaries,
+ * 2 chunk prefix, 3 scan output, 4 per-element kernel.
+ * sg2_profile_enable(1) starts collecting (at most SG2_PROF_MAX_CALLS calls are
+ * kept), sg2_profile_read waits for the recorded events, adds each stage's
+ * elapsed milliseconds over the collected calls into ms[SG2_PROF_STAGES],
+ * stores the number of calls and clears the collection. */
+#define SG2_PROF_STAGES 5
+#define SG2_PROF_MAX_CALLS 256
+int sg2_profile_enable(int on);
+int sg2_profile_read(float* ms, int* calls);
+
 #ifdef __cplusplus
 }
 #endif

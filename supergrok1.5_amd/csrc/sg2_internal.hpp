@@ -78,6 +78,9 @@ struct Plan {
     Sg2Weights W;
 };
 
+// records a profiling event (no-op unless profiling is enabled)
+void prof_mark(int idx, hipStream_t st);
+
 int launch_sort(const Plan& pl, hipStream_t st);
 int launch_scan(const Plan& pl, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);

@@ -285,10 +285,13 @@ int launch_scan(const Plan& pl, hipStream_t st) {
         hipLaunchKernelGGL(k_scan<false>, dim3(2 * pl.wchunks), dim3(SCAN_THREADS), 0, st, pl);
         SG_LAUNCH_CHECK("k_scan<summary>");
     }
+    prof_mark(2, st);
     hipLaunchKernelGGL(k_chunk_prefix, dim3(2 * pl.P), dim3(SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_chunk_prefix");
+    prof_mark(3, st);
     hipLaunchKernelGGL(k_scan<true>, dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_scan<out>");
+    prof_mark(4, st);
     return 0;
 }
 

@@ -14,6 +14,14 @@ namespace {
 
 int g_chunk_len = 1024;
 
+// ---- optional per-stage timing with HIP events on the step's stream
+constexpr int PROF_MARKS = SG2_PROF_STAGES + 1;
+struct Prof {
+    bool on = false;
+    int calls = 0;
+    std::vector<hipEvent_t> ev;     // [SG2_PROF_MAX_CALLS][PROF_MARKS], created on first enable
+} g_prof;
+
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
     size_t off_tables, off_keys[2], off_vals[2], off_spine, off_blocksums, off_summ, off_hstart, off_ctx, bytes;
@@ -71,9 +79,43 @@ int check_dims(const SgDims* d) {
 }
 
 }  // namespace
+
+void prof_mark(int idx, hipStream_t st) {
+    if (!g_prof.on || g_prof.calls >= SG2_PROF_MAX_CALLS) return;
+    (void)hipEventRecord(g_prof.ev[(size_t)g_prof.calls * PROF_MARKS + idx], st);
+}
 }  // namespace sg2
 
 extern "C" {
+
+int sg2_profile_enable(int on) {
+    using namespace sg2;
+    if (on && g_prof.ev.empty()) {
+        g_prof.ev.resize((size_t)SG2_PROF_MAX_CALLS * PROF_MARKS);
+        for (auto& e : g_prof.ev) SG_HIP_CHECK(hipEventCreate(&e));
+    }
+    g_prof.on = on != 0;
+    g_prof.calls = 0;
+    return 0;
+}
+
+int sg2_profile_read(float* ms, int* calls) {
+    using namespace sg2;
+    if (!ms || !calls) return sg::fail("NULL argument");
+    for (int k = 0; k < SG2_PROF_STAGES; k++) ms[k] = 0.0f;
+    *calls = g_prof.calls;
+    for (int c = 0; c < g_prof.calls; c++) {
+        hipEvent_t* e = &g_prof.ev[(size_t)c * PROF_MARKS];
+        SG_HIP_CHECK(hipEventSynchronize(e[PROF_MARKS - 1]));
+        for (int k = 0; k < SG2_PROF_STAGES; k++) {
+            float t = 0.0f;
+            SG_HIP_CHECK(hipEventElapsedTime(&t, e[k], e[k + 1]));
+            ms[k] += t;
+        }
+    }
+    g_prof.calls = 0;
+    return 0;
+}
 
 const char* sg_last_error(void) { return sg::last_error().c_str(); }
 
@@ -173,13 +215,17 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
     pl.W = *weights;
 
+    prof_mark(0, st);
     if (launch_sort(pl, st)) return 1;
+    prof_mark(1, st);
     if (debug && debug->perm)
         SG_HIP_CHECK(hipMemcpyAsync(debug->perm, pl.vals[0], 4 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
     if (launch_scan(pl, st)) return 1;
     if (debug && debug->ctx)
         SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * DM, hipMemcpyDeviceToDevice, st));
     if (launch_elem(pl, expert_counts, debug ? debug->expert_idx : nullptr, st)) return 1;
+    prof_mark(5, st);
+    if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;
     return 0;
 }
 

@@ -47,7 +47,9 @@ class Sg2Debug(C.Structure):
     _fields_ = [("perm", C.c_void_p), ("expert_idx", C.c_void_p), ("ctx", C.c_void_p)]
 
 
-EXPORTS = ("sg_last_error", "sg2_set_chunk_len", "sg2_get_chunk_len", "sg2_workspace_bytes", "sg2_batched_step")
+EXPORTS = ("sg_last_error", "sg2_set_chunk_len", "sg2_get_chunk_len", "sg2_workspace_bytes", "sg2_batched_step",
+           "sg2_profile_enable", "sg2_profile_read")
+SG2_PROF_STAGES = ("sort", "scan_summary", "chunk_prefix", "scan_output", "elementwise")
 
 _lib = None
 
@@ -68,6 +70,20 @@ def lib():
                                        C.POINTER(Sg2Debug), C.c_void_p]
         _lib = L
     return _lib
+
+
+def profile_enable(on=True):
+    if lib().sg2_profile_enable(1 if on else 0) != 0:
+        raise RuntimeError(last_error())
+
+
+def profile_read():
+    """(dict stage -> total ms, number of calls) since profile_enable(True)."""
+    ms = (C.c_float * len(SG2_PROF_STAGES))()
+    calls = C.c_int(0)
+    if lib().sg2_profile_read(ms, C.byref(calls)) != 0:
+        raise RuntimeError(last_error())
+    return {n: float(ms[k]) for k, n in enumerate(SG2_PROF_STAGES)}, calls.value
 
 
 def last_error():
