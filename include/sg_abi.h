@@ -112,6 +112,131 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
 int sg2_profile_enable(int on);
 int sg2_profile_read(float* ms, int* calls);
 
+/* ======================= Grokfast / SuperGrok v1.5 ======================== */
+
+/* Scratch for the elementwise entry points below (tables + reduction
+ * partials) for n tensors with these sizes. */
+size_t sg_elemwise_workspace_bytes(int num_tensors, const int64_t* numels);
+
+/* Grokfast EMA filter + amplification over all tensors in one launch:
+ *   ema = alpha*ema + (1-alpha)*g ;  grad <- g + lamb*ema   (grad overwritten)
+ * Replaces launch_fused_grokfast_ema (csrc/grokfast_kernels.cu:20-60) called
+ * per tensor by grokfast_fused_step (csrc/ops.cpp:514-532). */
+typedef struct SgGrokfastTensor {
+    void* grad;        /* [numel] dtype, overwritten with the amplified gradient */
+    float* ema;        /* [numel] fp32 */
+    int64_t numel;
+    int32_t dtype;
+} SgGrokfastTensor;
+int sg_grokfast_ema(int num_tensors, const SgGrokfastTensor* tensors, float alpha, float lamb,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* The whole Grokfast.step body in one pass: the EMA/amplify above followed by
+ * the AdamW update of adamw_step (grokking_optimizers/_adamw_helper.py:12-22,
+ * called from grokking_optimizers/grokfast.py:124-143): p *= 1-lr*wd first,
+ * bias corrections from the per-tensor step computed in double as Python
+ * does.  grad is still overwritten with the amplified gradient. */
+typedef struct SgGrokfastAdamTensor {
+    void* param;       /* [numel] dtype */
+    void* grad;        /* [numel] dtype */
+    float* ema;        /* [numel] fp32 */
+    float* exp_avg;    /* [numel] fp32 */
+    float* exp_avg_sq; /* [numel] fp32 */
+    int64_t numel;
+    int32_t dtype;
+    int32_t step;      /* already incremented, >= 1 */
+} SgGrokfastAdamTensor;
+int sg_grokfast_adamw_step(int num_tensors, const SgGrokfastAdamTensor* tensors, float alpha, float lamb,
+                           double lr, double beta1, double beta2, double eps, double weight_decay,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* SuperGrok v1.5 full step over all tensors: global-norm gradient clip
+ * (coef = c/(norm+1e-6) when norm > c, gradients rescaled in place) with the
+ * norm reduced on the device, then mu EMA, the 2->H->1 sharpness meta-net,
+ * Adam and progressive weight decay in one pass.  Replaces
+ * clip_grad_norms_device_side (csrc/ops.cpp:23-55) and
+ * launch_fused_supergrok15_full_step (csrc/supergrok15_kernels.cu:323-459)
+ * behind supergrok15_fused_step (csrc/ops.cpp:83-152).
+ * gelu_mode 0: exact erf GELU (the reference's CPU path, csrc/ops.cpp:140);
+ * gelu_mode 1: z/(1+exp(-1.702 z)) (its GPU kernel, supergrok15_kernels.cu:380). */
+typedef struct Sg15Tensor {
+    void* param;            /* [numel] dtype */
+    void* grad;             /* [numel] dtype, rescaled in place when clipping is active */
+    const void* sharpness;  /* [numel] dtype */
+    float* exp_avg;         /* [numel] fp32 */
+    float* exp_avg_sq;      /* [numel] fp32 */
+    float* mu;              /* [numel] fp32 */
+    int64_t numel;
+    int32_t dtype;
+    float alpha, beta1, bc1, bc2;
+} Sg15Tensor;
+typedef struct Sg15Net {
+    const float* W1;        /* [hidden,2] */
+    const float* b1;        /* [hidden]   */
+    const float* W2;        /* [1,hidden] */
+    const float* b2;        /* [1]        */
+    int32_t hidden;         /* <= 256 */
+    float rescale;
+    int32_t gelu_mode;
+} Sg15Net;
+int sg15_fused_step(int num_tensors, const Sg15Tensor* tensors, const Sg15Net* net, float lamb_eff, float beta2,
+                    float lr, float wd_eff, float eps, float grad_clip_norm, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* SAM ascent step p += rho/(||g||+1e-12) * g with the global norm reduced on
+ * the device: replaces compute_sam_grad_norm_device_side + launch_sam_perturb
+ * (csrc/ops.cpp:58-75,154-177; csrc/supergrok15_kernels.cu:151-162).  The
+ * caller clones the parameters beforehand. */
+typedef struct Sg15SamTensor {
+    void* param;
+    const void* grad;
+    int64_t numel;
+    int32_t dtype;
+} Sg15SamTensor;
+int sg15_sam_perturb(int num_tensors, const Sg15SamTensor* tensors, float rho, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/* sharpness = |g_sam - g| ; param <- backup.  Replaces launch_sharpness_restore
+ * (csrc/supergrok15_kernels.cu:170-184, csrc/ops.cpp:179-204). */
+typedef struct Sg15RestoreTensor {
+    void* param;
+    void* sharpness;
+    const void* backup;
+    const void* sam_grad;
+    const void* normal_grad;
+    int64_t numel;
+    int32_t dtype;
+} Sg15RestoreTensor;
+int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ================================ Muon ==================================== */
+
+/* One 2-D parameter of the Muon step: the i-th entries of the vectors of
+ * muon_fused_step (csrc/ops.h:510-514).  buf is the fp32 momentum buffer
+ * (grokking_optimizers/muon.py:145-147). */
+typedef struct SgMuonMatrix {
+    void* param;        /* [rows,cols] dtype, updated in place */
+    const void* grad;   /* [rows,cols] dtype                   */
+    float* buf;         /* [rows,cols] fp32, updated           */
+    int64_t rows, cols;
+    int32_t dtype;
+} SgMuonMatrix;
+
+size_t sg_muon_workspace_bytes(int num_matrices, const SgMuonMatrix* mats);
+
+/* Muon step for all matrices: buf = momentum*buf + g; X = buf/(||buf||_F+1e-7)
+ * with the norm reduced on the device; ns_steps quintic Newton-Schulz
+ * iterations X <- aX + b(XX^T)X + c(XX^T)^2 X with (a,b,c) = (3.4445, -4.7750,
+ * 2.0315); p = (p - 0.2*lr*X) * (1 - lr*wd).  The iterations run as bf16 MFMA
+ * GEMMs with fp32 accumulation, on the Gram matrix of the smaller dimension
+ * (X^T X for tall matrices; the same product re-associated).  Replaces the
+ * body of muon_fused_step (csrc/ops.cpp:663-746: ATen norm + host sync,
+ * three torch::mm per iteration, muon_ns_combine_kernel and
+ * muon_update_kernel, csrc/muon_kernels.cu:37-72). */
+int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, float lr, float wd, int ns_steps,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,6 +27,8 @@
  *   sg_sigmoid   1/(1+expf(-x))   :970-971
  *   sg_silu      z/(1+expf(-z))   :263,559,777
  *   sg_abar_pair trapezoidal A_bar for the even/odd member of a RoPE pair, :228,431-432
+ *   sg_gelu_erf  exact GELU of the CPU path      csrc/ops.cpp:140 (torch::gelu)
+ *   sg_gelu_sigmoid  z/(1+expf(-1.702 z))         csrc/supergrok15_kernels.cu:380
  */
 #ifndef SG_MATH_H_
 #define SG_MATH_H_
@@ -174,5 +176,29 @@ SG_HD float sg_tanh(float x) {
     }
     return y;
 }
+
+/* erfc(x): Chebyshev fit with exponential prefactor (Numerical Recipes
+ * "erfcc"), fractional error below 1.2e-7 for every x. */
+SG_HD float sg_erfc(float x) {
+    const float ax = sg_abs(x);
+    const float t = 1.0f / sg_fma(0.5f, ax, 1.0f);
+    float p = 0.17087277f;
+    p = sg_fma(p, t, -0.82215223f);
+    p = sg_fma(p, t, 1.48851587f);
+    p = sg_fma(p, t, -1.13520398f);
+    p = sg_fma(p, t, 0.27886807f);
+    p = sg_fma(p, t, -0.18628806f);
+    p = sg_fma(p, t, 0.09678418f);
+    p = sg_fma(p, t, 0.37409196f);
+    p = sg_fma(p, t, 1.00002368f);
+    p = sg_fma(p, t, -1.26551223f);
+    const float r = t * sg_exp(sg_fma(-ax, ax, p));
+    return (x >= 0.0f) ? r : 2.0f - r;
+}
+
+/* exact GELU: 0.5 z (1 + erf(z/sqrt2)) = 0.5 z erfc(-z/sqrt2) */
+SG_HD float sg_gelu_erf(float z) { return (0.5f * z) * sg_erfc(z * -0.707106781186547524f); }
+/* the sigmoid approximation of GELU used by the reference's GPU kernel */
+SG_HD float sg_gelu_sigmoid(float z) { return z / (1.0f + sg_exp(-1.702f * z)); }
 
 #endif /* SG_MATH_H_ */

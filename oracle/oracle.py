@@ -32,7 +32,8 @@ def lib():
         if not os.path.exists(_LIB):
             build()
         _lib = C.CDLL(_LIB)
-        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos"):
+        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf",
+                  "gelu_sigmoid"):
             f = getattr(_lib, "orc_" + n)
             f.restype = C.c_float
             f.argtypes = [C.c_float]
@@ -105,3 +106,47 @@ def sg2_step(weights, state, grad, sharp, scalars, dims=None, precision=32, chun
     if rc != 0:
         raise RuntimeError("orc_sg2_step: unsupported dims (status %d)" % rc)
     return out
+
+
+# ------------------------------------------------------------------ Grokfast / SuperGrok v1.5
+def _f32(a):
+    assert a.dtype == np.float32 and a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def grokfast_ema(grad, ema, alpha, lamb):
+    """In place on float32 arrays: ema update, grad <- grad + lamb*ema."""
+    lib().orc_grokfast_ema(_f32(grad), _f32(ema), C.c_int64(grad.size), C.c_float(alpha), C.c_float(lamb))
+
+
+def grokfast_adamw(param, grad, ema, ea, easq, step, alpha, lamb, lr, beta1, beta2, eps, wd):
+    lib().orc_grokfast_adamw(_f32(param), _f32(grad), _f32(ema), _f32(ea), _f32(easq), C.c_int64(param.size),
+                             C.c_int(step), C.c_float(alpha), C.c_float(lamb), C.c_double(lr), C.c_double(beta1),
+                             C.c_double(beta2), C.c_double(eps), C.c_double(wd))
+
+
+def sg15_clip_coef(grads, clip):
+    """(coef, clip_on) of the global-norm clip: coef = clip/(norm+1e-6) when norm > clip."""
+    tot = sum(float(np.sum(g.astype(np.float64) ** 2)) for g in grads)
+    norm = np.float32(np.sqrt(tot))
+    if clip > 0 and norm > np.float32(clip):
+        return float(np.float32(clip) / (norm + np.float32(1e-6))), 1
+    return 1.0, 0
+
+
+def sg15_step(params, grads, sharps, eas, easqs, mus, net, per_tensor, lamb_eff, beta2, lr, wd_eff, eps, clip,
+              gelu_mode=0):
+    """All tensors, in place.  net = (W1[H,2], b1[H], W2[1,H], b2[1], rescale); per_tensor: list of dicts
+    alpha, beta1, bc1, bc2."""
+    coef, on = sg15_clip_coef(grads, clip)
+    W1, b1, W2, b2, rescale = net
+    W1, b1, W2, b2 = [np.ascontiguousarray(w, np.float32) for w in (W1, b1, W2, b2)]
+    f = C.c_float
+    for p, g, s, ea, easq, mu, sc in zip(params, grads, sharps, eas, easqs, mus, per_tensor):
+        if p.size == 0:
+            continue
+        lib().orc_sg15_step(_f32(p), _f32(g), _f32(s), _f32(ea), _f32(easq), _f32(mu), C.c_int64(p.size), _f32(W1),
+                            _f32(b1), _f32(W2), _f32(b2), C.c_int(b1.size), f(rescale), C.c_int(gelu_mode),
+                            f(sc["alpha"]), f(sc["beta1"]), f(sc["bc1"]), f(sc["bc2"]), f(lamb_eff), f(beta2), f(lr),
+                            f(wd_eff), f(eps), f(coef), C.c_int(on))
+    return coef, on

@@ -1,0 +1,403 @@
+// Muon step: momentum, Frobenius normalisation, quintic Newton-Schulz
+// orthogonalisation as bf16 MFMA GEMMs with fp32 accumulation, parameter
+// update.  Replaces the body of muon_fused_step (csrc/ops.cpp:663-746 of the
+// reference: ATen norm + one host sync, three torch::mm per iteration,
+// muon_ns_combine_kernel / muon_update_kernel of csrc/muon_kernels.cu:37-72).
+//
+// Every matrix is worked on in its "wide" orientation Y [m x n] (m = min dim)
+// so the Gram matrix is always the small m x m one:
+//     G = Y Y^T            H = b G + c G G            Y <- a Y + H Y
+// (for a tall parameter X this is X^T X and X (bG + cG^2): the reference's
+// X X^T form re-associated, 6 m^2 n instead of 6 n^2 m flops per iteration).
+// All three products are "NT" GEMMs (both operands K-contiguous) once the
+// transpose Y^T is kept next to Y; it is refreshed by a small LDS transpose
+// kernel after every iteration.  Work buffers are zero-padded to multiples of
+// 128 so the GEMM needs no edge handling (zero rows/columns stay zero through
+// the iteration).
+//
+// GEMM: 128x128 output tile per 256-thread workgroup, 4 waves as 2x2, each
+// wave 64x64 = 2x2 MFMA 32x32x16 bf16 tiles (64 fp32 accumulators per lane),
+// K tiles of 64 staged through double-buffered LDS with 144-byte row stride
+// (conflict-free 16-byte operand fetches), next tile prefetched into registers
+// while the current one is multiplied.  Tile index -> XCD-contiguous order so
+// that the workgroups sharing operand panels share an L2.
+#include <cmath>
+#include <vector>
+
+#include "sg_common.hpp"
+
+namespace sgmu {
+namespace {
+
+typedef uint16_t bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int BT = 128;            // GEMM tile (M and N)
+constexpr int BK = 64;             // GEMM K tile
+constexpr int LDS_ROW = BK + 8;    // bf16 elements per LDS row (144 bytes)
+constexpr int ETILE = 4096;        // elements per tile of the elementwise kernels
+constexpr float NS_A = 3.4445f, NS_B = -4.7750f, NS_C = 2.0315f;
+
+struct Mat {
+    void* param;
+    const void* grad;
+    float* buf;
+    bf16_t *Y, *YT, *G, *H;       // [mp x np], [np x mp], [mp x mp], [mp x mp]
+    int rows, cols, dtype;
+    int m, n, mp, np;              // min / max dim and their padded sizes
+    int wide;                      // rows <= cols
+    int etile0;                    // first elementwise tile of this matrix
+    int pad_;
+};
+
+struct Batch {
+    const Mat* mats;
+    const int* etile_prefix;       // [P+1] elementwise tiles (rows*cols / ETILE)
+    const int* gtile_prefix[3];    // [P+1] GEMM output tiles for the three products
+    const int* ttile_prefix;       // [P+1] 64x64 transpose tiles of Y
+    int P, etiles, gtiles[3], ttiles;
+    double* partials;              // [etiles]
+    float* inv_norm;               // [P]
+};
+
+// ---- momentum + sum of squares ------------------------------------------------
+__device__ __forceinline__ double block_sum(double v, double* sm) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v += __shfl_down(v, d, 64);
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const double r = (sm[0] + sm[1]) + (sm[2] + sm[3]);
+    __syncthreads();
+    return r;
+}
+
+__global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum) {
+    __shared__ double sm[4];
+    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
+    const Mat& M = B.mats[mi];
+    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
+    const int cnt = min(ETILE, M.rows * M.cols - start);
+    float acc = 0.0f;
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int i = start + k;
+        const float b = sg_fma(momentum, M.buf[i], sg::load_elem(M.grad, M.dtype, i));
+        M.buf[i] = b;
+        acc = sg_fma(b, b, acc);
+    }
+    const double tot = block_sum((double)acc, sm);
+    if (threadIdx.x == 0) B.partials[blockIdx.x] = tot;
+}
+
+__global__ __launch_bounds__(256) void k_norm(Batch B) {
+    __shared__ double sm[4];
+    const int mi = blockIdx.x;
+    double acc = 0.0;
+    for (int k = B.etile_prefix[mi] + (int)threadIdx.x; k < B.etile_prefix[mi + 1]; k += 256) acc += B.partials[k];
+    const double tot = block_sum(acc, sm);
+    if (threadIdx.x == 0) B.inv_norm[mi] = 1.0f / ((float)sqrt(tot) + 1e-7f);
+}
+
+// X = buf * inv_norm as bf16, written in the parameter's own orientation into
+// Y (wide) or YT (tall); the other one follows from k_transpose.
+__global__ __launch_bounds__(256) void k_normalize(Batch B) {
+    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
+    const Mat& M = B.mats[mi];
+    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
+    const int cnt = min(ETILE, M.rows * M.cols - start);
+    const float inv = B.inv_norm[mi];
+    bf16_t* dst = M.wide ? M.Y : M.YT;
+    const int ld = M.wide ? M.np : M.mp;
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int i = start + k, r = i / M.cols, c = i - r * M.cols;
+        dst[(size_t)r * ld + c] = sg::f_to_bf16_bits(M.buf[i] * inv);
+    }
+}
+
+// dst[c][r] = src[r][c] over the padded buffers, 64x64 tiles through LDS.
+// to_yt != 0: Y -> YT, else YT -> Y.
+__global__ __launch_bounds__(256) void k_transpose(Batch B, int to_yt, int only_tall, int only_wide) {
+    __shared__ bf16_t t[64][66];
+    const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
+    const Mat& M = B.mats[mi];
+    if ((only_tall && M.wide) || (only_wide && !M.wide)) return;
+    const int R = to_yt ? M.mp : M.np, C = to_yt ? M.np : M.mp;     // source is [R x C]
+    const bf16_t* src = to_yt ? M.Y : M.YT;
+    bf16_t* dst = to_yt ? M.YT : M.Y;
+    const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
+    const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
+    (void)R;
+    for (int k = threadIdx.x; k < 64 * 64; k += 256) {
+        const int r = k >> 6, c = k & 63;
+        t[r][c] = src[(size_t)(tr0 + r) * C + tc0 + c];
+    }
+    __syncthreads();
+    for (int k = threadIdx.x; k < 64 * 64; k += 256) {
+        const int r = k >> 6, c = k & 63;     // output row r (= source column), column c (= source row)
+        dst[(size_t)(tc0 + r) * R + tr0 + c] = t[c][r];
+    }
+}
+
+// ---- NT GEMM  C[M x N] = A[M x K] * B[N x K]^T  with fused epilogues ---------------
+enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
+
+template <int EPI>
+__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
+    __shared__ __attribute__((aligned(16))) bf16_t sA[2][BT * LDS_ROW];
+    __shared__ __attribute__((aligned(16))) bf16_t sB[2][BT * LDS_ROW];
+
+    // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs
+    const int nblk = gridDim.x;
+    int lb = blockIdx.x;
+    if (nblk % 8 == 0) lb = (blockIdx.x % 8) * (nblk / 8) + blockIdx.x / 8;
+    const int* __restrict__ prefix = Bt.gtile_prefix[EPI];
+    const int mi = sg::upper_seg(prefix, Bt.P, lb);
+    const Mat& Mt = Bt.mats[mi];
+    const int tile = lb - prefix[mi];
+
+    const bf16_t *A, *B;
+    bf16_t* C;
+    int K, lda, ldb, ldc, tn_count;
+    if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; tn_count = Mt.mp / BT; }
+    else if (EPI == EPI_POLY) { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; tn_count = Mt.mp / BT; }
+    else { A = Mt.H; B = Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np; tn_count = Mt.np / BT; }
+    const int tm = tile / tn_count, tn = tile % tn_count;
+    A += (size_t)tm * BT * lda;
+    B += (size_t)tn * BT * ldb;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    // global -> register staging: 4 x 16 bytes of A and of B per thread per K tile
+    uint4 ra[4], rb[4];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
+            ra[i] = *reinterpret_cast<const uint4*>(A + (size_t)row * lda + k0 + kc * 8);
+            rb[i] = *reinterpret_cast<const uint4*>(B + (size_t)row * ldb + k0 + kc * 8);
+        }
+    };
+    auto sstore = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
+            *reinterpret_cast<uint4*>(&sA[buf][row * LDS_ROW + kc * 8]) = ra[i];
+            *reinterpret_cast<uint4*>(&sB[buf][row * LDS_ROW + kc * 8]) = rb[i];
+        }
+    };
+
+    gload(0);
+    sstore(0);
+    __syncthreads();
+    const int nk = K / BK;
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) gload((kt + 1) * BK);
+        const bf16_t* a_base = &sA[cur][(wm * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 8];
+        const bf16_t* b_base = &sB[cur][(wn * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 8];
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; kk++) {
+            bf16x8 av[2], bv[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                av[i] = *reinterpret_cast<const bf16x8*>(a_base + i * 32 * LDS_ROW + kk * 16);
+                bv[i] = *reinterpret_cast<const bf16x8*>(b_base + i * 32 * LDS_ROW + kk * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) sstore(cur ^ 1);
+        __syncthreads();
+    }
+
+    // epilogue: accumulator element e of tile (i,j): row = 8*(e/4) + 4*(lane/32) + e%4, col = lane%32
+    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : Mt.Y;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int row = tm * BT + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                const int col = tn * BT + wn * 64 + j * 32 + (lane & 31);
+                const size_t o = (size_t)row * ldc + col;
+                float v = acc[i][j][e];
+                if (EPI == EPI_POLY) v = sg_fma(NS_C, v, NS_B * sg::bf16_bits_to_f(aux[o]));
+                if (EPI == EPI_APPLY) v = sg_fma(NS_A, sg::bf16_bits_to_f(aux[o]), v);
+                C[o] = sg::f_to_bf16_bits(v);
+            }
+}
+
+// p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
+__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay) {
+    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
+    const Mat& M = B.mats[mi];
+    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
+    const int cnt = min(ETILE, M.rows * M.cols - start);
+    const bf16_t* X = M.wide ? M.Y : M.YT;
+    const int ld = M.wide ? M.np : M.mp;
+    // the reference's scalar arithmetic (csrc/ops.cpp:729-734)
+    const float max_dim = (float)max(M.rows, M.cols);
+    const float scale_factor = 0.2f * sqrtf(max_dim);
+    const float neg_lr_scale = -lr * scale_factor / sqrtf(max_dim);
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int i = start + k, r = i / M.cols, c = i - r * M.cols;
+        float o = sg::bf16_bits_to_f(X[(size_t)r * ld + c]);
+        if (M.dtype == SG_F16) o = __half2float(__float2half_rn(o));     // X.to(p.dtype)
+        const float p = sg::load_elem(M.param, M.dtype, i);
+        sg::store_elem(M.param, M.dtype, i, sg_fma(neg_lr_scale, o, p) * decay);
+    }
+}
+
+__global__ __launch_bounds__(256) void k_zero(uint4* p, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+inline int round_up(int x, int a) { return (x + a - 1) / a * a; }
+
+struct Layout {
+    int P;
+    std::vector<Mat> mats;
+    std::vector<int> pre_e, pre_g[3], pre_t;
+    size_t off_mats, off_pre_e, off_pre_g[3], off_pre_t, off_partials, off_inv, off_buffers, bytes;
+};
+
+int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
+    L->P = P;
+    L->mats.resize(P);
+    L->pre_e.assign(P + 1, 0);
+    for (int k = 0; k < 3; k++) L->pre_g[k].assign(P + 1, 0);
+    L->pre_t.assign(P + 1, 0);
+    size_t o = 0;
+    auto take = [&](size_t b) { size_t r = o; o = sg::align_up(o + b, 256); return r; };
+    L->off_mats = take(sizeof(Mat) * (size_t)P);
+    L->off_pre_e = take(sizeof(int) * (size_t)(P + 1));
+    for (int k = 0; k < 3; k++) L->off_pre_g[k] = take(sizeof(int) * (size_t)(P + 1));
+    L->off_pre_t = take(sizeof(int) * (size_t)(P + 1));
+    int64_t etiles = 0;
+    for (int i = 0; i < P; i++) {
+        const SgMuonMatrix& s = in[i];
+        if (s.rows <= 0 || s.cols <= 0 || s.rows * s.cols > 0x7fffffff) return sg::fail("matrix %d: bad shape %lld x %lld", i, (long long)s.rows, (long long)s.cols);
+        if (s.dtype != SG_F32 && s.dtype != SG_F16 && s.dtype != SG_BF16) return sg::fail("matrix %d: bad dtype %d", i, s.dtype);
+        Mat& M = L->mats[i];
+        M.param = s.param; M.grad = s.grad; M.buf = s.buf;
+        M.rows = (int)s.rows; M.cols = (int)s.cols; M.dtype = s.dtype;
+        M.wide = s.rows <= s.cols;
+        M.m = (int)std::min(s.rows, s.cols); M.n = (int)std::max(s.rows, s.cols);
+        M.mp = round_up(M.m, BT); M.np = round_up(M.n, BT);
+        M.pad_ = 0;
+        const int et = (int)((s.rows * s.cols + ETILE - 1) / ETILE);
+        M.etile0 = (int)etiles;
+        etiles += et;
+        L->pre_e[i + 1] = L->pre_e[i] + et;
+        L->pre_g[EPI_GRAM][i + 1] = L->pre_g[EPI_GRAM][i] + (M.mp / BT) * (M.mp / BT);
+        L->pre_g[EPI_POLY][i + 1] = L->pre_g[EPI_POLY][i] + (M.mp / BT) * (M.mp / BT);
+        L->pre_g[EPI_APPLY][i + 1] = L->pre_g[EPI_APPLY][i] + (M.mp / BT) * (M.np / BT);
+        L->pre_t[i + 1] = L->pre_t[i] + (M.mp / 64) * (M.np / 64);
+    }
+    L->off_partials = take(sizeof(double) * (size_t)(etiles + 1));
+    L->off_inv = take(sizeof(float) * (size_t)P);
+    L->off_buffers = o;
+    for (int i = 0; i < P; i++) {
+        Mat& M = L->mats[i];
+        // offsets for now; turned into pointers once the workspace base is known
+        M.Y = (bf16_t*)take(2 * (size_t)M.mp * M.np);
+        M.YT = (bf16_t*)take(2 * (size_t)M.mp * M.np);
+        M.G = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
+        M.H = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
+    }
+    L->bytes = o;
+    return 0;
+}
+
+}  // namespace
+}  // namespace sgmu
+
+extern "C" {
+
+size_t sg_muon_workspace_bytes(int num_matrices, const SgMuonMatrix* mats) {
+    if (num_matrices <= 0 || !mats) return 0;
+    sgmu::Layout L;
+    if (sgmu::make_layout(num_matrices, mats, &L)) return 0;
+    return L.bytes;
+}
+
+int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, float lr, float wd, int ns_steps, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+    using namespace sgmu;
+    if (num_matrices <= 0) return 0;
+    if (!mats) return sg::fail("NULL argument");
+    if (ns_steps < 0) return sg::fail("ns_steps must be >= 0");
+    for (int i = 0; i < num_matrices; i++)
+        if (!mats[i].param || !mats[i].grad || !mats[i].buf) return sg::fail("matrix %d: NULL pointer", i);
+    Layout L;
+    if (make_layout(num_matrices, mats, &L)) return 1;
+    if (!workspace || workspace_bytes < L.bytes) return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
+    if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    unsigned char* ws = static_cast<unsigned char*>(workspace);
+    const int P = L.P;
+    for (auto& M : L.mats) {
+        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.YT = (bf16_t*)(ws + (size_t)M.YT);
+        M.G = (bf16_t*)(ws + (size_t)M.G); M.H = (bf16_t*)(ws + (size_t)M.H);
+    }
+    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, hipMemcpyHostToDevice, st));
+    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_e, L.pre_e.data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
+    for (int k = 0; k < 3; k++)
+        SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_g[k], L.pre_g[k].data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
+    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_t, L.pre_t.data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
+    Batch B;
+    B.mats = reinterpret_cast<const Mat*>(ws + L.off_mats);
+    B.etile_prefix = reinterpret_cast<const int*>(ws + L.off_pre_e);
+    for (int k = 0; k < 3; k++) B.gtile_prefix[k] = reinterpret_cast<const int*>(ws + L.off_pre_g[k]);
+    B.ttile_prefix = reinterpret_cast<const int*>(ws + L.off_pre_t);
+    B.P = P;
+    B.etiles = L.pre_e[P];
+    for (int k = 0; k < 3; k++) B.gtiles[k] = L.pre_g[k][P];
+    B.ttiles = L.pre_t[P];
+    B.partials = reinterpret_cast<double*>(ws + L.off_partials);
+    B.inv_norm = reinterpret_cast<float*>(ws + L.off_inv);
+
+    // padded work buffers start from zero (a fill kernel, not a memset node, so the call stays capturable)
+    bool any_pad = false;
+    for (const auto& M : L.mats) any_pad = any_pad || M.mp != M.m || M.np != M.n;
+    if (any_pad) {
+        const size_t n16 = (L.bytes - L.off_buffers) / 16;
+        hipLaunchKernelGGL(k_zero, dim3((unsigned)std::min<size_t>((n16 + 255) / 256, 65535)), dim3(256), 0, st,
+                           reinterpret_cast<uint4*>(ws + L.off_buffers), n16);
+    }
+
+    hipLaunchKernelGGL(k_momentum, dim3(B.etiles), dim3(256), 0, st, B, momentum);
+    hipLaunchKernelGGL(k_norm, dim3(P), dim3(256), 0, st, B);
+    hipLaunchKernelGGL(k_normalize, dim3(B.etiles), dim3(256), 0, st, B);
+    SG_LAUNCH_CHECK("muon prologue");
+    if (ns_steps > 0) {
+        // wide matrices: YT from Y; tall matrices: Y from YT
+        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 1, 0, 1);
+        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 0, 1, 0);
+        SG_LAUNCH_CHECK("muon transpose");
+    }
+    for (int it = 0; it < ns_steps; it++) {
+        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), 0, st, B);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), 0, st, B);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), 0, st, B);
+        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 1, 0, 0);    // YT <- Y^T for every matrix
+        SG_LAUNCH_CHECK("muon newton-schulz");
+    }
+    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd);
+    SG_LAUNCH_CHECK("k_update");
+    return 0;
+}
+
+}  // extern "C"

@@ -1,1 +1,21 @@
-"""MI355X-native fused optimizer steps behind the grokking_optimizers API."""
+"""grokking_optimizers on MI355X: the Grokfast, SuperGrok v1.5, SuperGrok v2 and
+Muon optimizer classes of peterc04/SuperGrok1.5, with every fused step running
+as hand-written HIP (libsg_hip.so) behind the reference's `_ops` extension
+surface.  As in the reference (grokking_optimizers/__init__.py:13-20 there),
+importing fails unless the compiled extension is present; there is no Python
+or CPU fallback.
+"""
+try:
+    from grokking_optimizers import _ops  # noqa: F401
+except ImportError as e:  # pragma: no cover
+    raise ImportError(
+        "grokking_optimizers needs its compiled extension (_ops) and libsg_hip.so; "
+        "build them with `python __graft_entry__.py` at the repository root (%s)" % e)
+
+from grokking_optimizers.grokfast import Grokfast
+from grokking_optimizers.muon import Muon
+from grokking_optimizers.supergrok15 import SuperGrok15, SharpnessMetaNet
+from grokking_optimizers.supergrok2 import SuperGrok2
+from grokking_optimizers.mamba3_peer_metanet import Mamba3PEERMetaNet
+
+__all__ = ["Grokfast", "Muon", "SuperGrok15", "SharpnessMetaNet", "SuperGrok2", "Mamba3PEERMetaNet"]

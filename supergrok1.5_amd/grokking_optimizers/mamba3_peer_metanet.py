@@ -1,0 +1,140 @@
+"""Parameter container of the SuperGrok v2 meta-network: bidirectional Mamba-3
+scan blocks, per-element GRU, 4-head PEER product-key router and the expert
+pool.  Same sub-module / parameter names, shapes and initialisation as the
+reference (grokking_optimizers/mamba3_peer_metanet.py:44-269), so state dicts
+are interchangeable; `get_weights` (:515-567 there) exports the tensors in the
+layout the fused step consumes, and `_recycle_dead_experts` (:437-491 there)
+is the host-side expert recycling.
+
+The arithmetic of the network runs inside the fused HIP step
+(`_ops.supergrok2_mamba_peer_batched_step`); this module has no forward pass
+of its own.
+"""
+import math
+
+import torch
+import torch.nn as nn
+
+
+class Mamba3ScanBlock(nn.Module):
+    def __init__(self, d_model: int = 8, d_state: int = 16, expand: int = 2):
+        super().__init__()
+        assert d_state % 2 == 0, "d_state must be even for paired RoPE"
+        self.d_model, self.d_state, self.d_inner = d_model, d_state, d_model * expand
+        di = self.d_inner
+        self.in_proj = nn.Linear(d_model, 2 * di, bias=False)
+        self.dt_proj = nn.Linear(di, di, bias=True)
+        self.B_proj = nn.Linear(di, d_state, bias=False)
+        self.C_proj = nn.Linear(di, d_state, bias=False)
+        self.A_log = nn.Parameter(torch.log(torch.linspace(1, d_state, d_state)).unsqueeze(0).repeat(di, 1))
+        self.D = nn.Parameter(torch.ones(di))
+        self.rope_freq = nn.Parameter(torch.randn(di, d_state // 2) * 0.01)
+        self.out_proj = nn.Linear(di, d_model, bias=False)
+
+    def export(self):
+        f = lambda t: t.detach().float().contiguous()
+        return [f(self.in_proj.weight), f(self.dt_proj.weight), f(self.dt_proj.bias), f(self.B_proj.weight),
+                f(self.C_proj.weight), f(self.A_log), f(self.D), f(self.rope_freq), f(self.out_proj.weight)]
+
+
+class MiniGRU(nn.Module):
+    def __init__(self, input_dim: int, hidden_dim: int = 4):
+        super().__init__()
+        self.hidden_dim = hidden_dim
+        self.W_z = nn.Linear(input_dim + hidden_dim, hidden_dim)
+        self.W_r = nn.Linear(input_dim + hidden_dim, hidden_dim)
+        self.W_h = nn.Linear(input_dim + hidden_dim, hidden_dim)
+
+
+class Mamba3PEERMetaNet(nn.Module):
+    def __init__(self, d_model: int = 8, d_state: int = 16, mamba_expand: int = 2, num_peer_heads: int = 4,
+                 num_experts: int = 144, expert_hidden: int = 16, gru_hidden: int = 4, rescale: float = 0.1,
+                 recycle_interval: int = 100, recycle_threshold: float = 0.001):
+        super().__init__()
+        self.d_model, self.d_state = d_model, d_state
+        self.num_peer_heads, self.num_experts = num_peer_heads, num_experts
+        self.expert_hidden, self.gru_hidden = expert_hidden, gru_hidden
+        self.rescale = rescale
+        self.recycle_interval, self.recycle_threshold = recycle_interval, recycle_threshold
+        self.pk_dim = int(math.sqrt(num_experts))
+        assert self.pk_dim * self.pk_dim == num_experts, f"num_experts must be perfect square, got {num_experts}"
+        self.input_proj = nn.Linear(2, d_model, bias=True)
+        self.mamba_fwd = Mamba3ScanBlock(d_model, d_state, mamba_expand)
+        self.mamba_bwd = Mamba3ScanBlock(d_model, d_state, mamba_expand)
+        self.gru = MiniGRU(2 + 2 * d_model, gru_hidden)
+        peer_in = gru_hidden + 2 * d_model + 2
+        self.peer_queries = nn.ModuleList([nn.Linear(peer_in, d_model, bias=False) for _ in range(num_peer_heads)])
+        mk_keys = lambda: nn.ParameterList([nn.Parameter(torch.randn(self.pk_dim, d_model // 2) * 0.02)
+                                            for _ in range(num_peer_heads)])
+        self.product_keys_A = mk_keys()
+        self.product_keys_B = mk_keys()
+        self.expert_W1 = nn.Parameter(torch.randn(num_experts, expert_hidden, 1) * 0.02)
+        self.expert_b1 = nn.Parameter(torch.zeros(num_experts, expert_hidden))
+        self.expert_W2 = nn.Parameter(torch.randn(num_experts, 1, expert_hidden) * 0.02)
+        self.expert_b2 = nn.Parameter(torch.zeros(num_experts, 1))
+        self.register_buffer("expert_counts", torch.zeros(num_experts, dtype=torch.int32))
+        self.register_buffer("step_counter", torch.tensor(0, dtype=torch.long))
+
+    def get_weights(self):
+        f = lambda t: t.detach().float().contiguous()
+        names = ("in_proj", "dt_proj_W", "dt_proj_b", "B_proj", "C_proj", "A_log", "D", "rope_freq", "out_proj")
+        w = {"input_proj_W": f(self.input_proj.weight), "input_proj_b": f(self.input_proj.bias)}
+        for tag, blk in (("fwd", self.mamba_fwd), ("bwd", self.mamba_bwd)):
+            w.update({f"mamba_{tag}_{n}": t for n, t in zip(names, blk.export())})
+        for g, lin in (("z", self.gru.W_z), ("r", self.gru.W_r), ("h", self.gru.W_h)):
+            w[f"gru_W_{g}"], w[f"gru_b_{g}"] = f(lin.weight), f(lin.bias)
+        w["peer_queries"] = [f(q.weight) for q in self.peer_queries]
+        w["product_keys_A"] = [f(k) for k in self.product_keys_A]
+        w["product_keys_B"] = [f(k) for k in self.product_keys_B]
+        for n in ("expert_W1", "expert_b1", "expert_W2", "expert_b2"):
+            w[n] = f(getattr(self, n))
+        w.update(rescale=self.rescale, d_model=self.d_model, d_state=self.d_state, d_inner=self.mamba_fwd.d_inner,
+                 pk_dim=self.pk_dim, expert_hidden=self.expert_hidden, gru_hidden=self.gru_hidden,
+                 num_peer_heads=self.num_peer_heads, num_experts=self.num_experts)
+        return w
+
+    def flat_weights(self):
+        """The 33 tensors in the argument order of _ops.supergrok2_mamba_peer_batched_step."""
+        w = self.get_weights()
+        out = [w["input_proj_W"], w["input_proj_b"]]
+        for tag in ("fwd", "bwd"):
+            out += [w[f"mamba_{tag}_{n}"] for n in ("in_proj", "dt_proj_W", "dt_proj_b", "B_proj", "C_proj", "A_log",
+                                                    "D", "rope_freq", "out_proj")]
+        out += [w["gru_W_z"], w["gru_b_z"], w["gru_W_r"], w["gru_b_r"], w["gru_W_h"], w["gru_b_h"]]
+        out += [torch.stack(w["peer_queries"]), torch.stack(w["product_keys_A"]), torch.stack(w["product_keys_B"])]
+        E = self.num_experts
+        out += [w["expert_W1"].reshape(E, -1), w["expert_b1"], w["expert_W2"].reshape(E, -1), w["expert_b2"].reshape(-1)]
+        return out
+
+    @torch.no_grad()
+    def _recycle_dead_experts(self):
+        """Experts with fewer than recycle_threshold of the activations are replaced by a noisy clone of
+        an expert sampled in proportion to its count; a product key is re-drawn only when every expert
+        sharing it is dead.  Returns True if anything changed.  Random draws, in order: one multinomial,
+        then per dead expert (ascending index) W1, b1, W2, b2 noise, then key A redraws per head, then
+        key B redraws per head -- the sequence of the reference (mamba3_peer_metanet.py:453-488)."""
+        total = self.expert_counts.sum().item()
+        if total == 0:
+            return False
+        dead = (self.expert_counts.float() / total) < self.recycle_threshold
+        if not dead.any():
+            self.expert_counts.zero_()
+            return False
+        top = torch.multinomial(self.expert_counts.float(), 1).item()
+        pk, H = self.pk_dim, self.num_peer_heads
+        for i in dead.nonzero(as_tuple=True)[0].tolist():
+            for name in ("expert_W1", "expert_b1", "expert_W2", "expert_b2"):
+                t = getattr(self, name).data
+                t[i] = t[top] + 0.01 * torch.randn_like(t[i])
+            a, b = divmod(i, pk)
+            if dead[a * pk:(a + 1) * pk].all():
+                for h in range(H):
+                    row = self.product_keys_A[h].data[a]
+                    self.product_keys_A[h].data[a] = torch.randn_like(row) * 0.02
+            cols = torch.arange(0, self.num_experts, pk, device=dead.device) + b
+            if dead[cols[cols < self.num_experts]].all():
+                for h in range(H):
+                    row = self.product_keys_B[h].data[b]
+                    self.product_keys_B[h].data[b] = torch.randn_like(row) * 0.02
+        self.expert_counts.zero_()
+        return True

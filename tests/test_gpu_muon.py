@@ -1,0 +1,109 @@
+"""GPU parity of the Muon step (bf16 MFMA Newton-Schulz behind `_ops.muon_fused_step`)
+with the fp32 CPU restatement and the reference's golden vectors.
+
+Gates: momentum buffer within 1e-4 relative; orthogonalised update within 2e-2
+relative Frobenius norm of the fp32 iteration (bf16 operands, fp32 accumulation);
+updated parameters within one bf16 ulp (bf16 params) or 2e-2*0.2*lr (fp32 params)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import rel_close
+from oracle import muon_oracle
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _ops():
+    from grokking_optimizers import _ops
+    return _ops
+
+
+def _bf16(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).float().numpy()
+
+
+def _run_case(shapes, dt, steps, seed, lr=0.02, wd=1.0, momentum=0.95, ns=5):
+    ops = _ops()
+    gen = torch.Generator().manual_seed(seed)
+    p0 = [(torch.randn(*s, generator=gen) * 0.02).to(dt) for s in shapes]
+    params = [p.clone().cuda() for p in p0]
+    bufs = [torch.zeros(s, device="cuda") for s in shapes]
+    rp = [p.float().numpy().copy() for p in p0]
+    rb = [np.zeros(s, np.float32) for s in shapes]
+    for t in range(steps):
+        grads = [(torch.randn(*s, generator=gen) * 1e-3).to(dt) for s in shapes]
+        print("muon step", t, shapes, dt, flush=True)
+        ops.muon_fused_step(params, [g.cuda() for g in grads], bufs, momentum, lr, wd, ns)
+        torch.cuda.synchronize()
+        for i, s in enumerate(shapes):
+            old = rp[i]
+            new_p, X = muon_oracle.muon_step(old, grads[i].float().numpy(), rb[i], momentum, lr, wd, ns)
+            ok, r = rel_close(bufs[i].cpu().numpy(), rb[i], 1e-4, 1e-7)
+            assert ok, ("buf", t, i, r)
+            got = params[i].float().cpu().numpy()
+            # recover the applied update: p_new/decay - p_old = -0.2*lr*X
+            decay = np.float32(1.0) - np.float32(lr) * np.float32(wd)
+            if dt == torch.float32:
+                X_gpu = (got / decay - old) / (-0.2 * lr)
+                rel_f = np.linalg.norm(X_gpu - X) / np.linalg.norm(X)
+                assert rel_f < 2e-2, ("X frobenius", t, i, rel_f)
+                sv = np.linalg.svd(X_gpu.astype(np.float64), compute_uv=False)
+                assert sv.min() > 0.5 and sv.max() < 1.3, (sv.min(), sv.max())
+            else:
+                want = _bf16(new_p) if dt == torch.bfloat16 else new_p.astype(np.float16).astype(np.float32)
+                ulp = np.abs(want) * (2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10) + 1e-12
+                nd = np.abs(got - want) / ulp
+                assert nd.max() <= 1.01, ("param ulps", t, i, nd.max())
+                # keep the fp32 trajectory of the checker aligned with the 16-bit parameters of the device
+                new_p = got
+            rp[i] = got if dt != torch.float32 else new_p
+            if dt == torch.float32:
+                params[i].copy_(torch.from_numpy(new_p).cuda())      # re-sync so the next step starts identical
+
+
+def test_small_shapes_all_dtypes():
+    shapes = [(24, 40), (40, 24), (16, 16), (130, 70), (1, 5)]
+    for dt in (torch.float32, torch.bfloat16, torch.float16):
+        _run_case(shapes, dt, 2, seed=1)
+
+
+def test_reference_golden_f32():
+    ops = _ops()
+    z = np.load(os.path.join(GOLD, "ref_muon.npz"))
+    P = int(z["n"])
+    params = [torch.from_numpy(z[f"f32_p_in_{i}"]).cuda() for i in range(P)]
+    bufs = [torch.zeros_like(p) for p in params]
+    grads = [torch.from_numpy(z[f"f32_g_0_{i}"]).cuda() for i in range(P)]
+    ops.muon_fused_step(params, grads, bufs, float(z["momentum"]), float(z["lr"]), float(z["wd"]), int(z["ns_steps"]))
+    for i in range(P):
+        ok, r = rel_close(bufs[i].cpu().numpy(), z[f"f32_buf_0_{i}"], 1e-4, 1e-7)
+        assert ok, r
+        p_in, want = z[f"f32_p_in_{i}"], z[f"f32_p_0_{i}"]
+        upd_ref, upd_got = want / 0.98 - p_in, params[i].cpu().numpy() / 0.98 - p_in
+        assert np.linalg.norm(upd_got - upd_ref) / np.linalg.norm(upd_ref) < 2e-2
+
+
+def test_config5_sized_matrices():
+    """One wide 1024x4096 and one tall 4096x1024 bf16 matrix, 5 Newton-Schulz iterations, two steps."""
+    _run_case([(1024, 4096), (4096, 1024)], torch.bfloat16, 2, seed=5)
+    # fp32 parameters expose the orthogonalised update itself
+    _run_case([(1024, 4096)], torch.float32, 1, seed=6)
+
+
+def test_class_and_errors():
+    from grokking_optimizers import Muon
+    ops = _ops()
+    w = torch.nn.Parameter((torch.randn(64, 96) * 0.02).cuda())
+    b = torch.nn.Parameter(torch.zeros(96).cuda())
+    opt = Muon([w], [b], lr=0.02, weight_decay=0.0)
+    for _ in range(2):
+        w.grad, b.grad = torch.randn_like(w) * 1e-3, torch.randn_like(b) * 1e-3
+        opt.step()
+    assert opt.state[w]["momentum_buffer"].dtype == torch.float32 and "exp_avg" in opt.state[b]
+    assert bool(torch.isfinite(w).all())
+    with pytest.raises(RuntimeError, match="2-D"):
+        ops.muon_fused_step([torch.zeros(4, device="cuda")], [torch.ones(4, device="cuda")], [torch.zeros(4, device="cuda")], 0.9, 0.1, 0.0, 5)
