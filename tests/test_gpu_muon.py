@@ -3,7 +3,8 @@ with the fp32 CPU restatement and the reference's golden vectors.
 
 Gates: momentum buffer within 1e-4 relative; orthogonalised update within 2e-2
 relative Frobenius norm of the fp32 iteration (bf16 operands, fp32 accumulation);
-updated parameters within one bf16 ulp (bf16 params) or 2e-2*0.2*lr (fp32 params)."""
+updated 16-bit parameters within one ulp of the stored value plus the deviation of
+the update (fp32 parameters expose the update itself, checked in Frobenius norm)."""
 import os
 
 import numpy as np
@@ -55,9 +56,12 @@ def _run_case(shapes, dt, steps, seed, lr=0.02, wd=1.0, momentum=0.95, ns=5):
                 assert sv.min() > 0.5 and sv.max() < 1.3, (sv.min(), sv.max())
             else:
                 want = _bf16(new_p) if dt == torch.bfloat16 else new_p.astype(np.float16).astype(np.float32)
-                ulp = np.abs(want) * (2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10) + 1e-12
-                nd = np.abs(got - want) / ulp
-                assert nd.max() <= 1.01, ("param ulps", t, i, nd.max())
+                # one rounding step of the stored parameter + the bf16-vs-fp32 Newton-Schulz deviation of the
+                # update itself (elementwise bound: 10% of the largest update entry; Frobenius: 2e-2, above)
+                ulp = np.maximum(np.abs(want), np.abs(got)) * (2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10)
+                tol = ulp + 0.1 * 0.2 * lr * np.abs(X).max() + 1e-12
+                nd = np.abs(got - want) / tol
+                assert nd.max() <= 1.0, ("param tolerance", t, i, nd.max())
                 # keep the fp32 trajectory of the checker aligned with the 16-bit parameters of the device
                 new_p = got
             rp[i] = got if dt != torch.float32 else new_p
