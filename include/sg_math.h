@@ -131,6 +131,23 @@ SG_HD void sg_sincos(float th, float* s_out, float* c_out) {
     *c_out = sg_i2f((int32_t)((uint32_t)sg_f2i(c0) ^ ((((uint32_t)q + 1u) & 2u) << 30)));
 }
 
+/* sg_sincos for |theta| < 0.78: the reduction multiple is then 0, so the
+ * general routine reduces to the two polynomials; the results are bit for
+ * bit those of sg_sincos.  Lets a wavefront skip the reduction and quadrant
+ * logic when all its lanes hold small angles. */
+SG_HD void sg_sincos_small(float th, float* s_out, float* c_out) {
+    const float z = th * th;
+    float sp = -1.9515295891e-4f;
+    sp = sg_fma(sp, z, 8.3321608736e-3f);
+    sp = sg_fma(sp, z, -1.6666654611e-1f);
+    *s_out = sg_fma(sp * z, th, th);
+    float cp = 2.443315711809948e-5f;
+    cp = sg_fma(cp, z, -1.388731625493765e-3f);
+    cp = sg_fma(cp, z, 4.166664568298827e-2f);
+    *c_out = sg_fma(cp * z, z, sg_fma(z, -0.5f, 1.0f));
+}
+#define SG_SINCOS_SMALL_LIMIT 0.78f
+
 /* 1/d for normal positive d: bit-trick seed + three Newton steps (~5e-8 rel). */
 SG_HD float sg_rcp_pos(float d) {
     float r = sg_i2f(0x7EF311C7 - sg_f2i(d));

@@ -32,7 +32,7 @@ def lib():
         if not os.path.exists(_LIB):
             build()
         _lib = C.CDLL(_LIB)
-        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf",
+        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf", "sin_small", "cos_small",
                   "gelu_sigmoid"):
             f = getattr(_lib, "orc_" + n)
             f.restype = C.c_float

@@ -514,6 +514,8 @@ float orc_tanh(float x) { return sg_tanh(x); }
 float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }
 float orc_cos(float x) { float s, c; sg_sincos(x, &s, &c); return c; }
 float orc_rcp_pos(float x) { return sg_rcp_pos(x); }
+float orc_sin_small(float x) { float s, c; sg_sincos_small(x, &s, &c); return s; }
+float orc_cos_small(float x) { float s, c; sg_sincos_small(x, &s, &c); return c; }
 float orc_abar(float dt, float A) { float e, o; sg_abar_pair(dt, 0.5f * A, 0.5f * A, &e, &o); return e; }
 uint16_t orc_f_to_f16(float f) { return f_to_f16(f); }
 float orc_f16_to_f(uint16_t h) { return f16_to_f(h); }

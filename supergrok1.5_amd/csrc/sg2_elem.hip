@@ -11,7 +11,7 @@
 // over a P+1 entry prefix table.  The 144 expert MLPs live in LDS (records of
 // 48 floats padded to 52 so that random per-lane experts spread over the
 // banks); GRU / query / key weights are wave-uniform and come in through
-// scalar loads.  expert_counts is accumulated in an LDS histogram and flushed
+// scalar loads (constant address space).  expert_counts is accumulated in an LDS histogram and flushed
 // once per workgroup (the reference issues one global atomic per element and
 // head).
 #include "sg2_internal.hpp"
@@ -46,18 +46,18 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
     }
     __syncthreads();
 
-    const float* __restrict__ Wz = pl.W.w[W_GRU_WZ];
-    const float* __restrict__ bz = pl.W.w[W_GRU_BZ];
-    const float* __restrict__ Wr = pl.W.w[W_GRU_WR];
-    const float* __restrict__ br = pl.W.w[W_GRU_BR];
-    const float* __restrict__ Wh = pl.W.w[W_GRU_WH];
-    const float* __restrict__ bh = pl.W.w[W_GRU_BH];
-    const float* __restrict__ Wq = pl.W.w[W_PEER_Q];
-    const float* __restrict__ KA = pl.W.w[W_KEYS_A];
-    const float* __restrict__ KB = pl.W.w[W_KEYS_B];
+    const sg::cfloat_p Wz = sg::as_const(pl.W.w[W_GRU_WZ]);
+    const sg::cfloat_p bz = sg::as_const(pl.W.w[W_GRU_BZ]);
+    const sg::cfloat_p Wr = sg::as_const(pl.W.w[W_GRU_WR]);
+    const sg::cfloat_p br = sg::as_const(pl.W.w[W_GRU_BR]);
+    const sg::cfloat_p Wh = sg::as_const(pl.W.w[W_GRU_WH]);
+    const sg::cfloat_p bh = sg::as_const(pl.W.w[W_GRU_BH]);
+    const sg::cfloat_p Wq = sg::as_const(pl.W.w[W_PEER_Q]);
+    const sg::cfloat_p KA = sg::as_const(pl.W.w[W_KEYS_A]);
+    const sg::cfloat_p KB = sg::as_const(pl.W.w[W_KEYS_B]);
 
     for (int tile = blockIdx.x; tile < pl.elem_tiles; tile += gridDim.x) {
-        const int ti = sg::upper_seg(pl.elem_tile_prefix, pl.P, tile);
+        const int ti = sg::upper_seg(sg::as_const(pl.elem_tile_prefix), pl.P, tile);
         const TensorDev& T = pl.tensors[ti];
         const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
         const int cnt = min(ELEM_TILE, T.numel - start);
@@ -84,8 +84,8 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             float zg[GH], rg[GH], hnew[GH];
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const float* wz = Wz + j * GRL;
-                const float* wr = Wr + j * GRL;
+                const sg::cfloat_p wz = Wz + j * GRL;
+                const sg::cfloat_p wr = Wr + j * GRL;
                 float vz = bz[j], vr = br[j];
                 vz = sg_fma(wz[0], g, vz); vz = sg_fma(wz[1], s, vz);
                 vr = sg_fma(wr[0], g, vr); vr = sg_fma(wr[1], s, vr);
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             }
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const float* wh = Wh + j * GRL;
+                const sg::cfloat_p wh = Wh + j * GRL;
                 float v = bh[j];
                 v = sg_fma(wh[0], g, v); v = sg_fma(wh[1], s, v);
 #pragma unroll
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 float query[DM];
 #pragma unroll
                 for (int dd = 0; dd < DM; dd++) {
-                    const float* qr = Wq + (hh * DM + dd) * PIN;
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
                     float v = 0.0f;
 #pragma unroll
                     for (int q = 0; q < GH; q++) v = sg_fma(qr[q], hnew[q], v);
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 int best[2];
 #pragma unroll
                 for (int hf = 0; hf < 2; hf++) {
-                    const float* keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
                     int bi = 0;
                     float bs = -1e30f;
 #pragma unroll

@@ -21,19 +21,31 @@
 // Per-timestep projections (in_proj, dt, B, C) are recomputed in both passes
 // for tiles of 64 timesteps and staged through LDS instead of being
 // materialised in HBM (the reference writes 320 B per element per direction).
+//
+// The kernels are bound by fp32 VALU issue, not by HBM: per (timestep, column,
+// pair) one shared reciprocal, one sin/cos pair and the 2x2 update.  The
+// recurrence loop therefore works on blocks of 8 timesteps: all LDS operands of
+// the block are fetched first, the state-independent coefficients of the 8
+// steps are computed as independent instruction streams, and only the short
+// h-update chain is serial.  When every lane of the wave holds a small
+// rotation angle the sin/cos range reduction is skipped (bit-identical
+// results, see sg_sincos_small).
 #include "sg2_internal.hpp"
 
 namespace sg2 {
 namespace {
 
 constexpr int LDS_STRIDE = SCAN_TT + 1;   // [row][timestep] rows padded so the 8 rows a wave reads sit in 8 banks
+constexpr int UB = 8;                     // timesteps per unrolled block of the recurrence
 
 struct DirW {
-    const float *in_proj, *dt_W, *dt_b, *Bp, *Cp, *A_log, *D, *rope, *out_proj;
+    sg::cfloat_p in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj;
 };
 __device__ __forceinline__ DirW dir_weights(const Sg2Weights& W, int dir) {
     const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-    return {W.w[b], W.w[b + 1], W.w[b + 2], W.w[b + 3], W.w[b + 4], W.w[b + 5], W.w[b + 6], W.w[b + 7], W.w[b + 8]};
+    return {sg::as_const(W.w[b]),     sg::as_const(W.w[b + 1]), sg::as_const(W.w[b + 2]),
+            sg::as_const(W.w[b + 3]), sg::as_const(W.w[b + 4]), sg::as_const(W.w[b + 5]),
+            sg::as_const(W.w[b + 6]), sg::as_const(W.w[b + 7]), sg::as_const(W.w[b + 8])};
 }
 
 __device__ __forceinline__ float dpp_quad_swap1(float v) {   // lane ^ 1
@@ -45,7 +57,12 @@ __device__ __forceinline__ float dpp_quad_swap2(float v) {   // lane ^ 2
 __device__ __forceinline__ float dpp_half_mirror(float v) {  // lane -> 7 - lane within each group of 8
     return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0x141, 0xF, 0xF, true));
 }
-
+// sum over the 8 lanes of a (column) group, as the balanced tree ((0+1)+(2+3)) + ((4+5)+(6+7))
+__device__ __forceinline__ float pair_tree_sum(float y) {
+    y = y + dpp_quad_swap1(y);
+    y = y + dpp_quad_swap2(y);
+    return y + dpp_half_mirror(y);
+}
 
 // Projections of one timestep (x = projected input, 8 floats).  Both halves of
 // the workgroup compute the 16 x-branch values; each then produces its half
@@ -65,8 +82,7 @@ __device__ __forceinline__ void project_tile(const DirW& w, const float (&x)[DM]
     }
 #pragma unroll
     for (int q = 0; q < DI / 2; q++) {
-        constexpr int base = HALF * (DI / 2);
-        const int jj = base + q;
+        const int jj = HALF * (DI / 2) + q;
         float a = w.dt_b[jj];
 #pragma unroll
         for (int k = 0; k < DI; k++) a = sg_fma(w.dt_W[jj * DI + k], xb[k], a);
@@ -99,6 +115,53 @@ __device__ __forceinline__ void project_tile(const DirW& w, const float (&x)[DM]
     }
 }
 
+// scan state of one lane: OUT -> (he,ho) only; summary -> also the two columns of M
+struct LaneState {
+    float he, ho, c0e, c0o, c1e, c1o;
+};
+
+template <bool OUT>
+__device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, float sn, float cs, float be, float bo) {
+    if (!OUT) {
+        float re = sg_fma(S.c0e, cs, -(S.c0o * sn)), ro = sg_fma(S.c0o, cs, S.c0e * sn);
+        S.c0e = ae * re;
+        S.c0o = ao * ro;
+        re = sg_fma(S.c1e, cs, -(S.c1o * sn));
+        ro = sg_fma(S.c1o, cs, S.c1e * sn);
+        S.c1e = ae * re;
+        S.c1o = ao * ro;
+    }
+    const float re = sg_fma(S.he, cs, -(S.ho * sn));
+    const float ro = sg_fma(S.ho, cs, S.he * sn);
+    S.he = sg_fma(ae, re, be);
+    S.ho = sg_fma(ao, ro, bo);
+}
+
+// UB consecutive timesteps (all valid): coefficients first, then the serial chain
+template <bool OUT, bool SMALL_ANGLE>
+__device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&xv)[UB], const float (&Be)[UB],
+                                            const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
+                                            float hAo, float freq, float (&y)[UB]) {
+    float ae[UB], ao[UB], sn[UB], cs[UB], be[UB], bo[UB];
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+        sg_abar_pair(dt[u], hAe, hAo, &ae[u], &ao[u]);
+        if (SMALL_ANGLE) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
+        else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
+        be[u] = (dt[u] * Be[u]) * xv[u];
+        bo[u] = (dt[u] * Bo[u]) * xv[u];
+    }
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+        step_update<OUT>(S, ae[u], ao[u], sn[u], cs[u], be[u], bo[u]);
+        if (OUT) y[u] = sg_fma(S.ho, Co[u], S.he * Ce[u]);
+    }
+    if (OUT) {
+#pragma unroll
+        for (int u = 0; u < UB; u++) y[u] = pair_tree_sum(y[u]);
+    }
+}
+
 template <bool OUT>
 __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
     __shared__ float s_dt[DI * LDS_STRIDE];
@@ -111,34 +174,34 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
     const int per_dir = OUT ? pl.chunks : pl.wchunks;
     const int dir = (int)blockIdx.x >= per_dir ? 1 : 0;
     const int cidx = (int)blockIdx.x - dir * per_dir;
-    const int* __restrict__ prefix = OUT ? pl.chunk_prefix : pl.wchunk_prefix;
+    const sg::cint_p prefix = sg::as_const(OUT ? pl.chunk_prefix : pl.wchunk_prefix);
     const int ti = sg::upper_seg(prefix, pl.P, cidx);
     const int c = cidx - prefix[ti];                       // chunk within the tensor
     const TensorDev& T = pl.tensors[ti];
     const int N = T.numel, dtype = T.dtype, off = T.off;
+    const void* const t_grad = T.grad;
+    const void* const t_sharp = T.sharp;
     const int u0 = c * pl.chunk_len;                       // first scan step of the chunk
     const int u1 = min(u0 + pl.chunk_len, N);
     const DirW w = dir_weights(pl.W, dir);
     const int32_t* __restrict__ perm = pl.vals[0] + off;
+    const sg::cfloat_p Wi = sg::as_const(pl.W.w[W_IN_W]);
+    const sg::cfloat_p bi = sg::as_const(pl.W.w[W_IN_B]);
 
     const int tid = threadIdx.x;
     const int tu = tid & (SCAN_TT - 1);                                   // projection role: timestep of the tile
     const int half = __builtin_amdgcn_readfirstlane(tid >> 6);           // projection role: which half of the outputs
     const int j = tid >> 3, p = tid & 7;                                  // scan role
 
-    const float hAe = 0.5f * -sg_exp(w.A_log[j * DS + 2 * p]);
-    const float hAo = 0.5f * -sg_exp(w.A_log[j * DS + 2 * p + 1]);
-    const float freq = w.rope[j * HP + p];
+    const float hAe = 0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
+    const float hAo = 0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
+    const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
 
-    // scan state: OUT -> (he,ho);  summary -> columns (c0e,c0o),(c1e,c1o) and offset (be,bo)
-    float he, ho, c0e = 1.0f, c0o = 0.0f, c1e = 0.0f, c1o = 1.0f;
+    LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     if (OUT) {
         const float* hs = pl.hstart + ((size_t)(dir * pl.chunks + cidx) * 2) * SCAN_THREADS;
-        he = hs[tid];
-        ho = hs[SCAN_THREADS + tid];
-    } else {
-        he = 0.0f;
-        ho = 0.0f;
+        S.he = hs[tid];
+        S.ho = hs[SCAN_THREADS + tid];
     }
 
     for (int tile0 = u0; tile0 < u1; tile0 += SCAN_TT) {
@@ -154,11 +217,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
                 const int t = dir ? (N - 1 - u) : u;
                 orig = perm[t];
                 orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
-                g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, orig));
-                s = sg::finite_or_zero(sg::load_elem(T.sharp, dtype, orig));
+                g = sg::finite_or_zero(sg::load_elem(t_grad, dtype, orig));
+                s = sg::finite_or_zero(sg::load_elem(t_sharp, dtype, orig));
             }
-            const float* __restrict__ Wi = pl.W.w[W_IN_W];
-            const float* __restrict__ bi = pl.W.w[W_IN_B];
 #pragma unroll
             for (int k = 0; k < DM; k++) x[k] = sg_fma(Wi[2 * k + 1], s, Wi[2 * k] * g) + bi[k];
         }
@@ -175,35 +236,38 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
         const float* __restrict__ r_Bo = s_B + (2 * p + 1) * LDS_STRIDE;
         const float* __restrict__ r_Ce = s_C + (OUT ? (2 * p) * LDS_STRIDE : 0);
         const float* __restrict__ r_Co = s_C + (OUT ? (2 * p + 1) * LDS_STRIDE : 0);
-#pragma unroll 4
-        for (int k = 0; k < cnt; k++) {
-            const float dt = r_dt[k], xv = r_xb[k];
+        int k0 = 0;
+        for (; k0 + UB <= cnt; k0 += UB) {
+            float dt[UB], xv[UB], Be[UB], Bo[UB], Ce[UB], Co[UB], y[UB];
+            bool small = true;
+#pragma unroll
+            for (int q = 0; q < UB; q++) {
+                dt[q] = r_dt[k0 + q];
+                xv[q] = r_xb[k0 + q];
+                Be[q] = r_Be[k0 + q];
+                Bo[q] = r_Bo[k0 + q];
+                Ce[q] = OUT ? r_Ce[k0 + q] : 0.0f;
+                Co[q] = OUT ? r_Co[k0 + q] : 0.0f;
+                small = small && (sg_abs(dt[q] * freq) < SG_SINCOS_SMALL_LIMIT);
+            }
+            if (__builtin_amdgcn_ballot_w64(!small) == 0)
+                block_steps<OUT, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+            else
+                block_steps<OUT, false>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+            if (OUT && p == 0) {
+#pragma unroll
+                for (int q = 0; q < UB; q++) s_y[j * LDS_STRIDE + k0 + q] = y[q];
+            }
+        }
+        for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
+            const float dt = r_dt[k0], xv = r_xb[k0];
             float ae, ao, sn, cs;
             sg_abar_pair(dt, hAe, hAo, &ae, &ao);
             sg_sincos(dt * freq, &sn, &cs);
-            const float be = (dt * r_Be[k]) * xv, bo = (dt * r_Bo[k]) * xv;
+            step_update<OUT>(S, ae, ao, sn, cs, (dt * r_Be[k0]) * xv, (dt * r_Bo[k0]) * xv);
             if (OUT) {
-                const float re = sg_fma(he, cs, -(ho * sn));
-                const float ro = sg_fma(ho, cs, he * sn);
-                he = sg_fma(ae, re, be);
-                ho = sg_fma(ao, ro, bo);
-                float y = sg_fma(ho, r_Co[k], he * r_Ce[k]);
-                y = y + dpp_quad_swap1(y);
-                y = y + dpp_quad_swap2(y);
-                y = y + dpp_half_mirror(y);
-                if (p == 0) s_y[j * LDS_STRIDE + k] = y;
-            } else {
-                float re = sg_fma(c0e, cs, -(c0o * sn)), ro = sg_fma(c0o, cs, c0e * sn);
-                c0e = ae * re;
-                c0o = ao * ro;
-                re = sg_fma(c1e, cs, -(c1o * sn));
-                ro = sg_fma(c1o, cs, c1e * sn);
-                c1e = ae * re;
-                c1o = ao * ro;
-                re = sg_fma(he, cs, -(ho * sn));
-                ro = sg_fma(ho, cs, he * sn);
-                he = sg_fma(ae, re, be);
-                ho = sg_fma(ao, ro, bo);
+                const float y = pair_tree_sum(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
+                if (p == 0) s_y[j * LDS_STRIDE + k0] = y;
             }
         }
         __syncthreads();
@@ -218,10 +282,14 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
             float cx[DM / 2];
 #pragma unroll
             for (int q = 0; q < DM / 2; q++) {
-                const int dd = half * (DM / 2) + q;
                 float a = 0.0f;
+                if (half == 0) {
 #pragma unroll
-                for (int jj = 0; jj < DI; jj++) a = sg_fma(w.out_proj[dd * DI + jj], o[jj], a);
+                    for (int jj = 0; jj < DI; jj++) a = sg_fma(w.out_proj[q * DI + jj], o[jj], a);
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < DI; jj++) a = sg_fma(w.out_proj[(DM / 2 + q) * DI + jj], o[jj], a);
+                }
                 cx[q] = a;
             }
             if (valid) {
@@ -235,45 +303,79 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
     if (OUT) {
         if (u1 == N) {   // last chunk in scan order: new carried state of the tensor
             float* st = dir ? T.mbwd : T.mfwd;
-            st[j * DS + 2 * p] = he;
-            st[j * DS + 2 * p + 1] = ho;
+            st[j * DS + 2 * p] = S.he;
+            st[j * DS + 2 * p + 1] = S.ho;
         }
     } else {
         float* sm = pl.summaries + (size_t)(dir * pl.wchunks + cidx) * 6 * SCAN_THREADS;
-        sm[0 * SCAN_THREADS + tid] = c0e;   // M = [c0e c1e; c0o c1o]
-        sm[1 * SCAN_THREADS + tid] = c0o;
-        sm[2 * SCAN_THREADS + tid] = c1e;
-        sm[3 * SCAN_THREADS + tid] = c1o;
-        sm[4 * SCAN_THREADS + tid] = he;
-        sm[5 * SCAN_THREADS + tid] = ho;
+        sm[0 * SCAN_THREADS + tid] = S.c0e;   // M = [c0e c1e; c0o c1o]
+        sm[1 * SCAN_THREADS + tid] = S.c0o;
+        sm[2 * SCAN_THREADS + tid] = S.c1e;
+        sm[3 * SCAN_THREADS + tid] = S.c1o;
+        sm[4 * SCAN_THREADS + tid] = S.he;
+        sm[5 * SCAN_THREADS + tid] = S.ho;
     }
 }
 
-// start state of every chunk: h_{c+1} = M_c h_c + b_c, from the carried state
-__global__ __launch_bounds__(SCAN_THREADS) void k_chunk_prefix(Plan pl) {
+// Start state of every chunk: h_{c+1} = M_c h_c + b_c, applied in order from
+// the carried state of the tensor.  One workgroup per (tensor, direction).
+// The recurrence itself is a handful of fmas per chunk; what matters is the
+// latency of fetching 3 KB of summaries per chunk, so eight 128-lane groups
+// stream batches of 32 chunks into LDS (next batch prefetched into registers)
+// and group 0 applies them.
+constexpr int PREFIX_GROUPS = 8;
+constexpr int PREFIX_BATCH = 32;
+constexpr int PREFIX_PER_GROUP = PREFIX_BATCH / PREFIX_GROUPS;
+
+__global__ __launch_bounds__(PREFIX_GROUPS * SCAN_THREADS) void k_chunk_prefix(Plan pl) {
+    __shared__ float lds[PREFIX_BATCH * 6 * SCAN_THREADS];     // 96 KB
     const int ti = blockIdx.x % pl.P, dir = blockIdx.x / pl.P;
     const TensorDev& T = pl.tensors[ti];
     if (T.numel == 0) return;
-    const int tid = threadIdx.x, j = tid >> 3, p = tid & 7;
-    const float* st = dir ? T.mbwd : T.mfwd;
-    float he = st[j * DS + 2 * p], ho = st[j * DS + 2 * p + 1];
-    float* hs = pl.hstart + ((size_t)(dir * pl.chunks + pl.chunk_prefix[ti]) * 2) * SCAN_THREADS;
-    const float* sm = pl.summaries + (size_t)(dir * pl.wchunks + pl.wchunk_prefix[ti]) * 6 * SCAN_THREADS;
-    hs[tid] = he;
-    hs[SCAN_THREADS + tid] = ho;
-    const int nc = T.nchunks;
-#pragma unroll 4
-    for (int c = 0; c + 1 < nc; c++) {
-        const float* m = sm + (size_t)c * 6 * SCAN_THREADS;
-        const float m0 = m[tid], m1 = m[SCAN_THREADS + tid], m2 = m[2 * SCAN_THREADS + tid];
-        const float m3 = m[3 * SCAN_THREADS + tid], m4 = m[4 * SCAN_THREADS + tid], m5 = m[5 * SCAN_THREADS + tid];
-        const float ne = sg_fma(m0, he, sg_fma(m2, ho, m4));
-        const float no = sg_fma(m1, he, sg_fma(m3, ho, m5));
-        he = ne;
-        ho = no;
-        float* h1 = hs + (size_t)(c + 1) * 2 * SCAN_THREADS;
-        h1[tid] = he;
-        h1[SCAN_THREADS + tid] = ho;
+    const int lane = threadIdx.x % SCAN_THREADS, grp = threadIdx.x / SCAN_THREADS;
+    const int j = lane >> 3, p = lane & 7;
+    float* __restrict__ hs = pl.hstart + ((size_t)(dir * pl.chunks + pl.chunk_prefix[ti]) * 2) * SCAN_THREADS;
+    const float* __restrict__ sm = pl.summaries + (size_t)(dir * pl.wchunks + pl.wchunk_prefix[ti]) * 6 * SCAN_THREADS;
+    const int ns = T.nchunks - 1;                               // summaries to apply
+    float he = 0.0f, ho = 0.0f;
+    if (grp == 0) {
+        const float* st = dir ? T.mbwd : T.mfwd;
+        he = st[j * DS + 2 * p];
+        ho = st[j * DS + 2 * p + 1];
+        hs[lane] = he;
+        hs[SCAN_THREADS + lane] = ho;
+    }
+    float r[PREFIX_PER_GROUP][6];
+    auto prefetch = [&](int b) {
+#pragma unroll
+        for (int q = 0; q < PREFIX_PER_GROUP; q++) {
+            const int c = b * PREFIX_BATCH + grp + PREFIX_GROUPS * q;
+#pragma unroll
+            for (int k = 0; k < 6; k++) r[q][k] = (c < ns) ? sm[((size_t)c * 6 + k) * SCAN_THREADS + lane] : 0.0f;
+        }
+    };
+    prefetch(0);
+    for (int b = 0; b * PREFIX_BATCH < ns; b++) {
+#pragma unroll
+        for (int q = 0; q < PREFIX_PER_GROUP; q++)
+#pragma unroll
+            for (int k = 0; k < 6; k++) lds[((grp + PREFIX_GROUPS * q) * 6 + k) * SCAN_THREADS + lane] = r[q][k];
+        __syncthreads();
+        prefetch(b + 1);
+        if (grp == 0) {
+            const int lim = min(PREFIX_BATCH, ns - b * PREFIX_BATCH);
+            for (int cc = 0; cc < lim; cc++) {
+                const float* m = lds + cc * 6 * SCAN_THREADS + lane;
+                const float ne = sg_fma(m[0], he, sg_fma(m[2 * SCAN_THREADS], ho, m[4 * SCAN_THREADS]));
+                const float no = sg_fma(m[SCAN_THREADS], he, sg_fma(m[3 * SCAN_THREADS], ho, m[5 * SCAN_THREADS]));
+                he = ne;
+                ho = no;
+                float* h1 = hs + (size_t)(b * PREFIX_BATCH + cc + 1) * 2 * SCAN_THREADS;
+                h1[lane] = he;
+                h1[SCAN_THREADS + lane] = ho;
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -286,7 +388,7 @@ int launch_scan(const Plan& pl, hipStream_t st) {
         SG_LAUNCH_CHECK("k_scan<summary>");
     }
     prof_mark(2, st);
-    hipLaunchKernelGGL(k_chunk_prefix, dim3(2 * pl.P), dim3(SCAN_THREADS), 0, st, pl);
+    hipLaunchKernelGGL(k_chunk_prefix, dim3(2 * pl.P), dim3(PREFIX_GROUPS * SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_chunk_prefix");
     prof_mark(3, st);
     hipLaunchKernelGGL(k_scan<true>, dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);

@@ -59,8 +59,18 @@ __device__ __forceinline__ void store_elem(void* p, int dtype, int64_t i, float 
 }
 __device__ __forceinline__ float finite_or_zero(float v) { return sg_isfinite(v) ? v : 0.0f; }
 
+// Read-only tables and weights are read through the constant address space: a
+// wave-uniform index then becomes a scalar load (s_load_dword*), which the
+// compiler will not emit for plain global pointers in a kernel that also
+// stores to global memory.  Only for memory no kernel of the same launch writes.
+typedef const __attribute__((address_space(4))) float* cfloat_p;
+typedef const __attribute__((address_space(4))) int* cint_p;
+__device__ __forceinline__ cfloat_p as_const(const float* p) { return (cfloat_p)p; }
+__device__ __forceinline__ cint_p as_const(const int* p) { return (cint_p)p; }
+
 // largest i in [0, n) with prefix[i] <= x   (prefix is non-decreasing, prefix[0] == 0)
-__device__ __forceinline__ int upper_seg(const int* __restrict__ prefix, int n, int x) {
+template <class P>
+__device__ __forceinline__ int upper_seg(P prefix, int n, int x) {
     int lo = 0, hi = n;
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;

@@ -71,6 +71,16 @@ def test_sincos():
     assert L.orc_sin(0.0) == 0.0 and L.orc_cos(0.0) == 1.0
 
 
+def test_small_angle_sincos_is_bitwise_the_general_one():
+    xs = np.concatenate([RNG.uniform(-0.78, 0.78, 50000), RNG.uniform(-1e-3, 1e-3, 5000),
+                         [0.0, -0.0, 0.7799999, -0.7799999, 1e-30, -1e-30]]).astype(np.float32)
+    for x in xs:
+        x = float(x)
+        assert abs(x) < 0.78
+        assert np.float32(L.orc_sin_small(x)).tobytes() == np.float32(L.orc_sin(x)).tobytes(), x
+        assert np.float32(L.orc_cos_small(x)).tobytes() == np.float32(L.orc_cos(x)).tobytes(), x
+
+
 def test_rcp_and_abar():
     ds = np.exp(RNG.uniform(0, 60, 20000))
     assert _maxrel(L.orc_rcp_pos, lambda d: 1.0 / d, ds) < 1.5e-7
