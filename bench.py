@@ -76,13 +76,83 @@ def cpu_baseline(sample_elems_target=1_000_000):
                       "fp32 C++ restatement, %.1f s" % (pick[0], pick[-1], tot, dt)}
 
 
+def bench_other(args, dev):
+    """Secondary measurements: the Grokfast, SuperGrok v1.5 and Muon fused steps through `_ops`."""
+    import torch
+    import workloads as wl
+    from grokking_optimizers import _ops
+    K, Wm = args.steps, args.warmup
+    if args.workload == "muon":
+        shapes = [(1024, 4096)] * 12 + [(4096, 1024)] * 12
+        gen = torch.Generator().manual_seed(0)
+        params = [(torch.randn(*s, generator=gen) * 0.02).to(torch.bfloat16).to(dev) for s in shapes]
+        grads = [(torch.randn(*s, generator=gen) * 1e-3).to(torch.bfloat16).to(dev) for s in shapes]
+        bufs = [torch.zeros(s, device=dev) for s in shapes]
+        step = lambda: _ops.muon_fused_step(params, grads, bufs, 0.95, 0.02, 1.0, 5)
+        units, unit = 5 * sum(6 * min(s) ** 2 * max(s) for s in shapes), "FLOP/s"      # 6 min^2 max per NS iteration
+        name, dtype, bound, peak = "Muon step, 12x[1024,4096] + 12x[4096,1024], 5 Newton-Schulz iterations", "bf16", "mfma", 2500.0
+    else:
+        shapes = wl.shared14_shapes()
+        params = [p.reshape(-1).to(dev) for p in wl.make_params(shapes, seed=0)]
+        grads0 = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.01 if args.workload == "sg15" else 0.0)]
+        z = lambda: [torch.zeros_like(p) for p in params]
+        n = sum(p.numel() for p in params)
+        if args.workload == "grokfast":
+            emas, ms, vs = z(), z(), z()
+            grads = [g.clone() for g in grads0]
+            t = [0]
+
+            def step():
+                t[0] += 1
+                _ops.grokfast_adamw_fused_step(params, grads, emas, ms, vs, [t[0]] * len(params), 0.98, 2.0, 1e-3, 0.9, 0.98, 1e-8, 1.0)
+            name = "Grokfast fused step (EMA + amplify + AdamW), 14 tensors, %d elements" % n
+        else:
+            eas, easqs, mus, sharps = z(), z(), z(), z()
+            gen = torch.Generator().manual_seed(3)
+            H = 32
+            W1, b1 = (torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev)
+            W2, b2 = (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)
+            grads = [g.clone() for g in grads0]
+            P = len(params)
+
+            def step():
+                _ops.supergrok15_fused_step(params, grads, eas, easqs, mus, sharps, [0] * P, [0.98] * P,
+                                            [0.9 * 0.9 ** i for i in range(P)], W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8,
+                                            2.0, 1.0, 0.5, 1.0)
+            name = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip), 14 tensors, %d elements" % n
+        units, unit, dtype, bound, peak = n, "elements/s", "f32", "hbm", HBM_PEAK_GBS
+    for _ in range(Wm):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(K):
+        step()
+    torch.cuda.synchronize()
+    el = (time.perf_counter() - t0) / K
+    out = {"metric": "secondary: " + args.workload, "value": units / el, "unit": unit, "n_gpus": 1, "steps": K, "warmup": Wm,
+           "ms_per_step": 1e3 * el, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+           "data": "synthetic", "config": {"workload": name}}
+    if bound == "mfma":
+        out["roofline"] = {"bound": "mfma", "achieved": units / el / 1e12, "peak": peak, "unit": "TFLOP/s",
+                           "frac": units / el / 1e12 / peak, "traffic": None}
+    else:
+        out["roofline"] = {"bound": "hbm", "achieved": 40 * units / el / 1e9, "peak": peak, "unit": "GB/s",
+                           "frac": 40 * units / el / 1e9 / peak, "traffic": None}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14"])
+    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon"],
+                    help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
+                         "grokfast / sg15 / muon time the other fused steps of BASELINE configs 1, 2 and 5")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain device copy of 1 GiB (a reference point for scaling the FETCH_SIZE / "
+                         "WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box here has one GPU and the path uses no collectives; "
@@ -94,11 +164,20 @@ def main():
     from sg2_harness import per_tensor_scalars, shared_scalars
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
+    if args.workload in ("grokfast", "sg15", "muon"):
+        print(json.dumps(bench_other(args, dev)))
+        return
     shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev)
     total = sum(p.numel() for p in st["params"])
     step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
                          st["counts"])
     shared = shared_scalars()
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     t = 0
     for _ in range(args.warmup):
         t += 1

@@ -68,7 +68,8 @@ struct Plan {
     int elem_tiles, sort_tiles, chunks, wchunks;
     int chunk_len;
     uint32_t* keys[2];
-    int32_t* vals[2];
+    int32_t* vals[2];              // element index within the tensor | sign bit of the gradient in bit 31
+    float* ssorted;                // [total] sharpness gathered into sorted order
     uint32_t* spine;               // [256 * sort_tiles] per-tile digit counts, layout [segment][digit][tile]
     uint32_t* blocksums;
     float* summaries;              // [2][wchunks][6][128]
@@ -81,7 +82,7 @@ struct Plan {
 // records a profiling event (no-op unless profiling is enabled)
 void prof_mark(int idx, hipStream_t st);
 
-int launch_sort(const Plan& pl, hipStream_t st);
+int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st);
 int launch_scan(const Plan& pl, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
 

@@ -21,6 +21,9 @@
 // Per-timestep projections (in_proj, dt, B, C) are recomputed in both passes
 // for tiles of 64 timesteps and staged through LDS instead of being
 // materialised in HBM (the reference writes 320 B per element per direction).
+// The inputs of a timestep come coalesced from the sort's own output: the key
+// is |g|, the payload carries the sign of g and the element index, and the
+// sharpness has been gathered into sorted order once.
 //
 // The kernels are bound by fp32 VALU issue, not by HBM: per (timestep, column,
 // pair) one shared reciprocal, one sin/cos pair and the 2x2 update.  The
@@ -36,7 +39,15 @@ namespace sg2 {
 namespace {
 
 constexpr int LDS_STRIDE = SCAN_TT + 1;   // [row][timestep] rows padded so the 8 rows a wave reads sit in 8 banks
-constexpr int UB = 8;                     // timesteps per unrolled block of the recurrence
+#ifndef SG2_SCAN_UB
+#define SG2_SCAN_UB 8
+#endif
+constexpr int UB = SG2_SCAN_UB;           // timesteps per unrolled block of the recurrence
+#ifdef SG2_SCAN_WAVES
+#define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
+#else
+#define SG2_SCAN_ATTR
+#endif
 
 struct DirW {
     sg::cfloat_p in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj;
@@ -163,7 +174,7 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
 }
 
 template <bool OUT>
-__global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
+__global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     __shared__ float s_dt[DI * LDS_STRIDE];
     __shared__ float s_xb[DI * LDS_STRIDE];
     __shared__ float s_B[DS * LDS_STRIDE];
@@ -178,13 +189,13 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
     const int ti = sg::upper_seg(prefix, pl.P, cidx);
     const int c = cidx - prefix[ti];                       // chunk within the tensor
     const TensorDev& T = pl.tensors[ti];
-    const int N = T.numel, dtype = T.dtype, off = T.off;
-    const void* const t_grad = T.grad;
-    const void* const t_sharp = T.sharp;
+    const int N = T.numel, off = T.off;
     const int u0 = c * pl.chunk_len;                       // first scan step of the chunk
     const int u1 = min(u0 + pl.chunk_len, N);
     const DirW w = dir_weights(pl.W, dir);
-    const int32_t* __restrict__ perm = pl.vals[0] + off;
+    const uint32_t* __restrict__ skey = pl.keys[0] + off;      // sorted |g| bits
+    const int32_t* __restrict__ sval = pl.vals[0] + off;       // element index | sign of g
+    const float* __restrict__ ssrt = pl.ssorted + off;          // sharpness in sorted order
     const sg::cfloat_p Wi = sg::as_const(pl.W.w[W_IN_W]);
     const sg::cfloat_p bi = sg::as_const(pl.W.w[W_IN_B]);
 
@@ -215,10 +226,11 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_scan(Plan pl) {
             float g = 0.0f, s = 0.0f;
             if (valid) {
                 const int t = dir ? (N - 1 - u) : u;
-                orig = perm[t];
+                const int32_t v = sval[t];
+                orig = v & 0x7fffffff;
                 orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
-                g = sg::finite_or_zero(sg::load_elem(t_grad, dtype, orig));
-                s = sg::finite_or_zero(sg::load_elem(t_sharp, dtype, orig));
+                g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
+                s = ssrt[t];
             }
 #pragma unroll
             for (int k = 0; k < DM; k++) x[k] = sg_fma(Wi[2 * k + 1], s, Wi[2 * k] * g) + bi[k];

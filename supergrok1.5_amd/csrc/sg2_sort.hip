@@ -36,8 +36,10 @@ __global__ __launch_bounds__(256) void k_keys(Plan pl) {
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int i = start + k;
         const float g = sg::finite_or_zero(sg::load_elem(T.grad, T.dtype, i));
+        // key = |g| bits; the sign rides in bit 31 of the payload so that the sorted (key, payload)
+        // pair gives back g exactly and the scan never has to gather gradients from element order
         pl.keys[0][T.off + i] = (uint32_t)sg_f2i(sg_abs(g));
-        pl.vals[0][T.off + i] = i;
+        pl.vals[0][T.off + i] = i | (sg_f2i(g) & (int32_t)0x80000000);
     }
 }
 
@@ -206,9 +208,26 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
     }
 }
 
+// After the sort: sharpness gathered into sorted order (one random read per element, once, instead of
+// one per scan pass and direction), and optionally the plain permutation for inspection.
+__global__ __launch_bounds__(256) void k_gather_sorted(Plan pl, int32_t* __restrict__ dbg_perm) {
+    const int tile = blockIdx.x;
+    const int ti = sg::upper_seg(sg::as_const(pl.elem_tile_prefix), pl.P, tile);
+    const TensorDev& T = pl.tensors[ti];
+    const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
+    const int cnt = min(ELEM_TILE, T.numel - start);
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int t = T.off + start + k;
+        int idx = pl.vals[0][t] & 0x7fffffff;
+        idx = ((unsigned)idx < (unsigned)T.numel) ? idx : 0;       // never index outside the tensor
+        pl.ssorted[t] = sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, idx));
+        if (dbg_perm) dbg_perm[t] = idx;
+    }
+}
+
 }  // namespace
 
-int launch_sort(const Plan& pl, hipStream_t st) {
+int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st) {
     if (pl.total == 0) return 0;
     hipLaunchKernelGGL(k_keys, dim3(pl.elem_tiles), dim3(256), 0, st, pl);
     SG_LAUNCH_CHECK("k_keys");
@@ -223,7 +242,10 @@ int launch_sort(const Plan& pl, hipStream_t st) {
         hipLaunchKernelGGL(k_scatter, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
         SG_LAUNCH_CHECK("radix pass");
     }
-    return 0;   // result is back in keys[0] / vals[0]
+    // result is back in keys[0] / vals[0]
+    hipLaunchKernelGGL(k_gather_sorted, dim3(pl.elem_tiles), dim3(256), 0, st, pl, dbg_perm);
+    SG_LAUNCH_CHECK("k_gather_sorted");
+    return 0;
 }
 
 }  // namespace sg2

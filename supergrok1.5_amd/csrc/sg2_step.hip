@@ -24,7 +24,7 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_spine, off_blocksums, off_summ, off_hstart, off_ctx, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_ctx, bytes;
     size_t tables_bytes;
 };
 
@@ -51,6 +51,7 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
     L->off_tables = take(L->tables_bytes);
     for (int k = 0; k < 2; k++) L->off_keys[k] = take(4 * (size_t)total);
     for (int k = 0; k < 2; k++) L->off_vals[k] = take(4 * (size_t)total);
+    L->off_ssorted = take(4 * (size_t)total);
     L->off_spine = take(4 * 256 * (size_t)stl);
     L->off_blocksums = take(4 * (size_t)(L->nb + 1));
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * SCAN_THREADS);
@@ -206,6 +207,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
         pl.keys[k] = reinterpret_cast<uint32_t*>(ws + L.off_keys[k]);
         pl.vals[k] = reinterpret_cast<int32_t*>(ws + L.off_vals[k]);
     }
+    pl.ssorted = reinterpret_cast<float*>(ws + L.off_ssorted);
     pl.spine = reinterpret_cast<uint32_t*>(ws + L.off_spine);
     pl.blocksums = reinterpret_cast<uint32_t*>(ws + L.off_blocksums);
     pl.summaries = reinterpret_cast<float*>(ws + L.off_summ);
@@ -216,10 +218,8 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.W = *weights;
 
     prof_mark(0, st);
-    if (launch_sort(pl, st)) return 1;
+    if (launch_sort(pl, debug ? debug->perm : nullptr, st)) return 1;
     prof_mark(1, st);
-    if (debug && debug->perm)
-        SG_HIP_CHECK(hipMemcpyAsync(debug->perm, pl.vals[0], 4 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
     if (launch_scan(pl, st)) return 1;
     if (debug && debug->ctx)
         SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * DM, hipMemcpyDeviceToDevice, st));
