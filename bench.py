@@ -19,6 +19,10 @@ for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd"), os.path.join(ROOT, "test
 
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch (read + written) on the 25M-element workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs scaled by a 1 GiB copy (profiles/sg2_step_scale50_pmc_traffic.txt); not measured by this script
+PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.675e9 + 1.626e9, "scan_summary": 0.619e9 + 0.150e9,
+                             "elementwise": 2.603e9 + 0.801e9}
 FLOP_PER_ELEMENT = 30e3         # arithmetic actually required per element (both scan directions + elementwise)
 VALU_PEAK_TFLOPS = 157.3
 
@@ -214,7 +218,8 @@ def main():
                                % (len(shapes), total, "BASELINE configs[3]" if args.workload == "scale50" else "configs[2] set"),
                    "chunk_len": _cabi.lib().sg2_get_chunk_len()},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if args.workload == "scale50" else None,
                      "kernel_ms": stage_avg[dom]},
         "step_hbm_frac": BYTES_PER_ELEMENT * value / 1e9 / HBM_PEAK_GBS,
         "step_valu_frac": FLOP_PER_ELEMENT * value / 1e12 / VALU_PEAK_TFLOPS,
