@@ -153,6 +153,8 @@ def main():
     ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps of BASELINE configs 1, 2 and 5")
+    ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
+    ap.add_argument("--window", type=int, default=-1, help="scan summary window (-1: library default, 0: off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 1 GiB (a reference point for scaling the FETCH_SIZE / "
@@ -171,6 +173,8 @@ def main():
     if args.workload in ("grokfast", "sg15", "muon"):
         print(json.dumps(bench_other(args, dev)))
         return
+    if _cabi.lib().sg2_set_chunk_len(args.chunk_len) or _cabi.lib().sg2_set_scan_window(args.window):
+        raise SystemExit(_cabi.last_error())
     shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev)
     total = sum(p.numel() for p in st["params"])
     step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
@@ -216,7 +220,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SuperGrok v2 full step, %d tensors, %d elements (%s), fp32, bilevel off"
                                % (len(shapes), total, "BASELINE configs[3]" if args.workload == "scale50" else "configs[2] set"),
-                   "chunk_len": _cabi.lib().sg2_get_chunk_len()},
+                   "chunk_len": _cabi.chunk_len_for([p.numel() for p in st["params"]]), "summary_window": _cabi.lib().sg2_get_scan_window()},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if args.workload == "scale50" else None,

@@ -81,10 +81,22 @@ typedef struct Sg2Debug {
 const char* sg_last_error(void);
 
 /* Length (timesteps) of the scan chunks a tensor's sorted sequence is cut
- * into; a multiple of 64.  0 restores the default (1024).  Affects results
- * only by re-association of the chunk products. */
+ * into; a multiple of 64.  0 (the default) lets each call choose 4096, 2048
+ * or 1024 from the amount of work; sg2_chunk_len_for tells what a call with
+ * these tensor sizes will use.  Affects results only by re-association of the
+ * chunk products. */
 int sg2_set_chunk_len(int chunk_len);
 int sg2_get_chunk_len(void);
+int sg2_chunk_len_for(int num_tensors, const int64_t* numels);
+
+/* Summary window of the scan (timesteps, a multiple of 64; 0 disables, a
+ * negative value restores the default 256).  The recurrence contracts, so the
+ * 2x2 part of a chunk summary taken over only its last `window` steps is
+ * normally far below fp32 resolution; when every entry is below 2^-100 the
+ * chunk summary is (0, b_window), otherwise the whole chunk is accumulated.
+ * Takes effect when window < chunk_len. */
+int sg2_set_scan_window(int window);
+int sg2_get_scan_window(void);
 
 /* Bytes of scratch the batched step needs for these tensor sizes. */
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);

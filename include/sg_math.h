@@ -162,18 +162,19 @@ SG_HD float sg_rcp_pos(float d) {
 
 /* Trapezoidal discretisation for the two states of one RoPE pair:
  *   A_bar = (1 + dt*A/2) / (1 - dt*A/2 + 1e-8)
- * hA_e and hA_o are A/2 (exact halving).  A < 0 and dt >= 0, so the
- * denominator is >= 1 and the "+1e-8f" of the reference is below half an ulp
- * of it: adding it never changes an fp32 value >= 1, so it is dropped.  One shared reciprocal
- * serves both members of the pair. */
-SG_HD void sg_abar_pair(float dt, float hA_e, float hA_o, float* ab_e, float* ab_o) {
-    const float n_e = sg_fma(dt, hA_e, 1.0f);
-    const float d_e = sg_fma(-dt, hA_e, 1.0f);
-    const float n_o = sg_fma(dt, hA_o, 1.0f);
-    const float d_o = sg_fma(-dt, hA_o, 1.0f);
+ * With t = -dt*A/2 >= 0 (A < 0, dt >= 0) this is (1-t)/(1+t) = 2/(1+t) - 1.
+ * nhA_e and nhA_o are -A/2 (exact halving and negation).  The denominator is
+ * >= 1, so the "+1e-8f" of the reference is below half an ulp of it: adding it
+ * never changes an fp32 value >= 1, and it is dropped.  One shared reciprocal
+ * serves both members of the pair:
+ *   r = 1/((1+t_e)(1+t_o));  A_bar_e = 2 r (1+t_o) - 1;  A_bar_o = 2 r (1+t_e) - 1. */
+SG_HD void sg_abar_pair(float dt, float nhA_e, float nhA_o, float* ab_e, float* ab_o) {
+    const float d_e = sg_fma(dt, nhA_e, 1.0f);
+    const float d_o = sg_fma(dt, nhA_o, 1.0f);
     const float r = sg_rcp_pos(d_e * d_o);
-    *ab_e = (n_e * d_o) * r;
-    *ab_o = (n_o * d_e) * r;
+    const float r2 = r + r;
+    *ab_e = sg_fma(d_o, r2, -1.0f);
+    *ab_o = sg_fma(d_e, r2, -1.0f);
 }
 
 SG_HD float sg_tanh(float x) {

@@ -63,7 +63,7 @@ def sort_perm(g):
     return perm
 
 
-def sg2_step(weights, state, grad, sharp, scalars, dims=None, precision=32, chunk_len=0,
+def sg2_step(weights, state, grad, sharp, scalars, dims=None, precision=32, chunk_len=0, window=0,
              expert_counts=None, debug=False):
     """One SuperGrok v2 step on one tensor, in place on `state`.
 
@@ -97,7 +97,7 @@ def sg2_step(weights, state, grad, sharp, scalars, dims=None, precision=32, chun
         out["margin"] = np.empty((N, H, 2), np.float32)
         out["smart"] = np.empty(N, np.float32)
     rc = L.orc_sg2_step(
-        C.c_int(precision), C.c_int64(chunk_len), warr, _ptr(darr), C.c_int(dtype),
+        C.c_int(precision), C.c_int64(chunk_len), C.c_int64(window), warr, _ptr(darr), C.c_int(dtype),
         _ptr(state["param"]), _ptr(grad), _ptr(sharp), _ptr(state["exp_avg"]),
         _ptr(state["exp_avg_sq"]), _ptr(state["mu"]), _ptr(state["gru"]),
         _ptr(state["mamba_fwd"]), _ptr(state["mamba_bwd"]), C.c_int64(N), _ptr(sarr),

@@ -46,15 +46,15 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
     }
     __syncthreads();
 
-    const sg::cfloat_p Wz = sg::as_const(pl.W.w[W_GRU_WZ]);
-    const sg::cfloat_p bz = sg::as_const(pl.W.w[W_GRU_BZ]);
-    const sg::cfloat_p Wr = sg::as_const(pl.W.w[W_GRU_WR]);
-    const sg::cfloat_p br = sg::as_const(pl.W.w[W_GRU_BR]);
-    const sg::cfloat_p Wh = sg::as_const(pl.W.w[W_GRU_WH]);
-    const sg::cfloat_p bh = sg::as_const(pl.W.w[W_GRU_BH]);
-    const sg::cfloat_p Wq = sg::as_const(pl.W.w[W_PEER_Q]);
-    const sg::cfloat_p KA = sg::as_const(pl.W.w[W_KEYS_A]);
-    const sg::cfloat_p KB = sg::as_const(pl.W.w[W_KEYS_B]);
+    const sg::cfloat_p Wz0 = sg::as_const(pl.W.w[W_GRU_WZ]);
+    const sg::cfloat_p bz0 = sg::as_const(pl.W.w[W_GRU_BZ]);
+    const sg::cfloat_p Wr0 = sg::as_const(pl.W.w[W_GRU_WR]);
+    const sg::cfloat_p br0 = sg::as_const(pl.W.w[W_GRU_BR]);
+    const sg::cfloat_p Wh0 = sg::as_const(pl.W.w[W_GRU_WH]);
+    const sg::cfloat_p bh0 = sg::as_const(pl.W.w[W_GRU_BH]);
+    const sg::cfloat_p Wq0 = sg::as_const(pl.W.w[W_PEER_Q]);
+    const sg::cfloat_p KA0 = sg::as_const(pl.W.w[W_KEYS_A]);
+    const sg::cfloat_p KB0 = sg::as_const(pl.W.w[W_KEYS_B]);
 
     for (int tile = blockIdx.x; tile < pl.elem_tiles; tile += gridDim.x) {
         const int ti = sg::upper_seg(sg::as_const(pl.elem_tile_prefix), pl.P, tile);
@@ -67,6 +67,10 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
 
         for (int k = threadIdx.x; k < cnt; k += ELEM_THREADS) {
             const int i = start + k;
+            // the weights are re-read (scalar loads, cache hits) for every element instead of being hoisted
+            const int zo = sg::opaque_zero();
+            const sg::cfloat_p Wz = Wz0 + zo, bz = bz0 + zo, Wr = Wr0 + zo, br = br0 + zo, Wh = Wh0 + zo, bh = bh0 + zo;
+            const sg::cfloat_p Wq = Wq0 + zo, KA = KA0 + zo, KB = KB0 + zo;
             const float g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, i));
             const float s = sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i));
             float cf[DM], cb[DM], hold[GH];

@@ -67,6 +67,7 @@ struct Plan {
     int total;                     // sum of numel
     int elem_tiles, sort_tiles, chunks, wchunks;
     int chunk_len;
+    int window;                    // summary window (0: whole chunk), see k_scan<false>
     uint32_t* keys[2];
     int32_t* vals[2];              // element index within the tensor | sign bit of the gradient in bit 31
     float* ssorted;                // [total] sharpness gathered into sorted order

@@ -11,7 +11,13 @@
 // backward one).  One 128-lane workgroup owns one chunk; lane (j,p) owns
 // column j and RoPE pair p, i.e. the two states h[j][2p], h[j][2p+1].
 //   k_scan<false>  every chunk but the last of a tensor: 2x2 affine summary
-//                  (M,b) of the chunk, accumulated from the identity.
+//                  (M,b) of the chunk, accumulated from the identity.  The
+//                  recurrence contracts (|A_bar| < 1), so the summary is first
+//                  taken over the last `window` steps only; if every |entry| of
+//                  that window's M, in all 128 lanes, is below 2^-100 the chunk
+//                  summary is (0, b_window) -- the state entering the window
+//                  is multiplied by less than 2^-100 -- otherwise the whole
+//                  chunk is accumulated.
 //   k_chunk_prefix start state of each chunk: summaries applied in order to
 //                  the carried state of the tensor.
 //   k_scan<true>   every chunk replayed from its start state: y = h.C, gate,
@@ -159,8 +165,9 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
         sg_abar_pair(dt[u], hAe, hAo, &ae[u], &ao[u]);
         if (SMALL_ANGLE) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
         else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
-        be[u] = (dt[u] * Be[u]) * xv[u];
-        bo[u] = (dt[u] * Bo[u]) * xv[u];
+        const float ux = dt[u] * xv[u];
+        be[u] = ux * Be[u];
+        bo[u] = ux * Bo[u];
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
@@ -192,7 +199,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const int N = T.numel, off = T.off;
     const int u0 = c * pl.chunk_len;                       // first scan step of the chunk
     const int u1 = min(u0 + pl.chunk_len, N);
-    const DirW w = dir_weights(pl.W, dir);
+    const DirW w0 = dir_weights(pl.W, dir);
     const uint32_t* __restrict__ skey = pl.keys[0] + off;      // sorted |g| bits
     const int32_t* __restrict__ sval = pl.vals[0] + off;       // element index | sign of g
     const float* __restrict__ ssrt = pl.ssorted + off;          // sharpness in sorted order
@@ -204,8 +211,9 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const int half = __builtin_amdgcn_readfirstlane(tid >> 6);           // projection role: which half of the outputs
     const int j = tid >> 3, p = tid & 7;                                  // scan role
 
-    const float hAe = 0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
-    const float hAo = 0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
+    // -A/2 with A = -exp(A_log): the two poles of this lane's pair
+    const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
+    const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
     const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
@@ -215,8 +223,19 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         S.ho = hs[SCAN_THREADS + tid];
     }
 
-    for (int tile0 = u0; tile0 < u1; tile0 += SCAN_TT) {
+    int first = u0;
+    bool windowed = false;
+    if (!OUT && pl.window > 0 && pl.window < pl.chunk_len) {
+        first = u1 - pl.window;
+        windowed = true;
+    }
+    for (;;) {
+    for (int tile0 = first; tile0 < u1; tile0 += SCAN_TT) {
         const int cnt = min(SCAN_TT, u1 - tile0);
+        // the projection weights are re-read (scalar loads, cache hits) in every tile instead of being hoisted
+        const int zo = sg::opaque_zero();
+        const DirW w = {w0.in_proj + zo, w0.dt_W + zo, w0.dt_b + zo, w0.Bp + zo, w0.Cp + zo,
+                        w0.A_log + zo, w0.D + zo, w0.rope + zo, w0.out_proj + zo};
         // ---------------- phase A: projections of SCAN_TT timesteps -> LDS
         const int u = tile0 + tu;
         const bool valid = u < u1;
@@ -276,7 +295,8 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             float ae, ao, sn, cs;
             sg_abar_pair(dt, hAe, hAo, &ae, &ao);
             sg_sincos(dt * freq, &sn, &cs);
-            step_update<OUT>(S, ae, ao, sn, cs, (dt * r_Be[k0]) * xv, (dt * r_Bo[k0]) * xv);
+            const float ux = dt * xv;
+            step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             if (OUT) {
                 const float y = pair_tree_sum(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
                 if (p == 0) s_y[j * LDS_STRIDE + k0] = y;
@@ -310,6 +330,18 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             }
             __syncthreads();
         }
+    }
+    if (OUT || !windowed) break;
+    {   // did the window contract?  (a NaN counts as "no")
+        const float mx = sg_max(sg_max(sg_abs(S.c0e), sg_abs(S.c0o)), sg_max(sg_abs(S.c1e), sg_abs(S.c1o)));
+        if (!__syncthreads_or(!(mx < 7.888609052210118e-31f))) {
+            S.c0e = S.c0o = S.c1e = S.c1o = 0.0f;
+            break;
+        }
+        windowed = false;
+        first = u0;
+        S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
+    }
     }
 
     if (OUT) {

@@ -12,7 +12,21 @@
 namespace sg2 {
 namespace {
 
-int g_chunk_len = 1024;
+int g_chunk_len = 0;      // 0: chosen per call from the amount of work, see auto_chunk_len
+int g_window = 256;
+
+// Longer chunks mean fewer summaries (less work in the first scan pass and the prefix), shorter chunks
+// mean more workgroups.  Take the longest of 4096 / 2048 / 1024 that still gives the replay pass about
+// four full waves of workgroups on 256 CUs.
+int auto_chunk_len(int P, const int64_t* numels) {
+    for (int L = 4096; L > 1024; L >>= 1) {
+        int64_t wgs = 0;
+        for (int i = 0; i < P; i++) wgs += 2 * ((numels[i] + L - 1) / L);
+        if (wgs >= 8192) return L;
+    }
+    return 1024;
+}
+int effective_chunk_len(int P, const int64_t* numels) { return g_chunk_len > 0 ? g_chunk_len : auto_chunk_len(P, numels); }
 
 // ---- optional per-stage timing with HIP events on the step's stream
 constexpr int PROF_MARKS = SG2_PROF_STAGES + 1;
@@ -121,17 +135,28 @@ int sg2_profile_read(float* ms, int* calls) {
 const char* sg_last_error(void) { return sg::last_error().c_str(); }
 
 int sg2_set_chunk_len(int chunk_len) {
-    if (chunk_len == 0) chunk_len = 1024;
-    if (chunk_len < sg2::SCAN_TT || chunk_len % sg2::SCAN_TT) return sg::fail("chunk_len must be a positive multiple of %d", sg2::SCAN_TT);
+    if (chunk_len < 0 || chunk_len % sg2::SCAN_TT) return sg::fail("chunk_len must be 0 (automatic) or a positive multiple of %d", sg2::SCAN_TT);
     sg2::g_chunk_len = chunk_len;
     return 0;
 }
 int sg2_get_chunk_len(void) { return sg2::g_chunk_len; }
+int sg2_chunk_len_for(int num_tensors, const int64_t* numels) {
+    if (num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
+    return sg2::effective_chunk_len(num_tensors, numels);
+}
+
+int sg2_set_scan_window(int window) {
+    if (window < 0) window = 256;
+    if (window % sg2::SCAN_TT) return sg::fail("scan window must be a multiple of %d (0 disables it)", sg2::SCAN_TT);
+    sg2::g_window = window;
+    return 0;
+}
+int sg2_get_scan_window(void) { return sg2::g_window; }
 
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;
-    if (sg2::make_layout(num_tensors, numels, sg2::g_chunk_len, &L)) return 0;
+    if (sg2::make_layout(num_tensors, numels, sg2::effective_chunk_len(num_tensors, numels), &L)) return 0;
     return L.bytes;
 }
 
@@ -159,8 +184,9 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
             if (((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
         }
     }
+    const int chunk_len = effective_chunk_len(P, numels.data());
     Layout L;
-    if (make_layout(P, numels.data(), g_chunk_len, &L)) return 1;
+    if (make_layout(P, numels.data(), chunk_len, &L)) return 1;
     if (L.total == 0) return 0;
     if (!workspace || workspace_bytes < L.bytes)
         return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
@@ -176,7 +202,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     for (int i = 0; i < P; i++) {
         const Sg2Tensor& t = tensors[i];
         const int n = (int)t.numel;
-        const int nc = (n + g_chunk_len - 1) / g_chunk_len;
+        const int nc = (n + chunk_len - 1) / chunk_len;
         TensorDev& d = td[i];
         d.param = t.param; d.grad = t.grad; d.sharp = t.sharpness;
         d.ea = t.exp_avg; d.easq = t.exp_avg_sq; d.mu = t.mu; d.gru = t.gru_state;
@@ -202,7 +228,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.chunk_prefix = dpre + 2 * (P + 1);
     pl.wchunk_prefix = dpre + 3 * (P + 1);
     pl.P = P; pl.total = L.total; pl.elem_tiles = L.elem_tiles; pl.sort_tiles = L.sort_tiles;
-    pl.chunks = L.chunks; pl.wchunks = L.wchunks; pl.chunk_len = g_chunk_len;
+    pl.chunks = L.chunks; pl.wchunks = L.wchunks; pl.chunk_len = chunk_len; pl.window = g_window;
     for (int k = 0; k < 2; k++) {
         pl.keys[k] = reinterpret_cast<uint32_t*>(ws + L.off_keys[k]);
         pl.vals[k] = reinterpret_cast<int32_t*>(ws + L.off_vals[k]);

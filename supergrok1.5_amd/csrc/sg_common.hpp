@@ -68,6 +68,15 @@ typedef const __attribute__((address_space(4))) int* cint_p;
 __device__ __forceinline__ cfloat_p as_const(const float* p) { return (cfloat_p)p; }
 __device__ __forceinline__ cint_p as_const(const int* p) { return (cint_p)p; }
 
+// A zero the optimiser cannot see through, held in a scalar register.  Adding it to a weight pointer
+// inside a loop keeps the loop-invariant scalar loads where they are used: hoisted out of the loop,
+// a thousand of them would be spilled from SGPRs into VGPR lanes and read back with v_readlane.
+__device__ __forceinline__ int opaque_zero() {
+    int z = 0;
+    asm volatile("" : "+s"(z));
+    return z;
+}
+
 // largest i in [0, n) with prefix[i] <= x   (prefix is non-decreasing, prefix[0] == 0)
 template <class P>
 __device__ __forceinline__ int upper_seg(P prefix, int n, int x) {

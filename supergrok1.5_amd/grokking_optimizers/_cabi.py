@@ -47,7 +47,7 @@ class Sg2Debug(C.Structure):
     _fields_ = [("perm", C.c_void_p), ("expert_idx", C.c_void_p), ("ctx", C.c_void_p)]
 
 
-EXPORTS = ("sg_last_error", "sg2_set_chunk_len", "sg2_get_chunk_len", "sg2_workspace_bytes", "sg2_batched_step",
+EXPORTS = ("sg_last_error", "sg2_set_chunk_len", "sg2_get_chunk_len", "sg2_set_scan_window", "sg2_get_scan_window", "sg2_chunk_len_for", "sg2_workspace_bytes", "sg2_batched_step",
            "sg2_profile_enable", "sg2_profile_read")
 SG2_PROF_STAGES = ("sort", "scan_summary", "chunk_prefix", "scan_output", "elementwise")
 
@@ -62,6 +62,7 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.sg_last_error.restype = C.c_char_p
         L.sg2_set_chunk_len.argtypes = [C.c_int]
+        L.sg2_set_scan_window.argtypes = [C.c_int]
         L.sg2_workspace_bytes.restype = C.c_size_t
         L.sg2_workspace_bytes.argtypes = [C.POINTER(SgDims), C.c_int, C.POINTER(C.c_int64)]
         L.sg2_batched_step.restype = C.c_int
@@ -93,6 +94,12 @@ def last_error():
 def make_dims(dims=None):
     d = dict(DEFAULT_DIMS if dims is None else dims)
     return SgDims(*[d[n] for n in DIM_NAMES])
+
+
+def chunk_len_for(numels):
+    """Scan chunk length a call with these tensor sizes uses (the configured one, or the automatic choice)."""
+    arr = (C.c_int64 * len(numels))(*numels)
+    return lib().sg2_chunk_len_for(len(numels), arr)
 
 
 def workspace_bytes(numels, dims=None):

@@ -67,7 +67,12 @@ class Sg2Case:
         self.step_fn(gg, ss, per_tensor, shared)
         torch.cuda.synchronize()
 
-    def oracle_step(self, grads, sharps, per_tensor, shared, chunk_len, precision=32, threads=8):
+    def oracle_step(self, grads, sharps, per_tensor, shared, chunk_len, precision=32, threads=8, window=None):
+        from grokking_optimizers import _cabi
+        if window is None:
+            window = _cabi.lib().sg2_get_scan_window()
+        if chunk_len is None:
+            chunk_len = _cabi.chunk_len_for([wl.numel(s) for s in self.shapes])
         dbg = [None] * self.P
         counts = [np.zeros_like(self.counts_np) for _ in range(self.P)]
 
@@ -78,7 +83,7 @@ class Sg2Case:
             s = to_np(sharps[i].reshape(-1).to(self.dtypes[i]))
             if self.np[i]["exp_avg"].size == 0:
                 return
-            dbg[i] = orc.sg2_step(self.Wnp, self.np[i], g, s, sc, precision=precision, chunk_len=chunk_len,
+            dbg[i] = orc.sg2_step(self.Wnp, self.np[i], g, s, sc, precision=precision, chunk_len=chunk_len, window=window,
                                   expert_counts=counts[i], debug=True)
         with ThreadPoolExecutor(threads) as ex:
             list(ex.map(one, range(self.P)))
