@@ -4,7 +4,8 @@
 A "step" is one call of sg2_batched_step (sort -> bidirectional scan -> GRU ->
 PEER -> expert MLP -> Adam/WD) over the whole synthetic parameter set, with
 parameters, gradients, moments and meta-net weights already resident in HBM.
-Prints ONE JSON line; see DESIGN.md for how each field is derived.
+Prints ONE JSON line: whole-step throughput, the roofline figures of the dominant kernel (timed by HIP
+events on the step's stream), and a single-core CPU baseline on a bounded sample.
 """
 import argparse
 import json
@@ -20,7 +21,7 @@ for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd"), os.path.join(ROOT, "test
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (read + written) on the 25M-element workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs scaled by a 1 GiB copy (profiles/sg2_step_scale50_pmc_traffic.txt); not measured by this script
+# runs scaled by what the same counters read for a 1 GiB device copy; not measured by this script
 PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.675e9 + 1.626e9, "scan_summary": 0.619e9 + 0.150e9,
                              "elementwise": 2.603e9 + 0.801e9}
 FLOP_PER_ELEMENT = 30e3         # arithmetic actually required per element (both scan directions + elementwise)
@@ -152,7 +153,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
-                         "grokfast / sg15 / muon time the other fused steps of BASELINE configs 1, 2 and 5")
+                         "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
     ap.add_argument("--window", type=int, default=-1, help="scan summary window (-1: library default, 0: off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -219,7 +220,7 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SuperGrok v2 full step, %d tensors, %d elements (%s), fp32, bilevel off"
-                               % (len(shapes), total, "BASELINE configs[3]" if args.workload == "scale50" else "configs[2] set"),
+                               % (len(shapes), total, "50 log-uniform tensors" if args.workload == "scale50" else "2-layer transformer set"),
                    "chunk_len": _cabi.chunk_len_for([p.numel() for p in st["params"]]), "summary_window": _cabi.lib().sg2_get_scan_window()},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
