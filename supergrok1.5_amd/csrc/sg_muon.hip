@@ -12,15 +12,18 @@
 // All three products are "NT" GEMMs (both operands K-contiguous) once the
 // transpose Y^T is kept next to Y; it is refreshed by a small LDS transpose
 // kernel after every iteration.  Work buffers are zero-padded to multiples of
-// 128 so the GEMM needs no edge handling (zero rows/columns stay zero through
+// 256 so the GEMM needs no edge handling (zero rows/columns stay zero through
 // the iteration).
 //
-// GEMM: 128x128 output tile per 256-thread workgroup, 4 waves as 2x2, each
-// wave 64x64 = 2x2 MFMA 32x32x16 bf16 tiles (64 fp32 accumulators per lane),
-// K tiles of 64 staged through double-buffered LDS with 144-byte row stride
+// GEMM: 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each
+// wave 128x128 = 4x4 MFMA 32x32x16 bf16 tiles (256 fp32 accumulators per
+// lane), K tiles of 64 staged through LDS with 144-byte row stride
 // (conflict-free 16-byte operand fetches), next tile prefetched into registers
-// while the current one is multiplied.  Tile index -> XCD-contiguous order so
-// that the workgroups sharing operand panels share an L2.
+// while the current one is multiplied.  256x256x64 gives 128 flop per byte
+// fetched, which keeps the MFMA pipe ahead of the ~64 B/clk a CU can pull from
+// L2; the symmetric products (G and G*G) compute only the tiles on or above
+// the diagonal.  Tile index -> XCD-contiguous order so that the workgroups
+// sharing operand panels share an L2.
 #include <cmath>
 #include <vector>
 
@@ -33,9 +36,11 @@ typedef uint16_t bf16_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-constexpr int BT = 128;            // GEMM tile (M and N)
+constexpr int BT = 256;            // GEMM tile (M and N)
 constexpr int BK = 64;             // GEMM K tile
 constexpr int LDS_ROW = BK + 8;    // bf16 elements per LDS row (144 bytes)
+constexpr int GEMM_LDS_BYTES = 2 * 2 * BT * LDS_ROW * 2;   // two stages of {A tile, B tile}: 147,456 bytes of the CU's 160 KB
+static_assert(BK == 64, "the K loop of k_gemm_nt is written for four 16-wide steps");
 constexpr int ETILE = 4096;        // elements per tile of the elementwise kernels
 constexpr float NS_A = 3.4445f, NS_B = -4.7750f, NS_C = 2.0315f;
 
@@ -139,103 +144,146 @@ __global__ __launch_bounds__(256) void k_transpose(Batch B, int to_yt, int only_
 }
 
 // ---- NT GEMM  C[M x N] = A[M x K] * B[N x K]^T  with fused epilogues ---------------
+// 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
+// 32x32x16 tiles (256 fp32 accumulators per lane; one wave per SIMD, the whole register file).
+// Per 16-wide k step a wave fetches 4+4 16-byte operands from LDS for 16 MFMAs.  The next K tile
+// is prefetched from global memory into registers while the current one is multiplied.
+// The Gram and polynomial products are symmetric: only tiles on or above the diagonal are
+// computed, each off-diagonal tile is also stored transposed.
 enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint16_t bf16r(float v) {   // round to nearest even, NaN kept quiet; no branches
+    const uint32_t u = (uint32_t)sg_f2i(v);
+    const uint32_t rne = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    const uint32_t nan = (u >> 16) | 0x40u;
+    return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne);
+}
 
 template <int EPI>
 __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
-    __shared__ __attribute__((aligned(16))) bf16_t sA[2][BT * LDS_ROW];
-    __shared__ __attribute__((aligned(16))) bf16_t sB[2][BT * LDS_ROW];
+    constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
+    constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
+    // LDS: two stages of {A tile, B tile}, each tile BT rows of LDS_ROW elements
+    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
+    constexpr int TILE_ELEMS = BT * LDS_ROW;
 
     // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs
     const int nblk = gridDim.x;
     int lb = blockIdx.x;
     if (nblk % 8 == 0) lb = (blockIdx.x % 8) * (nblk / 8) + blockIdx.x / 8;
-    const int* __restrict__ prefix = Bt.gtile_prefix[EPI];
+    const sg::cint_p prefix = sg::as_const(Bt.gtile_prefix[EPI]);
     const int mi = sg::upper_seg(prefix, Bt.P, lb);
     const Mat& Mt = Bt.mats[mi];
-    const int tile = lb - prefix[mi];
+    int tile = lb - prefix[mi];
 
     const bf16_t *A, *B;
     bf16_t* C;
-    int K, lda, ldb, ldc, tn_count;
-    if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; tn_count = Mt.mp / BT; }
-    else if (EPI == EPI_POLY) { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; tn_count = Mt.mp / BT; }
-    else { A = Mt.H; B = Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np; tn_count = Mt.np / BT; }
-    const int tm = tile / tn_count, tn = tile % tn_count;
+    int K, lda, ldb, ldc, tm, tn;
+    if (EPI == EPI_APPLY) {
+        A = Mt.H; B = Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np;
+        const int tn_count = Mt.np / BT;
+        tm = tile / tn_count;
+        tn = tile % tn_count;
+    } else {
+        if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; }
+        else { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; }
+        const int nt = Mt.mp / BT;      // upper-triangular enumeration: row tm holds nt - tm tiles
+        tm = 0;
+        while (tile >= nt - tm) { tile -= nt - tm; tm++; }
+        tn = tm + tile;
+    }
     A += (size_t)tm * BT * lda;
     B += (size_t)tn * BT * ldb;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    f32x16 acc[2][2];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // global -> register staging: 4 x 16 bytes of A and of B per thread per K tile
-    uint4 ra[4], rb[4];
-    auto gload = [&](int k0) {
+    // One operand tile of the next K step is in flight in registers at a time: A is fetched
+    // while the first half of the current K tile is multiplied and stored into the other LDS
+    // stage, then B during the second half.  One barrier per K tile.
+    u32x4 rg[CH];    // native vector type: the array is promoted to registers (HIP's uint4 struct is not)
+    const uint32_t voff_a = (uint32_t)(((tid >> 3) * lda + (tid & 7) * 8) * 2);
+    const uint32_t voff_b = (uint32_t)(((tid >> 3) * ldb + (tid & 7) * 8) * 2);
+    const int soff = (tid >> 3) * LDS_ROW + (tid & 7) * 8;
+    auto gload = [&](const bf16_t* base, int ld, uint32_t voff, int k0) {
+        const char* p = reinterpret_cast<const char*>(base + k0);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
-            ra[i] = *reinterpret_cast<const uint4*>(A + (size_t)row * lda + k0 + kc * 8);
-            rb[i] = *reinterpret_cast<const uint4*>(B + (size_t)row * ldb + k0 + kc * 8);
-        }
+        for (int i = 0; i < CH; i++) rg[i] = *reinterpret_cast<const u32x4*>(p + (size_t)i * 32 * ld * 2 + voff);
     };
-    auto sstore = [&](int buf) {
+    auto sstore = [&](bf16_t* tile) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
-            *reinterpret_cast<uint4*>(&sA[buf][row * LDS_ROW + kc * 8]) = ra[i];
-            *reinterpret_cast<uint4*>(&sB[buf][row * LDS_ROW + kc * 8]) = rb[i];
-        }
+        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&tile[soff + i * 32 * LDS_ROW]) = rg[i];
+    };
+    const int a_off = (wm * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
+    const int b_off = TILE_ELEMS + (wn * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
+    auto mma = [&](const bf16_t* stage, int kk) {
+        bf16x8 av[TM], bv[TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const bf16x8*>(stage + a_off + i * 32 * LDS_ROW + kk * 16);
+#pragma unroll
+        for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
     };
 
-    gload(0);
-    sstore(0);
+    gload(A, lda, voff_a, 0);
+    sstore(smem);
+    gload(B, ldb, voff_b, 0);
+    sstore(smem + TILE_ELEMS);
     __syncthreads();
     const int nk = K / BK;
     for (int kt = 0; kt < nk; kt++) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) gload((kt + 1) * BK);
-        const bf16_t* a_base = &sA[cur][(wm * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 8];
-        const bf16_t* b_base = &sB[cur][(wn * 64 + (lane & 31)) * LDS_ROW + (lane >> 5) * 8];
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
-            bf16x8 av[2], bv[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                av[i] = *reinterpret_cast<const bf16x8*>(a_base + i * 32 * LDS_ROW + kk * 16);
-                bv[i] = *reinterpret_cast<const bf16x8*>(b_base + i * 32 * LDS_ROW + kk * 16);
-            }
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) sstore(cur ^ 1);
+        const bf16_t* cur = smem + (kt & 1) * 2 * TILE_ELEMS;
+        bf16_t* nxt = smem + ((kt + 1) & 1) * 2 * TILE_ELEMS;
+        const bool more = kt + 1 < nk;
+        if (more) gload(A, lda, voff_a, (kt + 1) * BK);
+        mma(cur, 0);
+        mma(cur, 1);
+        if (more) { sstore(nxt); gload(B, ldb, voff_b, (kt + 1) * BK); }
+        mma(cur, 2);
+        mma(cur, 3);
+        if (more) sstore(nxt + TILE_ELEMS);
         __syncthreads();
     }
 
     // epilogue: accumulator element e of tile (i,j): row = 8*(e/4) + 4*(lane/32) + e%4, col = lane%32
     const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : Mt.Y;
+    const bool mirror = (EPI != EPI_APPLY) && tm != tn;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < TN; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                const int row = tm * BT + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                const int col = tn * BT + wn * 64 + j * 32 + (lane & 31);
-                const size_t o = (size_t)row * ldc + col;
-                float v = acc[i][j][e];
-                if (EPI == EPI_POLY) v = sg_fma(NS_C, v, NS_B * sg::bf16_bits_to_f(aux[o]));
-                if (EPI == EPI_APPLY) v = sg_fma(NS_A, sg::bf16_bits_to_f(aux[o]), v);
-                C[o] = sg::f_to_bf16_bits(v);
+            for (int q = 0; q < 4; q++) {
+                const int row0 = tm * BT + wm * (BT / 2) + i * 32 + 8 * q + 4 * (lane >> 5);
+                const int col = tn * BT + wn * (BT / 2) + j * 32 + (lane & 31);
+                uint16_t o[4];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const size_t off = (size_t)(row0 + r) * ldc + col;
+                    float v = acc[i][j][4 * q + r];
+                    if (EPI == EPI_POLY) v = sg_fma(NS_C, v, NS_B * sg::bf16_bits_to_f(aux[off]));
+                    if (EPI == EPI_APPLY) v = sg_fma(NS_A, sg::bf16_bits_to_f(aux[off]), v);
+                    o[r] = bf16r(v);
+                    C[off] = o[r];
+                }
+                if (mirror) {   // C[col][row0 .. row0+3]
+                    uint2 pk;
+                    pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+                    pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+                    *reinterpret_cast<uint2*>(C + (size_t)col * ldc + row0) = pk;
+                }
             }
 }
 
@@ -301,8 +349,9 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         M.etile0 = (int)etiles;
         etiles += et;
         L->pre_e[i + 1] = L->pre_e[i] + et;
-        L->pre_g[EPI_GRAM][i + 1] = L->pre_g[EPI_GRAM][i] + (M.mp / BT) * (M.mp / BT);
-        L->pre_g[EPI_POLY][i + 1] = L->pre_g[EPI_POLY][i] + (M.mp / BT) * (M.mp / BT);
+        const int nt = M.mp / BT, tri = nt * (nt + 1) / 2;      // symmetric products: tiles on or above the diagonal
+        L->pre_g[EPI_GRAM][i + 1] = L->pre_g[EPI_GRAM][i] + tri;
+        L->pre_g[EPI_POLY][i + 1] = L->pre_g[EPI_POLY][i] + tri;
         L->pre_g[EPI_APPLY][i + 1] = L->pre_g[EPI_APPLY][i] + (M.mp / BT) * (M.np / BT);
         L->pre_t[i + 1] = L->pre_t[i] + (M.mp / 64) * (M.np / 64);
     }
@@ -369,6 +418,18 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
     B.partials = reinterpret_cast<double*>(ws + L.off_partials);
     B.inv_norm = reinterpret_cast<float*>(ws + L.off_inv);
 
+    {   // the GEMM needs more LDS than the default per-kernel limit: raise it once per device
+        static bool raised[64] = {};
+        int dev = 0;
+        SG_HIP_CHECK(hipGetDevice(&dev));
+        if (dev >= 0 && dev < 64 && !raised[dev]) {
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_GRAM>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_POLY>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_APPLY>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
+            raised[dev] = true;
+        }
+    }
+
     // padded work buffers start from zero (a fill kernel, not a memset node, so the call stays capturable)
     bool any_pad = false;
     for (const auto& M : L.mats) any_pad = any_pad || M.mp != M.m || M.np != M.n;
@@ -389,9 +450,9 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
         SG_LAUNCH_CHECK("muon transpose");
     }
     for (int it = 0; it < ns_steps; it++) {
-        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), 0, st, B);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), 0, st, B);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), 0, st, B);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B);
         hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 1, 0, 0);    // YT <- Y^T for every matrix
         SG_LAUNCH_CHECK("muon newton-schulz");
     }
