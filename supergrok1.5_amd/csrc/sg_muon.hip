@@ -28,6 +28,7 @@
 #include <vector>
 
 #include "sg_common.hpp"
+#include <type_traits>
 
 namespace sgmu {
 namespace {
@@ -152,12 +153,15 @@ __global__ __launch_bounds__(256) void k_transpose(Batch B, int to_yt, int only_
 // computed, each off-diagonal tile is also stored transposed.
 enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// explicit global address space: a generic (flat) load would count against the LDS wait counter as well
+typedef const __attribute__((address_space(1))) u32x4* gvec_p;
 
-__device__ __forceinline__ uint16_t bf16r(float v) {   // round to nearest even, NaN kept quiet; no branches
+__device__ __forceinline__ uint32_t bf16r(float v) {   // round to nearest even, NaN kept quiet; no branches
     const uint32_t u = (uint32_t)sg_f2i(v);
     const uint32_t rne = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
     const uint32_t nan = (u >> 16) | 0x40u;
-    return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne);
+    return ((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne;
 }
 
 template <int EPI>
@@ -168,10 +172,13 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
     constexpr int TILE_ELEMS = BT * LDS_ROW;
 
-    // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs
+    // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs,
+    // so that tiles that run together on an XCD share operand panels in its L2
     const int nblk = gridDim.x;
     int lb = blockIdx.x;
     if (nblk % 8 == 0) lb = (blockIdx.x % 8) * (nblk / 8) + blockIdx.x / 8;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
     const sg::cint_p prefix = sg::as_const(Bt.gtile_prefix[EPI]);
     const int mi = sg::upper_seg(prefix, Bt.P, lb);
     const Mat& Mt = Bt.mats[mi];
@@ -182,9 +189,17 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     int K, lda, ldb, ldc, tm, tn;
     if (EPI == EPI_APPLY) {
         A = Mt.H; B = Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np;
-        const int tn_count = Mt.np / BT;
-        tm = tile / tn_count;
-        tn = tile % tn_count;
+        // bands of 8 tile columns: 32 tiles that run together span 4 x 8 tiles instead of 2 x 16,
+        // which halves the panel bytes they pull into L2
+        const int ntm = Mt.mp / BT, ntn = Mt.np / BT;
+        if (ntn % 8 == 0) {
+            const int band = tile / (ntm * 8), w = tile % (ntm * 8);
+            tm = w / 8;
+            tn = band * 8 + w % 8;
+        } else {
+            tm = tile / ntn;
+            tn = tile % ntn;
+        }
     } else {
         if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; }
         else { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; }
@@ -196,9 +211,6 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     A += (size_t)tm * BT * lda;
     B += (size_t)tn * BT * ldb;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-
     f32x16 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -207,84 +219,224 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // One operand tile of the next K step is in flight in registers at a time: A is fetched
-    // while the first half of the current K tile is multiplied and stored into the other LDS
-    // stage, then B during the second half.  One barrier per K tile.
-    u32x4 rg[CH];    // native vector type: the array is promoted to registers (HIP's uint4 struct is not)
+    // Global -> register -> LDS pipeline two K tiles deep: while tile kt is multiplied out of
+    // one LDS stage, tile kt+1 moves from its register set into the other stage and the loads of
+    // tile kt+3 are issued into the set just freed; tile kt+2 stays in flight in the other set.
+    // A load has two K tiles of MFMA work (~4000 cycles) to arrive.  One barrier per K tile.
+    u32x4 ra[2][CH], rb[2][CH];
     const uint32_t voff_a = (uint32_t)(((tid >> 3) * lda + (tid & 7) * 8) * 2);
     const uint32_t voff_b = (uint32_t)(((tid >> 3) * ldb + (tid & 7) * 8) * 2);
     const int soff = (tid >> 3) * LDS_ROW + (tid & 7) * 8;
-    auto gload = [&](const bf16_t* base, int ld, uint32_t voff, int k0) {
-        const char* p = reinterpret_cast<const char*>(base + k0);
+    auto gload_a = [&](int set, int kt) {
+        const char* pa = reinterpret_cast<const char*>(A + kt * BK);
 #pragma unroll
-        for (int i = 0; i < CH; i++) rg[i] = *reinterpret_cast<const u32x4*>(p + (size_t)i * 32 * ld * 2 + voff);
+        for (int i = 0; i < CH; i++) ra[set][i] = *(gvec_p)(pa + (size_t)i * 32 * lda * 2 + voff_a);
     };
-    auto sstore = [&](bf16_t* tile) {
+    auto gload_b = [&](int set, int kt) {
+        const char* pb = reinterpret_cast<const char*>(B + kt * BK);
 #pragma unroll
-        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&tile[soff + i * 32 * LDS_ROW]) = rg[i];
+        for (int i = 0; i < CH; i++) rb[set][i] = *(gvec_p)(pb + (size_t)i * 32 * ldb * 2 + voff_b);
+    };
+    auto sstore_a = [&](int set, bf16_t* stage) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[soff + i * 32 * LDS_ROW]) = ra[set][i];
+    };
+    auto sstore_b = [&](int set, bf16_t* stage) {
+#pragma unroll
+        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[TILE_ELEMS + soff + i * 32 * LDS_ROW]) = rb[set][i];
     };
     const int a_off = (wm * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
     const int b_off = TILE_ELEMS + (wn * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
-    auto mma = [&](const bf16_t* stage, int kk) {
-        bf16x8 av[TM], bv[TN];
+    // MFMA operands are double-buffered in registers: the LDS reads of the next 16-wide k step are
+    // in flight while the 16 MFMAs of the current one issue (one wave per SIMD, nothing else hides them)
+    bf16x8 av[2][TM], bv[2][TN];
+    auto lds_load = [&](const bf16_t* stage, int kk, int s) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) av[i] = *reinterpret_cast<const bf16x8*>(stage + a_off + i * 32 * LDS_ROW + kk * 16);
+        for (int i = 0; i < TM; i++) av[s][i] = *reinterpret_cast<const bf16x8*>(stage + a_off + i * 32 * LDS_ROW + kk * 16);
 #pragma unroll
-        for (int j = 0; j < TN; j++) bv[j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+        for (int j = 0; j < TN; j++) bv[s][j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+    };
+    auto mma = [&](int s) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i], bv[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[s][i], bv[s][j], acc[i][j], 0, 0, 0);
     };
 
-    gload(A, lda, voff_a, 0);
-    sstore(smem);
-    gload(B, ldb, voff_b, 0);
-    sstore(smem + TILE_ELEMS);
+    const int nk = K / BK;      // a multiple of 4: K is a multiple of 256
+    gload_a(0, 0); gload_b(0, 0);
+    sstore_a(0, smem); sstore_b(0, smem);
+    gload_a(1, 1); gload_b(1, 1);
+    gload_a(0, 2); gload_b(0, 2);
     __syncthreads();
-    const int nk = K / BK;
-    for (int kt = 0; kt < nk; kt++) {
+    // One wave per SIMD issues in order, so a burst of memory instructions leaves the MFMA pipe
+    // idle while it issues.  Each K tile is four phases of 16 MFMAs; the LDS reads of the next k
+    // step, the LDS writes of tile kt+1 and the global loads of tile kt+3 are dealt between the
+    // MFMAs of a phase with sched_group_barrier (masks: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS
+    // read, 0x200 LDS write).  The steady-state body issues everything unconditionally (a static
+    // wait count has to be right on every path); the last four K tiles are peeled.
+    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : Mt.Y;
+    const int gcol0 = tn * BT + wn * (BT / 2);
+    auto ktile = [&](int kt, auto set_c, auto store_c, auto load_c) {
+        constexpr int S = decltype(set_c)::value;       // register set holding tile kt+1
+#ifdef SGX_NOLOAD
+        constexpr bool LD = false;
+#else
+        constexpr bool LD = decltype(load_c)::value != 0;
+#endif
+#ifdef SGX_NOSTORE
+        constexpr bool ST = false;
+#else
+        constexpr bool ST = decltype(store_c)::value != 0;
+#endif
         const bf16_t* cur = smem + (kt & 1) * 2 * TILE_ELEMS;
         bf16_t* nxt = smem + ((kt + 1) & 1) * 2 * TILE_ELEMS;
-        const bool more = kt + 1 < nk;
-        if (more) gload(A, lda, voff_a, (kt + 1) * BK);
-        mma(cur, 0);
-        mma(cur, 1);
-        if (more) { sstore(nxt); gload(B, ldb, voff_b, (kt + 1) * BK); }
-        mma(cur, 2);
-        mma(cur, 3);
-        if (more) sstore(nxt + TILE_ELEMS);
-        __syncthreads();
-    }
-
-    // epilogue: accumulator element e of tile (i,j): row = 8*(e/4) + 4*(lane/32) + e%4, col = lane%32
-    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : Mt.Y;
-    const bool mirror = (EPI != EPI_APPLY) && tm != tn;
+#ifdef SGX_NOLDSREAD
+        if (kt == 0)
+#endif
+        lds_load(cur, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 0: k step 0 | read k step 1
+#ifdef SGX_NOLDSREAD
+        if (kt == 0)
+#endif
+        lds_load(cur, 1, 1);
+        mma(0);
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+        for (int g = 0; g < 8; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 1: k step 1 | read k step 2, write A of tile kt+1
+#ifdef SGX_NOLDSREAD
+        if (kt == 0)
+#endif
+        lds_load(cur, 2, 0);
+        if (ST) sstore_a(S, nxt);
+        mma(1);
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 2: k step 2 | read k step 3, write B of tile kt+1, load A of tile kt+3
+#ifdef SGX_NOLDSREAD
+        if (kt == 0)
+#endif
+        lds_load(cur, 3, 1);
+        if (ST) sstore_b(S, nxt);
+        if (LD) gload_a(S, kt + 3);
+        mma(0);
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // phase 3: k step 3 | load B of tile kt+3
+        if (LD) gload_b(S, kt + 3);
+        mma(1);
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#ifndef SGX_NOBARRIER
+        __syncthreads();
+#endif
+    };
+    using c0 = std::integral_constant<int, 0>;
+    using c1 = std::integral_constant<int, 1>;
+    int kt = 0;
+    for (; kt + 4 < nk; kt += 2) {
+        ktile(kt, c1{}, c1{}, c1{});
+        ktile(kt + 1, c0{}, c1{}, c1{});
+    }
+    ktile(kt, c1{}, c1{}, c1{});        // kt = nk-4: loads the last tile
+    ktile(kt + 1, c0{}, c1{}, c0{});
+    ktile(kt + 2, c1{}, c1{}, c0{});
+    ktile(kt + 3, c0{}, c0{}, c0{});
+
+    // ---- epilogue, staged through LDS (free after the last barrier) so that global memory sees
+    // 16-byte accesses along rows.  Accumulator element e of MFMA tile (i,j) is
+    // row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.  One 32-row block of the wave's 128x128
+    // tile at a time: fp32 block -> LDS, read back as 8-column chunks, combine with the auxiliary
+    // operand, round to bf16 and store.  Off-diagonal tiles of the symmetric products also store
+    // the transposed block: the rounded values go back into the staged block and are read down
+    // its columns.  Every wave stages in its own LDS region and LDS executes a wave's
+    // instructions in order, so no workgroup barrier is needed, only the compiler kept from
+    // reordering (wave_barrier).
+    constexpr int EP_ROW = 128 + 4;     // floats per staged row
+    static_assert(4 * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
+    float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EP_ROW);
+    const bool mirror = (EPI != EPI_APPLY) && tm != tn;     // uniform over the workgroup
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int grow0 = tm * BT + wm * (BT / 2) + i * 32;
 #pragma unroll
         for (int j = 0; j < TN; j++)
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int row0 = tm * BT + wm * (BT / 2) + i * 32 + 8 * q + 4 * (lane >> 5);
-                const int col = tn * BT + wn * (BT / 2) + j * 32 + (lane & 31);
-                uint16_t o[4];
+            for (int e = 0; e < 16; e++)
+                ep[(8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * EP_ROW + 32 * j + (lane & 31)] = acc[i][j][e];
+        // the auxiliary operand (G for the polynomial, Y for the apply step, which updates Y in
+        // place): all of this block's chunks are fetched before its first store so the loads overlap
+        u32x4 ax[8];
+        if (EPI != EPI_GRAM) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    const size_t off = (size_t)(row0 + r) * ldc + col;
-                    float v = acc[i][j][4 * q + r];
-                    if (EPI == EPI_POLY) v = sg_fma(NS_C, v, NS_B * sg::bf16_bits_to_f(aux[off]));
-                    if (EPI == EPI_APPLY) v = sg_fma(NS_A, sg::bf16_bits_to_f(aux[off]), v);
-                    o[r] = bf16r(v);
-                    C[off] = o[r];
-                }
-                if (mirror) {   // C[col][row0 .. row0+3]
-                    uint2 pk;
-                    pk.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-                    pk.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-                    *reinterpret_cast<uint2*>(C + (size_t)col * ldc + row0) = pk;
+            for (int c = 0; c < 8; c++) {
+                const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
+                ax[c] = *(gvec_p)(aux + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
+            f32x4* src = reinterpret_cast<f32x4*>(&ep[row * EP_ROW + c8 * 8]);
+            const f32x4 lo = src[0], hi = src[1];
+            float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            if (EPI != EPI_GRAM) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const uint32_t w = ax[c][k >> 1];
+                    const float x = sg_i2f((int32_t)((k & 1) ? (w & 0xffff0000u) : (w << 16)));
+                    v[k] = (EPI == EPI_POLY) ? sg_fma(NS_C, v[k], NS_B * x) : sg_fma(NS_A, x, v[k]);
                 }
             }
+            uint32_t o[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) o[k] = bf16r(v[k]);
+            u32x4 out;
+#pragma unroll
+            for (int k = 0; k < 4; k++) out[k] = o[2 * k] | (o[2 * k + 1] << 16);
+            *reinterpret_cast<u32x4*>(C + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8) = out;
+            if (mirror) {   // rounded values (as bf16 bit patterns) back into the staged block
+                u32x4 b0 = {o[0], o[1], o[2], o[3]}, b1 = {o[4], o[5], o[6], o[7]};
+                reinterpret_cast<u32x4*>(src)[0] = b0;
+                reinterpret_cast<u32x4*>(src)[1] = b1;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (mirror) {
+            const uint32_t* epb = reinterpret_cast<const uint32_t*>(ep);
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const int id = lane + 64 * c, col = id >> 2, r8 = id & 3;
+                u32x4 t;
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    t[k] = epb[(r8 * 8 + 2 * k) * EP_ROW + col] | (epb[(r8 * 8 + 2 * k + 1) * EP_ROW + col] << 16);
+                *reinterpret_cast<u32x4*>(C + (size_t)(gcol0 + col) * ldc + grow0 + r8 * 8) = t;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
 }
 
 // p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
@@ -422,7 +574,9 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
         static bool raised[64] = {};
         int dev = 0;
         SG_HIP_CHECK(hipGetDevice(&dev));
-        if (dev >= 0 && dev < 64 && !raised[dev]) {
+        if (dev < 0 || dev >= 64) return sg::fail("device index %d out of range", dev);
+        if (!raised[dev]) {
+
             SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_GRAM>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
             SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_POLY>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
             SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_nt<EPI_APPLY>), hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES));
