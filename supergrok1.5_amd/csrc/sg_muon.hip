@@ -10,16 +10,20 @@
 // (for a tall parameter X this is X^T X and X (bG + cG^2): the reference's
 // X X^T form re-associated, 6 m^2 n instead of 6 n^2 m flops per iteration).
 // All three products are "NT" GEMMs (both operands K-contiguous) once the
-// transpose Y^T is kept next to Y; it is refreshed by a small LDS transpose
-// kernel after every iteration.  Work buffers are zero-padded to multiples of
+// transpose Y^T is kept next to Y; the apply step's epilogue writes the new Y
+// and, into the other of two Y^T buffers, its transpose (the current Y^T is
+// still being read as the B operand by other workgroups).  An LDS transpose
+// kernel is only needed once, after normalisation.  Work buffers are
+// zero-padded to multiples of
 // 256 so the GEMM needs no edge handling (zero rows/columns stay zero through
 // the iteration).
 //
 // GEMM: 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each
 // wave 128x128 = 4x4 MFMA 32x32x16 bf16 tiles (256 fp32 accumulators per
 // lane), K tiles of 64 staged through LDS with 144-byte row stride
-// (conflict-free 16-byte operand fetches), next tile prefetched into registers
-// while the current one is multiplied.  256x256x64 gives 128 flop per byte
+// (conflict-free 16-byte operand fetches, two stages), the tiles of the next
+// K steps in flight in two register sets while the current one is multiplied,
+// memory instructions dealt between the MFMAs.  256x256x64 gives 128 flop per byte
 // fetched, which keeps the MFMA pipe ahead of the ~64 B/clk a CU can pull from
 // L2; the symmetric products (G and G*G) compute only the tiles on or above
 // the diagonal.  Tile index -> XCD-contiguous order so that the workgroups
@@ -50,11 +54,12 @@ struct Mat {
     const void* grad;
     float* buf;
     bf16_t *Y, *YT, *G, *H;       // [mp x np], [np x mp], [mp x mp], [mp x mp]
+    bf16_t* YT2;                   // second [np x mp] buffer: the apply step reads one transposed copy and writes the other
     int rows, cols, dtype;
     int m, n, mp, np;              // min / max dim and their padded sizes
     int wide;                      // rows <= cols
     int etile0;                    // first elementwise tile of this matrix
-    int pad_;
+    int vec8;                      // cols % 8 == 0 and param/grad/buf 16-byte aligned: elementwise kernels move 8 elements per lane
 };
 
 struct Batch {
@@ -78,20 +83,71 @@ __device__ __forceinline__ double block_sum(double v, double* sm) {
     return r;
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// eight consecutive elements in the tensor's storage type; i a multiple of 8, base 16-byte aligned
+__device__ __forceinline__ void load8(const void* p, int dtype, size_t i, float v[8]) {
+    if (dtype == SG_F32) {
+        const f32x4* q = reinterpret_cast<const f32x4*>(static_cast<const float*>(p) + i);
+        const f32x4 a = q[0], b = q[1];
+#pragma unroll
+        for (int k = 0; k < 4; k++) { v[k] = a[k]; v[4 + k] = b[k]; }
+    } else {
+        const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p) + i);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const uint16_t h = (uint16_t)((k & 1) ? (w[k >> 1] >> 16) : (w[k >> 1] & 0xffffu));
+            v[k] = (dtype == SG_F16) ? __half2float(__ushort_as_half(h)) : sg::bf16_bits_to_f(h);
+        }
+    }
+}
+__device__ __forceinline__ void store8(void* p, int dtype, size_t i, const float v[8]) {
+    if (dtype == SG_F32) {
+        f32x4* q = reinterpret_cast<f32x4*>(static_cast<float*>(p) + i);
+        q[0] = f32x4{v[0], v[1], v[2], v[3]};
+        q[1] = f32x4{v[4], v[5], v[6], v[7]};
+    } else {
+        u32x4 w;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t lo = (dtype == SG_F16) ? __half_as_ushort(__float2half_rn(v[2 * k])) : sg::f_to_bf16_bits(v[2 * k]);
+            const uint32_t hi = (dtype == SG_F16) ? __half_as_ushort(__float2half_rn(v[2 * k + 1])) : sg::f_to_bf16_bits(v[2 * k + 1]);
+            w[k] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(p) + i) = w;
+    }
+}
+
 __global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum) {
     __shared__ double sm[4];
     const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
     const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
     const int cnt = min(ETILE, M.rows * M.cols - start);
-    float acc = 0.0f;
-    for (int k = threadIdx.x; k < cnt; k += 256) {
-        const int i = start + k;
-        const float b = sg_fma(momentum, M.buf[i], sg::load_elem(M.grad, M.dtype, i));
-        M.buf[i] = b;
-        acc = sg_fma(b, b, acc);
+    double acc = 0.0;
+    if (M.vec8) {
+        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
+            const size_t i = (size_t)start + k;
+            float g[8], b[8], part = 0.0f;
+            load8(M.grad, M.dtype, i, g);
+            load8(M.buf, SG_F32, i, b);
+#pragma unroll
+            for (int e = 0; e < 8; e++) { b[e] = sg_fma(momentum, b[e], g[e]); part = sg_fma(b[e], b[e], part); }
+            store8(M.buf, SG_F32, i, b);
+            acc += (double)part;
+        }
+    } else {
+        float part = 0.0f;
+        for (int k = threadIdx.x; k < cnt; k += 256) {
+            const int i = start + k;
+            const float b = sg_fma(momentum, M.buf[i], sg::load_elem(M.grad, M.dtype, i));
+            M.buf[i] = b;
+            part = sg_fma(b, b, part);
+        }
+        acc = (double)part;
     }
-    const double tot = block_sum((double)acc, sm);
+    const double tot = block_sum(acc, sm);
     if (threadIdx.x == 0) B.partials[blockIdx.x] = tot;
 }
 
@@ -114,6 +170,17 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
     const float inv = B.inv_norm[mi];
     bf16_t* dst = M.wide ? M.Y : M.YT;
     const int ld = M.wide ? M.np : M.mp;
+    if (M.vec8) {
+        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
+            const int i = start + k, r = i / M.cols, c = i - r * M.cols;      // 8 elements of one row
+            float b[8];
+            load8(M.buf, SG_F32, (size_t)i, b);
+#pragma unroll
+            for (int e = 0; e < 8; e++) b[e] *= inv;
+            store8(dst, SG_BF16, (size_t)r * ld + c, b);
+        }
+        return;
+    }
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int i = start + k, r = i / M.cols, c = i - r * M.cols;
         dst[(size_t)r * ld + c] = sg::f_to_bf16_bits(M.buf[i] * inv);
@@ -152,8 +219,6 @@ __global__ __launch_bounds__(256) void k_transpose(Batch B, int to_yt, int only_
 // The Gram and polynomial products are symmetric: only tiles on or above the diagonal are
 // computed, each off-diagonal tile is also stored transposed.
 enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 // explicit global address space: a generic (flat) load would count against the LDS wait counter as well
 typedef const __attribute__((address_space(1))) u32x4* gvec_p;
 
@@ -165,7 +230,7 @@ __device__ __forceinline__ uint32_t bf16r(float v) {   // round to nearest even,
 }
 
 template <int EPI>
-__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
+__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_iter) {
     constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
     constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
     // LDS: two stages of {A tile, B tile}, each tile BT rows of LDS_ROW elements
@@ -185,10 +250,11 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     int tile = lb - prefix[mi];
 
     const bf16_t *A, *B;
-    bf16_t* C;
-    int K, lda, ldb, ldc, tm, tn;
+    bf16_t *C, *CT;         // CT: where the transposed tile goes (the symmetric products mirror into C itself)
+    int K, lda, ldb, ldc, ldct, tm, tn;
     if (EPI == EPI_APPLY) {
-        A = Mt.H; B = Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np;
+        A = Mt.H; B = yt_sel ? Mt.YT2 : Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np;
+        CT = yt_sel ? Mt.YT : Mt.YT2; ldct = Mt.mp;
         // bands of 8 tile columns: 32 tiles that run together span 4 x 8 tiles instead of 2 x 16,
         // which halves the panel bytes they pull into L2
         const int ntm = Mt.mp / BT, ntn = Mt.np / BT;
@@ -203,6 +269,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     } else {
         if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; }
         else { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; }
+        CT = C; ldct = ldc;
         const int nt = Mt.mp / BT;      // upper-triangular enumeration: row tm holds nt - tm tiles
         tm = 0;
         while (tile >= nt - tm) { tile -= nt - tm; tm++; }
@@ -279,27 +346,12 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     const int gcol0 = tn * BT + wn * (BT / 2);
     auto ktile = [&](int kt, auto set_c, auto store_c, auto load_c) {
         constexpr int S = decltype(set_c)::value;       // register set holding tile kt+1
-#ifdef SGX_NOLOAD
-        constexpr bool LD = false;
-#else
-        constexpr bool LD = decltype(load_c)::value != 0;
-#endif
-#ifdef SGX_NOSTORE
-        constexpr bool ST = false;
-#else
-        constexpr bool ST = decltype(store_c)::value != 0;
-#endif
+        constexpr bool LD = decltype(load_c)::value != 0, ST = decltype(store_c)::value != 0;
         const bf16_t* cur = smem + (kt & 1) * 2 * TILE_ELEMS;
         bf16_t* nxt = smem + ((kt + 1) & 1) * 2 * TILE_ELEMS;
-#ifdef SGX_NOLDSREAD
-        if (kt == 0)
-#endif
         lds_load(cur, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         // phase 0: k step 0 | read k step 1
-#ifdef SGX_NOLDSREAD
-        if (kt == 0)
-#endif
         lds_load(cur, 1, 1);
         mma(0);
 #pragma unroll
@@ -309,9 +361,6 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
         }
         __builtin_amdgcn_sched_barrier(0);
         // phase 1: k step 1 | read k step 2, write A of tile kt+1
-#ifdef SGX_NOLDSREAD
-        if (kt == 0)
-#endif
         lds_load(cur, 2, 0);
         if (ST) sstore_a(S, nxt);
         mma(1);
@@ -323,9 +372,6 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
         }
         __builtin_amdgcn_sched_barrier(0);
         // phase 2: k step 2 | read k step 3, write B of tile kt+1, load A of tile kt+3
-#ifdef SGX_NOLDSREAD
-        if (kt == 0)
-#endif
         lds_load(cur, 3, 1);
         if (ST) sstore_b(S, nxt);
         if (LD) gload_a(S, kt + 3);
@@ -347,9 +393,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
             if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-#ifndef SGX_NOBARRIER
         __syncthreads();
-#endif
     };
     using c0 = std::integral_constant<int, 0>;
     using c1 = std::integral_constant<int, 1>;
@@ -375,7 +419,10 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
     constexpr int EP_ROW = 128 + 4;     // floats per staged row
     static_assert(4 * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
     float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EP_ROW);
-    const bool mirror = (EPI != EPI_APPLY) && tm != tn;     // uniform over the workgroup
+    // uniform over the workgroup.  The apply step keeps the transposed copy of Y current for the
+    // next iteration's B operand; after the last iteration only tall matrices still need it (their
+    // parameter update reads the transposed orientation).
+    const bool mirror = (EPI == EPI_APPLY) ? (!last_iter || !Mt.wide) : (tm != tn);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int grow0 = tm * BT + wm * (BT / 2) + i * 32;
@@ -432,7 +479,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
 #pragma unroll
                 for (int k = 0; k < 4; k++)
                     t[k] = epb[(r8 * 8 + 2 * k) * EP_ROW + col] | (epb[(r8 * 8 + 2 * k + 1) * EP_ROW + col] << 16);
-                *reinterpret_cast<u32x4*>(C + (size_t)(gcol0 + col) * ldc + grow0 + r8 * 8) = t;
+                *reinterpret_cast<u32x4*>(CT + (size_t)(gcol0 + col) * ldct + grow0 + r8 * 8) = t;
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -440,17 +487,32 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt) {
 }
 
 // p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
-__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay) {
+__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int yt_sel) {
     const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
     const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
     const int cnt = min(ETILE, M.rows * M.cols - start);
-    const bf16_t* X = M.wide ? M.Y : M.YT;
+    const bf16_t* X = M.wide ? M.Y : (yt_sel ? M.YT2 : M.YT);
     const int ld = M.wide ? M.np : M.mp;
     // the reference's scalar arithmetic (csrc/ops.cpp:729-734)
     const float max_dim = (float)max(M.rows, M.cols);
     const float scale_factor = 0.2f * sqrtf(max_dim);
     const float neg_lr_scale = -lr * scale_factor / sqrtf(max_dim);
+    if (M.vec8) {
+        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
+            const int i = start + k, r = i / M.cols, c = i - r * M.cols;
+            float o[8], p[8];
+            load8(X, SG_BF16, (size_t)r * ld + c, o);
+            load8(M.param, M.dtype, (size_t)i, p);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                if (M.dtype == SG_F16) o[e] = __half2float(__float2half_rn(o[e]));
+                p[e] = sg_fma(neg_lr_scale, o[e], p[e]) * decay;
+            }
+            store8(M.param, M.dtype, (size_t)i, p);
+        }
+        return;
+    }
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int i = start + k, r = i / M.cols, c = i - r * M.cols;
         float o = sg::bf16_bits_to_f(X[(size_t)r * ld + c]);
@@ -494,9 +556,9 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         M.param = s.param; M.grad = s.grad; M.buf = s.buf;
         M.rows = (int)s.rows; M.cols = (int)s.cols; M.dtype = s.dtype;
         M.wide = s.rows <= s.cols;
+        M.vec8 = (s.cols % 8 == 0) && ((((uintptr_t)s.param | (uintptr_t)s.grad | (uintptr_t)s.buf) & 15u) == 0);
         M.m = (int)std::min(s.rows, s.cols); M.n = (int)std::max(s.rows, s.cols);
         M.mp = round_up(M.m, BT); M.np = round_up(M.n, BT);
-        M.pad_ = 0;
         const int et = (int)((s.rows * s.cols + ETILE - 1) / ETILE);
         M.etile0 = (int)etiles;
         etiles += et;
@@ -515,6 +577,7 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         // offsets for now; turned into pointers once the workspace base is known
         M.Y = (bf16_t*)take(2 * (size_t)M.mp * M.np);
         M.YT = (bf16_t*)take(2 * (size_t)M.mp * M.np);
+        M.YT2 = (bf16_t*)take(2 * (size_t)M.mp * M.np);
         M.G = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
         M.H = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
     }
@@ -550,7 +613,7 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     const int P = L.P;
     for (auto& M : L.mats) {
-        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.YT = (bf16_t*)(ws + (size_t)M.YT);
+        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.YT = (bf16_t*)(ws + (size_t)M.YT); M.YT2 = (bf16_t*)(ws + (size_t)M.YT2);
         M.G = (bf16_t*)(ws + (size_t)M.G); M.H = (bf16_t*)(ws + (size_t)M.H);
     }
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, hipMemcpyHostToDevice, st));
@@ -604,13 +667,13 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
         SG_LAUNCH_CHECK("muon transpose");
     }
     for (int it = 0; it < ns_steps; it++) {
-        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B);
-        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 1, 0, 0);    // YT <- Y^T for every matrix
+        const int sel = it & 1, last = it + 1 == ns_steps;
+        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         SG_LAUNCH_CHECK("muon newton-schulz");
     }
-    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd);
+    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1);
     SG_LAUNCH_CHECK("k_update");
     return 0;
 }
