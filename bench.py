@@ -22,7 +22,7 @@ BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (read + written) on the 25M-element workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs scaled by what the same counters read for a 1 GiB device copy; not measured by this script
-PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.675e9 + 1.626e9, "scan_summary": 0.619e9 + 0.150e9,
+PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.625e9 + 1.612e9, "scan_summary": 0.042e9 + 0.037e9,
                              "elementwise": 2.603e9 + 0.801e9}
 FLOP_PER_ELEMENT = 30e3         # arithmetic actually required per element (both scan directions + elementwise)
 VALU_PEAK_TFLOPS = 157.3
