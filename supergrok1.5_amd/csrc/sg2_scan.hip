@@ -44,11 +44,14 @@
 namespace sg2 {
 namespace {
 
-constexpr int LDS_STRIDE = SCAN_TT + 1;   // [row][timestep] rows padded so the 8 rows a wave reads sit in 8 banks
+constexpr int LDS_STRIDE = SCAN_TT + 4;   // [row][timestep] rows: 16-byte aligned (the recurrence fetches 4 timesteps per LDS read)
+                                          // and padded so the 8 rows a wave reads start 4 banks apart
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 #ifndef SG2_SCAN_UB
 #define SG2_SCAN_UB 8
 #endif
 constexpr int UB = SG2_SCAN_UB;           // timesteps per unrolled block of the recurrence
+static_assert(UB % 4 == 0 && SCAN_TT % UB == 0 && SCAN_TT == 64, "blocks are fetched 4 timesteps per LDS read; one ballot covers a tile");
 #ifdef SG2_SCAN_WAVES
 #define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
 #else
@@ -86,9 +89,13 @@ __device__ __forceinline__ float pair_tree_sum(float y) {
 // of dt / B (/ C / gate) and publishes its half of the x-branch rows.  HALF is
 // a template parameter so that every weight index is a compile-time constant
 // (scalar loads) and the register array is never indexed dynamically.
+// Returns whether every rotation angle of this timestep, over this half's columns, is small enough
+// for sg_sincos_small (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
+// rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
 template <bool OUT, int HALF>
-__device__ __forceinline__ void project_tile(const DirW& w, const float (&x)[DM], int tu, float* s_dt, float* s_xb,
-                                             float* s_B, float* s_C, float* s_gate) {
+__device__ __forceinline__ bool project_tile(const DirW& w, const float (&x)[DM], int tu, float* s_dt, float* s_xb,
+                                             float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
+    bool small = true;
     float xb[DI];
 #pragma unroll
     for (int jj = 0; jj < DI; jj++) {
@@ -103,7 +110,9 @@ __device__ __forceinline__ void project_tile(const DirW& w, const float (&x)[DM]
         float a = w.dt_b[jj];
 #pragma unroll
         for (int k = 0; k < DI; k++) a = sg_fma(w.dt_W[jj * DI + k], xb[k], a);
-        s_dt[jj * LDS_STRIDE + tu] = sg_softplus(a);
+        const float dtv = sg_softplus(a);
+        small = small && (dtv * s_fmax[jj] < SG_SINCOS_SMALL_LIMIT);
+        s_dt[jj * LDS_STRIDE + tu] = dtv;
         s_xb[jj * LDS_STRIDE + tu] = xb[jj];
     }
 #pragma unroll
@@ -130,6 +139,7 @@ __device__ __forceinline__ void project_tile(const DirW& w, const float (&x)[DM]
             s_gate[jj * LDS_STRIDE + tu] = sg_silu(z);
         }
     }
+    return small;
 }
 
 // scan state of one lane: OUT -> (he,ho) only; summary -> also the two columns of M
@@ -182,12 +192,14 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
 
 template <bool OUT>
 __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
-    __shared__ float s_dt[DI * LDS_STRIDE];
-    __shared__ float s_xb[DI * LDS_STRIDE];
-    __shared__ float s_B[DS * LDS_STRIDE];
-    __shared__ float s_C[OUT ? DS * LDS_STRIDE : 1];
-    __shared__ float s_gate[OUT ? DI * LDS_STRIDE : 1];
-    __shared__ float s_y[OUT ? DI * LDS_STRIDE : 1];
+    __shared__ __attribute__((aligned(16))) float s_dt[DI * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_xb[DI * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_B[DS * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_C[OUT ? DS * LDS_STRIDE : 1];
+    __shared__ __attribute__((aligned(16))) float s_gate[OUT ? DI * LDS_STRIDE : 1];
+    __shared__ __attribute__((aligned(16))) float s_y[OUT ? DI * LDS_STRIDE : 1];
+    __shared__ float s_fmax[DI];
+    __shared__ unsigned long long s_large[2];      // per projection half: bit t set = timestep t of the tile needs the full sin/cos
 
     const int per_dir = OUT ? pl.chunks : pl.wchunks;
     const int dir = (int)blockIdx.x >= per_dir ? 1 : 0;
@@ -215,6 +227,15 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
     const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
     const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
+
+    {   // largest |frequency| of each column's 8 pairs
+        float f = sg_abs(freq);
+        f = sg_max(f, dpp_quad_swap1(f));
+        f = sg_max(f, dpp_quad_swap2(f));
+        f = sg_max(f, dpp_half_mirror(f));
+        if (p == 0) s_fmax[j] = f;
+        __syncthreads();
+    }
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     if (OUT) {
@@ -254,11 +275,17 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
 #pragma unroll
             for (int k = 0; k < DM; k++) x[k] = sg_fma(Wi[2 * k + 1], s, Wi[2 * k] * g) + bi[k];
         }
+        bool small_t;
         if (half == 0)
-            project_tile<OUT, 0>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate);
+            small_t = project_tile<OUT, 0>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
         else
-            project_tile<OUT, 1>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate);
+            small_t = project_tile<OUT, 1>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
+        {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
+            const unsigned long long large = __builtin_amdgcn_ballot_w64(!small_t);
+            if (tu == 0) s_large[half] = large;
+        }
         __syncthreads();
+        const unsigned long long large = s_large[half];
 
         // ---------------- phase B: the recurrence over the tile, lane = (j,p)
         const float* __restrict__ r_dt = s_dt + j * LDS_STRIDE;
@@ -270,24 +297,26 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         int k0 = 0;
         for (; k0 + UB <= cnt; k0 += UB) {
             float dt[UB], xv[UB], Be[UB], Bo[UB], Ce[UB], Co[UB], y[UB];
-            bool small = true;
 #pragma unroll
-            for (int q = 0; q < UB; q++) {
-                dt[q] = r_dt[k0 + q];
-                xv[q] = r_xb[k0 + q];
-                Be[q] = r_Be[k0 + q];
-                Bo[q] = r_Bo[k0 + q];
-                Ce[q] = OUT ? r_Ce[k0 + q] : 0.0f;
-                Co[q] = OUT ? r_Co[k0 + q] : 0.0f;
-                small = small && (sg_abs(dt[q] * freq) < SG_SINCOS_SMALL_LIMIT);
+            for (int q = 0; q < UB; q += 4) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(r_dt + k0 + q), b = *reinterpret_cast<const f32x4*>(r_xb + k0 + q);
+                const f32x4 c = *reinterpret_cast<const f32x4*>(r_Be + k0 + q), d = *reinterpret_cast<const f32x4*>(r_Bo + k0 + q);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { dt[q + e] = a[e]; xv[q + e] = b[e]; Be[q + e] = c[e]; Bo[q + e] = d[e]; Ce[q + e] = 0.0f; Co[q + e] = 0.0f; }
+                if (OUT) {
+                    const f32x4 f = *reinterpret_cast<const f32x4*>(r_Ce + k0 + q), g = *reinterpret_cast<const f32x4*>(r_Co + k0 + q);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { Ce[q + e] = f[e]; Co[q + e] = g[e]; }
+                }
             }
-            if (__builtin_amdgcn_ballot_w64(!small) == 0)
+            if (((large >> k0) & ((1ull << UB) - 1)) == 0)
                 block_steps<OUT, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             else
                 block_steps<OUT, false>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             if (OUT && p == 0) {
 #pragma unroll
-                for (int q = 0; q < UB; q++) s_y[j * LDS_STRIDE + k0 + q] = y[q];
+                for (int q = 0; q < UB; q += 4)
+                    *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + q]) = f32x4{y[q], y[q + 1], y[q + 2], y[q + 3]};
             }
         }
         for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
