@@ -51,7 +51,7 @@ def build_workload(name, device):
     return shapes, state, grad_sets, sharps, weights
 
 
-def cpu_baseline(sample_elems_target=1_000_000):
+def cpu_baseline(sample_elems_target=4_000_000):
     """The CPU restatement of the reference's algorithm (sequential scan, the
     path grokking_optimizers/supergrok2.py:430-470 takes on CPU) timed on one
     host core over a bounded sample of the same parameter set."""
