@@ -222,6 +222,98 @@ typedef struct Sg15RestoreTensor {
 int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/* ================== the other fused steps of the reference ================== */
+
+/* One tensor of an Adam-family fused step: the i-th entries of the tensor
+ * vectors of the reference's *_fused_step functions.  Fields an entry point
+ * does not use are ignored (may be NULL / 0). */
+typedef struct SgFamilyTensor {
+    void* param;        /* [numel] dtype, updated in place */
+    void* grad;         /* [numel] dtype; rescaled in place when global-norm clipping is active */
+    float* exp_avg;     /* [numel] fp32 */
+    float* exp_avg_sq;  /* [numel] fp32 (not Lion) */
+    float* aux;         /* [numel] fp32: GrokAdamW ema, Prodigy s, SuperGrok v1.1 mu */
+    const void* aux2;   /* Prodigy: param_init [numel] fp32; SuperGrok v1.1: sharpness [numel] dtype */
+    int64_t numel;
+    int32_t dtype;
+    float bc1, bc2;     /* 1 - beta1^step, 1 - beta2^step as the caller computed them */
+    float alpha, beta1; /* SuperGrok v1.1 per-layer values */
+} SgFamilyTensor;
+
+/* 1 -> H -> 1 ReLU amplifier of NeuralGrok (first and last Linear of its _Amplifier). */
+typedef struct SgAmplifier {
+    const float* W1;    /* [hidden,1] */
+    const float* b1;    /* [hidden]   */
+    const float* W2;    /* [1,hidden] */
+    const float* b2;    /* [1]        */
+    int32_t hidden;     /* <= 256 */
+} SgAmplifier;
+
+/* Workspace for every entry point of this section: the elementwise bookkeeping
+ * plus one float per element (SuperGrok v1.1 keeps the smart gradient there
+ * between its two passes). */
+size_t sg_family_workspace_bytes(int num_tensors, const int64_t* numels);
+
+/* GrokAdamW: global-norm clip, ema = alpha*ema + (1-alpha)*g, g' = g + lamb*ema,
+ * AdamW on g'.  Replaces grokadamw_fused_step (csrc/ops.cpp:311-353;
+ * launch_fused_grokadamw_step, csrc/grokadamw_kernels.cu). */
+int sg_grokadamw_step(int num_tensors, const SgFamilyTensor* tensors, float alpha, float lamb, float beta1, float beta2,
+                      float lr, float wd, float eps, float grad_clip_norm, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/* NeuralGrok: global-norm clip, g' = g * (alpha_amp * MLP(g) + beta_amp), AdamW
+ * on g' in one pass.  Replaces neuralgrok_fused_step (csrc/ops.cpp:360-417;
+ * fused_neuralgrok_full_step_kernel, csrc/neuralgrok_kernels.cu). */
+int sg_neuralgrok_step(int num_tensors, const SgFamilyTensor* tensors, const SgAmplifier* amp, float alpha_amp,
+                       float beta_amp, float beta1, float beta2, float lr, float wd, float eps, float grad_clip_norm,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* Prodigy: num = sum g.(p - p0), den = sum s reduced on the device;
+ * d_lr <- max(d_lr, |num|/(den+1e-12)) when den > 1e-30; then the d_lr-scaled
+ * Adam step.  The new d_lr is computed on the device, consumed by the step
+ * kernel from device memory, and copied to *d_lr_out (the call synchronises
+ * the stream for that copy, as the reference's own single sync does).
+ * Replaces prodigy_fused_step (csrc/ops.cpp:424-506; csrc/prodigy_kernels.cu:50-170). */
+int sg_prodigy_step(int num_tensors, const SgFamilyTensor* tensors, float d_lr, float beta1, float beta2, float lr,
+                    float wd, float eps, float* d_lr_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Lion: p -= lr*(sign(beta1*m + (1-beta1)*g) + wd*p); m = beta2*m + (1-beta2)*g.
+ * Replaces lion_fused_step (csrc/ops.cpp:536-560; csrc/lion_kernels.cu:20-56). */
+int sg_lion_step(int num_tensors, const SgFamilyTensor* tensors, float lr, float beta1, float beta2, float wd,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* SuperGrok v1.1: global-norm clip; mu EMA and the 2->H->1 meta-net (pass 1,
+ * smart gradient kept in the workspace); per tensor the cosine gate
+ * sigmoid(T * <smart,mu> / (|smart||mu| + 1e-8)) from sums reduced on the
+ * device, lamb_eff = ramp*gate*lamb (0 when ramp <= 0); Adam with decoupled
+ * decay (pass 2).  No host synchronisation: the reference reads the gate back
+ * once per tensor.  Replaces supergrok11_fused_step (csrc/ops.cpp:209-288;
+ * csrc/supergrok11_kernels.cu).  net->gelu_mode as for sg15_fused_step. */
+int sg11_fused_step(int num_tensors, const SgFamilyTensor* tensors, const Sg15Net* net, float beta2, float lr, float wd,
+                    float eps, float lamb, float ramp, float gate_temperature, float grad_clip_norm, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+/* LookSAM.  The ascent step is sg15_sam_perturb (looksam_perturb_all is the same
+ * computation, csrc/ops.cpp:566-590). */
+typedef struct SgLookSamTensor {
+    void* a;            /* restore: param;  directions: v_dir (fp32);      adjust: grad (dtype)  */
+    const void* b;      /* restore: backup; directions: sam_grad (dtype);  adjust: v_dir (fp32)  */
+    const void* c;      /*                  directions: normal_grad (dtype)                      */
+    int64_t numel;
+    int32_t dtype;
+} SgLookSamTensor;
+/* param <- backup (looksam_restore_all, csrc/ops.cpp:592-605). */
+int sg_looksam_restore(int num_tensors, const SgLookSamTensor* tensors, void* workspace, size_t workspace_bytes,
+                       void* stream);
+/* v = (g_sam - g)/|g_sam - g| per tensor, left untouched when the norm is below
+ * 1e-12; norms reduced on the device (looksam_compute_directions,
+ * csrc/ops.cpp:607-630; launch_looksam_direction). */
+int sg_looksam_directions(int num_tensors, const SgLookSamTensor* tensors, void* workspace, size_t workspace_bytes,
+                          void* stream);
+/* g += la*|g| * v per tensor (looksam_adjust_grads, csrc/ops.cpp:632-652). */
+int sg_looksam_adjust(int num_tensors, const SgLookSamTensor* tensors, float la, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
 /* ================================ Muon ==================================== */
 
 /* One 2-D parameter of the Muon step: the i-th entries of the vectors of

@@ -373,6 +373,215 @@ void supergrok2_mamba_peer_step(
         num_experts, expert_counts);
 }
 
+
+// ---- the other fused steps (csrc/ops.h:408-508 of the reference: same names, same argument order) ----------
+
+namespace {
+struct FamilyArgs {
+    std::vector<SgFamilyTensor> ts;
+    std::vector<int64_t> numels;
+    const torch::Tensor* first = nullptr;
+    torch::Tensor ws;
+    void make_ws() { ws = make_workspace(sg_family_workspace_bytes((int)ts.size(), numels.data()), *first); }
+};
+
+// fills one SgFamilyTensor per tensor with a gradient; aux/aux2 may be NULL lists
+void gather_family(const char* fn, FamilyArgs* A, std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads,
+                   std::vector<torch::Tensor>* eas, std::vector<torch::Tensor>* easqs, std::vector<torch::Tensor>* aux,
+                   std::vector<torch::Tensor>* aux2, bool aux2_f32, const std::vector<float>* bc1, const std::vector<float>* bc2,
+                   const std::vector<float>* alphas, const std::vector<float>* beta1s) {
+    for (size_t i = 0; i < params.size(); i++) {
+        if (!grads[i].defined() || grads[i].numel() == 0) continue;
+        check_gpu(params[i], fn, "param");
+        check_gpu(grads[i], fn, "grad");
+        TORCH_CHECK(params[i].scalar_type() == grads[i].scalar_type(), fn, ": param/grad dtype mismatch");
+        TORCH_CHECK(params[i].numel() == grads[i].numel(), fn, ": param/grad size mismatch");
+        SgFamilyTensor t = {};
+        t.param = params[i].data_ptr();
+        t.grad = grads[i].data_ptr();
+        if (eas) { check_f32((*eas)[i], fn, "exp_avg"); t.exp_avg = (*eas)[i].data_ptr<float>(); }
+        if (easqs) { check_f32((*easqs)[i], fn, "exp_avg_sq"); t.exp_avg_sq = (*easqs)[i].data_ptr<float>(); }
+        if (aux) { check_f32((*aux)[i], fn, "state"); t.aux = (*aux)[i].data_ptr<float>(); }
+        if (aux2) {
+            if (aux2_f32) check_f32((*aux2)[i], fn, "param_init");
+            else {
+                check_gpu((*aux2)[i], fn, "sharpness");
+                TORCH_CHECK((*aux2)[i].scalar_type() == grads[i].scalar_type(), fn, ": sharpness must have the gradient's dtype");
+            }
+            TORCH_CHECK((*aux2)[i].numel() == grads[i].numel(), fn, ": size mismatch");
+            t.aux2 = (*aux2)[i].data_ptr();
+        }
+        t.numel = grads[i].numel();
+        t.dtype = dtype_code(grads[i], "grad");
+        t.bc1 = bc1 ? (*bc1)[i] : 1.0f;
+        t.bc2 = bc2 ? (*bc2)[i] : 1.0f;
+        t.alpha = alphas ? (*alphas)[i] : 0.0f;
+        t.beta1 = beta1s ? (*beta1s)[i] : 0.0f;
+        A->ts.push_back(t);
+        A->numels.push_back(t.numel);
+        if (!A->first) A->first = &grads[i];
+    }
+}
+
+void bias_corrections(const std::vector<int64_t>& steps, float beta1, float beta2, std::vector<float>* bc1, std::vector<float>* bc2) {
+    for (int64_t st : steps) {      // float pow, as the reference computes them (csrc/ops.cpp:333-334)
+        bc1->push_back(1.0f - std::pow(beta1, static_cast<float>(st)));
+        bc2->push_back(1.0f - std::pow(beta2, static_cast<float>(st)));
+    }
+}
+}  // namespace
+
+void grokadamw_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
+                          std::vector<torch::Tensor>& exp_avg_sqs, std::vector<torch::Tensor>& emas, std::vector<int64_t>& steps,
+                          float alpha, float lamb, float beta1, float beta2, float lr, float wd, float eps, float grad_clip_norm) {
+    const char* fn = "grokadamw_fused_step";
+    std::vector<float> bc1, bc2;
+    bias_corrections(steps, beta1, beta2, &bc1, &bc2);
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, &exp_avg_sqs, &emas, nullptr, false, &bc1, &bc2, nullptr, nullptr);
+    if (A.ts.empty()) return;
+    A.make_ws();
+    check_status(sg_grokadamw_step((int)A.ts.size(), A.ts.data(), alpha, lamb, beta1, beta2, lr, wd, eps, grad_clip_norm, A.ws.data_ptr(),
+                                   (size_t)A.ws.numel(), current_stream(*A.first)), fn);
+}
+
+void neuralgrok_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
+                           std::vector<torch::Tensor>& exp_avg_sqs, std::vector<int64_t>& steps, torch::Tensor W1, torch::Tensor b1,
+                           torch::Tensor W2, torch::Tensor b2, float alpha_amp, float beta_amp, int hidden_dim, float beta1, float beta2,
+                           float lr, float wd, float eps, float grad_clip_norm) {
+    const char* fn = "neuralgrok_fused_step";
+    std::vector<float> bc1, bc2;
+    bias_corrections(steps, beta1, beta2, &bc1, &bc2);
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, &exp_avg_sqs, nullptr, nullptr, false, &bc1, &bc2, nullptr, nullptr);
+    if (A.ts.empty()) return;
+    auto W1f = W1.to(torch::kFloat32).contiguous(), b1f = b1.to(torch::kFloat32).contiguous();
+    auto W2f = W2.to(torch::kFloat32).contiguous(), b2f = b2.to(torch::kFloat32).contiguous();
+    check_f32(W1f, fn, "W1"); check_f32(b1f, fn, "b1"); check_f32(W2f, fn, "W2"); check_f32(b2f, fn, "b2");
+    TORCH_CHECK(W1f.numel() == hidden_dim && b1f.numel() == hidden_dim && W2f.numel() == hidden_dim && b2f.numel() == 1, fn,
+                ": amplifier weight shapes do not match hidden_dim");
+    SgAmplifier amp = {W1f.data_ptr<float>(), b1f.data_ptr<float>(), W2f.data_ptr<float>(), b2f.data_ptr<float>(), hidden_dim};
+    A.make_ws();
+    check_status(sg_neuralgrok_step((int)A.ts.size(), A.ts.data(), &amp, alpha_amp, beta_amp, beta1, beta2, lr, wd, eps, grad_clip_norm,
+                                    A.ws.data_ptr(), (size_t)A.ws.numel(), current_stream(*A.first)), fn);
+}
+
+float prodigy_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
+                         std::vector<torch::Tensor>& exp_avg_sqs, std::vector<torch::Tensor>& s_bufs,
+                         std::vector<torch::Tensor>& param_inits, std::vector<int64_t>& steps, float d_lr, float beta1, float beta2,
+                         float lr, float wd, float eps) {
+    const char* fn = "prodigy_fused_step";
+    std::vector<float> bc1, bc2;
+    bias_corrections(steps, beta1, beta2, &bc1, &bc2);
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, &exp_avg_sqs, &s_bufs, &param_inits, true, &bc1, &bc2, nullptr, nullptr);
+    if (A.ts.empty()) return d_lr;
+    A.make_ws();
+    float out = d_lr;
+    check_status(sg_prodigy_step((int)A.ts.size(), A.ts.data(), d_lr, beta1, beta2, lr, wd, eps, &out, A.ws.data_ptr(), (size_t)A.ws.numel(),
+                                 current_stream(*A.first)), fn);
+    return out;
+}
+
+void lion_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs, float lr,
+                     float beta1, float beta2, float wd) {
+    const char* fn = "lion_fused_step";
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, nullptr, nullptr, nullptr, false, nullptr, nullptr, nullptr, nullptr);
+    if (A.ts.empty()) return;
+    A.make_ws();
+    check_status(sg_lion_step((int)A.ts.size(), A.ts.data(), lr, beta1, beta2, wd, A.ws.data_ptr(), (size_t)A.ws.numel(),
+                              current_stream(*A.first)), fn);
+}
+
+void supergrok11_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
+                            std::vector<torch::Tensor>& exp_avg_sqs, std::vector<torch::Tensor>& mus,
+                            std::vector<torch::Tensor>& sharpness_cache, std::vector<int64_t>& steps, std::vector<float>& layer_alphas,
+                            std::vector<float>& layer_beta1s, torch::Tensor W1, torch::Tensor b1, torch::Tensor W2, torch::Tensor b2,
+                            float rescale, int hidden_dim, float beta2, float lr, float wd_eff, float eps, float lamb, float ramp,
+                            float gate_temperature, float grad_clip_norm) {
+    const char* fn = "supergrok11_fused_step";
+    std::vector<float> bc1(params.size(), 1.0f), bc2(params.size(), 1.0f);
+    for (size_t i = 0; i < params.size(); i++) {
+        if (!grads[i].defined() || grads[i].numel() == 0) continue;
+        steps[i] += 1;   // pybind's copy of the Python list, exactly as in the reference (csrc/ops.cpp:237)
+        const float step = static_cast<float>(steps[i]);
+        bc1[i] = 1.0f - std::pow(layer_beta1s[i], step);
+        bc2[i] = 1.0f - std::pow(beta2, step);
+    }
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, &exp_avg_sqs, &mus, &sharpness_cache, false, &bc1, &bc2, &layer_alphas, &layer_beta1s);
+    if (A.ts.empty()) return;
+    auto W1f = W1.to(torch::kFloat32).contiguous(), b1f = b1.to(torch::kFloat32).contiguous();
+    auto W2f = W2.to(torch::kFloat32).contiguous(), b2f = b2.to(torch::kFloat32).contiguous();
+    check_f32(W1f, fn, "W1"); check_f32(b1f, fn, "b1"); check_f32(W2f, fn, "W2"); check_f32(b2f, fn, "b2");
+    TORCH_CHECK(W1f.numel() == 2 * hidden_dim && b1f.numel() == hidden_dim && W2f.numel() == hidden_dim && b2f.numel() == 1, fn,
+                ": meta-net weight shapes do not match hidden_dim");
+    Sg15Net net = {W1f.data_ptr<float>(), b1f.data_ptr<float>(), W2f.data_ptr<float>(), b2f.data_ptr<float>(), hidden_dim, rescale,
+                   g_sg15_gelu_mode};
+    A.make_ws();
+    check_status(sg11_fused_step((int)A.ts.size(), A.ts.data(), &net, beta2, lr, wd_eff, eps, lamb, ramp, gate_temperature, grad_clip_norm,
+                                 A.ws.data_ptr(), (size_t)A.ws.numel(), current_stream(*A.first)), fn);
+}
+
+std::vector<torch::Tensor> supergrok11_sam_perturb_all(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, float rho) {
+    return supergrok15_sam_perturb_all(params, grads, rho);
+}
+void supergrok11_sharpness_restore_all(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& sharpness_cache,
+                                       std::vector<torch::Tensor>& backups, std::vector<torch::Tensor>& sam_grads,
+                                       std::vector<torch::Tensor>& normal_grads) {
+    supergrok15_sharpness_restore_all(params, sharpness_cache, backups, sam_grads, normal_grads);
+}
+
+std::vector<torch::Tensor> looksam_perturb_all(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, float rho) {
+    return supergrok15_sam_perturb_all(params, grads, rho);
+}
+
+namespace {
+void looksam_call(const char* fn, int mode, std::vector<torch::Tensor>& a, std::vector<torch::Tensor>& b, std::vector<torch::Tensor>* c, float la) {
+    std::vector<SgLookSamTensor> ts;
+    std::vector<int64_t> numels;
+    const torch::Tensor* first = nullptr;
+    for (size_t i = 0; i < a.size(); i++) {
+        // mode 0: a=param, b=backup; mode 1: a=v_dir, b=sam_grad, c=normal_grad; mode 2: a=grad, b=v_dir
+        const torch::Tensor& typed = (mode == 1) ? b[i] : a[i];
+        if (!a[i].defined() || !b[i].defined() || a[i].numel() == 0 || b[i].numel() == 0) continue;
+        if (mode == 1 && (!(*c)[i].defined() || (*c)[i].numel() == 0)) continue;
+        check_gpu(a[i], fn, "tensor");
+        check_gpu(b[i], fn, "tensor");
+        if (mode == 0) TORCH_CHECK(a[i].scalar_type() == b[i].scalar_type(), fn, ": param/backup dtype mismatch");
+        if (mode == 1) {
+            check_f32(a[i], fn, "v_dir");
+            check_gpu((*c)[i], fn, "normal_grad");
+            TORCH_CHECK(b[i].scalar_type() == (*c)[i].scalar_type(), fn, ": gradient dtype mismatch");
+        }
+        if (mode == 2) check_f32(b[i], fn, "v_dir");
+        TORCH_CHECK(a[i].numel() == b[i].numel(), fn, ": size mismatch");
+        ts.push_back({a[i].data_ptr(), b[i].data_ptr(), mode == 1 ? (*c)[i].data_ptr() : nullptr, typed.numel(), dtype_code(typed, "tensor")});
+        numels.push_back(typed.numel());
+        if (!first) first = &a[i];
+    }
+    if (ts.empty()) return;
+    auto ws = make_workspace(sg_family_workspace_bytes((int)ts.size(), numels.data()), *first);
+    int rc = 0;
+    if (mode == 0) rc = sg_looksam_restore((int)ts.size(), ts.data(), ws.data_ptr(), (size_t)ws.numel(), current_stream(*first));
+    if (mode == 1) rc = sg_looksam_directions((int)ts.size(), ts.data(), ws.data_ptr(), (size_t)ws.numel(), current_stream(*first));
+    if (mode == 2) rc = sg_looksam_adjust((int)ts.size(), ts.data(), la, ws.data_ptr(), (size_t)ws.numel(), current_stream(*first));
+    check_status(rc, fn);
+}
+}  // namespace
+
+void looksam_restore_all(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& backups) {
+    looksam_call("looksam_restore_all", 0, params, backups, nullptr, 0.0f);
+}
+void looksam_compute_directions(std::vector<torch::Tensor>& v_dirs, std::vector<torch::Tensor>& sam_grads,
+                                std::vector<torch::Tensor>& normal_grads) {
+    looksam_call("looksam_compute_directions", 1, v_dirs, sam_grads, &normal_grads, 0.0f);
+}
+void looksam_adjust_grads(std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& v_dirs, float la) {
+    looksam_call("looksam_adjust_grads", 2, grads, v_dirs, nullptr, la);
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "Grokking optimizers: fused steps on MI355X (hand-written HIP behind the reference's _ops surface)";
     m.def("supergrok15_fused_step", &supergrok15_fused_step, "SuperGrok1.5: fused clip + mu + meta-net + gating + adam + progressive wd",
@@ -383,6 +592,30 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("supergrok15_sam_perturb_all", &supergrok15_sam_perturb_all, py::arg("params"), py::arg("grads"), py::arg("rho"));
     m.def("supergrok15_sharpness_restore_all", &supergrok15_sharpness_restore_all, py::arg("params"), py::arg("sharpness_cache"),
           py::arg("backups"), py::arg("sam_grads"), py::arg("normal_grads"));
+    m.def("supergrok11_fused_step", &supergrok11_fused_step, "SuperGrok1.1: fused clip + mu + meta-net + cosine gate + adam",
+          py::arg("params"), py::arg("grads"), py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("mus"), py::arg("sharpness_cache"),
+          py::arg("steps"), py::arg("layer_alphas"), py::arg("layer_beta1s"), py::arg("W1"), py::arg("b1"), py::arg("W2"), py::arg("b2"),
+          py::arg("rescale"), py::arg("hidden_dim"), py::arg("beta2"), py::arg("lr"), py::arg("wd_eff"), py::arg("eps"), py::arg("lamb"),
+          py::arg("ramp"), py::arg("gate_temperature"), py::arg("grad_clip_norm"));
+    m.def("supergrok11_sam_perturb_all", &supergrok11_sam_perturb_all, py::arg("params"), py::arg("grads"), py::arg("rho"));
+    m.def("supergrok11_sharpness_restore_all", &supergrok11_sharpness_restore_all, py::arg("params"), py::arg("sharpness_cache"),
+          py::arg("backups"), py::arg("sam_grads"), py::arg("normal_grads"));
+    m.def("grokadamw_fused_step", &grokadamw_fused_step, "GrokAdamW: fused EMA filter + amplification + Adam", py::arg("params"),
+          py::arg("grads"), py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("emas"), py::arg("steps"), py::arg("alpha"),
+          py::arg("lamb"), py::arg("beta1"), py::arg("beta2"), py::arg("lr"), py::arg("wd"), py::arg("eps"), py::arg("grad_clip_norm"));
+    m.def("neuralgrok_fused_step", &neuralgrok_fused_step, "NeuralGrok: fused MLP amplifier + Adam", py::arg("params"), py::arg("grads"),
+          py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("steps"), py::arg("W1"), py::arg("b1"), py::arg("W2"), py::arg("b2"),
+          py::arg("alpha_amp"), py::arg("beta_amp"), py::arg("hidden_dim"), py::arg("beta1"), py::arg("beta2"), py::arg("lr"),
+          py::arg("wd"), py::arg("eps"), py::arg("grad_clip_norm"));
+    m.def("prodigy_fused_step", &prodigy_fused_step, "Prodigy: distance-aware self-tuning Adam; returns the new d_lr", py::arg("params"),
+          py::arg("grads"), py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("s_bufs"), py::arg("param_inits"), py::arg("steps"),
+          py::arg("d_lr"), py::arg("beta1"), py::arg("beta2"), py::arg("lr"), py::arg("wd"), py::arg("eps"));
+    m.def("lion_fused_step", &lion_fused_step, "Lion: fused sign-momentum step", py::arg("params"), py::arg("grads"), py::arg("exp_avgs"),
+          py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("wd"));
+    m.def("looksam_perturb_all", &looksam_perturb_all, py::arg("params"), py::arg("grads"), py::arg("rho"));
+    m.def("looksam_restore_all", &looksam_restore_all, py::arg("params"), py::arg("backups"));
+    m.def("looksam_compute_directions", &looksam_compute_directions, py::arg("v_dirs"), py::arg("sam_grads"), py::arg("normal_grads"));
+    m.def("looksam_adjust_grads", &looksam_adjust_grads, py::arg("grads"), py::arg("v_dirs"), py::arg("la"));
     m.def("supergrok15_set_gelu_mode", &supergrok15_set_gelu_mode, py::arg("mode"));
     m.def("grokfast_fused_step", &grokfast_fused_step, "Grokfast: fused EMA update + gradient amplification", py::arg("grads"),
           py::arg("ema_bufs"), py::arg("alpha"), py::arg("lamb"));

@@ -13,159 +13,10 @@
 
 #include "sg_common.hpp"
 
+#include "sg_elemwise.hpp"
+
 namespace sgew {
 namespace {
-
-constexpr int TILE = 4096;
-constexpr int THREADS = 256;
-constexpr int MAX_HIDDEN = 256;
-
-struct Red {            // result of the device-side norm reduction
-    double norm_sq;
-    float norm;         // sqrt(norm_sq)
-    float coef;         // clip coefficient (1 when clipping is inactive)
-    int clip_on;
-    int pad_;
-};
-
-struct Layout {
-    int n, tiles;
-    size_t off_recs, off_nrecs, off_prefix, off_partials, off_red, bytes;
-};
-constexpr size_t REC_BYTES = 96;   // upper bound of any per-tensor record below
-constexpr size_t NREC_BYTES = 24;  // view of a record used by the norm reduction
-
-int make_layout(int n, const int64_t* numels, Layout* L) {
-    int64_t tiles = 0, total = 0;
-    for (int i = 0; i < n; i++) {
-        if (numels[i] < 0 || numels[i] > 0x7fffffff) return sg::fail("tensor %d: bad numel %lld", i, (long long)numels[i]);
-        tiles += (numels[i] + TILE - 1) / TILE;
-        total += numels[i];
-    }
-    if (tiles > 0x7fffffff) return sg::fail("too many elements");
-    L->n = n;
-    L->tiles = (int)tiles;
-    size_t o = 0;
-    auto take = [&](size_t b) { size_t r = o; o = sg::align_up(o + b, 256); return r; };
-    L->off_recs = take(REC_BYTES * (size_t)n);
-    L->off_nrecs = take(NREC_BYTES * (size_t)n);
-    L->off_prefix = take(sizeof(int) * (size_t)(n + 1));
-    L->off_partials = take(sizeof(double) * (size_t)(tiles + 1));
-    L->off_red = take(sizeof(Red));
-    L->bytes = o;
-    return 0;
-}
-
-template <class Rec>
-struct Batch {
-    const Rec* recs;
-    const int* prefix;
-    int n, tiles;
-    double* partials;
-    Red* red;
-    void* nrecs;      // device room for n norm-reduction views
-};
-
-// Upload records + tile prefix; fills the Batch.  Rec must have .numel.
-template <class Rec>
-int upload(const std::vector<Rec>& recs, void* workspace, size_t ws_bytes, hipStream_t st, Batch<Rec>* B) {
-    static_assert(sizeof(Rec) <= REC_BYTES, "record too large");
-    const int n = (int)recs.size();
-    std::vector<int64_t> numels(n);
-    for (int i = 0; i < n; i++) numels[i] = recs[i].numel;
-    Layout L;
-    if (make_layout(n, numels.data(), &L)) return 1;
-    if (!workspace || ws_bytes < L.bytes) return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, ws_bytes);
-    if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
-    std::vector<int> prefix(n + 1, 0);
-    for (int i = 0; i < n; i++) prefix[i + 1] = prefix[i] + (int)((numels[i] + TILE - 1) / TILE);
-    unsigned char* ws = static_cast<unsigned char*>(workspace);
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_recs, recs.data(), sizeof(Rec) * (size_t)n, hipMemcpyHostToDevice, st));
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_prefix, prefix.data(), sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, st));
-    B->recs = reinterpret_cast<const Rec*>(ws + L.off_recs);
-    B->prefix = reinterpret_cast<const int*>(ws + L.off_prefix);
-    B->n = n;
-    B->tiles = L.tiles;
-    B->partials = reinterpret_cast<double*>(ws + L.off_partials);
-    B->red = reinterpret_cast<Red*>(ws + L.off_red);
-    B->nrecs = ws + L.off_nrecs;
-    return 0;
-}
-
-template <class Rec>
-__device__ __forceinline__ const Rec& tile_rec(const Batch<Rec>& B, int tile, int* start, int* cnt) {
-    const int ti = sg::upper_seg(B.prefix, B.n, tile);
-    const Rec& R = B.recs[ti];
-    *start = (tile - B.prefix[ti]) * TILE;
-    *cnt = min(TILE, (int)R.numel - *start);
-    return R;
-}
-
-// ---- deterministic sum of squares -------------------------------------------
-__device__ __forceinline__ double block_sum(double v, double* sm /*[4]*/) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_down(v, d, 64);
-    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const double r = (sm[0] + sm[1]) + (sm[2] + sm[3]);
-    __syncthreads();
-    return r;
-}
-
-struct NormRec {
-    const void* grad;
-    int64_t numel;
-    int32_t dtype;
-};
-
-__global__ __launch_bounds__(THREADS) void k_sumsq_partial(Batch<NormRec> B) {
-    __shared__ double sm[4];
-    int start, cnt;
-    const NormRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
-    float acc = 0.0f;
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
-        const float g = sg::load_elem(R.grad, R.dtype, start + k);
-        acc = sg_fma(g, g, acc);
-    }
-    const double tot = block_sum((double)acc, sm);
-    if (threadIdx.x == 0) B.partials[blockIdx.x] = tot;
-}
-
-// clip_norm > 0: clipping semantics of clip_grad_norms_device_side; rho_mode: nothing extra (norm is read by the consumer)
-__global__ __launch_bounds__(THREADS) void k_sumsq_final(const double* __restrict__ partials, int tiles, float clip_norm, Red* red) {
-    __shared__ double sm[4];
-    double acc = 0.0;
-    for (int k = threadIdx.x; k < tiles; k += THREADS) acc += partials[k];
-    const double tot = block_sum(acc, sm);
-    if (threadIdx.x == 0) {
-        const float norm = (float)sqrt(tot);
-        red->norm_sq = tot;
-        red->norm = norm;
-        const bool on = clip_norm > 0.0f && norm > clip_norm;
-        red->clip_on = on ? 1 : 0;
-        red->coef = on ? clip_norm / (norm + 1e-6f) : 1.0f;
-    }
-}
-
-template <class Rec>
-int reduce_sumsq(const std::vector<Rec>& recs, const Batch<Rec>& B, float clip_norm, hipStream_t st) {
-    static_assert(sizeof(NormRec) == NREC_BYTES, "NormRec layout");
-    std::vector<NormRec> nr(recs.size());
-    for (size_t i = 0; i < recs.size(); i++) nr[i] = {recs[i].grad, recs[i].numel, recs[i].dtype};
-    SG_HIP_CHECK(hipMemcpyAsync(B.nrecs, nr.data(), sizeof(NormRec) * nr.size(), hipMemcpyHostToDevice, st));
-    Batch<NormRec> NB;
-    NB.recs = reinterpret_cast<const NormRec*>(B.nrecs);
-    NB.prefix = B.prefix;
-    NB.n = B.n;
-    NB.tiles = B.tiles;
-    NB.partials = B.partials;
-    NB.red = B.red;
-    NB.nrecs = nullptr;
-    hipLaunchKernelGGL(k_sumsq_partial, dim3(B.tiles), dim3(THREADS), 0, st, NB);
-    hipLaunchKernelGGL(k_sumsq_final, dim3(1), dim3(THREADS), 0, st, B.partials, B.tiles, clip_norm, B.red);
-    SG_LAUNCH_CHECK("sumsq");
-    return 0;
-}
 
 // ---- Grokfast ------------------------------------------------------------------
 struct GfRec {
@@ -299,11 +150,6 @@ __global__ __launch_bounds__(THREADS) void k_restore(Batch<RestoreRec> B) {
         sg::store_elem(R.sharp, R.dtype, i, sg_abs(sgv - ng));
         sg::store_elem(R.param, R.dtype, i, sg::load_elem(R.backup, R.dtype, i));
     }
-}
-
-int check_dtype(int i, int dtype) {
-    if (dtype != SG_F32 && dtype != SG_F16 && dtype != SG_BF16) return sg::fail("tensor %d: bad dtype %d", i, dtype);
-    return 0;
 }
 
 }  // namespace

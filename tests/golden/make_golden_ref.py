@@ -1,5 +1,6 @@
 """Writes tests/golden/ref_*.npz: inputs and outputs of the reference's own CPU
-code for the Grokfast, SuperGrok v1.5 and Muon steps.
+code for the Grokfast, SuperGrok v1.5, Muon, SuperGrok v1.1, GrokAdamW,
+NeuralGrok, Prodigy, Lion and LookSAM steps.
 
 The outputs come from oracle/_ref/ref_ops*.so, which oracle/Makefile.ref
 compiles from the reference's csrc/ops.cpp (CPU-only, where it lies under
@@ -113,10 +114,141 @@ def muon():
     np.savez_compressed(os.path.join(HERE, "ref_muon.npz"), **out)
 
 
+def family():
+    """The remaining fused steps (csrc/ops.cpp:209-656): SuperGrok v1.1, GrokAdamW, NeuralGrok, Prodigy, Lion, LookSAM."""
+    out = {}
+    sizes = [50, 257, 1, 1000]
+    P = len(sizes)
+
+    def put(tag, t, name, tensors):
+        for i, x in enumerate(tensors):
+            out[f"{tag}_{name}_{t}_{i}"] = x.detach().float().numpy().copy()
+
+    # GrokAdamW: step 1 trips the global-norm clip
+    gen = torch.Generator().manual_seed(21)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    eas, easqs, emas = ([torch.zeros(n) for n in sizes] for _ in range(3))
+    cfg = dict(alpha=0.98, lamb=5.0, beta1=0.9, beta2=0.98, lr=1e-3, wd=1.0, eps=1e-8, clip=1.0)
+    out.update({f"gaw_{k}": v for k, v in cfg.items()})
+    put("gaw", "in", "p", params)
+    for t in range(3):
+        grads = [rnd(gen, n, std=0.3 if t == 1 else 1e-3) for n in sizes]
+        put("gaw", t, "g_in", grads)
+        ref_ops.grokadamw_fused_step(params, grads, eas, easqs, emas, [t + 1] * P, cfg["alpha"], cfg["lamb"], cfg["beta1"],
+                                     cfg["beta2"], cfg["lr"], cfg["wd"], cfg["eps"], cfg["clip"])
+        for name, ts in (("g_out", grads), ("p", params), ("ea", eas), ("easq", easqs), ("ema", emas)):
+            put("gaw", t, name, ts)
+
+    # NeuralGrok
+    gen = torch.Generator().manual_seed(22)
+    H = 8
+    W1, b1, W2, b2 = rnd(gen, H, 1, std=0.5), rnd(gen, H, std=0.1), rnd(gen, 1, H, std=0.5), rnd(gen, 1, std=0.1)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    eas, easqs = ([torch.zeros(n) for n in sizes] for _ in range(2))
+    cfg = dict(alpha_amp=10.0, beta_amp=4.0, beta1=0.9, beta2=0.98, lr=1e-3, wd=1.0, eps=1e-8, clip=1.0)
+    out.update({f"ng_{k}": v for k, v in cfg.items()})
+    out.update(ng_W1=W1.numpy(), ng_b1=b1.numpy(), ng_W2=W2.numpy(), ng_b2=b2.numpy(), ng_H=H)
+    put("ng", "in", "p", params)
+    for t in range(3):
+        grads = [rnd(gen, n, std=0.3 if t == 1 else 1e-3) for n in sizes]
+        put("ng", t, "g_in", grads)
+        ref_ops.neuralgrok_fused_step(params, grads, eas, easqs, [t + 1] * P, W1, b1, W2, b2, cfg["alpha_amp"], cfg["beta_amp"], H,
+                                      cfg["beta1"], cfg["beta2"], cfg["lr"], cfg["wd"], cfg["eps"], cfg["clip"])
+        for name, ts in (("g_out", grads), ("p", params), ("ea", eas), ("easq", easqs)):
+            put("ng", t, name, ts)
+
+    # Prodigy: d_lr is returned and fed back
+    gen = torch.Generator().manual_seed(23)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    inits = [p.clone() for p in params]
+    eas, easqs, ss = ([torch.zeros(n) for n in sizes] for _ in range(3))
+    cfg = dict(beta1=0.9, beta2=0.999, lr=1e-3, wd=0.0, eps=1e-8, d_lr0=1e-6)
+    out.update({f"pr_{k}": v for k, v in cfg.items()})
+    put("pr", "in", "p", params)
+    d_lr = cfg["d_lr0"]
+    for t in range(4):
+        grads = [rnd(gen, n, std=1e-2) for n in sizes]
+        put("pr", t, "g_in", grads)
+        d_lr = ref_ops.prodigy_fused_step(params, grads, eas, easqs, ss, inits, [t + 1] * P, d_lr, cfg["beta1"], cfg["beta2"],
+                                          cfg["lr"], cfg["wd"], cfg["eps"])
+        out[f"pr_d_lr_{t}"] = d_lr
+        for name, ts in (("p", params), ("ea", eas), ("easq", easqs), ("s", ss)):
+            put("pr", t, name, ts)
+
+    # Lion (an exactly-zero gradient and momentum exercises sign(0) = 0)
+    gen = torch.Generator().manual_seed(24)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    eas = [torch.zeros(n) for n in sizes]
+    cfg = dict(lr=1e-4, beta1=0.9, beta2=0.99, wd=3.0)
+    out.update({f"li_{k}": v for k, v in cfg.items()})
+    put("li", "in", "p", params)
+    for t in range(3):
+        grads = [rnd(gen, n, std=1e-3) for n in sizes]
+        if t == 0:
+            grads[1][:7] = 0.0
+        put("li", t, "g_in", grads)
+        ref_ops.lion_fused_step(params, grads, eas, cfg["lr"], cfg["beta1"], cfg["beta2"], cfg["wd"])
+        for name, ts in (("p", params), ("ea", eas)):
+            put("li", t, name, ts)
+
+    # SuperGrok v1.1 (steps travel by value through the binding, exactly as for v1.5)
+    gen = torch.Generator().manual_seed(25)
+    H = 8
+    W1, b1, W2, b2 = rnd(gen, H, 2, std=0.5), rnd(gen, H, std=0.1), rnd(gen, 1, H, std=0.5), rnd(gen, 1, std=0.1)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    eas, easqs, mus = ([torch.zeros(n) for n in sizes] for _ in range(3))
+    alphas = [0.98] * P
+    beta1s = [0.9 * 0.9 ** i for i in range(P)]
+    cfg = dict(rescale=0.1, beta2=0.999, lr=1e-3, wd=1.0, eps=1e-8, lamb=5.0, ramp=0.5, temp=5.0, clip=1.0)
+    out.update({f"s11_{k}": v for k, v in cfg.items()})
+    out.update(s11_W1=W1.numpy(), s11_b1=b1.numpy(), s11_W2=W2.numpy(), s11_b2=b2.numpy(), s11_H=H,
+               s11_alphas=np.array(alphas), s11_beta1s=np.array(beta1s))
+    put("s11", "in", "p", params)
+    for t in range(3):
+        grads = [rnd(gen, n, std=0.3 if t == 1 else 1e-3) for n in sizes]
+        sharps = [rnd(gen, n, std=1e-3).abs() for n in sizes]
+        put("s11", t, "g_in", grads)
+        put("s11", t, "sharp", sharps)
+        steps = [t] * P
+        ref_ops.supergrok11_fused_step(params, grads, eas, easqs, mus, sharps, steps, alphas, beta1s, W1, b1, W2, b2, cfg["rescale"], H,
+                                       cfg["beta2"], cfg["lr"], cfg["wd"], cfg["eps"], cfg["lamb"], cfg["ramp"], cfg["temp"],
+                                       cfg["clip"])
+        for name, ts in (("g_out", grads), ("p", params), ("ea", eas), ("easq", easqs), ("mu", mus)):
+            put("s11", t, name, ts)
+
+    # LookSAM helpers
+    gen = torch.Generator().manual_seed(26)
+    params = [rnd(gen, n, std=0.02) for n in sizes]
+    grads = [rnd(gen, n, std=1e-3) for n in sizes]
+    put("ls", "in", "p", params)
+    put("ls", "in", "g", grads)
+    out["ls_rho"] = 0.05
+    backups = ref_ops.looksam_perturb_all(params, grads, 0.05)
+    put("ls", "pert", "p", params)
+    put("ls", "pert", "backup", backups)
+    ref_ops.looksam_restore_all(params, backups)
+    put("ls", "rest", "p", params)
+    sam_grads = [rnd(gen, n, std=1e-3) for n in sizes]
+    sam_grads[2] = grads[2].clone()          # zero difference: that direction is left as it was
+    v_dirs = [torch.full((n,), 0.25) for n in sizes]
+    put("ls", "dir", "sam_g", sam_grads)
+    put("ls", "dir", "v_in", v_dirs)
+    ref_ops.looksam_compute_directions(v_dirs, sam_grads, grads)
+    put("ls", "dir", "v_out", v_dirs)        # unchanged: the CPU branch rebinds its by-value copy of the list
+    vd = [rnd(gen, n) for n in sizes]
+    vd = [v / v.norm() for v in vd]
+    put("ls", "adj", "v", vd)
+    out["ls_la"] = 0.7
+    ref_ops.looksam_adjust_grads(grads, vd, 0.7)
+    put("ls", "adj", "g_out", grads)
+    np.savez_compressed(os.path.join(HERE, "ref_family.npz"), **out)
+
+
 if __name__ == "__main__":
     grokfast()
     sg15()
     muon()
+    family()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
