@@ -256,7 +256,9 @@ size_t sg_family_workspace_bytes(int num_tensors, const int64_t* numels);
 
 /* GrokAdamW: global-norm clip, ema = alpha*ema + (1-alpha)*g, g' = g + lamb*ema,
  * AdamW on g'.  Replaces grokadamw_fused_step (csrc/ops.cpp:311-353;
- * launch_fused_grokadamw_step, csrc/grokadamw_kernels.cu). */
+ * launch_fused_grokadamw_step, csrc/grokadamw_kernels.cu).  With lamb == 0 the
+ * aux (ema) pointers may be NULL and the step is plain AdamW: the update of
+ * grokking_optimizers/_adamw_helper.py:12-22 as one launch. */
 int sg_grokadamw_step(int num_tensors, const SgFamilyTensor* tensors, float alpha, float lamb, float beta1, float beta2,
                       float lr, float wd, float eps, float grad_clip_norm, void* workspace, size_t workspace_bytes,
                       void* stream);

@@ -445,6 +445,25 @@ void grokadamw_fused_step(std::vector<torch::Tensor>& params, std::vector<torch:
                                    (size_t)A.ws.numel(), current_stream(*A.first)), fn);
 }
 
+// AdamW over a list of tensors as one launch: what adamw_step of the reference's
+// grokking_optimizers/_adamw_helper.py:12-22 does with six ATen calls per tensor (bias corrections in double).
+void adamw_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
+                      std::vector<torch::Tensor>& exp_avg_sqs, std::vector<int64_t>& steps, double lr, double beta1, double beta2,
+                      double eps, double wd) {
+    const char* fn = "adamw_fused_step";
+    std::vector<float> bc1, bc2;
+    for (int64_t st : steps) {
+        bc1.push_back((float)(1.0 - std::pow(beta1, (double)st)));
+        bc2.push_back((float)(1.0 - std::pow(beta2, (double)st)));
+    }
+    FamilyArgs A;
+    gather_family(fn, &A, params, grads, &exp_avgs, &exp_avg_sqs, nullptr, nullptr, false, &bc1, &bc2, nullptr, nullptr);
+    if (A.ts.empty()) return;
+    A.make_ws();
+    check_status(sg_grokadamw_step((int)A.ts.size(), A.ts.data(), 0.0f, 0.0f, (float)beta1, (float)beta2, (float)lr, (float)wd, (float)eps,
+                                   0.0f, A.ws.data_ptr(), (size_t)A.ws.numel(), current_stream(*A.first)), fn);
+}
+
 void neuralgrok_fused_step(std::vector<torch::Tensor>& params, std::vector<torch::Tensor>& grads, std::vector<torch::Tensor>& exp_avgs,
                            std::vector<torch::Tensor>& exp_avg_sqs, std::vector<int64_t>& steps, torch::Tensor W1, torch::Tensor b1,
                            torch::Tensor W2, torch::Tensor b2, float alpha_amp, float beta_amp, int hidden_dim, float beta1, float beta2,
@@ -610,6 +629,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("prodigy_fused_step", &prodigy_fused_step, "Prodigy: distance-aware self-tuning Adam; returns the new d_lr", py::arg("params"),
           py::arg("grads"), py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("s_bufs"), py::arg("param_inits"), py::arg("steps"),
           py::arg("d_lr"), py::arg("beta1"), py::arg("beta2"), py::arg("lr"), py::arg("wd"), py::arg("eps"));
+    m.def("adamw_fused_step", &adamw_fused_step, "AdamW over a tensor list in one launch", py::arg("params"), py::arg("grads"),
+          py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("steps"), py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("eps"),
+          py::arg("wd"));
     m.def("lion_fused_step", &lion_fused_step, "Lion: fused sign-momentum step", py::arg("params"), py::arg("grads"), py::arg("exp_avgs"),
           py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("wd"));
     m.def("looksam_perturb_all", &looksam_perturb_all, py::arg("params"), py::arg("grads"), py::arg("rho"));

@@ -61,9 +61,13 @@ __global__ __launch_bounds__(THREADS) void k_grokadamw(Batch<FamRec> B, float al
     for (int k = threadIdx.x; k < cnt; k += THREADS) {
         const int i = start + k;
         const float g = clipped_grad(R, i, clip_on, coef);
-        const float e = sg_fma(alpha, R.aux[i], (1.0f - alpha) * g);
-        R.aux[i] = e;
-        adam_update(R, i, sg_fma(lamb, e, g), beta1, beta2, eps, decay, step_size);
+        float fg = g;
+        if (R.aux) {        // no EMA buffer: plain AdamW
+            const float e = sg_fma(alpha, R.aux[i], (1.0f - alpha) * g);
+            R.aux[i] = e;
+            fg = sg_fma(lamb, e, g);
+        }
+        adam_update(R, i, fg, beta1, beta2, eps, decay, step_size);
     }
 }
 
@@ -345,7 +349,8 @@ int sg_grokadamw_step(int num_tensors, const SgFamilyTensor* tensors, float alph
     using namespace sgew;
     if (num_tensors <= 0) return 0;
     std::vector<FamRec> recs;
-    if (collect(num_tensors, tensors, N_PARAM | N_GRAD | N_EA | N_EASQ | N_AUX, &recs) || check_bc(recs)) return 1;
+    // the EMA buffer may be NULL for every tensor when lamb == 0: the step is then plain AdamW
+    if (collect(num_tensors, tensors, N_PARAM | N_GRAD | N_EA | N_EASQ | (lamb != 0.0f ? N_AUX : 0), &recs) || check_bc(recs)) return 1;
     if (recs.empty()) return 0;
     hipStream_t st = (hipStream_t)stream;
     Batch<FamRec> B;

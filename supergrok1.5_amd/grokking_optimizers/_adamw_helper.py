@@ -1,15 +1,15 @@
-"""AdamW over a list of tensors with ATen ops: the update Muon applies to its
-non-2D parameter group (reference: grokking_optimizers/_adamw_helper.py:12-22;
-decay first, bias corrections in Python double, denom = sqrt(v/bc2) + eps)."""
+"""AdamW over a list of tensors: the update Muon applies to its non-2D parameter
+group and LookSAM applies in `step()` (reference:
+grokking_optimizers/_adamw_helper.py:12-22; decay first, bias corrections in
+Python double, denom = sqrt(v/bc2) + eps).  One fused launch over all tensors
+(`_ops.adamw_fused_step`) instead of six ATen calls per tensor."""
 import torch
+
+from grokking_optimizers import _ops
 
 
 @torch.no_grad()
 def adamw_step(params, grads, exp_avgs, exp_avg_sqs, steps, lr, beta1, beta2, eps, wd):
-    for p, g, m, v, t in zip(params, grads, exp_avgs, exp_avg_sqs, steps):
-        bc1, bc2 = 1.0 - beta1 ** t, 1.0 - beta2 ** t
-        m.mul_(beta1).add_(g, alpha=1 - beta1)
-        v.mul_(beta2).addcmul_(g, g, value=1 - beta2)
-        denom = (v / bc2).sqrt().add_(eps)
-        p.mul_(1 - lr * wd)
-        p.addcdiv_(m, denom, value=-(lr / bc1))
+    if params:
+        _ops.adamw_fused_step(list(params), list(grads), list(exp_avgs), list(exp_avg_sqs), [int(t) for t in steps],
+                              float(lr), float(beta1), float(beta2), float(eps), float(wd))
