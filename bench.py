@@ -82,7 +82,7 @@ def cpu_baseline(sample_elems_target=4_000_000):
 
 
 def bench_other(args, dev):
-    """Secondary measurements: the Grokfast, SuperGrok v1.5 and Muon fused steps through `_ops`."""
+    """Secondary measurements: the other fused steps through `_ops`."""
     import torch
     import workloads as wl
     from grokking_optimizers import _ops
@@ -111,7 +111,7 @@ def bench_other(args, dev):
                 t[0] += 1
                 _ops.grokfast_adamw_fused_step(params, grads, emas, ms, vs, [t[0]] * len(params), 0.98, 2.0, 1e-3, 0.9, 0.98, 1e-8, 1.0)
             name = "Grokfast fused step (EMA + amplify + AdamW), 14 tensors, %d elements" % n
-        else:
+        elif args.workload == "sg15":
             eas, easqs, mus, sharps = z(), z(), z(), z()
             gen = torch.Generator().manual_seed(3)
             H = 32
@@ -125,6 +125,53 @@ def bench_other(args, dev):
                                             [0.9 * 0.9 ** i for i in range(P)], W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8,
                                             2.0, 1.0, 0.5, 1.0)
             name = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip), 14 tensors, %d elements" % n
+        else:
+            # the other fused steps, on the 50-tensor / 25 M-element set so that HBM traffic, not launch latency, is measured
+            shapes = wl.scale50_shapes()
+            params = [p.reshape(-1).to(dev) for p in wl.make_params(shapes, seed=0)]
+            grads = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.005, tail="student3")]
+            n = sum(p.numel() for p in params)
+            P = len(params)
+            a, b, c, d = z(), z(), z(), z()
+            gen = torch.Generator().manual_seed(3)
+            t = [0]
+            if args.workload == "grokadamw":
+                def step():
+                    t[0] += 1
+                    _ops.grokadamw_fused_step(params, grads, a, b, c, [t[0]] * P, 0.98, 5.0, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
+                bytes_per_elem, what = 36, "GrokAdamW fused step (clip + EMA + amplify + AdamW)"
+            elif args.workload == "neuralgrok":
+                H = 128
+                W = [(torch.randn(H, 1, generator=gen) * 0.5).to(dev), torch.zeros(H, device=dev),
+                     (torch.randn(1, H, generator=gen) * 0.1).to(dev), torch.zeros(1, device=dev)]
+
+                def step():
+                    t[0] += 1
+                    _ops.neuralgrok_fused_step(params, grads, a, b, [t[0]] * P, *W, 10.0, 4.0, H, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
+                bytes_per_elem, what = 28, "NeuralGrok fused step (clip + 1->128->1 amplifier + AdamW)"
+            elif args.workload == "prodigy":
+                inits = [p.clone() for p in params]
+                dl = [1e-6]
+
+                def step():
+                    t[0] += 1
+                    dl[0] = _ops.prodigy_fused_step(params, grads, a, b, c, inits, [t[0]] * P, dl[0], 0.9, 0.999, 1e-3, 0.0, 1e-8)
+                bytes_per_elem, what = 52, "Prodigy fused step (d_lr reduction pass + Adam pass, one host read of d_lr)"
+            elif args.workload == "lion":
+                def step():
+                    _ops.lion_fused_step(params, grads, a, 1e-4, 0.9, 0.99, 3.0)
+                bytes_per_elem, what = 20, "Lion fused step"
+            else:
+                H = 32
+                W = [(torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev),
+                     (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)]
+                beta1s = [0.9 * 0.9 ** i for i in range(P)]
+
+                def step():
+                    _ops.supergrok11_fused_step(params, grads, a, b, c, d, [0] * P, [0.98] * P, beta1s, *W, 0.1, H, 0.999, 1e-3, 1.0,
+                                                1e-8, 5.0, 1.0, 5.0, 1.0)
+                bytes_per_elem, what = 52, "SuperGrok v1.1 full step (H=32, exact GELU, device-side clip and cosine gates)"
+            name = "%s, 50 tensors, %d elements" % (what, n)
         units, unit, dtype, bound, peak = n, "elements/s", "f32", "hbm", HBM_PEAK_GBS
     for _ in range(Wm):
         step()
@@ -141,8 +188,9 @@ def bench_other(args, dev):
         out["roofline"] = {"bound": "mfma", "achieved": units / el / 1e12, "peak": peak, "unit": "TFLOP/s",
                            "frac": units / el / 1e12 / peak, "traffic": None}
     else:
-        out["roofline"] = {"bound": "hbm", "achieved": 40 * units / el / 1e9, "peak": peak, "unit": "GB/s",
-                           "frac": 40 * units / el / 1e9 / peak, "traffic": None}
+        bpe = locals().get("bytes_per_elem", 40)       # algorithmic bytes per element of the step
+        out["roofline"] = {"bound": "hbm", "achieved": bpe * units / el / 1e9, "peak": peak, "unit": "GB/s",
+                           "frac": bpe * units / el / 1e9 / peak, "traffic": None, "bytes_per_element": bpe}
     return out
 
 
@@ -151,7 +199,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon"],
+    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
@@ -171,7 +219,7 @@ def main():
     from sg2_harness import per_tensor_scalars, shared_scalars
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
-    if args.workload in ("grokfast", "sg15", "muon"):
+    if args.workload not in ("scale50", "shared14"):
         print(json.dumps(bench_other(args, dev)))
         return
     if _cabi.lib().sg2_set_chunk_len(args.chunk_len) or _cabi.lib().sg2_set_scan_window(args.window):

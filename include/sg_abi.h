@@ -316,6 +316,21 @@ int sg_looksam_directions(int num_tensors, const SgLookSamTensor* tensors, void*
 int sg_looksam_adjust(int num_tensors, const SgLookSamTensor* tensors, float la, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* Pre-pass of the SuperGrok v2 step, per tensor: out = g * c/(|g|+1e-12) when
+ * |g| > c, else g; non-finite entries of the result become 0.  Norms are
+ * reduced on the device.  Replaces the two host syncs per tensor of
+ * grokking_optimizers/supergrok2.py:316-321 (grad.norm() > clip, then
+ * isfinite(grad).all()).  out is a separate tensor, as the reference makes one;
+ * workspace: sg_family_workspace_bytes. */
+typedef struct Sg2ClipTensor {
+    const void* grad;   /* [numel] dtype */
+    void* out;          /* [numel] dtype */
+    int64_t numel;
+    int32_t dtype;
+} Sg2ClipTensor;
+int sg2_clip_grads(int num_tensors, const Sg2ClipTensor* tensors, float max_norm, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
 /* ================================ Muon ==================================== */
 
 /* One 2-D parameter of the Muon step: the i-th entries of the vectors of

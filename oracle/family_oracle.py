@@ -11,12 +11,15 @@ what the corresponding host function of the reference's csrc/ops.cpp computes:
   prodigy_step           prodigy_fused_step                   ops.cpp:424-506
   lion_step              lion_fused_step                      ops.cpp:536-560
   sg11_step              supergrok11_fused_step               ops.cpp:209-288
+  sg2_clip               SuperGrok2.step pre-pass             grokking_optimizers/supergrok2.py:316-321
   looksam_perturb        looksam_perturb_all                  ops.cpp:566-590
   looksam_directions     looksam_compute_directions           ops.cpp:607-630
   looksam_adjust         looksam_adjust_grads                 ops.cpp:632-652
 
 Pinned by tests/golden/ref_family.npz, which holds inputs and outputs of the
-reference's own CPU code for every function above (tests/test_oracle_family.py).
+reference's own CPU code for every ops.cpp function above
+(tests/test_oracle_family.py); sg2_clip, which restates Python, is pinned there
+against the same three torch expressions evaluated by torch on the CPU.
 Tensors are lists of 1-D float32 arrays and are updated in place, like the
 reference updates its tensor lists.
 """
@@ -150,6 +153,16 @@ def sg11_step(params, grads, eas, easqs, mus, sharps, steps, alphas, beta1s, W1,
         lamb_eff = F(ramp) * gate * F(lamb) if ramp > 0 else F(0)
         fg = smart + lamb_eff * mu
         _adam(p, ea, easq, fg, beta1s[i], beta2, lr, wd, eps, _bc(beta1s[i], st), _bc(beta2, st))
+
+
+def sg2_clip(grads, max_norm):
+    """Per-tensor pre-pass of the v2 step (grokking_optimizers/supergrok2.py:316-321): returns new arrays."""
+    out = []
+    for g in grads:
+        n = _norm([g])
+        h = g * (F(max_norm) / (n + F(1e-12))) if n > F(max_norm) else g.copy()
+        out.append(np.where(np.isfinite(h), h, F(0)).astype(F))
+    return out
 
 
 def looksam_perturb(params, grads, rho):

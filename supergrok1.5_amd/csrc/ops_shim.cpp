@@ -601,6 +601,29 @@ void looksam_adjust_grads(std::vector<torch::Tensor>& grads, std::vector<torch::
     looksam_call("looksam_adjust_grads", 2, grads, v_dirs, nullptr, la);
 }
 
+// Per-tensor clip + non-finite guard of the v2 pre-pass (grokking_optimizers/supergrok2.py:316-321 of the
+// reference), for all tensors in three launches and without host syncs.  Returns new tensors.
+std::vector<torch::Tensor> supergrok2_clip_grads(std::vector<torch::Tensor>& grads, float max_norm) {
+    const char* fn = "supergrok2_clip_grads";
+    std::vector<torch::Tensor> out;
+    std::vector<Sg2ClipTensor> ts;
+    std::vector<int64_t> numels;
+    const torch::Tensor* first = nullptr;
+    for (size_t i = 0; i < grads.size(); i++) {
+        if (!grads[i].defined()) { out.push_back(grads[i]); continue; }
+        check_gpu(grads[i], fn, "grad");
+        out.push_back(torch::empty_like(grads[i]));
+        if (grads[i].numel() == 0) continue;
+        ts.push_back({grads[i].data_ptr(), out.back().data_ptr(), grads[i].numel(), dtype_code(grads[i], "grad")});
+        numels.push_back(grads[i].numel());
+        if (!first) first = &grads[i];
+    }
+    if (ts.empty()) return out;
+    auto ws = make_workspace(sg_family_workspace_bytes((int)ts.size(), numels.data()), *first);
+    check_status(sg2_clip_grads((int)ts.size(), ts.data(), max_norm, ws.data_ptr(), (size_t)ws.numel(), current_stream(*first)), fn);
+    return out;
+}
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "Grokking optimizers: fused steps on MI355X (hand-written HIP behind the reference's _ops surface)";
     m.def("supergrok15_fused_step", &supergrok15_fused_step, "SuperGrok1.5: fused clip + mu + meta-net + gating + adam + progressive wd",
@@ -632,6 +655,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("adamw_fused_step", &adamw_fused_step, "AdamW over a tensor list in one launch", py::arg("params"), py::arg("grads"),
           py::arg("exp_avgs"), py::arg("exp_avg_sqs"), py::arg("steps"), py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("eps"),
           py::arg("wd"));
+    m.def("supergrok2_clip_grads", &supergrok2_clip_grads, "SuperGrok2 pre-pass: per-tensor norm clip + non-finite guard, device-side",
+          py::arg("grads"), py::arg("max_norm"));
     m.def("lion_fused_step", &lion_fused_step, "Lion: fused sign-momentum step", py::arg("params"), py::arg("grads"), py::arg("exp_avgs"),
           py::arg("lr"), py::arg("beta1"), py::arg("beta2"), py::arg("wd"));
     m.def("looksam_perturb_all", &looksam_perturb_all, py::arg("params"), py::arg("grads"), py::arg("rho"));

@@ -291,6 +291,27 @@ __global__ __launch_bounds__(THREADS) void k_ls_adjust(Batch<FamRec> B, float la
     }
 }
 
+// ---- SuperGrok v2 pre-pass: per-tensor norm clip + non-finite guard ------------------------------------------
+// FamRec roles: grad = input gradient, param = output (a new tensor, as the reference makes one)
+__global__ __launch_bounds__(THREADS) void k_sg2_clip(Batch<FamRec> B, float max_norm) {
+    int start, cnt;
+    const int ti = sg::upper_seg(B.prefix, B.n, (int)blockIdx.x);
+    const FamRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
+    // a NaN norm compares false (no clip); an infinite one gives scale 0 and the guard below zeroes what 0*inf leaves
+    const float norm = (float)sqrt(B.tred[ti].s[0]);
+    const float scale = (norm > max_norm) ? max_norm / (norm + 1e-12f) : 1.0f;
+    for (int k = threadIdx.x; k < cnt; k += THREADS) {
+        const int i = start + k;
+        float g = sg::load_elem(R.grad, R.dtype, i);
+        if (scale != 1.0f) {
+            g = g * scale;
+            if (R.dtype == SG_F16) g = __half2float(__float2half_rn(g));        // the product is a tensor of the gradient's type
+            if (R.dtype == SG_BF16) g = sg::bf16_bits_to_f(sg::f_to_bf16_bits(g));
+        }
+        sg::store_elem(R.param, R.dtype, i, sg::finite_or_zero(g));
+    }
+}
+
 // ---- host side ---------------------------------------------------------------------------------------------
 enum Need { N_PARAM = 1, N_GRAD = 2, N_EA = 4, N_EASQ = 8, N_AUX = 16, N_AUX2 = 32 };
 
@@ -450,6 +471,34 @@ int sg11_fused_step(int num_tensors, const SgFamilyTensor* tensors, const Sg15Ne
     hipLaunchKernelGGL(k_sum_tiles, dim3(B.n), dim3(THREADS), 0, st, B, 1);
     hipLaunchKernelGGL(k_sg11_adam, dim3(B.tiles), dim3(THREADS), 0, st, B, beta2, lr, eps, 1.0f - lr * wd, lamb, ramp, gate_temperature);
     SG_LAUNCH_CHECK("k_sg11");
+    return 0;
+}
+
+int sg2_clip_grads(int num_tensors, const Sg2ClipTensor* tensors, float max_norm, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace sgew;
+    if (num_tensors <= 0) return 0;
+    if (!tensors) return sg::fail("NULL argument");
+    std::vector<FamRec> recs;
+    for (int i = 0; i < num_tensors; i++) {
+        const Sg2ClipTensor& t = tensors[i];
+        if (t.numel == 0) continue;
+        if (!t.grad || !t.out) return sg::fail("tensor %d: NULL pointer", i);
+        if (check_dtype(i, t.dtype)) return 1;
+        FamRec r = {};
+        r.grad = const_cast<void*>(t.grad);
+        r.param = t.out;
+        r.numel = t.numel;
+        r.dtype = t.dtype;
+        recs.push_back(r);
+    }
+    if (recs.empty()) return 0;
+    hipStream_t st = (hipStream_t)stream;
+    Batch<FamRec> B;
+    if (upload(recs, workspace, workspace_bytes, st, &B)) return 1;
+    hipLaunchKernelGGL(k_ls_grad_sumsq, dim3(B.tiles), dim3(THREADS), 0, st, B);
+    hipLaunchKernelGGL(k_sum_tiles, dim3(B.n), dim3(THREADS), 0, st, B, 1);
+    hipLaunchKernelGGL(k_sg2_clip, dim3(B.tiles), dim3(THREADS), 0, st, B, max_norm);
+    SG_LAUNCH_CHECK("k_sg2_clip");
     return 0;
 }
 

@@ -125,3 +125,19 @@ def test_class_clip_matches_formula():
     out = opt._clip([g_big, g_small])
     want = g_big * (0.5 / (g_big.norm() + 1e-12))
     assert torch.allclose(out[0], want, rtol=1e-6, atol=0) and torch.equal(out[1], g_small)
+    # against the CPU checker, with non-finite entries, several tiles and 16-bit gradients
+    import numpy as np
+    from oracle import family_oracle as fo
+    r = np.random.RandomState(4)
+    cases = [r.randn(9000).astype(np.float32), (r.randn(5000) * 1e-4).astype(np.float32), r.randn(4096).astype(np.float32),
+             r.randn(70).astype(np.float32), r.randn(1).astype(np.float32) * 3]
+    cases[2][100] = np.nan
+    cases[3][7] = -np.inf
+    got = opt._clip([torch.from_numpy(c).cuda() for c in cases])
+    for a, b in zip(got, fo.sg2_clip(cases, 0.5)):
+        assert np.allclose(a.cpu().numpy(), b, rtol=1e-6, atol=0)
+    h = [torch.from_numpy(c).cuda().to(torch.bfloat16) for c in cases[:2]]
+    got = opt._clip(h)
+    want = fo.sg2_clip([x.float().cpu().numpy() for x in h], 0.5)
+    for a, b in zip(got, want):
+        assert a.dtype == torch.bfloat16 and np.allclose(a.float().cpu().numpy(), b, rtol=2 ** -7, atol=0)
