@@ -1,0 +1,65 @@
+/* Composed per-timestep projections of one SuperGrok v2 scan direction.
+ *
+ * Every linear quantity of a timestep is an affine function of the element's
+ * (gradient, sharpness) pair, because the 8-vector fed to the scan is itself
+ * x = W_in [g, s]^T + b_in (input_proj_sort_kernel,
+ * csrc/supergrok2_mamba_peer_kernels.cu:92-117 of the reference) and in_proj,
+ * dt_proj, B_proj and C_proj (:138-200 there) are applied to it without a
+ * nonlinearity in between:
+ *     xb_j = in_proj[j,:] x            z_j = in_proj[d_inner+j,:] x
+ *     dt_raw_j = dt_W[j,:] xb + dt_b   B_s = B_proj[s,:] xb     C_s = C_proj[s,:] xb
+ * This header composes those maps once per call into coefficient triples
+ * (c_g, c_s, c_0) - accumulated in double, in a fixed order, rounded to float -
+ * so that a timestep costs two fmas per output, v = fma(c_g, g, fma(c_s, s, c_0)),
+ * instead of a chain of small matrix products.  The device kernel and the CPU
+ * checker both include this file (double +,* only, no contraction), so their
+ * coefficients are bit-identical.
+ */
+#ifndef SG2_COMPOSE_H_
+#define SG2_COMPOSE_H_
+#include "sg_math.h"
+
+enum { SG2_COMP_XB = 0, SG2_COMP_Z = 1, SG2_COMP_DT = 2, SG2_COMP_B = 3, SG2_COMP_C = 4, SG2_COMP_GROUPS = 5 };
+#define SG2_COMP_MAX_INNER 32
+#define SG2_COMP_MAX_MODEL 16
+
+/* Coefficient triple of output `row` of `group`.  Win [d_model,2], bin [d_model],
+ * in_proj [2*d_inner, d_model], dt_W [d_inner,d_inner], dt_b [d_inner],
+ * Bp / Cp [d_state, d_inner]. */
+SG_HD void sg2_compose_one(int group, int row, int d_model, int d_inner, const float* Win, const float* bin,
+                           const float* in_proj, const float* dt_W, const float* dt_b, const float* Bp, const float* Cp,
+                           float out[3]) {
+    double src[SG2_COMP_MAX_MODEL][3];
+    for (int k = 0; k < d_model; k++) {
+        src[k][0] = (double)Win[2 * k];
+        src[k][1] = (double)Win[2 * k + 1];
+        src[k][2] = (double)bin[k];
+    }
+    if (group == SG2_COMP_XB || group == SG2_COMP_Z) {
+        const float* w = in_proj + (size_t)(group == SG2_COMP_Z ? d_inner + row : row) * d_model;
+        for (int c = 0; c < 3; c++) {
+            double acc = 0.0;
+            for (int k = 0; k < d_model; k++) acc = acc + (double)w[k] * src[k][c];
+            out[c] = (float)acc;
+        }
+        return;
+    }
+    double xb[SG2_COMP_MAX_INNER][3];
+    for (int j = 0; j < d_inner; j++)
+        for (int c = 0; c < 3; c++) {
+            double acc = 0.0;
+            for (int k = 0; k < d_model; k++) acc = acc + (double)in_proj[(size_t)j * d_model + k] * src[k][c];
+            xb[j][c] = acc;
+        }
+    const float* w = (group == SG2_COMP_DT ? dt_W : (group == SG2_COMP_B ? Bp : Cp)) + (size_t)row * d_inner;
+    for (int c = 0; c < 3; c++) {
+        double acc = (group == SG2_COMP_DT && c == 2) ? (double)dt_b[row] : 0.0;
+        for (int j = 0; j < d_inner; j++) acc = acc + (double)w[j] * xb[j][c];
+        out[c] = (float)acc;
+    }
+}
+
+/* value of a composed output for one element */
+SG_HD float sg2_comp_eval(const float* c, float g, float s) { return sg_fma(c[0], g, sg_fma(c[1], s, c[2])); }
+
+#endif /* SG2_COMPOSE_H_ */

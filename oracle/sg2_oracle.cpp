@@ -70,6 +70,7 @@
 #include <vector>
 
 #include "../include/sg_math.h"
+#include "../include/sg2_compose.h"
 
 namespace {
 
@@ -196,6 +197,9 @@ void sort_perm(const float* g, int64_t N, int32_t* perm) {
 template <class O>
 struct DirW {
     const float *in_proj, *dt_W, *dt_b, *Bp, *Cp, *A_log, *D, *rope, *out_proj;
+    /* fp32 policy: composed coefficient triples [group][row][3] (include/sg2_compose.h), as the device uses them */
+    std::vector<float> comp;
+    int comp_rows;
 };
 
 template <class O>
@@ -203,10 +207,27 @@ struct StepProj {           /* per-timestep projections */
     typename O::R xb[32], z[32], dt[32], B[32], C[32];
 };
 
+/* gs: the element's (gradient, sharpness); x: its input projection.  The fp32 policy evaluates the composed
+ * affine maps from (g, s); the fp64 policy evaluates the reference's chain of projections from x literally. */
 template <class O>
-void project(const Dims& d, const DirW<O>& w, const typename O::R* x, bool need_zc, StepProj<O>& o) {
+void project(const Dims& d, const DirW<O>& w, const typename O::R* x, const float* gs, bool need_zc, StepProj<O>& o) {
     typedef typename O::R R;
     const int dm = d.d_model, di = d.d_inner, ds = d.d_state;
+    if (sizeof(R) == 4) {
+        const float* c = w.comp.data();
+        const int rows = w.comp_rows;
+        auto eval = [&](int group, int row) { return (R)sg2_comp_eval(c + ((size_t)group * rows + row) * 3, gs[0], gs[1]); };
+        for (int j = 0; j < di; j++) {
+            o.xb[j] = eval(SG2_COMP_XB, j);
+            o.z[j] = need_zc ? eval(SG2_COMP_Z, j) : (R)0;
+            o.dt[j] = O::softplus(eval(SG2_COMP_DT, j));
+        }
+        for (int s = 0; s < ds; s++) {
+            o.B[s] = eval(SG2_COMP_B, s);
+            o.C[s] = need_zc ? eval(SG2_COMP_C, s) : (R)0;
+        }
+        return;
+    }
     for (int j = 0; j < di; j++) {
         R a = 0, b = 0;
         for (int k = 0; k < dm; k++) a = O::fma((R)w.in_proj[j * dm + k], x[k], a);
@@ -233,7 +254,7 @@ void project(const Dims& d, const DirW<O>& w, const typename O::R* x, bool need_
 /* x: [N][d_model] in sorted order.  h: [d_inner][d_state] carried state,
  * updated in place.  ctx: [N][d_model], written at sorted position t. */
 template <class O>
-void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, int64_t N, bool reverse,
+void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const float* gs, int64_t N, bool reverse,
               int64_t chunk_len, int64_t window, typename O::R* h, typename O::R* ctx) {
     typedef typename O::R R;
     const int dm = d.d_model, di = d.d_inner, ds = d.d_state, hp = ds / 2;
@@ -260,7 +281,7 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, int64_t N
             }
             for (int64_t u = first; u < (c + 1) * chunk_len; u++) {
                 const int64_t t = reverse ? (N - 1 - u) : u;
-                project<O>(d, w, x + t * dm, false, sp);
+                project<O>(d, w, x + t * dm, gs + 2 * t, false, sp);
                 for (int j = 0; j < di; j++) {
                     const R dt = sp.dt[j], xb = sp.xb[j];
                     for (int p = 0; p < hp; p++) {
@@ -311,7 +332,7 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, int64_t N
         const int64_t u_end = std::min<int64_t>((c + 1) * chunk_len, N);
         for (int64_t u = c * chunk_len; u < u_end; u++) {
             const int64_t t = reverse ? (N - 1 - u) : u;
-            project<O>(d, w, x + t * dm, true, sp);
+            project<O>(d, w, x + t * dm, gs + 2 * t, true, sp);
             for (int j = 0; j < di; j++) {
                 const R dt = sp.dt[j], xb = sp.xb[j];
                 for (int p = 0; p < hp; p++) {
@@ -367,8 +388,11 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
 
     /* input projection, gathered into sorted order */
     std::vector<R> x((size_t)N * dm);
+    std::vector<float> gs_sorted((size_t)N * 2);
     for (int64_t t = 0; t < N; t++) {
         const R gv = g[perm[t]], sv = s[perm[t]];
+        gs_sorted[2 * t] = g[perm[t]];
+        gs_sorted[2 * t + 1] = s[perm[t]];
         for (int k = 0; k < dm; k++)
             x[t * dm + k] = O::fma((R)W[W_IN_W][2 * k + 1], sv, (R)W[W_IN_W][2 * k] * gv) + (R)W[W_IN_B][k];
     }
@@ -377,11 +401,19 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
     std::vector<R> hst[2];
     for (int dir = 0; dir < 2; dir++) {
         const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8]};
+        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0};
+        if (sizeof(R) == 4) {
+            w.comp_rows = std::max(di, ds);
+            w.comp.assign((size_t)SG2_COMP_GROUPS * w.comp_rows * 3, 0.0f);
+            for (int grp = 0; grp < SG2_COMP_GROUPS; grp++)
+                for (int row = 0; row < ((grp == SG2_COMP_B || grp == SG2_COMP_C) ? ds : di); row++)
+                    sg2_compose_one(grp, row, dm, di, W[W_IN_W], W[W_IN_B], W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4],
+                                    &w.comp[((size_t)grp * w.comp_rows + row) * 3]);
+        }
         float* st = dir ? mbwd_io : mfwd_io;
         hst[dir].assign(st, st + di * ds);
         ctx_sorted[dir].resize((size_t)N * dm);
-        scan_dir<O>(d, w, x.data(), N, dir == 1, chunk_len, window, hst[dir].data(), ctx_sorted[dir].data());
+        scan_dir<O>(d, w, x.data(), gs_sorted.data(), N, dir == 1, chunk_len, window, hst[dir].data(), ctx_sorted[dir].data());
         for (int i = 0; i < di * ds; i++) st[i] = (float)hst[dir][i];
     }
     /* unsort: element perm[t] takes the context computed at sorted position t */

@@ -75,6 +75,7 @@ struct Plan {
     uint32_t* blocksums;
     float* summaries;              // [2][wchunks][6][128]
     float* hstart;                 // [2][chunks][2][128]
+    float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
     float* ctx;                    // [2][total][DM]
     float decay, beta2, eps, rescale;
     Sg2Weights W;

@@ -40,6 +40,7 @@
 // rotation angle the sin/cos range reduction is skipped (bit-identical
 // results, see sg_sincos_small).
 #include "sg2_internal.hpp"
+#include "../../include/sg2_compose.h"
 
 namespace sg2 {
 namespace {
@@ -84,59 +85,54 @@ __device__ __forceinline__ float pair_tree_sum(float y) {
     return y + dpp_half_mirror(y);
 }
 
-// Projections of one timestep (x = projected input, 8 floats).  Both halves of
-// the workgroup compute the 16 x-branch values; each then produces its half
-// of dt / B (/ C / gate) and publishes its half of the x-branch rows.  HALF is
-// a template parameter so that every weight index is a compile-time constant
-// (scalar loads) and the register array is never indexed dynamically.
+// Composed coefficient triples (see sg2_compose.h), one thread per (direction, group, row).
+__global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
+    static_assert(DI == 16 && DS == 16, "k_compose: 16 rows per group");
+    const int dir = threadIdx.x / (SG2_COMP_GROUPS * 16), r = threadIdx.x % (SG2_COMP_GROUPS * 16);
+    const int group = r / 16, row = r % 16;
+    const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+    float out[3];
+    sg2_compose_one(group, row, DM, DI, pl.W.w[W_IN_W], pl.W.w[W_IN_B], pl.W.w[b], pl.W.w[b + 1], pl.W.w[b + 2], pl.W.w[b + 3],
+                    pl.W.w[b + 4], out);
+    float* dst = pl.comp + (size_t)threadIdx.x * 3;
+    dst[0] = out[0];
+    dst[1] = out[1];
+    dst[2] = out[2];
+}
+
+// Projections of one timestep from the element's (g, s).  Each half of the workgroup produces its
+// half of dt / x-branch / B (/ C / gate).  HALF is a template parameter so that every coefficient
+// index is a compile-time constant (scalar loads).  c points at this direction's coefficients.
 // Returns whether every rotation angle of this timestep, over this half's columns, is small enough
 // for sg_sincos_small (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
 template <bool OUT, int HALF>
-__device__ __forceinline__ bool project_tile(const DirW& w, const float (&x)[DM], int tu, float* s_dt, float* s_xb,
-                                             float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
+__device__ __forceinline__ bool project_tile(sg::cfloat_p c, float g, float s, int tu, float* s_dt, float* s_xb, float* s_B,
+                                             float* s_C, float* s_gate, const float* s_fmax) {
+    auto eval = [&](int group, int row) {
+        const sg::cfloat_p t = c + (group * 16 + row) * 3;
+        return sg_fma(t[0], g, sg_fma(t[1], s, t[2]));
+    };
     bool small = true;
-    float xb[DI];
-#pragma unroll
-    for (int jj = 0; jj < DI; jj++) {
-        float a = 0.0f;
-#pragma unroll
-        for (int k = 0; k < DM; k++) a = sg_fma(w.in_proj[jj * DM + k], x[k], a);
-        xb[jj] = a;
-    }
 #pragma unroll
     for (int q = 0; q < DI / 2; q++) {
         const int jj = HALF * (DI / 2) + q;
-        float a = w.dt_b[jj];
-#pragma unroll
-        for (int k = 0; k < DI; k++) a = sg_fma(w.dt_W[jj * DI + k], xb[k], a);
-        const float dtv = sg_softplus(a);
+        const float dtv = sg_softplus(eval(SG2_COMP_DT, jj));
         small = small && (dtv * s_fmax[jj] < SG_SINCOS_SMALL_LIMIT);
         s_dt[jj * LDS_STRIDE + tu] = dtv;
-        s_xb[jj * LDS_STRIDE + tu] = xb[jj];
+        s_xb[jj * LDS_STRIDE + tu] = eval(SG2_COMP_XB, jj);
     }
 #pragma unroll
     for (int q = 0; q < DS / 2; q++) {
         const int ss = HALF * (DS / 2) + q;
-        float a = 0.0f;
-#pragma unroll
-        for (int k = 0; k < DI; k++) a = sg_fma(w.Bp[ss * DI + k], xb[k], a);
-        s_B[ss * LDS_STRIDE + tu] = a;
-        if (OUT) {
-            float b = 0.0f;
-#pragma unroll
-            for (int k = 0; k < DI; k++) b = sg_fma(w.Cp[ss * DI + k], xb[k], b);
-            s_C[ss * LDS_STRIDE + tu] = b;
-        }
+        s_B[ss * LDS_STRIDE + tu] = eval(SG2_COMP_B, ss);
+        if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(SG2_COMP_C, ss);
     }
     if (OUT) {
 #pragma unroll
         for (int q = 0; q < DI / 2; q++) {
             const int jj = HALF * (DI / 2) + q;
-            float z = 0.0f;
-#pragma unroll
-            for (int k = 0; k < DM; k++) z = sg_fma(w.in_proj[(jj + DI) * DM + k], x[k], z);
-            s_gate[jj * LDS_STRIDE + tu] = sg_silu(z);
+            s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(SG2_COMP_Z, jj));
         }
     }
     return small;
@@ -215,8 +211,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const uint32_t* __restrict__ skey = pl.keys[0] + off;      // sorted |g| bits
     const int32_t* __restrict__ sval = pl.vals[0] + off;       // element index | sign of g
     const float* __restrict__ ssrt = pl.ssorted + off;          // sharpness in sorted order
-    const sg::cfloat_p Wi = sg::as_const(pl.W.w[W_IN_W]);
-    const sg::cfloat_p bi = sg::as_const(pl.W.w[W_IN_B]);
+    const sg::cfloat_p comp0 = sg::as_const(pl.comp) + dir * (SG2_COMP_GROUPS * 16 * 3);
 
     const int tid = threadIdx.x;
     const int tu = tid & (SCAN_TT - 1);                                   // projection role: timestep of the tile
@@ -253,33 +248,29 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     for (;;) {
     for (int tile0 = first; tile0 < u1; tile0 += SCAN_TT) {
         const int cnt = min(SCAN_TT, u1 - tile0);
-        // the projection weights are re-read (scalar loads, cache hits) in every tile instead of being hoisted
+        // the coefficients are re-read (scalar loads, cache hits) in every tile instead of being hoisted
         const int zo = sg::opaque_zero();
         const DirW w = {w0.in_proj + zo, w0.dt_W + zo, w0.dt_b + zo, w0.Bp + zo, w0.Cp + zo,
                         w0.A_log + zo, w0.D + zo, w0.rope + zo, w0.out_proj + zo};
+        const sg::cfloat_p comp = comp0 + zo;
         // ---------------- phase A: projections of SCAN_TT timesteps -> LDS
         const int u = tile0 + tu;
         const bool valid = u < u1;
         int orig = 0;
-        float x[DM];
-        {
-            float g = 0.0f, s = 0.0f;
-            if (valid) {
-                const int t = dir ? (N - 1 - u) : u;
-                const int32_t v = sval[t];
-                orig = v & 0x7fffffff;
-                orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
-                g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
-                s = ssrt[t];
-            }
-#pragma unroll
-            for (int k = 0; k < DM; k++) x[k] = sg_fma(Wi[2 * k + 1], s, Wi[2 * k] * g) + bi[k];
+        float g = 0.0f, sh = 0.0f;
+        if (valid) {
+            const int t = dir ? (N - 1 - u) : u;
+            const int32_t v = sval[t];
+            orig = v & 0x7fffffff;
+            orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
+            g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
+            sh = ssrt[t];
         }
         bool small_t;
         if (half == 0)
-            small_t = project_tile<OUT, 0>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
+            small_t = project_tile<OUT, 0>(comp, g, sh, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
         else
-            small_t = project_tile<OUT, 1>(w, x, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
+            small_t = project_tile<OUT, 1>(comp, g, sh, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
         {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!small_t);
             if (tu == 0) s_large[half] = large;
@@ -456,6 +447,8 @@ __global__ __launch_bounds__(PREFIX_GROUPS * SCAN_THREADS) void k_chunk_prefix(P
 
 int launch_scan(const Plan& pl, hipStream_t st) {
     if (pl.total == 0) return 0;
+    hipLaunchKernelGGL(k_compose, dim3(1), dim3(2 * SG2_COMP_GROUPS * 16), 0, st, pl);
+    SG_LAUNCH_CHECK("k_compose");
     if (pl.wchunks > 0) {
         hipLaunchKernelGGL(k_scan<false>, dim3(2 * pl.wchunks), dim3(SCAN_THREADS), 0, st, pl);
         SG_LAUNCH_CHECK("k_scan<summary>");

@@ -38,7 +38,7 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_ctx, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_ctx, bytes;
     size_t tables_bytes;
 };
 
@@ -70,6 +70,7 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
     L->off_blocksums = take(4 * (size_t)(L->nb + 1));
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * SCAN_THREADS);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * SCAN_THREADS);
+    L->off_comp = take(4 * 2 * 5 * 16 * 3);
     L->off_ctx = take(4 * 2 * (size_t)total * DM);
     L->bytes = o;
     return 0;
@@ -238,6 +239,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.blocksums = reinterpret_cast<uint32_t*>(ws + L.off_blocksums);
     pl.summaries = reinterpret_cast<float*>(ws + L.off_summ);
     pl.hstart = reinterpret_cast<float*>(ws + L.off_hstart);
+    pl.comp = reinterpret_cast<float*>(ws + L.off_comp);
     pl.ctx = reinterpret_cast<float*>(ws + L.off_ctx);
     pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
