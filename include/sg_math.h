@@ -177,6 +177,36 @@ SG_HD void sg_abar_pair(float dt, float nhA_e, float nhA_o, float* ab_e, float* 
     *ab_o = sg_fma(d_e, r2, -1.0f);
 }
 
+/* The same A_bar values for a block of n <= 16 consecutive timesteps of one lane with ONE reciprocal
+ * (simultaneous inversion): with D_k = (1+t_e,k)(1+t_o,k) and prefix products P_k = D_0 ... D_k,
+ *   1/D_k = (1/P_{n-1}) * (D_{k+1} ... D_{n-1}) * P_{k-1}.
+ * sg_abar_block_prefix forms d_e, d_o and P and returns P_{n-1}; the caller uses the block form only
+ * while that product is below SG_ABAR_BLOCK_LIMIT (all D_k >= 1, so a finite small last product
+ * means every partial product is finite too), and sg_abar_pair per timestep otherwise.  Results differ
+ * from sg_abar_pair in the last bits (a few more roundings), so both sides of a parity comparison must
+ * group the timesteps the same way. */
+#define SG_ABAR_BLOCK_LIMIT 1e30f
+SG_HD float sg_abar_block_prefix(int n, const float* dt, float nhA_e, float nhA_o, float* d_e, float* d_o, float* P) {
+    float acc = 1.0f;
+    for (int k = 0; k < n; k++) {
+        d_e[k] = sg_fma(dt[k], nhA_e, 1.0f);
+        d_o[k] = sg_fma(dt[k], nhA_o, 1.0f);
+        acc = (k == 0) ? d_e[k] * d_o[k] : acc * (d_e[k] * d_o[k]);
+        P[k] = acc;
+    }
+    return acc;
+}
+SG_HD void sg_abar_block_finish(int n, const float* d_e, const float* d_o, const float* P, float* ab_e, float* ab_o) {
+    float r = sg_rcp_pos(P[n - 1]);
+    for (int k = n - 1; k >= 0; k--) {
+        const float inv = (k > 0) ? r * P[k - 1] : r;      /* 1/D_k */
+        if (k > 0) r = r * (d_e[k] * d_o[k]);
+        const float r2 = inv + inv;
+        ab_e[k] = sg_fma(d_o[k], r2, -1.0f);
+        ab_o[k] = sg_fma(d_e[k], r2, -1.0f);
+    }
+}
+
 SG_HD float sg_tanh(float x) {
     const float ax = sg_abs(x);
     float y;

@@ -251,6 +251,75 @@ void project(const Dims& d, const DirW<O>& w, const typename O::R* x, const floa
     }
 }
 
+/* Coefficients of up to 64 consecutive scan steps (one tile of the device kernel): projections, A_bar and
+ * sin/cos per (step, column, pair).  The fp32 policy groups the A_bar exactly like the device: blocks of 8
+ * steps counted from the tile start share one reciprocal per lane (sg_abar_block_*), unless some lane of the
+ * block's 64-lane wave (lanes ordered column-major, 8 pairs per column) exceeds SG_ABAR_BLOCK_LIMIT; the ragged
+ * end of a tile and the fp64 policy take the per-step formula. */
+template <class O>
+struct TileCoef {
+    std::vector<StepProj<O>> sp;
+    std::vector<typename O::R> ae, ao, sn, cs;
+};
+enum { ORC_TILE = 64, ORC_BLOCK = 8, ORC_WAVE = 64 };
+
+template <class O>
+void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typename O::R>& A, const typename O::R* x,
+                       const float* gs, int64_t N, bool reverse, int64_t u0, int cnt, bool need_zc, TileCoef<O>& tc) {
+    typedef typename O::R R;
+    const int dm = d.d_model, di = d.d_inner, ds = d.d_state, hp = ds / 2, lanes = di * hp;
+    tc.sp.resize(ORC_TILE);
+    tc.ae.resize((size_t)ORC_TILE * lanes);
+    tc.ao.resize((size_t)ORC_TILE * lanes);
+    tc.sn.resize((size_t)ORC_TILE * lanes);
+    tc.cs.resize((size_t)ORC_TILE * lanes);
+    for (int k = 0; k < cnt; k++) {
+        const int64_t u = u0 + k, t = reverse ? (N - 1 - u) : u;
+        project<O>(d, w, x + t * dm, gs + 2 * t, need_zc, tc.sp[k]);
+        for (int j = 0; j < di; j++)
+            for (int p = 0; p < hp; p++)
+                O::sincos(tc.sp[k].dt[j] * (R)w.rope[j * hp + p], &tc.sn[(size_t)k * lanes + j * hp + p],
+                          &tc.cs[(size_t)k * lanes + j * hp + p]);
+    }
+    int k0 = 0;
+    if (sizeof(R) == 4) {
+        std::vector<float> de((size_t)lanes * ORC_BLOCK), dod((size_t)lanes * ORC_BLOCK), P((size_t)lanes * ORC_BLOCK);
+        for (; k0 + ORC_BLOCK <= cnt; k0 += ORC_BLOCK) {
+            for (int wave0 = 0; wave0 < lanes; wave0 += ORC_WAVE) {
+                const int wave1 = std::min(lanes, wave0 + ORC_WAVE);
+                bool block_ok = true;
+                for (int l = wave0; l < wave1; l++) {
+                    const int j = l / hp, p = l % hp;
+                    float dts[ORC_BLOCK];
+                    for (int q = 0; q < ORC_BLOCK; q++) dts[q] = (float)tc.sp[k0 + q].dt[j];
+                    const float last = sg_abar_block_prefix(ORC_BLOCK, dts, -0.5f * (float)A[j * ds + 2 * p], -0.5f * (float)A[j * ds + 2 * p + 1],
+                                                            &de[(size_t)l * ORC_BLOCK], &dod[(size_t)l * ORC_BLOCK], &P[(size_t)l * ORC_BLOCK]);
+                    if (!(last < SG_ABAR_BLOCK_LIMIT)) block_ok = false;
+                }
+                for (int l = wave0; l < wave1; l++) {
+                    const int j = l / hp, p = l % hp;
+                    float e[ORC_BLOCK], o[ORC_BLOCK];
+                    if (block_ok) {
+                        sg_abar_block_finish(ORC_BLOCK, &de[(size_t)l * ORC_BLOCK], &dod[(size_t)l * ORC_BLOCK], &P[(size_t)l * ORC_BLOCK], e, o);
+                    } else {
+                        for (int q = 0; q < ORC_BLOCK; q++)
+                            sg_abar_pair((float)tc.sp[k0 + q].dt[j], -0.5f * (float)A[j * ds + 2 * p], -0.5f * (float)A[j * ds + 2 * p + 1], &e[q], &o[q]);
+                    }
+                    for (int q = 0; q < ORC_BLOCK; q++) {
+                        tc.ae[(size_t)(k0 + q) * lanes + l] = (R)e[q];
+                        tc.ao[(size_t)(k0 + q) * lanes + l] = (R)o[q];
+                    }
+                }
+            }
+        }
+    }
+    for (; k0 < cnt; k0++)
+        for (int j = 0; j < di; j++)
+            for (int p = 0; p < hp; p++)
+                O::abar_pair(tc.sp[k0].dt[j], A[j * ds + 2 * p], A[j * ds + 2 * p + 1], &tc.ae[(size_t)k0 * lanes + j * hp + p],
+                             &tc.ao[(size_t)k0 * lanes + j * hp + p]);
+}
+
 /* x: [N][d_model] in sorted order.  h: [d_inner][d_state] carried state,
  * updated in place.  ctx: [N][d_model], written at sorted position t. */
 template <class O>
@@ -267,7 +336,7 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
 
     std::vector<R> hstart((size_t)nchunks * di * ds);
     std::copy(h, h + di * ds, hstart.begin());
-    StepProj<O> sp;
+    TileCoef<O> tc;
 
     /* pass 1 + 2: summaries of chunks 0..nchunks-2, start states of 1..nchunks-1 */
     std::vector<R> sm(di * hp * 6);
@@ -279,23 +348,25 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
                 R* m = &sm[i * 6];
                 m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 1; m[4] = 0; m[5] = 0;   /* col0=(m0,m1) col1=(m2,m3) b=(m4,m5) */
             }
-            for (int64_t u = first; u < (c + 1) * chunk_len; u++) {
-                const int64_t t = reverse ? (N - 1 - u) : u;
-                project<O>(d, w, x + t * dm, gs + 2 * t, false, sp);
-                for (int j = 0; j < di; j++) {
-                    const R dt = sp.dt[j], xb = sp.xb[j];
-                    for (int p = 0; p < hp; p++) {
-                        R ae, ao, sn, cs;
-                        O::abar_pair(dt, A[j * ds + 2 * p], A[j * ds + 2 * p + 1], &ae, &ao);
-                        O::sincos(dt * (R)w.rope[j * hp + p], &sn, &cs);
-                        const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
-                        R* m = &sm[(j * hp + p) * 6];
-                        for (int v = 0; v < 3; v++) {
-                            const R ve = m[2 * v], vo = m[2 * v + 1];
-                            const R re = O::fma(ve, cs, -(vo * sn));
-                            const R ro = O::fma(vo, cs, ve * sn);
-                            if (v < 2) { m[2 * v] = ae * re; m[2 * v + 1] = ao * ro; }
-                            else { m[4] = O::fma(ae, re, be); m[5] = O::fma(ao, ro, bo); }
+            for (int64_t tile0 = first; tile0 < (c + 1) * chunk_len; tile0 += ORC_TILE) {
+                const int cnt = (int)std::min<int64_t>(ORC_TILE, (c + 1) * chunk_len - tile0);
+                tile_coefficients<O>(d, w, A, x, gs, N, reverse, tile0, cnt, false, tc);
+                for (int k = 0; k < cnt; k++) {
+                    const StepProj<O>& sp = tc.sp[k];
+                    for (int j = 0; j < di; j++) {
+                        const R dt = sp.dt[j], xb = sp.xb[j];
+                        for (int p = 0; p < hp; p++) {
+                            const size_t li = (size_t)k * di * hp + j * hp + p;
+                            const R ae = tc.ae[li], ao = tc.ao[li], sn = tc.sn[li], cs = tc.cs[li];
+                            const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
+                            R* m = &sm[(j * hp + p) * 6];
+                            for (int v = 0; v < 3; v++) {
+                                const R ve = m[2 * v], vo = m[2 * v + 1];
+                                const R re = O::fma(ve, cs, -(vo * sn));
+                                const R ro = O::fma(vo, cs, ve * sn);
+                                if (v < 2) { m[2 * v] = ae * re; m[2 * v + 1] = ao * ro; }
+                                else { m[4] = O::fma(ae, re, be); m[5] = O::fma(ao, ro, bo); }
+                            }
                         }
                     }
                 }
@@ -330,33 +401,36 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
     for (int64_t c = 0; c < nchunks; c++) {
         std::copy(&hstart[(size_t)c * di * ds], &hstart[(size_t)c * di * ds] + di * ds, hc.begin());
         const int64_t u_end = std::min<int64_t>((c + 1) * chunk_len, N);
-        for (int64_t u = c * chunk_len; u < u_end; u++) {
-            const int64_t t = reverse ? (N - 1 - u) : u;
-            project<O>(d, w, x + t * dm, gs + 2 * t, true, sp);
-            for (int j = 0; j < di; j++) {
-                const R dt = sp.dt[j], xb = sp.xb[j];
-                for (int p = 0; p < hp; p++) {
-                    R ae, ao, sn, cs;
-                    O::abar_pair(dt, A[j * ds + 2 * p], A[j * ds + 2 * p + 1], &ae, &ao);
-                    O::sincos(dt * (R)w.rope[j * hp + p], &sn, &cs);
-                    const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
-                    const R he = hc[j * ds + 2 * p], ho = hc[j * ds + 2 * p + 1];
-                    const R re = O::fma(he, cs, -(ho * sn));
-                    const R ro = O::fma(ho, cs, he * sn);
-                    const R ne = O::fma(ae, re, be), no = O::fma(ao, ro, bo);
-                    hc[j * ds + 2 * p] = ne;
-                    hc[j * ds + 2 * p + 1] = no;
-                    yp[p] = O::fma(no, sp.C[2 * p + 1], ne * sp.C[2 * p]);
+        for (int64_t tile0 = c * chunk_len; tile0 < u_end; tile0 += ORC_TILE) {
+            const int cnt = (int)std::min<int64_t>(ORC_TILE, u_end - tile0);
+            tile_coefficients<O>(d, w, A, x, gs, N, reverse, tile0, cnt, true, tc);
+            for (int k = 0; k < cnt; k++) {
+                const int64_t u = tile0 + k, t = reverse ? (N - 1 - u) : u;
+                const StepProj<O>& sp = tc.sp[k];
+                for (int j = 0; j < di; j++) {
+                    const R dt = sp.dt[j], xb = sp.xb[j];
+                    for (int p = 0; p < hp; p++) {
+                        const size_t li = (size_t)k * di * hp + j * hp + p;
+                        const R ae = tc.ae[li], ao = tc.ao[li], sn = tc.sn[li], cs = tc.cs[li];
+                        const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
+                        const R he = hc[j * ds + 2 * p], ho = hc[j * ds + 2 * p + 1];
+                        const R re = O::fma(he, cs, -(ho * sn));
+                        const R ro = O::fma(ho, cs, he * sn);
+                        const R ne = O::fma(ae, re, be), no = O::fma(ao, ro, bo);
+                        hc[j * ds + 2 * p] = ne;
+                        hc[j * ds + 2 * p + 1] = no;
+                        yp[p] = O::fma(no, sp.C[2 * p + 1], ne * sp.C[2 * p]);
+                    }
+                    /* balanced pairwise sum over the RoPE pairs (stride 1, 2, 4, ...) */
+                    for (int st = 1; st < hp; st *= 2)
+                        for (int p = 0; p + st < hp; p += 2 * st) yp[p] = yp[p] + yp[p + st];
+                    out[j] = O::fma(yp[0], O::silu(sp.z[j]), (R)w.D[j] * xb);
                 }
-                /* balanced pairwise sum over the RoPE pairs (stride 1, 2, 4, ...) */
-                for (int st = 1; st < hp; st *= 2)
-                    for (int p = 0; p + st < hp; p += 2 * st) yp[p] = yp[p] + yp[p + st];
-                out[j] = O::fma(yp[0], O::silu(sp.z[j]), (R)w.D[j] * xb);
-            }
-            for (int dd = 0; dd < dm; dd++) {
-                R a = 0;
-                for (int j = 0; j < di; j++) a = O::fma((R)w.out_proj[dd * di + j], out[j], a);
-                ctx[t * dm + dd] = a;
+                for (int dd = 0; dd < dm; dd++) {
+                    R a = 0;
+                    for (int j = 0; j < di; j++) a = O::fma((R)w.out_proj[dd * di + j], out[j], a);
+                    ctx[t * dm + dd] = a;
+                }
             }
         }
     }

@@ -101,14 +101,14 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
 }
 
 // Projections of one timestep from the element's (g, s).  Each half of the workgroup produces its
-// half of dt / x-branch / B (/ C / gate).  HALF is a template parameter so that every coefficient
+// half of dt / dt*x-branch / B (/ D*x-branch / C / gate).  HALF is a template parameter so that every coefficient
 // index is a compile-time constant (scalar loads).  c points at this direction's coefficients.
 // Returns whether every rotation angle of this timestep, over this half's columns, is small enough
 // for sg_sincos_small (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
 template <bool OUT, int HALF>
-__device__ __forceinline__ bool project_tile(sg::cfloat_p c, float g, float s, int tu, float* s_dt, float* s_xb, float* s_B,
-                                             float* s_C, float* s_gate, const float* s_fmax) {
+__device__ __forceinline__ bool project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt, float* s_ux,
+                                             float* s_dx, float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
     auto eval = [&](int group, int row) {
         const sg::cfloat_p t = c + (group * 16 + row) * 3;
         return sg_fma(t[0], g, sg_fma(t[1], s, t[2]));
@@ -119,8 +119,10 @@ __device__ __forceinline__ bool project_tile(sg::cfloat_p c, float g, float s, i
         const int jj = HALF * (DI / 2) + q;
         const float dtv = sg_softplus(eval(SG2_COMP_DT, jj));
         small = small && (dtv * s_fmax[jj] < SG_SINCOS_SMALL_LIMIT);
+        const float xbv = eval(SG2_COMP_XB, jj);
         s_dt[jj * LDS_STRIDE + tu] = dtv;
-        s_xb[jj * LDS_STRIDE + tu] = eval(SG2_COMP_XB, jj);
+        s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
+        if (OUT) s_dx[jj * LDS_STRIDE + tu] = Dw[jj] * xbv;
     }
 #pragma unroll
     for (int q = 0; q < DS / 2; q++) {
@@ -160,20 +162,30 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
     S.ho = sg_fma(ao, ro, bo);
 }
 
-// UB consecutive timesteps (all valid): coefficients first, then the serial chain
+// UB consecutive timesteps (all valid): coefficients first, then the serial chain.  ux = dt * x-branch
+// (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
+// (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
 template <bool OUT, bool SMALL_ANGLE>
-__device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&xv)[UB], const float (&Be)[UB],
+__device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, float (&y)[UB]) {
     float ae[UB], ao[UB], sn[UB], cs[UB], be[UB], bo[UB];
+    {
+        float d_e[UB], d_o[UB], P[UB];
+        const float last = sg_abar_block_prefix(UB, dt, hAe, hAo, d_e, d_o, P);
+        if (__builtin_amdgcn_ballot_w64(!(last < SG_ABAR_BLOCK_LIMIT)) == 0) {
+            sg_abar_block_finish(UB, d_e, d_o, P, ae, ao);
+        } else {
+#pragma unroll
+            for (int u = 0; u < UB; u++) sg_abar_pair(dt[u], hAe, hAo, &ae[u], &ao[u]);
+        }
+    }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
-        sg_abar_pair(dt[u], hAe, hAo, &ae[u], &ao[u]);
         if (SMALL_ANGLE) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
         else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
-        const float ux = dt[u] * xv[u];
-        be[u] = ux * Be[u];
-        bo[u] = ux * Bo[u];
+        be[u] = ux[u] * Be[u];
+        bo[u] = ux[u] * Bo[u];
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
@@ -189,11 +201,13 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
 template <bool OUT>
 __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     __shared__ __attribute__((aligned(16))) float s_dt[DI * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) float s_xb[DI * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_ux[DI * LDS_STRIDE];       // dt * x-branch
     __shared__ __attribute__((aligned(16))) float s_B[DS * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) float s_C[OUT ? DS * LDS_STRIDE : 1];
     __shared__ __attribute__((aligned(16))) float s_gate[OUT ? DI * LDS_STRIDE : 1];
-    __shared__ __attribute__((aligned(16))) float s_y[OUT ? DI * LDS_STRIDE : 1];
+    __shared__ __attribute__((aligned(16))) float s_dx[OUT ? DI * LDS_STRIDE : 1];   // D * x-branch (skip term)
+    // y of column j goes where dt of column j was: both are touched only by the 8 lanes of column j, in program order
+    float* const s_y = s_dt;
     __shared__ float s_fmax[DI];
     __shared__ unsigned long long s_large[2];      // per projection half: bit t set = timestep t of the tile needs the full sin/cos
 
@@ -268,9 +282,9 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         }
         bool small_t;
         if (half == 0)
-            small_t = project_tile<OUT, 0>(comp, g, sh, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
+            small_t = project_tile<OUT, 0>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         else
-            small_t = project_tile<OUT, 1>(comp, g, sh, tu, s_dt, s_xb, s_B, s_C, s_gate, s_fmax);
+            small_t = project_tile<OUT, 1>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!small_t);
             if (tu == 0) s_large[half] = large;
@@ -280,7 +294,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
 
         // ---------------- phase B: the recurrence over the tile, lane = (j,p)
         const float* __restrict__ r_dt = s_dt + j * LDS_STRIDE;
-        const float* __restrict__ r_xb = s_xb + j * LDS_STRIDE;
+        const float* __restrict__ r_ux = s_ux + j * LDS_STRIDE;
         const float* __restrict__ r_Be = s_B + (2 * p) * LDS_STRIDE;
         const float* __restrict__ r_Bo = s_B + (2 * p + 1) * LDS_STRIDE;
         const float* __restrict__ r_Ce = s_C + (OUT ? (2 * p) * LDS_STRIDE : 0);
@@ -290,7 +304,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             float dt[UB], xv[UB], Be[UB], Bo[UB], Ce[UB], Co[UB], y[UB];
 #pragma unroll
             for (int q = 0; q < UB; q += 4) {
-                const f32x4 a = *reinterpret_cast<const f32x4*>(r_dt + k0 + q), b = *reinterpret_cast<const f32x4*>(r_xb + k0 + q);
+                const f32x4 a = *reinterpret_cast<const f32x4*>(r_dt + k0 + q), b = *reinterpret_cast<const f32x4*>(r_ux + k0 + q);
                 const f32x4 c = *reinterpret_cast<const f32x4*>(r_Be + k0 + q), d = *reinterpret_cast<const f32x4*>(r_Bo + k0 + q);
 #pragma unroll
                 for (int e = 0; e < 4; e++) { dt[q + e] = a[e]; xv[q + e] = b[e]; Be[q + e] = c[e]; Bo[q + e] = d[e]; Ce[q + e] = 0.0f; Co[q + e] = 0.0f; }
@@ -311,11 +325,10 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             }
         }
         for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
-            const float dt = r_dt[k0], xv = r_xb[k0];
+            const float dt = r_dt[k0], ux = r_ux[k0];
             float ae, ao, sn, cs;
             sg_abar_pair(dt, hAe, hAo, &ae, &ao);
             sg_sincos(dt * freq, &sn, &cs);
-            const float ux = dt * xv;
             step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             if (OUT) {
                 const float y = pair_tree_sum(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
@@ -329,8 +342,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             float o[DI];
 #pragma unroll
             for (int jj = 0; jj < DI; jj++)
-                o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], s_gate[jj * LDS_STRIDE + tu],
-                               w.D[jj] * s_xb[jj * LDS_STRIDE + tu]);
+                o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], s_gate[jj * LDS_STRIDE + tu], s_dx[jj * LDS_STRIDE + tu]);
             float cx[DM / 2];
 #pragma unroll
             for (int q = 0; q < DM / 2; q++) {

@@ -111,6 +111,23 @@ def test_edge_cases():
             assert torch.isfinite(v.float()).all(), k
 
 
+def test_wide_dynamic_range_gradients():
+    """|g| log-uniform over 1e-6 .. 1e5: the largest step sizes overflow the product of A_bar denominators of an
+    8-step block, so the sorted sequence mixes blocks that share one reciprocal with blocks that fall back to
+    the per-step form; device and checker have to take the same decision for every block."""
+    shapes = [(3000,), (700,), (64, 130)]
+    case = Sg2Case(shapes, seed=11)
+    r = np.random.RandomState(5)
+    for t in range(1, 3):
+        grads = [torch.from_numpy((10.0 ** r.uniform(-6, 5, size=int(np.prod(s)))
+                                   * r.choice([-1.0, 1.0], size=int(np.prod(s)))).astype(np.float32)).reshape(s) for s in shapes]
+        sharps = [torch.zeros_like(g) for g in grads]
+        pt, sh = per_tensor_scalars(case.P, t, 0.0), shared_scalars(1.0)
+        print("wide range step", t, flush=True)
+        case.gpu_step(grads, sharps, pt, sh)
+        print("worst tolerance ratios", case.compare(case.oracle_step(grads, sharps, pt, sh, None), REL, FLOOR))
+
+
 def test_heavy_ties_sort_is_stable():
     """Quantised gradients: thousands of exact ties; permutation must equal the stable argsort."""
     shapes = [(20000,), (9000,)]
