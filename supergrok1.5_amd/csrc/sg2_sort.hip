@@ -184,9 +184,29 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
         }
     }
     __syncthreads();
-    {   // digit d = threadIdx.x: turn per-wave counts into per-wave destinations
+    // digit d = threadIdx.x: position of each wave's first key of digit d inside the tile's digit-sorted order
+    // (cnt[k][d]), start of digit d in that order (lbase[d]) and its distance to the global destination (gdelta[d])
+    __shared__ uint32_t lbase[256], gdelta[256], wsum[WAVES];
+    {
         const int d = threadIdx.x;
-        uint32_t run = pl.spine[tr.spine0 + d * tr.stride];
+        uint32_t tot = 0;
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) tot += cnt[k][d];
+        uint32_t inc = tot;     // inclusive scan over the 64 digits of this wave, then across the 4 waves
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += up;
+        }
+        if (lane == 63) wsum[w] = inc;
+        __syncthreads();
+        uint32_t before = 0;
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) before += (k < w) ? wsum[k] : 0u;
+        const uint32_t lb = before + inc - tot;
+        lbase[d] = lb;
+        gdelta[d] = pl.spine[tr.spine0 + d * tr.stride] - lb;     // global destination = gdelta[d] + local position (mod 2^32)
+        uint32_t run = lb;
 #pragma unroll
         for (int k = 0; k < WAVES; k++) {
             const uint32_t c = cnt[k][d];
@@ -195,15 +215,30 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
         }
     }
     __syncthreads();
-    uint32_t* __restrict__ kout = pl.keys[src ^ 1];
-    int32_t* __restrict__ vout = pl.vals[src ^ 1];
+    // reorder through LDS so that global stores go out in digit-sorted order: consecutive lanes then write
+    // consecutive addresses within each digit's run instead of 4-byte pieces all over the tile's 256 runs
+    __shared__ uint32_t skey[SORT_TILE];
+    __shared__ int32_t sval[SORT_TILE];
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int i = w * WAVE_ITEMS + r * 64 + lane;
         if (i < tr.cnt) {
-            const uint32_t dst = cnt[w][(key[r] >> shift) & 255u] + rank[r];
-            kout[dst] = key[r];
-            vout[dst] = val[r];
+            const uint32_t lp = cnt[w][(key[r] >> shift) & 255u] + rank[r];
+            skey[lp] = key[r];
+            sval[lp] = val[r];
+        }
+    }
+    __syncthreads();
+    uint32_t* __restrict__ kout = pl.keys[src ^ 1];
+    int32_t* __restrict__ vout = pl.vals[src ^ 1];
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int lp = r * SORT_THREADS + threadIdx.x;
+        if (lp < tr.cnt) {
+            const uint32_t kk = skey[lp];
+            const uint32_t dst = gdelta[(kk >> shift) & 255u] + (uint32_t)lp;
+            kout[dst] = kk;
+            vout[dst] = sval[lp];
         }
     }
 }
