@@ -130,7 +130,19 @@ __global__ __launch_bounds__(THREADS) void k_sumsq_partial(Batch<NormRec> B) {
     int start, cnt;
     const NormRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
     float acc = 0.0f;
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
+    int done = 0;
+    if (R.dtype == SG_F32 && ((uintptr_t)R.grad & 15u) == 0) {     // four elements per lane and access
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        done = cnt & ~3;
+        for (int k = threadIdx.x * 4; k < done; k += THREADS * 4) {
+            const f32x4 g = *reinterpret_cast<const f32x4*>(static_cast<const float*>(R.grad) + start + k);
+            acc = sg_fma(g[0], g[0], acc);
+            acc = sg_fma(g[1], g[1], acc);
+            acc = sg_fma(g[2], g[2], acc);
+            acc = sg_fma(g[3], g[3], acc);
+        }
+    }
+    for (int k = done + threadIdx.x; k < cnt; k += THREADS) {
         const float g = sg::load_elem(R.grad, R.dtype, start + k);
         acc = sg_fma(g, g, acc);
     }

@@ -27,7 +27,24 @@ struct FamRec {
     int64_t numel;
     int32_t dtype;
     float bc1, bc2, alpha, beta1;
+    int32_t vec4;          // fp32 tensor and every pointer 16-byte aligned: four elements per lane and access
 };
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4 ld4(const void* p, int i) { return *reinterpret_cast<const f32x4*>(static_cast<const float*>(p) + i); }
+__device__ __forceinline__ void st4(void* p, int i, f32x4 v) { *reinterpret_cast<f32x4*>(static_cast<float*>(p) + i) = v; }
+
+// Runs body(i) for every element of the tile; when the tensor allows 16-byte accesses, body4(i) handles four
+// consecutive elements per lane and body(i) only the ragged end.
+template <class B1, class B4>
+__device__ __forceinline__ void for_tile(const FamRec& R, int start, int cnt, B1 body, B4 body4) {
+    int done = 0;
+    if (R.vec4) {
+        done = cnt & ~3;
+        for (int k = threadIdx.x * 4; k < done; k += THREADS * 4) body4(start + k);
+    }
+    for (int k = done + threadIdx.x; k < cnt; k += THREADS) body(start + k);
+}
 
 // clipped gradient, written back in place when clipping is active (clip_grad_norms_device_side, csrc/ops.cpp:23-55)
 __device__ __forceinline__ float clipped_grad(const FamRec& R, int i, bool clip_on, float coef) {
@@ -38,17 +55,44 @@ __device__ __forceinline__ float clipped_grad(const FamRec& R, int i, bool clip_
     }
     return g;
 }
+__device__ __forceinline__ f32x4 clipped_grad4(const FamRec& R, int i, bool clip_on, float coef) {
+    f32x4 g = ld4(R.grad, i);
+    if (clip_on) {
+        g = g * coef;
+        st4(R.grad, i, g);
+    }
+    return g;
+}
 
 // decoupled decay, then the Adam step: p*(1 - lr*wd) - (lr/bc1) * ea / (sqrt(easq/bc2) + eps)
+__device__ __forceinline__ float adam_core(float fg, float p, float& ea, float& easq, float beta1, float beta2, float bc2,
+                                           float eps_eff, float decay, float step_size) {
+    ea = sg_fma(beta1, ea, (1.0f - beta1) * fg);
+    easq = sg_fma(beta2, easq, ((1.0f - beta2) * fg) * fg);
+    const float denom = __builtin_sqrtf(easq / bc2) + eps_eff;
+    return sg_fma(p, decay, -((step_size * ea) / denom));
+}
 __device__ __forceinline__ void adam_update(const FamRec& R, int i, float fg, float beta1, float beta2, float eps_eff, float decay,
                                             float step_size) {
-    const float ea = sg_fma(beta1, R.ea[i], (1.0f - beta1) * fg);
-    const float easq = sg_fma(beta2, R.easq[i], ((1.0f - beta2) * fg) * fg);
+    float ea = R.ea[i], easq = R.easq[i];
+    const float p = adam_core(fg, sg::load_elem(R.param, R.dtype, i), ea, easq, beta1, beta2, R.bc2, eps_eff, decay, step_size);
     R.ea[i] = ea;
     R.easq[i] = easq;
-    const float denom = __builtin_sqrtf(easq / R.bc2) + eps_eff;
-    const float p = sg::load_elem(R.param, R.dtype, i);
-    sg::store_elem(R.param, R.dtype, i, sg_fma(p, decay, -((step_size * ea) / denom)));
+    sg::store_elem(R.param, R.dtype, i, p);
+}
+__device__ __forceinline__ void adam_update4(const FamRec& R, int i, f32x4 fg, float beta1, float beta2, float eps_eff, float decay,
+                                             float step_size) {
+    f32x4 ea = ld4(R.ea, i), easq = ld4(R.easq, i), p = ld4(R.param, i);
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        float a = ea[c], q = easq[c];
+        p[c] = adam_core(fg[c], p[c], a, q, beta1, beta2, R.bc2, eps_eff, decay, step_size);
+        ea[c] = a;
+        easq[c] = q;
+    }
+    st4(R.ea, i, ea);
+    st4(R.easq, i, easq);
+    st4(R.param, i, p);
 }
 
 __global__ __launch_bounds__(THREADS) void k_grokadamw(Batch<FamRec> B, float alpha, float lamb, float beta1, float beta2, float lr,
@@ -58,17 +102,31 @@ __global__ __launch_bounds__(THREADS) void k_grokadamw(Batch<FamRec> B, float al
     const float coef = B.red->coef;
     const bool clip_on = B.red->clip_on != 0;
     const float step_size = lr / R.bc1;
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
-        const int i = start + k;
-        const float g = clipped_grad(R, i, clip_on, coef);
-        float fg = g;
-        if (R.aux) {        // no EMA buffer: plain AdamW
-            const float e = sg_fma(alpha, R.aux[i], (1.0f - alpha) * g);
-            R.aux[i] = e;
-            fg = sg_fma(lamb, e, g);
-        }
-        adam_update(R, i, fg, beta1, beta2, eps, decay, step_size);
-    }
+    for_tile(R, start, cnt,
+        [&](int i) {
+            const float g = clipped_grad(R, i, clip_on, coef);
+            float fg = g;
+            if (R.aux) {        // no EMA buffer: plain AdamW
+                const float e = sg_fma(alpha, R.aux[i], (1.0f - alpha) * g);
+                R.aux[i] = e;
+                fg = sg_fma(lamb, e, g);
+            }
+            adam_update(R, i, fg, beta1, beta2, eps, decay, step_size);
+        },
+        [&](int i) {
+            const f32x4 g = clipped_grad4(R, i, clip_on, coef);
+            f32x4 fg = g;
+            if (R.aux) {
+                f32x4 e = ld4(R.aux, i);
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    e[c] = sg_fma(alpha, e[c], (1.0f - alpha) * g[c]);
+                    fg[c] = sg_fma(lamb, e[c], g[c]);
+                }
+                st4(R.aux, i, e);
+            }
+            adam_update4(R, i, fg, beta1, beta2, eps, decay, step_size);
+        });
 }
 
 __global__ __launch_bounds__(THREADS) void k_neuralgrok(Batch<FamRec> B, const float* __restrict__ W1, const float* __restrict__ b1,
@@ -94,17 +152,35 @@ __global__ __launch_bounds__(THREADS) void k_neuralgrok(Batch<FamRec> B, const f
     }
 }
 
+__device__ __forceinline__ void lion_core(float g, float& m, float& p, float lr, float beta1, float beta2, float wd) {
+    const float interp = sg_fma(beta1, m, (1.0f - beta1) * g);
+    const float s = interp > 0.0f ? 1.0f : (interp < 0.0f ? -1.0f : 0.0f);
+    p = sg_fma(-lr, sg_fma(wd, p, s), p);
+    m = sg_fma(beta2, m, (1.0f - beta2) * g);
+}
 __global__ __launch_bounds__(THREADS) void k_lion(Batch<FamRec> B, float lr, float beta1, float beta2, float wd) {
     int start, cnt;
     const FamRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
-        const int i = start + k;
-        const float g = sg::load_elem(R.grad, R.dtype, i), m = R.ea[i], p = sg::load_elem(R.param, R.dtype, i);
-        const float interp = sg_fma(beta1, m, (1.0f - beta1) * g);
-        const float s = interp > 0.0f ? 1.0f : (interp < 0.0f ? -1.0f : 0.0f);
-        sg::store_elem(R.param, R.dtype, i, sg_fma(-lr, sg_fma(wd, p, s), p));
-        R.ea[i] = sg_fma(beta2, m, (1.0f - beta2) * g);
-    }
+    for_tile(R, start, cnt,
+        [&](int i) {
+            float m = R.ea[i], p = sg::load_elem(R.param, R.dtype, i);
+            lion_core(sg::load_elem(R.grad, R.dtype, i), m, p, lr, beta1, beta2, wd);
+            sg::store_elem(R.param, R.dtype, i, p);
+            R.ea[i] = m;
+        },
+        [&](int i) {
+            const f32x4 g = ld4(R.grad, i);
+            f32x4 m = ld4(R.ea, i), p = ld4(R.param, i);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                float mc = m[c], pc = p[c];
+                lion_core(g[c], mc, pc, lr, beta1, beta2, wd);
+                m[c] = mc;
+                p[c] = pc;
+            }
+            st4(R.param, i, p);
+            st4(R.ea, i, m);
+        });
 }
 
 // ---- reductions: up to three sums per tile, then one block per tensor (or one for the call) -------------
@@ -143,11 +219,19 @@ __global__ __launch_bounds__(THREADS) void k_prodigy_partial(Batch<FamRec> B) {
     const FamRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
     const float* p0 = static_cast<const float*>(R.aux2);
     float num = 0.0f, den = 0.0f;
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
-        const int i = start + k;
-        num = sg_fma(sg::load_elem(R.grad, R.dtype, i), sg::load_elem(R.param, R.dtype, i) - p0[i], num);
-        den += R.aux[i];
-    }
+    for_tile(R, start, cnt,
+        [&](int i) {
+            num = sg_fma(sg::load_elem(R.grad, R.dtype, i), sg::load_elem(R.param, R.dtype, i) - p0[i], num);
+            den += R.aux[i];
+        },
+        [&](int i) {
+            const f32x4 g = ld4(R.grad, i), p = ld4(R.param, i), q = ld4(p0, i), sv = ld4(R.aux, i);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                num = sg_fma(g[c], p[c] - q[c], num);
+                den += sv[c];
+            }
+        });
     tile_sums(B, (double)num, (double)den, 0.0);
 }
 
@@ -163,12 +247,22 @@ __global__ __launch_bounds__(THREADS) void k_prodigy(Batch<FamRec> B, float beta
     const FamRec& R = tile_rec(B, blockIdx.x, &start, &cnt);
     const float d_lr = B.tred[0].d_lr;
     const float decay = 1.0f - (lr * d_lr) * wd, step_size = lr / R.bc1, eps_eff = d_lr * eps;
-    for (int k = threadIdx.x; k < cnt; k += THREADS) {
-        const int i = start + k;
-        const float dg = d_lr * sg::load_elem(R.grad, R.dtype, i);
-        R.aux[i] = sg_fma(beta2, R.aux[i], ((1.0f - beta2) * dg) * dg);
-        adam_update(R, i, dg, beta1, beta2, eps_eff, decay, step_size);
-    }
+    for_tile(R, start, cnt,
+        [&](int i) {
+            const float dg = d_lr * sg::load_elem(R.grad, R.dtype, i);
+            R.aux[i] = sg_fma(beta2, R.aux[i], ((1.0f - beta2) * dg) * dg);
+            adam_update(R, i, dg, beta1, beta2, eps_eff, decay, step_size);
+        },
+        [&](int i) {
+            f32x4 dg = ld4(R.grad, i), sv = ld4(R.aux, i);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                dg[c] = d_lr * dg[c];
+                sv[c] = sg_fma(beta2, sv[c], ((1.0f - beta2) * dg[c]) * dg[c]);
+            }
+            st4(R.aux, i, sv);
+            adam_update4(R, i, dg, beta1, beta2, eps_eff, decay, step_size);
+        });
 }
 
 // ---- SuperGrok v1.1 -------------------------------------------------------------------------------------
@@ -324,7 +418,10 @@ int collect(int n, const SgFamilyTensor* ts, int need, std::vector<FamRec>* recs
             ((need & N_EASQ) && !t.exp_avg_sq) || ((need & N_AUX) && !t.aux) || ((need & N_AUX2) && !t.aux2))
             return sg::fail("tensor %d: NULL pointer", i);
         if (check_dtype(i, t.dtype)) return 1;
-        recs->push_back({t.param, t.grad, t.exp_avg, t.exp_avg_sq, t.aux, t.aux2, nullptr, t.numel, t.dtype, t.bc1, t.bc2, t.alpha, t.beta1});
+        const uintptr_t all = (uintptr_t)t.param | (uintptr_t)t.grad | (uintptr_t)t.exp_avg | (uintptr_t)t.exp_avg_sq | (uintptr_t)t.aux |
+                              (uintptr_t)t.aux2;
+        recs->push_back({t.param, t.grad, t.exp_avg, t.exp_avg_sq, t.aux, t.aux2, nullptr, t.numel, t.dtype, t.bc1, t.bc2, t.alpha, t.beta1,
+                         (t.dtype == SG_F32 && (all & 15u) == 0) ? 1 : 0});
     }
     return 0;
 }
