@@ -28,7 +28,7 @@ FLOP_PER_ELEMENT = 30e3         # arithmetic actually required per element (both
 VALU_PEAK_TFLOPS = 157.3
 
 
-def build_workload(name, device):
+def build_workload(name, device, nonzero_sharpness=False):
     import torch
     import workloads as wl
     from helpers import DIMS
@@ -46,7 +46,11 @@ def build_workload(name, device):
     for seed in (1, 2):
         g = wl.clip_per_tensor(wl.make_grads(shapes, seed=seed, tail_frac=0.005, tail="student3"))
         grad_sets.append([t.reshape(-1).to(device) for t in g])
+    # sharpness is 0 until a SAM probe has run (the optimizer's initial state and the configuration the metric is quoted on);
+    # --sharpness measures the step with a populated sharpness cache instead (one more random gather per element)
     sharps = [torch.zeros_like(p) for p in params]
+    if nonzero_sharpness:
+        sharps = [(g.abs() * 0.5).contiguous() for g in grad_sets[1]]
     weights = [w.to(device) for w in wl.meta_weights(7)]
     return shapes, state, grad_sets, sharps, weights
 
@@ -199,6 +203,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--sharpness", action="store_true", help="v2 workloads: non-zero sharpness cache (as after a SAM probe)")
     ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
@@ -224,7 +229,7 @@ def main():
         return
     if _cabi.lib().sg2_set_chunk_len(args.chunk_len) or _cabi.lib().sg2_set_scan_window(args.window):
         raise SystemExit(_cabi.last_error())
-    shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev)
+    shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev, args.sharpness)
     total = sum(p.numel() for p in st["params"])
     step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
                          st["counts"])

@@ -52,7 +52,8 @@ struct TensorDev {
     int dtype;
     int nchunks;    // scan chunks of this tensor
     float alpha, lamb, beta1, bc2, step_size;
-    int pad_[5];
+    int sharp_nonzero;   // uploaded as 0; set by k_keys when any (finite) sharpness entry of the tensor is not 0
+    int pad_[4];
 };
 static_assert(sizeof(TensorDev) == 128, "TensorDev layout");
 

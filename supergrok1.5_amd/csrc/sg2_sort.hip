@@ -33,6 +33,7 @@ __global__ __launch_bounds__(256) void k_keys(Plan pl) {
     const TensorDev& T = pl.tensors[ti];
     const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
     const int cnt = min(ELEM_TILE, T.numel - start);
+    bool nz = false;
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int i = start + k;
         const float g = sg::finite_or_zero(sg::load_elem(T.grad, T.dtype, i));
@@ -40,7 +41,11 @@ __global__ __launch_bounds__(256) void k_keys(Plan pl) {
         // pair gives back g exactly and the scan never has to gather gradients from element order
         pl.keys[0][T.off + i] = (uint32_t)sg_f2i(sg_abs(g));
         pl.vals[0][T.off + i] = i | (sg_f2i(g) & (int32_t)0x80000000);
+        nz = nz || (sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, i)) != 0.0f);
     }
+    // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
+    // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
+    if (__syncthreads_or(nz) && threadIdx.x == 0) atomicOr(const_cast<int*>(&T.sharp_nonzero), 1);
 }
 
 struct TileRef {
@@ -251,11 +256,16 @@ __global__ __launch_bounds__(256) void k_gather_sorted(Plan pl, int32_t* __restr
     const TensorDev& T = pl.tensors[ti];
     const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
     const int cnt = min(ELEM_TILE, T.numel - start);
+    const bool gather = T.sharp_nonzero != 0;      // all-zero sharpness: nothing to gather, the sorted copy is 0 as well
+    if (!gather && !dbg_perm) {
+        for (int k = threadIdx.x; k < cnt; k += 256) pl.ssorted[T.off + start + k] = 0.0f;
+        return;
+    }
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int t = T.off + start + k;
         int idx = pl.vals[0][t] & 0x7fffffff;
         idx = ((unsigned)idx < (unsigned)T.numel) ? idx : 0;       // never index outside the tensor
-        pl.ssorted[t] = sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, idx));
+        pl.ssorted[t] = gather ? sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, idx)) : 0.0f;
         if (dbg_perm) dbg_perm[t] = idx;
     }
 }

@@ -211,7 +211,8 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
         d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
         d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
         d.step_size = scalars->lr / t.bc1;
-        for (int k = 0; k < 5; k++) d.pad_[k] = 0;
+        d.sharp_nonzero = 0;
+        for (int k = 0; k < 4; k++) d.pad_[k] = 0;
         off += n;
         p_et[i + 1] = p_et[i] + (n + ELEM_TILE - 1) / ELEM_TILE;
         p_st[i + 1] = p_st[i] + (n + SORT_TILE - 1) / SORT_TILE;
