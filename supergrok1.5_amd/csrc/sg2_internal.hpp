@@ -52,8 +52,7 @@ struct TensorDev {
     int dtype;
     int nchunks;    // scan chunks of this tensor
     float alpha, lamb, beta1, bc2, step_size;
-    int sharp_nonzero;   // uploaded as 0; set by k_keys when any (finite) sharpness entry of the tensor is not 0
-    int pad_[4];
+    int pad_[5];
 };
 static_assert(sizeof(TensorDev) == 128, "TensorDev layout");
 
@@ -77,6 +76,7 @@ struct Plan {
     float* summaries;              // [2][wchunks][6][128]
     float* hstart;                 // [2][chunks][2][128]
     float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
+    int* sharp_nonzero;            // [P] uploaded as 0; set by k_keys when some (finite) sharpness entry of the tensor is not 0
     float* ctx;                    // [2][total][DM]
     float decay, beta2, eps, rescale;
     Sg2Weights W;

@@ -45,7 +45,11 @@ __global__ __launch_bounds__(256) void k_keys(Plan pl) {
     }
     // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
     // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
-    if (__syncthreads_or(nz) && threadIdx.x == 0) atomicOr(const_cast<int*>(&T.sharp_nonzero), 1);
+    // (plain store, and only while the flag still reads 0: every writer stores the same value)
+    if (__syncthreads_or(nz) && threadIdx.x == 0) {
+        volatile int* flag = pl.sharp_nonzero + ti;
+        if (*flag == 0) *flag = 1;
+    }
 }
 
 struct TileRef {
@@ -256,7 +260,7 @@ __global__ __launch_bounds__(256) void k_gather_sorted(Plan pl, int32_t* __restr
     const TensorDev& T = pl.tensors[ti];
     const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
     const int cnt = min(ELEM_TILE, T.numel - start);
-    const bool gather = T.sharp_nonzero != 0;      // all-zero sharpness: nothing to gather, the sorted copy is 0 as well
+    const bool gather = pl.sharp_nonzero[ti] != 0;      // all-zero sharpness: nothing to gather, the sorted copy is 0 as well
     if (!gather && !dbg_perm) {
         for (int k = threadIdx.x; k < cnt; k += 256) pl.ssorted[T.off + start + k] = 0.0f;
         return;

@@ -38,7 +38,7 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_ctx, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, bytes;
     size_t tables_bytes;
 };
 
@@ -71,6 +71,7 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * SCAN_THREADS);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * SCAN_THREADS);
     L->off_comp = take(4 * 2 * 5 * 16 * 3);
+    L->off_flags = take(4 * (size_t)P);        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * DM);
     L->bytes = o;
     return 0;
@@ -211,8 +212,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
         d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
         d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
         d.step_size = scalars->lr / t.bc1;
-        d.sharp_nonzero = 0;
-        for (int k = 0; k < 4; k++) d.pad_[k] = 0;
+        for (int k = 0; k < 5; k++) d.pad_[k] = 0;
         off += n;
         p_et[i + 1] = p_et[i] + (n + ELEM_TILE - 1) / ELEM_TILE;
         p_st[i + 1] = p_st[i] + (n + SORT_TILE - 1) / SORT_TILE;
@@ -221,6 +221,10 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     }
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_tables, blob.data(), L.tables_bytes, hipMemcpyHostToDevice, st));
+    {
+        const std::vector<int> zeros((size_t)P, 0);
+        SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_flags, zeros.data(), sizeof(int) * (size_t)P, hipMemcpyHostToDevice, st));
+    }
 
     Plan pl;
     pl.tensors = reinterpret_cast<const TensorDev*>(ws + L.off_tables);
@@ -241,6 +245,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.summaries = reinterpret_cast<float*>(ws + L.off_summ);
     pl.hstart = reinterpret_cast<float*>(ws + L.off_hstart);
     pl.comp = reinterpret_cast<float*>(ws + L.off_comp);
+    pl.sharp_nonzero = reinterpret_cast<int*>(ws + L.off_flags);
     pl.ctx = reinterpret_cast<float*>(ws + L.off_ctx);
     pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
