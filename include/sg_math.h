@@ -197,13 +197,14 @@ SG_HD float sg_abar_block_prefix(int n, const float* dt, float nhA_e, float nhA_
     return acc;
 }
 SG_HD void sg_abar_block_finish(int n, const float* d_e, const float* d_o, const float* P, float* ab_e, float* ab_o) {
+    /* the factor 2 of A_bar = 2/(1+t) - 1 rides on the running reciprocal (doubling is exact) */
     float r = sg_rcp_pos(P[n - 1]);
+    r = r + r;
     for (int k = n - 1; k >= 0; k--) {
-        const float inv = (k > 0) ? r * P[k - 1] : r;      /* 1/D_k */
+        const float inv2 = (k > 0) ? r * P[k - 1] : r;      /* 2/D_k */
         if (k > 0) r = r * (d_e[k] * d_o[k]);
-        const float r2 = inv + inv;
-        ab_e[k] = sg_fma(d_o[k], r2, -1.0f);
-        ab_o[k] = sg_fma(d_e[k], r2, -1.0f);
+        ab_e[k] = sg_fma(d_o[k], inv2, -1.0f);
+        ab_o[k] = sg_fma(d_e[k], inv2, -1.0f);
     }
 }
 

@@ -106,12 +106,13 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
 // Returns whether every rotation angle of this timestep, over this half's columns, is small enough
 // for sg_sincos_small (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
-template <bool OUT, int HALF>
-__device__ __forceinline__ bool project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt, float* s_ux,
-                                             float* s_dx, float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
+template <bool OUT, int HALF, bool HAS_S>
+__device__ __forceinline__ bool project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt,
+                                             float* s_ux, float* s_dx, float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
+    // HAS_S is false for a tensor whose sharpness is all zero: fma(c_s, 0, c_0) is c_0 itself, so the term is skipped
     auto eval = [&](int group, int row) {
         const sg::cfloat_p t = c + (group * 16 + row) * 3;
-        return sg_fma(t[0], g, sg_fma(t[1], s, t[2]));
+        return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]);
     };
     bool small = true;
 #pragma unroll
@@ -225,6 +226,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const uint32_t* __restrict__ skey = pl.keys[0] + off;      // sorted |g| bits
     const int32_t* __restrict__ sval = pl.vals[0] + off;       // element index | sign of g
     const float* __restrict__ ssrt = pl.ssorted + off;          // sharpness in sorted order
+    const bool has_s = __builtin_amdgcn_readfirstlane(pl.sharp_nonzero[ti]) != 0;
     const sg::cfloat_p comp0 = sg::as_const(pl.comp) + dir * (SG2_COMP_GROUPS * 16 * 3);
 
     const int tid = threadIdx.x;
@@ -281,10 +283,17 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             sh = ssrt[t];
         }
         bool small_t;
-        if (half == 0)
-            small_t = project_tile<OUT, 0>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-        else
-            small_t = project_tile<OUT, 1>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+        if (has_s) {
+            if (half == 0)
+                small_t = project_tile<OUT, 0, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+            else
+                small_t = project_tile<OUT, 1, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+        } else {
+            if (half == 0)
+                small_t = project_tile<OUT, 0, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+            else
+                small_t = project_tile<OUT, 1, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+        }
         {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!small_t);
             if (tu == 0) s_large[half] = large;
