@@ -160,6 +160,18 @@ SG_HD float sg_rcp_pos(float d) {
     return r;
 }
 
+/* sin and cos for |theta| < 0.3 with one polynomial term less each (least-squares fit on that
+ * interval; ~1 ulp).  NOT bit-identical to sg_sincos: both sides of a parity comparison must take
+ * this form for the same timesteps. */
+#define SG_SINCOS_TINY_LIMIT 0.3f
+SG_HD void sg_sincos_tiny(float th, float* s_out, float* c_out) {
+    const float z = th * th;
+    const float sp = sg_fma(0.0083154970780015f, z, -0.16666646301746368f);
+    *s_out = sg_fma(sp * z, th, th);
+    const float cp = sg_fma(-0.0013806807110086083f, z, 0.041666239500045776f);
+    *c_out = sg_fma(cp * z, z, sg_fma(z, -0.5f, 1.0f));
+}
+
 /* Trapezoidal discretisation for the two states of one RoPE pair:
  *   A_bar = (1 + dt*A/2) / (1 - dt*A/2 + 1e-8)
  * With t = -dt*A/2 >= 0 (A < 0, dt >= 0) this is (1-t)/(1+t) = 2/(1+t) - 1.

@@ -32,7 +32,7 @@ def lib():
         if not os.path.exists(_LIB):
             build()
         _lib = C.CDLL(_LIB)
-        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf", "sin_small", "cos_small",
+        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf", "sin_small", "cos_small", "sin_tiny", "cos_tiny",
                   "gelu_sigmoid"):
             f = getattr(_lib, "orc_" + n)
             f.restype = C.c_float

@@ -281,6 +281,29 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
                 O::sincos(tc.sp[k].dt[j] * (R)w.rope[j * hp + p], &tc.sn[(size_t)k * lanes + j * hp + p],
                           &tc.cs[(size_t)k * lanes + j * hp + p]);
     }
+    if (sizeof(R) == 4) {
+        /* blocks whose angles are all below SG_SINCOS_TINY_LIMIT, over the 8 steps and the columns of a wave, take
+         * sg_sincos_tiny (the device decides with dt * max_p |rope[j,p]| per column) */
+        std::vector<float> fmax(di, 0.0f);
+        for (int j = 0; j < di; j++)
+            for (int p = 0; p < hp; p++) fmax[j] = sg_max(fmax[j], sg_abs(w.rope[j * hp + p]));
+        for (int b0 = 0; b0 + ORC_BLOCK <= cnt; b0 += ORC_BLOCK)
+            for (int wave0 = 0; wave0 < lanes; wave0 += ORC_WAVE) {
+                const int wave1 = std::min(lanes, wave0 + ORC_WAVE);
+                bool tiny = true;
+                for (int q = 0; q < ORC_BLOCK && tiny; q++)
+                    for (int j = wave0 / hp; j <= (wave1 - 1) / hp; j++)
+                        if (!((float)tc.sp[b0 + q].dt[j] * fmax[j] < SG_SINCOS_TINY_LIMIT)) { tiny = false; break; }
+                if (!tiny) continue;
+                for (int q = 0; q < ORC_BLOCK; q++)
+                    for (int l = wave0; l < wave1; l++) {
+                        float sn, cs;
+                        sg_sincos_tiny((float)tc.sp[b0 + q].dt[l / hp] * w.rope[l], &sn, &cs);
+                        tc.sn[(size_t)(b0 + q) * lanes + l] = (R)sn;
+                        tc.cs[(size_t)(b0 + q) * lanes + l] = (R)cs;
+                    }
+            }
+    }
     int k0 = 0;
     if (sizeof(R) == 4) {
         std::vector<float> de((size_t)lanes * ORC_BLOCK), dod((size_t)lanes * ORC_BLOCK), P((size_t)lanes * ORC_BLOCK);
@@ -639,6 +662,8 @@ int orc_sg2_step(int precision, int64_t chunk_len, int64_t window, const float* 
 float orc_exp(float x) { return sg_exp(x); }
 float orc_log(float x) { return sg_log(x); }
 float orc_softplus(float x) { return sg_softplus(x); }
+float orc_sin_tiny(float x) { float s, c; sg_sincos_tiny(x, &s, &c); return s; }
+float orc_cos_tiny(float x) { float s, c; sg_sincos_tiny(x, &s, &c); return c; }
 float orc_sigmoid(float x) { return sg_sigmoid(x); }
 float orc_silu(float x) { return sg_silu(x); }
 float orc_tanh(float x) { return sg_tanh(x); }

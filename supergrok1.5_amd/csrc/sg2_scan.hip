@@ -53,11 +53,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #endif
 constexpr int UB = SG2_SCAN_UB;           // timesteps per unrolled block of the recurrence
 static_assert(UB % 4 == 0 && SCAN_TT % UB == 0 && SCAN_TT == 64, "blocks are fetched 4 timesteps per LDS read; one ballot covers a tile");
-#ifdef SG2_SCAN_WAVES
-#define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
-#else
-#define SG2_SCAN_ATTR
+// Three waves per SIMD (168 VGPRs) is where the kernels stop gaining from occupancy; keep the
+// register allocation from drifting just past that boundary.
+#ifndef SG2_SCAN_WAVES
+#define SG2_SCAN_WAVES 3
 #endif
+#define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
 
 struct DirW {
     sg::cfloat_p in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj;
@@ -103,23 +104,25 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
 // Projections of one timestep from the element's (g, s).  Each half of the workgroup produces its
 // half of dt / dt*x-branch / B (/ D*x-branch / C / gate).  HALF is a template parameter so that every coefficient
 // index is a compile-time constant (scalar loads).  c points at this direction's coefficients.
-// Returns whether every rotation angle of this timestep, over this half's columns, is small enough
-// for sg_sincos_small (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
+// Returns bit 0: every rotation angle of this timestep, over this half's columns, is small enough for
+// sg_sincos_small; bit 1: small enough for sg_sincos_tiny (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
 template <bool OUT, int HALF, bool HAS_S>
-__device__ __forceinline__ bool project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt,
+__device__ __forceinline__ int project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt,
                                              float* s_ux, float* s_dx, float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
     // HAS_S is false for a tensor whose sharpness is all zero: fma(c_s, 0, c_0) is c_0 itself, so the term is skipped
     auto eval = [&](int group, int row) {
         const sg::cfloat_p t = c + (group * 16 + row) * 3;
         return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]);
     };
-    bool small = true;
+    bool small = true, tiny = true;
 #pragma unroll
     for (int q = 0; q < DI / 2; q++) {
         const int jj = HALF * (DI / 2) + q;
         const float dtv = sg_softplus(eval(SG2_COMP_DT, jj));
-        small = small && (dtv * s_fmax[jj] < SG_SINCOS_SMALL_LIMIT);
+        const float amax = dtv * s_fmax[jj];
+        small = small && (amax < SG_SINCOS_SMALL_LIMIT);
+        tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
         const float xbv = eval(SG2_COMP_XB, jj);
         s_dt[jj * LDS_STRIDE + tu] = dtv;
         s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
@@ -138,7 +141,7 @@ __device__ __forceinline__ bool project_tile(sg::cfloat_p c, sg::cfloat_p Dw, fl
             s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(SG2_COMP_Z, jj));
         }
     }
-    return small;
+    return (small ? 1 : 0) | (tiny ? 2 : 0);
 }
 
 // scan state of one lane: OUT -> (he,ho) only; summary -> also the two columns of M
@@ -166,7 +169,8 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // UB consecutive timesteps (all valid): coefficients first, then the serial chain.  ux = dt * x-branch
 // (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
-template <bool OUT, bool SMALL_ANGLE>
+// ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny (its own values).
+template <bool OUT, int ANGLE>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, float (&y)[UB]) {
@@ -183,7 +187,8 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
-        if (SMALL_ANGLE) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
+        if (ANGLE == 2) sg_sincos_tiny(dt[u] * freq, &sn[u], &cs[u]);
+        else if (ANGLE == 1) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
         else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
         be[u] = ux[u] * Be[u];
         bo[u] = ux[u] * Bo[u];
@@ -211,6 +216,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     float* const s_y = s_dt;
     __shared__ float s_fmax[DI];
     __shared__ unsigned long long s_large[2];      // per projection half: bit t set = timestep t of the tile needs the full sin/cos
+    __shared__ unsigned long long s_nottiny[2];    // ... bit t set = timestep t is not eligible for sg_sincos_tiny
 
     const int per_dir = OUT ? pl.chunks : pl.wchunks;
     const int dir = (int)blockIdx.x >= per_dir ? 1 : 0;
@@ -282,24 +288,25 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
             sh = ssrt[t];
         }
-        bool small_t;
+        int angle_t;
         if (has_s) {
             if (half == 0)
-                small_t = project_tile<OUT, 0, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 0, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
             else
-                small_t = project_tile<OUT, 1, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 1, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         } else {
             if (half == 0)
-                small_t = project_tile<OUT, 0, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 0, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
             else
-                small_t = project_tile<OUT, 1, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 1, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         }
         {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
-            const unsigned long long large = __builtin_amdgcn_ballot_w64(!small_t);
-            if (tu == 0) s_large[half] = large;
+            const unsigned long long large = __builtin_amdgcn_ballot_w64(!(angle_t & 1));
+            const unsigned long long nottiny = __builtin_amdgcn_ballot_w64(!(angle_t & 2));
+            if (tu == 0) { s_large[half] = large; s_nottiny[half] = nottiny; }
         }
         __syncthreads();
-        const unsigned long long large = s_large[half];
+        const unsigned long long large = s_large[half], nottiny = s_nottiny[half];
 
         // ---------------- phase B: the recurrence over the tile, lane = (j,p)
         const float* __restrict__ r_dt = s_dt + j * LDS_STRIDE;
@@ -323,10 +330,13 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                     for (int e = 0; e < 4; e++) { Ce[q + e] = f[e]; Co[q + e] = g[e]; }
                 }
             }
-            if (((large >> k0) & ((1ull << UB) - 1)) == 0)
-                block_steps<OUT, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+            const unsigned long long blk = ((1ull << UB) - 1) << k0;
+            if ((nottiny & blk) == 0)
+                block_steps<OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+            else if ((large & blk) == 0)
+                block_steps<OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             else
-                block_steps<OUT, false>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             if (OUT && p == 0) {
 #pragma unroll
                 for (int q = 0; q < UB; q += 4)

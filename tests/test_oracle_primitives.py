@@ -81,6 +81,22 @@ def test_small_angle_sincos_is_bitwise_the_general_one():
         assert np.float32(L.orc_cos_small(x)).tobytes() == np.float32(L.orc_cos(x)).tobytes(), x
 
 
+def test_tiny_angle_sincos_against_libm():
+    """|theta| < 0.3 with one polynomial term less: ~1 ulp of sin (relative) and of cos (absolute), pure rotation
+    (s^2 + c^2 = 1 to rounding), odd/even symmetry."""
+    xs = np.concatenate([RNG.uniform(-0.3, 0.3, 50000), RNG.uniform(-1e-3, 1e-3, 5000), [0.0, 0.2999999, -0.2999999, 1e-30]])
+    ws = wc = wn = 0.0
+    for x in xs.astype(np.float32):
+        x = float(x)
+        s, c = L.orc_sin_tiny(x), L.orc_cos_tiny(x)
+        ws = max(ws, abs(s - math.sin(x)) / max(abs(x), 1e-30))
+        wc = max(wc, abs(c - math.cos(x)))
+        wn = max(wn, abs(s * s + c * c - 1.0))
+        assert L.orc_sin_tiny(-x) == -s and L.orc_cos_tiny(-x) == c
+    assert ws < 1.5e-7 and wc < 1.3e-7 and wn < 3e-7, (ws, wc, wn)
+    assert L.orc_sin_tiny(0.0) == 0.0 and L.orc_cos_tiny(0.0) == 1.0
+
+
 def test_rcp_and_abar():
     ds = np.exp(RNG.uniform(0, 60, 20000))
     assert _maxrel(L.orc_rcp_pos, lambda d: 1.0 / d, ds) < 1.5e-7
