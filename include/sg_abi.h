@@ -222,6 +222,37 @@ typedef struct Sg15RestoreTensor {
 int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, void* workspace,
                            size_t workspace_bytes, void* stream);
 
+/* ---- bilevel meta-net training: the scan, forward and backward ------------
+ *
+ * The reference trains the meta-net by differentiating smart_grad with respect
+ * to its weights (grokking_optimizers/supergrok2.py:516-1330 over
+ * supergrok2_bilevel_fwd_save / supergrok2_bilevel_backward, csrc/ops.h:232-371).
+ * Here the sequential part - sort and bidirectional scan - runs forward and
+ * backward in HIP; the per-element part (GRU, soft top-4 PEER routing, experts)
+ * is a handful of dense torch ops on the caller's side.
+ *
+ * sg2_bilevel_forward: sort + scan exactly as in sg2_batched_step, writing the
+ * two contexts of every element to ctx_out ([2][sum numel][d_model] floats,
+ * element order, tensors packed in call order) and keeping what the backward
+ * pass needs in the workspace.  Of Sg2Tensor only grad, sharpness,
+ * mamba_fwd_state, mamba_bwd_state, numel and dtype are read; the two states
+ * are OVERWRITTEN with the end-of-sequence states, so pass copies.
+ *
+ * sg2_bilevel_backward: same tensors and the SAME, untouched workspace; d_ctx
+ * has ctx_out's layout.  grads_out receives, per direction (forward first,
+ * SG2_BWD_STRIDE floats each):
+ *   [5][16][3]  composed projection coefficients (include/sg2_compose.h order)
+ *   [16][16]    A_log      [16][8] rope_freq      [16] D      [8][16] out_proj
+ * The caller maps the coefficient gradients back through the composition.
+ * A tensor is walked serially by one workgroup per direction (exact adjoint,
+ * no truncation). */
+#define SG2_BWD_STRIDE 768
+size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
+int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                        float* ctx_out, void* workspace, size_t workspace_bytes, void* stream);
+int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                         const float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ================== the other fused steps of the reference ================== */
 
 /* One tensor of an Adam-family fused step: the i-th entries of the tensor

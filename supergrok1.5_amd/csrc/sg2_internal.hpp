@@ -76,6 +76,7 @@ struct Plan {
     float* summaries;              // [2][wchunks][6][128]
     float* hstart;                 // [2][chunks][2][128]
     float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
+    float* htile;                  // bilevel: [2][tiles][2][128] state at the start of every 64-step tile, or NULL
     int* sharp_nonzero;            // [P] uploaded as 0; set by k_keys when some (finite) sharpness entry of the tensor is not 0
     float* ctx;                    // [2][total][DM]
     float decay, beta2, eps, rescale;
@@ -87,6 +88,10 @@ void prof_mark(int idx, hipStream_t st);
 
 int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st);
 int launch_scan(const Plan& pl, hipStream_t st);
+// tile index of scan step u of tensor ti (element offset off) in the per-tile state array of the bilevel path
+__host__ __device__ inline int htile_index(int off, int ti, int u) { return off / SCAN_TT + ti + u / SCAN_TT; }
+__host__ __device__ inline int htile_count(int total, int P) { return total / SCAN_TT + P + 1; }
+int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
 
 }  // namespace sg2

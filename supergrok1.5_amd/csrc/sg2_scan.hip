@@ -308,6 +308,11 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         __syncthreads();
         const unsigned long long large = s_large[half], nottiny = s_nottiny[half];
 
+        if (OUT && pl.htile != nullptr) {      // bilevel: keep the state entering this tile for the backward pass
+            float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, tile0)) * 2 * SCAN_THREADS;
+            ht[tid] = S.he;
+            ht[SCAN_THREADS + tid] = S.ho;
+        }
         // ---------------- phase B: the recurrence over the tile, lane = (j,p)
         const float* __restrict__ r_dt = s_dt + j * LDS_STRIDE;
         const float* __restrict__ r_ux = s_ux + j * LDS_STRIDE;

@@ -38,11 +38,11 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, off_htile, bytes;
     size_t tables_bytes;
 };
 
-int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
+int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bilevel = false) {
     int64_t total = 0, et = 0, stl = 0, ch = 0, wch = 0;
     for (int i = 0; i < P; i++) {
         const int64_t n = numels[i];
@@ -73,6 +73,8 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L) {
     L->off_comp = take(4 * 2 * 5 * 16 * 3);
     L->off_flags = take(4 * (size_t)P);        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * DM);
+    // bilevel only: state at the start of every 64-step tile, both directions (tile index = off/64 + tensor index + u/64)
+    L->off_htile = take(bilevel ? 4 * 2 * ((size_t)total / SCAN_TT + (size_t)P + 1) * 2 * SCAN_THREADS : 0);
     L->bytes = o;
     return 0;
 }
@@ -162,16 +164,22 @@ size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* n
     return L.bytes;
 }
 
-int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
-                     const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
-                     const Sg2Debug* debug, void* stream) {
-    using namespace sg2;
+}  // extern "C"
+
+namespace sg2 {
+// Validates the call, lays out the workspace, uploads the per-tensor records and fills the Plan.  full_step:
+// the optimizer-state pointers of every tensor are required; otherwise only grad, sharpness and the two Mamba
+// states (bilevel forward/backward).  Returns 0 with pl->total == 0 when there is nothing to do.
+int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const Sg2Scalars* scalars,
+               void* workspace, size_t workspace_bytes, bool full_step, bool bilevel, bool keep_flags, hipStream_t st, Plan* plp, Layout* Lp) {
+    Plan& pl = *plp;
+    Layout& L = *Lp;
+    pl.total = 0;
     if (check_dims(dims)) return 1;
     if (num_tensors == 0) return 0;
     if (num_tensors < 0 || !tensors || !weights || !scalars) return sg::fail("NULL argument");
     for (int k = 0; k < SG2_NUM_WEIGHTS; k++)
         if (!weights->w[k]) return sg::fail("weight pointer %d is NULL", k);
-    hipStream_t st = (hipStream_t)stream;
     const int P = num_tensors;
 
     std::vector<int64_t> numels(P);
@@ -179,21 +187,18 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
         const Sg2Tensor& t = tensors[i];
         numels[i] = t.numel;
         if (t.numel > 0) {
-            if (!t.param || !t.grad || !t.sharpness || !t.exp_avg || !t.exp_avg_sq || !t.mu || !t.gru_state ||
-                !t.mamba_fwd_state || !t.mamba_bwd_state)
-                return sg::fail("tensor %d: NULL pointer", i);
+            if (!t.grad || !t.sharpness || !t.mamba_fwd_state || !t.mamba_bwd_state) return sg::fail("tensor %d: NULL pointer", i);
+            if (full_step && (!t.param || !t.exp_avg || !t.exp_avg_sq || !t.mu || !t.gru_state)) return sg::fail("tensor %d: NULL pointer", i);
             if (t.dtype != SG_F32 && t.dtype != SG_F16 && t.dtype != SG_BF16) return sg::fail("tensor %d: bad dtype %d", i, t.dtype);
-            if (((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
+            if (full_step && ((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
         }
     }
     const int chunk_len = effective_chunk_len(P, numels.data());
-    Layout L;
-    if (make_layout(P, numels.data(), chunk_len, &L)) return 1;
+    if (make_layout(P, numels.data(), chunk_len, &L, bilevel)) return 1;
     if (L.total == 0) return 0;
     if (!workspace || workspace_bytes < L.bytes)
         return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
     if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
-
     // ---- host tables -> one blob -> device
     std::vector<unsigned char> blob(L.tables_bytes);
     TensorDev* td = reinterpret_cast<TensorDev*>(blob.data());
@@ -211,7 +216,7 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
         d.mfwd = t.mamba_fwd_state; d.mbwd = t.mamba_bwd_state;
         d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
         d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
-        d.step_size = scalars->lr / t.bc1;
+        d.step_size = full_step ? scalars->lr / t.bc1 : 0.0f;
         for (int k = 0; k < 5; k++) d.pad_[k] = 0;
         off += n;
         p_et[i + 1] = p_et[i] + (n + ELEM_TILE - 1) / ELEM_TILE;
@@ -221,12 +226,11 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     }
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_tables, blob.data(), L.tables_bytes, hipMemcpyHostToDevice, st));
-    {
+    if (!keep_flags) {
         const std::vector<int> zeros((size_t)P, 0);
         SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_flags, zeros.data(), sizeof(int) * (size_t)P, hipMemcpyHostToDevice, st));
     }
 
-    Plan pl;
     pl.tensors = reinterpret_cast<const TensorDev*>(ws + L.off_tables);
     const int* dpre = reinterpret_cast<const int*>(ws + L.off_tables + sizeof(TensorDev) * (size_t)P);
     pl.elem_tile_prefix = dpre;
@@ -251,6 +255,22 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
     pl.W = *weights;
 
+    pl.htile = bilevel ? reinterpret_cast<float*>(ws + L.off_htile) : nullptr;
+    return 0;
+}
+}  // namespace sg2
+
+extern "C" {
+
+int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                     const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
+                     const Sg2Debug* debug, void* stream) {
+    using namespace sg2;
+    hipStream_t st = (hipStream_t)stream;
+    Plan pl;
+    Layout L;
+    if (build_plan(dims, weights, num_tensors, tensors, scalars, workspace, workspace_bytes, true, false, false, st, &pl, &L)) return 1;
+    if (pl.total == 0) return 0;
     prof_mark(0, st);
     if (launch_sort(pl, debug ? debug->perm : nullptr, st)) return 1;
     prof_mark(1, st);
@@ -261,6 +281,43 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     prof_mark(5, st);
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;
     return 0;
+}
+
+size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
+    if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
+    sg2::Layout L;
+    if (sg2::make_layout(num_tensors, numels, sg2::effective_chunk_len(num_tensors, numels), &L, true)) return 0;
+    return L.bytes;
+}
+
+int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, float* ctx_out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace sg2;
+    hipStream_t st = (hipStream_t)stream;
+    Plan pl;
+    Layout L;
+    const Sg2Scalars none = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, false, st, &pl, &L)) return 1;
+    if (pl.total == 0) return 0;
+    if (!ctx_out) return sg::fail("ctx_out is NULL");
+    pl.ctx = ctx_out;
+    if (launch_sort(pl, nullptr, st)) return 1;
+    return launch_scan(pl, st);
+}
+
+int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const float* d_ctx,
+                         float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace sg2;
+    hipStream_t st = (hipStream_t)stream;
+    Plan pl;
+    Layout L;
+    const Sg2Scalars none = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (!grads_out) return sg::fail("grads_out is NULL");
+    // same layout as the forward call: sorted keys / payloads / sharpness, the sharpness flags, coefficients and tile
+    // states are still in place
+    if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, true, st, &pl, &L)) return 1;
+    if (pl.total > 0 && !d_ctx) return sg::fail("d_ctx is NULL");
+    return launch_bilevel_backward(pl, d_ctx, grads_out, st);
 }
 
 }  // extern "C"

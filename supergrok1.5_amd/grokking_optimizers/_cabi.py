@@ -69,6 +69,14 @@ def lib():
         L.sg2_batched_step.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
                                        C.POINTER(Sg2Scalars), C.c_void_p, C.c_void_p, C.c_size_t,
                                        C.POINTER(Sg2Debug), C.c_void_p]
+        L.sg2_bilevel_workspace_bytes.restype = C.c_size_t
+        L.sg2_bilevel_workspace_bytes.argtypes = [C.POINTER(SgDims), C.c_int, C.POINTER(C.c_int64)]
+        L.sg2_bilevel_forward.restype = C.c_int
+        L.sg2_bilevel_forward.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor), C.c_void_p,
+                                          C.c_void_p, C.c_size_t, C.c_void_p]
+        L.sg2_bilevel_backward.restype = C.c_int
+        L.sg2_bilevel_backward.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor), C.c_void_p,
+                                           C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         _lib = L
     return _lib
 
@@ -160,3 +168,61 @@ class Sg2Step:
                                     C.byref(self.debug) if self.debug is not None else None, stream)
         if rc != 0:
             raise RuntimeError("sg2_batched_step: " + last_error())
+
+
+SG2_BWD_STRIDE = 768        # floats per direction in the gradient block of sg2_bilevel_backward
+
+
+class Sg2Bilevel:
+    """sg2_bilevel_forward / sg2_bilevel_backward on a fixed list of tensors: the sort and the bidirectional scan of
+    the meta-net, differentiable with respect to the scan's weights.  forward() returns the two contexts of every
+    element ([2, sum numel, d_model], element order, tensors packed in call order); backward(d_ctx) returns the
+    gradient block [2, SG2_BWD_STRIDE] described in include/sg_abi.h.  The workspace is kept between the two."""
+
+    def __init__(self, weights, grads, sharps, mamba_fwd, mamba_bwd, dims=None):
+        self.dims = make_dims(dims)
+        self.weights = [w.detach().float().contiguous() for w in weights]
+        assert len(self.weights) == 33 and all(w.is_cuda for w in self.weights)
+        self.W = Sg2Weights()
+        for k, w in enumerate(self.weights):
+            self.W.w[k] = w.data_ptr()
+        self.P = len(grads)
+        self.grads = [g.contiguous() for g in grads]
+        self.sharps = [s.contiguous() for s in sharps]
+        # the entry points overwrite the states with the end-of-sequence ones: work on copies
+        self.mf = [m.detach().float().clone() for m in mamba_fwd]
+        self.mb = [m.detach().float().clone() for m in mamba_bwd]
+        self.numels = [g.numel() for g in self.grads]
+        self.total = sum(self.numels)
+        dev = self.grads[0].device
+        arr = (C.c_int64 * self.P)(*self.numels)
+        nbytes = lib().sg2_bilevel_workspace_bytes(C.byref(self.dims), self.P, arr)
+        if nbytes == 0 and self.total > 0:
+            raise RuntimeError(last_error())
+        self.workspace = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        self.tensors = (Sg2Tensor * self.P)()
+        for i in range(self.P):
+            t, g, s = self.tensors[i], self.grads[i], self.sharps[i]
+            assert g.dtype == s.dtype and g.is_cuda and s.is_cuda
+            t.grad, t.sharpness = g.data_ptr(), s.data_ptr()
+            t.mamba_fwd_state, t.mamba_bwd_state = self.mf[i].data_ptr(), self.mb[i].data_ptr()
+            t.numel, t.dtype = g.numel(), SG_DTYPE[g.dtype]
+        self.device = dev
+
+    def forward(self):
+        ctx = torch.empty(2, self.total, self.dims.d_model, dtype=torch.float32, device=self.device)
+        rc = lib().sg2_bilevel_forward(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, ctx.data_ptr(),
+                                       self.workspace.data_ptr(), self.workspace.numel(), torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError("sg2_bilevel_forward: " + last_error())
+        return ctx
+
+    def backward(self, d_ctx):
+        d_ctx = d_ctx.detach().float().contiguous()
+        assert d_ctx.shape == (2, self.total, self.dims.d_model) and d_ctx.is_cuda
+        out = torch.empty(2, SG2_BWD_STRIDE, dtype=torch.float32, device=self.device)
+        rc = lib().sg2_bilevel_backward(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, d_ctx.data_ptr(), out.data_ptr(),
+                                        self.workspace.data_ptr(), self.workspace.numel(), torch.cuda.current_stream().cuda_stream)
+        if rc != 0:
+            raise RuntimeError("sg2_bilevel_backward: " + last_error())
+        return out
