@@ -29,6 +29,33 @@ def compose_coefficients(Win, bin_, in_proj, dt_W, dt_b, Bp, Cp):
     return torch.stack([xb, z, dt, Bp.to(f) @ xb, Cp.to(f) @ xb], dim=0)
 
 
+def scan_weight_grads(block, W20):
+    """block: [2, SG2_BWD_STRIDE] from sg2_bilevel_backward; W20: the 20 scan weights (input_proj W, b, then the nine
+    tensors of each direction).  Returns the 20 gradients (float64): A_log / rope_freq / D / out_proj directly, the rest
+    by carrying the coefficient gradients through `compose_coefficients`."""
+    blk = block.double()
+    grads = [None] * 20
+    d_in_W = torch.zeros_like(W20[0], dtype=torch.float64)
+    d_in_b = torch.zeros_like(W20[1], dtype=torch.float64)
+    for d in range(2):
+        base = 2 + 9 * d
+        in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj = W20[base:base + 9]
+        o = 5 * GROUP_ROWS * 3
+        dcomp = blk[d, :o].reshape(5, GROUP_ROWS, 3)
+        d_alog = blk[d, o:o + A_log.numel()].reshape(A_log.shape); o += A_log.numel()
+        d_rope = blk[d, o:o + rope.numel()].reshape(rope.shape); o += rope.numel()
+        d_D = blk[d, o:o + D.numel()].reshape(D.shape); o += D.numel()
+        d_out_proj = blk[d, o:o + out_proj.numel()].reshape(out_proj.shape)
+        with torch.enable_grad():
+            raw = [t.detach().double().requires_grad_(True) for t in (W20[0], W20[1], in_proj, dt_W, dt_b, Bp, Cp)]
+            g = torch.autograd.grad(compose_coefficients(*raw), raw, grad_outputs=dcomp)
+        d_in_W += g[0]
+        d_in_b += g[1]
+        grads[base:base + 9] = [g[2], g[3], g[4], g[5], g[6], d_alog, d_D, d_rope, d_out_proj]
+    grads[0], grads[1] = d_in_W, d_in_b
+    return grads
+
+
 class ScanContexts(torch.autograd.Function):
     """(fwd_ctx, bwd_ctx) of every element of a list of tensors as a function of the 20 scan weights
     (input_proj W, b; then in_proj, dt_W, dt_b, B_proj, C_proj, A_log, D, rope_freq, out_proj for each direction)."""
@@ -43,28 +70,105 @@ class ScanContexts(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         W = ctx.saved_tensors
-        blk = ctx.plan.backward(d_out).double()                              # [2, SG2_BWD_STRIDE]
-        grads = [None] * 20
-        d_in_W = torch.zeros_like(W[0], dtype=torch.float64)
-        d_in_b = torch.zeros_like(W[1], dtype=torch.float64)
-        for d in range(2):
-            base = 2 + 9 * d
-            in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj = W[base:base + 9]
-            o = 0
-            dcomp = blk[d, o:o + 5 * GROUP_ROWS * 3].reshape(5, GROUP_ROWS, 3); o += 5 * GROUP_ROWS * 3
-            d_alog = blk[d, o:o + A_log.numel()].reshape(A_log.shape); o += A_log.numel()
-            d_rope = blk[d, o:o + rope.numel()].reshape(rope.shape); o += rope.numel()
-            d_D = blk[d, o:o + D.numel()].reshape(D.shape); o += D.numel()
-            d_out_proj = blk[d, o:o + out_proj.numel()].reshape(out_proj.shape)
-            with torch.enable_grad():
-                raw = [t.detach().double().requires_grad_(True) for t in (W[0], W[1], in_proj, dt_W, dt_b, Bp, Cp)]
-                comp = compose_coefficients(*raw)
-                g = torch.autograd.grad(comp, raw, grad_outputs=dcomp)
-            d_in_W += g[0]
-            d_in_b += g[1]
-            grads[base:base + 9] = [g[2], g[3], g[4], g[5], g[6], d_alog, d_D, d_rope, d_out_proj]
-        grads[0], grads[1] = d_in_W, d_in_b
+        grads = scan_weight_grads(ctx.plan.backward(d_out), W)
         return (None,) + tuple(gr.to(w.dtype) for gr, w in zip(grads, W))
+
+
+def scan_parameters(mn):
+    """The 20 scan parameters of a Mamba3PEERMetaNet in the order ScanContexts expects."""
+    out = [mn.input_proj.weight, mn.input_proj.bias]
+    for blk in (mn.mamba_fwd, mn.mamba_bwd):
+        out += [blk.in_proj.weight, blk.dt_proj.weight, blk.dt_proj.bias, blk.B_proj.weight, blk.C_proj.weight,
+                blk.A_log, blk.D, blk.rope_freq, blk.out_proj.weight]
+    return out
+
+
+def meta_dims(mn):
+    return dict(d_model=mn.d_model, d_state=mn.d_state, d_inner=mn.mamba_fwd.d_inner, gru_hidden=mn.gru_hidden,
+                num_heads=mn.num_peer_heads, pk_dim=mn.pk_dim, expert_hidden=mn.expert_hidden, num_experts=mn.num_experts)
+
+
+def make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd):
+    dev = grads[0].device
+    if dev.type != "cuda":
+        raise RuntimeError("the bilevel path of SuperGrok v2 needs GPU tensors: there is no CPU path")
+    shape = (mn.mamba_fwd.d_inner, mn.d_state)
+    zero = lambda m: torch.zeros(*shape, dtype=torch.float32, device=dev) if m is None else m
+    return _cabi.Sg2Bilevel(mn.flat_weights(), [g.reshape(-1) for g in grads], [s.reshape(-1).to(g.dtype) for s, g in zip(sharps, grads)],
+                            [zero(m) for m in mamba_fwd], [zero(m) for m in mamba_bwd], meta_dims(mn))
+
+
+def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
+    """GRU, soft top-k product-key routing (softmax of 10 x the k best scores of each sub-key, k*k experts per head)
+    and the expert MLPs for N elements: smart gradient [N] and new GRU state
+    (reference: Mamba3PEERMetaNet.forward_for_bilevel, mamba3_peer_metanet.py:395-436; GRU :178-192)."""
+    gru = mn.gru
+    xin = torch.cat([g.unsqueeze(-1), s.unsqueeze(-1), ctx_f, ctx_b], dim=-1)
+    xh = torch.cat([xin, gru_state], dim=-1)
+    z = torch.sigmoid(gru.W_z(xh))
+    r = torch.sigmoid(gru.W_r(xh))
+    cand = torch.tanh(gru.W_h(torch.cat([xin, r * gru_state], dim=-1)))
+    h_new = (1 - z) * gru_state + z * cand
+    pin = torch.cat([h_new, ctx_f, ctx_b, g.unsqueeze(-1), s.unsqueeze(-1)], dim=-1)
+    N, half, pk = g.numel(), mn.d_model // 2, mn.pk_dim
+    W1, b1 = mn.expert_W1.squeeze(-1), mn.expert_b1
+    W2, b2 = mn.expert_W2.squeeze(1), mn.expert_b2.squeeze(-1)
+    total = torch.zeros(N, device=g.device, dtype=torch.float32)
+    for h in range(mn.num_peer_heads):
+        q = mn.peer_queries[h](pin)
+        va, ia = (q[:, :half] @ mn.product_keys_A[h].T).topk(topk, dim=-1)
+        vb, ib = (q[:, half:] @ mn.product_keys_B[h].T).topk(topk, dim=-1)
+        wa, wb = torch.softmax(va * 10.0, dim=-1), torch.softmax(vb * 10.0, dim=-1)
+        idx = (ia.unsqueeze(2) * pk + ib.unsqueeze(1)).reshape(N, -1)
+        route = (wa.unsqueeze(2) * wb.unsqueeze(1)).reshape(N, -1)
+        act = torch.relu(W1[idx] * g.reshape(N, 1, 1) + b1[idx])
+        out = (W2[idx] * act).sum(-1) + b2[idx]
+        total = total + (route * out).sum(dim=1)
+    return g + mn.rescale * (total / mn.num_peer_heads), h_new
+
+
+def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
+    """Differentiable forward of one tensor: (smart_grad, new_gru); gradients reach every parameter of `mn`."""
+    g = grad.reshape(-1).float()
+    s = sharpness.reshape(-1).float()
+    plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
+    ctx = ScanContexts.apply(plan, *scan_parameters(mn))
+    smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float())
+    return smart.reshape(grad.shape).to(grad.dtype), h_new
+
+
+def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bwd, cotangents, chunk=1 << 17):
+    """Adds the gradient of  sum_p <smart_grad_p, cotangent_p>  with respect to every parameter of `mn` to its
+    .grad, for a list of tensors at once.  The scan runs once for all tensors (forward and adjoint in HIP); the
+    per-element part is differentiated in slices of `chunk` elements so that the activations autograd keeps
+    (about 20 KB per element) stay bounded, which is exact because the loss is a sum over elements."""
+    plan = make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd)
+    ctx = plan.forward()
+    d_ctx = torch.empty_like(ctx)
+    g_all = torch.cat([g.reshape(-1).float() for g in grads])
+    s_all = torch.cat([s.reshape(-1).float() for s in sharps])
+    h_all = torch.cat([h.float() for h in gru_states])
+    c_all = torch.cat([c.reshape(-1).float() for c in cotangents])
+    scan_ids = {id(p) for p in scan_parameters(mn)}
+    elem_params = [p for p in mn.parameters() if id(p) not in scan_ids and p.requires_grad]
+    total = g_all.numel()
+    for lo in range(0, total, chunk):
+        hi = min(total, lo + chunk)
+        cf = ctx[0, lo:hi].detach().requires_grad_(True)
+        cb = ctx[1, lo:hi].detach().requires_grad_(True)
+        with torch.enable_grad():
+            smart, _ = per_element(mn, g_all[lo:hi], s_all[lo:hi], cf, cb, h_all[lo:hi])
+            loss = (smart * c_all[lo:hi]).sum()
+        got = torch.autograd.grad(loss, [cf, cb] + elem_params, allow_unused=True)
+        d_ctx[0, lo:hi], d_ctx[1, lo:hi] = got[0], got[1]
+        for p, gr in zip(elem_params, got[2:]):
+            if gr is not None:
+                p.grad = gr if p.grad is None else p.grad + gr
+    scan_params = scan_parameters(mn)
+    for p, gr in zip(scan_params, scan_weight_grads(plan.backward(d_ctx), [p.detach() for p in scan_params])):
+        if p.requires_grad:
+            gr = gr.to(p.dtype)
+            p.grad = gr if p.grad is None else p.grad + gr
 
 
 def scan_contexts(weights33, scan_params, grads, sharps, mamba_fwd, mamba_bwd, dims=None):

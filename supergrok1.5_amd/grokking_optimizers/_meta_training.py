@@ -14,6 +14,7 @@ differentiate; here the perturbed copies require grad and the SAM gradient is
 taken with respect to them.
 """
 import torch
+import torch.nn as nn
 
 from grokking_optimizers import _ops
 
@@ -97,3 +98,47 @@ class MetaTraining:
 
     def get_global_step(self):
         return self._global_step
+
+
+class ScheduledTraining:
+    """The training-loop entry points SuperGrok v1.5 and v2 share (reference: supergrok15.py:415-478 and
+    supergrok2.py:1373-1440): expects sam_step, bilevel_step, step, the adaptive-frequency getters of GrokSchedule
+    and meta_net on self."""
+
+    def sam_meta_step(self, model, train_x, train_y, val_x, val_y, criterion, meta_optimizer):
+        return (self.sam_step(model, train_x, train_y, criterion),
+                self.bilevel_step(model, train_x, train_y, val_x, val_y, criterion, meta_optimizer))
+
+    def get_cached_alpha(self):
+        return self._cached_alpha
+
+    def get_effective_wd(self):
+        return self._get_effective_wd(self.param_groups[0]["weight_decay"]) if self.param_groups else 0.0
+
+    def step_full(self, model, train_x, train_y, val_x, val_y, criterion=None):
+        """Forward + backward + (at their adaptive frequencies) SAM probe and bilevel update + optimizer step;
+        returns the metrics it computed.  Unlike the reference, errors of the SAM probe and of the bilevel update
+        are not swallowed."""
+        criterion = nn.CrossEntropyLoss() if criterion is None else criterion
+        if not hasattr(self, "_auto_meta_opt"):
+            self._auto_meta_opt = torch.optim.Adam(self.meta_net.parameters(), lr=1e-4)
+        model.zero_grad()
+        logits = model(train_x)
+        loss = criterion(logits, train_y)
+        loss.backward()
+        metrics = {}
+        step_num = self._global_step + 1
+        if step_num % self._get_effective_sam_freq() == 0:
+            metrics["sam_loss"] = self.sam_step(model, train_x, train_y, criterion)
+        if step_num % self._get_effective_bilevel_freq() == 0:
+            metrics["val_loss"] = self.bilevel_step(model, train_x, train_y, val_x, val_y, criterion, self._auto_meta_opt)
+        kw = {}
+        if step_num % self.alpha_update_freq == 0 or step_num == 1:
+            with torch.no_grad():
+                kw["train_loss"] = metrics["train_loss"] = float(loss.item())
+                kw["train_acc"] = metrics["train_acc"] = float((logits.detach().argmax(-1) == train_y).float().mean().item())
+                if step_num % self.alpha_update_freq == 0:
+                    kw["val_loss"] = float(criterion(model(val_x), val_y).item())
+                    metrics.setdefault("val_loss", kw["val_loss"])
+        self.step(**kw)
+        return metrics

@@ -15,7 +15,7 @@ import torch.nn as nn
 from torch.optim import Optimizer
 
 from grokking_optimizers import _ops
-from grokking_optimizers._meta_training import MetaTraining
+from grokking_optimizers._meta_training import MetaTraining, ScheduledTraining
 from grokking_optimizers._schedule import GrokSchedule
 
 
@@ -45,7 +45,7 @@ class SharpnessMetaNet(nn.Module):
                 self.rescale.data.item())
 
 
-class SuperGrok15(GrokSchedule, MetaTraining, Optimizer):
+class SuperGrok15(GrokSchedule, MetaTraining, ScheduledTraining, Optimizer):
     def __init__(self, params, lr: float = 1e-3, betas: tuple = (0.9, 0.999), eps: float = 1e-8,
                  weight_decay: float = 1.0, alpha_init: float = 0.98, lamb: float = 2.0, gamma: float = 0.1,
                  gamma_alpha: float = 0.0, kappa: float = 0.1, warmup_steps: int = 100, warmup_ramp: int = 100,
@@ -131,39 +131,4 @@ class SuperGrok15(GrokSchedule, MetaTraining, Optimizer):
         """Bilevel meta-net update on the validation batch with the cached sharpness (supergrok15.py:354-413 there)."""
         return self._meta_update(model, val_x, val_y, criterion, meta_optimizer)
 
-    def sam_meta_step(self, model, train_x, train_y, val_x, val_y, criterion, meta_optimizer):
-        return (self.sam_step(model, train_x, train_y, criterion),
-                self.bilevel_step(model, train_x, train_y, val_x, val_y, criterion, meta_optimizer))
-
-    def get_cached_alpha(self):
-        return self._cached_alpha
-
-    def get_effective_wd(self):
-        return self._get_effective_wd(self.param_groups[0]["weight_decay"]) if self.param_groups else 0.0
-
-    def step_full(self, model, train_x, train_y, val_x, val_y, criterion=None):
-        """Forward + backward + (at their adaptive frequencies) SAM probe and bilevel update + optimizer step;
-        returns the metrics it computed (supergrok15.py:429-478 there)."""
-        criterion = nn.CrossEntropyLoss() if criterion is None else criterion
-        if not hasattr(self, "_auto_meta_opt"):
-            self._auto_meta_opt = torch.optim.Adam(self.meta_net.parameters(), lr=1e-4)
-        model.zero_grad()
-        logits = model(train_x)
-        loss = criterion(logits, train_y)
-        loss.backward()
-        metrics = {}
-        step_num = self._global_step + 1
-        if step_num % self._get_effective_sam_freq() == 0:
-            metrics["sam_loss"] = self.sam_step(model, train_x, train_y, criterion)
-        if step_num % self._get_effective_bilevel_freq() == 0:
-            metrics["val_loss"] = self.bilevel_step(model, train_x, train_y, val_x, val_y, criterion, self._auto_meta_opt)
-        kw = {}
-        if step_num % self.alpha_update_freq == 0 or step_num == 1:
-            with torch.no_grad():
-                kw["train_loss"] = metrics["train_loss"] = float(loss.item())
-                kw["train_acc"] = metrics["train_acc"] = float((logits.detach().argmax(-1) == train_y).float().mean().item())
-                if step_num % self.alpha_update_freq == 0:
-                    kw["val_loss"] = float(criterion(model(val_x), val_y).item())
-                    metrics.setdefault("val_loss", kw["val_loss"])
-        self.step(**kw)
-        return metrics
+    # sam_meta_step, get_cached_alpha, get_effective_wd and step_full come from ScheduledTraining

@@ -20,8 +20,10 @@ Differences, all on the host side:
     product keys are seen by the next step (the reference keeps using stale
     stacked copies until its cache is next invalidated);
   * parameters must live on the GPU: there is no Python fallback path.
-SAM and bilevel meta-training (`sam_step`, `bilevel_step`, `step_full`) are not
-part of this package.
+`sam_step`, `bilevel_step`, `sam_meta_step` and `step_full` are there too: the SAM
+probe through the fused perturb / sharpness ops, the bilevel update with the
+sort and scan of the meta-net in HIP forward and backward and the per-element
+part under torch autograd (grokking_optimizers/_bilevel.py).
 """
 from typing import Optional
 
@@ -30,11 +32,12 @@ import torch.nn as nn
 from torch.optim import Optimizer
 
 from grokking_optimizers import _ops
+from grokking_optimizers._meta_training import MetaTraining, ScheduledTraining
 from grokking_optimizers._schedule import GrokSchedule
 from grokking_optimizers.mamba3_peer_metanet import Mamba3PEERMetaNet
 
 
-class SuperGrok2(GrokSchedule, Optimizer):
+class SuperGrok2(GrokSchedule, MetaTraining, ScheduledTraining, Optimizer):
     def __init__(self, params, lr: float = 1e-3, betas: tuple = (0.9, 0.999), eps: float = 1e-8,
                  weight_decay: float = 1.0, alpha_init: float = 0.98, lamb: float = 2.0, gamma: float = 0.1,
                  gamma_alpha: float = 0.0, kappa: float = 0.1, warmup_steps: int = 100, warmup_ramp: int = 100,
@@ -162,7 +165,44 @@ class SuperGrok2(GrokSchedule, Optimizer):
                 self._weights_dirty = True
         return loss
 
-    def sam_step(self, *a, **k):
-        raise NotImplementedError("SAM and bilevel meta-training are outside this package; only the optimizer step is")
+    # sam_step comes from MetaTraining (supergrok2.py:474-514 of the reference); sam_meta_step, step_full and the
+    # getters from ScheduledTraining.
 
-    bilevel_step = step_full = sam_step
+    def bilevel_step(self, model, train_x, train_y, val_x, val_y, criterion, meta_optimizer):
+        """One meta-optimizer step on  -sum_p <smart_grad_p, val_grad_p / |val_grad_p|>  where smart_grad is the
+        meta-net's differentiable output (soft top-4 routing) on the training gradient, cached sharpness and
+        persistent states of every parameter (reference: supergrok2.py:516-1371).  The sort and the bidirectional
+        scan run in HIP forward and backward, for all parameters in one pass; .grad of the model is restored.
+        Returns the validation loss."""
+        from grokking_optimizers import _bilevel
+        self._ensure_state()
+        named = list(model.named_parameters())
+        saved = {n: p.grad.detach().clone() for n, p in named if p.grad is not None}
+        picked = [(n, p, self._param_to_idx[id(p)]) for n, p in named
+                  if n in saved and id(p) in self._param_to_idx and saved[n].numel() > 0]
+        if not picked:
+            return 0.0
+        model.zero_grad()
+        with torch.enable_grad():
+            val_loss = criterion(model(val_x), val_y)
+            val_loss.backward()
+        meta_optimizer.zero_grad()
+        grads, sharps, grus, mf, mb, cots = [], [], [], [], [], []
+        for n, p, i in picked:
+            if p.grad is None:
+                continue
+            vg = p.grad.detach().float()
+            norm = vg.norm()
+            grads.append(saved[n].reshape(-1).float().contiguous())
+            sharps.append(self._flat_sharpness[i].reshape(-1).float().contiguous())
+            grus.append(self._flat_gru_states[i])
+            mf.append(self._flat_mamba_fwd_states[i])
+            mb.append(self._flat_mamba_bwd_states[i])
+            cots.append(-torch.where(norm > 1e-12, vg / norm, vg).reshape(-1))
+        if grads:
+            _bilevel.accumulate_meta_gradients(self.meta_net, grads, sharps, grus, mf, mb, cots)
+            meta_optimizer.step()
+            self._weights_dirty = True
+        for n, p in named:
+            p.grad = saved.get(n)
+        return float(val_loss.item())

@@ -96,3 +96,162 @@ def test_zero_sharpness_and_zero_states():
 def test_several_chunks():
     """Chunk length 64: the forward pass runs summaries, chunk prefix and replay; the adjoint crosses chunk borders."""
     _case([(1000,), (257,), (640,)], seed=13, sharp=True, state_std=0.3, chunk_len=64)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# whole meta-net: differentiable forward (soft top-4 routing) and the optimizer's bilevel_step
+# ---------------------------------------------------------------------------------------------------------------
+def _ref_forward_for_bilevel(mn, grad, sharp, gru_state, hf, hb):
+    """float64 CPU statement of Mamba3PEERMetaNet.forward_for_bilevel (mamba3_peer_metanet.py:372-436 of the
+    reference) on a double copy `mn` of the module, with ref_fp64.scan_block as the scan."""
+    g, s = grad.reshape(-1), sharp.reshape(-1)
+    N = g.numel()
+    perm = torch.sort(g.abs().float(), stable=True).indices
+    x = mn.input_proj(torch.stack([g[perm], s[perm]], -1))
+    blk = lambda b: [b.in_proj.weight, b.dt_proj.weight, b.dt_proj.bias, b.B_proj.weight, b.C_proj.weight, b.A_log, b.D,
+                     b.rope_freq, b.out_proj.weight]
+    fo, _ = ref_fp64.scan_block(x, blk(mn.mamba_fwd), hf)
+    bo, _ = ref_fp64.scan_block(x.flip(0), blk(mn.mamba_bwd), hb)
+    unsort = torch.argsort(perm)
+    cf, cb = fo[unsort], bo.flip(0)[unsort]
+    xin = torch.cat([g[:, None], s[:, None], cf, cb], -1)
+    xh = torch.cat([xin, gru_state], -1)
+    z, r = torch.sigmoid(mn.gru.W_z(xh)), torch.sigmoid(mn.gru.W_r(xh))
+    hn = (1 - z) * gru_state + z * torch.tanh(mn.gru.W_h(torch.cat([xin, r * gru_state], -1)))
+    pin = torch.cat([hn, cf, cb, g[:, None], s[:, None]], -1)
+    total = torch.zeros(N, 1, dtype=torch.float64)
+    half = mn.d_model // 2
+    for h in range(mn.num_peer_heads):
+        q = mn.peer_queries[h](pin)
+        va, ia = (q[:, :half] @ mn.product_keys_A[h].T).topk(4, dim=-1)
+        vb, ib = (q[:, half:] @ mn.product_keys_B[h].T).topk(4, dim=-1)
+        sa, sb = torch.softmax(va * 10.0, -1), torch.softmax(vb * 10.0, -1)
+        idx = (ia.unsqueeze(2) * mn.pk_dim + ib.unsqueeze(1)).reshape(N, -1)
+        rw = (sa.unsqueeze(2) * sb.unsqueeze(1)).reshape(N, -1)
+        W1, b1, W2, b2 = mn.expert_W1[idx], mn.expert_b1[idx], mn.expert_W2[idx], mn.expert_b2[idx]
+        gx = g.reshape(N, 1, 1, 1).expand(-1, 16, -1, -1)
+        zz = torch.relu(torch.matmul(W1, gx).squeeze(-1) + b1)
+        out = torch.matmul(W2, zz.unsqueeze(-1)).squeeze(-1).squeeze(-1) + b2.squeeze(-1)
+        total = total + (rw * out).sum(1, keepdim=True)
+    return (g[:, None] + mn.rescale * total / mn.num_peer_heads).squeeze(-1), hn
+
+
+def _meta_net(seed, dev):
+    from grokking_optimizers import Mamba3PEERMetaNet
+    torch.manual_seed(seed)
+    mn = Mamba3PEERMetaNet()
+    with torch.no_grad():       # the initial keys and experts are nearly silent: give every part a visible gradient
+        for p in mn.parameters():
+            if p.dim() > 0 and float(p.abs().max()) < 0.05:
+                p.add_(torch.randn_like(p) * 0.2)
+    return mn.to(dev)
+
+
+def _grad_ratios(named_got, named_ref, rel):
+    worst = {}
+    for (n, got), (_, ref) in zip(named_got, named_ref):
+        got = torch.zeros_like(ref) if got is None else got.double().cpu()
+        scale = float(ref.abs().max())
+        worst[n] = round(float((got - ref).abs().max()) / (rel * scale + 1e-12), 3)
+    return worst
+
+
+def test_differentiable_forward_of_the_whole_meta_net():
+    """smart gradient, new GRU state and the gradient of <smart, R> with respect to every parameter of the meta-net,
+    one tensor, against the float64 statement; then the chunked accumulation over several tensors against the sum of
+    the per-tensor autograd gradients."""
+    import copy
+    from grokking_optimizers import _bilevel
+    dev = torch.device("cuda:0")
+    mn = _meta_net(5, dev)
+    mn64 = copy.deepcopy(mn).double().cpu()
+    gen = torch.Generator().manual_seed(17)
+    shapes = [(150,), (9, 11), (64,)]
+    data = []
+    for shp in shapes:
+        n = int(np.prod(shp))
+        data.append(dict(g=torch.randn(n, generator=gen) * 0.5, s=torch.rand(n, generator=gen) * 0.3,
+                         h=torch.randn(n, 4, generator=gen) * 0.5, hf=torch.randn(16, 16, generator=gen) * 0.3,
+                         hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
+    print("whole meta-net forward, shapes", shapes, flush=True)
+    ref_sum = None
+    for k, d in enumerate(data):
+        mn.zero_grad()
+        mn64.zero_grad()
+        smart, hn = _bilevel.forward_for_bilevel(mn, d["g"].to(dev), d["s"].to(dev), d["h"].to(dev), d["hf"].to(dev), d["hb"].to(dev))
+        (smart * d["R"].to(dev)).sum().backward()
+        rs, rh = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
+        (rs * d["R"].double()).sum().backward()
+        for name, got, ref in (("smart", smart, rs), ("gru", hn, rh)):
+            got, ref = got.detach().double().cpu(), ref.detach()
+            err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
+            assert bool((err <= tol).all()), (name, k, float((err / tol).max()))
+        ref_named = [(n, p.grad.clone()) for n, p in mn64.named_parameters()]
+        w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_named, 2e-4)
+        print("tensor", k, "worst gradient ratios", w, flush=True)
+        assert max(w.values()) <= 1.0, w
+        ref_sum = ref_named if ref_sum is None else [(n, a + b) for (n, a), (_, b) in zip(ref_sum, ref_named)]
+    mn.zero_grad()
+    _bilevel.accumulate_meta_gradients(mn, [d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data],
+                                       [d["h"].to(dev) for d in data], [d["hf"].to(dev) for d in data],
+                                       [d["hb"].to(dev) for d in data], [d["R"].to(dev) for d in data], chunk=100)
+    w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_sum, 2e-4)
+    print("chunked accumulation, worst gradient ratios", w, flush=True)
+    assert max(w.values()) <= 1.0, w
+
+
+def test_optimizer_bilevel_step_and_step_full():
+    """SuperGrok2.bilevel_step changes the meta-net along the gradient the accumulation returns, restores the model's
+    gradients and reports the validation loss; step_full with SAM and bilevel at every step runs and learns."""
+    import copy
+    from grokking_optimizers import SuperGrok2, _bilevel
+    dev = torch.device("cuda:0")
+    torch.manual_seed(3)
+    model = torch.nn.Sequential(torch.nn.Linear(12, 24), torch.nn.ReLU(), torch.nn.Linear(24, 5)).to(dev)
+    opt = SuperGrok2(model.parameters(), lr=1e-2, meta_net=_meta_net(8, dev), sam_freq_min=1, sam_freq_max=1,
+                     bilevel_freq_min=1, bilevel_freq_max=1, alpha_update_freq=2)
+    xs, ys = torch.randn(64, 12, device=dev), torch.randint(0, 5, (64,), device=dev)
+    xv, yv = torch.randn(32, 12, device=dev), torch.randint(0, 5, (32,), device=dev)
+    crit = torch.nn.CrossEntropyLoss()
+    print("bilevel_step on a 2-layer model", flush=True)
+    model.zero_grad()
+    crit(model(xs), ys).backward()
+    opt.step()                  # GRU and Mamba states away from zero (a zero GRU state hides the reset gate)
+    model.zero_grad()
+    crit(model(xs), ys).backward()
+    sam_loss = opt.sam_step(model, xs, ys, crit)
+    assert sam_loss > 0 and any(float(s.abs().max()) > 0 for s in opt._flat_sharpness)
+    before_grads = [p.grad.clone() for p in model.parameters()]
+    before_meta = copy.deepcopy(opt.meta_net.state_dict())
+    # expected meta gradient, from the same pieces
+    model.zero_grad()
+    crit(model(xv), yv).backward()
+    cots = []
+    for p in model.parameters():
+        vg = p.grad.detach().float()
+        cots.append(-(vg / vg.norm()).reshape(-1))
+    probe = copy.deepcopy(opt.meta_net)
+    _bilevel.accumulate_meta_gradients(probe, [g.reshape(-1) for g in before_grads], opt._flat_sharpness, opt._flat_gru_states,
+                                       opt._flat_mamba_fwd_states, opt._flat_mamba_bwd_states, cots)
+    for p, g in zip(model.parameters(), before_grads):
+        p.grad = g.clone()
+    meta_opt = torch.optim.SGD(opt.meta_net.parameters(), lr=0.5)
+    val = opt.bilevel_step(model, xs, ys, xv, yv, crit, meta_opt)
+    assert abs(val - float(crit(model(xv), yv).detach())) < 1e-5
+    for p, g in zip(model.parameters(), before_grads):
+        assert torch.equal(p.grad, g)
+    moved = 0
+    for (n, p), q in zip(opt.meta_net.named_parameters(), probe.parameters()):
+        want = before_meta[n] - 0.5 * (q.grad if q.grad is not None else torch.zeros_like(p))
+        scale = float(q.grad.abs().max()) if q.grad is not None else 0.0
+        assert float((p.detach() - want).abs().max()) <= 0.5 * 2e-4 * scale + 1e-7, n      # atomics: order of sums differs
+        moved += int(scale > 0)
+    assert moved == len(list(opt.meta_net.parameters())), moved
+    losses = []
+    for it in range(12):
+        m = opt.step_full(model, xs, ys, xv, yv, crit)
+        assert "sam_loss" in m and "val_loss" in m
+        with torch.no_grad():
+            losses.append(float(crit(model(xs), ys)))
+    print("step_full losses", [round(v, 4) for v in losses], flush=True)
+    assert all(np.isfinite(losses)) and losses[-1] < losses[0]
