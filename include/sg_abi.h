@@ -228,8 +228,9 @@ int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, vo
  * to its weights (grokking_optimizers/supergrok2.py:516-1330 over
  * supergrok2_bilevel_fwd_save / supergrok2_bilevel_backward, csrc/ops.h:232-371).
  * Here the sequential part - sort and bidirectional scan - runs forward and
- * backward in HIP; the per-element part (GRU, soft top-4 PEER routing, experts)
- * is a handful of dense torch ops on the caller's side.
+ * backward in HIP (sg2_bilevel_forward / sg2_bilevel_backward), and so does
+ * the per-element part - GRU, soft top-4 PEER routing, experts -
+ * (sg2_bilevel_elem, forward and backward in one pass).
  *
  * sg2_bilevel_forward: sort + scan exactly as in sg2_batched_step, writing the
  * two contexts of every element to ctx_out ([2][sum numel][d_model] floats,
@@ -252,6 +253,29 @@ int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_t
                         float* ctx_out, void* workspace, size_t workspace_bytes, void* stream);
 int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
                          const float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* sg2_bilevel_elem: the per-element part of Mamba3PEERMetaNet.forward_for_bilevel
+ * (grokking_optimizers/mamba3_peer_metanet.py:395-436 of the reference) and its
+ * derivative, for `total` elements given as flat fp32 arrays (all tensors of
+ * the call packed in the order of sg2_bilevel_forward's ctx_out):
+ *   grad, sharpness, cotangent [total]; ctx [2][total][d_model];
+ *   gru_state [total][gru_hidden] (read only).
+ * With smart_i = grad_i + rescale/heads * sum over heads of the softly routed
+ * expert outputs, it writes
+ *   smart_out [total]            (may be NULL)
+ *   d_ctx     [2][total][d_model]   d/d ctx of  sum_i cotangent_i * smart_i
+ *   grads_out [SG2_ELEM_GRAD_FLOATS], the same derivative for the weights:
+ *     gru W_z[4][22] b_z[4] W_r[4][22] b_r[4] W_h[4][22] b_h[4], peer queries
+ *     [4][8][22], product keys A [4][12][4], B [4][12][4], expert W1 [144][16],
+ *     b1 [144][16], W2 [144][16], b2 [144].
+ * Of `weights` only the GRU, query, key and expert entries are read.  ctx,
+ * gru_state and d_ctx must be 16-byte aligned; the workspace holds one row of
+ * partial sums per workgroup. */
+#define SG2_ELEM_GRAD_FLOATS 8420
+size_t sg2_bilevel_elem_workspace_bytes(int64_t total);
+int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
+                     const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
+                     float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ================== the other fused steps of the reference ================== */
 

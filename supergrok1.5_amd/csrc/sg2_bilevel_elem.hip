@@ -1,0 +1,422 @@
+// Per-element part of the bilevel meta-net update of SuperGrok v2, forward and backward in one pass: GRU, soft
+// top-4 product-key routing (softmax of 10 x the four best scores of each sub-key, 16 experts per head), expert
+// MLPs and the skip connection, followed at once by the gradients of  sum_i cot_i * smart_i  with respect to the
+// two scan contexts of every element and to every weight of this part.
+//
+// Stands in for the per-element kernels of launch_mamba3_peer_backward[_batched]
+// (csrc/supergrok2_mamba_peer_backward_kernels.cu of the reference, driven from
+// grokking_optimizers/supergrok2.py:516-1330); the arithmetic is that of Mamba3PEERMetaNet.forward_for_bilevel
+// (grokking_optimizers/mamba3_peer_metanet.py:395-436) and its autograd derivative.
+//
+// One lane per element, persistent grid over tiles of 256 elements.  Nothing is kept between forward and backward:
+// a lane holds its element's activations in registers, and the routing of a head is differentiated before the
+// next head is evaluated.  Weight gradients are sums over elements:
+//   * experts and product keys (rows chosen per element): float atomics on accumulators in LDS;
+//   * GRU and query matrices (dense outer products d (x) x): every lane leaves its d (44 values) and x (31 values)
+//     in LDS, then each lane of the workgroup owns up to four matrix entries and sums their products over the
+//     256 elements of the tile, keeping the running sums in registers for the life of the workgroup.
+// Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
+// order.  (Within a workgroup the LDS atomics arrive in no fixed order, so expert and key gradients can differ
+// in the last bits between runs.)
+#include "sg2_internal.hpp"
+
+namespace sg2 {
+namespace {
+
+constexpr int BE_THREADS = 256;
+constexpr int EXP_STRIDE = 52;          // floats per expert record in LDS: W1[16] b1[16] W2[16] b2 + pad
+constexpr int TOPK = 4;
+constexpr int XW = 31, DW = 45;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
+// x row: g, s, fwd ctx[8], bwd ctx[8], h_old[4], r*h_old[4], h_new[4], 1
+constexpr int X_G = 0, X_S = 1, X_CF = 2, X_CB = 10, X_H = 18, X_RH = 22, X_HN = 26, X_ONE = 30;
+// d row: d pre_z[4], d pre_r[4], d pre_h[4], d query[4 heads][8]
+constexpr int D_Z = 0, D_R = 4, D_H = 8, D_Q = 12;
+constexpr int N_DENSE = 3 * (GH * GRL + GH) + NH * DM * PIN;      // 276 + 704
+constexpr int OFF_KA = N_DENSE, OFF_KB = OFF_KA + NH * PK * (DM / 2);
+constexpr int OFF_W1 = OFF_KB + NH * PK * (DM / 2), OFF_B1 = OFF_W1 + NE * EH, OFF_W2 = OFF_B1 + NE * EH, OFF_B2 = OFF_W2 + NE * EH;
+constexpr int N_GRADS = OFF_B2 + NE;
+static_assert(N_GRADS == SG2_ELEM_GRAD_FLOATS, "gradient layout");
+constexpr int DENSE_PER_LANE = (N_DENSE + BE_THREADS - 1) / BE_THREADS;
+
+// (column of d, column of x) whose products make up dense gradient entry o, in the order
+// W_z[4][22] b_z[4] W_r[4][22] b_r[4] W_h[4][22] b_h[4] queries[4][8][22]
+__device__ __forceinline__ void dense_entry(int o, int* dcol, int* xcol) {
+    if (o < 3 * (GH * GRL + GH)) {
+        const int gate = o / (GH * GRL + GH), q = o % (GH * GRL + GH);
+        if (q >= GH * GRL) { *dcol = gate * GH + (q - GH * GRL); *xcol = X_ONE; return; }
+        const int j = q / GRL, c = q % GRL;
+        *dcol = gate * GH + j;
+        *xcol = (gate == 2 && c >= 2 + 2 * DM) ? X_RH + (c - 2 - 2 * DM) : c;     // the candidate sees r*h in place of h
+        return;
+    }
+    const int q = o - 3 * (GH * GRL + GH);
+    const int row = q / PIN, c = q % PIN;                 // row = head*8 + r; query input = h_new, fwd ctx, bwd ctx, g, s
+    *dcol = D_Q + row;
+    *xcol = c < GH ? X_HN + c : (c < GH + 2 * DM ? X_CF + (c - GH) : (c == GH + 2 * DM ? X_G : X_S));
+}
+
+struct ElemArgs {
+    const float *g, *s, *ctx, *gru, *cot;
+    float *smart, *d_ctx, *partials;
+    int total;
+    float rescale;
+    Sg2Weights W;
+};
+
+__global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float* s_exp = lds;                                   // [NE][EXP_STRIDE] weights
+    float* s_gexp = s_exp + NE * EXP_STRIDE;              // [NE][EXP_STRIDE] gradients, same layout
+    float* s_gkey = s_gexp + NE * EXP_STRIDE;             // [2][NH][PK][DM/2]
+    float* s_x = s_gkey + 2 * NH * PK * (DM / 2);         // [256][XW]
+    float* s_d = s_x + BE_THREADS * XW;                   // [256][DW]
+
+    const int tid = threadIdx.x;
+    {
+        const float* __restrict__ W1 = a.W.w[W_EXP_W1];
+        const float* __restrict__ B1 = a.W.w[W_EXP_B1];
+        const float* __restrict__ W2 = a.W.w[W_EXP_W2];
+        const float* __restrict__ B2 = a.W.w[W_EXP_B2];
+        for (int i = tid; i < NE * EXP_STRIDE; i += BE_THREADS) { s_gexp[i] = 0.0f; s_exp[i] = 0.0f; }
+        for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) s_gkey[i] = 0.0f;
+        __syncthreads();
+        for (int i = tid; i < NE * EH; i += BE_THREADS) {
+            const int e = i / EH, k = i % EH;
+            s_exp[e * EXP_STRIDE + k] = W1[i];
+            s_exp[e * EXP_STRIDE + EH + k] = B1[i];
+            s_exp[e * EXP_STRIDE + 2 * EH + k] = W2[i];
+        }
+        for (int i = tid; i < NE; i += BE_THREADS) s_exp[i * EXP_STRIDE + 3 * EH] = B2[i];
+    }
+    __syncthreads();
+
+    const sg::cfloat_p Wz = sg::as_const(a.W.w[W_GRU_WZ]), bz = sg::as_const(a.W.w[W_GRU_BZ]);
+    const sg::cfloat_p Wr = sg::as_const(a.W.w[W_GRU_WR]), br = sg::as_const(a.W.w[W_GRU_BR]);
+    const sg::cfloat_p Wh = sg::as_const(a.W.w[W_GRU_WH]), bh = sg::as_const(a.W.w[W_GRU_BH]);
+    const sg::cfloat_p Wq = sg::as_const(a.W.w[W_PEER_Q]);
+    const sg::cfloat_p KA = sg::as_const(a.W.w[W_KEYS_A]), KB = sg::as_const(a.W.w[W_KEYS_B]);
+
+    int dcol[DENSE_PER_LANE], xcol[DENSE_PER_LANE];
+    float dense[DENSE_PER_LANE];
+#pragma unroll
+    for (int q = 0; q < DENSE_PER_LANE; q++) {
+        const int o = tid + q * BE_THREADS;
+        dcol[q] = 0; xcol[q] = 0; dense[q] = 0.0f;
+        if (o < N_DENSE) dense_entry(o, &dcol[q], &xcol[q]);
+    }
+
+    const int tiles = (a.total + BE_THREADS - 1) / BE_THREADS;
+    const float kscale = a.rescale / (float)NH;
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const int i = tile * BE_THREADS + tid;
+        float* xrow = s_x + tid * XW;
+        float* drow = s_d + tid * DW;
+        if (i < a.total) {
+            const float g = a.g[i], s = a.s[i], cot = a.cot[i];
+            float cf[DM], cb[DM], h[GH];
+            {
+                const float4* pf = reinterpret_cast<const float4*>(a.ctx + (size_t)i * DM);
+                const float4* pb = reinterpret_cast<const float4*>(a.ctx + ((size_t)a.total + i) * DM);
+                const float4 a0 = pf[0], a1 = pf[1], b0 = pb[0], b1 = pb[1];
+                cf[0] = a0.x; cf[1] = a0.y; cf[2] = a0.z; cf[3] = a0.w; cf[4] = a1.x; cf[5] = a1.y; cf[6] = a1.z; cf[7] = a1.w;
+                cb[0] = b0.x; cb[1] = b0.y; cb[2] = b0.z; cb[3] = b0.w; cb[4] = b1.x; cb[5] = b1.y; cb[6] = b1.z; cb[7] = b1.w;
+                const float4 h4 = reinterpret_cast<const float4*>(a.gru)[i];
+                h[0] = h4.x; h[1] = h4.y; h[2] = h4.z; h[3] = h4.w;
+            }
+            // ---- GRU forward
+            float zg[GH], rg[GH], cand[GH], hn[GH];
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const sg::cfloat_p wz = Wz + j * GRL, wr = Wr + j * GRL;
+                float vz = bz[j], vr = br[j];
+                vz = sg_fma(wz[0], g, vz); vz = sg_fma(wz[1], s, vz);
+                vr = sg_fma(wr[0], g, vr); vr = sg_fma(wr[1], s, vr);
+#pragma unroll
+                for (int q = 0; q < DM; q++) { vz = sg_fma(wz[2 + q], cf[q], vz); vr = sg_fma(wr[2 + q], cf[q], vr); }
+#pragma unroll
+                for (int q = 0; q < DM; q++) { vz = sg_fma(wz[2 + DM + q], cb[q], vz); vr = sg_fma(wr[2 + DM + q], cb[q], vr); }
+#pragma unroll
+                for (int q = 0; q < GH; q++) { vz = sg_fma(wz[2 + 2 * DM + q], h[q], vz); vr = sg_fma(wr[2 + 2 * DM + q], h[q], vr); }
+                zg[j] = sg_sigmoid(vz);
+                rg[j] = sg_sigmoid(vr);
+            }
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const sg::cfloat_p wh = Wh + j * GRL;
+                float v = bh[j];
+                v = sg_fma(wh[0], g, v); v = sg_fma(wh[1], s, v);
+#pragma unroll
+                for (int q = 0; q < DM; q++) v = sg_fma(wh[2 + q], cf[q], v);
+#pragma unroll
+                for (int q = 0; q < DM; q++) v = sg_fma(wh[2 + DM + q], cb[q], v);
+#pragma unroll
+                for (int q = 0; q < GH; q++) v = sg_fma(wh[2 + 2 * DM + q], rg[q] * h[q], v);
+                cand[j] = sg_tanh(v);
+                hn[j] = sg_fma(zg[j], cand[j], (1.0f - zg[j]) * h[j]);
+            }
+            xrow[X_G] = g; xrow[X_S] = s; xrow[X_ONE] = 1.0f;
+#pragma unroll
+            for (int q = 0; q < DM; q++) { xrow[X_CF + q] = cf[q]; xrow[X_CB + q] = cb[q]; }
+#pragma unroll
+            for (int q = 0; q < GH; q++) { xrow[X_H + q] = h[q]; xrow[X_RH + q] = rg[q] * h[q]; xrow[X_HN + q] = hn[q]; }
+
+            // ---- heads: forward, then at once the head's backward
+            float total = 0.0f;
+            float dhn[GH] = {0.f, 0.f, 0.f, 0.f}, dcf[DM], dcb[DM];
+#pragma unroll
+            for (int q = 0; q < DM; q++) { dcf[q] = 0.0f; dcb[q] = 0.0f; }
+            const float kk = cot * kscale;                 // d loss / d head output
+#pragma unroll 1
+            for (int hh = 0; hh < NH; hh++) {
+                float query[DM];
+#pragma unroll
+                for (int dd = 0; dd < DM; dd++) {
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
+                    float v = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < GH; q++) v = sg_fma(qr[q], hn[q], v);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + q], cf[q], v);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + DM + q], cb[q], v);
+                    v = sg_fma(qr[GH + 2 * DM], g, v);
+                    v = sg_fma(qr[GH + 2 * DM + 1], s, v);
+                    query[dd] = v;
+                }
+                int idx[2][TOPK];
+                float wgt[2][TOPK];
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    float sc[PK];
+#pragma unroll
+                    for (int q = 0; q < PK; q++) {
+                        float dot = 0.0f;
+#pragma unroll
+                        for (int dd = 0; dd < DM / 2; dd++) dot = sg_fma(query[hf * (DM / 2) + dd], keys[q * (DM / 2) + dd], dot);
+                        sc[q] = dot;
+                    }
+                    // four best scores, ties to the lower index; softmax of 10 x score over them
+                    float val[TOPK];
+                    unsigned taken = 0u;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) {
+                        int bi = 0;
+                        float bs = -3.0e38f;
+#pragma unroll
+                        for (int q = 0; q < PK; q++) {
+                            const bool free_ = ((taken >> q) & 1u) == 0u;
+                            if (free_ && sc[q] > bs) { bs = sc[q]; bi = q; }
+                        }
+                        taken |= 1u << bi;
+                        idx[hf][k] = bi;
+                        val[k] = bs;
+                    }
+                    float den = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) { wgt[hf][k] = sg_exp(10.0f * (val[k] - val[0])); den += wgt[hf][k]; }
+                    const float inv = 1.0f / den;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) wgt[hf][k] *= inv;
+                }
+                // experts: out, and the gradients of their weights
+                float ra[TOPK] = {0.f, 0.f, 0.f, 0.f}, rb[TOPK] = {0.f, 0.f, 0.f, 0.f};
+                float head_out = 0.0f;
+#pragma unroll 1
+                for (int c = 0; c < TOPK * TOPK; c++) {
+                    const int ia = c >> 2, ib = c & 3;
+                    // the unrolled selects keep idx/wgt in registers (a dynamic index would send them to scratch)
+                    const int ea = ia == 0 ? idx[0][0] : ia == 1 ? idx[0][1] : ia == 2 ? idx[0][2] : idx[0][3];
+                    const int eb = ib == 0 ? idx[1][0] : ib == 1 ? idx[1][1] : ib == 2 ? idx[1][2] : idx[1][3];
+                    const float wa = ia == 0 ? wgt[0][0] : ia == 1 ? wgt[0][1] : ia == 2 ? wgt[0][2] : wgt[0][3];
+                    const float wb = ib == 0 ? wgt[1][0] : ib == 1 ? wgt[1][1] : ib == 2 ? wgt[1][2] : wgt[1][3];
+                    int e = ea * PK + eb;
+                    if (e >= NE) e = NE - 1;
+                    const float* rec = s_exp + e * EXP_STRIDE;
+                    float* grec = s_gexp + e * EXP_STRIDE;
+                    const float dout = kk * wa * wb;
+                    float out = rec[3 * EH];
+#pragma unroll
+                    for (int m = 0; m < EH; m++) {
+                        const float pre = sg_fma(rec[m], g, rec[EH + m]);
+                        if (pre > 0.0f) {
+                            const float w2 = rec[2 * EH + m];
+                            out = sg_fma(w2, pre, out);
+                            const float dpre = dout * w2;
+                            atomicAdd(&grec[2 * EH + m], dout * pre);
+                            atomicAdd(&grec[m], dpre * g);
+                            atomicAdd(&grec[EH + m], dpre);
+                        }
+                    }
+                    atomicAdd(&grec[3 * EH], dout);
+                    head_out = sg_fma(wa * wb, out, head_out);
+                    const float oa = wb * out, ob = wa * out;
+                    ra[0] += ia == 0 ? oa : 0.0f; ra[1] += ia == 1 ? oa : 0.0f; ra[2] += ia == 2 ? oa : 0.0f; ra[3] += ia == 3 ? oa : 0.0f;
+                    rb[0] += ib == 0 ? ob : 0.0f; rb[1] += ib == 1 ? ob : 0.0f; rb[2] += ib == 2 ? ob : 0.0f; rb[3] += ib == 3 ? ob : 0.0f;
+                }
+                total += head_out;
+                // routing backward: softmax, scores, keys, query
+                float dq[DM];
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    float* gk = s_gkey + (hf * NH + hh) * PK * (DM / 2);
+                    float mean = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) mean = sg_fma(wgt[hf][k], kk * (hf ? rb[k] : ra[k]), mean);
+#pragma unroll
+                    for (int dd = 0; dd < DM / 2; dd++) dq[hf * (DM / 2) + dd] = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) {
+                        const float dv = 10.0f * wgt[hf][k] * (kk * (hf ? rb[k] : ra[k]) - mean);
+                        const int row = idx[hf][k];
+#pragma unroll
+                        for (int dd = 0; dd < DM / 2; dd++) {
+                            dq[hf * (DM / 2) + dd] = sg_fma(dv, keys[row * (DM / 2) + dd], dq[hf * (DM / 2) + dd]);
+                            atomicAdd(&gk[row * (DM / 2) + dd], dv * query[hf * (DM / 2) + dd]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int dd = 0; dd < DM; dd++) {
+                    drow[D_Q + hh * DM + dd] = dq[dd];
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
+#pragma unroll
+                    for (int q = 0; q < GH; q++) dhn[q] = sg_fma(qr[q], dq[dd], dhn[q]);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) dcf[q] = sg_fma(qr[GH + q], dq[dd], dcf[q]);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) dcb[q] = sg_fma(qr[GH + DM + q], dq[dd], dcb[q]);
+                }
+            }
+            if (a.smart != nullptr) a.smart[i] = sg_fma(a.rescale, total / (float)NH, g);
+
+            // ---- GRU backward
+            float dpz[GH], dpr[GH], dph[GH], drh[GH] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                dpz[j] = (dhn[j] * (cand[j] - h[j])) * (zg[j] * (1.0f - zg[j]));
+                dph[j] = (dhn[j] * zg[j]) * (1.0f - cand[j] * cand[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const sg::cfloat_p wh = Wh + j * GRL;
+#pragma unroll
+                for (int q = 0; q < DM; q++) { dcf[q] = sg_fma(wh[2 + q], dph[j], dcf[q]); dcb[q] = sg_fma(wh[2 + DM + q], dph[j], dcb[q]); }
+#pragma unroll
+                for (int q = 0; q < GH; q++) drh[q] = sg_fma(wh[2 + 2 * DM + q], dph[j], drh[q]);
+            }
+#pragma unroll
+            for (int j = 0; j < GH; j++) dpr[j] = (drh[j] * h[j]) * (rg[j] * (1.0f - rg[j]));
+#pragma unroll
+            for (int j = 0; j < GH; j++) {
+                const sg::cfloat_p wz = Wz + j * GRL, wr = Wr + j * GRL;
+#pragma unroll
+                for (int q = 0; q < DM; q++) {
+                    dcf[q] = sg_fma(wz[2 + q], dpz[j], dcf[q]); dcf[q] = sg_fma(wr[2 + q], dpr[j], dcf[q]);
+                    dcb[q] = sg_fma(wz[2 + DM + q], dpz[j], dcb[q]); dcb[q] = sg_fma(wr[2 + DM + q], dpr[j], dcb[q]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < GH; j++) { drow[D_Z + j] = dpz[j]; drow[D_R + j] = dpr[j]; drow[D_H + j] = dph[j]; }
+            {
+                float4* of = reinterpret_cast<float4*>(a.d_ctx + (size_t)i * DM);
+                float4* ob = reinterpret_cast<float4*>(a.d_ctx + ((size_t)a.total + i) * DM);
+                of[0] = make_float4(dcf[0], dcf[1], dcf[2], dcf[3]); of[1] = make_float4(dcf[4], dcf[5], dcf[6], dcf[7]);
+                ob[0] = make_float4(dcb[0], dcb[1], dcb[2], dcb[3]); ob[1] = make_float4(dcb[4], dcb[5], dcb[6], dcb[7]);
+            }
+        } else {
+            for (int q = 0; q < XW; q++) xrow[q] = 0.0f;
+            for (int q = 0; q < DW; q++) drow[q] = 0.0f;
+        }
+        __syncthreads();
+        // ---- dense gradients: each lane's entries, summed over the tile's elements
+        for (int e = 0; e < BE_THREADS; e++) {
+#pragma unroll
+            for (int q = 0; q < DENSE_PER_LANE; q++) dense[q] = sg_fma(s_d[e * DW + dcol[q]], s_x[e * XW + xcol[q]], dense[q]);
+        }
+        __syncthreads();
+    }
+
+    // ---- this workgroup's sums -> its row of the partials buffer
+    float* out = a.partials + (size_t)blockIdx.x * N_GRADS;
+#pragma unroll
+    for (int q = 0; q < DENSE_PER_LANE; q++) {
+        const int o = tid + q * BE_THREADS;
+        if (o < N_DENSE) out[o] = dense[q];
+    }
+    for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) out[OFF_KA + i] = s_gkey[i];
+    for (int i = tid; i < NE * EH; i += BE_THREADS) {
+        const int e = i / EH, k = i % EH;
+        out[OFF_W1 + i] = s_gexp[e * EXP_STRIDE + k];
+        out[OFF_B1 + i] = s_gexp[e * EXP_STRIDE + EH + k];
+        out[OFF_W2 + i] = s_gexp[e * EXP_STRIDE + 2 * EH + k];
+    }
+    for (int i = tid; i < NE; i += BE_THREADS) out[OFF_B2 + i] = s_gexp[i * EXP_STRIDE + 3 * EH];
+}
+
+__global__ void k_sum_partials(const float* __restrict__ partials, int rows, float* __restrict__ out) {
+    const int o = blockIdx.x * blockDim.x + threadIdx.x;
+    if (o >= N_GRADS) return;
+    float acc = 0.0f;
+    for (int r = 0; r < rows; r++) acc += partials[(size_t)r * N_GRADS + o];
+    out[o] = acc;
+}
+
+constexpr int BE_LDS_BYTES = 4 * (2 * NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW));
+constexpr int BE_MAX_GROUPS = 512;
+
+int elem_groups(int64_t total) {
+    const int64_t tiles = (total + BE_THREADS - 1) / BE_THREADS;
+    return (int)(tiles < BE_MAX_GROUPS ? (tiles > 0 ? tiles : 1) : BE_MAX_GROUPS);
+}
+
+}  // namespace
+}  // namespace sg2
+
+extern "C" {
+
+size_t sg2_bilevel_elem_workspace_bytes(int64_t total) {
+    if (total < 0) return 0;
+    return sizeof(float) * (size_t)sg2::elem_groups(total) * sg2::N_GRADS;
+}
+
+int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
+                     const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
+                     float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace sg2;
+    hipStream_t st = (hipStream_t)stream;
+    if (check_dims(dims)) return 1;
+    if (!weights || !grads_out) return sg::fail("NULL argument");
+    if (total < 0 || total > 0x7fffffffLL - BE_THREADS) return sg::fail("element count %lld out of range", (long long)total);
+    for (int k = W_GRU_WZ; k < SG2_NUM_WEIGHTS; k++)
+        if (!weights->w[k]) return sg::fail("weight pointer %d is NULL", k);
+    const int groups = elem_groups(total);
+    if (!workspace || workspace_bytes < sizeof(float) * (size_t)groups * N_GRADS)
+        return sg::fail("workspace too small: need %zu bytes, got %zu", sizeof(float) * (size_t)groups * N_GRADS, workspace_bytes);
+    if (total > 0) {
+        if (!grad || !sharpness || !ctx || !gru_state || !cotangent || !d_ctx) return sg::fail("NULL argument");
+        if ((((uintptr_t)ctx | (uintptr_t)gru_state | (uintptr_t)d_ctx) & 15u) != 0) return sg::fail("ctx, gru_state and d_ctx must be 16-byte aligned");
+    }
+    {
+        static bool raised[64] = {};
+        int dev = 0;
+        SG_HIP_CHECK(hipGetDevice(&dev));
+        if (dev < 0 || dev >= 64) return sg::fail("device index %d out of range", dev);
+        if (!raised[dev]) {
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bilevel_elem), hipFuncAttributeMaxDynamicSharedMemorySize, BE_LDS_BYTES));
+            raised[dev] = true;
+        }
+    }
+    ElemArgs a;
+    a.g = grad; a.s = sharpness; a.ctx = ctx; a.gru = gru_state; a.cot = cotangent;
+    a.smart = smart_out; a.d_ctx = d_ctx; a.partials = static_cast<float*>(workspace);
+    a.total = (int)total; a.rescale = rescale; a.W = *weights;
+    hipLaunchKernelGGL(k_bilevel_elem, dim3(groups), dim3(BE_THREADS), BE_LDS_BYTES, st, a);
+    SG_LAUNCH_CHECK("k_bilevel_elem");
+    hipLaunchKernelGGL(k_sum_partials, dim3((N_GRADS + 255) / 256), dim3(256), 0, st, a.partials, groups, grads_out);
+    SG_LAUNCH_CHECK("k_sum_partials");
+    return 0;
+}
+
+}  // extern "C"

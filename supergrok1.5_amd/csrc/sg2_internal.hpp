@@ -91,6 +91,7 @@ int launch_scan(const Plan& pl, hipStream_t st);
 // tile index of scan step u of tensor ti (element offset off) in the per-tile state array of the bilevel path
 __host__ __device__ inline int htile_index(int off, int ti, int u) { return off / SCAN_TT + ti + u / SCAN_TT; }
 __host__ __device__ inline int htile_count(int total, int P) { return total / SCAN_TT + P + 1; }
+int check_dims(const SgDims* d);
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
 

@@ -79,6 +79,8 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bil
     return 0;
 }
 
+}  // namespace
+
 int check_dims(const SgDims* d) {
     if (!d) return sg::fail("dims is NULL");
     // the limits the reference enforces (csrc/supergrok2_mamba_peer_kernels.cu:1796-1801)
@@ -96,6 +98,8 @@ int check_dims(const SgDims* d) {
                         DM, DS, DI, GH, NH, PK, EH, NE);
     return 0;
 }
+
+namespace {
 
 }  // namespace
 

@@ -3,10 +3,14 @@
 grokking_optimizers/mamba3_peer_metanet.py:372-436, driven from
 grokking_optimizers/supergrok2.py:516-1371).
 
-The sequential part - magnitude sort and bidirectional Mamba-3 scan - runs in
-HIP, forward and backward (`ScanContexts`, over sg2_bilevel_forward /
-sg2_bilevel_backward); what follows per element (GRU, soft top-4 PEER routing,
-expert MLPs) is dense tensor algebra and is left to torch autograd.
+The optimizer's bilevel update (`accumulate_meta_gradients`) runs in HIP end to
+end: sort + bidirectional Mamba-3 scan (sg2_bilevel_forward), per-element GRU /
+soft top-4 PEER routing / expert MLPs forward and backward in one pass
+(sg2_bilevel_elem), then the exact adjoint of the scan (sg2_bilevel_backward).
+`forward_for_bilevel` is the module-level differentiable forward of one tensor:
+the scan as an autograd Function over the same two entry points, the per-element
+part as torch ops (`per_element`), which is also what the tests check
+sg2_bilevel_elem against.
 """
 import torch
 
@@ -137,38 +141,47 @@ def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, ma
     return smart.reshape(grad.shape).to(grad.dtype), h_new
 
 
-def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bwd, cotangents, chunk=1 << 17):
+def elem_parameters(mn):
+    """(parameter, shape in the gradient block of sg2_bilevel_elem) in the block's order."""
+    out = []
+    for lin in (mn.gru.W_z, mn.gru.W_r, mn.gru.W_h):
+        out += [lin.weight, lin.bias]
+    return out, list(mn.peer_queries), list(mn.product_keys_A), list(mn.product_keys_B), \
+        [mn.expert_W1, mn.expert_b1, mn.expert_W2, mn.expert_b2]
+
+
+def _add_grad(p, gr):
+    if p.requires_grad:
+        gr = gr.reshape(p.shape).to(p.dtype)
+        p.grad = gr.clone() if p.grad is None else p.grad + gr
+
+
+def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bwd, cotangents):
     """Adds the gradient of  sum_p <smart_grad_p, cotangent_p>  with respect to every parameter of `mn` to its
-    .grad, for a list of tensors at once.  The scan runs once for all tensors (forward and adjoint in HIP); the
-    per-element part is differentiated in slices of `chunk` elements so that the activations autograd keeps
-    (about 20 KB per element) stay bounded, which is exact because the loss is a sum over elements."""
+    .grad, for a list of tensors at once, all in HIP: scan forward (sg2_bilevel_forward), per-element forward and
+    backward (sg2_bilevel_elem), scan adjoint (sg2_bilevel_backward).  Returns the smart gradients (flat, packed)."""
     plan = make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd)
     ctx = plan.forward()
-    d_ctx = torch.empty_like(ctx)
     g_all = torch.cat([g.reshape(-1).float() for g in grads])
     s_all = torch.cat([s.reshape(-1).float() for s in sharps])
     h_all = torch.cat([h.float() for h in gru_states])
     c_all = torch.cat([c.reshape(-1).float() for c in cotangents])
-    scan_ids = {id(p) for p in scan_parameters(mn)}
-    elem_params = [p for p in mn.parameters() if id(p) not in scan_ids and p.requires_grad]
-    total = g_all.numel()
-    for lo in range(0, total, chunk):
-        hi = min(total, lo + chunk)
-        cf = ctx[0, lo:hi].detach().requires_grad_(True)
-        cb = ctx[1, lo:hi].detach().requires_grad_(True)
-        with torch.enable_grad():
-            smart, _ = per_element(mn, g_all[lo:hi], s_all[lo:hi], cf, cb, h_all[lo:hi])
-            loss = (smart * c_all[lo:hi]).sum()
-        got = torch.autograd.grad(loss, [cf, cb] + elem_params, allow_unused=True)
-        d_ctx[0, lo:hi], d_ctx[1, lo:hi] = got[0], got[1]
-        for p, gr in zip(elem_params, got[2:]):
-            if gr is not None:
-                p.grad = gr if p.grad is None else p.grad + gr
+    smart, d_ctx, blk = _cabi.bilevel_elem(plan.weights, g_all, s_all, ctx, h_all, c_all, float(mn.rescale), meta_dims(mn))
+    gru_p, queries, keys_a, keys_b, experts = elem_parameters(mn)
+    o = 0
+    for p in gru_p:
+        _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
+    for group in (queries, keys_a, keys_b):
+        for q in group:
+            p = q.weight if isinstance(q, torch.nn.Linear) else q
+            _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
+    for p in experts:
+        _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
+    assert o == _cabi.SG2_ELEM_GRAD_FLOATS
     scan_params = scan_parameters(mn)
     for p, gr in zip(scan_params, scan_weight_grads(plan.backward(d_ctx), [p.detach() for p in scan_params])):
-        if p.requires_grad:
-            gr = gr.to(p.dtype)
-            p.grad = gr if p.grad is None else p.grad + gr
+        _add_grad(p, gr)
+    return smart
 
 
 def scan_contexts(weights33, scan_params, grads, sharps, mamba_fwd, mamba_bwd, dims=None):

@@ -77,6 +77,11 @@ def lib():
         L.sg2_bilevel_backward.restype = C.c_int
         L.sg2_bilevel_backward.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor), C.c_void_p,
                                            C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.sg2_bilevel_elem_workspace_bytes.restype = C.c_size_t
+        L.sg2_bilevel_elem_workspace_bytes.argtypes = [C.c_int64]
+        L.sg2_bilevel_elem.restype = C.c_int
+        L.sg2_bilevel_elem.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int64] + [C.c_void_p] * 5 + [C.c_float] + \
+                                      [C.c_void_p] * 4 + [C.c_size_t, C.c_void_p]
         _lib = L
     return _lib
 
@@ -226,3 +231,32 @@ class Sg2Bilevel:
         if rc != 0:
             raise RuntimeError("sg2_bilevel_backward: " + last_error())
         return out
+
+
+SG2_ELEM_GRAD_FLOATS = 8420
+
+
+def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, dims=None, want_smart=True):
+    """sg2_bilevel_elem on flat fp32 GPU arrays: returns (smart [total] or None, d_ctx [2, total, d_model],
+    weight-gradient block [SG2_ELEM_GRAD_FLOATS])."""
+    d = make_dims(dims)
+    ws_ = [w.detach().float().contiguous() for w in weights]
+    W = Sg2Weights()
+    for k, w in enumerate(ws_):
+        W.w[k] = w.data_ptr()
+    arrs = [t.detach().float().contiguous() for t in (grad, sharpness, ctx, gru_state, cotangent)]
+    total = arrs[0].numel()
+    dev = arrs[0].device
+    assert all(t.is_cuda for t in arrs) and arrs[2].shape == (2, total, d.d_model) and arrs[3].shape == (total, d.gru_hidden)
+    assert arrs[1].numel() == total and arrs[4].numel() == total
+    smart = torch.empty(total, dtype=torch.float32, device=dev) if want_smart else None
+    d_ctx = torch.empty_like(arrs[2])
+    out = torch.empty(SG2_ELEM_GRAD_FLOATS, dtype=torch.float32, device=dev)
+    nbytes = lib().sg2_bilevel_elem_workspace_bytes(total)
+    work = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    rc = lib().sg2_bilevel_elem(C.byref(d), C.byref(W), total, *[t.data_ptr() for t in arrs], float(rescale),
+                                smart.data_ptr() if want_smart else None, d_ctx.data_ptr(), out.data_ptr(), work.data_ptr(),
+                                work.numel(), torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError("sg2_bilevel_elem: " + last_error())
+    return smart, d_ctx, out

@@ -22,8 +22,7 @@ Differences, all on the host side:
   * parameters must live on the GPU: there is no Python fallback path.
 `sam_step`, `bilevel_step`, `sam_meta_step` and `step_full` are there too: the SAM
 probe through the fused perturb / sharpness ops, the bilevel update with the
-sort and scan of the meta-net in HIP forward and backward and the per-element
-part under torch autograd (grokking_optimizers/_bilevel.py).
+meta-net differentiated in HIP (grokking_optimizers/_bilevel.py).
 """
 from typing import Optional
 
@@ -171,8 +170,8 @@ class SuperGrok2(GrokSchedule, MetaTraining, ScheduledTraining, Optimizer):
     def bilevel_step(self, model, train_x, train_y, val_x, val_y, criterion, meta_optimizer):
         """One meta-optimizer step on  -sum_p <smart_grad_p, val_grad_p / |val_grad_p|>  where smart_grad is the
         meta-net's differentiable output (soft top-4 routing) on the training gradient, cached sharpness and
-        persistent states of every parameter (reference: supergrok2.py:516-1371).  The sort and the bidirectional
-        scan run in HIP forward and backward, for all parameters in one pass; .grad of the model is restored.
+        persistent states of every parameter (reference: supergrok2.py:516-1371).  The meta-net runs in HIP forward and
+        backward, for all parameters in one pass; .grad of the model is restored.
         Returns the validation loss."""
         from grokking_optimizers import _bilevel
         self._ensure_state()

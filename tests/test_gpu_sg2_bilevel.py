@@ -158,8 +158,9 @@ def _grad_ratios(named_got, named_ref, rel):
 
 def test_differentiable_forward_of_the_whole_meta_net():
     """smart gradient, new GRU state and the gradient of <smart, R> with respect to every parameter of the meta-net,
-    one tensor, against the float64 statement; then the chunked accumulation over several tensors against the sum of
-    the per-tensor autograd gradients."""
+    one tensor at a time through the autograd form (HIP scan + torch per-element part), against the float64
+    statement; then the all-HIP accumulation over the three tensors at once (sg2_bilevel_forward, sg2_bilevel_elem,
+    sg2_bilevel_backward) against the sum of the float64 gradients and the float64 smart gradients."""
     import copy
     from grokking_optimizers import _bilevel
     dev = torch.device("cuda:0")
@@ -174,7 +175,7 @@ def test_differentiable_forward_of_the_whole_meta_net():
                          h=torch.randn(n, 4, generator=gen) * 0.5, hf=torch.randn(16, 16, generator=gen) * 0.3,
                          hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
     print("whole meta-net forward, shapes", shapes, flush=True)
-    ref_sum = None
+    ref_sum, ref_smart = None, []
     for k, d in enumerate(data):
         mn.zero_grad()
         mn64.zero_grad()
@@ -186,17 +187,22 @@ def test_differentiable_forward_of_the_whole_meta_net():
             got, ref = got.detach().double().cpu(), ref.detach()
             err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
             assert bool((err <= tol).all()), (name, k, float((err / tol).max()))
+        ref_smart.append(rs.detach())
         ref_named = [(n, p.grad.clone()) for n, p in mn64.named_parameters()]
         w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_named, 2e-4)
         print("tensor", k, "worst gradient ratios", w, flush=True)
         assert max(w.values()) <= 1.0, w
         ref_sum = ref_named if ref_sum is None else [(n, a + b) for (n, a), (_, b) in zip(ref_sum, ref_named)]
     mn.zero_grad()
-    _bilevel.accumulate_meta_gradients(mn, [d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data],
-                                       [d["h"].to(dev) for d in data], [d["hf"].to(dev) for d in data],
-                                       [d["hb"].to(dev) for d in data], [d["R"].to(dev) for d in data], chunk=100)
+    print("all-HIP accumulation over the three tensors", flush=True)
+    smart = _bilevel.accumulate_meta_gradients(mn, [d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data],
+                                               [d["h"].to(dev) for d in data], [d["hf"].to(dev) for d in data],
+                                               [d["hb"].to(dev) for d in data], [d["R"].to(dev) for d in data])
+    got, ref = smart.double().cpu(), torch.cat(ref_smart)
+    err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
+    assert bool((err <= tol).all()), ("smart", float((err / tol).max()))
     w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_sum, 2e-4)
-    print("chunked accumulation, worst gradient ratios", w, flush=True)
+    print("all-HIP accumulation, worst gradient ratios", w, flush=True)
     assert max(w.values()) <= 1.0, w
 
 
