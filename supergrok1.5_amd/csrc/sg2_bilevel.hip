@@ -9,21 +9,27 @@
 // the state entering every 64-step tile; the per-element part of the meta-net (GRU, soft top-4 PEER routing,
 // experts) is differentiated by torch autograd on the caller's side.
 //
-// One 128-lane workgroup per (tensor, direction) walks the tensor's tiles from the last scan step to the first,
-// lane (j,p) owning column j and RoPE pair p as in the forward kernels.  Per tile:
+// The adjoint state lambda obeys a linear recurrence over the scan steps in reverse, so a tensor is cut into the
+// chunks of the forward pass and handled in three launches, like the forward scan:
+//   k_adj_summary  per (chunk, direction): the affine map lambda_end-of-chunk -> lambda_start-of-chunk
+//                  (a 2x2 matrix and an offset per lane), which needs only d y of every step, not the states;
+//   k_adj_prefix   per (tensor, direction): composes the maps from the last chunk to the first, leaving the adjoint
+//                  state that arrives at the end of every chunk;
+//   k_bilevel_backward  per (chunk, direction), exact from that arriving state.  A 128-lane workgroup walks the
+//                  chunk's 64-step tiles from the last to the first, lane (j,p) owning column j and RoPE pair p
+//                  as in the forward kernels.  Per tile:
 //   1  projections of the 64 steps from (g, s) and the composed coefficients, with the derivatives of softplus
 //      and SiLU, and the incoming context gradients gathered from element order;
 //   2  the forward recurrence from the saved tile-start state, keeping the state after every step in LDS;
 //   3  per step and column: out, d out = out_proj^T d ctx, d y, d z, the D-skip part of d x-branch;
-//   4  the adjoint recurrence over the steps in reverse: lambda <- R(theta)^T diag(A_bar) lambda + d y C, with
+//   4  the adjoint recurrence over the steps in reverse: lambda <- R(theta)^T diag(A_bar) (lambda + d y C), with
 //      the gradients of dt, x-branch, B and C per step (reduced over pairs / columns) and of A_log and the RoPE
 //      frequencies per lane;
 //   5  sums over the tile's steps: composed-coefficient gradients d v (x) (g, s, 1), d D, d out_proj.
-// The adjoint state lambda is carried from tile to tile, so the result is exact (no truncation); the price is
-// that a tensor's steps are visited serially by one workgroup.  Gradients of the composed coefficients are
-// mapped back to input_proj / in_proj / dt_proj / B_proj / C_proj by the caller (the composition is a handful of
-// small matrix products).  Accumulation into the output arrays uses float atomics: sums over tensors arrive in
-// no fixed order.
+// Nothing is truncated: the result is the exact adjoint.  Gradients of the composed coefficients are mapped back
+// to input_proj / in_proj / dt_proj / B_proj / C_proj by the caller (the composition is a handful of small matrix
+// products).  Every workgroup keeps its sums in registers over the chunks it handles and writes them to its own
+// row of a partials buffer, which k_adj_sum_rows adds in a fixed order: the result is reproducible run to run.
 #include "sg2_internal.hpp"
 #include "../../include/sg2_compose.h"
 
@@ -52,7 +58,132 @@ __device__ __forceinline__ float pair_sum(float v) {             // sum over the
     return v;
 }
 
-__global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, const float* __restrict__ d_ctx, float* __restrict__ gout) {
+// What a (chunk, direction) needs to find its steps.
+struct ChunkRef {
+    int ti, N, off, ustart, uend;
+    bool has_s;
+    const uint32_t* skey;
+    const int32_t* sval;
+    const float* ssrt;
+    const float* dctx;
+};
+__device__ __forceinline__ ChunkRef chunk_ref(const Plan& pl, int chunk, int dir, const float* d_ctx) {
+    ChunkRef c;
+    c.ti = sg::upper_seg(sg::as_const(pl.chunk_prefix), pl.P, chunk);
+    const TensorDev& T = pl.tensors[c.ti];
+    c.N = T.numel;
+    c.off = T.off;
+    c.ustart = (chunk - pl.chunk_prefix[c.ti]) * pl.chunk_len;
+    c.uend = min(c.N, c.ustart + pl.chunk_len);
+    c.has_s = pl.sharp_nonzero[c.ti] != 0;        // all-zero sharpness is never gathered into sorted order
+    c.skey = pl.keys[0] + c.off;
+    c.sval = pl.vals[0] + c.off;
+    c.ssrt = pl.ssorted + c.off;
+    c.dctx = d_ctx + ((size_t)dir * pl.total + c.off) * DM;
+    return c;
+}
+// (g, s) and the element index of scan step u of a chunk's tensor; zeros past the end
+__device__ __forceinline__ void load_step(const ChunkRef& c, int dir, int u, bool valid, float* g, float* s, int* orig) {
+    *g = 0.0f; *s = 0.0f; *orig = 0;
+    if (valid) {
+        const int t = dir ? (c.N - 1 - u) : u;
+        const int32_t v = c.sval[t];
+        int o = v & 0x7fffffff;
+        *orig = ((unsigned)o < (unsigned)c.N) ? o : 0;
+        *g = sg_i2f((int32_t)c.skey[t] | (v & (int32_t)0x80000000));
+        *s = c.has_s ? c.ssrt[t] : 0.0f;
+    }
+}
+
+// lambda -> R(theta)^T diag(A_bar) lambda for one lane's pair
+__device__ __forceinline__ void adj_apply(float ae, float ao, float sn, float cs, float* xe, float* xo) {
+    const float dre = *xe * ae, dro = *xo * ao;
+    *xe = sg_fma(dre, cs, dro * sn);
+    *xo = sg_fma(dro, cs, -(dre * sn));
+}
+
+// ---- launch 1: affine map of the adjoint state across every chunk
+constexpr int SUMM_ROWS = 4;                     // LDS arrays of the summary kernel: dt, C, gate, d y
+__global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const float* __restrict__ d_ctx) {
+    __shared__ float rows[SUMM_ROWS * ROWS * BST];
+    __shared__ __attribute__((aligned(16))) float s_dctx[SCAN_TT * DM];
+    auto arr = [&](int a) { return rows + a * ROWS * BST; };
+    const int chunk = blockIdx.x, dir = blockIdx.y;
+    const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
+    const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+    const float* __restrict__ Alog = pl.W.w[b + 5];
+    const float* __restrict__ rope = pl.W.w[b + 7];
+    const float* __restrict__ Wout = pl.W.w[b + 8];
+    const float* __restrict__ comp = pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3);
+    const int tid = threadIdx.x;
+    const int tu = tid & (SCAN_TT - 1), half = tid >> 6;
+    const int j = tid >> 3, p = tid & 7;
+    const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
+    const float freq = rope[j * HP + p];
+    float u1e = 1.0f, u1o = 0.0f, u2e = 0.0f, u2o = 1.0f, ve = 0.0f, vo = 0.0f;
+    const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
+    for (int tile = ntiles - 1; tile >= 0; tile--) {
+        const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
+        {
+            const bool valid = tu < cnt;
+            float g, s;
+            int orig;
+            load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
+            const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
+            reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
+            for (int q = 0; q < ROWS / 2; q++) {
+                const int r = half * (ROWS / 2) + q;
+                arr(0)[r * BST + tu] = valid ? sg_softplus(sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s)) : 0.0f;
+                arr(1)[r * BST + tu] = sg2_comp_eval(comp + (SG2_COMP_C * 16 + r) * 3, g, s);
+                const float z = sg2_comp_eval(comp + (SG2_COMP_Z * 16 + r) * 3, g, s);
+                arr(2)[r * BST + tu] = z * sg_sigmoid(z);
+            }
+        }
+        __syncthreads();
+        for (int q = 0; q < ROWS / 2; q++) {
+            const int r = half * (ROWS / 2) + q;
+            float dout = 0.0f;
+#pragma unroll
+            for (int d = 0; d < DM; d++) dout = sg_fma(Wout[d * DI + r], s_dctx[tu * DM + d], dout);
+            arr(3)[r * BST + tu] = (tu < cnt) ? dout * arr(2)[r * BST + tu] : 0.0f;
+        }
+        __syncthreads();
+        for (int k = cnt - 1; k >= 0; k--) {
+            const float dt = arr(0)[j * BST + k], dy = arr(3)[j * BST + k];
+            float ae, ao, sn, cs;
+            sg_abar_pair(dt, a_e, a_o, &ae, &ao);
+            sg_sincos(dt * freq, &sn, &cs);
+            ve = sg_fma(dy, arr(1)[(2 * p) * BST + k], ve);
+            vo = sg_fma(dy, arr(1)[(2 * p + 1) * BST + k], vo);
+            adj_apply(ae, ao, sn, cs, &u1e, &u1o);
+            adj_apply(ae, ao, sn, cs, &u2e, &u2o);
+            adj_apply(ae, ao, sn, cs, &ve, &vo);
+        }
+        __syncthreads();
+    }
+    float* out = pl.adj_summ + (((size_t)dir * pl.chunks + chunk) * SCAN_THREADS + tid) * 6;
+    out[0] = u1e; out[1] = u1o; out[2] = u2e; out[3] = u2o; out[4] = ve; out[5] = vo;
+}
+
+// ---- launch 2: adjoint state arriving at the end of every chunk, last chunk of a tensor first
+__global__ __launch_bounds__(SCAN_THREADS) void k_adj_prefix(Plan pl) {
+    const int ti = blockIdx.x, dir = blockIdx.y, tid = threadIdx.x;
+    const int base = pl.chunk_prefix[ti], nc = pl.chunk_prefix[ti + 1] - base;
+    float le = 0.0f, lo = 0.0f;
+    for (int c = nc - 1; c >= 0; c--) {
+        const size_t at = ((size_t)dir * pl.chunks + base + c) * SCAN_THREADS + tid;
+        pl.adj_lam[at * 2] = le;
+        pl.adj_lam[at * 2 + 1] = lo;
+        const float* m = pl.adj_summ + at * 6;
+        const float ne = sg_fma(m[0], le, sg_fma(m[2], lo, m[4]));
+        const float no = sg_fma(m[1], le, sg_fma(m[3], lo, m[5]));
+        le = ne;
+        lo = no;
+    }
+}
+
+// ---- launch 3: the gradients, chunk by chunk
+__global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, const float* __restrict__ d_ctx) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* rows = lds;
     float* sH = lds + LDS_ROWS_FLOATS;
@@ -60,26 +191,13 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     float* s_gs = s_dctx + SCAN_TT * DM;
     auto arr = [&](int a) { return rows + a * ROWS * BST; };
 
-    const int ti = blockIdx.x % pl.P, dir = blockIdx.x / pl.P;
-    const TensorDev& T = pl.tensors[ti];
-    const int N = T.numel, off = T.off;
-    if (N == 0) return;
-    const bool has_s = pl.sharp_nonzero[ti] != 0;      // all-zero sharpness is never gathered into sorted order
+    const int dir = blockIdx.y;
     const int b = dir ? W_B_INPROJ : W_F_INPROJ;
     const float* __restrict__ Alog = pl.W.w[b + 5];
     const float* __restrict__ Dw = pl.W.w[b + 6];
     const float* __restrict__ rope = pl.W.w[b + 7];
     const float* __restrict__ Wout = pl.W.w[b + 8];
     const float* __restrict__ comp = pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3);
-    const uint32_t* __restrict__ skey = pl.keys[0] + off;
-    const int32_t* __restrict__ sval = pl.vals[0] + off;
-    const float* __restrict__ ssrt = pl.ssorted + off;
-    const float* __restrict__ dctx = d_ctx + ((size_t)dir * pl.total + off) * DM;
-    float* __restrict__ g_comp = gout + dir * SG2_BWD_STRIDE;
-    float* __restrict__ g_alog = g_comp + SG2_COMP_GROUPS * 16 * 3;
-    float* __restrict__ g_rope = g_alog + DI * DS;
-    float* __restrict__ g_D = g_rope + DI * HP;
-    float* __restrict__ g_wout = g_D + DI;
 
     const int tid = threadIdx.x;
     const int tu = tid & (SCAN_TT - 1), half = tid >> 6;          // projection role
@@ -87,30 +205,30 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
 
-    float le = 0.0f, lo = 0.0f;                      // adjoint of the state after the current step
     float acc_alog_e = 0.0f, acc_alog_o = 0.0f, acc_rope = 0.0f;
     float acc_c0 = 0.0f, acc_c1 = 0.0f, acc_c2 = 0.0f, acc_D = 0.0f, acc_wout = 0.0f;
 
-    const int ntiles = (N + SCAN_TT - 1) / SCAN_TT;
+  for (int chunk = blockIdx.x; chunk < pl.chunks; chunk += gridDim.x) {
+    const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
+    const int ti = c.ti, off = c.off;
+    float le, lo;                                    // adjoint of the state after the current step
+    {
+        const float* lam = pl.adj_lam + (((size_t)dir * pl.chunks + chunk) * SCAN_THREADS + tid) * 2;
+        le = lam[0];
+        lo = lam[1];
+    }
+    const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
     for (int tile = ntiles - 1; tile >= 0; tile--) {
-        const int u0 = tile * SCAN_TT, cnt = min(SCAN_TT, N - u0);
+        const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
         // ---- 1: projections, activation derivatives, incoming gradients
         {
-            const int u = u0 + tu;
             const bool valid = tu < cnt;
-            float g = 0.0f, s = 0.0f;
-            int orig = 0;
-            if (valid) {
-                const int t = dir ? (N - 1 - u) : u;
-                const int32_t v = sval[t];
-                orig = v & 0x7fffffff;
-                orig = ((unsigned)orig < (unsigned)N) ? orig : 0;
-                g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
-                s = has_s ? ssrt[t] : 0.0f;
-            }
+            float g, s;
+            int orig;
+            load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
             if (half == 0) { s_gs[2 * tu] = g; s_gs[2 * tu + 1] = s; }
             {
-                const float4 dv = valid ? reinterpret_cast<const float4*>(dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
                 reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
             }
             for (int q = 0; q < ROWS / 2; q++) {
@@ -248,17 +366,34 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         __syncthreads();
     }
 
-    atomicAdd(&g_alog[j * DS + 2 * p], acc_alog_e);
-    atomicAdd(&g_alog[j * DS + 2 * p + 1], acc_alog_o);
-    atomicAdd(&g_rope[j * HP + p], acc_rope);
+  }
+    // this workgroup's sums -> its row of the partials buffer (every entry of the row is written)
+    float* g_comp = pl.adj_part + ((size_t)dir * gridDim.x + blockIdx.x) * SG2_BWD_STRIDE;
+    float* g_alog = g_comp + SG2_COMP_GROUPS * 16 * 3;
+    float* g_rope = g_alog + DI * DS;
+    float* g_D = g_rope + DI * HP;
+    float* g_wout = g_D + DI;
+    g_alog[j * DS + 2 * p] = acc_alog_e;
+    g_alog[j * DS + 2 * p + 1] = acc_alog_o;
+    g_rope[j * HP + p] = acc_rope;
     if (tid < SG2_COMP_GROUPS * 16) {
-        atomicAdd(&g_comp[tid * 3 + 0], acc_c0);
-        atomicAdd(&g_comp[tid * 3 + 1], acc_c1);
-        atomicAdd(&g_comp[tid * 3 + 2], acc_c2);
+        g_comp[tid * 3 + 0] = acc_c0;
+        g_comp[tid * 3 + 1] = acc_c1;
+        g_comp[tid * 3 + 2] = acc_c2;
     } else if (tid < SG2_COMP_GROUPS * 16 + DI) {
-        atomicAdd(&g_D[tid - SG2_COMP_GROUPS * 16], acc_D);
+        g_D[tid - SG2_COMP_GROUPS * 16] = acc_D;
     }
-    atomicAdd(&g_wout[tid], acc_wout);
+    g_wout[tid] = acc_wout;
+}
+
+// ---- launch 4: rows of the partials buffer added in a fixed order
+__global__ void k_adj_sum_rows(const float* __restrict__ part, int rows_per_dir, float* __restrict__ out) {
+    const int o = blockIdx.x * blockDim.x + threadIdx.x;
+    if (o >= 2 * SG2_BWD_STRIDE) return;
+    const int dir = o / SG2_BWD_STRIDE, e = o % SG2_BWD_STRIDE;
+    float acc = 0.0f;
+    for (int r = 0; r < rows_per_dir; r++) acc += part[((size_t)dir * rows_per_dir + r) * SG2_BWD_STRIDE + e];
+    out[o] = acc;
 }
 
 __global__ void k_fill_zero(float* p, int n) {
@@ -281,11 +416,20 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
             raised[dev] = true;
         }
     }
-    hipLaunchKernelGGL(k_fill_zero, dim3(8), dim3(256), 0, st, grads_out, 2 * SG2_BWD_STRIDE);
-    SG_LAUNCH_CHECK("k_fill_zero");
-    if (pl.total == 0) return 0;
-    hipLaunchKernelGGL(k_bilevel_backward, dim3(2 * pl.P), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, d_ctx, grads_out);
+    if (pl.total == 0) {
+        hipLaunchKernelGGL(k_fill_zero, dim3(8), dim3(256), 0, st, grads_out, 2 * SG2_BWD_STRIDE);
+        SG_LAUNCH_CHECK("k_fill_zero");
+        return 0;
+    }
+    const int groups = pl.chunks < ADJ_GROUPS ? pl.chunks : ADJ_GROUPS;
+    hipLaunchKernelGGL(k_adj_summary, dim3(pl.chunks, 2), dim3(SCAN_THREADS), 0, st, pl, d_ctx);
+    SG_LAUNCH_CHECK("k_adj_summary");
+    hipLaunchKernelGGL(k_adj_prefix, dim3(pl.P, 2), dim3(SCAN_THREADS), 0, st, pl);
+    SG_LAUNCH_CHECK("k_adj_prefix");
+    hipLaunchKernelGGL(k_bilevel_backward, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, d_ctx);
     SG_LAUNCH_CHECK("k_bilevel_backward");
+    hipLaunchKernelGGL(k_adj_sum_rows, dim3((2 * SG2_BWD_STRIDE + 255) / 256), dim3(256), 0, st, pl.adj_part, groups, grads_out);
+    SG_LAUNCH_CHECK("k_adj_sum_rows");
     return 0;
 }
 

@@ -11,13 +11,16 @@
 // One lane per element, persistent grid over tiles of 256 elements.  Nothing is kept between forward and backward:
 // a lane holds its element's activations in registers, and the routing of a head is differentiated before the
 // next head is evaluated.  Weight gradients are sums over elements:
-//   * experts and product keys (rows chosen per element): float atomics on accumulators in LDS;
+//   * product keys (rows chosen per element): float atomics on accumulators in LDS;
+//   * experts (16 per element and head, chosen per element): gathered, not scattered.  Each lane owns nine
+//     (expert, hidden unit) pairs with their sums in registers and walks the tile's elements, whose routing
+//     weights of the head every lane has left in LDS as two 12-vectors (see the expert-gradient pass);
 //   * GRU and query matrices (dense outer products d (x) x): every lane leaves its d (44 values) and x (31 values)
 //     in LDS, then each lane of the workgroup owns up to four matrix entries and sums their products over the
 //     256 elements of the tile, keeping the running sums in registers for the life of the workgroup.
 // Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
-// order.  (Within a workgroup the LDS atomics arrive in no fixed order, so expert and key gradients can differ
-// in the last bits between runs.)
+// order.  (Within a workgroup the LDS atomics arrive in no fixed order, so the key gradients can differ in the last
+// bits between runs; everything else is summed in a fixed order.)
 #include "sg2_internal.hpp"
 
 namespace sg2 {
@@ -26,6 +29,9 @@ namespace {
 constexpr int BE_THREADS = 256;
 constexpr int EXP_STRIDE = 52;          // floats per expert record in LDS: W1[16] b1[16] W2[16] b2 + pad
 constexpr int TOPK = 4;
+constexpr int RW = 2 * PK + 1;          // staged routing row of a head: first-index weights[12] (times d loss/d head), second-index weights[12], mask of first indices
+constexpr int EXP_PER_LANE = NE * EH / BE_THREADS;     // (expert, hidden unit) pairs a lane accumulates
+static_assert(NE * EH % BE_THREADS == 0 && PK % 4 == 0, "expert pairs per lane");
 constexpr int XW = 31, DW = 45;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
 // x row: g, s, fwd ctx[8], bwd ctx[8], h_old[4], r*h_old[4], h_new[4], 1
 constexpr int X_G = 0, X_S = 1, X_CF = 2, X_CB = 10, X_H = 18, X_RH = 22, X_HN = 26, X_ONE = 30;
@@ -66,10 +72,10 @@ struct ElemArgs {
 __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* s_exp = lds;                                   // [NE][EXP_STRIDE] weights
-    float* s_gexp = s_exp + NE * EXP_STRIDE;              // [NE][EXP_STRIDE] gradients, same layout
-    float* s_gkey = s_gexp + NE * EXP_STRIDE;             // [2][NH][PK][DM/2]
+    float* s_gkey = s_exp + NE * EXP_STRIDE;              // [2][NH][PK][DM/2]
     float* s_x = s_gkey + 2 * NH * PK * (DM / 2);         // [256][XW]
     float* s_d = s_x + BE_THREADS * XW;                   // [256][DW]
+    float* s_rt = s_d + BE_THREADS * DW;                  // [256][RW]
 
     const int tid = threadIdx.x;
     {
@@ -77,7 +83,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         const float* __restrict__ B1 = a.W.w[W_EXP_B1];
         const float* __restrict__ W2 = a.W.w[W_EXP_W2];
         const float* __restrict__ B2 = a.W.w[W_EXP_B2];
-        for (int i = tid; i < NE * EXP_STRIDE; i += BE_THREADS) { s_gexp[i] = 0.0f; s_exp[i] = 0.0f; }
+        for (int i = tid; i < NE * EXP_STRIDE; i += BE_THREADS) s_exp[i] = 0.0f;
         for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) s_gkey[i] = 0.0f;
         __syncthreads();
         for (int i = tid; i < NE * EH; i += BE_THREADS) {
@@ -105,14 +111,35 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         if (o < N_DENSE) dense_entry(o, &dcol[q], &xcol[q]);
     }
 
+    // the lane's (expert, hidden unit) pairs: wave w owns the experts with first sub-key index 3w .. 3w+2; for first
+    // index 3w + r, round c covers second indices 4c .. 4c+3 (one per 16 lanes) x 16 hidden units.  Per pair: the
+    // expert's W1, b1 entry and three sums over elements of t = (routing weight if the unit is active else 0):
+    // sum t, sum t*g, sum t*pre, from which d b1 = W2*sum t, d W1 = W2*sum t*g, d W2 = sum t*pre.
+    constexpr int KA_PER_WAVE = PK / 4, ROUNDS = PK / 4;
+    static_assert(KA_PER_WAVE * ROUNDS == EXP_PER_LANE, "pairs per lane");
+    const int ka0 = __builtin_amdgcn_readfirstlane(KA_PER_WAVE * (tid >> 6));
+    const int kb_sub = (tid & 63) >> 4;
+    float ew1[EXP_PER_LANE], eb1[EXP_PER_LANE];
+    float st0[EXP_PER_LANE], st1[EXP_PER_LANE], stp[EXP_PER_LANE], sdo[EXP_PER_LANE];
+#pragma unroll
+    for (int q = 0; q < EXP_PER_LANE; q++) {
+        const int e = (ka0 + q / ROUNDS) * PK + 4 * (q % ROUNDS) + kb_sub, m = tid & (EH - 1);
+        ew1[q] = s_exp[e * EXP_STRIDE + m]; eb1[q] = s_exp[e * EXP_STRIDE + EH + m];
+        st0[q] = st1[q] = stp[q] = sdo[q] = 0.0f;
+    }
+
     const int tiles = (a.total + BE_THREADS - 1) / BE_THREADS;
     const float kscale = a.rescale / (float)NH;
     for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-        const int i = tile * BE_THREADS + tid;
+        // every lane runs the element code (the passes over the tile need whole workgroups): lanes past the end redo
+        // the last element with a zero cotangent, which zeroes everything they add, and store nothing
+        const bool valid = tile * BE_THREADS + tid < a.total;
+        const int i = valid ? tile * BE_THREADS + tid : a.total - 1;
         float* xrow = s_x + tid * XW;
         float* drow = s_d + tid * DW;
-        if (i < a.total) {
-            const float g = a.g[i], s = a.s[i], cot = a.cot[i];
+        float* rtrow = s_rt + tid * RW;
+        {
+            const float g = a.g[i], s = a.s[i], cot = valid ? a.cot[i] : 0.0f;
             float cf[DM], cb[DM], h[GH];
             {
                 const float4* pf = reinterpret_cast<const float4*>(a.ctx + (size_t)i * DM);
@@ -219,7 +246,19 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 #pragma unroll
                     for (int k = 0; k < TOPK; k++) wgt[hf][k] *= inv;
                 }
-                // experts: out, and the gradients of their weights
+                // experts: outputs per lane; their weight gradients in the pass below, from the staged routing weights
+#pragma unroll
+                for (int k = 0; k < 2 * PK; k++) rtrow[k] = 0.0f;
+                {
+                    int mask = 0;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) {
+                        rtrow[idx[0][k]] = kk * wgt[0][k];
+                        rtrow[PK + idx[1][k]] = wgt[1][k];
+                        mask |= 1 << idx[0][k];
+                    }
+                    rtrow[2 * PK] = __int_as_float(kk != 0.0f ? mask : 0);
+                }
                 float ra[TOPK] = {0.f, 0.f, 0.f, 0.f}, rb[TOPK] = {0.f, 0.f, 0.f, 0.f};
                 float head_out = 0.0f;
 #pragma unroll 1
@@ -233,27 +272,63 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     int e = ea * PK + eb;
                     if (e >= NE) e = NE - 1;
                     const float* rec = s_exp + e * EXP_STRIDE;
-                    float* grec = s_gexp + e * EXP_STRIDE;
-                    const float dout = kk * wa * wb;
                     float out = rec[3 * EH];
 #pragma unroll
-                    for (int m = 0; m < EH; m++) {
-                        const float pre = sg_fma(rec[m], g, rec[EH + m]);
-                        if (pre > 0.0f) {
-                            const float w2 = rec[2 * EH + m];
-                            out = sg_fma(w2, pre, out);
-                            const float dpre = dout * w2;
-                            atomicAdd(&grec[2 * EH + m], dout * pre);
-                            atomicAdd(&grec[m], dpre * g);
-                            atomicAdd(&grec[EH + m], dpre);
-                        }
-                    }
-                    atomicAdd(&grec[3 * EH], dout);
+                    for (int m = 0; m < EH; m++) out = sg_fma(rec[2 * EH + m], sg_max(sg_fma(rec[m], g, rec[EH + m]), 0.0f), out);
                     head_out = sg_fma(wa * wb, out, head_out);
                     const float oa = wb * out, ob = wa * out;
                     ra[0] += ia == 0 ? oa : 0.0f; ra[1] += ia == 1 ? oa : 0.0f; ra[2] += ia == 2 ? oa : 0.0f; ra[3] += ia == 3 ? oa : 0.0f;
                     rb[0] += ib == 0 ? ob : 0.0f; rb[1] += ib == 1 ? ob : 0.0f; rb[2] += ib == 2 ? ob : 0.0f; rb[3] += ib == 3 ? ob : 0.0f;
                 }
+                // Expert gradients.  The weight an element gives expert (ka, kb) of this head is the product
+                // (d loss/d head * wa)[ka] * wb[kb] of two 12-vectors with four non-zeros each, which every lane has
+                // just staged.  Scattering the 16 x 49 contributions of an element with LDS float atomics is far too
+                // slow (they retire about one lane per clock), and neighbours in element order share no routing, so
+                // the sums are gathered instead: a lane owns nine fixed (expert, hidden unit) pairs, keeps their sums
+                // in registers, and walks the tile's 256 elements.  A wave's pairs belong to three first indices:
+                // those the element did not pick are skipped with a scalar branch on the element's staged mask.
+                __syncthreads();
+                {
+                    // an element's staged values are fetched one element ahead of their use (two register sets)
+                    struct Staged { float a[KA_PER_WAVE], b[ROUNDS], g, mask; };
+                    auto fetch = [&](int el, Staged& v) {
+                        const float* row = s_rt + el * RW;
+                        v.mask = row[2 * PK];
+                        v.g = s_x[el * XW + X_G];
+#pragma unroll
+                        for (int r = 0; r < KA_PER_WAVE; r++) v.a[r] = row[ka0 + r];
+#pragma unroll
+                        for (int c = 0; c < ROUNDS; c++) v.b[c] = row[PK + 4 * c + kb_sub];
+                    };
+                    auto add = [&](const Staged& v) {
+                        const int mask = __builtin_amdgcn_readfirstlane(__float_as_int(v.mask)) >> ka0;
+#pragma unroll
+                        for (int r = 0; r < KA_PER_WAVE; r++) {
+                            if (((mask >> r) & 1) == 0) continue;          // scalar: the element did not pick this first index
+#pragma unroll
+                            for (int c = 0; c < ROUNDS; c++) {
+                                const int q = r * ROUNDS + c;
+                                const float dout = v.a[r] * v.b[c];
+                                const float pre = sg_fma(ew1[q], v.g, eb1[q]);
+                                const float t = pre > 0.0f ? dout : 0.0f;
+                                st0[q] += t;
+                                st1[q] = sg_fma(t, v.g, st1[q]);
+                                stp[q] = sg_fma(t, pre, stp[q]);
+                                sdo[q] += dout;
+                            }
+                        }
+                    };
+                    Staged v0, v1;
+                    fetch(0, v0);
+#pragma unroll 1
+                    for (int el = 0; el < BE_THREADS; el += 2) {
+                        fetch(el + 1, v1);
+                        add(v0);
+                        fetch(el + 2 < BE_THREADS ? el + 2 : el, v0);
+                        add(v1);
+                    }
+                }
+                __syncthreads();
                 total += head_out;
                 // routing backward: softmax, scores, keys, query
                 float dq[DM];
@@ -289,7 +364,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     for (int q = 0; q < DM; q++) dcb[q] = sg_fma(qr[GH + DM + q], dq[dd], dcb[q]);
                 }
             }
-            if (a.smart != nullptr) a.smart[i] = sg_fma(a.rescale, total / (float)NH, g);
+            if (valid && a.smart != nullptr) a.smart[i] = sg_fma(a.rescale, total / (float)NH, g);
 
             // ---- GRU backward
             float dpz[GH], dpr[GH], dph[GH], drh[GH] = {0.f, 0.f, 0.f, 0.f};
@@ -319,15 +394,12 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             }
 #pragma unroll
             for (int j = 0; j < GH; j++) { drow[D_Z + j] = dpz[j]; drow[D_R + j] = dpr[j]; drow[D_H + j] = dph[j]; }
-            {
+            if (valid) {
                 float4* of = reinterpret_cast<float4*>(a.d_ctx + (size_t)i * DM);
                 float4* ob = reinterpret_cast<float4*>(a.d_ctx + ((size_t)a.total + i) * DM);
                 of[0] = make_float4(dcf[0], dcf[1], dcf[2], dcf[3]); of[1] = make_float4(dcf[4], dcf[5], dcf[6], dcf[7]);
                 ob[0] = make_float4(dcb[0], dcb[1], dcb[2], dcb[3]); ob[1] = make_float4(dcb[4], dcb[5], dcb[6], dcb[7]);
             }
-        } else {
-            for (int q = 0; q < XW; q++) xrow[q] = 0.0f;
-            for (int q = 0; q < DW; q++) drow[q] = 0.0f;
         }
         __syncthreads();
         // ---- dense gradients: each lane's entries, summed over the tile's elements
@@ -346,13 +418,15 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         if (o < N_DENSE) out[o] = dense[q];
     }
     for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) out[OFF_KA + i] = s_gkey[i];
-    for (int i = tid; i < NE * EH; i += BE_THREADS) {
-        const int e = i / EH, k = i % EH;
-        out[OFF_W1 + i] = s_gexp[e * EXP_STRIDE + k];
-        out[OFF_B1 + i] = s_gexp[e * EXP_STRIDE + EH + k];
-        out[OFF_W2 + i] = s_gexp[e * EXP_STRIDE + 2 * EH + k];
+#pragma unroll
+    for (int q = 0; q < EXP_PER_LANE; q++) {
+        const int e = (ka0 + q / ROUNDS) * PK + 4 * (q % ROUNDS) + kb_sub, m = tid & (EH - 1);
+        const float w2 = s_exp[e * EXP_STRIDE + 2 * EH + m];
+        out[OFF_W1 + e * EH + m] = w2 * st1[q];
+        out[OFF_B1 + e * EH + m] = w2 * st0[q];
+        out[OFF_W2 + e * EH + m] = stp[q];
+        if (m == 0) out[OFF_B2 + e] = sdo[q];
     }
-    for (int i = tid; i < NE; i += BE_THREADS) out[OFF_B2 + i] = s_gexp[i * EXP_STRIDE + 3 * EH];
 }
 
 __global__ void k_sum_partials(const float* __restrict__ partials, int rows, float* __restrict__ out) {
@@ -363,7 +437,8 @@ __global__ void k_sum_partials(const float* __restrict__ partials, int rows, flo
     out[o] = acc;
 }
 
-constexpr int BE_LDS_BYTES = 4 * (2 * NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW));
+constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW));
+static_assert(BE_LDS_BYTES <= 160 * 1024, "LDS of k_bilevel_elem");
 constexpr int BE_MAX_GROUPS = 512;
 
 int elem_groups(int64_t total) {
