@@ -25,7 +25,8 @@
 //   4  the adjoint recurrence over the steps in reverse: lambda <- R(theta)^T diag(A_bar) (lambda + d y C), with
 //      the gradients of dt, x-branch, B and C per step (reduced over pairs / columns) and of A_log and the RoPE
 //      frequencies per lane;
-//   5  sums over the tile's steps: composed-coefficient gradients d v (x) (g, s, 1), d D, d out_proj.
+//   5  sums over the tile's steps: composed-coefficient gradients d v (x) (g, s, 1) of x-branch, z and dt (those of B
+//      and C are summed per lane during 4 and reduced over columns once per workgroup), d D, d out_proj.
 // Nothing is truncated: the result is the exact adjoint.  Gradients of the composed coefficients are mapped back
 // to input_proj / in_proj / dt_proj / B_proj / C_proj by the caller (the composition is a handful of small matrix
 // products).  Every workgroup keeps its sums in registers over the chunks it handles and writes them to its own
@@ -39,22 +40,27 @@ namespace {
 constexpr int BST = SCAN_TT + 4;                 // row stride of the [16][64] LDS arrays
 constexpr int ROWS = 16;
 // LDS arrays of ROWS x BST floats
-enum { A_DT, A_DSP, A_XB, A_B, A_C, A_GATE, A_DGATE, A_Y, A_DY, A_DZ, A_DXB, A_DDT, A_DB0, A_DB1, A_DC0, A_DC1, A_COUNT };
+enum { A_DT, A_DSP, A_XB, A_B, A_C, A_GATE, A_DGATE, A_Y, A_DY, A_DZ, A_DXB, A_DDT, A_COUNT };
 constexpr int LDS_ROWS_FLOATS = A_COUNT * ROWS * BST;
 constexpr int LDS_H_FLOATS = SCAN_TT * SCAN_THREADS * 2;          // state after every step of the tile
 constexpr int LDS_MISC_FLOATS = SCAN_TT * DM + SCAN_TT * 2;       // d ctx tile, (g, s) of the tile
 constexpr int BILEVEL_LDS_BYTES = 4 * (LDS_ROWS_FLOATS + LDS_H_FLOATS + LDS_MISC_FLOATS);
 
+// value of the lane whose index differs in one bit, by DPP where the pattern stays inside a row of 16 lanes
+template <int CTRL>
+__device__ __forceinline__ float dpp_get(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
 __device__ __forceinline__ float xor_sum_columns(float v) {      // sum over the 8 columns of a wave (lanes 8 apart)
-    v += __shfl_xor(v, 8, 64);
+    v += dpp_get<0x128>(v);              // row_ror:8 = lane ^ 8
     v += __shfl_xor(v, 16, 64);
     v += __shfl_xor(v, 32, 64);
     return v;
 }
 __device__ __forceinline__ float pair_sum(float v) {             // sum over the 8 pairs of a column (adjacent lanes)
-    v += __shfl_xor(v, 1, 64);
-    v += __shfl_xor(v, 2, 64);
-    v += __shfl_xor(v, 4, 64);
+    v += dpp_get<0xB1>(v);               // quad_perm [1,0,3,2] = lane ^ 1
+    v += dpp_get<0x4E>(v);               // quad_perm [2,3,0,1] = lane ^ 2
+    v += dpp_get<0x141>(v);              // row_half_mirror: lane 7-i of the 8; every quad already holds its sum
     return v;
 }
 
@@ -207,6 +213,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
 
     float acc_alog_e = 0.0f, acc_alog_o = 0.0f, acc_rope = 0.0f;
     float acc_c0 = 0.0f, acc_c1 = 0.0f, acc_c2 = 0.0f, acc_D = 0.0f, acc_wout = 0.0f;
+    float acc_bc[12];                 // this lane's column share of d B[2p], d B[2p+1], d C[2p], d C[2p+1] against (g, s, 1)
+#pragma unroll
+    for (int q = 0; q < 12; q++) acc_bc[q] = 0.0f;
 
   for (int chunk = blockIdx.x; chunk < pl.chunks; chunk += gridDim.x) {
     const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
@@ -283,10 +292,6 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             arr(A_GATE)[r * BST + tu] = valid ? sg_fma(y, gate, Dw[r] * xb) : 0.0f;     // out, for d out_proj
             arr(A_DGATE)[r * BST + tu] = valid ? dout : 0.0f;                           // d out, for d D
             arr(A_DDT)[r * BST + tu] = 0.0f;
-            arr(A_DB0)[r * BST + tu] = 0.0f;
-            arr(A_DB1)[r * BST + tu] = 0.0f;
-            arr(A_DC0)[r * BST + tu] = 0.0f;
-            arr(A_DC1)[r * BST + tu] = 0.0f;
         }
         __syncthreads();
 
@@ -304,7 +309,15 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             // y = sum h C
             le = sg_fma(dy, Ce, le);
             lo = sg_fma(dy, Co, lo);
-            const float dCe = xor_sum_columns(dy * he), dCo = xor_sum_columns(dy * ho);
+            // d C[2p], d C[2p+1] of this step are sums over the columns of dy*h, d B of lambda*dt*xb; what is wanted
+            // is their sum over steps against (g, s, 1), so each lane sums its own column's share over the steps
+            // and the columns are added once, when the workgroup is done
+            const float gk = s_gs[2 * k], sk = s_gs[2 * k + 1];
+            {
+                const float te = dy * he, to = dy * ho;
+                acc_bc[6] = sg_fma(te, gk, acc_bc[6]); acc_bc[7] = sg_fma(te, sk, acc_bc[7]); acc_bc[8] += te;
+                acc_bc[9] = sg_fma(to, gk, acc_bc[9]); acc_bc[10] = sg_fma(to, sk, acc_bc[10]); acc_bc[11] += to;
+            }
             // h' = A_bar * rot(h) + dt * xb * B
             const float re = sg_fma(pe, cs, -(po * sn)), ro = sg_fma(po, cs, pe * sn);
             // A_bar = 2/d - 1, d = 1 + dt*a: dA_bar/dd = -2/d^2 = -(A_bar+1)^2/2
@@ -320,19 +333,15 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             const float qb = sg_fma(le, Be, lo * Bo);
             ddt = sg_fma(qb, xb, ddt);
             const float ux = dt * xb;
-            const float dBe = xor_sum_columns(le * ux), dBo = xor_sum_columns(lo * ux);
+            {
+                const float te = le * ux, to = lo * ux;
+                acc_bc[0] = sg_fma(te, gk, acc_bc[0]); acc_bc[1] = sg_fma(te, sk, acc_bc[1]); acc_bc[2] += te;
+                acc_bc[3] = sg_fma(to, gk, acc_bc[3]); acc_bc[4] = sg_fma(to, sk, acc_bc[4]); acc_bc[5] += to;
+            }
             const float ddt_j = pair_sum(ddt), dxb_j = pair_sum(qb * dt);
             if (p == 0) {
                 arr(A_DDT)[j * BST + k] = ddt_j * arr(A_DSP)[j * BST + k];
                 arr(A_DXB)[j * BST + k] += dxb_j;
-            }
-            if ((tid & 63) < 8) {        // column 0 of the wave holds the wave's sums for pair p
-                float* db = arr(w ? A_DB1 : A_DB0);
-                float* dc = arr(w ? A_DC1 : A_DC0);
-                db[(2 * p) * BST + k] = dBe;
-                db[(2 * p + 1) * BST + k] = dBo;
-                dc[(2 * p) * BST + k] = dCe;
-                dc[(2 * p + 1) * BST + k] = dCo;
             }
             // lambda for the previous step
             const float nle = sg_fma(dre, cs, dro * sn), nlo = sg_fma(dro, cs, -(dre * sn));
@@ -341,27 +350,28 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         }
         __syncthreads();
 
-        // ---- 5: sums over the tile's steps
-        if (tid < SG2_COMP_GROUPS * 16) {
+        // ---- 5: sums over the tile's steps (steps past the end of the chunk hold zeros in every array read here)
+        if (tid < 3 * 16) {              // x-branch, z, dt (the first three coefficient groups)
             const int group = tid / 16, r = tid % 16;
-            for (int k = 0; k < cnt; k++) {
+#pragma unroll 8
+            for (int k = 0; k < SCAN_TT; k++) {
                 float dv;
                 if (group == SG2_COMP_XB) dv = arr(A_DXB)[r * BST + k];
                 else if (group == SG2_COMP_Z) dv = arr(A_DZ)[r * BST + k];
-                else if (group == SG2_COMP_DT) dv = arr(A_DDT)[r * BST + k];
-                else if (group == SG2_COMP_B) dv = arr(A_DB0)[r * BST + k] + arr(A_DB1)[r * BST + k];
-                else dv = arr(A_DC0)[r * BST + k] + arr(A_DC1)[r * BST + k];
+                else dv = arr(A_DDT)[r * BST + k];
                 acc_c0 = sg_fma(dv, s_gs[2 * k], acc_c0);
                 acc_c1 = sg_fma(dv, s_gs[2 * k + 1], acc_c1);
                 acc_c2 += dv;
             }
         } else if (tid < SG2_COMP_GROUPS * 16 + DI) {
             const int r = tid - SG2_COMP_GROUPS * 16;
-            for (int k = 0; k < cnt; k++) acc_D = sg_fma(arr(A_DGATE)[r * BST + k], arr(A_XB)[r * BST + k], acc_D);
+#pragma unroll 8
+            for (int k = 0; k < SCAN_TT; k++) acc_D = sg_fma(arr(A_DGATE)[r * BST + k], arr(A_XB)[r * BST + k], acc_D);
         }
         {
             const int d = tid >> 4, r = tid & 15;       // out_proj[d][r]
-            for (int k = 0; k < cnt; k++) acc_wout = sg_fma(s_dctx[k * DM + d], arr(A_GATE)[r * BST + k], acc_wout);
+#pragma unroll 8
+            for (int k = 0; k < SCAN_TT; k++) acc_wout = sg_fma(s_dctx[k * DM + d], arr(A_GATE)[r * BST + k], acc_wout);
         }
         __syncthreads();
     }
@@ -376,10 +386,24 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     g_alog[j * DS + 2 * p] = acc_alog_e;
     g_alog[j * DS + 2 * p + 1] = acc_alog_o;
     g_rope[j * HP + p] = acc_rope;
-    if (tid < SG2_COMP_GROUPS * 16) {
+    // B and C coefficient gradients: columns added within the wave, then the two waves through LDS
+#pragma unroll
+    for (int q = 0; q < 12; q++) acc_bc[q] = xor_sum_columns(acc_bc[q]);
+    __syncthreads();
+    if ((tid & 63) < 8) {             // column 0 of each wave holds the wave's sums for pair p
+#pragma unroll
+        for (int q = 0; q < 12; q++) lds[(w * 8 + p) * 12 + q] = acc_bc[q];
+    }
+    __syncthreads();
+    if (tid < 3 * 16) {
         g_comp[tid * 3 + 0] = acc_c0;
         g_comp[tid * 3 + 1] = acc_c1;
         g_comp[tid * 3 + 2] = acc_c2;
+    } else if (tid < SG2_COMP_GROUPS * 16) {
+        const int group = tid / 16, r = tid % 16;            // B: group 3, C: group 4; row r = 2*pair + (odd)
+        const int q0 = (group == SG2_COMP_C ? 6 : 0) + (r & 1) * 3;
+#pragma unroll
+        for (int c = 0; c < 3; c++) g_comp[tid * 3 + c] = lds[(r >> 1) * 12 + q0 + c] + lds[(8 + (r >> 1)) * 12 + q0 + c];
     } else if (tid < SG2_COMP_GROUPS * 16 + DI) {
         g_D[tid - SG2_COMP_GROUPS * 16] = acc_D;
     }
