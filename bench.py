@@ -129,6 +129,26 @@ def bench_other(args, dev):
                                             [0.9 * 0.9 ** i for i in range(P)], W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8,
                                             2.0, 1.0, 0.5, 1.0)
             name = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip), 14 tensors, %d elements" % n
+        elif args.workload == "bilevel":
+            # gradient of sum <smart_grad, cotangent> with respect to every weight of the v2 meta-net, for all tensors
+            # of the model at once: sort + scan forward, per-element forward/backward, scan adjoint, all in HIP
+            from grokking_optimizers import Mamba3PEERMetaNet, _bilevel
+            torch.manual_seed(0)
+            mn = Mamba3PEERMetaNet().to(dev)
+            sharps = [g.abs() * 0.5 for g in grads0]
+            grus = [torch.zeros(g.numel(), 4, device=dev) for g in grads0]
+            mf = [torch.zeros(16, 16, device=dev) for _ in grads0]
+            mb = [torch.zeros(16, 16, device=dev) for _ in grads0]
+            gen = torch.Generator().manual_seed(5)
+            cots = [torch.randn(g.numel(), generator=gen).to(dev) for g in grads0]
+
+            def step():
+                mn.zero_grad()
+                _bilevel.accumulate_meta_gradients(mn, grads0, sharps, grus, mf, mb, cots)
+            # per element: grad, sharpness, cotangent, GRU state read (28 B); both contexts written by the scan and read
+            # by the per-element pass, their gradients written by it and read by the adjoint (4 x 64 B)
+            bytes_per_elem = 284
+            name = "SuperGrok v2 bilevel meta-gradient pass (sort + scan, per-element forward/backward, scan adjoint), 14 tensors, %d elements" % n
         else:
             # the other fused steps, on the 50-tensor / 25 M-element set so that HBM traffic, not launch latency, is measured
             shapes = wl.scale50_shapes()
@@ -204,7 +224,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--sharpness", action="store_true", help="v2 workloads: non-zero sharpness cache (as after a SAM probe)")
-    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11"],
+    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11", "bilevel"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
