@@ -24,9 +24,15 @@
 //                  D skip, out_proj, and the 8-float context written straight
 //                  to the element's original position (the "unsort").  The
 //                  last chunk stores the new carried state.
-// Per-timestep projections (in_proj, dt, B, C) are recomputed in both passes
-// for tiles of 64 timesteps and staged through LDS instead of being
-// materialised in HBM (the reference writes 320 B per element per direction).
+//   k_compose      runs first: the input of a timestep is two numbers (g, s)
+//                  and every projection of the block is linear in their 8-float
+//                  input projection, so input_proj, in_proj, dt_proj, B_proj and
+//                  C_proj are folded into 5 x 16 coefficient triples per
+//                  direction (include/sg2_compose.h).
+// Per-timestep projections (x-branch, z, dt, B, C) are evaluated from those
+// triples in both passes for tiles of 64 timesteps and staged through LDS
+// instead of being materialised in HBM (the reference writes 320 B per
+// element per direction).
 // The inputs of a timestep come coalesced from the sort's own output: the key
 // is |g|, the payload carries the sign of g and the element index, and the
 // sharpness has been gathered into sorted order once.
@@ -36,9 +42,15 @@
 // recurrence loop therefore works on blocks of 8 timesteps: all LDS operands of
 // the block are fetched first, the state-independent coefficients of the 8
 // steps are computed as independent instruction streams, and only the short
-// h-update chain is serial.  When every lane of the wave holds a small
-// rotation angle the sin/cos range reduction is skipped (bit-identical
-// results, see sg_sincos_small).
+// h-update chain is serial.  The A_bar denominators of a lane's 8 steps are
+// inverted together (one division per block, sg_abar_block_*).  When every
+// lane of the wave holds a small rotation angle the sin/cos range reduction is
+// skipped (bit-identical results, see sg_sincos_small); when every angle of
+// the block is below 0.3 a shorter polynomial pair is used (sg_sincos_tiny,
+// not bit-identical to the general form: the choice depends on the angles only
+// and the CPU checker makes the same one).
+// For the bilevel pass k_scan<true> also stores the state entering every
+// 64-step tile (Plan::htile), which the adjoint kernels restart from.
 #include "sg2_internal.hpp"
 #include "../../include/sg2_compose.h"
 

@@ -1,7 +1,10 @@
 // C-ABI entry points of the SuperGrok v2 batched step: validation, workspace
 // carving, the small per-call table upload and the launch sequence
-//   keys -> 4 radix passes -> chunk summaries -> chunk prefix -> scan output
-//   -> per-element GRU/PEER/expert/Adam.
+//   keys -> 4 radix passes -> sharpness gather -> coefficient composition
+//   -> chunk summaries -> chunk prefix -> scan output
+//   -> per-element GRU/PEER/expert/Adam,
+// and of the scan part of the bilevel pass (the same sort + scan with the
+// tile-start states kept, and its adjoint).
 // Stands behind supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877 of
 // the reference) in place of launch_mamba3_peer_batched_step
 // (csrc/supergrok2_mamba_peer_kernels.cu:1754-2117).
