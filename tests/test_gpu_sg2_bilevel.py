@@ -93,6 +93,12 @@ def test_zero_sharpness_and_zero_states():
     _case([(200,), (64,), (65,)], seed=12, sharp=False, state_std=0.0)
 
 
+def test_automatic_chunk_length_on_longer_tensors():
+    """5000 + 3000 elements at the chunk length the library picks by itself (several chunks per tensor, partial last
+    tiles): the chunk-parallel adjoint (summaries, prefix, replay) against float64 autograd."""
+    _case([(5000,), (3000,)], seed=14, sharp=True, state_std=0.3)
+
+
 def test_several_chunks():
     """Chunk length 64: the forward pass runs summaries, chunk prefix and replay; the adjoint crosses chunk borders."""
     _case([(1000,), (257,), (640,)], seed=13, sharp=True, state_std=0.3, chunk_len=64)
