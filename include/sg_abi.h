@@ -240,14 +240,14 @@ int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, vo
  * are OVERWRITTEN with the end-of-sequence states, so pass copies.
  *
  * sg2_bilevel_backward: same tensors and the SAME, untouched workspace; d_ctx
- * has ctx_out's layout.  grads_out receives, per direction (forward first,
- * SG2_BWD_STRIDE floats each):
- *   [5][16][3]  composed projection coefficients (include/sg2_compose.h order)
- *   [16][16]    A_log      [16][8] rope_freq      [16] D      [8][16] out_proj
- * The caller maps the coefficient gradients back through the composition.
- * A tensor is walked serially by one workgroup per direction (exact adjoint,
- * no truncation). */
-#define SG2_BWD_STRIDE 768
+ * has ctx_out's layout.  grads_out receives SG2_SCAN_GRAD_FLOATS floats, the
+ * gradients of the 20 scan weights in the order of Sg2Weights:
+ *   input_proj W [8][2], b [8]; then for the forward and the backward block
+ *   in_proj [32][8], dt_proj W [16][16], b [16], B_proj [16][16], C_proj
+ *   [16][16], A_log [16][16], D [16], rope_freq [16][8], out_proj [8][16].
+ * The adjoint is exact (no truncation window); sums over elements are formed in
+ * a fixed order, so the result is reproducible run to run. */
+#define SG2_SCAN_GRAD_FLOATS 3160
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
 int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
                         float* ctx_out, void* workspace, size_t workspace_bytes, void* stream);

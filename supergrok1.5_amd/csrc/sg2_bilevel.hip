@@ -27,9 +27,9 @@
 //      frequencies per lane;
 //   5  sums over the tile's steps: composed-coefficient gradients d v (x) (g, s, 1) of x-branch, z and dt (those of B
 //      and C are summed per lane during 4 and reduced over columns once per workgroup), d D, d out_proj.
-// Nothing is truncated: the result is the exact adjoint.  Gradients of the composed coefficients are mapped back
-// to input_proj / in_proj / dt_proj / B_proj / C_proj by the caller (the composition is a handful of small matrix
-// products).  Every workgroup keeps its sums in registers over the chunks it handles and writes them to its own
+// Nothing is truncated: the result is the exact adjoint.  Gradients of the composed coefficients are carried back
+// to input_proj / in_proj / dt_proj / B_proj / C_proj by a last one-workgroup kernel (k_compose_backward, the
+// transpose of the composition).  Every workgroup keeps its sums in registers over the chunks it handles and writes them to its own
 // row of a partials buffer, which k_adj_sum_rows adds in a fixed order: the result is reproducible run to run.
 #include "sg2_internal.hpp"
 #include "../../include/sg2_compose.h"
@@ -420,6 +420,84 @@ __global__ void k_adj_sum_rows(const float* __restrict__ part, int rows_per_dir,
     out[o] = acc;
 }
 
+// ---- launch 5: from the gradients of the composed coefficients to those of the weights they were composed from
+// (the transpose of sg2_compose_one), and the final layout: input_proj W [8][2], b [8]; then per direction in_proj
+// [32][8], dt_proj W [16][16], b [16], B_proj [16][16], C_proj [16][16], A_log [16][16], D [16], rope_freq [16][8],
+// out_proj [8][16].  One workgroup; blk is k_adj_sum_rows' output ([2][SG2_BWD_STRIDE]).
+//   src = [W_in | b_in] (8x3);  xb = in_proj[:16] src;  z = in_proj[16:] src;  dt = dt_W xb + [0 0 dt_b];  B = B_proj xb;  C = C_proj xb
+__global__ __launch_bounds__(256) void k_compose_backward(Plan pl, const float* __restrict__ blk, float* __restrict__ out) {
+    static_assert(DM == 8 && DI == 16 && DS == 16 && SG2_COMP_GROUPS == 5, "k_compose_backward: fixed dimensions");
+    __shared__ float s_src[DM][3], s_xb[DI][3], s_d[SG2_COMP_GROUPS][16][3], s_dxb[DI][3];
+    const int tid = threadIdx.x;
+    constexpr int PER_DIR = 2 * DI * DM + DI * DI + DI + 2 * DS * DI + DI * DS + DI + DI * HP + DM * DI;
+    static_assert(2 * DM + DM + 2 * PER_DIR == SG2_SCAN_GRAD_FLOATS, "gradient layout");
+    if (tid < DM * 3) s_src[tid / 3][tid % 3] = (tid % 3 < 2) ? pl.W.w[W_IN_W][(tid / 3) * 2 + tid % 3] : pl.W.w[W_IN_B][tid / 3];
+    float dsrc = 0.0f;                              // thread (d, c) for tid < 24, summed over both directions
+    for (int dir = 0; dir < 2; dir++) {
+        const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+        const float* __restrict__ in_proj = pl.W.w[b];
+        const float* __restrict__ dtW = pl.W.w[b + 1];
+        const float* __restrict__ Bp = pl.W.w[b + 3];
+        const float* __restrict__ Cp = pl.W.w[b + 4];
+        const float* __restrict__ g = blk + dir * SG2_BWD_STRIDE;
+        float* __restrict__ o = out + 3 * DM + dir * PER_DIR;
+        __syncthreads();
+        if (tid < SG2_COMP_GROUPS * 16 * 3) (&s_d[0][0][0])[tid] = g[tid];
+        if (tid < DI * 3) (&s_xb[0][0])[tid] = pl.comp[dir * (SG2_COMP_GROUPS * 16 * 3) + SG2_COMP_XB * 16 * 3 + tid];
+        __syncthreads();
+        {   // dt_W, B_proj, C_proj: d W[r][k] = sum_c d v[r][c] * xb[k][c]
+            const int r = tid >> 4, k = tid & 15;
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 3; c++) {
+                a0 = sg_fma(s_d[SG2_COMP_DT][r][c], s_xb[k][c], a0);
+                a1 = sg_fma(s_d[SG2_COMP_B][r][c], s_xb[k][c], a1);
+                a2 = sg_fma(s_d[SG2_COMP_C][r][c], s_xb[k][c], a2);
+            }
+            o[2 * DI * DM + tid] = a0;
+            o[2 * DI * DM + DI * DI + DI + tid] = a1;
+            o[2 * DI * DM + DI * DI + DI + DS * DI + tid] = a2;
+            if (tid < DI) o[2 * DI * DM + DI * DI + tid] = s_d[SG2_COMP_DT][tid][2];      // dt_b
+        }
+        if (tid < DI * 3) {   // d xb[k][c] = d xb-coefficients + dt_W^T d dt + B_proj^T d B + C_proj^T d C
+            const int k = tid / 3, c = tid % 3;
+            float a = s_d[SG2_COMP_XB][k][c];
+            for (int r = 0; r < 16; r++) {
+                a = sg_fma(dtW[r * DI + k], s_d[SG2_COMP_DT][r][c], a);
+                a = sg_fma(Bp[r * DI + k], s_d[SG2_COMP_B][r][c], a);
+                a = sg_fma(Cp[r * DI + k], s_d[SG2_COMP_C][r][c], a);
+            }
+            s_dxb[k][c] = a;
+        }
+        __syncthreads();
+        {   // in_proj [32][8]: rows 0..15 from d xb, rows 16..31 from d z
+            const int r = tid >> 3, d = tid & 7;
+            float a = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 3; c++) a = sg_fma(r < DI ? s_dxb[r][c] : s_d[SG2_COMP_Z][r - DI][c], s_src[d][c], a);
+            o[tid] = a;
+        }
+        if (tid < DM * 3) {
+            const int d = tid / 3, c = tid % 3;
+            for (int r = 0; r < DI; r++) {
+                dsrc = sg_fma(in_proj[r * DM + d], s_dxb[r][c], dsrc);
+                dsrc = sg_fma(in_proj[(DI + r) * DM + d], s_d[SG2_COMP_Z][r][c], dsrc);
+            }
+        }
+        // A_log, D, rope_freq, out_proj pass through (the block holds them as A_log, rope_freq, D, out_proj)
+        const float* ga = g + SG2_COMP_GROUPS * 16 * 3;
+        float* oa = o + 2 * DI * DM + DI * DI + DI + 2 * DS * DI;
+        oa[tid] = ga[tid];                                                        // A_log [16][16]
+        if (tid < DI) oa[DI * DS + tid] = ga[DI * DS + DI * HP + tid];            // D
+        if (tid < DI * HP) oa[DI * DS + DI + tid] = ga[DI * DS + tid];            // rope_freq
+        if (tid < DM * DI) oa[DI * DS + DI + DI * HP + tid] = ga[DI * DS + DI * HP + DI + tid];   // out_proj
+    }
+    if (tid < DM * 3) {
+        const int d = tid / 3, c = tid % 3;
+        if (c < 2) out[d * 2 + c] = dsrc; else out[2 * DM + d] = dsrc;
+    }
+}
+
 __global__ void k_fill_zero(float* p, int n) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0.0f;
 }
@@ -428,7 +506,7 @@ __global__ void k_fill_zero(float* p, int n) {
 
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st) {
     static_assert(DM * DI == SCAN_THREADS, "one thread per out_proj entry");
-    static_assert(SG2_BWD_STRIDE == SG2_COMP_GROUPS * 16 * 3 + DI * DS + DI * HP + DI + DM * DI, "gradient layout");
+    static_assert(SG2_BWD_STRIDE == SG2_COMP_GROUPS * 16 * 3 + DI * DS + DI * HP + DI + DM * DI, "layout of the per-direction sums");
     {
         static bool raised[64] = {};
         int dev = 0;
@@ -441,7 +519,7 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
         }
     }
     if (pl.total == 0) {
-        hipLaunchKernelGGL(k_fill_zero, dim3(8), dim3(256), 0, st, grads_out, 2 * SG2_BWD_STRIDE);
+        hipLaunchKernelGGL(k_fill_zero, dim3(8), dim3(256), 0, st, grads_out, SG2_SCAN_GRAD_FLOATS);
         SG_LAUNCH_CHECK("k_fill_zero");
         return 0;
     }
@@ -452,8 +530,10 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
     SG_LAUNCH_CHECK("k_adj_prefix");
     hipLaunchKernelGGL(k_bilevel_backward, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, d_ctx);
     SG_LAUNCH_CHECK("k_bilevel_backward");
-    hipLaunchKernelGGL(k_adj_sum_rows, dim3((2 * SG2_BWD_STRIDE + 255) / 256), dim3(256), 0, st, pl.adj_part, groups, grads_out);
+    hipLaunchKernelGGL(k_adj_sum_rows, dim3((2 * SG2_BWD_STRIDE + 255) / 256), dim3(256), 0, st, pl.adj_part, groups, pl.adj_blk);
     SG_LAUNCH_CHECK("k_adj_sum_rows");
+    hipLaunchKernelGGL(k_compose_backward, dim3(1), dim3(256), 0, st, pl, pl.adj_blk, grads_out);
+    SG_LAUNCH_CHECK("k_compose_backward");
     return 0;
 }
 

@@ -79,6 +79,7 @@ struct Plan {
     float* htile;                  // bilevel: [2][tiles][2][128] state at the start of every 64-step tile, or NULL
     float* adj_summ;               // bilevel: [2][chunks][128][6] adjoint transfer map of every chunk
     float* adj_lam;                // bilevel: [2][chunks][128][2] adjoint state arriving at the end of every chunk
+    float* adj_blk;                // bilevel: [2][SG2_BWD_STRIDE] sums of adj_part's rows
     float* adj_part;               // bilevel: [2][ADJ_GROUPS][SG2_BWD_STRIDE] per-workgroup gradient sums
     int* sharp_nonzero;            // [P] uploaded as 0; set by k_keys when some (finite) sharpness entry of the tensor is not 0
     float* ctx;                    // [2][total][DM]
@@ -94,6 +95,8 @@ int launch_scan(const Plan& pl, hipStream_t st);
 // tile index of scan step u of tensor ti (element offset off) in the per-tile state array of the bilevel path
 __host__ __device__ inline int htile_index(int off, int ti, int u) { return off / SCAN_TT + ti + u / SCAN_TT; }
 __host__ __device__ inline int htile_count(int total, int P) { return total / SCAN_TT + P + 1; }
+// floats per direction of the adjoint kernels' sums: composed coefficients [5][16][3], A_log [16][16], rope_freq [16][8], D [16], out_proj [8][16]
+constexpr int SG2_BWD_STRIDE = 768;
 constexpr int ADJ_GROUPS = 512;    // workgroups per direction of the adjoint replay (upper bound)
 int check_dims(const SgDims* d);
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st);

@@ -41,7 +41,7 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, off_htile, off_adj_summ, off_adj_lam, off_adj_part, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, off_htile, off_adj_summ, off_adj_lam, off_adj_part, off_adj_blk, bytes;
     size_t tables_bytes;
 };
 
@@ -81,6 +81,7 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bil
     L->off_adj_summ = take(bilevel ? 4 * 2 * (size_t)L->chunks * SCAN_THREADS * 6 : 0);
     L->off_adj_lam = take(bilevel ? 4 * 2 * (size_t)L->chunks * SCAN_THREADS * 2 : 0);
     L->off_adj_part = take(bilevel ? 4 * 2 * (size_t)ADJ_GROUPS * SG2_BWD_STRIDE : 0);
+    L->off_adj_blk = take(bilevel ? 4 * 2 * (size_t)SG2_BWD_STRIDE : 0);
     L->bytes = o;
     return 0;
 }
@@ -269,6 +270,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.adj_summ = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_summ) : nullptr;
     pl.adj_lam = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_lam) : nullptr;
     pl.adj_part = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_part) : nullptr;
+    pl.adj_blk = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_blk) : nullptr;
     return 0;
 }
 }  // namespace sg2

@@ -6,7 +6,8 @@ grokking_optimizers/supergrok2.py:516-1371).
 The optimizer's bilevel update (`accumulate_meta_gradients`) runs in HIP end to
 end: sort + bidirectional Mamba-3 scan (sg2_bilevel_forward), per-element GRU /
 soft top-4 PEER routing / expert MLPs forward and backward in one pass
-(sg2_bilevel_elem), then the exact adjoint of the scan (sg2_bilevel_backward).
+(sg2_bilevel_elem), then the exact adjoint of the scan down to the gradients
+of the scan's weights (sg2_bilevel_backward).
 `forward_for_bilevel` is the module-level differentiable forward of one tensor:
 the scan as an autograd Function over the same two entry points, the per-element
 part as torch ops (`per_element`), which is also what the tests check
@@ -16,48 +17,14 @@ import torch
 
 from grokking_optimizers import _cabi
 
-GROUP_ROWS = 16
-
-
-def compose_coefficients(Win, bin_, in_proj, dt_W, dt_b, Bp, Cp):
-    """[5, 16, 3] coefficient triples (c_g, c_s, c_0) of x-branch, z, dt_raw, B, C as affine functions of an
-    element's (gradient, sharpness): the same composition include/sg2_compose.h performs on the device, as
-    differentiable torch algebra (float64), used to carry the coefficient gradients back to the raw weights."""
-    f = torch.float64
-    src = torch.cat([Win.to(f), bin_.to(f).unsqueeze(1)], dim=1)            # [d_model, 3]
-    di = dt_W.shape[0]
-    xb = in_proj.to(f)[:di] @ src                                            # [d_inner, 3]
-    z = in_proj.to(f)[di:] @ src
-    dt = dt_W.to(f) @ xb
-    dt = dt + torch.stack([torch.zeros_like(dt_b, dtype=f), torch.zeros_like(dt_b, dtype=f), dt_b.to(f)], dim=1)
-    return torch.stack([xb, z, dt, Bp.to(f) @ xb, Cp.to(f) @ xb], dim=0)
-
-
-def scan_weight_grads(block, W20):
-    """block: [2, SG2_BWD_STRIDE] from sg2_bilevel_backward; W20: the 20 scan weights (input_proj W, b, then the nine
-    tensors of each direction).  Returns the 20 gradients (float64): A_log / rope_freq / D / out_proj directly, the rest
-    by carrying the coefficient gradients through `compose_coefficients`."""
-    blk = block.double()
-    grads = [None] * 20
-    d_in_W = torch.zeros_like(W20[0], dtype=torch.float64)
-    d_in_b = torch.zeros_like(W20[1], dtype=torch.float64)
-    for d in range(2):
-        base = 2 + 9 * d
-        in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj = W20[base:base + 9]
-        o = 5 * GROUP_ROWS * 3
-        dcomp = blk[d, :o].reshape(5, GROUP_ROWS, 3)
-        d_alog = blk[d, o:o + A_log.numel()].reshape(A_log.shape); o += A_log.numel()
-        d_rope = blk[d, o:o + rope.numel()].reshape(rope.shape); o += rope.numel()
-        d_D = blk[d, o:o + D.numel()].reshape(D.shape); o += D.numel()
-        d_out_proj = blk[d, o:o + out_proj.numel()].reshape(out_proj.shape)
-        with torch.enable_grad():
-            raw = [t.detach().double().requires_grad_(True) for t in (W20[0], W20[1], in_proj, dt_W, dt_b, Bp, Cp)]
-            g = torch.autograd.grad(compose_coefficients(*raw), raw, grad_outputs=dcomp)
-        d_in_W += g[0]
-        d_in_b += g[1]
-        grads[base:base + 9] = [g[2], g[3], g[4], g[5], g[6], d_alog, d_D, d_rope, d_out_proj]
-    grads[0], grads[1] = d_in_W, d_in_b
-    return grads
+def split_flat(flat, params):
+    """Views of one flat gradient tensor, one per parameter, in order (no copies, no kernels)."""
+    out, o = [], 0
+    for p in params:
+        out.append(flat[o:o + p.numel()].view(p.shape))
+        o += p.numel()
+    assert o == flat.numel()
+    return out
 
 
 class ScanContexts(torch.autograd.Function):
@@ -74,8 +41,7 @@ class ScanContexts(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_out):
         W = ctx.saved_tensors
-        grads = scan_weight_grads(ctx.plan.backward(d_out), W)
-        return (None,) + tuple(gr.to(w.dtype) for gr, w in zip(grads, W))
+        return (None,) + tuple(gr.to(w.dtype) for gr, w in zip(split_flat(ctx.plan.backward(d_out), W), W))
 
 
 def scan_parameters(mn):
@@ -142,18 +108,20 @@ def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, ma
 
 
 def elem_parameters(mn):
-    """(parameter, shape in the gradient block of sg2_bilevel_elem) in the block's order."""
+    """The parameters of the per-element part in the order of sg2_bilevel_elem's gradient block."""
     out = []
     for lin in (mn.gru.W_z, mn.gru.W_r, mn.gru.W_h):
         out += [lin.weight, lin.bias]
-    return out, list(mn.peer_queries), list(mn.product_keys_A), list(mn.product_keys_B), \
-        [mn.expert_W1, mn.expert_b1, mn.expert_W2, mn.expert_b2]
+    out += [q.weight for q in mn.peer_queries] + list(mn.product_keys_A) + list(mn.product_keys_B)
+    return out + [mn.expert_W1, mn.expert_b1, mn.expert_W2, mn.expert_b2]
 
 
-def _add_grad(p, gr):
-    if p.requires_grad:
-        gr = gr.reshape(p.shape).to(p.dtype)
-        p.grad = gr.clone() if p.grad is None else p.grad + gr
+def _add_grads(params, flat):
+    """p.grad (+)= its slice of `flat`; a parameter without a gradient gets a view of the flat tensor."""
+    for p, gr in zip(params, split_flat(flat, params)):
+        if p.requires_grad:
+            gr = gr if gr.dtype == p.dtype else gr.to(p.dtype)
+            p.grad = gr if p.grad is None else p.grad + gr
 
 
 def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bwd, cotangents):
@@ -167,20 +135,8 @@ def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bw
     h_all = torch.cat([h.float() for h in gru_states])
     c_all = torch.cat([c.reshape(-1).float() for c in cotangents])
     smart, d_ctx, blk = _cabi.bilevel_elem(plan.weights, g_all, s_all, ctx, h_all, c_all, float(mn.rescale), meta_dims(mn))
-    gru_p, queries, keys_a, keys_b, experts = elem_parameters(mn)
-    o = 0
-    for p in gru_p:
-        _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
-    for group in (queries, keys_a, keys_b):
-        for q in group:
-            p = q.weight if isinstance(q, torch.nn.Linear) else q
-            _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
-    for p in experts:
-        _add_grad(p, blk[o:o + p.numel()]); o += p.numel()
-    assert o == _cabi.SG2_ELEM_GRAD_FLOATS
-    scan_params = scan_parameters(mn)
-    for p, gr in zip(scan_params, scan_weight_grads(plan.backward(d_ctx), [p.detach() for p in scan_params])):
-        _add_grad(p, gr)
+    _add_grads(elem_parameters(mn), blk)
+    _add_grads(scan_parameters(mn), plan.backward(d_ctx))
     return smart
 
 

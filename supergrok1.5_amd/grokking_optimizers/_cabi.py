@@ -175,14 +175,15 @@ class Sg2Step:
             raise RuntimeError("sg2_batched_step: " + last_error())
 
 
-SG2_BWD_STRIDE = 768        # floats per direction in the gradient block of sg2_bilevel_backward
+SG2_SCAN_GRAD_FLOATS = 3160  # gradients of the 20 scan weights, flat, in the order of Sg2Weights
 
 
 class Sg2Bilevel:
     """sg2_bilevel_forward / sg2_bilevel_backward on a fixed list of tensors: the sort and the bidirectional scan of
     the meta-net, differentiable with respect to the scan's weights.  forward() returns the two contexts of every
     element ([2, sum numel, d_model], element order, tensors packed in call order); backward(d_ctx) returns the
-    gradient block [2, SG2_BWD_STRIDE] described in include/sg_abi.h.  The workspace is kept between the two."""
+    gradients of the 20 scan weights as one flat tensor [SG2_SCAN_GRAD_FLOATS] (layout in include/sg_abi.h).  The
+    workspace is kept between the two."""
 
     def __init__(self, weights, grads, sharps, mamba_fwd, mamba_bwd, dims=None):
         self.dims = make_dims(dims)
@@ -225,7 +226,7 @@ class Sg2Bilevel:
     def backward(self, d_ctx):
         d_ctx = d_ctx.detach().float().contiguous()
         assert d_ctx.shape == (2, self.total, self.dims.d_model) and d_ctx.is_cuda
-        out = torch.empty(2, SG2_BWD_STRIDE, dtype=torch.float32, device=self.device)
+        out = torch.empty(SG2_SCAN_GRAD_FLOATS, dtype=torch.float32, device=self.device)
         rc = lib().sg2_bilevel_backward(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, d_ctx.data_ptr(), out.data_ptr(),
                                         self.workspace.data_ptr(), self.workspace.numel(), torch.cuda.current_stream().cuda_stream)
         if rc != 0:
