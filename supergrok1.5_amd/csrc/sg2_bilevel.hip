@@ -6,7 +6,7 @@
 // (csrc/supergrok2_mamba_peer_backward_kernels.cu:2512-3624 of the reference, called from
 // grokking_optimizers/supergrok2.py:516-1330).  The forward pass is the production scan itself
 // (sg2_bilevel_forward: sort + summaries + prefix + replay, carried states untouched), which additionally keeps
-// the state entering every 64-step tile; the per-element part of the meta-net (GRU, soft top-4 PEER routing,
+// the state entering every 32nd step; the per-element part of the meta-net (GRU, soft top-4 PEER routing,
 // experts) is differentiated by torch autograd on the caller's side.
 //
 // The adjoint state lambda obeys a linear recurrence over the scan steps in reverse, so a tensor is cut into the
@@ -16,9 +16,9 @@
 //   k_adj_prefix   per (tensor, direction): composes the maps from the last chunk to the first, leaving the adjoint
 //                  state that arrives at the end of every chunk;
 //   k_bilevel_backward  per (chunk, direction), exact from that arriving state.  A 128-lane workgroup walks the
-//                  chunk's 64-step tiles from the last to the first, lane (j,p) owning column j and RoPE pair p
+//                  chunk's 32-step tiles from the last to the first, lane (j,p) owning column j and RoPE pair p
 //                  as in the forward kernels.  Per tile:
-//   1  projections of the 64 steps from (g, s) and the composed coefficients, with the derivatives of softplus
+//   1  projections of the 32 steps from (g, s) and the composed coefficients, with the derivatives of softplus
 //      and SiLU, and the incoming context gradients gathered from element order;
 //   2  the forward recurrence from the saved tile-start state, keeping the state after every step in LDS;
 //   3  per step and column: out, d out = out_proj^T d ctx, d y, d z, the D-skip part of d x-branch;
@@ -41,9 +41,14 @@ constexpr int BST = SCAN_TT + 4;                 // row stride of the [16][64] L
 constexpr int ROWS = 16;
 // LDS arrays of ROWS x BST floats
 enum { A_DT, A_DSP, A_XB, A_B, A_C, A_GATE, A_DGATE, A_Y, A_DY, A_DZ, A_DXB, A_DDT, A_COUNT };
-constexpr int LDS_ROWS_FLOATS = A_COUNT * ROWS * BST;
-constexpr int LDS_H_FLOATS = SCAN_TT * SCAN_THREADS * 2;          // state after every step of the tile
-constexpr int LDS_MISC_FLOATS = SCAN_TT * DM + SCAN_TT * 2;       // d ctx tile, (g, s) of the tile
+// The gradient kernel works on tiles of BT = HT_STEP steps (half a forward tile), which keeps its LDS below half
+// a CU's so that two workgroups share a CU.
+constexpr int BT = HT_STEP;
+constexpr int BBST = BT + 1;                     // row stride of its [16][BT] arrays (odd: the 16 rows a step reads hit 16 banks)
+constexpr int LDS_ROWS_FLOATS = A_COUNT * ROWS * BBST;
+constexpr int LDS_H_FLOATS = BT * SCAN_THREADS * 2;               // state after every step of the tile
+constexpr int LDS_MISC_FLOATS = BT * DM + BT * 2;                 // d ctx tile, (g, s) of the tile
+static_assert(SCAN_THREADS == 4 * BT && ROWS % 4 == 0 && (LDS_ROWS_FLOATS + LDS_H_FLOATS) % 4 == 0, "projection roles, float4 alignment");
 constexpr int BILEVEL_LDS_BYTES = 4 * (LDS_ROWS_FLOATS + LDS_H_FLOATS + LDS_MISC_FLOATS);
 
 // value of the lane whose index differs in one bit, by DPP where the pattern stays inside a row of 16 lanes
@@ -194,8 +199,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     float* rows = lds;
     float* sH = lds + LDS_ROWS_FLOATS;
     float* s_dctx = sH + LDS_H_FLOATS;
-    float* s_gs = s_dctx + SCAN_TT * DM;
-    auto arr = [&](int a) { return rows + a * ROWS * BST; };
+    float* s_gs = s_dctx + BT * DM;
+    auto arr = [&](int a) { return rows + a * ROWS * BBST; };
 
     const int dir = blockIdx.y;
     const int b = dir ? W_B_INPROJ : W_F_INPROJ;
@@ -206,7 +211,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     const float* __restrict__ comp = pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3);
 
     const int tid = threadIdx.x;
-    const int tu = tid & (SCAN_TT - 1), half = tid >> 6;          // projection role
+    const int tu = tid & (BT - 1), part = tid >> 5;               // projection role: step tu, rows 4*part .. 4*part+3
     const int j = tid >> 3, p = tid & 7, w = tid >> 6;             // recurrence role
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
@@ -226,32 +231,32 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         le = lam[0];
         lo = lam[1];
     }
-    const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
+    const int ntiles = (c.uend - c.ustart + BT - 1) / BT;
     for (int tile = ntiles - 1; tile >= 0; tile--) {
-        const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
+        const int u0 = c.ustart + tile * BT, cnt = min(BT, c.uend - u0);
         // ---- 1: projections, activation derivatives, incoming gradients
         {
             const bool valid = tu < cnt;
             float g, s;
             int orig;
             load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
-            if (half == 0) { s_gs[2 * tu] = g; s_gs[2 * tu + 1] = s; }
-            {
-                const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
-                reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
+            if (part == 0) { s_gs[2 * tu] = g; s_gs[2 * tu + 1] = s; }
+            if (part < DM / 4) {
+                const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[part] : make_float4(0.f, 0.f, 0.f, 0.f);
+                reinterpret_cast<float4*>(s_dctx + tu * DM)[part] = dv;
             }
-            for (int q = 0; q < ROWS / 2; q++) {
-                const int r = half * (ROWS / 2) + q;
+            for (int q = 0; q < ROWS / 4; q++) {
+                const int r = part * (ROWS / 4) + q;
                 const float raw = sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s);
-                arr(A_DT)[r * BST + tu] = valid ? sg_softplus(raw) : 0.0f;
-                arr(A_DSP)[r * BST + tu] = (raw > 20.0f) ? 1.0f : sg_sigmoid(raw);
-                arr(A_XB)[r * BST + tu] = valid ? sg2_comp_eval(comp + (SG2_COMP_XB * 16 + r) * 3, g, s) : 0.0f;
-                arr(A_B)[r * BST + tu] = sg2_comp_eval(comp + (SG2_COMP_B * 16 + r) * 3, g, s);
-                arr(A_C)[r * BST + tu] = sg2_comp_eval(comp + (SG2_COMP_C * 16 + r) * 3, g, s);
+                arr(A_DT)[r * BBST + tu] = valid ? sg_softplus(raw) : 0.0f;
+                arr(A_DSP)[r * BBST + tu] = (raw > 20.0f) ? 1.0f : sg_sigmoid(raw);
+                arr(A_XB)[r * BBST + tu] = valid ? sg2_comp_eval(comp + (SG2_COMP_XB * 16 + r) * 3, g, s) : 0.0f;
+                arr(A_B)[r * BBST + tu] = sg2_comp_eval(comp + (SG2_COMP_B * 16 + r) * 3, g, s);
+                arr(A_C)[r * BBST + tu] = sg2_comp_eval(comp + (SG2_COMP_C * 16 + r) * 3, g, s);
                 const float z = sg2_comp_eval(comp + (SG2_COMP_Z * 16 + r) * 3, g, s);
                 const float sz = sg_sigmoid(z);
-                arr(A_GATE)[r * BST + tu] = z * sz;
-                arr(A_DGATE)[r * BST + tu] = sz * sg_fma(z, 1.0f - sz, 1.0f);
+                arr(A_GATE)[r * BBST + tu] = z * sz;
+                arr(A_DGATE)[r * BBST + tu] = sz * sg_fma(z, 1.0f - sz, 1.0f);
             }
         }
         __syncthreads();
@@ -262,44 +267,44 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         {
             float he = hs_e, ho = hs_o;
             for (int k = 0; k < cnt; k++) {
-                const float dt = arr(A_DT)[j * BST + k];
+                const float dt = arr(A_DT)[j * BBST + k];
                 float ae, ao, sn, cs;
                 sg_abar_pair(dt, a_e, a_o, &ae, &ao);
                 sg_sincos(dt * freq, &sn, &cs);
-                const float ux = dt * arr(A_XB)[j * BST + k];
+                const float ux = dt * arr(A_XB)[j * BBST + k];
                 const float re = sg_fma(he, cs, -(ho * sn)), ro = sg_fma(ho, cs, he * sn);
-                he = sg_fma(ae, re, ux * arr(A_B)[(2 * p) * BST + k]);
-                ho = sg_fma(ao, ro, ux * arr(A_B)[(2 * p + 1) * BST + k]);
+                he = sg_fma(ae, re, ux * arr(A_B)[(2 * p) * BBST + k]);
+                ho = sg_fma(ao, ro, ux * arr(A_B)[(2 * p + 1) * BBST + k]);
                 sH[(k * SCAN_THREADS + tid) * 2] = he;
                 sH[(k * SCAN_THREADS + tid) * 2 + 1] = ho;
-                const float y = pair_sum(sg_fma(ho, arr(A_C)[(2 * p + 1) * BST + k], he * arr(A_C)[(2 * p) * BST + k]));
-                if (p == 0) arr(A_Y)[j * BST + k] = y;
+                const float y = pair_sum(sg_fma(ho, arr(A_C)[(2 * p + 1) * BBST + k], he * arr(A_C)[(2 * p) * BBST + k]));
+                if (p == 0) arr(A_Y)[j * BBST + k] = y;
             }
         }
         __syncthreads();
 
         // ---- 3: per step and column: out, d out, d y, d z, D-skip part of d x-branch
-        for (int q = 0; q < ROWS / 2; q++) {
-            const int r = half * (ROWS / 2) + q;
+        for (int q = 0; q < ROWS / 4; q++) {
+            const int r = part * (ROWS / 4) + q;
             float dout = 0.0f;
 #pragma unroll
             for (int d = 0; d < DM; d++) dout = sg_fma(Wout[d * DI + r], s_dctx[tu * DM + d], dout);
-            const float y = arr(A_Y)[r * BST + tu], gate = arr(A_GATE)[r * BST + tu], xb = arr(A_XB)[r * BST + tu];
+            const float y = arr(A_Y)[r * BBST + tu], gate = arr(A_GATE)[r * BBST + tu], xb = arr(A_XB)[r * BBST + tu];
             const bool valid = tu < cnt;
-            arr(A_DY)[r * BST + tu] = valid ? dout * gate : 0.0f;
-            arr(A_DZ)[r * BST + tu] = valid ? (dout * y) * arr(A_DGATE)[r * BST + tu] : 0.0f;
-            arr(A_DXB)[r * BST + tu] = valid ? dout * Dw[r] : 0.0f;
-            arr(A_GATE)[r * BST + tu] = valid ? sg_fma(y, gate, Dw[r] * xb) : 0.0f;     // out, for d out_proj
-            arr(A_DGATE)[r * BST + tu] = valid ? dout : 0.0f;                           // d out, for d D
-            arr(A_DDT)[r * BST + tu] = 0.0f;
+            arr(A_DY)[r * BBST + tu] = valid ? dout * gate : 0.0f;
+            arr(A_DZ)[r * BBST + tu] = valid ? (dout * y) * arr(A_DGATE)[r * BBST + tu] : 0.0f;
+            arr(A_DXB)[r * BBST + tu] = valid ? dout * Dw[r] : 0.0f;
+            arr(A_GATE)[r * BBST + tu] = valid ? sg_fma(y, gate, Dw[r] * xb) : 0.0f;     // out, for d out_proj
+            arr(A_DGATE)[r * BBST + tu] = valid ? dout : 0.0f;                           // d out, for d D
+            arr(A_DDT)[r * BBST + tu] = 0.0f;
         }
         __syncthreads();
 
         // ---- 4: adjoint recurrence, last step of the tile first
         for (int k = cnt - 1; k >= 0; k--) {
-            const float dt = arr(A_DT)[j * BST + k], xb = arr(A_XB)[j * BST + k], dy = arr(A_DY)[j * BST + k];
-            const float Be = arr(A_B)[(2 * p) * BST + k], Bo = arr(A_B)[(2 * p + 1) * BST + k];
-            const float Ce = arr(A_C)[(2 * p) * BST + k], Co = arr(A_C)[(2 * p + 1) * BST + k];
+            const float dt = arr(A_DT)[j * BBST + k], xb = arr(A_XB)[j * BBST + k], dy = arr(A_DY)[j * BBST + k];
+            const float Be = arr(A_B)[(2 * p) * BBST + k], Bo = arr(A_B)[(2 * p + 1) * BBST + k];
+            const float Ce = arr(A_C)[(2 * p) * BBST + k], Co = arr(A_C)[(2 * p + 1) * BBST + k];
             const float he = sH[(k * SCAN_THREADS + tid) * 2], ho = sH[(k * SCAN_THREADS + tid) * 2 + 1];
             const float pe = (k > 0) ? sH[((k - 1) * SCAN_THREADS + tid) * 2] : hs_e;
             const float po = (k > 0) ? sH[((k - 1) * SCAN_THREADS + tid) * 2 + 1] : hs_o;
@@ -340,8 +345,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             }
             const float ddt_j = pair_sum(ddt), dxb_j = pair_sum(qb * dt);
             if (p == 0) {
-                arr(A_DDT)[j * BST + k] = ddt_j * arr(A_DSP)[j * BST + k];
-                arr(A_DXB)[j * BST + k] += dxb_j;
+                arr(A_DDT)[j * BBST + k] = ddt_j * arr(A_DSP)[j * BBST + k];
+                arr(A_DXB)[j * BBST + k] += dxb_j;
             }
             // lambda for the previous step
             const float nle = sg_fma(dre, cs, dro * sn), nlo = sg_fma(dro, cs, -(dre * sn));
@@ -354,11 +359,11 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         if (tid < 3 * 16) {              // x-branch, z, dt (the first three coefficient groups)
             const int group = tid / 16, r = tid % 16;
 #pragma unroll 8
-            for (int k = 0; k < SCAN_TT; k++) {
+            for (int k = 0; k < BT; k++) {
                 float dv;
-                if (group == SG2_COMP_XB) dv = arr(A_DXB)[r * BST + k];
-                else if (group == SG2_COMP_Z) dv = arr(A_DZ)[r * BST + k];
-                else dv = arr(A_DDT)[r * BST + k];
+                if (group == SG2_COMP_XB) dv = arr(A_DXB)[r * BBST + k];
+                else if (group == SG2_COMP_Z) dv = arr(A_DZ)[r * BBST + k];
+                else dv = arr(A_DDT)[r * BBST + k];
                 acc_c0 = sg_fma(dv, s_gs[2 * k], acc_c0);
                 acc_c1 = sg_fma(dv, s_gs[2 * k + 1], acc_c1);
                 acc_c2 += dv;
@@ -366,12 +371,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         } else if (tid < SG2_COMP_GROUPS * 16 + DI) {
             const int r = tid - SG2_COMP_GROUPS * 16;
 #pragma unroll 8
-            for (int k = 0; k < SCAN_TT; k++) acc_D = sg_fma(arr(A_DGATE)[r * BST + k], arr(A_XB)[r * BST + k], acc_D);
+            for (int k = 0; k < BT; k++) acc_D = sg_fma(arr(A_DGATE)[r * BBST + k], arr(A_XB)[r * BBST + k], acc_D);
         }
         {
             const int d = tid >> 4, r = tid & 15;       // out_proj[d][r]
 #pragma unroll 8
-            for (int k = 0; k < SCAN_TT; k++) acc_wout = sg_fma(s_dctx[k * DM + d], arr(A_GATE)[r * BST + k], acc_wout);
+            for (int k = 0; k < BT; k++) acc_wout = sg_fma(s_dctx[k * DM + d], arr(A_GATE)[r * BBST + k], acc_wout);
         }
         __syncthreads();
     }

@@ -76,7 +76,7 @@ struct Plan {
     float* summaries;              // [2][wchunks][6][128]
     float* hstart;                 // [2][chunks][2][128]
     float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
-    float* htile;                  // bilevel: [2][tiles][2][128] state at the start of every 64-step tile, or NULL
+    float* htile;                  // bilevel: [2][htile_count][2][128] state entering every HT_STEP-th step, or NULL
     float* adj_summ;               // bilevel: [2][chunks][128][6] adjoint transfer map of every chunk
     float* adj_lam;                // bilevel: [2][chunks][128][2] adjoint state arriving at the end of every chunk
     float* adj_blk;                // bilevel: [2][SG2_BWD_STRIDE] sums of adj_part's rows
@@ -92,9 +92,11 @@ void prof_mark(int idx, hipStream_t st);
 
 int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st);
 int launch_scan(const Plan& pl, hipStream_t st);
-// tile index of scan step u of tensor ti (element offset off) in the per-tile state array of the bilevel path
-__host__ __device__ inline int htile_index(int off, int ti, int u) { return off / SCAN_TT + ti + u / SCAN_TT; }
-__host__ __device__ inline int htile_count(int total, int P) { return total / SCAN_TT + P + 1; }
+// bilevel path: the forward scan keeps the state entering every HT_STEP-th step of a tensor; index of scan step u
+// (a multiple of HT_STEP) of tensor ti (element offset off) in that array, and the array's length
+constexpr int HT_STEP = 32;
+__host__ __device__ inline int htile_index(int off, int ti, int u) { return off / HT_STEP + ti + u / HT_STEP; }
+__host__ __device__ inline int htile_count(int total, int P) { return total / HT_STEP + P + 1; }
 // floats per direction of the adjoint kernels' sums: composed coefficients [5][16][3], A_log [16][16], rope_freq [16][8], D [16], out_proj [8][16]
 constexpr int SG2_BWD_STRIDE = 768;
 constexpr int ADJ_GROUPS = 512;    // workgroups per direction of the adjoint replay (upper bound)

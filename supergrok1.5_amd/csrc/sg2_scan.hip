@@ -49,8 +49,8 @@
 // the block is below 0.3 a shorter polynomial pair is used (sg_sincos_tiny,
 // not bit-identical to the general form: the choice depends on the angles only
 // and the CPU checker makes the same one).
-// For the bilevel pass k_scan<true> also stores the state entering every
-// 64-step tile (Plan::htile), which the adjoint kernels restart from.
+// For the bilevel pass k_scan<true, true> also stores the state entering every
+// 32nd step (Plan::htile), which the adjoint kernels restart from.
 #include "sg2_internal.hpp"
 #include "../../include/sg2_compose.h"
 
@@ -65,6 +65,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #endif
 constexpr int UB = SG2_SCAN_UB;           // timesteps per unrolled block of the recurrence
 static_assert(UB % 4 == 0 && SCAN_TT % UB == 0 && SCAN_TT == 64, "blocks are fetched 4 timesteps per LDS read; one ballot covers a tile");
+static_assert(HT_STEP % UB == 0 && SCAN_TT % HT_STEP == 0 && SCAN_TT / HT_STEP <= 2, "kept states fall on block borders: tile start and at most one more");
 // Three waves per SIMD (168 VGPRs) is where the kernels stop gaining from occupancy; keep the
 // register allocation from drifting just past that boundary.
 #ifndef SG2_SCAN_WAVES
@@ -216,7 +217,8 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
 }
 
-template <bool OUT>
+// KEEP (bilevel pass, OUT only): also store the state entering every HT_STEP-th step for the adjoint kernels.
+template <bool OUT, bool KEEP = false>
 __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     __shared__ __attribute__((aligned(16))) float s_dt[DI * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) float s_ux[DI * LDS_STRIDE];       // dt * x-branch
@@ -320,11 +322,12 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         __syncthreads();
         const unsigned long long large = s_large[half], nottiny = s_nottiny[half];
 
-        if (OUT && pl.htile != nullptr) {      // bilevel: keep the state entering this tile for the backward pass
-            float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, tile0)) * 2 * SCAN_THREADS;
+        auto keep_state = [&](int u) {
+            float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, u)) * 2 * SCAN_THREADS;
             ht[tid] = S.he;
             ht[SCAN_THREADS + tid] = S.ho;
-        }
+        };
+        if (KEEP) keep_state(tile0);
         // ---------------- phase B: the recurrence over the tile, lane = (j,p)
         const float* __restrict__ r_dt = s_dt + j * LDS_STRIDE;
         const float* __restrict__ r_ux = s_ux + j * LDS_STRIDE;
@@ -334,6 +337,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float* __restrict__ r_Co = s_C + (OUT ? (2 * p + 1) * LDS_STRIDE : 0);
         int k0 = 0;
         for (; k0 + UB <= cnt; k0 += UB) {
+            if (KEEP && k0 == HT_STEP) keep_state(tile0 + HT_STEP);
             float dt[UB], xv[UB], Be[UB], Bo[UB], Ce[UB], Co[UB], y[UB];
 #pragma unroll
             for (int q = 0; q < UB; q += 4) {
@@ -360,6 +364,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                     *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + q]) = f32x4{y[q], y[q + 1], y[q + 2], y[q + 3]};
             }
         }
+        if (KEEP && k0 == HT_STEP && cnt > HT_STEP) keep_state(tile0 + HT_STEP);      // the ragged end starts right there
         for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
             const float dt = r_dt[k0], ux = r_ux[k0];
             float ae, ao, sn, cs;
@@ -498,14 +503,17 @@ int launch_scan(const Plan& pl, hipStream_t st) {
     hipLaunchKernelGGL(k_compose, dim3(1), dim3(2 * SG2_COMP_GROUPS * 16), 0, st, pl);
     SG_LAUNCH_CHECK("k_compose");
     if (pl.wchunks > 0) {
-        hipLaunchKernelGGL(k_scan<false>, dim3(2 * pl.wchunks), dim3(SCAN_THREADS), 0, st, pl);
+        hipLaunchKernelGGL((k_scan<false, false>), dim3(2 * pl.wchunks), dim3(SCAN_THREADS), 0, st, pl);
         SG_LAUNCH_CHECK("k_scan<summary>");
     }
     prof_mark(2, st);
     hipLaunchKernelGGL(k_chunk_prefix, dim3(2 * pl.P), dim3(PREFIX_GROUPS * SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_chunk_prefix");
     prof_mark(3, st);
-    hipLaunchKernelGGL(k_scan<true>, dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
+    if (pl.htile != nullptr)
+        hipLaunchKernelGGL((k_scan<true, true>), dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
+    else
+        hipLaunchKernelGGL((k_scan<true, false>), dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_scan<out>");
     prof_mark(4, st);
     return 0;

@@ -76,8 +76,8 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bil
     L->off_comp = take(4 * 2 * 5 * 16 * 3);
     L->off_flags = take(4 * (size_t)P);        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * DM);
-    // bilevel only: state at the start of every 64-step tile, both directions (tile index = off/64 + tensor index + u/64)
-    L->off_htile = take(bilevel ? 4 * 2 * ((size_t)total / SCAN_TT + (size_t)P + 1) * 2 * SCAN_THREADS : 0);
+    // bilevel only: state entering every HT_STEP-th step, both directions
+    L->off_htile = take(bilevel ? 4 * 2 * (size_t)htile_count((int)total, P) * 2 * SCAN_THREADS : 0);
     L->off_adj_summ = take(bilevel ? 4 * 2 * (size_t)L->chunks * SCAN_THREADS * 6 : 0);
     L->off_adj_lam = take(bilevel ? 4 * 2 * (size_t)L->chunks * SCAN_THREADS * 2 : 0);
     L->off_adj_part = take(bilevel ? 4 * 2 * (size_t)ADJ_GROUPS * SG2_BWD_STRIDE : 0);

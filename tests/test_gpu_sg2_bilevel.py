@@ -89,6 +89,12 @@ def test_small_tensors_with_sharpness_and_carried_states():
     _case([(300,), (70,), (1,), (129,), (5, 13)], seed=11, sharp=True, state_std=0.3)
 
 
+def test_ragged_tile_ends():
+    """Lengths that end 1..7 steps after a multiple of 32 or 64 (the forward pass keeps a state every 32 steps, and the
+    last steps of a tensor run through its scalar tail loop)."""
+    _case([(99,), (33,), (97,), (39,), (64 + 32,), (32,), (31,), (64 + 39,)], seed=15, sharp=True, state_std=0.3)
+
+
 def test_zero_sharpness_and_zero_states():
     _case([(200,), (64,), (65,)], seed=12, sharp=False, state_std=0.0)
 
