@@ -415,14 +415,19 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     g_wout[tid] = acc_wout;
 }
 
-// ---- launch 4: rows of the partials buffer added in a fixed order
-__global__ void k_adj_sum_rows(const float* __restrict__ part, int rows_per_dir, float* __restrict__ out) {
-    const int o = blockIdx.x * blockDim.x + threadIdx.x;
-    if (o >= 2 * SG2_BWD_STRIDE) return;
+// ---- launch 4: rows of the partials buffer added in a fixed order (64 entries per workgroup, four lanes per entry
+// each taking every fourth row, then the four partial sums in order)
+__global__ __launch_bounds__(256) void k_adj_sum_rows(const float* __restrict__ part, int rows_per_dir, float* __restrict__ out) {
+    __shared__ float s_part[4][64];
+    const int col = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + col;          // 2 * SG2_BWD_STRIDE is a multiple of 64
     const int dir = o / SG2_BWD_STRIDE, e = o % SG2_BWD_STRIDE;
     float acc = 0.0f;
-    for (int r = 0; r < rows_per_dir; r++) acc += part[((size_t)dir * rows_per_dir + r) * SG2_BWD_STRIDE + e];
-    out[o] = acc;
+#pragma unroll 4
+    for (int r = slice; r < rows_per_dir; r += 4) acc += part[((size_t)dir * rows_per_dir + r) * SG2_BWD_STRIDE + e];
+    s_part[slice][col] = acc;
+    __syncthreads();
+    if (slice == 0) out[o] = ((s_part[0][col] + s_part[1][col]) + s_part[2][col]) + s_part[3][col];
 }
 
 // ---- launch 5: from the gradients of the composed coefficients to those of the weights they were composed from
@@ -535,7 +540,8 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
     SG_LAUNCH_CHECK("k_adj_prefix");
     hipLaunchKernelGGL(k_bilevel_backward, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, d_ctx);
     SG_LAUNCH_CHECK("k_bilevel_backward");
-    hipLaunchKernelGGL(k_adj_sum_rows, dim3((2 * SG2_BWD_STRIDE + 255) / 256), dim3(256), 0, st, pl.adj_part, groups, pl.adj_blk);
+    static_assert((2 * SG2_BWD_STRIDE) % 64 == 0, "k_adj_sum_rows: whole workgroups");
+    hipLaunchKernelGGL(k_adj_sum_rows, dim3(2 * SG2_BWD_STRIDE / 64), dim3(256), 0, st, pl.adj_part, groups, pl.adj_blk);
     SG_LAUNCH_CHECK("k_adj_sum_rows");
     hipLaunchKernelGGL(k_compose_backward, dim3(1), dim3(256), 0, st, pl, pl.adj_blk, grads_out);
     SG_LAUNCH_CHECK("k_compose_backward");

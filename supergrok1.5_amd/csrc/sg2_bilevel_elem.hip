@@ -429,12 +429,20 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     }
 }
 
-__global__ void k_sum_partials(const float* __restrict__ partials, int rows, float* __restrict__ out) {
-    const int o = blockIdx.x * blockDim.x + threadIdx.x;
-    if (o >= N_GRADS) return;
+// Rows of the partials buffer added in a fixed order: 64 entries per workgroup, four lanes per entry each taking
+// every fourth row, then the four partial sums in order.
+__global__ __launch_bounds__(256) void k_sum_partials(const float* __restrict__ partials, int rows, float* __restrict__ out) {
+    __shared__ float s_part[4][64];
+    const int col = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + col;
     float acc = 0.0f;
-    for (int r = 0; r < rows; r++) acc += partials[(size_t)r * N_GRADS + o];
-    out[o] = acc;
+    if (o < N_GRADS) {
+#pragma unroll 4
+        for (int r = slice; r < rows; r += 4) acc += partials[(size_t)r * N_GRADS + o];
+    }
+    s_part[slice][col] = acc;
+    __syncthreads();
+    if (slice == 0 && o < N_GRADS) out[o] = ((s_part[0][col] + s_part[1][col]) + s_part[2][col]) + s_part[3][col];
 }
 
 constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW));
@@ -489,7 +497,7 @@ int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t tota
     a.total = (int)total; a.rescale = rescale; a.W = *weights;
     hipLaunchKernelGGL(k_bilevel_elem, dim3(groups), dim3(BE_THREADS), BE_LDS_BYTES, st, a);
     SG_LAUNCH_CHECK("k_bilevel_elem");
-    hipLaunchKernelGGL(k_sum_partials, dim3((N_GRADS + 255) / 256), dim3(256), 0, st, a.partials, groups, grads_out);
+    hipLaunchKernelGGL(k_sum_partials, dim3((N_GRADS + 63) / 64), dim3(256), 0, st, a.partials, groups, grads_out);
     SG_LAUNCH_CHECK("k_sum_partials");
     return 0;
 }
