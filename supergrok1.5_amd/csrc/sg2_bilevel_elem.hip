@@ -8,16 +8,17 @@
 // grokking_optimizers/supergrok2.py:516-1330); the arithmetic is that of Mamba3PEERMetaNet.forward_for_bilevel
 // (grokking_optimizers/mamba3_peer_metanet.py:395-436) and its autograd derivative.
 //
-// One lane per element, persistent grid over tiles of 256 elements.  Nothing is kept between forward and backward:
+// One lane per element, persistent grid over tiles of 128 elements (two 128-lane workgroups share a CU, so one
+// workgroup's passes over its tile overlap the other's per-element arithmetic).  Nothing is kept between forward and backward:
 // a lane holds its element's activations in registers, and the routing of a head is differentiated before the
 // next head is evaluated.  Weight gradients are sums over elements:
 //   * product keys (rows chosen per element): float atomics on accumulators in LDS;
-//   * experts (16 per element and head, chosen per element): gathered, not scattered.  Each lane owns nine
+//   * experts (16 per element and head, chosen per element): gathered, not scattered.  Each lane owns 18
 //     (expert, hidden unit) pairs with their sums in registers and walks the tile's elements, whose routing
 //     weights of the head every lane has left in LDS as two 12-vectors (see the expert-gradient pass);
-//   * GRU and query matrices (dense outer products d (x) x): every lane leaves its d (44 values) and x (31 values)
-//     in LDS, then each lane of the workgroup owns up to four matrix entries and sums their products over the
-//     256 elements of the tile, keeping the running sums in registers for the life of the workgroup.
+//   * GRU and query matrices (dense outer products d (x) x): every lane leaves its x (31 values) and, per head
+//     and once more for the GRU, its d (8 / 12 values) in LDS; each lane of the workgroup owns up to two entries
+//     of the head's query matrix and three of the GRU matrices and sums their products over the tile's elements.
 // Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
 // order.  (Within a workgroup the LDS atomics arrive in no fixed order, so the key gradients can differ in the last
 // bits between runs; everything else is summed in a fixed order.)
@@ -26,38 +27,39 @@
 namespace sg2 {
 namespace {
 
-constexpr int BE_THREADS = 256;
+constexpr int BE_THREADS = 128;         // two waves; LDS is sized so that two workgroups share a CU
+constexpr int BE_WAVES = BE_THREADS / 64;
 constexpr int EXP_STRIDE = 52;          // floats per expert record in LDS: W1[16] b1[16] W2[16] b2 + pad
 constexpr int TOPK = 4;
 constexpr int RW = 2 * PK + 1;          // staged routing row of a head: first-index weights[12] (times d loss/d head), second-index weights[12], mask of first indices
 constexpr int EXP_PER_LANE = NE * EH / BE_THREADS;     // (expert, hidden unit) pairs a lane accumulates
-static_assert(NE * EH % BE_THREADS == 0 && PK % 4 == 0, "expert pairs per lane");
-constexpr int XW = 31, DW = 45;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
+static_assert(NE * EH % BE_THREADS == 0 && PK % 4 == 0 && PK % BE_WAVES == 0, "expert pairs per lane");
+constexpr int XW = 31, DW = 13;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
 // x row: g, s, fwd ctx[8], bwd ctx[8], h_old[4], r*h_old[4], h_new[4], 1
 constexpr int X_G = 0, X_S = 1, X_CF = 2, X_CB = 10, X_H = 18, X_RH = 22, X_HN = 26, X_ONE = 30;
-// d row: d pre_z[4], d pre_r[4], d pre_h[4], d query[4 heads][8]
-constexpr int D_Z = 0, D_R = 4, D_H = 8, D_Q = 12;
-constexpr int N_DENSE = 3 * (GH * GRL + GH) + NH * DM * PIN;      // 276 + 704
+// d row, reused: d query[8] of the current head, then d pre_z[4], d pre_r[4], d pre_h[4] of the GRU
+constexpr int D_Z = 0, D_R = 4, D_H = 8;
+constexpr int N_GRU = 3 * (GH * GRL + GH), N_QHEAD = DM * PIN;     // 276 GRU entries, 176 query entries per head
+constexpr int N_DENSE = N_GRU + NH * N_QHEAD;                      // 276 + 704
 constexpr int OFF_KA = N_DENSE, OFF_KB = OFF_KA + NH * PK * (DM / 2);
 constexpr int OFF_W1 = OFF_KB + NH * PK * (DM / 2), OFF_B1 = OFF_W1 + NE * EH, OFF_W2 = OFF_B1 + NE * EH, OFF_B2 = OFF_W2 + NE * EH;
 constexpr int N_GRADS = OFF_B2 + NE;
 static_assert(N_GRADS == SG2_ELEM_GRAD_FLOATS, "gradient layout");
-constexpr int DENSE_PER_LANE = (N_DENSE + BE_THREADS - 1) / BE_THREADS;
+constexpr int GRU_PER_LANE = (N_GRU + BE_THREADS - 1) / BE_THREADS, Q_PER_LANE = (N_QHEAD + BE_THREADS - 1) / BE_THREADS;
 
-// (column of d, column of x) whose products make up dense gradient entry o, in the order
-// W_z[4][22] b_z[4] W_r[4][22] b_r[4] W_h[4][22] b_h[4] queries[4][8][22]
-__device__ __forceinline__ void dense_entry(int o, int* dcol, int* xcol) {
-    if (o < 3 * (GH * GRL + GH)) {
-        const int gate = o / (GH * GRL + GH), q = o % (GH * GRL + GH);
-        if (q >= GH * GRL) { *dcol = gate * GH + (q - GH * GRL); *xcol = X_ONE; return; }
-        const int j = q / GRL, c = q % GRL;
-        *dcol = gate * GH + j;
-        *xcol = (gate == 2 && c >= 2 + 2 * DM) ? X_RH + (c - 2 - 2 * DM) : c;     // the candidate sees r*h in place of h
-        return;
-    }
-    const int q = o - 3 * (GH * GRL + GH);
-    const int row = q / PIN, c = q % PIN;                 // row = head*8 + r; query input = h_new, fwd ctx, bwd ctx, g, s
-    *dcol = D_Q + row;
+// (column of d, column of x) whose products make up GRU gradient entry o, in the order
+// W_z[4][22] b_z[4] W_r[4][22] b_r[4] W_h[4][22] b_h[4]
+__device__ __forceinline__ void gru_entry(int o, int* dcol, int* xcol) {
+    const int gate = o / (GH * GRL + GH), q = o % (GH * GRL + GH);
+    if (q >= GH * GRL) { *dcol = gate * GH + (q - GH * GRL); *xcol = X_ONE; return; }
+    const int j = q / GRL, c = q % GRL;
+    *dcol = gate * GH + j;
+    *xcol = (gate == 2 && c >= 2 + 2 * DM) ? X_RH + (c - 2 - 2 * DM) : c;     // the candidate sees r*h in place of h
+}
+// same for entry o = r*22 + c of a head's query matrix [8][22]; query input = h_new, fwd ctx, bwd ctx, g, s
+__device__ __forceinline__ void query_entry(int o, int* dcol, int* xcol) {
+    const int c = o % PIN;
+    *dcol = o / PIN;
     *xcol = c < GH ? X_HN + c : (c < GH + 2 * DM ? X_CF + (c - GH) : (c == GH + 2 * DM ? X_G : X_S));
 }
 
@@ -75,7 +77,8 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     float* s_gkey = s_exp + NE * EXP_STRIDE;              // [2][NH][PK][DM/2]
     float* s_x = s_gkey + 2 * NH * PK * (DM / 2);         // [256][XW]
     float* s_d = s_x + BE_THREADS * XW;                   // [256][DW]
-    float* s_rt = s_d + BE_THREADS * DW;                  // [256][RW]
+    float* s_rt = s_d + BE_THREADS * DW;                  // [128][RW]
+    float* s_gq = s_rt + BE_THREADS * RW;                 // [NH][8][22] query-matrix gradients of this workgroup
 
     const int tid = threadIdx.x;
     {
@@ -85,6 +88,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         const float* __restrict__ B2 = a.W.w[W_EXP_B2];
         for (int i = tid; i < NE * EXP_STRIDE; i += BE_THREADS) s_exp[i] = 0.0f;
         for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) s_gkey[i] = 0.0f;
+        for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) s_gq[i] = 0.0f;
         __syncthreads();
         for (int i = tid; i < NE * EH; i += BE_THREADS) {
             const int e = i / EH, k = i % EH;
@@ -102,20 +106,26 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     const sg::cfloat_p Wq = sg::as_const(a.W.w[W_PEER_Q]);
     const sg::cfloat_p KA = sg::as_const(a.W.w[W_KEYS_A]), KB = sg::as_const(a.W.w[W_KEYS_B]);
 
-    int dcol[DENSE_PER_LANE], xcol[DENSE_PER_LANE];
-    float dense[DENSE_PER_LANE];
+    // the lane's entries of the GRU gradients (sums kept in registers) and of a head's query matrix (summed per
+    // tile and head, then added to s_gq)
+    int gdcol[GRU_PER_LANE], gxcol[GRU_PER_LANE], qdcol[Q_PER_LANE], qxcol[Q_PER_LANE];
+    float gsum[GRU_PER_LANE];
 #pragma unroll
-    for (int q = 0; q < DENSE_PER_LANE; q++) {
-        const int o = tid + q * BE_THREADS;
-        dcol[q] = 0; xcol[q] = 0; dense[q] = 0.0f;
-        if (o < N_DENSE) dense_entry(o, &dcol[q], &xcol[q]);
+    for (int q = 0; q < GRU_PER_LANE; q++) {
+        gdcol[q] = 0; gxcol[q] = 0; gsum[q] = 0.0f;
+        if (tid + q * BE_THREADS < N_GRU) gru_entry(tid + q * BE_THREADS, &gdcol[q], &gxcol[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < Q_PER_LANE; q++) {
+        qdcol[q] = 0; qxcol[q] = 0;
+        if (tid + q * BE_THREADS < N_QHEAD) query_entry(tid + q * BE_THREADS, &qdcol[q], &qxcol[q]);
     }
 
-    // the lane's (expert, hidden unit) pairs: wave w owns the experts with first sub-key index 3w .. 3w+2; for first
-    // index 3w + r, round c covers second indices 4c .. 4c+3 (one per 16 lanes) x 16 hidden units.  Per pair: the
+    // the lane's (expert, hidden unit) pairs: wave w owns the experts with first sub-key index 6w .. 6w+5; for first
+    // index 6w + r, round c covers second indices 4c .. 4c+3 (one per 16 lanes) x 16 hidden units.  Per pair: the
     // expert's W1, b1 entry and three sums over elements of t = (routing weight if the unit is active else 0):
     // sum t, sum t*g, sum t*pre, from which d b1 = W2*sum t, d W1 = W2*sum t*g, d W2 = sum t*pre.
-    constexpr int KA_PER_WAVE = PK / 4, ROUNDS = PK / 4;
+    constexpr int KA_PER_WAVE = PK / BE_WAVES, ROUNDS = PK / 4;
     static_assert(KA_PER_WAVE * ROUNDS == EXP_PER_LANE, "pairs per lane");
     const int ka0 = __builtin_amdgcn_readfirstlane(KA_PER_WAVE * (tid >> 6));
     const int kb_sub = (tid & 63) >> 4;
@@ -280,12 +290,46 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     ra[0] += ia == 0 ? oa : 0.0f; ra[1] += ia == 1 ? oa : 0.0f; ra[2] += ia == 2 ? oa : 0.0f; ra[3] += ia == 3 ? oa : 0.0f;
                     rb[0] += ib == 0 ? ob : 0.0f; rb[1] += ib == 1 ? ob : 0.0f; rb[2] += ib == 2 ? ob : 0.0f; rb[3] += ib == 3 ? ob : 0.0f;
                 }
+                total += head_out;
+                // routing backward: softmax, scores, keys, query
+                float dq[DM];
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    float* gk = s_gkey + (hf * NH + hh) * PK * (DM / 2);
+                    float mean = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) mean = sg_fma(wgt[hf][k], kk * (hf ? rb[k] : ra[k]), mean);
+#pragma unroll
+                    for (int dd = 0; dd < DM / 2; dd++) dq[hf * (DM / 2) + dd] = 0.0f;
+#pragma unroll
+                    for (int k = 0; k < TOPK; k++) {
+                        const float dv = 10.0f * wgt[hf][k] * (kk * (hf ? rb[k] : ra[k]) - mean);
+                        const int row = idx[hf][k];
+#pragma unroll
+                        for (int dd = 0; dd < DM / 2; dd++) {
+                            dq[hf * (DM / 2) + dd] = sg_fma(dv, keys[row * (DM / 2) + dd], dq[hf * (DM / 2) + dd]);
+                            atomicAdd(&gk[row * (DM / 2) + dd], dv * query[hf * (DM / 2) + dd]);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int dd = 0; dd < DM; dd++) {
+                    drow[dd] = dq[dd];
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
+#pragma unroll
+                    for (int q = 0; q < GH; q++) dhn[q] = sg_fma(qr[q], dq[dd], dhn[q]);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) dcf[q] = sg_fma(qr[GH + q], dq[dd], dcf[q]);
+#pragma unroll
+                    for (int q = 0; q < DM; q++) dcb[q] = sg_fma(qr[GH + DM + q], dq[dd], dcb[q]);
+                }
                 // Expert gradients.  The weight an element gives expert (ka, kb) of this head is the product
                 // (d loss/d head * wa)[ka] * wb[kb] of two 12-vectors with four non-zeros each, which every lane has
                 // just staged.  Scattering the 16 x 49 contributions of an element with LDS float atomics is far too
                 // slow (they retire about one lane per clock), and neighbours in element order share no routing, so
-                // the sums are gathered instead: a lane owns nine fixed (expert, hidden unit) pairs, keeps their sums
-                // in registers, and walks the tile's 256 elements.  A wave's pairs belong to three first indices:
+                // the sums are gathered instead: a lane owns 18 fixed (expert, hidden unit) pairs, keeps their sums
+                // in registers, and walks the tile's 128 elements.  A wave's pairs belong to six first indices:
                 // those the element did not pick are skipped with a scalar branch on the element's staged mask.
                 __syncthreads();
                 {
@@ -328,41 +372,20 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                         add(v1);
                     }
                 }
-                __syncthreads();
-                total += head_out;
-                // routing backward: softmax, scores, keys, query
-                float dq[DM];
+                // this head's query-matrix gradients: d query (x) query input over the tile's elements
+                {
+                    float qs[Q_PER_LANE];
 #pragma unroll
-                for (int hf = 0; hf < 2; hf++) {
-                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
-                    float* gk = s_gkey + (hf * NH + hh) * PK * (DM / 2);
-                    float mean = 0.0f;
+                    for (int q = 0; q < Q_PER_LANE; q++) qs[q] = 0.0f;
+                    for (int e = 0; e < BE_THREADS; e++) {
 #pragma unroll
-                    for (int k = 0; k < TOPK; k++) mean = sg_fma(wgt[hf][k], kk * (hf ? rb[k] : ra[k]), mean);
-#pragma unroll
-                    for (int dd = 0; dd < DM / 2; dd++) dq[hf * (DM / 2) + dd] = 0.0f;
-#pragma unroll
-                    for (int k = 0; k < TOPK; k++) {
-                        const float dv = 10.0f * wgt[hf][k] * (kk * (hf ? rb[k] : ra[k]) - mean);
-                        const int row = idx[hf][k];
-#pragma unroll
-                        for (int dd = 0; dd < DM / 2; dd++) {
-                            dq[hf * (DM / 2) + dd] = sg_fma(dv, keys[row * (DM / 2) + dd], dq[hf * (DM / 2) + dd]);
-                            atomicAdd(&gk[row * (DM / 2) + dd], dv * query[hf * (DM / 2) + dd]);
-                        }
+                        for (int q = 0; q < Q_PER_LANE; q++) qs[q] = sg_fma(s_d[e * DW + qdcol[q]], s_x[e * XW + qxcol[q]], qs[q]);
                     }
+#pragma unroll
+                    for (int q = 0; q < Q_PER_LANE; q++)
+                        if (tid + q * BE_THREADS < N_QHEAD) s_gq[hh * N_QHEAD + tid + q * BE_THREADS] += qs[q];      // one owner per entry
                 }
-#pragma unroll
-                for (int dd = 0; dd < DM; dd++) {
-                    drow[D_Q + hh * DM + dd] = dq[dd];
-                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
-#pragma unroll
-                    for (int q = 0; q < GH; q++) dhn[q] = sg_fma(qr[q], dq[dd], dhn[q]);
-#pragma unroll
-                    for (int q = 0; q < DM; q++) dcf[q] = sg_fma(qr[GH + q], dq[dd], dcf[q]);
-#pragma unroll
-                    for (int q = 0; q < DM; q++) dcb[q] = sg_fma(qr[GH + DM + q], dq[dd], dcb[q]);
-                }
+                __syncthreads();
             }
             if (valid && a.smart != nullptr) a.smart[i] = sg_fma(a.rescale, total / (float)NH, g);
 
@@ -402,10 +425,10 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             }
         }
         __syncthreads();
-        // ---- dense gradients: each lane's entries, summed over the tile's elements
+        // ---- GRU gradients: each lane's entries, summed over the tile's elements
         for (int e = 0; e < BE_THREADS; e++) {
 #pragma unroll
-            for (int q = 0; q < DENSE_PER_LANE; q++) dense[q] = sg_fma(s_d[e * DW + dcol[q]], s_x[e * XW + xcol[q]], dense[q]);
+            for (int q = 0; q < GRU_PER_LANE; q++) gsum[q] = sg_fma(s_d[e * DW + gdcol[q]], s_x[e * XW + gxcol[q]], gsum[q]);
         }
         __syncthreads();
     }
@@ -413,10 +436,12 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     // ---- this workgroup's sums -> its row of the partials buffer
     float* out = a.partials + (size_t)blockIdx.x * N_GRADS;
 #pragma unroll
-    for (int q = 0; q < DENSE_PER_LANE; q++) {
+    for (int q = 0; q < GRU_PER_LANE; q++) {
         const int o = tid + q * BE_THREADS;
-        if (o < N_DENSE) out[o] = dense[q];
+        if (o < N_GRU) out[o] = gsum[q];
     }
+    __syncthreads();
+    for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) out[N_GRU + i] = s_gq[i];
     for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) out[OFF_KA + i] = s_gkey[i];
 #pragma unroll
     for (int q = 0; q < EXP_PER_LANE; q++) {
@@ -445,9 +470,9 @@ __global__ __launch_bounds__(256) void k_sum_partials(const float* __restrict__ 
     if (slice == 0 && o < N_GRADS) out[o] = ((s_part[0][col] + s_part[1][col]) + s_part[2][col]) + s_part[3][col];
 }
 
-constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW));
-static_assert(BE_LDS_BYTES <= 160 * 1024, "LDS of k_bilevel_elem");
-constexpr int BE_MAX_GROUPS = 512;
+constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD);
+static_assert(2 * BE_LDS_BYTES <= 160 * 1024, "two workgroups of k_bilevel_elem per CU");
+constexpr int BE_MAX_GROUPS = 1024;
 
 int elem_groups(int64_t total) {
     const int64_t tiles = (total + BE_THREADS - 1) / BE_THREADS;
