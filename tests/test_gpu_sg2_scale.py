@@ -61,3 +61,64 @@ def test_scale50_properties_and_determinism():
         for x, y in zip(a, b):
             assert torch.equal(x, y)
     assert torch.equal(counts, again[8])
+
+
+def test_bilevel_pass_at_scale_linearity_and_chunking():
+    """The bilevel meta-gradient pass on the full 50-tensor set (25 M elements, up to 1024 chunks per tensor), through
+    properties that do not need a CPU answer: the gradients are linear in the cotangent; a different chunk length
+    (another decomposition of the same sums) gives the same result; everything except the product-key gradients
+    (LDS atomics) repeats bit for bit."""
+    from grokking_optimizers import Mamba3PEERMetaNet, _bilevel, _cabi
+    dev = torch.device("cuda:0")
+    shapes = wl.scale50_shapes()
+    torch.manual_seed(11)
+    mn = Mamba3PEERMetaNet().to(dev)
+    with torch.no_grad():
+        for p in mn.parameters():
+            if p.dim() > 0 and float(p.abs().max()) < 0.05:
+                p.add_(torch.randn_like(p) * 0.2)
+    grads = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=3, std=0.3)]
+    sharps = [g.abs() * 0.5 for g in grads]
+    gen = torch.Generator().manual_seed(4)
+    grus = [(torch.randn(g.numel(), 4, generator=gen) * 0.5).to(dev) for g in grads]
+    mf = [(torch.randn(16, 16, generator=gen) * 0.3).to(dev) for _ in grads]
+    mb = [(torch.randn(16, 16, generator=gen) * 0.3).to(dev) for _ in grads]
+    c1 = [torch.randn(g.numel(), generator=gen).to(dev) for g in grads]
+    c2 = [torch.randn(g.numel(), generator=gen).to(dev) for g in grads]
+
+    def run(cots):
+        mn.zero_grad()
+        smart = _bilevel.accumulate_meta_gradients(mn, grads, sharps, grus, mf, mb, cots)
+        torch.cuda.synchronize()
+        return smart, {n: p.grad.clone() for n, p in mn.named_parameters()}
+
+    print("bilevel at scale: cotangent 1", flush=True)
+    s1, g1 = run(c1)
+    print("bilevel at scale: cotangent 2", flush=True)
+    s2, g2 = run(c2)
+    print("bilevel at scale: sum of both", flush=True)
+    s3, g3 = run([a + b for a, b in zip(c1, c2)])
+    assert torch.equal(s1, s2) and torch.equal(s1, s3) and bool(torch.isfinite(s1).all())     # smart does not depend on the cotangent
+    for n in g1:
+        want = g1[n].double() + g2[n].double()
+        scale = float(want.abs().max())
+        assert bool(torch.isfinite(g3[n]).all()) and scale > 0, n
+        assert float((g3[n].double() - want).abs().max()) <= 2e-4 * scale, (n, scale)
+    print("bilevel at scale: repeat", flush=True)
+    s1b, g1b = run(c1)
+    assert torch.equal(s1, s1b)
+    for n in g1:
+        if "product_keys" in n:
+            assert float((g1[n] - g1b[n]).abs().max()) <= 1e-5 * float(g1[n].abs().max()), n
+        else:
+            assert torch.equal(g1[n], g1b[n]), n
+    print("bilevel at scale: chunk length 1024", flush=True)
+    assert _cabi.lib().sg2_set_chunk_len(1024) == 0
+    try:
+        s1c, g1c = run(c1)
+    finally:
+        _cabi.lib().sg2_set_chunk_len(0)
+    assert float((s1c - s1).abs().max()) <= 1e-4 * float(s1.abs().max())
+    for n in g1:
+        scale = float(g1[n].abs().max())
+        assert float((g1c[n].double() - g1[n].double()).abs().max()) <= 2e-4 * scale, (n, scale)
