@@ -218,6 +218,32 @@ def bench_other(args, dev):
     return out
 
 
+def class_step_ms(shapes, grad_sets, dev, steps, warmup):
+    """Wall time of SuperGrok2.step() itself (per-tensor clip on the device, scalar schedules, the 51-argument
+    `_ops` call), same tensors and gradients, the module's own initial meta-weights, recycling off."""
+    import torch
+    from grokking_optimizers import SuperGrok2
+    import workloads as wl
+    params = [torch.nn.Parameter(p.to(dev)) for p in wl.make_params(shapes, seed=0)]
+    opt = SuperGrok2(params, lr=1e-3, recycle_interval=0)
+    t = 0
+
+    def one():
+        nonlocal t
+        t += 1
+        for p, g in zip(params, grad_sets[t & 1]):
+            p.grad = g.view(p.shape)
+        opt.step()
+    for _ in range(warmup):
+        one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    return 1e3 * (time.perf_counter() - t0) / steps
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -303,6 +329,7 @@ def main():
         "step_valu_frac": FLOP_PER_ELEMENT * value / 1e12 / VALU_PEAK_TFLOPS,
         "stage_ms": stage_avg,
     }
+    out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
