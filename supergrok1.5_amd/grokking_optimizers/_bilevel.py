@@ -98,13 +98,15 @@ def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
 
 
 def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
-    """Differentiable forward of one tensor: (smart_grad, new_gru); gradients reach every parameter of `mn`."""
+    """Differentiable forward of one tensor, the reference's return values: (smart_grad, new_gru, new_mamba_fwd_state,
+    new_mamba_bwd_state); gradients reach every parameter of `mn` (the two new states are plain tensors: nothing in
+    the reference differentiates through them)."""
     g = grad.reshape(-1).float()
     s = sharpness.reshape(-1).float()
     plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
     ctx = ScanContexts.apply(plan, *scan_parameters(mn))
     smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float())
-    return smart.reshape(grad.shape).to(grad.dtype), h_new
+    return smart.reshape(grad.shape).to(grad.dtype), h_new, plan.mf[0], plan.mb[0]
 
 
 def elem_parameters(mn):

@@ -7,8 +7,10 @@ layout the fused step consumes, and `_recycle_dead_experts` (:437-491 there)
 is the host-side expert recycling.
 
 The arithmetic of the network runs inside the fused HIP step
-(`_ops.supergrok2_mamba_peer_batched_step`); this module has no forward pass
-of its own.
+(`_ops.supergrok2_mamba_peer_batched_step`); this module has no `forward` of
+its own.  `forward_for_bilevel` (:372-436 there) is the differentiable variant
+with soft top-4 routing: sort and scan in HIP (forward and adjoint), the
+per-element part as torch ops.
 """
 import math
 
@@ -92,6 +94,12 @@ class Mamba3PEERMetaNet(nn.Module):
                  pk_dim=self.pk_dim, expert_hidden=self.expert_hidden, gru_hidden=self.gru_hidden,
                  num_peer_heads=self.num_peer_heads, num_experts=self.num_experts)
         return w
+
+    def forward_for_bilevel(self, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
+        """(smart_grad, new_gru_state, new_mamba_fwd_state, new_mamba_bwd_state), differentiable with respect to
+        every parameter of the module; GPU tensors only."""
+        from grokking_optimizers import _bilevel
+        return _bilevel.forward_for_bilevel(self, grad, sharpness, gru_state, mamba_fwd_state, mamba_bwd_state)
 
     def flat_weights(self):
         """The 33 tensors in the argument order of _ops.supergrok2_mamba_peer_batched_step."""

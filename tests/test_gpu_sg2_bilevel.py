@@ -122,8 +122,8 @@ def _ref_forward_for_bilevel(mn, grad, sharp, gru_state, hf, hb):
     x = mn.input_proj(torch.stack([g[perm], s[perm]], -1))
     blk = lambda b: [b.in_proj.weight, b.dt_proj.weight, b.dt_proj.bias, b.B_proj.weight, b.C_proj.weight, b.A_log, b.D,
                      b.rope_freq, b.out_proj.weight]
-    fo, _ = ref_fp64.scan_block(x, blk(mn.mamba_fwd), hf)
-    bo, _ = ref_fp64.scan_block(x.flip(0), blk(mn.mamba_bwd), hb)
+    fo, new_f = ref_fp64.scan_block(x, blk(mn.mamba_fwd), hf)
+    bo, new_b = ref_fp64.scan_block(x.flip(0), blk(mn.mamba_bwd), hb)
     unsort = torch.argsort(perm)
     cf, cb = fo[unsort], bo.flip(0)[unsort]
     xin = torch.cat([g[:, None], s[:, None], cf, cb], -1)
@@ -145,7 +145,7 @@ def _ref_forward_for_bilevel(mn, grad, sharp, gru_state, hf, hb):
         zz = torch.relu(torch.matmul(W1, gx).squeeze(-1) + b1)
         out = torch.matmul(W2, zz.unsqueeze(-1)).squeeze(-1).squeeze(-1) + b2.squeeze(-1)
         total = total + (rw * out).sum(1, keepdim=True)
-    return (g[:, None] + mn.rescale * total / mn.num_peer_heads).squeeze(-1), hn
+    return (g[:, None] + mn.rescale * total / mn.num_peer_heads).squeeze(-1), hn, new_f, new_b
 
 
 def _meta_net(seed, dev):
@@ -191,11 +191,11 @@ def test_differentiable_forward_of_the_whole_meta_net():
     for k, d in enumerate(data):
         mn.zero_grad()
         mn64.zero_grad()
-        smart, hn = _bilevel.forward_for_bilevel(mn, d["g"].to(dev), d["s"].to(dev), d["h"].to(dev), d["hf"].to(dev), d["hb"].to(dev))
+        smart, hn, nf, nb = mn.forward_for_bilevel(d["g"].to(dev), d["s"].to(dev), d["h"].to(dev), d["hf"].to(dev), d["hb"].to(dev))
         (smart * d["R"].to(dev)).sum().backward()
-        rs, rh = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
+        rs, rh, rf, rb = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
         (rs * d["R"].double()).sum().backward()
-        for name, got, ref in (("smart", smart, rs), ("gru", hn, rh)):
+        for name, got, ref in (("smart", smart, rs), ("gru", hn, rh), ("mamba_fwd", nf, rf), ("mamba_bwd", nb, rb)):
             got, ref = got.detach().double().cpu(), ref.detach()
             err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
             assert bool((err <= tol).all()), (name, k, float((err / tol).max()))
