@@ -71,7 +71,8 @@ def make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd):
 def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
     """GRU, soft top-k product-key routing (softmax of 10 x the k best scores of each sub-key, k*k experts per head)
     and the expert MLPs for N elements: smart gradient [N] and new GRU state
-    (reference: Mamba3PEERMetaNet.forward_for_bilevel, mamba3_peer_metanet.py:395-436; GRU :178-192)."""
+    (reference: Mamba3PEERMetaNet.forward_for_bilevel, mamba3_peer_metanet.py:395-436; GRU :178-192).
+    topk=0: the hard top-1 routing of the optimizer step (Mamba3PEERMetaNet.forward, :319-367 there)."""
     gru = mn.gru
     xin = torch.cat([g.unsqueeze(-1), s.unsqueeze(-1), ctx_f, ctx_b], dim=-1)
     xh = torch.cat([xin, gru_state], dim=-1)
@@ -86,6 +87,10 @@ def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
     total = torch.zeros(N, device=g.device, dtype=torch.float32)
     for h in range(mn.num_peer_heads):
         q = mn.peer_queries[h](pin)
+        if topk == 0:
+            e = (q[:, :half] @ mn.product_keys_A[h].T).argmax(dim=-1) * pk + (q[:, half:] @ mn.product_keys_B[h].T).argmax(dim=-1)
+            total = total + (W2[e] * torch.relu(W1[e] * g.unsqueeze(-1) + b1[e])).sum(-1) + b2[e]
+            continue
         va, ia = (q[:, :half] @ mn.product_keys_A[h].T).topk(topk, dim=-1)
         vb, ib = (q[:, half:] @ mn.product_keys_B[h].T).topk(topk, dim=-1)
         wa, wb = torch.softmax(va * 10.0, dim=-1), torch.softmax(vb * 10.0, dim=-1)
@@ -95,6 +100,17 @@ def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
         out = (W2[idx] * act).sum(-1) + b2[idx]
         total = total + (route * out).sum(dim=1)
     return g + mn.rescale * (total / mn.num_peer_heads), h_new
+
+
+def forward(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
+    """The step's own forward (hard top-1 routing) as a module call, for callers that use the meta-net outside the
+    fused step: same return values as the reference's Mamba3PEERMetaNet.forward."""
+    g = grad.reshape(-1).float()
+    s = sharpness.reshape(-1).float()
+    plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
+    ctx = ScanContexts.apply(plan, *scan_parameters(mn))
+    smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float(), topk=0)
+    return smart.reshape(grad.shape).to(grad.dtype), h_new, plan.mf[0], plan.mb[0]
 
 
 def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):

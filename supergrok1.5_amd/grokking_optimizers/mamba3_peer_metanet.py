@@ -7,10 +7,10 @@ layout the fused step consumes, and `_recycle_dead_experts` (:437-491 there)
 is the host-side expert recycling.
 
 The arithmetic of the network runs inside the fused HIP step
-(`_ops.supergrok2_mamba_peer_batched_step`); this module has no `forward` of
-its own.  `forward_for_bilevel` (:372-436 there) is the differentiable variant
-with soft top-4 routing: sort and scan in HIP (forward and adjoint), the
-per-element part as torch ops.
+(`_ops.supergrok2_mamba_peer_batched_step`).  `forward` (:275-370 there) and
+`forward_for_bilevel` (:372-436 there, soft top-4 routing) are kept for callers
+that use the module outside the optimizer: sort and scan in HIP (forward and
+adjoint), the per-element part as torch ops; GPU tensors only.
 """
 import math
 
@@ -94,6 +94,12 @@ class Mamba3PEERMetaNet(nn.Module):
                  pk_dim=self.pk_dim, expert_hidden=self.expert_hidden, gru_hidden=self.gru_hidden,
                  num_peer_heads=self.num_peer_heads, num_experts=self.num_experts)
         return w
+
+    def forward(self, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
+        """(smart_grad, new_gru_state, new_mamba_fwd_state, new_mamba_bwd_state) with the step's hard top-1 routing.
+        Unlike the reference it does not update expert_counts: only the fused step does."""
+        from grokking_optimizers import _bilevel
+        return _bilevel.forward(self, grad, sharpness, gru_state, mamba_fwd_state, mamba_bwd_state)
 
     def forward_for_bilevel(self, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
         """(smart_grad, new_gru_state, new_mamba_fwd_state, new_mamba_bwd_state), differentiable with respect to

@@ -273,3 +273,26 @@ def test_optimizer_bilevel_step_and_step_full():
             losses.append(float(crit(model(xs), ys)))
     print("step_full losses", [round(v, 4) for v in losses], flush=True)
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
+
+
+def test_module_forward_matches_the_float64_step():
+    """Mamba3PEERMetaNet.forward (hard top-1 routing, HIP scan + torch per-element part) against the float64
+    restatement of the step: smart gradient, new GRU state, both new Mamba states; expert choices may differ only at
+    near-ties, which the tolerance on smart (1e-4 of its scale) would expose."""
+    dev = torch.device("cuda:0")
+    mn = _meta_net(21, dev)
+    gen = torch.Generator().manual_seed(22)
+    n = 333
+    g, s = torch.randn(n, generator=gen) * 0.5, torch.rand(n, generator=gen) * 0.3
+    h = torch.randn(n, 4, generator=gen) * 0.5
+    hf, hb = torch.randn(16, 16, generator=gen) * 0.3, torch.randn(16, 16, generator=gen) * 0.3
+    print("module forward, N", n, flush=True)
+    smart, hn, nf, nb = mn(g.to(dev), s.to(dev), h.to(dev), hf.to(dev), hb.to(dev))
+    dims = dict(d_model=8, gru_hidden=4, num_heads=4, pk_dim=12)
+    sc = dict(rescale=mn.rescale, alpha=0.0, lamb_eff=0.0, beta1=0.9, beta2=0.999, bc1=1.0, bc2=1.0, eps=1e-8, lr=0.0, wd_eff=0.0)
+    z = torch.zeros(n)
+    ref = ref_fp64.step([w.cpu() for w in mn.flat_weights()], z, g, s, z, z, z, h, hf, hb, sc, dims)
+    for name, got, want in (("smart", smart, ref["smart"]), ("gru", hn, ref["gru"]), ("mamba_fwd", nf, ref["mamba_fwd"]),
+                            ("mamba_bwd", nb, ref["mamba_bwd"])):
+        got = got.detach().double().cpu()
+        assert float((got - want).abs().max()) <= 1e-4 * float(want.abs().max()) + 1e-7, name
