@@ -12,16 +12,15 @@
 // workgroup's passes over its tile overlap the other's per-element arithmetic).  Nothing is kept between forward and backward:
 // a lane holds its element's activations in registers, and the routing of a head is differentiated before the
 // next head is evaluated.  Weight gradients are sums over elements:
-//   * product keys (rows chosen per element): float atomics on accumulators in LDS;
 //   * experts (16 per element and head, chosen per element): gathered, not scattered.  Each lane owns 18
 //     (expert, hidden unit) pairs with their sums in registers and walks the tile's elements, whose routing
 //     weights of the head every lane has left in LDS as two 12-vectors (see the expert-gradient pass);
 //   * GRU and query matrices (dense outer products d (x) x): every lane leaves its x (31 values) and, per head
 //     and once more for the GRU, its d (8 / 12 values) in LDS; each lane of the workgroup owns up to two entries
-//     of the head's query matrix and three of the GRU matrices and sums their products over the tile's elements.
+//     of the head's query matrix and three of the GRU matrices and sums their products over the tile's elements;
+//   * product keys (rows chosen per element): the same, with d score scattered into a 12-vector per sub-key.
 // Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
-// order.  (Within a workgroup the LDS atomics arrive in no fixed order, so the key gradients can differ in the last
-// bits between runs; everything else is summed in a fixed order.)
+// order.  No atomics anywhere: every sum is formed in a fixed order and the result repeats bit for bit.
 #include "sg2_internal.hpp"
 
 namespace sg2 {
@@ -291,12 +290,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     rb[0] += ib == 0 ? ob : 0.0f; rb[1] += ib == 1 ? ob : 0.0f; rb[2] += ib == 2 ? ob : 0.0f; rb[3] += ib == 3 ? ob : 0.0f;
                 }
                 total += head_out;
-                // routing backward: softmax, scores, keys, query
-                float dq[DM];
+                // routing backward: softmax, scores, query (the product keys' own gradients: see the end of the head)
+                float dq[DM], dv[2][TOPK];
 #pragma unroll
                 for (int hf = 0; hf < 2; hf++) {
                     const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
-                    float* gk = s_gkey + (hf * NH + hh) * PK * (DM / 2);
                     float mean = 0.0f;
 #pragma unroll
                     for (int k = 0; k < TOPK; k++) mean = sg_fma(wgt[hf][k], kk * (hf ? rb[k] : ra[k]), mean);
@@ -304,13 +302,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     for (int dd = 0; dd < DM / 2; dd++) dq[hf * (DM / 2) + dd] = 0.0f;
 #pragma unroll
                     for (int k = 0; k < TOPK; k++) {
-                        const float dv = 10.0f * wgt[hf][k] * (kk * (hf ? rb[k] : ra[k]) - mean);
+                        dv[hf][k] = 10.0f * wgt[hf][k] * (kk * (hf ? rb[k] : ra[k]) - mean);
                         const int row = idx[hf][k];
 #pragma unroll
-                        for (int dd = 0; dd < DM / 2; dd++) {
-                            dq[hf * (DM / 2) + dd] = sg_fma(dv, keys[row * (DM / 2) + dd], dq[hf * (DM / 2) + dd]);
-                            atomicAdd(&gk[row * (DM / 2) + dd], dv * query[hf * (DM / 2) + dd]);
-                        }
+                        for (int dd = 0; dd < DM / 2; dd++)
+                            dq[hf * (DM / 2) + dd] = sg_fma(dv[hf][k], keys[row * (DM / 2) + dd], dq[hf * (DM / 2) + dd]);
                     }
                 }
 #pragma unroll
@@ -384,6 +380,25 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 #pragma unroll
                     for (int q = 0; q < Q_PER_LANE; q++)
                         if (tid + q * BE_THREADS < N_QHEAD) s_gq[hh * N_QHEAD + tid + q * BE_THREADS] += qs[q];      // one owner per entry
+                }
+                __syncthreads();
+                // product-key gradients, d score (x) query half, the same way: the staged rows are free now, so each
+                // lane leaves d score as two 12-vectors (four non-zeros each) and its query; 96 lanes own one entry each
+#pragma unroll
+                for (int k = 0; k < 2 * PK; k++) rtrow[k] = 0.0f;
+#pragma unroll
+                for (int k = 0; k < TOPK; k++) {
+                    rtrow[idx[0][k]] = dv[0][k];
+                    rtrow[PK + idx[1][k]] = dv[1][k];
+                }
+#pragma unroll
+                for (int dd = 0; dd < DM; dd++) drow[dd] = query[dd];
+                __syncthreads();
+                if (tid < 2 * PK * (DM / 2)) {
+                    const int hf = tid / (PK * (DM / 2)), row = (tid / (DM / 2)) % PK, dd = tid % (DM / 2);
+                    float acc = 0.0f;
+                    for (int e = 0; e < BE_THREADS; e++) acc = sg_fma(s_rt[e * RW + hf * PK + row], s_d[e * DW + hf * (DM / 2) + dd], acc);
+                    s_gkey[(hf * NH + hh) * PK * (DM / 2) + row * (DM / 2) + dd] += acc;
                 }
                 __syncthreads();
             }
