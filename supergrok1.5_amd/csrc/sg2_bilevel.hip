@@ -131,9 +131,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
     const int j = tid >> 3, p = tid & 7;
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
-    float u1e = 1.0f, u1o = 0.0f, u2e = 0.0f, u2o = 1.0f, ve = 0.0f, vo = 0.0f;
+    if (chunk == pl.chunk_prefix[c.ti]) return;    // nothing lies before a tensor's first chunk: its map is never applied
+    float u1e, u1o, u2e, u2o, ve, vo;
     const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
-    for (int tile = ntiles - 1; tile >= 0; tile--) {
+    // The map contracts like the forward recurrence, so - as in the forward summary pass - it is first taken over the
+    // `window` steps at the start of the chunk only (the end of this reverse sweep).  If every entry of that matrix,
+    // in all 128 lanes, is below 2^-100, whatever arrives from later steps is multiplied by less than that: the
+    // chunk's map is (0, v_window).  Otherwise the whole chunk is swept.
+    const int wtiles = (pl.window > 0) ? pl.window / SCAN_TT : 0;
+    int first_tile = (wtiles > 0 && ntiles > wtiles) ? wtiles - 1 : ntiles - 1;
+    for (;;) {
+      u1e = 1.0f; u1o = 0.0f; u2e = 0.0f; u2o = 1.0f; ve = 0.0f; vo = 0.0f;
+      for (int tile = first_tile; tile >= 0; tile--) {
         const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
         {
             const bool valid = tu < cnt;
@@ -172,6 +181,11 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
         }
         __syncthreads();
     }
+      if (first_tile == ntiles - 1) break;
+      const float big = sg_max(sg_max(sg_abs(u1e), sg_abs(u1o)), sg_max(sg_abs(u2e), sg_abs(u2o)));
+      if (__syncthreads_and(big < 0x1p-100f)) { u1e = u1o = u2e = u2o = 0.0f; break; }
+      first_tile = ntiles - 1;
+    }
     float* out = pl.adj_summ + (((size_t)dir * pl.chunks + chunk) * SCAN_THREADS + tid) * 6;
     out[0] = u1e; out[1] = u1o; out[2] = u2e; out[3] = u2o; out[4] = ve; out[5] = vo;
 }
@@ -185,6 +199,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_prefix(Plan pl) {
         const size_t at = ((size_t)dir * pl.chunks + base + c) * SCAN_THREADS + tid;
         pl.adj_lam[at * 2] = le;
         pl.adj_lam[at * 2 + 1] = lo;
+        if (c == 0) break;
         const float* m = pl.adj_summ + at * 6;
         const float ne = sg_fma(m[0], le, sg_fma(m[2], lo, m[4]));
         const float no = sg_fma(m[1], le, sg_fma(m[3], lo, m[5]));

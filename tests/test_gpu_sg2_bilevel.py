@@ -40,13 +40,17 @@ def _reference(W, grads, sharps, mf, mb, R):
     return ctx, [w.grad for w in Wd]
 
 
-def _case(shapes, seed, sharp, state_std, chunk_len=None):
+def _case(shapes, seed, sharp, state_std, chunk_len=None, a_log=None):
     from grokking_optimizers import _bilevel, _cabi
     dev = torch.device("cuda:0")
     if chunk_len is not None:
         assert _cabi.lib().sg2_set_chunk_len(chunk_len) == 0
     try:
-        W = [w.to(dev) for w in wl.meta_weights(seed)]
+        W = wl.meta_weights(seed)
+        if a_log is not None:
+            for base in (2, 11):
+                W[base + 5].fill_(a_log)
+        W = [w.to(dev) for w in W]
         grads = [g.to(dev) for g in wl.make_grads(shapes, seed=seed + 1, std=0.5)]
         sharps = [(g.abs() * 0.5).to(dev) if sharp else torch.zeros_like(g, device=dev)
                   for g in wl.make_grads(shapes, seed=seed + 2, std=0.5)]
@@ -103,6 +107,12 @@ def test_automatic_chunk_length_on_longer_tensors():
     """5000 + 3000 elements at the chunk length the library picks by itself (several chunks per tensor, partial last
     tiles): the chunk-parallel adjoint (summaries, prefix, replay) against float64 autograd."""
     _case([(5000,), (3000,)], seed=14, sharp=True, state_std=0.3)
+
+
+def test_barely_contracting_poles_fall_back_to_whole_chunk_summaries():
+    """A_log = -12: A_bar stays within 1e-5 of 1, so neither the forward nor the adjoint summary may be taken over a
+    window; both must redo the whole chunk (chunk length 512, window 256)."""
+    _case([(3000,), (1500,)], seed=16, sharp=True, state_std=0.3, chunk_len=512, a_log=-12.0)
 
 
 def test_several_chunks():
