@@ -47,7 +47,7 @@ constexpr int BT = HT_STEP;
 constexpr int BBST = BT + 1;                     // row stride of its [16][BT] arrays (odd: the 16 rows a step reads hit 16 banks)
 constexpr int LDS_ROWS_FLOATS = A_COUNT * ROWS * BBST;
 constexpr int LDS_H_FLOATS = BT * SCAN_THREADS * 2;               // state after every step of the tile
-constexpr int LDS_MISC_FLOATS = BT * DM + BT * 2;                 // d ctx tile, (g, s) of the tile
+constexpr int LDS_MISC_FLOATS = BT * DM + BT * 2 + DI;            // d ctx tile, (g, s) of the tile, per-column frequency bound
 static_assert(SCAN_THREADS == 4 * BT && ROWS % 4 == 0 && (LDS_ROWS_FLOATS + LDS_H_FLOATS) % 4 == 0, "projection roles, float4 alignment");
 constexpr int BILEVEL_LDS_BYTES = 4 * (LDS_ROWS_FLOATS + LDS_H_FLOATS + LDS_MISC_FLOATS);
 
@@ -106,6 +106,21 @@ __device__ __forceinline__ void load_step(const ChunkRef& c, int dir, int u, boo
     }
 }
 
+// sin/cos of a rotation angle; `tiny` (uniform over the workgroup) says that every angle of the tile is below the limit
+// of the short polynomial pair, which the forward pass uses for such blocks as well
+__device__ __forceinline__ void rot_sincos(bool tiny, float th, float* sn, float* cs) {
+    if (tiny) sg_sincos_tiny(th, sn, cs); else sg_sincos(th, sn, cs);
+}
+// per column, the largest |rope frequency| of its 8 pairs (dt >= 0: dt*fmax bounds every angle of the column)
+__device__ __forceinline__ void fill_fmax(float* s_fmax, const float* __restrict__ rope) {
+    if (threadIdx.x < DI) {
+        float m = 0.0f;
+        for (int p = 0; p < HP; p++) m = sg_max(m, sg_abs(rope[threadIdx.x * HP + p]));
+        s_fmax[threadIdx.x] = m;
+    }
+    __syncthreads();
+}
+
 // lambda -> R(theta)^T diag(A_bar) lambda for one lane's pair
 __device__ __forceinline__ void adj_apply(float ae, float ao, float sn, float cs, float* xe, float* xo) {
     const float dre = *xe * ae, dro = *xo * ao;
@@ -118,6 +133,7 @@ constexpr int SUMM_ROWS = 4;                     // LDS arrays of the summary ke
 __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const float* __restrict__ d_ctx) {
     __shared__ float rows[SUMM_ROWS * ROWS * BST];
     __shared__ __attribute__((aligned(16))) float s_dctx[SCAN_TT * DM];
+    __shared__ float s_fmax[DI];
     auto arr = [&](int a) { return rows + a * ROWS * BST; };
     const int chunk = blockIdx.x, dir = blockIdx.y;
     const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
@@ -132,6 +148,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
     if (chunk == pl.chunk_prefix[c.ti]) return;    // nothing lies before a tensor's first chunk: its map is never applied
+    fill_fmax(s_fmax, rope);
     float u1e, u1o, u2e, u2o, ve, vo;
     const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
     // The map contracts like the forward recurrence, so - as in the forward summary pass - it is first taken over the
@@ -144,6 +161,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
       u1e = 1.0f; u1o = 0.0f; u2e = 0.0f; u2o = 1.0f; ve = 0.0f; vo = 0.0f;
       for (int tile = first_tile; tile >= 0; tile--) {
         const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
+        bool small = true;
         {
             const bool valid = tu < cnt;
             float g, s;
@@ -153,13 +171,15 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
             reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
             for (int q = 0; q < ROWS / 2; q++) {
                 const int r = half * (ROWS / 2) + q;
-                arr(0)[r * BST + tu] = valid ? sg_softplus(sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s)) : 0.0f;
+                const float dtv = valid ? sg_softplus(sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s)) : 0.0f;
+                small = small && (dtv * s_fmax[r] < SG_SINCOS_TINY_LIMIT);
+                arr(0)[r * BST + tu] = dtv;
                 arr(1)[r * BST + tu] = sg2_comp_eval(comp + (SG2_COMP_C * 16 + r) * 3, g, s);
                 const float z = sg2_comp_eval(comp + (SG2_COMP_Z * 16 + r) * 3, g, s);
                 arr(2)[r * BST + tu] = z * sg_sigmoid(z);
             }
         }
-        __syncthreads();
+        const bool tiny = __syncthreads_and(small);
         for (int q = 0; q < ROWS / 2; q++) {
             const int r = half * (ROWS / 2) + q;
             float dout = 0.0f;
@@ -172,7 +192,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
             const float dt = arr(0)[j * BST + k], dy = arr(3)[j * BST + k];
             float ae, ao, sn, cs;
             sg_abar_pair(dt, a_e, a_o, &ae, &ao);
-            sg_sincos(dt * freq, &sn, &cs);
+            rot_sincos(tiny, dt * freq, &sn, &cs);
             ve = sg_fma(dy, arr(1)[(2 * p) * BST + k], ve);
             vo = sg_fma(dy, arr(1)[(2 * p + 1) * BST + k], vo);
             adj_apply(ae, ao, sn, cs, &u1e, &u1o);
@@ -215,6 +235,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     float* sH = lds + LDS_ROWS_FLOATS;
     float* s_dctx = sH + LDS_H_FLOATS;
     float* s_gs = s_dctx + BT * DM;
+    float* s_fmax = s_gs + BT * 2;
     auto arr = [&](int a) { return rows + a * ROWS * BBST; };
 
     const int dir = blockIdx.y;
@@ -231,6 +252,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
 
+    fill_fmax(s_fmax, rope);
     float acc_alog_e = 0.0f, acc_alog_o = 0.0f, acc_rope = 0.0f;
     float acc_c0 = 0.0f, acc_c1 = 0.0f, acc_c2 = 0.0f, acc_D = 0.0f, acc_wout = 0.0f;
     float acc_bc[12];                 // this lane's column share of d B[2p], d B[2p+1], d C[2p], d C[2p+1] against (g, s, 1)
@@ -250,6 +272,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     for (int tile = ntiles - 1; tile >= 0; tile--) {
         const int u0 = c.ustart + tile * BT, cnt = min(BT, c.uend - u0);
         // ---- 1: projections, activation derivatives, incoming gradients
+        bool small = true;
         {
             const bool valid = tu < cnt;
             float g, s;
@@ -263,7 +286,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             for (int q = 0; q < ROWS / 4; q++) {
                 const int r = part * (ROWS / 4) + q;
                 const float raw = sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s);
-                arr(A_DT)[r * BBST + tu] = valid ? sg_softplus(raw) : 0.0f;
+                const float dtv = valid ? sg_softplus(raw) : 0.0f;
+                small = small && (dtv * s_fmax[r] < SG_SINCOS_TINY_LIMIT);
+                arr(A_DT)[r * BBST + tu] = dtv;
                 arr(A_DSP)[r * BBST + tu] = (raw > 20.0f) ? 1.0f : sg_sigmoid(raw);
                 arr(A_XB)[r * BBST + tu] = valid ? sg2_comp_eval(comp + (SG2_COMP_XB * 16 + r) * 3, g, s) : 0.0f;
                 arr(A_B)[r * BBST + tu] = sg2_comp_eval(comp + (SG2_COMP_B * 16 + r) * 3, g, s);
@@ -274,7 +299,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                 arr(A_DGATE)[r * BBST + tu] = sz * sg_fma(z, 1.0f - sz, 1.0f);
             }
         }
-        __syncthreads();
+        const bool tiny = __syncthreads_and(small);
 
         // ---- 2: forward recurrence over the tile, states kept
         const float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, u0)) * 2 * SCAN_THREADS;
@@ -285,7 +310,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                 const float dt = arr(A_DT)[j * BBST + k];
                 float ae, ao, sn, cs;
                 sg_abar_pair(dt, a_e, a_o, &ae, &ao);
-                sg_sincos(dt * freq, &sn, &cs);
+                rot_sincos(tiny, dt * freq, &sn, &cs);
                 const float ux = dt * arr(A_XB)[j * BBST + k];
                 const float re = sg_fma(he, cs, -(ho * sn)), ro = sg_fma(ho, cs, he * sn);
                 he = sg_fma(ae, re, ux * arr(A_B)[(2 * p) * BBST + k]);
@@ -325,7 +350,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             const float po = (k > 0) ? sH[((k - 1) * SCAN_THREADS + tid) * 2 + 1] : hs_o;
             float ae, ao, sn, cs;
             sg_abar_pair(dt, a_e, a_o, &ae, &ao);
-            sg_sincos(dt * freq, &sn, &cs);
+            rot_sincos(tiny, dt * freq, &sn, &cs);
             // y = sum h C
             le = sg_fma(dy, Ce, le);
             lo = sg_fma(dy, Co, lo);
