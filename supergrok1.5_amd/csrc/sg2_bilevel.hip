@@ -253,6 +253,20 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     const float freq = rope[j * HP + p];
 
     fill_fmax(s_fmax, rope);
+    // this lane's rows of the composed coefficients, of out_proj^T and of D, kept in registers: the barriers inside
+    // the tile loop would otherwise make every tile fetch them again
+    float cw[SG2_COMP_GROUPS][ROWS / 4][3], wo[ROWS / 4][DM], dwr[ROWS / 4];
+#pragma unroll
+    for (int q = 0; q < ROWS / 4; q++) {
+        const int r = part * (ROWS / 4) + q;
+#pragma unroll
+        for (int gq = 0; gq < SG2_COMP_GROUPS; gq++)
+#pragma unroll
+            for (int e = 0; e < 3; e++) cw[gq][q][e] = comp[(gq * 16 + r) * 3 + e];
+#pragma unroll
+        for (int d = 0; d < DM; d++) wo[q][d] = Wout[d * DI + r];
+        dwr[q] = Dw[r];
+    }
     float acc_alog_e = 0.0f, acc_alog_o = 0.0f, acc_rope = 0.0f;
     float acc_c0 = 0.0f, acc_c1 = 0.0f, acc_c2 = 0.0f, acc_D = 0.0f, acc_wout = 0.0f;
     float acc_bc[12];                 // this lane's column share of d B[2p], d B[2p+1], d C[2p], d C[2p+1] against (g, s, 1)
@@ -283,17 +297,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                 const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[part] : make_float4(0.f, 0.f, 0.f, 0.f);
                 reinterpret_cast<float4*>(s_dctx + tu * DM)[part] = dv;
             }
+#pragma unroll
             for (int q = 0; q < ROWS / 4; q++) {
                 const int r = part * (ROWS / 4) + q;
-                const float raw = sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s);
+                const float raw = sg2_comp_eval(cw[SG2_COMP_DT][q], g, s);
                 const float dtv = valid ? sg_softplus(raw) : 0.0f;
                 small = small && (dtv * s_fmax[r] < SG_SINCOS_TINY_LIMIT);
                 arr(A_DT)[r * BBST + tu] = dtv;
                 arr(A_DSP)[r * BBST + tu] = (raw > 20.0f) ? 1.0f : sg_sigmoid(raw);
-                arr(A_XB)[r * BBST + tu] = valid ? sg2_comp_eval(comp + (SG2_COMP_XB * 16 + r) * 3, g, s) : 0.0f;
-                arr(A_B)[r * BBST + tu] = sg2_comp_eval(comp + (SG2_COMP_B * 16 + r) * 3, g, s);
-                arr(A_C)[r * BBST + tu] = sg2_comp_eval(comp + (SG2_COMP_C * 16 + r) * 3, g, s);
-                const float z = sg2_comp_eval(comp + (SG2_COMP_Z * 16 + r) * 3, g, s);
+                arr(A_XB)[r * BBST + tu] = valid ? sg2_comp_eval(cw[SG2_COMP_XB][q], g, s) : 0.0f;
+                arr(A_B)[r * BBST + tu] = sg2_comp_eval(cw[SG2_COMP_B][q], g, s);
+                arr(A_C)[r * BBST + tu] = sg2_comp_eval(cw[SG2_COMP_C][q], g, s);
+                const float z = sg2_comp_eval(cw[SG2_COMP_Z][q], g, s);
                 const float sz = sg_sigmoid(z);
                 arr(A_GATE)[r * BBST + tu] = z * sz;
                 arr(A_DGATE)[r * BBST + tu] = sz * sg_fma(z, 1.0f - sz, 1.0f);
@@ -324,17 +339,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         __syncthreads();
 
         // ---- 3: per step and column: out, d out, d y, d z, D-skip part of d x-branch
+#pragma unroll
         for (int q = 0; q < ROWS / 4; q++) {
             const int r = part * (ROWS / 4) + q;
             float dout = 0.0f;
 #pragma unroll
-            for (int d = 0; d < DM; d++) dout = sg_fma(Wout[d * DI + r], s_dctx[tu * DM + d], dout);
+            for (int d = 0; d < DM; d++) dout = sg_fma(wo[q][d], s_dctx[tu * DM + d], dout);
             const float y = arr(A_Y)[r * BBST + tu], gate = arr(A_GATE)[r * BBST + tu], xb = arr(A_XB)[r * BBST + tu];
             const bool valid = tu < cnt;
             arr(A_DY)[r * BBST + tu] = valid ? dout * gate : 0.0f;
             arr(A_DZ)[r * BBST + tu] = valid ? (dout * y) * arr(A_DGATE)[r * BBST + tu] : 0.0f;
-            arr(A_DXB)[r * BBST + tu] = valid ? dout * Dw[r] : 0.0f;
-            arr(A_GATE)[r * BBST + tu] = valid ? sg_fma(y, gate, Dw[r] * xb) : 0.0f;     // out, for d out_proj
+            arr(A_DXB)[r * BBST + tu] = valid ? dout * dwr[q] : 0.0f;
+            arr(A_GATE)[r * BBST + tu] = valid ? sg_fma(y, gate, dwr[q] * xb) : 0.0f;     // out, for d out_proj
             arr(A_DGATE)[r * BBST + tu] = valid ? dout : 0.0f;                           // d out, for d D
             arr(A_DDT)[r * BBST + tu] = 0.0f;
         }
