@@ -12,7 +12,11 @@
 namespace sgew {
 namespace {
 
-constexpr int TILE = 4096;
+// Elements per workgroup.  Large calls use 4096 (16 per lane: few, long workgroups stream best); small calls use
+// shorter tiles so that there are several workgroups per CU and few elements in series per lane (the v1.5 / v1.1
+// steps spend ~1500 instructions per element).  A function of the call's total size only, so the workspace
+// layout, the upload and the kernels agree.
+inline int tile_for(int64_t total) { return total >= (8 << 20) ? 4096 : (total >= (1 << 20) ? 1024 : 256); }
 constexpr int THREADS = 256;
 constexpr int MAX_HIDDEN = 256;
 
@@ -31,7 +35,7 @@ struct TRed {           // up to three sums of one tensor (or of the whole call,
 };
 
 struct Layout {
-    int n, tiles;
+    int n, tiles, tile;
     size_t off_recs, off_nrecs, off_prefix, off_partials, off_red, off_tred, bytes;
     int64_t total;
 };
@@ -42,9 +46,11 @@ inline int make_layout(int n, const int64_t* numels, Layout* L) {
     int64_t tiles = 0, total = 0;
     for (int i = 0; i < n; i++) {
         if (numels[i] < 0 || numels[i] > 0x7fffffff) return sg::fail("tensor %d: bad numel %lld", i, (long long)numels[i]);
-        tiles += (numels[i] + TILE - 1) / TILE;
         total += numels[i];
     }
+    const int TILE = tile_for(total);
+    for (int i = 0; i < n; i++) tiles += (numels[i] + TILE - 1) / TILE;
+    L->tile = TILE;
     if (tiles > 0x7fffffff) return sg::fail("too many elements");
     L->n = n;
     L->tiles = (int)tiles;
@@ -65,7 +71,7 @@ template <class Rec>
 struct Batch {
     const Rec* recs;
     const int* prefix;
-    int n, tiles;
+    int n, tiles, tile;
     double* partials;
     Red* red;
     TRed* tred;
@@ -84,7 +90,7 @@ int upload(const std::vector<Rec>& recs, void* workspace, size_t ws_bytes, hipSt
     if (!workspace || ws_bytes < L.bytes) return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, ws_bytes);
     if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
     std::vector<int> prefix(n + 1, 0);
-    for (int i = 0; i < n; i++) prefix[i + 1] = prefix[i] + (int)((numels[i] + TILE - 1) / TILE);
+    for (int i = 0; i < n; i++) prefix[i + 1] = prefix[i] + (int)((numels[i] + L.tile - 1) / L.tile);
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_recs, recs.data(), sizeof(Rec) * (size_t)n, hipMemcpyHostToDevice, st));
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_prefix, prefix.data(), sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, st));
@@ -92,6 +98,7 @@ int upload(const std::vector<Rec>& recs, void* workspace, size_t ws_bytes, hipSt
     B->prefix = reinterpret_cast<const int*>(ws + L.off_prefix);
     B->n = n;
     B->tiles = L.tiles;
+    B->tile = L.tile;
     B->partials = reinterpret_cast<double*>(ws + L.off_partials);
     B->red = reinterpret_cast<Red*>(ws + L.off_red);
     B->tred = reinterpret_cast<TRed*>(ws + L.off_tred);
@@ -103,8 +110,8 @@ template <class Rec>
 __device__ __forceinline__ const Rec& tile_rec(const Batch<Rec>& B, int tile, int* start, int* cnt) {
     const int ti = sg::upper_seg(B.prefix, B.n, tile);
     const Rec& R = B.recs[ti];
-    *start = (tile - B.prefix[ti]) * TILE;
-    *cnt = min(TILE, (int)R.numel - *start);
+    *start = (tile - B.prefix[ti]) * B.tile;
+    *cnt = min(B.tile, (int)R.numel - *start);
     return R;
 }
 
@@ -177,6 +184,7 @@ int reduce_sumsq(const std::vector<Rec>& recs, const Batch<Rec>& B, float clip_n
     NB.prefix = B.prefix;
     NB.n = B.n;
     NB.tiles = B.tiles;
+    NB.tile = B.tile;
     NB.partials = B.partials;
     NB.red = B.red;
     NB.tred = B.tred;
