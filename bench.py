@@ -85,118 +85,157 @@ def cpu_baseline(sample_elems_target=4_000_000):
                       "fp32 C++ restatement, %.1f s" % (pick[0], pick[-1], tot, dt)}
 
 
-def bench_other(args, dev):
-    """Secondary measurements: the other fused steps through `_ops`."""
+def build_step(workload, ops, dev, limit=None):
+    """One secondary workload as a closure over `ops` (this package's `_ops`, or the reference's own CPU build: the
+    function names and argument orders are the same) on tensors living on `dev`.  limit: use only the first tensors
+    of the set, up to that many elements (the bounded CPU sample)."""
     import torch
     import workloads as wl
-    from grokking_optimizers import _ops
-    K, Wm = args.steps, args.warmup
-    if args.workload == "muon":
+
+    def take(shapes):
+        if limit is None:
+            return shapes
+        out, tot = [], 0
+        for sh in shapes:
+            if out and tot + wl.numel(sh) > limit:
+                break
+            out.append(sh)
+            tot += wl.numel(sh)
+        return out
+
+    W = dict(dtype="f32", bound="hbm", peak=HBM_PEAK_GBS, unit="elements/s", bytes_per_elem=40)
+    if workload == "muon":
         shapes = [(1024, 4096)] * 12 + [(4096, 1024)] * 12
+        if limit is not None:
+            shapes = [(1024, 4096), (4096, 1024)]
         gen = torch.Generator().manual_seed(0)
         params = [(torch.randn(*s, generator=gen) * 0.02).to(torch.bfloat16).to(dev) for s in shapes]
         grads = [(torch.randn(*s, generator=gen) * 1e-3).to(torch.bfloat16).to(dev) for s in shapes]
         bufs = [torch.zeros(s, device=dev) for s in shapes]
-        step = lambda: _ops.muon_fused_step(params, grads, bufs, 0.95, 0.02, 1.0, 5)
-        units, unit = 5 * sum(6 * min(s) ** 2 * max(s) for s in shapes), "FLOP/s"      # 6 min^2 max per NS iteration
-        name, dtype, bound, peak = "Muon step, 12x[1024,4096] + 12x[4096,1024], 5 Newton-Schulz iterations", "bf16", "mfma", 2500.0
+        W.update(step=lambda: ops.muon_fused_step(params, grads, bufs, 0.95, 0.02, 1.0, 5),
+                 units=5 * sum(6 * min(s) ** 2 * max(s) for s in shapes), unit="FLOP/s",       # 6 min^2 max per NS iteration
+                 name="Muon step, %d x [1024,4096] + %d x [4096,1024], 5 Newton-Schulz iterations" % (len(shapes) // 2, len(shapes) // 2),
+                 dtype="bf16", bound="mfma", peak=2500.0)
+        return W
+    small = workload in ("grokfast", "sg15", "bilevel")
+    shapes = take(wl.shared14_shapes() if small else wl.scale50_shapes())
+    params = [p.reshape(-1).to(dev) for p in wl.make_params(shapes, seed=0)]
+    if small:
+        grads = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.01 if workload == "sg15" else 0.0)]
     else:
-        shapes = wl.shared14_shapes()
-        params = [p.reshape(-1).to(dev) for p in wl.make_params(shapes, seed=0)]
-        grads0 = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.01 if args.workload == "sg15" else 0.0)]
-        z = lambda: [torch.zeros_like(p) for p in params]
-        n = sum(p.numel() for p in params)
-        if args.workload == "grokfast":
-            emas, ms, vs = z(), z(), z()
-            grads = [g.clone() for g in grads0]
-            t = [0]
+        # the other fused steps, on the 50-tensor / 25 M-element set so that HBM traffic, not launch latency, is measured
+        grads = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.005, tail="student3")]
+    z = lambda: [torch.zeros_like(p) for p in params]
+    n = sum(p.numel() for p in params)
+    P = len(params)
+    a, b, c, d = z(), z(), z(), z()
+    gen = torch.Generator().manual_seed(3)
+    t = [0]
+    setname = "%d tensors, %d elements" % (P, n)
+    if workload == "grokfast":
+        def step():
+            t[0] += 1
+            ops.grokfast_adamw_fused_step(params, grads, a, b, c, [t[0]] * P, 0.98, 2.0, 1e-3, 0.9, 0.98, 1e-8, 1.0)
+        what = "Grokfast fused step (EMA + amplify + AdamW)"
+    elif workload == "sg15":
+        H = 32
+        W1, b1 = (torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev)
+        W2, b2 = (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)
 
-            def step():
-                t[0] += 1
-                _ops.grokfast_adamw_fused_step(params, grads, emas, ms, vs, [t[0]] * len(params), 0.98, 2.0, 1e-3, 0.9, 0.98, 1e-8, 1.0)
-            name = "Grokfast fused step (EMA + amplify + AdamW), 14 tensors, %d elements" % n
-        elif args.workload == "sg15":
-            eas, easqs, mus, sharps = z(), z(), z(), z()
-            gen = torch.Generator().manual_seed(3)
-            H = 32
-            W1, b1 = (torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev)
-            W2, b2 = (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)
-            grads = [g.clone() for g in grads0]
-            P = len(params)
+        def step():
+            ops.supergrok15_fused_step(params, grads, a, b, c, d, [0] * P, [0.98] * P, [0.9 * 0.9 ** i for i in range(P)],
+                                       W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8, 2.0, 1.0, 0.5, 1.0)
+        what = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip)"
+    elif workload == "bilevel":
+        # gradient of sum <smart_grad, cotangent> with respect to every weight of the v2 meta-net, for all tensors
+        # of the model at once: sort + scan forward, per-element forward/backward, scan adjoint, all in HIP
+        from grokking_optimizers import Mamba3PEERMetaNet, _bilevel
+        torch.manual_seed(0)
+        mn = Mamba3PEERMetaNet().to(dev)
+        sharps = [g.abs() * 0.5 for g in grads]
+        grus = [torch.zeros(g.numel(), 4, device=dev) for g in grads]
+        mf = [torch.zeros(16, 16, device=dev) for _ in grads]
+        mb = [torch.zeros(16, 16, device=dev) for _ in grads]
+        cots = [torch.randn(g.numel(), generator=torch.Generator().manual_seed(5)).to(dev) for g in grads]
 
-            def step():
-                _ops.supergrok15_fused_step(params, grads, eas, easqs, mus, sharps, [0] * P, [0.98] * P,
-                                            [0.9 * 0.9 ** i for i in range(P)], W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8,
-                                            2.0, 1.0, 0.5, 1.0)
-            name = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip), 14 tensors, %d elements" % n
-        elif args.workload == "bilevel":
-            # gradient of sum <smart_grad, cotangent> with respect to every weight of the v2 meta-net, for all tensors
-            # of the model at once: sort + scan forward, per-element forward/backward, scan adjoint, all in HIP
-            from grokking_optimizers import Mamba3PEERMetaNet, _bilevel
-            torch.manual_seed(0)
-            mn = Mamba3PEERMetaNet().to(dev)
-            sharps = [g.abs() * 0.5 for g in grads0]
-            grus = [torch.zeros(g.numel(), 4, device=dev) for g in grads0]
-            mf = [torch.zeros(16, 16, device=dev) for _ in grads0]
-            mb = [torch.zeros(16, 16, device=dev) for _ in grads0]
-            gen = torch.Generator().manual_seed(5)
-            cots = [torch.randn(g.numel(), generator=gen).to(dev) for g in grads0]
+        def step():
+            mn.zero_grad()
+            _bilevel.accumulate_meta_gradients(mn, grads, sharps, grus, mf, mb, cots)
+        # per element: grad, sharpness, cotangent, GRU state read (28 B); both contexts written by the scan and read
+        # by the per-element pass, their gradients written by it and read by the adjoint (4 x 64 B)
+        W["bytes_per_elem"] = 284
+        what = "SuperGrok v2 bilevel meta-gradient pass (sort + scan, per-element forward/backward, scan adjoint)"
+    elif workload == "grokadamw":
+        def step():
+            t[0] += 1
+            ops.grokadamw_fused_step(params, grads, a, b, c, [t[0]] * P, 0.98, 5.0, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
+        W["bytes_per_elem"], what = 36, "GrokAdamW fused step (clip + EMA + amplify + AdamW)"
+    elif workload == "neuralgrok":
+        H = 128
+        Wn = [(torch.randn(H, 1, generator=gen) * 0.5).to(dev), torch.zeros(H, device=dev),
+              (torch.randn(1, H, generator=gen) * 0.1).to(dev), torch.zeros(1, device=dev)]
 
-            def step():
-                mn.zero_grad()
-                _bilevel.accumulate_meta_gradients(mn, grads0, sharps, grus, mf, mb, cots)
-            # per element: grad, sharpness, cotangent, GRU state read (28 B); both contexts written by the scan and read
-            # by the per-element pass, their gradients written by it and read by the adjoint (4 x 64 B)
-            bytes_per_elem = 284
-            name = "SuperGrok v2 bilevel meta-gradient pass (sort + scan, per-element forward/backward, scan adjoint), 14 tensors, %d elements" % n
-        else:
-            # the other fused steps, on the 50-tensor / 25 M-element set so that HBM traffic, not launch latency, is measured
-            shapes = wl.scale50_shapes()
-            params = [p.reshape(-1).to(dev) for p in wl.make_params(shapes, seed=0)]
-            grads = [g.reshape(-1).to(dev) for g in wl.make_grads(shapes, seed=1, tail_frac=0.005, tail="student3")]
-            n = sum(p.numel() for p in params)
-            P = len(params)
-            a, b, c, d = z(), z(), z(), z()
-            gen = torch.Generator().manual_seed(3)
-            t = [0]
-            if args.workload == "grokadamw":
-                def step():
-                    t[0] += 1
-                    _ops.grokadamw_fused_step(params, grads, a, b, c, [t[0]] * P, 0.98, 5.0, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
-                bytes_per_elem, what = 36, "GrokAdamW fused step (clip + EMA + amplify + AdamW)"
-            elif args.workload == "neuralgrok":
-                H = 128
-                W = [(torch.randn(H, 1, generator=gen) * 0.5).to(dev), torch.zeros(H, device=dev),
-                     (torch.randn(1, H, generator=gen) * 0.1).to(dev), torch.zeros(1, device=dev)]
+        def step():
+            t[0] += 1
+            ops.neuralgrok_fused_step(params, grads, a, b, [t[0]] * P, *Wn, 10.0, 4.0, H, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
+        W["bytes_per_elem"], what = 28, "NeuralGrok fused step (clip + 1->128->1 amplifier + AdamW)"
+    elif workload == "prodigy":
+        inits = [p.clone() for p in params]
+        dl = [1e-6]
 
-                def step():
-                    t[0] += 1
-                    _ops.neuralgrok_fused_step(params, grads, a, b, [t[0]] * P, *W, 10.0, 4.0, H, 0.9, 0.98, 1e-3, 1.0, 1e-8, 1.0)
-                bytes_per_elem, what = 28, "NeuralGrok fused step (clip + 1->128->1 amplifier + AdamW)"
-            elif args.workload == "prodigy":
-                inits = [p.clone() for p in params]
-                dl = [1e-6]
+        def step():
+            t[0] += 1
+            dl[0] = ops.prodigy_fused_step(params, grads, a, b, c, inits, [t[0]] * P, dl[0], 0.9, 0.999, 1e-3, 0.0, 1e-8)
+        W["bytes_per_elem"], what = 52, "Prodigy fused step (d_lr reduction pass + Adam pass, one host read of d_lr)"
+    elif workload == "lion":
+        def step():
+            ops.lion_fused_step(params, grads, a, 1e-4, 0.9, 0.99, 3.0)
+        W["bytes_per_elem"], what = 20, "Lion fused step"
+    else:
+        H = 32
+        Ws = [(torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev),
+              (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)]
+        beta1s = [0.9 * 0.9 ** i for i in range(P)]
 
-                def step():
-                    t[0] += 1
-                    dl[0] = _ops.prodigy_fused_step(params, grads, a, b, c, inits, [t[0]] * P, dl[0], 0.9, 0.999, 1e-3, 0.0, 1e-8)
-                bytes_per_elem, what = 52, "Prodigy fused step (d_lr reduction pass + Adam pass, one host read of d_lr)"
-            elif args.workload == "lion":
-                def step():
-                    _ops.lion_fused_step(params, grads, a, 1e-4, 0.9, 0.99, 3.0)
-                bytes_per_elem, what = 20, "Lion fused step"
-            else:
-                H = 32
-                W = [(torch.randn(H, 2, generator=gen) * 0.01).to(dev), torch.zeros(H, device=dev),
-                     (torch.randn(1, H, generator=gen) * 0.01).to(dev), torch.zeros(1, device=dev)]
-                beta1s = [0.9 * 0.9 ** i for i in range(P)]
+        def step():
+            ops.supergrok11_fused_step(params, grads, a, b, c, d, [0] * P, [0.98] * P, beta1s, *Ws, 0.1, H, 0.999, 1e-3, 1.0,
+                                       1e-8, 5.0, 1.0, 5.0, 1.0)
+        W["bytes_per_elem"], what = 52, "SuperGrok v1.1 full step (H=32, exact GELU, device-side clip and cosine gates)"
+    W.update(step=step, units=n, name="%s, %s" % (what, setname))
+    return W
 
-                def step():
-                    _ops.supergrok11_fused_step(params, grads, a, b, c, d, [0] * P, [0.98] * P, beta1s, *W, 0.1, H, 0.999, 1e-3, 1.0,
-                                                1e-8, 5.0, 1.0, 5.0, 1.0)
-                bytes_per_elem, what = 52, "SuperGrok v1.1 full step (H=32, exact GELU, device-side clip and cosine gates)"
-            name = "%s, 50 tensors, %d elements" % (what, n)
-        units, unit, dtype, bound, peak = n, "elements/s", "f32", "hbm", HBM_PEAK_GBS
+
+def cpu_reference_baseline(workload):
+    """The reference's own CPU code (its csrc/ops.cpp compiled without CUDA into oracle/_ref by oracle/Makefile.ref),
+    timed on a bounded sample of the same workload.  None when that build is not there or has no such step."""
+    import torch
+    ref_dir = os.path.join(ROOT, "oracle", "_ref")
+    if workload in ("bilevel", "grokfast") or not os.path.isdir(ref_dir):
+        return None       # the reference has no CPU op for these (Grokfast's AdamW half is Python there)
+    sys.path.insert(0, ref_dir)
+    try:
+        import ref_ops
+    except ImportError:
+        return None
+    W = build_step(workload, ref_ops, "cpu", limit=4_000_000)
+    W["step"]()                                   # warm-up (allocations, thread pool)
+    steps, t0 = 0, time.perf_counter()
+    while steps < 200 and (steps < 3 or time.perf_counter() - t0 < 5.0):
+        W["step"]()
+        steps += 1
+    el = (time.perf_counter() - t0) / steps
+    return {"value": W["units"] / el, "unit": W["unit"], "cores": torch.get_num_threads(), "kind": "reference",
+            "sample": "%s; %d step(s) of the reference's CPU path (ATen ops, %d threads), %.1f s" %
+                      (W["name"], steps, torch.get_num_threads(), el * steps)}
+
+
+def bench_other(args, dev):
+    """Secondary measurements: the other fused steps through `_ops`."""
+    import torch
+    from grokking_optimizers import _ops
+    K, Wm = args.steps, args.warmup
+    W = build_step(args.workload, _ops, dev)
+    step, units = W["step"], W["units"]
     for _ in range(Wm):
         step()
     torch.cuda.synchronize()
@@ -205,16 +244,20 @@ def bench_other(args, dev):
         step()
     torch.cuda.synchronize()
     el = (time.perf_counter() - t0) / K
-    out = {"metric": "secondary: " + args.workload, "value": units / el, "unit": unit, "n_gpus": 1, "steps": K, "warmup": Wm,
-           "ms_per_step": 1e3 * el, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
-           "data": "synthetic", "config": {"workload": name}}
-    if bound == "mfma":
-        out["roofline"] = {"bound": "mfma", "achieved": units / el / 1e12, "peak": peak, "unit": "TFLOP/s",
-                           "frac": units / el / 1e12 / peak, "traffic": None}
+    out = {"metric": "secondary: " + args.workload, "value": units / el, "unit": W["unit"], "n_gpus": 1, "steps": K, "warmup": Wm,
+           "ms_per_step": 1e3 * el, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": W["dtype"],
+           "data": "synthetic", "config": {"workload": W["name"]}}
+    if W["bound"] == "mfma":
+        out["roofline"] = {"bound": "mfma", "achieved": units / el / 1e12, "peak": W["peak"], "unit": "TFLOP/s",
+                           "frac": units / el / 1e12 / W["peak"], "traffic": None}
     else:
-        bpe = locals().get("bytes_per_elem", 40)       # algorithmic bytes per element of the step
-        out["roofline"] = {"bound": "hbm", "achieved": bpe * units / el / 1e9, "peak": peak, "unit": "GB/s",
-                           "frac": bpe * units / el / 1e9 / peak, "traffic": None, "bytes_per_element": bpe}
+        bpe = W["bytes_per_elem"]                      # algorithmic bytes per element of the step
+        out["roofline"] = {"bound": "hbm", "achieved": bpe * units / el / 1e9, "peak": W["peak"], "unit": "GB/s",
+                           "frac": bpe * units / el / 1e9 / W["peak"], "traffic": None, "bytes_per_element": bpe}
+    if not args.no_cpu_baseline:
+        base = cpu_reference_baseline(args.workload)
+        if base is not None:
+            out["cpu_baseline"] = base
     return out
 
 
