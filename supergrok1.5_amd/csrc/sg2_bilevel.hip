@@ -320,20 +320,42 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         const float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, u0)) * 2 * SCAN_THREADS;
         const float hs_e = ht[tid], hs_o = ht[SCAN_THREADS + tid];
         {
+            // in blocks of FB steps: operands and the state-independent coefficients of the whole block first (independent
+            // instruction streams), then the short serial state update.  Steps past the end of the chunk are
+            // identities (dt = 0, x-branch = 0) whose results nobody reads.
+            constexpr int FB = 8;
+            static_assert(BT % FB == 0, "whole blocks");
             float he = hs_e, ho = hs_o;
-            for (int k = 0; k < cnt; k++) {
-                const float dt = arr(A_DT)[j * BBST + k];
-                float ae, ao, sn, cs;
-                sg_abar_pair(dt, a_e, a_o, &ae, &ao);
-                rot_sincos(tiny, dt * freq, &sn, &cs);
-                const float ux = dt * arr(A_XB)[j * BBST + k];
-                const float re = sg_fma(he, cs, -(ho * sn)), ro = sg_fma(ho, cs, he * sn);
-                he = sg_fma(ae, re, ux * arr(A_B)[(2 * p) * BBST + k]);
-                ho = sg_fma(ao, ro, ux * arr(A_B)[(2 * p + 1) * BBST + k]);
-                sH[(k * SCAN_THREADS + tid) * 2] = he;
-                sH[(k * SCAN_THREADS + tid) * 2 + 1] = ho;
-                const float y = pair_sum(sg_fma(ho, arr(A_C)[(2 * p + 1) * BBST + k], he * arr(A_C)[(2 * p) * BBST + k]));
-                if (p == 0) arr(A_Y)[j * BBST + k] = y;
+            for (int k0 = 0; k0 < cnt; k0 += FB) {
+                float dtv[FB], uxv[FB], Bev[FB], Bov[FB], Cev[FB], Cov[FB], aev[FB], aov[FB], snv[FB], csv[FB], yv[FB];
+#pragma unroll
+                for (int q = 0; q < FB; q++) {
+                    const int k = k0 + q;
+                    dtv[q] = arr(A_DT)[j * BBST + k];
+                    uxv[q] = dtv[q] * arr(A_XB)[j * BBST + k];
+                    Bev[q] = arr(A_B)[(2 * p) * BBST + k]; Bov[q] = arr(A_B)[(2 * p + 1) * BBST + k];
+                    Cev[q] = arr(A_C)[(2 * p) * BBST + k]; Cov[q] = arr(A_C)[(2 * p + 1) * BBST + k];
+                }
+#pragma unroll
+                for (int q = 0; q < FB; q++) {
+                    sg_abar_pair(dtv[q], a_e, a_o, &aev[q], &aov[q]);
+                    rot_sincos(tiny, dtv[q] * freq, &snv[q], &csv[q]);
+                }
+#pragma unroll
+                for (int q = 0; q < FB; q++) {
+                    const float re = sg_fma(he, csv[q], -(ho * snv[q])), ro = sg_fma(ho, csv[q], he * snv[q]);
+                    he = sg_fma(aev[q], re, uxv[q] * Bev[q]);
+                    ho = sg_fma(aov[q], ro, uxv[q] * Bov[q]);
+                    sH[((k0 + q) * SCAN_THREADS + tid) * 2] = he;
+                    sH[((k0 + q) * SCAN_THREADS + tid) * 2 + 1] = ho;
+                    yv[q] = sg_fma(ho, Cov[q], he * Cev[q]);
+                }
+#pragma unroll
+                for (int q = 0; q < FB; q++) yv[q] = pair_sum(yv[q]);
+                if (p == 0) {
+#pragma unroll
+                    for (int q = 0; q < FB; q++) arr(A_Y)[j * BBST + k0 + q] = yv[q];
+                }
             }
         }
         __syncthreads();
@@ -357,57 +379,83 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         __syncthreads();
 
         // ---- 4: adjoint recurrence, last step of the tile first
-        for (int k = cnt - 1; k >= 0; k--) {
-            const float dt = arr(A_DT)[j * BBST + k], xb = arr(A_XB)[j * BBST + k], dy = arr(A_DY)[j * BBST + k];
-            const float Be = arr(A_B)[(2 * p) * BBST + k], Bo = arr(A_B)[(2 * p + 1) * BBST + k];
-            const float Ce = arr(A_C)[(2 * p) * BBST + k], Co = arr(A_C)[(2 * p + 1) * BBST + k];
-            const float he = sH[(k * SCAN_THREADS + tid) * 2], ho = sH[(k * SCAN_THREADS + tid) * 2 + 1];
-            const float pe = (k > 0) ? sH[((k - 1) * SCAN_THREADS + tid) * 2] : hs_e;
-            const float po = (k > 0) ? sH[((k - 1) * SCAN_THREADS + tid) * 2 + 1] : hs_o;
-            float ae, ao, sn, cs;
-            sg_abar_pair(dt, a_e, a_o, &ae, &ao);
-            rot_sincos(tiny, dt * freq, &sn, &cs);
-            // y = sum h C
-            le = sg_fma(dy, Ce, le);
-            lo = sg_fma(dy, Co, lo);
-            // d C[2p], d C[2p+1] of this step are sums over the columns of dy*h, d B of lambda*dt*xb; what is wanted
-            // is their sum over steps against (g, s, 1), so each lane sums its own column's share over the steps
-            // and the columns are added once, when the workgroup is done
-            const float gk = s_gs[2 * k], sk = s_gs[2 * k + 1];
-            {
-                const float te = dy * he, to = dy * ho;
-                acc_bc[6] = sg_fma(te, gk, acc_bc[6]); acc_bc[7] = sg_fma(te, sk, acc_bc[7]); acc_bc[8] += te;
-                acc_bc[9] = sg_fma(to, gk, acc_bc[9]); acc_bc[10] = sg_fma(to, sk, acc_bc[10]); acc_bc[11] += to;
+        // (blocks of RB steps, operands and coefficients of the block first, as in step 2)
+        constexpr int RB = 8;
+        static_assert(BT % RB == 0, "whole blocks");
+        for (int k0 = ((cnt - 1) / RB) * RB; k0 >= 0; k0 -= RB) {
+            float dtv[RB], xbv[RB], dyv[RB], Bev[RB], Bov[RB], Cev[RB], Cov[RB], gkv[RB], skv[RB], hev[RB + 1], hov[RB + 1];
+            float aev[RB], aov[RB], snv[RB], csv[RB];
+#pragma unroll
+            for (int q = 0; q < RB; q++) {
+                const int k = k0 + q;
+                dtv[q] = arr(A_DT)[j * BBST + k]; xbv[q] = arr(A_XB)[j * BBST + k]; dyv[q] = arr(A_DY)[j * BBST + k];
+                Bev[q] = arr(A_B)[(2 * p) * BBST + k]; Bov[q] = arr(A_B)[(2 * p + 1) * BBST + k];
+                Cev[q] = arr(A_C)[(2 * p) * BBST + k]; Cov[q] = arr(A_C)[(2 * p + 1) * BBST + k];
+                gkv[q] = s_gs[2 * k]; skv[q] = s_gs[2 * k + 1];
+                hev[q + 1] = sH[(k * SCAN_THREADS + tid) * 2]; hov[q + 1] = sH[(k * SCAN_THREADS + tid) * 2 + 1];
             }
-            // h' = A_bar * rot(h) + dt * xb * B
-            const float re = sg_fma(pe, cs, -(po * sn)), ro = sg_fma(po, cs, pe * sn);
-            // A_bar = 2/d - 1, d = 1 + dt*a: dA_bar/dd = -2/d^2 = -(A_bar+1)^2/2
-            const float dd_e = (le * re) * (-0.5f * (ae + 1.0f) * (ae + 1.0f));
-            const float dd_o = (lo * ro) * (-0.5f * (ao + 1.0f) * (ao + 1.0f));
-            float ddt = sg_fma(dd_e, a_e, dd_o * a_o);
-            acc_alog_e = sg_fma(dd_e * dt, a_e, acc_alog_e);
-            acc_alog_o = sg_fma(dd_o * dt, a_o, acc_alog_o);
-            const float dre = le * ae, dro = lo * ao;
-            const float dth = sg_fma(dro, re, -(dre * ro));        // d re/d theta = -ro, d ro/d theta = re
-            ddt = sg_fma(dth, freq, ddt);
-            acc_rope = sg_fma(dth, dt, acc_rope);
-            const float qb = sg_fma(le, Be, lo * Bo);
-            ddt = sg_fma(qb, xb, ddt);
-            const float ux = dt * xb;
-            {
-                const float te = le * ux, to = lo * ux;
-                acc_bc[0] = sg_fma(te, gk, acc_bc[0]); acc_bc[1] = sg_fma(te, sk, acc_bc[1]); acc_bc[2] += te;
-                acc_bc[3] = sg_fma(to, gk, acc_bc[3]); acc_bc[4] = sg_fma(to, sk, acc_bc[4]); acc_bc[5] += to;
+            hev[0] = (k0 > 0) ? sH[((k0 - 1) * SCAN_THREADS + tid) * 2] : hs_e;
+            hov[0] = (k0 > 0) ? sH[((k0 - 1) * SCAN_THREADS + tid) * 2 + 1] : hs_o;
+#pragma unroll
+            for (int q = 0; q < RB; q++) {
+                sg_abar_pair(dtv[q], a_e, a_o, &aev[q], &aov[q]);
+                rot_sincos(tiny, dtv[q] * freq, &snv[q], &csv[q]);
             }
-            const float ddt_j = pair_sum(ddt), dxb_j = pair_sum(qb * dt);
+            float ddtv[RB], dxbv[RB];
+#pragma unroll
+            for (int q = RB - 1; q >= 0; q--) {
+                const bool live = k0 + q < cnt;                  // steps past the end of the chunk leave lambda alone
+                const float dt = dtv[q], xb = xbv[q], dy = dyv[q], ae = aev[q], ao = aov[q], sn = snv[q], cs = csv[q];
+                const float he = hev[q + 1], ho = hov[q + 1], pe = hev[q], po = hov[q], gk = gkv[q], sk = skv[q];
+                // y = sum h C
+                le = sg_fma(dy, Cev[q], le);
+                lo = sg_fma(dy, Cov[q], lo);
+                // d C[2p], d C[2p+1] of this step are sums over the columns of dy*h, d B of lambda*dt*xb; what is wanted
+                // is their sum over steps against (g, s, 1), so each lane sums its own column's share over the steps
+                // and the columns are added once, when the workgroup is done
+                {
+                    const float te = dy * he, to = dy * ho;
+                    acc_bc[6] = sg_fma(te, gk, acc_bc[6]); acc_bc[7] = sg_fma(te, sk, acc_bc[7]); acc_bc[8] += te;
+                    acc_bc[9] = sg_fma(to, gk, acc_bc[9]); acc_bc[10] = sg_fma(to, sk, acc_bc[10]); acc_bc[11] += to;
+                }
+                // h' = A_bar * rot(h) + dt * xb * B
+                const float re = sg_fma(pe, cs, -(po * sn)), ro = sg_fma(po, cs, pe * sn);
+                // A_bar = 2/d - 1, d = 1 + dt*a: dA_bar/dd = -2/d^2 = -(A_bar+1)^2/2
+                const float dd_e = (le * re) * (-0.5f * (ae + 1.0f) * (ae + 1.0f));
+                const float dd_o = (lo * ro) * (-0.5f * (ao + 1.0f) * (ao + 1.0f));
+                float ddt = sg_fma(dd_e, a_e, dd_o * a_o);
+                acc_alog_e = sg_fma(dd_e * dt, a_e, acc_alog_e);
+                acc_alog_o = sg_fma(dd_o * dt, a_o, acc_alog_o);
+                const float dre = le * ae, dro = lo * ao;
+                const float dth = sg_fma(dro, re, -(dre * ro));        // d re/d theta = -ro, d ro/d theta = re
+                ddt = sg_fma(dth, freq, ddt);
+                acc_rope = sg_fma(dth, dt, acc_rope);
+                const float qb = sg_fma(le, Bev[q], lo * Bov[q]);
+                ddt = sg_fma(qb, xb, ddt);
+                const float ux = dt * xb;
+                {
+                    const float te = le * ux, to = lo * ux;
+                    acc_bc[0] = sg_fma(te, gk, acc_bc[0]); acc_bc[1] = sg_fma(te, sk, acc_bc[1]); acc_bc[2] += te;
+                    acc_bc[3] = sg_fma(to, gk, acc_bc[3]); acc_bc[4] = sg_fma(to, sk, acc_bc[4]); acc_bc[5] += to;
+                }
+                ddtv[q] = ddt;
+                dxbv[q] = qb * dt;
+                // lambda for the previous step
+                const float nle = sg_fma(dre, cs, dro * sn), nlo = sg_fma(dro, cs, -(dre * sn));
+                le = live ? nle : le;
+                lo = live ? nlo : lo;
+            }
+#pragma unroll
+            for (int q = 0; q < RB; q++) { ddtv[q] = pair_sum(ddtv[q]); dxbv[q] = pair_sum(dxbv[q]); }
             if (p == 0) {
-                arr(A_DDT)[j * BBST + k] = ddt_j * arr(A_DSP)[j * BBST + k];
-                arr(A_DXB)[j * BBST + k] += dxb_j;
+#pragma unroll
+                for (int q = 0; q < RB; q++) {
+                    if (k0 + q < cnt) {
+                        arr(A_DDT)[j * BBST + k0 + q] = ddtv[q] * arr(A_DSP)[j * BBST + k0 + q];
+                        arr(A_DXB)[j * BBST + k0 + q] += dxbv[q];
+                    }
+                }
             }
-            // lambda for the previous step
-            const float nle = sg_fma(dre, cs, dro * sn), nlo = sg_fma(dro, cs, -(dre * sn));
-            le = nle;
-            lo = nlo;
         }
         __syncthreads();
 
