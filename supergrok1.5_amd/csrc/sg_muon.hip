@@ -160,54 +160,30 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
     if (threadIdx.x == 0) B.inv_norm[mi] = 1.0f / ((float)sqrt(tot) + 1e-7f);
 }
 
-// X = buf * inv_norm as bf16, written in the parameter's own orientation into
-// Y (wide) or YT (tall); the other one follows from k_transpose.
+// X = buf * inv_norm as bf16, written in both orientations at once: Y ([mp x np], the wide orientation) and its
+// transpose YT ([np x mp]).  One 64x64 tile of the parameter's own orientation per workgroup: rows are read and
+// written along the fast axis, the transposed copy goes through LDS.  The zero padding of both buffers is written
+// here as well.
 __global__ __launch_bounds__(256) void k_normalize(Batch B) {
-    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
-    const Mat& M = B.mats[mi];
-    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
-    const int cnt = min(ETILE, M.rows * M.cols - start);
-    const float inv = B.inv_norm[mi];
-    bf16_t* dst = M.wide ? M.Y : M.YT;
-    const int ld = M.wide ? M.np : M.mp;
-    if (M.vec8) {
-        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
-            const int i = start + k, r = i / M.cols, c = i - r * M.cols;      // 8 elements of one row
-            float b[8];
-            load8(M.buf, SG_F32, (size_t)i, b);
-#pragma unroll
-            for (int e = 0; e < 8; e++) b[e] *= inv;
-            store8(dst, SG_BF16, (size_t)r * ld + c, b);
-        }
-        return;
-    }
-    for (int k = threadIdx.x; k < cnt; k += 256) {
-        const int i = start + k, r = i / M.cols, c = i - r * M.cols;
-        dst[(size_t)r * ld + c] = sg::f_to_bf16_bits(M.buf[i] * inv);
-    }
-}
-
-// dst[c][r] = src[r][c] over the padded buffers, 64x64 tiles through LDS.
-// to_yt != 0: Y -> YT, else YT -> Y.
-__global__ __launch_bounds__(256) void k_transpose(Batch B, int to_yt, int only_tall, int only_wide) {
     __shared__ bf16_t t[64][66];
     const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
-    if ((only_tall && M.wide) || (only_wide && !M.wide)) return;
-    const int R = to_yt ? M.mp : M.np, C = to_yt ? M.np : M.mp;     // source is [R x C]
-    const bf16_t* src = to_yt ? M.Y : M.YT;
-    bf16_t* dst = to_yt ? M.YT : M.Y;
+    const float inv = B.inv_norm[mi];
+    bf16_t* own = M.wide ? M.Y : M.YT;            // [R x C] in the parameter's orientation, padded
+    bf16_t* other = M.wide ? M.YT : M.Y;          // [C x R]
+    const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
     const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
     const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
-    (void)R;
     for (int k = threadIdx.x; k < 64 * 64; k += 256) {
-        const int r = k >> 6, c = k & 63;
-        t[r][c] = src[(size_t)(tr0 + r) * C + tc0 + c];
+        const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
+        const bf16_t v = (r < M.rows && c < M.cols) ? sg::f_to_bf16_bits(M.buf[(size_t)r * M.cols + c] * inv) : (bf16_t)0;
+        own[(size_t)r * C + c] = v;
+        t[k >> 6][k & 63] = v;
     }
     __syncthreads();
     for (int k = threadIdx.x; k < 64 * 64; k += 256) {
-        const int r = k >> 6, c = k & 63;     // output row r (= source column), column c (= source row)
-        dst[(size_t)(tc0 + r) * R + tr0 + c] = t[c][r];
+        const int r = k >> 6, c = k & 63;     // output row r (= own column), column c (= own row)
+        other[(size_t)(tc0 + r) * R + tr0 + c] = t[c][r];
     }
 }
 
@@ -658,14 +634,8 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
 
     hipLaunchKernelGGL(k_momentum, dim3(B.etiles), dim3(256), 0, st, B, momentum);
     hipLaunchKernelGGL(k_norm, dim3(P), dim3(256), 0, st, B);
-    hipLaunchKernelGGL(k_normalize, dim3(B.etiles), dim3(256), 0, st, B);
+    hipLaunchKernelGGL(k_normalize, dim3(B.ttiles), dim3(256), 0, st, B);
     SG_LAUNCH_CHECK("muon prologue");
-    if (ns_steps > 0) {
-        // wide matrices: YT from Y; tall matrices: Y from YT
-        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 1, 0, 1);
-        hipLaunchKernelGGL(k_transpose, dim3(B.ttiles), dim3(256), 0, st, B, 0, 1, 0);
-        SG_LAUNCH_CHECK("muon transpose");
-    }
     for (int it = 0; it < ns_steps; it++) {
         const int sel = it & 1, last = it + 1 == ns_steps;
         hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
