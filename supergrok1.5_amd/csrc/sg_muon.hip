@@ -174,6 +174,34 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
     const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
     const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
     const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
+    const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && (M.cols & 3) == 0 && (((uintptr_t)M.buf) & 15u) == 0;
+    if (full) {
+        // interior tile: a lane moves 16 consecutive elements of a row (four 16-byte loads, two 16-byte stores)
+        const int lr = threadIdx.x >> 2, c0 = (threadIdx.x & 3) * 16;
+        const float4* src = reinterpret_cast<const float4*>(M.buf + (size_t)(tr0 + lr) * M.cols + tc0 + c0);
+        uint32_t pk[8];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float4 v = src[q];
+            const uint32_t b0 = sg::f_to_bf16_bits(v.x * inv), b1 = sg::f_to_bf16_bits(v.y * inv);
+            const uint32_t b2 = sg::f_to_bf16_bits(v.z * inv), b3 = sg::f_to_bf16_bits(v.w * inv);
+            pk[2 * q] = b0 | (b1 << 16);
+            pk[2 * q + 1] = b2 | (b3 << 16);
+            t[lr][c0 + 4 * q] = (bf16_t)b0; t[lr][c0 + 4 * q + 1] = (bf16_t)b1;
+            t[lr][c0 + 4 * q + 2] = (bf16_t)b2; t[lr][c0 + 4 * q + 3] = (bf16_t)b3;
+        }
+        uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
+        dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        __syncthreads();
+        // transposed copy: output row lr (= own column), 16 consecutive output columns (= own rows)
+#pragma unroll
+        for (int q = 0; q < 8; q++) pk[q] = (uint32_t)t[c0 + 2 * q][lr] | ((uint32_t)t[c0 + 2 * q + 1][lr] << 16);
+        uint4* dt = reinterpret_cast<uint4*>(other + (size_t)(tc0 + lr) * R + tr0 + c0);
+        dt[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+        dt[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        return;
+    }
     for (int k = threadIdx.x; k < 64 * 64; k += 256) {
         const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
         const bf16_t v = (r < M.rows && c < M.cols) ? sg::f_to_bf16_bits(M.buf[(size_t)r * M.cols + c] * inv) : (bf16_t)0;
