@@ -26,28 +26,34 @@ def build():
     subprocess.check_call(["make", "-s", "-C", _HERE])
 
 
+def load(path):
+    """CDLL of a build of the checker with the return types set (tests also load deliberately broken builds)."""
+    L = C.CDLL(path)
+    for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf", "sin_small", "cos_small", "sin_tiny", "cos_tiny",
+              "gelu_sigmoid"):
+        f = getattr(L, "orc_" + n)
+        f.restype = C.c_float
+        f.argtypes = [C.c_float]
+    L.orc_abar.restype = C.c_float
+    L.orc_abar.argtypes = [C.c_float, C.c_float]
+    L.orc_f_to_f16.restype = C.c_uint16
+    L.orc_f_to_f16.argtypes = [C.c_float]
+    L.orc_f16_to_f.restype = C.c_float
+    L.orc_f16_to_f.argtypes = [C.c_uint16]
+    L.orc_f_to_bf16.restype = C.c_uint16
+    L.orc_f_to_bf16.argtypes = [C.c_float]
+    L.orc_bf16_to_f.restype = C.c_float
+    L.orc_bf16_to_f.argtypes = [C.c_uint16]
+    L.orc_sg2_step.restype = C.c_int
+    return L
+
+
 def lib():
     global _lib
     if _lib is None:
         if not os.path.exists(_LIB):
             build()
-        _lib = C.CDLL(_LIB)
-        for n in ("exp", "log", "softplus", "sigmoid", "silu", "tanh", "sin", "cos", "rcp_pos", "erfc", "gelu_erf", "sin_small", "cos_small", "sin_tiny", "cos_tiny",
-                  "gelu_sigmoid"):
-            f = getattr(_lib, "orc_" + n)
-            f.restype = C.c_float
-            f.argtypes = [C.c_float]
-        _lib.orc_abar.restype = C.c_float
-        _lib.orc_abar.argtypes = [C.c_float, C.c_float]
-        _lib.orc_f_to_f16.restype = C.c_uint16
-        _lib.orc_f_to_f16.argtypes = [C.c_float]
-        _lib.orc_f16_to_f.restype = C.c_float
-        _lib.orc_f16_to_f.argtypes = [C.c_uint16]
-        _lib.orc_f_to_bf16.restype = C.c_uint16
-        _lib.orc_f_to_bf16.argtypes = [C.c_float]
-        _lib.orc_bf16_to_f.restype = C.c_float
-        _lib.orc_bf16_to_f.argtypes = [C.c_uint16]
-        _lib.orc_sg2_step.restype = C.c_int
+        _lib = load(_LIB)
     return _lib
 
 

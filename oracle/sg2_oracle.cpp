@@ -60,8 +60,14 @@
  * Parity status: the reference's tests hold no golden vectors for this path
  * (tests/test_supergrok2.py checks finiteness and run-to-run determinism
  * only) and its CUDA kernels cannot run here, so every function below is
- * pinned by the independent checks in tests/test_oracle_*.py (numpy/torch
- * restatements, closed forms, library routines), not by reference outputs.
+ * pinned by checks that do not share its code: numpy's stable argsort and a
+ * brute-force rank (sort); closed forms of the recurrence, structural
+ * identities and torch.optim.AdamW (tests/test_oracle_sg2.py); special cases
+ * in which the mathematics fixes the per-element part -- GRU gates closed or
+ * open, one input column at a time, PEER winners known by construction with
+ * exact ties, hand-evaluated expert MLPs, the index clamp, the sense of the
+ * RoPE rotation -- each shown to fail on a build of this file with the
+ * corresponding mistake injected (tests/test_oracle_sg2_pins.py).
  */
 #include <algorithm>
 #include <cmath>

@@ -74,7 +74,7 @@ def step(weights, param, grad, sharp, ea, easq, mu, gru, mfwd, mbwd, sc, dims):
         q = pin @ W[26][hh].T
         ia = (q[:, : dm // 2] @ W[27][hh].T).argmax(-1)
         ib = (q[:, dm // 2:] @ W[28][hh].T).argmax(-1)
-        e = ia * pk + ib
+        e = torch.clamp(ia * pk + ib, max=W1.shape[0] - 1)     # csrc/supergrok2_mamba_peer_kernels.cu:1050-1051
         eidx[:, hh] = e
         zz = torch.relu(W1[e] * g[:, None] + b1[e])
         total = total + (W2[e] * zz).sum(-1) + b2[e]
@@ -87,3 +87,39 @@ def step(weights, param, grad, sharp, ea, easq, mu, gru, mfwd, mbwd, sc, dims):
     p_n = param.reshape(-1).to(F) * (1 - sc["lr"] * sc["wd_eff"]) - (sc["lr"] / sc["bc1"]) * ea_n / denom
     return dict(param=p_n, exp_avg=ea_n, exp_avg_sq=easq_n, mu=mu_n, gru=hn, mamba_fwd=hf, mamba_bwd=hb,
                 perm=perm, expert_idx=eidx, ctx_f=cf, ctx_b=cb, smart=smart)
+
+
+def forward_for_bilevel(W, grad, sharp, gru, mfwd, mbwd, rescale, dims, topk=4):
+    """Differentiable forward with soft top-k routing (grokking_optimizers/mamba3_peer_metanet.py:372-436 of the
+    reference): softmax of 10 x the k best scores of each sub-key, k*k experts per head weighted by the product.
+    W: the 33 weight tensors in `_ops` argument order (float64, may require grad).
+    Returns (smart_grad, new_gru, new_mamba_fwd, new_mamba_bwd)."""
+    dm, H, pk = dims["d_model"], dims["num_heads"], dims["pk_dim"]
+    g, s = grad.reshape(-1).to(F), sharp.reshape(-1).to(F)
+    N = g.numel()
+    perm = torch.sort(g.abs().float(), stable=True).indices
+    x = torch.stack([g[perm], s[perm]], -1) @ W[0].T + W[1]
+    fo, new_f = scan_block(x, W[2:11], mfwd)
+    bo, new_b = scan_block(x.flip(0), W[11:20], mbwd)
+    unsort = torch.argsort(perm)
+    cf, cb = fo[unsort], bo.flip(0)[unsort]
+    Wz, bz, Wr, br, Wh, bh = W[20:26]
+    h = gru.to(F)
+    xin = torch.cat([g[:, None], s[:, None], cf, cb], -1)
+    xh = torch.cat([xin, h], -1)
+    z, r = torch.sigmoid(xh @ Wz.T + bz), torch.sigmoid(xh @ Wr.T + br)
+    hn = (1 - z) * h + z * torch.tanh(torch.cat([xin, r * h], -1) @ Wh.T + bh)
+    pin = torch.cat([hn, cf, cb, g[:, None], s[:, None]], -1)
+    W1, b1, W2, b2 = W[29], W[30], W[31], W[32]
+    total = torch.zeros(N, dtype=F)
+    for hh in range(H):
+        q = pin @ W[26][hh].T
+        va, ia = (q[:, : dm // 2] @ W[27][hh].T).topk(topk, dim=-1)
+        vb, ib = (q[:, dm // 2:] @ W[28][hh].T).topk(topk, dim=-1)
+        sa, sb = torch.softmax(va * 10.0, -1), torch.softmax(vb * 10.0, -1)
+        idx = (ia.unsqueeze(2) * pk + ib.unsqueeze(1)).reshape(N, -1)
+        rw = (sa.unsqueeze(2) * sb.unsqueeze(1)).reshape(N, -1)
+        zz = torch.relu(W1[idx] * g[:, None, None] + b1[idx])
+        out = (W2[idx] * zz).sum(-1) + b2[idx]
+        total = total + (rw * out).sum(1)
+    return g + rescale * total / H, hn, new_f, new_b

@@ -125,37 +125,18 @@ def test_several_chunks():
 # ---------------------------------------------------------------------------------------------------------------
 def _ref_forward_for_bilevel(mn, grad, sharp, gru_state, hf, hb):
     """float64 CPU statement of Mamba3PEERMetaNet.forward_for_bilevel (mamba3_peer_metanet.py:372-436 of the
-    reference) on a double copy `mn` of the module, with ref_fp64.scan_block as the scan."""
-    g, s = grad.reshape(-1), sharp.reshape(-1)
-    N = g.numel()
-    perm = torch.sort(g.abs().float(), stable=True).indices
-    x = mn.input_proj(torch.stack([g[perm], s[perm]], -1))
+    reference) on a double copy `mn` of the module: ref_fp64.forward_for_bilevel (pinned by the closed forms of
+    tests/test_oracle_sg2_pins.py) over the module's own parameters, so that autograd reaches them."""
     blk = lambda b: [b.in_proj.weight, b.dt_proj.weight, b.dt_proj.bias, b.B_proj.weight, b.C_proj.weight, b.A_log, b.D,
                      b.rope_freq, b.out_proj.weight]
-    fo, new_f = ref_fp64.scan_block(x, blk(mn.mamba_fwd), hf)
-    bo, new_b = ref_fp64.scan_block(x.flip(0), blk(mn.mamba_bwd), hb)
-    unsort = torch.argsort(perm)
-    cf, cb = fo[unsort], bo.flip(0)[unsort]
-    xin = torch.cat([g[:, None], s[:, None], cf, cb], -1)
-    xh = torch.cat([xin, gru_state], -1)
-    z, r = torch.sigmoid(mn.gru.W_z(xh)), torch.sigmoid(mn.gru.W_r(xh))
-    hn = (1 - z) * gru_state + z * torch.tanh(mn.gru.W_h(torch.cat([xin, r * gru_state], -1)))
-    pin = torch.cat([hn, cf, cb, g[:, None], s[:, None]], -1)
-    total = torch.zeros(N, 1, dtype=torch.float64)
-    half = mn.d_model // 2
-    for h in range(mn.num_peer_heads):
-        q = mn.peer_queries[h](pin)
-        va, ia = (q[:, :half] @ mn.product_keys_A[h].T).topk(4, dim=-1)
-        vb, ib = (q[:, half:] @ mn.product_keys_B[h].T).topk(4, dim=-1)
-        sa, sb = torch.softmax(va * 10.0, -1), torch.softmax(vb * 10.0, -1)
-        idx = (ia.unsqueeze(2) * mn.pk_dim + ib.unsqueeze(1)).reshape(N, -1)
-        rw = (sa.unsqueeze(2) * sb.unsqueeze(1)).reshape(N, -1)
-        W1, b1, W2, b2 = mn.expert_W1[idx], mn.expert_b1[idx], mn.expert_W2[idx], mn.expert_b2[idx]
-        gx = g.reshape(N, 1, 1, 1).expand(-1, 16, -1, -1)
-        zz = torch.relu(torch.matmul(W1, gx).squeeze(-1) + b1)
-        out = torch.matmul(W2, zz.unsqueeze(-1)).squeeze(-1).squeeze(-1) + b2.squeeze(-1)
-        total = total + (rw * out).sum(1, keepdim=True)
-    return (g[:, None] + mn.rescale * total / mn.num_peer_heads).squeeze(-1), hn, new_f, new_b
+    E = mn.num_experts
+    W = ([mn.input_proj.weight, mn.input_proj.bias] + blk(mn.mamba_fwd) + blk(mn.mamba_bwd) +
+         [mn.gru.W_z.weight, mn.gru.W_z.bias, mn.gru.W_r.weight, mn.gru.W_r.bias, mn.gru.W_h.weight, mn.gru.W_h.bias] +
+         [torch.stack([q.weight for q in mn.peer_queries]), torch.stack(list(mn.product_keys_A)),
+          torch.stack(list(mn.product_keys_B))] +
+         [mn.expert_W1.reshape(E, -1), mn.expert_b1, mn.expert_W2.reshape(E, -1), mn.expert_b2.reshape(-1)])
+    dims = dict(d_model=mn.d_model, num_heads=mn.num_peer_heads, pk_dim=mn.pk_dim)
+    return ref_fp64.forward_for_bilevel(W, grad, sharp, gru_state, hf, hb, mn.rescale, dims)
 
 
 def _meta_net(seed, dev):
