@@ -14,24 +14,23 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd"), os.path.join(ROOT, "tests")):
+for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch (read + written) on the 25M-element workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs scaled by what the same counters read for a 1 GiB device copy; not measured by this script
+# HBM bytes per launch (read + written) on the 25M-element workload: constants copied from the rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE summary under profiles/ (scaled by what the same counters read for a 1 GiB device copy);
+# not measured by this script and valid for the default workload only
 PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.625e9 + 1.612e9, "scan_summary": 0.042e9 + 0.037e9,
                              "elementwise": 2.603e9 + 0.801e9}
-FLOP_PER_ELEMENT = 30e3         # arithmetic actually required per element (both scan directions + elementwise)
-VALU_PEAK_TFLOPS = 157.3
 
 
-def build_workload(name, device, nonzero_sharpness=False):
+def build_workload(name, device, nonzero_sharpness=False, weights="bench"):
     import torch
     import workloads as wl
-    from helpers import DIMS
+    DIMS = wl.DEFAULT_DIMS
     shapes = {"scale50": wl.scale50_shapes, "shared14": wl.shared14_shapes}[name]()
     gh, di, ds = DIMS["gru_hidden"], DIMS["d_inner"], DIMS["d_state"]
     params = [p.reshape(-1).to(device) for p in wl.make_params(shapes, seed=0)]
@@ -51,7 +50,9 @@ def build_workload(name, device, nonzero_sharpness=False):
     sharps = [torch.zeros_like(p) for p in params]
     if nonzero_sharpness:
         sharps = [(g.abs() * 0.5).contiguous() for g in grad_sets[1]]
-    weights = [w.to(device) for w in wl.meta_weights(7)]
+    # "bench": N(0, 0.1) in every tensor (the configuration the metric is quoted on); "module": the optimizer's own
+    # initial meta-net (A_log = log(1..16), default Linear weights)
+    weights = [w.to(device) for w in (wl.meta_weights(7) if weights == "bench" else wl.module_weights(0))]
     return shapes, state, grad_sets, sharps, weights
 
 
@@ -61,7 +62,6 @@ def cpu_baseline(sample_elems_target=4_000_000):
     host core over a bounded sample of the same parameter set."""
     import numpy as np
     import workloads as wl
-    from helpers import default_scalars, f32_scalars, fresh_state_np
     from oracle import oracle as orc
     shapes = wl.scale50_shapes()
     pick, tot = [], 0
@@ -75,10 +75,16 @@ def cpu_baseline(sample_elems_target=4_000_000):
     params = wl.make_params([shapes[i] for i in pick], seed=0)
     grads = wl.make_grads([shapes[i] for i in pick], seed=1, tail_frac=0.005, tail="student3")
     t0 = time.perf_counter()
+    D = wl.DEFAULT_DIMS
     for k, i in enumerate(pick):
-        st = fresh_state_np(params[k].numpy())
         g = grads[k].numpy().reshape(-1)
-        orc.sg2_step(W, st, g, np.zeros_like(g), f32_scalars(default_scalars(i=i)), precision=32, chunk_len=0)
+        n = g.size
+        st = dict(param=params[k].numpy().reshape(-1).copy(), exp_avg=np.zeros(n, np.float32), exp_avg_sq=np.zeros(n, np.float32),
+                  mu=np.zeros(n, np.float32), gru=np.zeros((n, D["gru_hidden"]), np.float32),
+                  mamba_fwd=np.zeros((D["d_inner"], D["d_state"]), np.float32),
+                  mamba_bwd=np.zeros((D["d_inner"], D["d_state"]), np.float32))
+        sc = dict(wl.per_tensor_scalars(i + 1, 1)[i], **wl.shared_scalars())
+        orc.sg2_step(W, st, g, np.zeros_like(g), sc, precision=32, chunk_len=0)
     dt = time.perf_counter() - t0
     return {"value": tot / dt, "unit": "elements/s", "cores": 1, "kind": "port",
             "sample": "tensors %d..%d of the 50-tensor set (%d elements), 1 step, sequential scan, "
@@ -298,7 +304,12 @@ def main():
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
     ap.add_argument("--window", type=int, default=-1, help="scan summary window (-1: library default, 0: off)")
+    ap.add_argument("--weights", default="bench", choices=["bench", "module"],
+                    help="v2 workloads: meta-net weights N(0, 0.1) (default, the measured configuration) or the optimizer's own initialisation")
+    ap.add_argument("--boundary", default="ops", choices=["ops", "cabi"],
+                    help="v2 workloads: time the torch-extension call _ops.supergrok2_mamba_peer_batched_step (default) or the bare C-ABI call")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-class-step", action="store_true", help="skip the wall time of SuperGrok2.step() (keeps a kernel trace to the C-ABI steps)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 1 GiB (a reference point for scaling the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -310,7 +321,7 @@ def main():
 
     import torch
     from grokking_optimizers import _cabi
-    from sg2_harness import per_tensor_scalars, shared_scalars
+    from workloads import per_tensor_scalars, shared_scalars
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     if args.workload not in ("scale50", "shared14"):
@@ -318,10 +329,23 @@ def main():
         return
     if _cabi.lib().sg2_set_chunk_len(args.chunk_len) or _cabi.lib().sg2_set_scan_window(args.window):
         raise SystemExit(_cabi.last_error())
-    shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev, args.sharpness)
+    shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev, args.sharpness, args.weights)
     total = sum(p.numel() for p in st["params"])
-    step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
-                         st["counts"])
+    D = _cabi.DEFAULT_DIMS
+    if args.boundary == "cabi":
+        step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
+                             st["counts"])
+    else:
+        # the reference's own entry point: supergrok2_mamba_peer_batched_step of the torch extension, 51 arguments
+        from grokking_optimizers import _ops
+
+        def step(grads, sharps_, per_tensor, sh):
+            col = lambda k: [float(sc[k]) for sc in per_tensor]
+            _ops.supergrok2_mamba_peer_batched_step(
+                st["params"], grads, sharps_, st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"], *weights,
+                col("alpha"), col("lamb_eff"), col("beta1"), col("bc1"), col("bc2"), sh["rescale"], sh["beta2"], sh["lr"],
+                sh["wd_eff"], sh["eps"], D["d_model"], D["d_state"], D["d_inner"], D["gru_hidden"], D["num_heads"],
+                D["pk_dim"], D["expert_hidden"], D["num_experts"], st["counts"])
     shared = shared_scalars()
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -363,16 +387,18 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "SuperGrok v2 full step, %d tensors, %d elements (%s), fp32, bilevel off"
                                % (len(shapes), total, "50 log-uniform tensors" if args.workload == "scale50" else "2-layer transformer set"),
-                   "chunk_len": _cabi.chunk_len_for([p.numel() for p in st["params"]]), "summary_window": _cabi.lib().sg2_get_scan_window()},
+                   "chunk_len": _cabi.chunk_len_for([p.numel() for p in st["params"]]), "summary_window": _cabi.lib().sg2_get_scan_window(),
+                   "timed_call": "_ops.supergrok2_mamba_peer_batched_step" if args.boundary == "ops" else "sg2_batched_step (C ABI)",
+                   "meta_weights": "N(0, 0.1), seed 7" if args.weights == "bench" else "Mamba3PEERMetaNet() initialisation, seed 0"},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if args.workload == "scale50" else None,
+                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if (args.workload, args.weights) == ("scale50", "bench") else None,
                      "kernel_ms": stage_avg[dom]},
         "step_hbm_frac": BYTES_PER_ELEMENT * value / 1e9 / HBM_PEAK_GBS,
-        "step_valu_frac": FLOP_PER_ELEMENT * value / 1e12 / VALU_PEAK_TFLOPS,
         "stage_ms": stage_avg,
     }
-    out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
+    if not args.no_class_step:
+        out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

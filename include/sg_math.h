@@ -102,7 +102,10 @@ SG_HD float sg_log(float u) {
 
 /* softplus with the reference's guard: raw > 20 passes through. */
 SG_HD float sg_softplus(float x) {
-    return (x > 20.0f) ? x : sg_log(1.0f + sg_exp(x));
+    /* evaluated unconditionally and selected (sg_exp clamps its argument, so the unused value is finite): a
+     * data-dependent branch here would split the callers' code at every call */
+    const float y = sg_log(1.0f + sg_exp(x));
+    return (x > 20.0f) ? x : y;
 }
 
 SG_HD float sg_sigmoid(float x) { return 1.0f / (1.0f + sg_exp(-x)); }

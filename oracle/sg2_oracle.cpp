@@ -48,14 +48,17 @@
  * chunking (ceil(N/512) steps per thread, Blelloch tree over 512 summaries)
  * is one more member of this family: all of them differ from the sequential
  * result only by re-association of the affine products.
- * window > 0 (a multiple of 64, < chunk_len): the summary of a chunk is first
- * accumulated over its last `window` steps only.  The recurrence contracts
- * (|A_bar| < 1), so the 2x2 part M of that window summary is usually
- * vanishingly small; if every |entry| of M in all (j,p) is below 2^-100 the
- * chunk summary is taken as (0, b_window) -- whatever state entered the window
- * is multiplied by less than 2^-100, far below fp32 resolution -- otherwise the
- * summary is recomputed over the whole chunk.  window <= 0 always uses the
- * whole chunk.
+ * window > 0 (a multiple of 64, < chunk_len): the summary of a chunk is built
+ * backwards in blocks of `window` steps.  The last block is summarised from
+ * the identity; the recurrence contracts (|A_bar| < 1), so the 2x2 part M of
+ * that summary is usually vanishingly small: if every |entry| of M in all
+ * (j,p) is below 2^-100 the chunk summary is taken as (0, b) -- whatever state
+ * entered the block is multiplied by less than 2^-100, far below fp32
+ * resolution.  Otherwise the block before it is summarised from the identity
+ * and the summary so far is applied on top (M, b) <- (M_late M_early,
+ * M_late b_early + b_late), and the test is repeated, until it passes or the
+ * chunk start is reached (then the summary is the exact one, re-associated by
+ * blocks).  window <= 0 accumulates the whole chunk in one block.
  *
  * Parity status: the reference's tests hold no golden vectors for this path
  * (tests/test_supergrok2.py checks finiteness and run-to-run determinism
@@ -369,16 +372,20 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
 
     /* pass 1 + 2: summaries of chunks 0..nchunks-2, start states of 1..nchunks-1 */
     std::vector<R> sm(di * hp * 6);
+    std::vector<R> late(di * hp * 6);
     for (int64_t c = 0; c + 1 < nchunks; c++) {
-        const bool try_window = window > 0 && window < chunk_len;
-        for (int attempt = try_window ? 0 : 1; attempt < 2; attempt++) {
-            const int64_t first = (attempt == 0) ? (c + 1) * chunk_len - window : c * chunk_len;
+        /* the chunk is walked backwards in blocks of `window` steps: each block is summarised from the identity, the
+         * summary of everything after it is applied on top, and the walk stops once the 2x2 part has contracted */
+        const int64_t u0 = c * chunk_len, u1 = (c + 1) * chunk_len;
+        int64_t blk_end = u1, blk_first = (window > 0 && window < chunk_len) ? std::max(u0, u1 - window) : u0;
+        bool have_late = false;
+        for (;;) {
             for (int i = 0; i < di * hp; i++) {
                 R* m = &sm[i * 6];
                 m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 1; m[4] = 0; m[5] = 0;   /* col0=(m0,m1) col1=(m2,m3) b=(m4,m5) */
             }
-            for (int64_t tile0 = first; tile0 < (c + 1) * chunk_len; tile0 += ORC_TILE) {
-                const int cnt = (int)std::min<int64_t>(ORC_TILE, (c + 1) * chunk_len - tile0);
+            for (int64_t tile0 = blk_first; tile0 < blk_end; tile0 += ORC_TILE) {
+                const int cnt = (int)std::min<int64_t>(ORC_TILE, blk_end - tile0);
                 tile_coefficients<O>(d, w, A, x, gs, N, reverse, tile0, cnt, false, tc);
                 for (int k = 0; k < cnt; k++) {
                     const StepProj<O>& sp = tc.sp[k];
@@ -400,19 +407,34 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
                     }
                 }
             }
-            if (attempt == 0) {
-                bool contracted = true;      /* every |M entry| < 2^-100 (a NaN counts as not contracted) */
-                for (int i = 0; i < di * hp && contracted; i++)
-                    for (int k = 0; k < 4; k++) {
-                        const R a = sm[i * 6 + k] < 0 ? -sm[i * 6 + k] : sm[i * 6 + k];
-                        if (!(a < (R)7.888609052210118e-31)) { contracted = false; break; }
-                    }
-                if (contracted) {
-                    for (int i = 0; i < di * hp; i++)
-                        for (int k = 0; k < 4; k++) sm[i * 6 + k] = 0;
-                    break;
+            if (have_late)       /* sm covers [blk_first, blk_end), late covers [blk_end, u1): both = late o sm */
+                for (int i = 0; i < di * hp; i++) {
+                    const R* L = &late[i * 6];
+                    R* m = &sm[i * 6];
+                    const R e0 = m[0], e1 = m[1], e2 = m[2], e3 = m[3], e4 = m[4], e5 = m[5];
+                    m[0] = O::fma(L[0], e0, L[2] * e1);
+                    m[1] = O::fma(L[1], e0, L[3] * e1);
+                    m[2] = O::fma(L[0], e2, L[2] * e3);
+                    m[3] = O::fma(L[1], e2, L[3] * e3);
+                    m[4] = O::fma(L[0], e4, O::fma(L[2], e5, L[4]));
+                    m[5] = O::fma(L[1], e4, O::fma(L[3], e5, L[5]));
                 }
+            if (blk_first == u0) break;
+            bool contracted = true;      /* every |M entry| < 2^-100 (a NaN counts as not contracted) */
+            for (int i = 0; i < di * hp && contracted; i++)
+                for (int k = 0; k < 4; k++) {
+                    const R a = sm[i * 6 + k] < 0 ? -sm[i * 6 + k] : sm[i * 6 + k];
+                    if (!(a < (R)7.888609052210118e-31)) { contracted = false; break; }
+                }
+            if (contracted) {
+                for (int i = 0; i < di * hp; i++)
+                    for (int k = 0; k < 4; k++) sm[i * 6 + k] = 0;
+                break;
             }
+            late = sm;
+            have_late = true;
+            blk_end = blk_first;
+            blk_first = std::max(u0, blk_first - window);
         }
         const R* h0 = &hstart[(size_t)c * di * ds];
         R* h1 = &hstart[(size_t)(c + 1) * di * ds];

@@ -333,8 +333,12 @@ void supergrok2_mamba_peer_batched_step(
         t.bc1 = bc1s[i];
         t.bc2 = bc2s[i];
     }
+    int64_t total = 0;
+    for (size_t i = 0; i < P; i++) total += numels[i];
     const size_t bytes = sg2_workspace_bytes(&dims, (int)P, numels.data());
-    TORCH_CHECK(bytes > 0 || std::string(sg_last_error()).empty(), fn, ": ", sg_last_error());
+    // 0 bytes with elements to process means the library refused the call (its message is fresh); with no elements
+    // at all there is no message to report: the call below validates the dimensions and returns
+    TORCH_CHECK(bytes > 0 || total == 0, fn, ": ", sg_last_error());
     auto ws = make_workspace(bytes, params[0]);
     Sg2Scalars sc = {rescale, beta2, lr, wd_eff, eps};
     check_status(sg2_batched_step(&dims, &W, (int)P, ts.data(), &sc, expert_counts.data_ptr<int32_t>(), ws.data_ptr(),

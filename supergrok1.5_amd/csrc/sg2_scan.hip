@@ -73,16 +73,6 @@ static_assert(HT_STEP % UB == 0 && SCAN_TT % HT_STEP == 0 && SCAN_TT / HT_STEP <
 #endif
 #define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
 
-struct DirW {
-    sg::cfloat_p in_proj, dt_W, dt_b, Bp, Cp, A_log, D, rope, out_proj;
-};
-__device__ __forceinline__ DirW dir_weights(const Sg2Weights& W, int dir) {
-    const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-    return {sg::as_const(W.w[b]),     sg::as_const(W.w[b + 1]), sg::as_const(W.w[b + 2]),
-            sg::as_const(W.w[b + 3]), sg::as_const(W.w[b + 4]), sg::as_const(W.w[b + 5]),
-            sg::as_const(W.w[b + 6]), sg::as_const(W.w[b + 7]), sg::as_const(W.w[b + 8])};
-}
-
 __device__ __forceinline__ float dpp_quad_swap1(float v) {   // lane ^ 1
     return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0xB1, 0xF, 0xF, true));
 }
@@ -115,46 +105,62 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
 }
 
 // Projections of one timestep from the element's (g, s).  Each half of the workgroup produces its
-// half of dt / dt*x-branch / B (/ D*x-branch / C / gate).  HALF is a template parameter so that every coefficient
-// index is a compile-time constant (scalar loads).  c points at this direction's coefficients.
+// half of dt / dt*x-branch / B (/ D*x-branch / C / gate).  HALF is a template parameter so that every row
+// index is a compile-time constant.  The coefficient triple of an output row sits in the four padding floats of the
+// LDS row it produces (staged once per workgroup, see stage_coefficients): one 16-byte broadcast read per output,
+// no scalar loads in the loop (a scalar load can only be waited for with lgkmcnt(0), which also drains the LDS queue).
 // Returns bit 0: every rotation angle of this timestep, over this half's columns, is small enough for
 // sg_sincos_small; bit 1: small enough for sg_sincos_tiny (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
 template <bool OUT, int HALF, bool HAS_S>
-__device__ __forceinline__ int project_tile(sg::cfloat_p c, sg::cfloat_p Dw, float g, float s, int tu, float* s_dt,
-                                             float* s_ux, float* s_dx, float* s_B, float* s_C, float* s_gate, const float* s_fmax) {
+__device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_dt, float* s_ux, float* s_dx, float* s_B,
+                                             float* s_C, float* s_gate, const float* s_fmax) {
     // HAS_S is false for a tensor whose sharpness is all zero: fma(c_s, 0, c_0) is c_0 itself, so the term is skipped
-    auto eval = [&](int group, int row) {
-        const sg::cfloat_p t = c + (group * 16 + row) * 3;
-        return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]);
-    };
+    auto eval = [&](const f32x4 t) { return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]); };
+    auto coef = [&](const float* arr, int row) { return *reinterpret_cast<const f32x4*>(arr + row * LDS_STRIDE + SCAN_TT); };
     bool small = true, tiny = true;
 #pragma unroll
     for (int q = 0; q < DI / 2; q++) {
         const int jj = HALF * (DI / 2) + q;
-        const float dtv = sg_softplus(eval(SG2_COMP_DT, jj));
+        const float dtv = sg_softplus(eval(coef(s_dt, jj)));
         const float amax = dtv * s_fmax[jj];
         small = small && (amax < SG_SINCOS_SMALL_LIMIT);
         tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
-        const float xbv = eval(SG2_COMP_XB, jj);
+        const f32x4 cx = coef(s_ux, jj);              // x-branch coefficients; [3] = D of this column
+        const float xbv = eval(cx);
         s_dt[jj * LDS_STRIDE + tu] = dtv;
         s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
-        if (OUT) s_dx[jj * LDS_STRIDE + tu] = Dw[jj] * xbv;
+        if (OUT) s_dx[jj * LDS_STRIDE + tu] = cx[3] * xbv;
     }
 #pragma unroll
     for (int q = 0; q < DS / 2; q++) {
         const int ss = HALF * (DS / 2) + q;
-        s_B[ss * LDS_STRIDE + tu] = eval(SG2_COMP_B, ss);
-        if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(SG2_COMP_C, ss);
+        s_B[ss * LDS_STRIDE + tu] = eval(coef(s_B, ss));
+        if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(coef(s_C, ss));
     }
     if (OUT) {
 #pragma unroll
         for (int q = 0; q < DI / 2; q++) {
             const int jj = HALF * (DI / 2) + q;
-            s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(SG2_COMP_Z, jj));
+            s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(coef(s_gate, jj)));
         }
     }
     return (small ? 1 : 0) | (tiny ? 2 : 0);
+}
+
+// Once per workgroup: the composed coefficient triples of this direction (and D) into the padding of the LDS rows.
+template <bool OUT>
+__device__ __forceinline__ void stage_coefficients(const float* __restrict__ comp, const float* __restrict__ Dw, int tid, float* s_dt,
+                                                   float* s_ux, float* s_B, float* s_C, float* s_gate) {
+    static_assert(DI == 16 && DS == 16 && SG2_COMP_GROUPS * 16 <= SCAN_THREADS, "one thread per (group, row)");
+    if (tid < SG2_COMP_GROUPS * 16) {
+        const int group = tid / 16, row = tid % 16;
+        float* arr = group == SG2_COMP_XB ? s_ux : group == SG2_COMP_DT ? s_dt : group == SG2_COMP_B ? s_B : group == SG2_COMP_C ? s_C : s_gate;
+        if (OUT || (group != SG2_COMP_C && group != SG2_COMP_Z)) {
+            const float* t = comp + (group * 16 + row) * 3;
+            *reinterpret_cast<f32x4*>(arr + row * LDS_STRIDE + SCAN_TT) = f32x4{t[0], t[1], t[2], group == SG2_COMP_XB ? Dw[row] : 0.0f};
+        }
+    }
 }
 
 // scan state of one lane: OUT -> (he,ho) only; summary -> also the two columns of M
@@ -229,6 +235,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     // y of column j goes where dt of column j was: both are touched only by the 8 lanes of column j, in program order
     float* const s_y = s_dt;
     __shared__ float s_fmax[DI];
+    __shared__ __attribute__((aligned(16))) float s_wout[OUT ? DM * DI : 4];      // out_proj of this direction
     __shared__ unsigned long long s_large[2];      // per projection half: bit t set = timestep t of the tile needs the full sin/cos
     __shared__ unsigned long long s_nottiny[2];    // ... bit t set = timestep t is not eligible for sg_sincos_tiny
 
@@ -242,12 +249,10 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const int N = T.numel, off = T.off;
     const int u0 = c * pl.chunk_len;                       // first scan step of the chunk
     const int u1 = min(u0 + pl.chunk_len, N);
-    const DirW w0 = dir_weights(pl.W, dir);
     const uint32_t* __restrict__ skey = pl.keys[0] + off;      // sorted |g| bits
     const int32_t* __restrict__ sval = pl.vals[0] + off;       // element index | sign of g
     const float* __restrict__ ssrt = pl.ssorted + off;          // sharpness in sorted order
     const bool has_s = __builtin_amdgcn_readfirstlane(pl.sharp_nonzero[ti]) != 0;
-    const sg::cfloat_p comp0 = sg::as_const(pl.comp) + dir * (SG2_COMP_GROUPS * 16 * 3);
 
     const int tid = threadIdx.x;
     const int tu = tid & (SCAN_TT - 1);                                   // projection role: timestep of the tile
@@ -265,6 +270,9 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         f = sg_max(f, dpp_quad_swap2(f));
         f = sg_max(f, dpp_half_mirror(f));
         if (p == 0) s_fmax[j] = f;
+        stage_coefficients<OUT>(pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3), pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_B, s_C, s_gate);
+        static_assert(DM * DI == SCAN_THREADS, "one out_proj entry per thread");
+        if (OUT) s_wout[tid] = pl.W.w[dir ? W_B_OUT : W_F_OUT][tid];
         __syncthreads();
     }
 
@@ -275,44 +283,53 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         S.ho = hs[SCAN_THREADS + tid];
     }
 
-    int first = u0;
-    bool windowed = false;
-    if (!OUT && pl.window > 0 && pl.window < pl.chunk_len) {
-        first = u1 - pl.window;
-        windowed = true;
-    }
-    for (;;) {
-    for (int tile0 = first; tile0 < u1; tile0 += SCAN_TT) {
-        const int cnt = min(SCAN_TT, u1 - tile0);
-        // the coefficients are re-read (scalar loads, cache hits) in every tile instead of being hoisted
-        const int zo = sg::opaque_zero();
-        const DirW w = {w0.in_proj + zo, w0.dt_W + zo, w0.dt_b + zo, w0.Bp + zo, w0.Cp + zo,
-                        w0.A_log + zo, w0.D + zo, w0.rope + zo, w0.out_proj + zo};
-        const sg::cfloat_p comp = comp0 + zo;
-        // ---------------- phase A: projections of SCAN_TT timesteps -> LDS
+    // Summary pass: the chunk is walked backwards in blocks of `window` steps.  Each block is summarised from the
+    // identity and the summary of everything after it (`late`) is applied on top; as soon as the 2x2 part of the
+    // running summary has contracted below 2^-100 the steps before the block cannot matter and the walk stops.
+    int blk_end = u1;
+    int blk_first = u0;
+    if (!OUT && pl.window > 0 && pl.window < pl.chunk_len) blk_first = max(u0, u1 - pl.window);
+    LaneState late = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
+    bool have_late = false;
+    // inputs of one tile (sorted |g| bits, payload, sorted sharpness) for this lane's timestep; zero beyond the block
+    uint32_t nx_key = 0;
+    int32_t nx_val = 0;
+    float nx_sh = 0.0f;
+    auto load_inputs = [&](int tile0) {
         const int u = tile0 + tu;
-        const bool valid = u < u1;
-        int orig = 0;
-        float g = 0.0f, sh = 0.0f;
-        if (valid) {
+        if (u < blk_end) {
             const int t = dir ? (N - 1 - u) : u;
-            const int32_t v = sval[t];
-            orig = v & 0x7fffffff;
-            orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
-            g = sg_i2f((int32_t)skey[t] | (v & (int32_t)0x80000000));
-            sh = ssrt[t];
+            nx_key = skey[t];
+            nx_val = sval[t];
+            nx_sh = ssrt[t];
         }
+    };
+    for (;;) {
+    load_inputs(blk_first);
+    for (int tile0 = blk_first; tile0 < blk_end; tile0 += SCAN_TT) {
+        const int cnt = min(SCAN_TT, blk_end - tile0);
+        // ---------------- phase A: projections of SCAN_TT timesteps -> LDS
+        // this tile's inputs were requested one tile ago (or just before the loop); request the next tile's now
+        const uint32_t kbits = nx_key;
+        const int32_t v = nx_val;
+        const float shv = nx_sh;
+        const bool valid = tile0 + tu < blk_end;
+        if (tile0 + SCAN_TT < blk_end) load_inputs(tile0 + SCAN_TT);
+        int orig = v & 0x7fffffff;
+        orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
+        const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
+        const float sh = valid ? shv : 0.0f;
         int angle_t;
         if (has_s) {
             if (half == 0)
-                angle_t = project_tile<OUT, 0, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 0, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
             else
-                angle_t = project_tile<OUT, 1, true>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 1, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         } else {
             if (half == 0)
-                angle_t = project_tile<OUT, 0, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 0, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
             else
-                angle_t = project_tile<OUT, 1, false>(comp, w.D, g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<OUT, 1, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
         }
         {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!(angle_t & 1));
@@ -387,13 +404,16 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             float cx[DM / 2];
 #pragma unroll
             for (int q = 0; q < DM / 2; q++) {
+                // row (DM/2) * half + q of out_proj: the same address for every lane of the wave (broadcast reads)
+                const float* wr = s_wout + (half * (DM / 2) + q) * DI;
                 float a = 0.0f;
-                if (half == 0) {
 #pragma unroll
-                    for (int jj = 0; jj < DI; jj++) a = sg_fma(w.out_proj[q * DI + jj], o[jj], a);
-                } else {
-#pragma unroll
-                    for (int jj = 0; jj < DI; jj++) a = sg_fma(w.out_proj[(DM / 2 + q) * DI + jj], o[jj], a);
+                for (int m = 0; m < DI; m += 4) {
+                    const f32x4 w4 = *reinterpret_cast<const f32x4*>(wr + m);
+                    a = sg_fma(w4[0], o[m], a);
+                    a = sg_fma(w4[1], o[m + 1], a);
+                    a = sg_fma(w4[2], o[m + 2], a);
+                    a = sg_fma(w4[3], o[m + 3], a);
                 }
                 cx[q] = a;
             }
@@ -404,17 +424,29 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             __syncthreads();
         }
     }
-    if (OUT || !windowed) break;
-    {   // did the window contract?  (a NaN counts as "no")
+    if (OUT) break;
+    if (have_late) {     // S covers [blk_first, blk_end), late covers [blk_end, u1): the summary of both is late o S
+        const LaneState E = S;
+        S.c0e = sg_fma(late.c0e, E.c0e, late.c1e * E.c0o);
+        S.c0o = sg_fma(late.c0o, E.c0e, late.c1o * E.c0o);
+        S.c1e = sg_fma(late.c0e, E.c1e, late.c1e * E.c1o);
+        S.c1o = sg_fma(late.c0o, E.c1e, late.c1o * E.c1o);
+        S.he = sg_fma(late.c0e, E.he, sg_fma(late.c1e, E.ho, late.he));
+        S.ho = sg_fma(late.c0o, E.he, sg_fma(late.c1o, E.ho, late.ho));
+    }
+    if (blk_first == u0) break;       // the whole chunk is covered
+    {   // has the running summary contracted?  (a NaN counts as "no")
         const float mx = sg_max(sg_max(sg_abs(S.c0e), sg_abs(S.c0o)), sg_max(sg_abs(S.c1e), sg_abs(S.c1o)));
         if (!__syncthreads_or(!(mx < 7.888609052210118e-31f))) {
             S.c0e = S.c0o = S.c1e = S.c1o = 0.0f;
             break;
         }
-        windowed = false;
-        first = u0;
-        S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     }
+    late = S;
+    have_late = true;
+    blk_end = blk_first;
+    blk_first = max(u0, blk_first - pl.window);
+    S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     }
 
     if (OUT) {

@@ -21,7 +21,14 @@ int g_window = 256;
 // Longer chunks mean fewer summaries (less work in the first scan pass and the prefix), shorter chunks
 // mean more workgroups.  Take the longest of 4096 / 2048 / 1024 that still gives the replay pass about
 // four full waves of workgroups on 256 CUs.
-int auto_chunk_len(int P, const int64_t* numels) {
+// tensor sizes of a call, either as a plain array (the *_bytes queries) or read from the tensor records (no copy)
+struct Numels {
+    const int64_t* plain;
+    const Sg2Tensor* tensors;
+    int64_t operator[](int i) const { return plain ? plain[i] : tensors[i].numel; }
+};
+
+int auto_chunk_len(int P, Numels numels) {
     for (int L = 4096; L > 1024; L >>= 1) {
         int64_t wgs = 0;
         for (int i = 0; i < P; i++) wgs += 2 * ((numels[i] + L - 1) / L);
@@ -29,7 +36,7 @@ int auto_chunk_len(int P, const int64_t* numels) {
     }
     return 1024;
 }
-int effective_chunk_len(int P, const int64_t* numels) { return g_chunk_len > 0 ? g_chunk_len : auto_chunk_len(P, numels); }
+int effective_chunk_len(int P, Numels numels) { return g_chunk_len > 0 ? g_chunk_len : auto_chunk_len(P, numels); }
 
 // ---- optional per-stage timing with HIP events on the step's stream
 constexpr int PROF_MARKS = SG2_PROF_STAGES + 1;
@@ -45,7 +52,7 @@ struct Layout {
     size_t tables_bytes;
 };
 
-int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bilevel = false) {
+int make_layout(int P, Numels numels, int chunk_len, Layout* L, bool bilevel = false) {
     int64_t total = 0, et = 0, stl = 0, ch = 0, wch = 0;
     for (int i = 0; i < P; i++) {
         const int64_t n = numels[i];
@@ -84,6 +91,34 @@ int make_layout(int P, const int64_t* numels, int chunk_len, Layout* L, bool bil
     L->off_adj_blk = take(bilevel ? 4 * 2 * (size_t)SG2_BWD_STRIDE : 0);
     L->bytes = o;
     return 0;
+}
+
+
+// Per-call tables travel as kernel arguments: UPLOAD_RECS tensor records and their entries of the four prefix
+// tables (tiles of the elementwise kernels, sort tiles, scan chunks, chunks with a summary) per launch.
+constexpr int UPLOAD_RECS = 24;
+struct TableChunk {
+    TensorDev rec[UPLOAD_RECS];
+    int pre[4][UPLOAD_RECS];       // prefix table q, entries i0+1 .. i0+cnt
+    TensorDev* dst_rec;
+    int* dst_pre;                  // four tables of P+1 ints, back to back
+    int* flags;                    // per-tensor "sharpness is not all zero" flags to clear, or NULL to keep them
+    int i0, cnt, P;
+};
+static_assert(sizeof(TableChunk) <= 3600, "kernel arguments stay well below 4 KB");
+
+__global__ __launch_bounds__(256) void k_tables(TableChunk c) {
+    constexpr int WORDS = sizeof(TensorDev) / 4;
+    const int* src = reinterpret_cast<const int*>(c.rec);
+    int* dst = reinterpret_cast<int*>(c.dst_rec + c.i0);
+    for (int w = threadIdx.x; w < c.cnt * WORDS; w += 256) dst[w] = src[w];
+    for (int w = threadIdx.x; w < 4 * c.cnt; w += 256) {
+        const int q = w / c.cnt, k = w % c.cnt;
+        c.dst_pre[q * (c.P + 1) + c.i0 + 1 + k] = c.pre[q][k];
+    }
+    if (c.i0 == 0 && threadIdx.x < 4) c.dst_pre[threadIdx.x * (c.P + 1)] = 0;
+    if (c.flags != nullptr)
+        for (int k = threadIdx.x; k < c.cnt; k += 256) c.flags[c.i0 + k] = 0;
 }
 
 }  // namespace
@@ -157,7 +192,7 @@ int sg2_set_chunk_len(int chunk_len) {
 int sg2_get_chunk_len(void) { return sg2::g_chunk_len; }
 int sg2_chunk_len_for(int num_tensors, const int64_t* numels) {
     if (num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
-    return sg2::effective_chunk_len(num_tensors, numels);
+    return sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr});
 }
 
 int sg2_set_scan_window(int window) {
@@ -171,7 +206,7 @@ int sg2_get_scan_window(void) { return sg2::g_window; }
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;
-    if (sg2::make_layout(num_tensors, numels, sg2::effective_chunk_len(num_tensors, numels), &L)) return 0;
+    if (sg2::make_layout(num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L)) return 0;
     return L.bytes;
 }
 
@@ -193,10 +228,9 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
         if (!weights->w[k]) return sg::fail("weight pointer %d is NULL", k);
     const int P = num_tensors;
 
-    std::vector<int64_t> numels(P);
+    const Numels numels = {nullptr, tensors};
     for (int i = 0; i < P; i++) {
         const Sg2Tensor& t = tensors[i];
-        numels[i] = t.numel;
         if (t.numel > 0) {
             if (!t.grad || !t.sharpness || !t.mamba_fwd_state || !t.mamba_bwd_state) return sg::fail("tensor %d: NULL pointer", i);
             if (full_step && (!t.param || !t.exp_avg || !t.exp_avg_sq || !t.mu || !t.gru_state)) return sg::fail("tensor %d: NULL pointer", i);
@@ -204,42 +238,47 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
             if (full_step && ((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
         }
     }
-    const int chunk_len = effective_chunk_len(P, numels.data());
-    if (make_layout(P, numels.data(), chunk_len, &L, bilevel)) return 1;
+    const int chunk_len = effective_chunk_len(P, numels);
+    if (make_layout(P, numels, chunk_len, &L, bilevel)) return 1;
     if (L.total == 0) return 0;
     if (!workspace || workspace_bytes < L.bytes)
         return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
     if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
-    // ---- host tables -> one blob -> device
-    std::vector<unsigned char> blob(L.tables_bytes);
-    TensorDev* td = reinterpret_cast<TensorDev*>(blob.data());
-    int* pre = reinterpret_cast<int*>(blob.data() + sizeof(TensorDev) * (size_t)P);
-    int *p_et = pre, *p_st = pre + (P + 1), *p_ch = pre + 2 * (P + 1), *p_wc = pre + 3 * (P + 1);
-    p_et[0] = p_st[0] = p_ch[0] = p_wc[0] = 0;
-    int off = 0;
-    for (int i = 0; i < P; i++) {
-        const Sg2Tensor& t = tensors[i];
-        const int n = (int)t.numel;
-        const int nc = (n + chunk_len - 1) / chunk_len;
-        TensorDev& d = td[i];
-        d.param = t.param; d.grad = t.grad; d.sharp = t.sharpness;
-        d.ea = t.exp_avg; d.easq = t.exp_avg_sq; d.mu = t.mu; d.gru = t.gru_state;
-        d.mfwd = t.mamba_fwd_state; d.mbwd = t.mamba_bwd_state;
-        d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
-        d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
-        d.step_size = full_step ? scalars->lr / t.bc1 : 0.0f;
-        for (int k = 0; k < 5; k++) d.pad_[k] = 0;
-        off += n;
-        p_et[i + 1] = p_et[i] + (n + ELEM_TILE - 1) / ELEM_TILE;
-        p_st[i + 1] = p_st[i] + (n + SORT_TILE - 1) / SORT_TILE;
-        p_ch[i + 1] = p_ch[i] + nc;
-        p_wc[i + 1] = p_wc[i] + (nc > 0 ? nc - 1 : 0);
-    }
+    // ---- per-tensor records and the four prefix tables: written by k_tables from kernel arguments, UPLOAD_RECS
+    // tensors per launch (no host-to-device copy: nothing here blocks the host or depends on the lifetime of host
+    // memory, and the call can be recorded into a graph)
     unsigned char* ws = static_cast<unsigned char*>(workspace);
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_tables, blob.data(), L.tables_bytes, hipMemcpyHostToDevice, st));
-    if (!keep_flags) {
-        const std::vector<int> zeros((size_t)P, 0);
-        SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_flags, zeros.data(), sizeof(int) * (size_t)P, hipMemcpyHostToDevice, st));
+    {
+        TensorDev* d_rec = reinterpret_cast<TensorDev*>(ws + L.off_tables);
+        int* d_pre = reinterpret_cast<int*>(ws + L.off_tables + sizeof(TensorDev) * (size_t)P);
+        int* d_flags = keep_flags ? nullptr : reinterpret_cast<int*>(ws + L.off_flags);
+        int off = 0, run[4] = {0, 0, 0, 0};
+        for (int i0 = 0; i0 < P; i0 += UPLOAD_RECS) {
+            TableChunk c;
+            c.dst_rec = d_rec; c.dst_pre = d_pre; c.flags = d_flags;
+            c.i0 = i0; c.cnt = P - i0 < UPLOAD_RECS ? P - i0 : UPLOAD_RECS; c.P = P;
+            for (int k = 0; k < c.cnt; k++) {
+                const Sg2Tensor& t = tensors[i0 + k];
+                const int n = (int)t.numel;
+                const int nc = (n + chunk_len - 1) / chunk_len;
+                TensorDev& d = c.rec[k];
+                d.param = t.param; d.grad = t.grad; d.sharp = t.sharpness;
+                d.ea = t.exp_avg; d.easq = t.exp_avg_sq; d.mu = t.mu; d.gru = t.gru_state;
+                d.mfwd = t.mamba_fwd_state; d.mbwd = t.mamba_bwd_state;
+                d.off = off; d.numel = n; d.dtype = t.dtype; d.nchunks = nc;
+                d.alpha = t.alpha_mu; d.lamb = t.lamb_eff; d.beta1 = t.beta1; d.bc2 = t.bc2;
+                d.step_size = full_step ? scalars->lr / t.bc1 : 0.0f;
+                for (int q = 0; q < 5; q++) d.pad_[q] = 0;
+                off += n;
+                run[0] += (n + ELEM_TILE - 1) / ELEM_TILE;
+                run[1] += (n + SORT_TILE - 1) / SORT_TILE;
+                run[2] += nc;
+                run[3] += nc > 0 ? nc - 1 : 0;
+                for (int q = 0; q < 4; q++) c.pre[q][k] = run[q];
+            }
+            hipLaunchKernelGGL(k_tables, dim3(1), dim3(256), 0, st, c);
+            SG_LAUNCH_CHECK("k_tables");
+        }
     }
 
     pl.tensors = reinterpret_cast<const TensorDev*>(ws + L.off_tables);
@@ -273,15 +312,9 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.adj_blk = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_blk) : nullptr;
     return 0;
 }
-}  // namespace sg2
 
-extern "C" {
-
-int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
-                     const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
-                     const Sg2Debug* debug, void* stream) {
-    using namespace sg2;
-    hipStream_t st = (hipStream_t)stream;
+int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const Sg2Scalars* scalars,
+             int32_t* expert_counts, void* workspace, size_t workspace_bytes, const Sg2Debug* debug, hipStream_t st) {
     Plan pl;
     Layout L;
     if (build_plan(dims, weights, num_tensors, tensors, scalars, workspace, workspace_bytes, true, false, false, st, &pl, &L)) return 1;
@@ -297,11 +330,21 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;
     return 0;
 }
+}  // namespace sg2
+
+extern "C" {
+
+int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                     const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
+                     const Sg2Debug* debug, void* stream) {
+    return sg2::run_step(dims, weights, num_tensors, tensors, scalars, expert_counts, workspace, workspace_bytes, debug,
+                         (hipStream_t)stream);
+}
 
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;
-    if (sg2::make_layout(num_tensors, numels, sg2::effective_chunk_len(num_tensors, numels), &L, true)) return 0;
+    if (sg2::make_layout(num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L, true)) return 0;
     return L.bytes;
 }
 

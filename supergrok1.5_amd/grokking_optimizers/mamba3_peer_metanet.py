@@ -121,6 +121,28 @@ class Mamba3PEERMetaNet(nn.Module):
         return out
 
     @torch.no_grad()
+    def load_flat_weights(self, weights):
+        """Inverse of flat_weights: copies 33 tensors in `_ops` argument order into the module's parameters."""
+        W = list(weights)
+        assert len(W) == 33
+        self.input_proj.weight.copy_(W[0])
+        self.input_proj.bias.copy_(W[1])
+        for base, blk in ((2, self.mamba_fwd), (11, self.mamba_bwd)):
+            for k, prm in enumerate((blk.in_proj.weight, blk.dt_proj.weight, blk.dt_proj.bias, blk.B_proj.weight,
+                                     blk.C_proj.weight, blk.A_log, blk.D, blk.rope_freq, blk.out_proj.weight)):
+                prm.copy_(W[base + k].reshape(prm.shape))
+        for k, lin in enumerate((self.gru.W_z, self.gru.W_r, self.gru.W_h)):
+            lin.weight.copy_(W[20 + 2 * k])
+            lin.bias.copy_(W[21 + 2 * k])
+        for h in range(self.num_peer_heads):
+            self.peer_queries[h].weight.copy_(W[26][h])
+            self.product_keys_A[h].copy_(W[27][h])
+            self.product_keys_B[h].copy_(W[28][h])
+        for k, name in enumerate(("expert_W1", "expert_b1", "expert_W2", "expert_b2")):
+            prm = getattr(self, name)
+            prm.copy_(W[29 + k].reshape(prm.shape))
+
+    @torch.no_grad()
     def _recycle_dead_experts(self):
         """Experts with fewer than recycle_threshold of the activations are replaced by a noisy clone of
         an expert sampled in proportion to its count; a product key is re-drawn only when every expert

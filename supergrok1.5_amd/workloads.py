@@ -5,6 +5,7 @@ device path and a CPU checker can be handed identical bits.
 """
 import math
 
+import numpy as np
 import torch
 
 DEFAULT_DIMS = dict(d_model=8, d_state=16, d_inner=16, gru_hidden=4, num_heads=4, pk_dim=12,
@@ -107,3 +108,32 @@ def clip_per_tensor(grads, max_norm=1.0):
         n = g.norm()
         out.append(g * (max_norm / (n + 1e-12)) if n > max_norm else g)
     return out
+
+
+def per_tensor_scalars(P, step, lamb_eff=0.0):
+    """Per-tensor scalars of optimizer step `step` as the optimizer class derives them (alpha 0.98, beta1_i =
+    0.9 * 0.9^i, bias corrections), rounded to fp32 as they cross the extension boundary."""
+    out = []
+    for i in range(P):
+        b1 = float(np.float32(0.9 * 0.9 ** i))
+        out.append(dict(alpha=float(np.float32(0.98)), lamb_eff=float(np.float32(lamb_eff)), beta1=b1,
+                        bc1=float(np.float32(1.0 - b1 ** step)), bc2=float(np.float32(1.0 - 0.999 ** step))))
+    return out
+
+
+def shared_scalars(wd_eff=1.0, rescale=0.1):
+    f = lambda v: float(np.float32(v))
+    return dict(rescale=f(rescale), beta2=f(0.999), lr=f(1e-3), wd_eff=f(wd_eff), eps=f(1e-8))
+
+
+def module_weights(seed=0):
+    """The 33 meta-net weight tensors as Mamba3PEERMetaNet() initialises them (the reference's initialisation:
+    A_log = log(1..16), default nn.Linear weights, keys and experts N(0, 0.02)), in `_ops` argument order."""
+    from grokking_optimizers import Mamba3PEERMetaNet
+    state = torch.random.get_rng_state()
+    torch.manual_seed(seed)
+    try:
+        mn = Mamba3PEERMetaNet()
+    finally:
+        torch.random.set_rng_state(state)
+    return [w.clone() for w in mn.flat_weights()]

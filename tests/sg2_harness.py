@@ -121,15 +121,4 @@ class Sg2Case:
         return worst
 
 
-def per_tensor_scalars(P, step, lamb_eff=0.0):
-    out = []
-    for i in range(P):
-        b1 = float(np.float32(0.9 * 0.9 ** i))
-        out.append(dict(alpha=float(np.float32(0.98)), lamb_eff=float(np.float32(lamb_eff)), beta1=b1,
-                        bc1=float(np.float32(1.0 - b1 ** step)), bc2=float(np.float32(1.0 - 0.999 ** step))))
-    return out
-
-
-def shared_scalars(wd_eff=1.0, rescale=0.1):
-    f = lambda v: float(np.float32(v))
-    return dict(rescale=f(rescale), beta2=f(0.999), lr=f(1e-3), wd_eff=f(wd_eff), eps=f(1e-8))
+per_tensor_scalars, shared_scalars = wl.per_tensor_scalars, wl.shared_scalars

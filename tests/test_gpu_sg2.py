@@ -63,8 +63,8 @@ def test_multi_chunk_small_chunks():
 
 
 def test_windowed_summaries_accept_and_fall_back():
-    """Window 64 on chunks of 256: accepted with the N(0,0.1) weights; with barely contracting poles
-    (A_log = -12) every window fails its 2^-100 test and the whole chunk is accumulated instead."""
+    """Window 64 on chunks of 256: the first block is accepted with the N(0,0.1) weights; with barely contracting
+    poles (A_log = -12) no block passes the 2^-100 test and the walk covers the whole chunk."""
     from grokking_optimizers import _cabi
     shapes = [(3000,), (64, 65), (700,)]
     assert _cabi.lib().sg2_set_chunk_len(256) == 0 and _cabi.lib().sg2_set_scan_window(64) == 0
@@ -78,6 +78,36 @@ def test_windowed_summaries_accept_and_fall_back():
     assert _cabi.lib().sg2_set_scan_window(0) == 0
     case = Sg2Case(shapes, seed=23, random_state=True)
     print("window off", _run_steps(case, 1, chunk_len=256))
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_module_initialised_weights_over_several_chunks(seed):
+    """The optimizer's own initial meta-net (A_log = log(1..16), default Linear weights: poles with dt*|A|/2 > 1,
+    i.e. negative A_bar, and columns whose 256-step window has not contracted) on tensors of several chunks, with
+    gradients of order one so that dt varies along the sequence; chunk lengths 1024 (automatic) and 512."""
+    from grokking_optimizers import _cabi
+    shapes = [(9000,), (64, 130), (3000,), (700,)]
+    W = wl.module_weights(seed)
+    for cl in (None, 512):
+        assert _cabi.lib().sg2_set_chunk_len(cl or 0) == 0
+        case = Sg2Case(shapes, seed=30 + seed, random_state=True, weights=W)
+        w = _run_steps(case, 2, chunk_len=cl, sharp=True, lamb_eff=2.0, wd_eff=4.5, grad_std=0.5 if cl else 1e-3)
+        print("module weights seed", seed, "chunk", cl, "worst tolerance ratios", w)
+
+
+def test_adaptive_window_needs_several_blocks():
+    """A_log = log(1..16) with dt about 1.7: |A_bar| of the fast poles is close to 1 again, a 64-step block does not
+    contract to 2^-100 and the summary walk has to go back several blocks (device and checker must stop at the same
+    block: the results are bit-identical or the comparison of the contexts fails)."""
+    from grokking_optimizers import _cabi
+    shapes = [(3000,), (64, 65)]
+    W = wl.meta_weights(7)
+    for base in (2, 11):
+        W[base + 5].copy_(torch.log(torch.arange(1, 17, dtype=torch.float32))[None, :].expand(16, 16))
+        W[base + 2].fill_(1.5)
+    assert _cabi.lib().sg2_set_chunk_len(512) == 0 and _cabi.lib().sg2_set_scan_window(64) == 0
+    case = Sg2Case(shapes, seed=41, random_state=True, weights=W)
+    print("several blocks", _run_steps(case, 2, chunk_len=512, sharp=True, lamb_eff=2.0))
 
 
 def test_shared14_one_step_default_chunk():

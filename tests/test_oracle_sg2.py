@@ -124,30 +124,37 @@ def test_chunked_scan_matches_sequential(n, chunk):
 
 
 def test_windowed_summaries_match_full_chunks():
-    """Chunk summaries taken over the last 64/128 steps only (accepted when the window's 2x2 part is below
-    2^-100) give the sequential result to rounding; weights that barely contract make every window fail
-    its test, and the fallback is then bit-identical to plain chunking."""
+    """Chunk summaries built backwards in blocks of 64/128 steps, stopping once the 2x2 part is below 2^-100, give
+    the sequential result to rounding -- for strongly contracting weights (the first block suffices), for poles that
+    need several blocks (the reference's initialisation A = -1..-16 with a large dt: |A_bar| close to 1 again), and
+    for weights that barely contract (the walk reaches the chunk start: the exact summary, re-associated)."""
     n = 1500
     W = weights_np()
     st = random_state_np(n, 11)
     g, s = _grad(n, 12), np.abs(_grad(n, 13))
     sc = default_scalars()
-    for prec, rel in ((64, 1e-9), (32, 2e-5)):
-        seq, dseq = _run_oracle(W, st, g, s, sc, prec, 0)
-        for win in (64, 128):
-            a, da = _run_oracle(W, st, g, s, sc, prec, 256, window=win)
-            ok, ratio = rel_close(dseq["ctx"], da["ctx"], rel=rel, floor=1e-7 if prec == 32 else 1e-12)
-            assert ok, (prec, win, ratio)
-            for k in ("mamba_fwd", "mamba_bwd"):
-                ok, ratio = rel_close(seq[k], a[k], rel=rel * 10, floor=1e-7)
-                assert ok, (prec, win, k, ratio)
-    # strongly contracting weights: the window is really used (result differs in the last bits from plain chunking
-    # at most; here we only require that it stays within rounding), weakly contracting: identical to plain chunking
+    Winit = [w.copy() for w in W]
+    for base in (2, 11):
+        Winit[base + 5][:] = np.log(np.arange(1, 17, dtype=np.float32))[None, :]     # A_log = log(1..16)
+        Winit[base + 2][:] = 1.5                                                       # dt about softplus(1.5) = 1.7
     Wslow = [w.copy() for w in W]
     for base in (2, 11):
-        Wslow[base + 5][:] = -12.0            # A_log: A = -6e-6, A_bar ~ 1 - 4e-6: no contraction within a window
+        Wslow[base + 5][:] = -12.0            # A = -6e-6, A_bar ~ 1 - 4e-6: no contraction within a chunk
+    for Wx in (W, Winit, Wslow):
+        for prec, rel in ((64, 1e-9), (32, 2e-5)):
+            seq, dseq = _run_oracle(Wx, st, g, s, sc, prec, 0)
+            for win in (64, 128):
+                a, da = _run_oracle(Wx, st, g, s, sc, prec, 256, window=win)
+                ok, ratio = rel_close(dseq["ctx"], da["ctx"], rel=rel, floor=1e-7 if prec == 32 else 1e-12)
+                assert ok, (prec, win, ratio)
+                for k in ("mamba_fwd", "mamba_bwd"):
+                    # entries of a barely contracting state are sums of 1500 inputs with cancellation: the floor
+                    # follows the size of the state (fp32 sequential is itself 1e-4 of it away from float64)
+                    ok, ratio = rel_close(seq[k], a[k], rel=rel * 10, floor=max(1e-7, 1e-5 * float(np.abs(seq[k]).max())))
+                    assert ok, (prec, win, k, ratio)
+    # a window as long as the chunk, or none, is plain chunking bit for bit
     plain, dplain = _run_oracle(Wslow, st, g, s, sc, 32, 256)
-    win, dwin = _run_oracle(Wslow, st, g, s, sc, 32, 256, window=64)
+    win, dwin = _run_oracle(Wslow, st, g, s, sc, 32, 256, window=256)
     assert np.array_equal(dplain["ctx"], dwin["ctx"]) and np.array_equal(plain["mamba_fwd"], win["mamba_fwd"])
 
 
