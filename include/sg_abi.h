@@ -90,11 +90,11 @@ int sg2_get_chunk_len(void);
 int sg2_chunk_len_for(int num_tensors, const int64_t* numels);
 
 /* Summary window of the scan (timesteps, a multiple of 64; 0 disables, a
- * negative value restores the default 256).  The recurrence contracts, so the
- * 2x2 part of a chunk summary taken over only its last `window` steps is
- * normally far below fp32 resolution; when every entry is below 2^-100 the
- * chunk summary is (0, b_window), otherwise the whole chunk is accumulated.
- * Takes effect when window < chunk_len. */
+ * negative value restores the default 256).  The recurrence contracts, so a
+ * chunk summary is built backwards in blocks of `window` steps and the walk
+ * stops as soon as every entry of the 2x2 part of the running summary is below
+ * 2^-100 (the chunk summary is then (0, b)); a chunk that never contracts is
+ * covered completely.  Takes effect when window < chunk_len. */
 int sg2_set_scan_window(int window);
 int sg2_get_scan_window(void);
 
@@ -110,6 +110,23 @@ size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* n
 int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors,
                      const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
                      void* workspace, size_t workspace_bytes, const Sg2Debug* debug, void* stream);
+
+/* sg2_batched_step without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The scratch lives in a static device array of SG2_STATIC_SCRATCH_BYTES inside
+ * the library (one copy per GPU the library runs on, held until the process
+ * ends); the call allocates and frees nothing, on the device or through any
+ * library.  Calls whose tensors need more scratch than that (about 700 000
+ * elements in total; sg2_workspace_bytes tells) are rejected with an error.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one
+ * GPU (different streams or threads) race; calls on one stream are ordered.
+ * Same kernels and results as sg2_batched_step. */
+#define SG2_STATIC_SCRATCH_BYTES (64u << 20)
+size_t sg2_static_scratch_bytes(void);
+int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int num_tensors,
+                            const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
+                            const Sg2Debug* debug, void* stream);
 
 /* Per-stage device timing of sg2_batched_step with HIP events recorded on the
  * step's own stream (no counterpart in the reference, which has no profiling

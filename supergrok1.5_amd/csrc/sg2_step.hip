@@ -8,6 +8,7 @@
 // Stands behind supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877 of
 // the reference) in place of launch_mamba3_peer_batched_step
 // (csrc/supergrok2_mamba_peer_kernels.cu:1754-2117).
+#include <mutex>
 #include <vector>
 
 #include "sg2_internal.hpp"
@@ -330,6 +331,28 @@ int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, con
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;
     return 0;
 }
+
+// Scratch of sg2_batched_step_static: one array per GPU the library runs on, held until the process ends.  The
+// array's name is only a handle in host code; its device address is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[SG2_STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+std::mutex g_scratch_mutex;
+
+int static_scratch_address(void** out) {
+    int dev = -1;
+    SG_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return sg::fail("device index %d outside 0..%d", dev, MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        SG_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return sg::fail("hipGetSymbolAddress returned NULL for the static scratch buffer");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
 }  // namespace sg2
 
 extern "C" {
@@ -339,6 +362,26 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
                      const Sg2Debug* debug, void* stream) {
     return sg2::run_step(dims, weights, num_tensors, tensors, scalars, expert_counts, workspace, workspace_bytes, debug,
                          (hipStream_t)stream);
+}
+
+size_t sg2_static_scratch_bytes(void) { return SG2_STATIC_SCRATCH_BYTES; }
+
+int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                            const Sg2Scalars* scalars, int32_t* expert_counts, const Sg2Debug* debug, void* stream) {
+    using namespace sg2;
+    if (check_dims(dims)) return 1;
+    if (num_tensors < 0 || (num_tensors > 0 && !tensors)) return sg::fail("NULL argument");
+    Layout L;
+    const Numels numels = {nullptr, tensors};
+    if (make_layout(num_tensors, numels, effective_chunk_len(num_tensors, numels), &L)) return 1;
+    if (L.bytes > SG2_STATIC_SCRATCH_BYTES)
+        return sg::fail("sg2_batched_step_static: these tensors need %zu bytes of scratch, the library's static buffer holds %zu "
+                        "(about 700 000 elements per call); use sg2_batched_step with a caller-provided workspace",
+                        L.bytes, (size_t)SG2_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    if (static_scratch_address(&ws)) return 1;
+    return run_step(dims, weights, num_tensors, tensors, scalars, expert_counts, ws, SG2_STATIC_SCRATCH_BYTES, debug,
+                    (hipStream_t)stream);
 }
 
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {

@@ -69,6 +69,10 @@ def lib():
         L.sg2_batched_step.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
                                        C.POINTER(Sg2Scalars), C.c_void_p, C.c_void_p, C.c_size_t,
                                        C.POINTER(Sg2Debug), C.c_void_p]
+        L.sg2_static_scratch_bytes.restype = C.c_size_t
+        L.sg2_batched_step_static.restype = C.c_int
+        L.sg2_batched_step_static.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
+                                              C.POINTER(Sg2Scalars), C.c_void_p, C.POINTER(Sg2Debug), C.c_void_p]
         L.sg2_bilevel_workspace_bytes.restype = C.c_size_t
         L.sg2_bilevel_workspace_bytes.argtypes = [C.POINTER(SgDims), C.c_int, C.POINTER(C.c_int64)]
         L.sg2_bilevel_forward.restype = C.c_int
