@@ -267,6 +267,41 @@ def bench_other(args, dev):
     return out
 
 
+def bench_probe(dev):
+    """Issue rate of plain fp32 vector instructions (sg_probe_valu): wave64 instructions per nanosecond and SIMD for
+    fma / mul / add / DPP-add streams with every SIMD of the chip busy, by resident waves per SIMD; and the shader
+    clock the part holds meanwhile (ticks of the in-kernel clock per nanosecond of the launch)."""
+    import ctypes as C
+    import torch
+    from grokking_optimizers import _cabi
+    L = _cabi.lib()
+    L.sg_probe_workspace_bytes.restype = C.c_size_t
+    L.sg_probe_valu.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_float), C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                                C.c_void_p, C.c_size_t, C.c_void_p]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ws = torch.empty(L.sg_probe_workspace_bytes(cus, 8), dtype=torch.uint8, device=dev)
+    rows, best = [], 0.0
+    for ncu in (cus,):
+        for op, name in enumerate(("fma", "mul", "add", "add_dpp")):
+            for w in (1, 2, 3, 4, 8):
+                ms, ticks, instr = C.c_float(), C.c_double(), C.c_double()
+                if L.sg_probe_valu(op, ncu, w, 2000, C.byref(ms), C.byref(ticks), C.byref(instr), ws.data_ptr(), ws.numel(),
+                                   torch.cuda.current_stream().cuda_stream) != 0:
+                    raise RuntimeError(_cabi.last_error())
+                rate = instr.value * w / (ms.value * 1e6)            # per SIMD: w waves share one
+                rows.append({"op": name, "cus": ncu, "waves_per_simd": w, "ms": round(ms.value, 4),
+                             "instr_per_ns_per_simd": round(rate, 4),
+                             "clock_ticks_per_instr_per_simd": round(ticks.value / instr.value / w, 3),
+                             "clock_ticks_per_ns": round(ticks.value / (ms.value * 1e6), 3)})
+                if ncu == cus:
+                    best = max(best, rate)
+    return {"metric": "secondary: valu-probe", "value": best, "unit": "wave64 instructions/ns/SIMD (whole chip, best case)",
+            "n_gpus": 1, "steps": 1, "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "plain fp32 VALU instruction streams, 8 independent accumulators per lane, %d CUs" % cus},
+            "rows": rows}
+
+
 def class_step_ms(shapes, grad_sets, dev, steps, warmup):
     """Wall time of SuperGrok2.step() itself (per-tensor clip on the device, scalar schedules, the 51-argument
     `_ops` call), same tensors and gradients, the module's own initial meta-weights, recycling off."""
@@ -299,7 +334,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--sharpness", action="store_true", help="v2 workloads: non-zero sharpness cache (as after a SAM probe)")
-    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11", "bilevel"],
+    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11", "bilevel", "valu-probe"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
@@ -324,6 +359,9 @@ def main():
     from workloads import per_tensor_scalars, shared_scalars
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
+    if args.workload == "valu-probe":
+        print(json.dumps(bench_probe(dev)))
+        return
     if args.workload not in ("scale50", "shared14"):
         print(json.dumps(bench_other(args, dev)))
         return

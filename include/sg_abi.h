@@ -141,6 +141,18 @@ int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int n
 int sg2_profile_enable(int on);
 int sg2_profile_read(float* ms, int* calls);
 
+/* Issue-rate probe of the fp32 vector ALU (measurement aid, no counterpart in
+ * the reference): `iters` x 128 independent wave64 instructions of one kind
+ * per wave (op 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_add_f32 with a DPP
+ * operand; plain, not packed) on num_cus x waves_per_simd workgroups of four
+ * waves, i.e. waves_per_simd waves on every SIMD of num_cus compute units
+ * when the dispatcher spreads them evenly.  Synchronises the stream.  Returns
+ * the elapsed milliseconds of the launch, the shader-clock ticks a wave took
+ * on average and the instructions each wave issued. */
+size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd);
+int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
+                  double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ======================= Grokfast / SuperGrok v1.5 ======================== */
 
 /* Scratch for the elementwise entry points below (tables + reduction

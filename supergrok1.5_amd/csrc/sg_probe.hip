@@ -1,0 +1,90 @@
+// Issue-rate probe of the fp32 vector ALU: what one MI355X sustains in wave64 instructions per nanosecond and
+// SIMD for plain (non-packed) fma / mul / add / DPP-add streams, as a function of the waves resident per SIMD and
+// of the share of the chip that is busy.  It is the yardstick the arithmetic-bound kernels of this library
+// (the v2 scan and per-element kernels) are priced against; the reference has nothing comparable.
+#include "sg_common.hpp"
+
+namespace {
+
+constexpr int PROBE_ILP = 8;       // independent accumulators per lane: no instruction waits for its predecessor
+constexpr int PROBE_UNROLL = 16;
+
+template <int OP>
+__global__ __launch_bounds__(256) void k_probe(float* sink, long long* ticks, int iters, float a, float b) {
+    float acc[PROBE_ILP];
+#pragma unroll
+    for (int k = 0; k < PROBE_ILP; k++) acc[k] = threadIdx.x * 1e-3f + k + 1.0f;
+    const long long t0 = clock64();
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int r = 0; r < PROBE_UNROLL; r++) {
+#pragma unroll
+            for (int k = 0; k < PROBE_ILP; k++) {
+                if (OP == 0) acc[k] = __builtin_fmaf(acc[k], a, b);
+                else if (OP == 1) acc[k] = acc[k] * a;
+                else if (OP == 2) acc[k] = acc[k] + a;
+                else acc[k] = acc[k] + sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(acc[k]), 0xB1, 0xF, 0xF, true));
+            }
+        }
+    }
+    const long long t1 = clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PROBE_ILP; k++) s += acc[k];
+    if (s == 12345.678f) sink[0] = s;       // keeps the arithmetic alive
+    if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd) {
+    if (num_cus <= 0 || waves_per_simd <= 0) return 0;
+    return 256 + sizeof(long long) * (size_t)num_cus * (size_t)waves_per_simd;
+}
+
+int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
+                  double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream) {
+    hipStream_t st = (hipStream_t)stream;
+    if (op < 0 || op > 3) return sg::fail("op must be 0 (fma), 1 (mul), 2 (add) or 3 (add with a DPP operand)");
+    if (num_cus <= 0 || num_cus > 1024 || waves_per_simd <= 0 || waves_per_simd > 8 || iters <= 0 || iters > 100000)
+        return sg::fail("probe size out of range");
+    if (!ms_out || !ticks_per_wave_out || !instr_per_wave_out) return sg::fail("NULL argument");
+    const int blocks = num_cus * waves_per_simd;         // 256 threads = one wave on each of the four SIMDs of a CU
+    if (!workspace || workspace_bytes < sg_probe_workspace_bytes(num_cus, waves_per_simd)) return sg::fail("workspace too small");
+    float* sink = static_cast<float*>(workspace);
+    long long* ticks = reinterpret_cast<long long*>(static_cast<unsigned char*>(workspace) + 256);
+    hipEvent_t e0, e1;
+    SG_HIP_CHECK(hipEventCreate(&e0));
+    SG_HIP_CHECK(hipEventCreate(&e1));
+    auto launch = [&](int n) {
+        switch (op) {
+            case 0: hipLaunchKernelGGL(k_probe<0>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 1: hipLaunchKernelGGL(k_probe<1>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 2: hipLaunchKernelGGL(k_probe<2>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            default: hipLaunchKernelGGL(k_probe<3>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+        }
+    };
+    launch(8);                                            // warm-up: code object load, clocks
+    SG_HIP_CHECK(hipEventRecord(e0, st));
+    launch(iters);
+    SG_HIP_CHECK(hipEventRecord(e1, st));
+    SG_LAUNCH_CHECK("k_probe");
+    SG_HIP_CHECK(hipEventSynchronize(e1));
+    SG_HIP_CHECK(hipEventElapsedTime(ms_out, e0, e1));
+    double sum = 0.0;
+    for (int b0 = 0; b0 < blocks; b0 += 256) {
+        long long h[256];
+        const int n = blocks - b0 < 256 ? blocks - b0 : 256;
+        SG_HIP_CHECK(hipMemcpy(h, ticks + b0, sizeof(long long) * n, hipMemcpyDeviceToHost));
+        for (int k = 0; k < n; k++) sum += (double)h[k];
+    }
+    *ticks_per_wave_out = sum / blocks;
+    *instr_per_wave_out = (double)iters * PROBE_UNROLL * PROBE_ILP;
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return 0;
+}
+
+}  // extern "C"
