@@ -278,6 +278,40 @@ int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, vo
  * a fixed order, so the result is reproducible run to run. */
 #define SG2_SCAN_GRAD_FLOATS 3160
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
+
+/* The same pair with the quantities the reference's own bilevel entry points
+ * exchange with their Python caller (supergrok2_bilevel_fwd_save[_batched] /
+ * supergrok2_bilevel_backward[_batched], csrc/ops.h:232-371; caller
+ * grokking_optimizers/supergrok2.py:646-1040).
+ * sg2_bilevel_forward_ex: ctx_out may be NULL; `extra` (may be NULL, and any of
+ * its members) receives
+ *   scan_out_fwd / scan_out_bwd [sum numel][d_inner]  the gated scan output
+ *            y*silu(z) + D*x of every step, before out_proj, in scan order
+ *            (forward: sorted position t; backward: step u = N-1-t), tensors
+ *            packed in call order -- the reference's fwd/bwd_scan_out_packed;
+ *   x_sorted [sum numel][d_model]     W_in [g, s] + b_in in sorted order;
+ *   perm     [sum numel]              sorted position -> element index.
+ * sg2_bilevel_backward_ex: exactly one of d_ctx (as above) and the pair
+ * d_scan_out_fwd / d_scan_out_bwd (scan_out's layout; out_proj then stays with
+ * the caller and its gradient is returned as zeros) is given.  dx_out (optional, with row_dx) receives
+ * [2][sum numel][d_model]: each direction's gradient with respect to x_sorted,
+ * in sorted order; row_dx is [2][80][d_model], the derivative of the 80
+ * pre-activation rows of each direction (x-branch, z, dt, B, C: 16 each) with
+ * respect to x, i.e. in_proj[:16], in_proj[16:], dt_W in_proj[:16],
+ * B_proj in_proj[:16], C_proj in_proj[:16].
+ * The backward call uses the chunk length and window of the forward call on the
+ * same workspace, whatever the settings are by then. */
+typedef struct Sg2BilevelExtra {
+    float* scan_out_fwd;
+    float* scan_out_bwd;
+    float* x_sorted;
+    int32_t* perm;
+} Sg2BilevelExtra;
+int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                           float* ctx_out, const Sg2BilevelExtra* extra, void* workspace, size_t workspace_bytes, void* stream);
+int sg2_bilevel_backward_ex(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                            const float* d_ctx, const float* d_scan_out_fwd, const float* d_scan_out_bwd, const float* row_dx,
+                            float* dx_out, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
 int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
                         float* ctx_out, void* workspace, size_t workspace_bytes, void* stream);
 int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,

@@ -1,4 +1,4 @@
-"""Builds the torch extension grokking_optimizers/_ops*.so from ops_shim.cpp.
+"""Builds the torch extension grokking_optimizers/_ops*.so from ops_shim.cpp and ops_bilevel.cpp.
 
 Plain g++ against the installed torch headers (no hipify step, no JIT cache):
 the shim contains no device code, it only forwards to libsg_hip.so, which it
@@ -25,7 +25,7 @@ def main():
            "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
            "-I" + os.path.join(tdir, "include"), "-I" + os.path.join(tdir, "include", "torch", "csrc", "api", "include"),
            "-I" + sysconfig.get_paths()["include"], "-I" + os.path.join(rocm, "include"),
-           os.path.join(HERE, "ops_shim.cpp"), "-o", out,
+           os.path.join(HERE, "ops_shim.cpp"), os.path.join(HERE, "ops_bilevel.cpp"), "-o", out,
            "-L" + tdir + "/lib", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip", "-ltorch_hip",
            "-L" + os.path.join(PKG, "lib"), "-lsg_hip",
            "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath," + tdir + "/lib", "-Wno-unused-variable"]

@@ -628,6 +628,27 @@ std::vector<torch::Tensor> supergrok2_clip_grads(std::vector<torch::Tensor>& gra
     return out;
 }
 
+// ---- the reference's bilevel entry points (ops_bilevel.cpp)
+void supergrok2_bilevel_fwd_save_batched(
+    std::vector<torch::Tensor>, std::vector<torch::Tensor>, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int, int, int, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int);
+void supergrok2_bilevel_backward_batched(
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, int, int, int, int, int);
+void supergrok2_bilevel_fwd_save(
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int, int, int, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, int);
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "Grokking optimizers: fused steps on MI355X (hand-written HIP behind the reference's _ops surface)";
     m.def("supergrok15_fused_step", &supergrok15_fused_step, "SuperGrok1.5: fused clip + mu + meta-net + gating + adam + progressive wd",
@@ -705,4 +726,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("beta2"), py::arg("lr"), py::arg("wd_eff"), py::arg("eps"), py::arg("d_model"), py::arg("d_state"),
           py::arg("d_inner"), py::arg("gru_hidden"), py::arg("num_heads"), py::arg("pk_dim"), py::arg("expert_hidden"),
           py::arg("num_experts"), py::arg("expert_counts"));
+    // bilevel meta-training: the reference's names and argument lists (csrc/ops.cpp:1072-1085 there)
+    m.def("supergrok2_bilevel_fwd_save", &supergrok2_bilevel_fwd_save, "SuperGrok2 bilevel: forward scan with state saving for backward");
+    m.def("supergrok2_bilevel_fwd_save_batched", &supergrok2_bilevel_fwd_save_batched,
+          "SuperGrok2 bilevel: batched forward scan with state saving");
+    m.def("supergrok2_bilevel_backward_batched", &supergrok2_bilevel_backward_batched, "SuperGrok2 bilevel: batched backward through scan");
+    m.def("supergrok2_bilevel_backward", [](py::args, py::kwargs) {
+        throw std::runtime_error(
+            "supergrok2_bilevel_backward (one tensor, whole meta-net) is not provided: its argument list carries the saved gate values of "
+            "the GRU instead of the GRU biases, and the HIP per-element kernel recomputes the forward pass from the weights. Use "
+            "supergrok2_bilevel_fwd_save_batched / supergrok2_bilevel_backward_batched (which the reference's caller prefers whenever they "
+            "exist), or SuperGrok2.bilevel_step of this package.");
+    }, "SuperGrok2 bilevel: full backward through meta-net (raises: see the message)");
 }

@@ -50,6 +50,18 @@ constexpr int LDS_H_FLOATS = BT * SCAN_THREADS * 2;               // state after
 constexpr int LDS_MISC_FLOATS = BT * DM + BT * 2 + DI;            // d ctx tile, (g, s) of the tile, per-column frequency bound
 static_assert(SCAN_THREADS == 4 * BT && ROWS % 4 == 0 && (LDS_ROWS_FLOATS + LDS_H_FLOATS) % 4 == 0, "projection roles, float4 alignment");
 constexpr int BILEVEL_LDS_BYTES = 4 * (LDS_ROWS_FLOATS + LDS_H_FLOATS + LDS_MISC_FLOATS);
+// with the gradient of the input projection as an output: per-step sums over the columns of the B / C shares of each
+// wave ([2 waves][BT][d B even, d B odd, d C even, d C odd][8 pairs]) and d(pre-activation row)/d x ([80][DM])
+constexpr int LDS_DX_FLOATS = 2 * BT * 4 * HP + SG2_COMP_GROUPS * 16 * DM;
+constexpr int BILEVEL_DX_LDS_BYTES = BILEVEL_LDS_BYTES + 4 * LDS_DX_FLOATS;
+
+// What comes in and goes out besides the weight gradients.  Exactly one of d_ctx / d_scan is given.
+struct AdjIO {
+    const float* d_ctx;     // [2][total][DM]  gradient w.r.t. the two contexts, element order
+    const float* d_scan[2]; // per direction [total][DI]  gradient w.r.t. the gated scan output (before out_proj), scan order
+    const float* rx;        // [2][SG2_COMP_GROUPS*16][DM]  d(pre-activation row)/d x of each direction (only with dx)
+    float* dx;              // [2][total][DM]  out, optional: each direction's gradient w.r.t. the input projection x, sorted order
+};
 
 // value of the lane whose index differs in one bit, by DPP where the pattern stays inside a row of 16 lanes
 template <int CTRL>
@@ -77,8 +89,9 @@ struct ChunkRef {
     const int32_t* sval;
     const float* ssrt;
     const float* dctx;
+    const float* dscan;      // this tensor's rows of d_scan for this direction, indexed by scan step
 };
-__device__ __forceinline__ ChunkRef chunk_ref(const Plan& pl, int chunk, int dir, const float* d_ctx) {
+__device__ __forceinline__ ChunkRef chunk_ref(const Plan& pl, int chunk, int dir, const AdjIO& io) {
     ChunkRef c;
     c.ti = sg::upper_seg(sg::as_const(pl.chunk_prefix), pl.P, chunk);
     const TensorDev& T = pl.tensors[c.ti];
@@ -90,7 +103,8 @@ __device__ __forceinline__ ChunkRef chunk_ref(const Plan& pl, int chunk, int dir
     c.skey = pl.keys[0] + c.off;
     c.sval = pl.vals[0] + c.off;
     c.ssrt = pl.ssorted + c.off;
-    c.dctx = d_ctx + ((size_t)dir * pl.total + c.off) * DM;
+    c.dctx = io.d_ctx ? io.d_ctx + ((size_t)dir * pl.total + c.off) * DM : nullptr;
+    c.dscan = io.d_scan[dir] ? io.d_scan[dir] + (size_t)c.off * DI : nullptr;
     return c;
 }
 // (g, s) and the element index of scan step u of a chunk's tensor; zeros past the end
@@ -130,13 +144,13 @@ __device__ __forceinline__ void adj_apply(float ae, float ao, float sn, float cs
 
 // ---- launch 1: affine map of the adjoint state across every chunk
 constexpr int SUMM_ROWS = 4;                     // LDS arrays of the summary kernel: dt, C, gate, d y
-__global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const float* __restrict__ d_ctx) {
+__global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, AdjIO io) {
     __shared__ float rows[SUMM_ROWS * ROWS * BST];
     __shared__ __attribute__((aligned(16))) float s_dctx[SCAN_TT * DM];
     __shared__ float s_fmax[DI];
     auto arr = [&](int a) { return rows + a * ROWS * BST; };
     const int chunk = blockIdx.x, dir = blockIdx.y;
-    const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
+    const ChunkRef c = chunk_ref(pl, chunk, dir, io);
     const int b = dir ? W_B_INPROJ : W_F_INPROJ;
     const float* __restrict__ Alog = pl.W.w[b + 5];
     const float* __restrict__ rope = pl.W.w[b + 7];
@@ -167,8 +181,10 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
             float g, s;
             int orig;
             load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
-            const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
-            reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
+            if (c.dctx != nullptr) {
+                const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[half] : make_float4(0.f, 0.f, 0.f, 0.f);
+                reinterpret_cast<float4*>(s_dctx + tu * DM)[half] = dv;
+            }
             for (int q = 0; q < ROWS / 2; q++) {
                 const int r = half * (ROWS / 2) + q;
                 const float dtv = valid ? sg_softplus(sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s)) : 0.0f;
@@ -183,8 +199,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, const flo
         for (int q = 0; q < ROWS / 2; q++) {
             const int r = half * (ROWS / 2) + q;
             float dout = 0.0f;
+            if (c.dscan != nullptr) {
+                if (tu < cnt) dout = c.dscan[(size_t)(u0 + tu) * DI + r];
+            } else {
 #pragma unroll
-            for (int d = 0; d < DM; d++) dout = sg_fma(Wout[d * DI + r], s_dctx[tu * DM + d], dout);
+                for (int d = 0; d < DM; d++) dout = sg_fma(Wout[d * DI + r], s_dctx[tu * DM + d], dout);
+            }
             arr(3)[r * BST + tu] = (tu < cnt) ? dout * arr(2)[r * BST + tu] : 0.0f;
         }
         __syncthreads();
@@ -229,13 +249,16 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_prefix(Plan pl) {
 }
 
 // ---- launch 3: the gradients, chunk by chunk
-__global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, const float* __restrict__ d_ctx) {
+template <bool DX>
+__global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, AdjIO io) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* rows = lds;
     float* sH = lds + LDS_ROWS_FLOATS;
     float* s_dctx = sH + LDS_H_FLOATS;
     float* s_gs = s_dctx + BT * DM;
     float* s_fmax = s_gs + BT * 2;
+    float* s_bc = s_fmax + DI;                       // DX only
+    float* s_rx = s_bc + 2 * BT * 4 * HP;            // DX only
     auto arr = [&](int a) { return rows + a * ROWS * BBST; };
 
     const int dir = blockIdx.y;
@@ -252,6 +275,9 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
     const float freq = rope[j * HP + p];
 
+    if (DX) {
+        for (int i = threadIdx.x; i < SG2_COMP_GROUPS * 16 * DM; i += SCAN_THREADS) s_rx[i] = io.rx[(size_t)dir * SG2_COMP_GROUPS * 16 * DM + i];
+    }
     fill_fmax(s_fmax, rope);
     // this lane's rows of the composed coefficients, of out_proj^T and of D, kept in registers: the barriers inside
     // the tile loop would otherwise make every tile fetch them again
@@ -274,7 +300,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
     for (int q = 0; q < 12; q++) acc_bc[q] = 0.0f;
 
   for (int chunk = blockIdx.x; chunk < pl.chunks; chunk += gridDim.x) {
-    const ChunkRef c = chunk_ref(pl, chunk, dir, d_ctx);
+    const ChunkRef c = chunk_ref(pl, chunk, dir, io);
     const int ti = c.ti, off = c.off;
     float le, lo;                                    // adjoint of the state after the current step
     {
@@ -293,7 +319,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             int orig;
             load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
             if (part == 0) { s_gs[2 * tu] = g; s_gs[2 * tu + 1] = s; }
-            if (part < DM / 4) {
+            if (part < DM / 4 && c.dctx != nullptr) {
                 const float4 dv = valid ? reinterpret_cast<const float4*>(c.dctx + (size_t)orig * DM)[part] : make_float4(0.f, 0.f, 0.f, 0.f);
                 reinterpret_cast<float4*>(s_dctx + tu * DM)[part] = dv;
             }
@@ -361,12 +387,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
         __syncthreads();
 
         // ---- 3: per step and column: out, d out, d y, d z, D-skip part of d x-branch
+        float4 dscan4 = make_float4(0.f, 0.f, 0.f, 0.f);          // d out of this lane's four rows when it comes in directly
+        if (c.dscan != nullptr && tu < cnt) dscan4 = reinterpret_cast<const float4*>(c.dscan + (size_t)(u0 + tu) * DI)[part];
 #pragma unroll
         for (int q = 0; q < ROWS / 4; q++) {
             const int r = part * (ROWS / 4) + q;
             float dout = 0.0f;
+            if (c.dscan != nullptr) {
+                dout = q == 0 ? dscan4.x : q == 1 ? dscan4.y : q == 2 ? dscan4.z : dscan4.w;
+            } else {
 #pragma unroll
-            for (int d = 0; d < DM; d++) dout = sg_fma(wo[q][d], s_dctx[tu * DM + d], dout);
+                for (int d = 0; d < DM; d++) dout = sg_fma(wo[q][d], s_dctx[tu * DM + d], dout);
+            }
             const float y = arr(A_Y)[r * BBST + tu], gate = arr(A_GATE)[r * BBST + tu], xb = arr(A_XB)[r * BBST + tu];
             const bool valid = tu < cnt;
             arr(A_DY)[r * BBST + tu] = valid ? dout * gate : 0.0f;
@@ -402,6 +434,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                 rot_sincos(tiny, dtv[q] * freq, &snv[q], &csv[q]);
             }
             float ddtv[RB], dxbv[RB];
+            float shBe[DX ? RB : 1], shBo[DX ? RB : 1], shCe[DX ? RB : 1], shCo[DX ? RB : 1];     // this column's share of d B / d C per step
 #pragma unroll
             for (int q = RB - 1; q >= 0; q--) {
                 const bool live = k0 + q < cnt;                  // steps past the end of the chunk leave lambda alone
@@ -417,6 +450,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                     const float te = dy * he, to = dy * ho;
                     acc_bc[6] = sg_fma(te, gk, acc_bc[6]); acc_bc[7] = sg_fma(te, sk, acc_bc[7]); acc_bc[8] += te;
                     acc_bc[9] = sg_fma(to, gk, acc_bc[9]); acc_bc[10] = sg_fma(to, sk, acc_bc[10]); acc_bc[11] += to;
+                    if (DX) { shCe[q] = te; shCo[q] = to; }
                 }
                 // h' = A_bar * rot(h) + dt * xb * B
                 const float re = sg_fma(pe, cs, -(po * sn)), ro = sg_fma(po, cs, pe * sn);
@@ -437,6 +471,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
                     const float te = le * ux, to = lo * ux;
                     acc_bc[0] = sg_fma(te, gk, acc_bc[0]); acc_bc[1] = sg_fma(te, sk, acc_bc[1]); acc_bc[2] += te;
                     acc_bc[3] = sg_fma(to, gk, acc_bc[3]); acc_bc[4] = sg_fma(to, sk, acc_bc[4]); acc_bc[5] += to;
+                    if (DX) { shBe[q] = te; shBo[q] = to; }
                 }
                 ddtv[q] = ddt;
                 dxbv[q] = qb * dt;
@@ -447,6 +482,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
             }
 #pragma unroll
             for (int q = 0; q < RB; q++) { ddtv[q] = pair_sum(ddtv[q]); dxbv[q] = pair_sum(dxbv[q]); }
+            if (DX) {
+                // d B[2p], d B[2p+1], d C[2p], d C[2p+1] of every step: columns of the wave added here, the two waves in step 6
+#pragma unroll
+                for (int q = 0; q < RB; q++) {
+                    const float s0 = xor_sum_columns(shBe[q]), s1 = xor_sum_columns(shBo[q]);
+                    const float s2 = xor_sum_columns(shCe[q]), s3 = xor_sum_columns(shCo[q]);
+                    if ((tid & 63) < HP) {
+                        float* dst = s_bc + ((w * BT + k0 + q) * 4) * HP + p;
+                        dst[0] = s0; dst[HP] = s1; dst[2 * HP] = s2; dst[3 * HP] = s3;
+                    }
+                }
+            }
             if (p == 0) {
 #pragma unroll
                 for (int q = 0; q < RB; q++) {
@@ -477,10 +524,38 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_bilevel_backward(Plan pl, cons
 #pragma unroll 8
             for (int k = 0; k < BT; k++) acc_D = sg_fma(arr(A_DGATE)[r * BBST + k], arr(A_XB)[r * BBST + k], acc_D);
         }
-        {
+        if (c.dscan == nullptr) {
             const int d = tid >> 4, r = tid & 15;       // out_proj[d][r]
 #pragma unroll 8
             for (int k = 0; k < BT; k++) acc_wout = sg_fma(s_dctx[k * DM + d], arr(A_GATE)[r * BBST + k], acc_wout);
+        }
+        // ---- 6 (optional): gradient w.r.t. the input projection x of every step of the tile,
+        //      d x = sum over the 80 pre-activation rows of (d row) * d row/d x; lane (tu, part) forms entries 2*part, 2*part+1
+        if (DX) {
+            if (tu < cnt) {
+                float a0 = 0.0f, a1 = 0.0f;
+                const float* rx = s_rx + 2 * part;
+#pragma unroll 4
+                for (int r = 0; r < 16; r++) {
+                    const float dxb = arr(A_DXB)[r * BBST + tu], dz = arr(A_DZ)[r * BBST + tu], ddt = arr(A_DDT)[r * BBST + tu];
+                    const int pr = r >> 1, odd = r & 1;
+                    const float dB = s_bc[((0 * BT + tu) * 4 + odd) * HP + pr] + s_bc[((1 * BT + tu) * 4 + odd) * HP + pr];
+                    const float dC = s_bc[((0 * BT + tu) * 4 + 2 + odd) * HP + pr] + s_bc[((1 * BT + tu) * 4 + 2 + odd) * HP + pr];
+                    const float* r0 = rx + (SG2_COMP_XB * 16 + r) * DM;
+                    const float* r1 = rx + (SG2_COMP_Z * 16 + r) * DM;
+                    const float* r2 = rx + (SG2_COMP_DT * 16 + r) * DM;
+                    const float* r3 = rx + (SG2_COMP_B * 16 + r) * DM;
+                    const float* r4 = rx + (SG2_COMP_C * 16 + r) * DM;
+                    a0 = sg_fma(dxb, r0[0], a0); a1 = sg_fma(dxb, r0[1], a1);
+                    a0 = sg_fma(dz, r1[0], a0); a1 = sg_fma(dz, r1[1], a1);
+                    a0 = sg_fma(ddt, r2[0], a0); a1 = sg_fma(ddt, r2[1], a1);
+                    a0 = sg_fma(dB, r3[0], a0); a1 = sg_fma(dB, r3[1], a1);
+                    a0 = sg_fma(dC, r4[0], a0); a1 = sg_fma(dC, r4[1], a1);
+                }
+                const int u = u0 + tu, t = dir ? (c.N - 1 - u) : u;
+                float2* dst = reinterpret_cast<float2*>(io.dx + ((size_t)dir * pl.total + off + t) * DM) + part;
+                *dst = make_float2(a0, a1);
+            }
         }
         __syncthreads();
     }
@@ -616,9 +691,45 @@ __global__ void k_fill_zero(float* p, int n) {
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0.0f;
 }
 
+// x = W_in [g, s] + b_in of every sorted position (the scan's 8-float input, which the forward kernels never
+// materialise), for callers that keep the reference's interface.  One thread per element.
+__global__ __launch_bounds__(256) void k_x_sorted(Plan pl, float* __restrict__ x_out) {
+    const int tile = blockIdx.x;
+    const int ti = sg::upper_seg(sg::as_const(pl.elem_tile_prefix), pl.P, tile);
+    const TensorDev& T = pl.tensors[ti];
+    const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
+    const int cnt = min(ELEM_TILE, T.numel - start);
+    const bool has_s = pl.sharp_nonzero[ti] != 0;
+    const float* __restrict__ Win = pl.W.w[W_IN_W];
+    const float* __restrict__ bin = pl.W.w[W_IN_B];
+    for (int k = threadIdx.x; k < cnt; k += 256) {
+        const int t = T.off + start + k;
+        const int32_t v = pl.vals[0][t];
+        const float g = sg_i2f((int32_t)pl.keys[0][t] | (v & (int32_t)0x80000000));
+        const float s = has_s ? pl.ssorted[t] : 0.0f;
+        float4 lo, hi;
+        float x[DM];
+#pragma unroll
+        for (int d = 0; d < DM; d++) x[d] = sg_fma(Win[2 * d + 1], s, Win[2 * d] * g) + bin[d];
+        lo = make_float4(x[0], x[1], x[2], x[3]);
+        hi = make_float4(x[4], x[5], x[6], x[7]);
+        reinterpret_cast<float4*>(x_out + (size_t)t * DM)[0] = lo;
+        reinterpret_cast<float4*>(x_out + (size_t)t * DM)[1] = hi;
+    }
+}
+
 }  // namespace
 
-int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st) {
+int launch_x_sorted(const Plan& pl, float* x_out, hipStream_t st) {
+    static_assert(DM == 8, "k_x_sorted: two float4 per element");
+    if (pl.total == 0) return 0;
+    hipLaunchKernelGGL(k_x_sorted, dim3(pl.elem_tiles), dim3(256), 0, st, pl, x_out);
+    SG_LAUNCH_CHECK("k_x_sorted");
+    return 0;
+}
+
+int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* const d_scan[2], const float* rx, float* dx, float* grads_out,
+                            hipStream_t st) {
     static_assert(DM * DI == SCAN_THREADS, "one thread per out_proj entry");
     static_assert(SG2_BWD_STRIDE == SG2_COMP_GROUPS * 16 * 3 + DI * DS + DI * HP + DI + DM * DI, "layout of the per-direction sums");
     {
@@ -627,8 +738,10 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
         SG_HIP_CHECK(hipGetDevice(&dev));
         if (dev < 0 || dev >= 64) return sg::fail("device index %d out of range", dev);
         if (!raised[dev]) {
-            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bilevel_backward), hipFuncAttributeMaxDynamicSharedMemorySize,
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bilevel_backward<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                              BILEVEL_LDS_BYTES));
+            SG_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k_bilevel_backward<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             BILEVEL_DX_LDS_BYTES));
             raised[dev] = true;
         }
     }
@@ -637,12 +750,16 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out
         SG_LAUNCH_CHECK("k_fill_zero");
         return 0;
     }
+    const AdjIO io = {d_ctx, {d_scan ? d_scan[0] : nullptr, d_scan ? d_scan[1] : nullptr}, rx, dx};
     const int groups = pl.chunks < ADJ_GROUPS ? pl.chunks : ADJ_GROUPS;
-    hipLaunchKernelGGL(k_adj_summary, dim3(pl.chunks, 2), dim3(SCAN_THREADS), 0, st, pl, d_ctx);
+    hipLaunchKernelGGL(k_adj_summary, dim3(pl.chunks, 2), dim3(SCAN_THREADS), 0, st, pl, io);
     SG_LAUNCH_CHECK("k_adj_summary");
     hipLaunchKernelGGL(k_adj_prefix, dim3(pl.P, 2), dim3(SCAN_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_adj_prefix");
-    hipLaunchKernelGGL(k_bilevel_backward, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, d_ctx);
+    if (dx != nullptr)
+        hipLaunchKernelGGL(k_bilevel_backward<true>, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_DX_LDS_BYTES, st, pl, io);
+    else
+        hipLaunchKernelGGL(k_bilevel_backward<false>, dim3(groups, 2), dim3(SCAN_THREADS), BILEVEL_LDS_BYTES, st, pl, io);
     SG_LAUNCH_CHECK("k_bilevel_backward");
     static_assert((2 * SG2_BWD_STRIDE) % 64 == 0, "k_adj_sum_rows: whole workgroups");
     hipLaunchKernelGGL(k_adj_sum_rows, dim3(2 * SG2_BWD_STRIDE / 64), dim3(256), 0, st, pl.adj_part, groups, pl.adj_blk);

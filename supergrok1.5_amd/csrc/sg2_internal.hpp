@@ -77,6 +77,7 @@ struct Plan {
     float* hstart;                 // [2][chunks][2][128]
     float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
     float* htile;                  // bilevel: [2][htile_count][2][128] state entering every HT_STEP-th step, or NULL
+    float* scan_out[2];            // bilevel, optional (NULL): per direction [total][DI] gated scan output of every step, in scan order
     float* adj_summ;               // bilevel: [2][chunks][128][6] adjoint transfer map of every chunk
     float* adj_lam;                // bilevel: [2][chunks][128][2] adjoint state arriving at the end of every chunk
     float* adj_blk;                // bilevel: [2][SG2_BWD_STRIDE] sums of adj_part's rows
@@ -101,7 +102,10 @@ __host__ __device__ inline int htile_count(int total, int P) { return total / HT
 constexpr int SG2_BWD_STRIDE = 768;
 constexpr int ADJ_GROUPS = 512;    // workgroups per direction of the adjoint replay (upper bound)
 int check_dims(const SgDims* d);
-int launch_bilevel_backward(const Plan& pl, const float* d_ctx, float* grads_out, hipStream_t st);
+// exactly one of d_ctx (element order, after out_proj) / d_scan (scan order, before out_proj) is given; dx (with rx) is optional
+int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* const d_scan[2], const float* rx, float* dx, float* grads_out,
+                            hipStream_t st);
+int launch_x_sorted(const Plan& pl, float* x_out, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
 
 }  // namespace sg2

@@ -420,6 +420,12 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             if (valid) {
                 float4* dst = reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM) + half;
                 *dst = make_float4(cx[0], cx[1], cx[2], cx[3]);
+                if (KEEP && pl.scan_out[dir] != nullptr) {
+                    // the gated scan output itself (before out_proj), at the step's position in scan order; this half's 8 columns
+                    float4* so = reinterpret_cast<float4*>(pl.scan_out[dir] + ((size_t)off + tile0 + tu) * DI) + 2 * half;
+                    so[0] = half ? make_float4(o[8], o[9], o[10], o[11]) : make_float4(o[0], o[1], o[2], o[3]);
+                    so[1] = half ? make_float4(o[12], o[13], o[14], o[15]) : make_float4(o[4], o[5], o[6], o[7]);
+                }
             }
             __syncthreads();
         }

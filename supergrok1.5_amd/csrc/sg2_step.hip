@@ -8,6 +8,8 @@
 // Stands behind supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877 of
 // the reference) in place of launch_mamba3_peer_batched_step
 // (csrc/supergrok2_mamba_peer_kernels.cu:1754-2117).
+#include <atomic>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -16,8 +18,16 @@
 namespace sg2 {
 namespace {
 
-int g_chunk_len = 0;      // 0: chosen per call from the amount of work, see auto_chunk_len
-int g_window = 256;
+// process-wide settings (atomic: a call reads each once; changing them while other threads are inside a call only
+// affects calls that start later)
+std::atomic<int> g_chunk_len{0};      // 0: chosen per call from the amount of work, see auto_chunk_len
+std::atomic<int> g_window{256};
+
+// What the forward call of the bilevel pass laid out in a workspace, so that the backward call addresses it the same
+// way whatever the settings are by then.  Keyed by the workspace address.
+struct BilevelRecord { int chunk_len, window, P, total; };
+std::mutex g_bilevel_mutex;
+std::map<const void*, BilevelRecord> g_bilevel_records;
 
 // Longer chunks mean fewer summaries (less work in the first scan pass and the prefix), shorter chunks
 // mean more workgroups.  Take the longest of 4096 / 2048 / 1024 that still gives the replay pass about
@@ -37,7 +47,10 @@ int auto_chunk_len(int P, Numels numels) {
     }
     return 1024;
 }
-int effective_chunk_len(int P, Numels numels) { return g_chunk_len > 0 ? g_chunk_len : auto_chunk_len(P, numels); }
+int effective_chunk_len(int P, Numels numels) {
+    const int set = g_chunk_len.load();
+    return set > 0 ? set : auto_chunk_len(P, numels);
+}
 
 // ---- optional per-stage timing with HIP events on the step's stream
 constexpr int PROF_MARKS = SG2_PROF_STAGES + 1;
@@ -190,7 +203,7 @@ int sg2_set_chunk_len(int chunk_len) {
     sg2::g_chunk_len = chunk_len;
     return 0;
 }
-int sg2_get_chunk_len(void) { return sg2::g_chunk_len; }
+int sg2_get_chunk_len(void) { return sg2::g_chunk_len.load(); }
 int sg2_chunk_len_for(int num_tensors, const int64_t* numels) {
     if (num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     return sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr});
@@ -202,7 +215,7 @@ int sg2_set_scan_window(int window) {
     sg2::g_window = window;
     return 0;
 }
-int sg2_get_scan_window(void) { return sg2::g_window; }
+int sg2_get_scan_window(void) { return sg2::g_window.load(); }
 
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
@@ -218,7 +231,8 @@ namespace sg2 {
 // the optimizer-state pointers of every tensor are required; otherwise only grad, sharpness and the two Mamba
 // states (bilevel forward/backward).  Returns 0 with pl->total == 0 when there is nothing to do.
 int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const Sg2Scalars* scalars,
-               void* workspace, size_t workspace_bytes, bool full_step, bool bilevel, bool keep_flags, hipStream_t st, Plan* plp, Layout* Lp) {
+               void* workspace, size_t workspace_bytes, bool full_step, bool bilevel, bool keep_flags, hipStream_t st, Plan* plp, Layout* Lp,
+               int chunk_override = 0, int window_override = -1) {
     Plan& pl = *plp;
     Layout& L = *Lp;
     pl.total = 0;
@@ -239,7 +253,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
             if (full_step && ((uintptr_t)t.gru_state & 15u) != 0) return sg::fail("tensor %d: gru_state must be 16-byte aligned", i);
         }
     }
-    const int chunk_len = effective_chunk_len(P, numels);
+    const int chunk_len = chunk_override > 0 ? chunk_override : effective_chunk_len(P, numels);
     if (make_layout(P, numels, chunk_len, &L, bilevel)) return 1;
     if (L.total == 0) return 0;
     if (!workspace || workspace_bytes < L.bytes)
@@ -289,7 +303,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.chunk_prefix = dpre + 2 * (P + 1);
     pl.wchunk_prefix = dpre + 3 * (P + 1);
     pl.P = P; pl.total = L.total; pl.elem_tiles = L.elem_tiles; pl.sort_tiles = L.sort_tiles;
-    pl.chunks = L.chunks; pl.wchunks = L.wchunks; pl.chunk_len = chunk_len; pl.window = g_window;
+    pl.chunks = L.chunks; pl.wchunks = L.wchunks; pl.chunk_len = chunk_len; pl.window = window_override >= 0 ? window_override : g_window.load();
     for (int k = 0; k < 2; k++) {
         pl.keys[k] = reinterpret_cast<uint32_t*>(ws + L.off_keys[k]);
         pl.vals[k] = reinterpret_cast<int32_t*>(ws + L.off_vals[k]);
@@ -307,6 +321,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.W = *weights;
 
     pl.htile = bilevel ? reinterpret_cast<float*>(ws + L.off_htile) : nullptr;
+    pl.scan_out[0] = pl.scan_out[1] = nullptr;
     pl.adj_summ = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_summ) : nullptr;
     pl.adj_lam = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_lam) : nullptr;
     pl.adj_part = bilevel ? reinterpret_cast<float*>(ws + L.off_adj_part) : nullptr;
@@ -391,34 +406,71 @@ size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const in
     return L.bytes;
 }
 
-int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, float* ctx_out,
-                        void* workspace, size_t workspace_bytes, void* stream) {
+int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, float* ctx_out,
+                           const Sg2BilevelExtra* extra, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace sg2;
     hipStream_t st = (hipStream_t)stream;
     Plan pl;
     Layout L;
     const Sg2Scalars none = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, false, st, &pl, &L)) return 1;
+    {
+        std::lock_guard<std::mutex> lock(g_bilevel_mutex);
+        if (g_bilevel_records.size() > 64) g_bilevel_records.clear();       // forgotten workspaces: bounded memory
+        g_bilevel_records[workspace] = BilevelRecord{pl.total > 0 ? pl.chunk_len : 0, pl.total > 0 ? pl.window : 0, num_tensors, pl.total};
+    }
     if (pl.total == 0) return 0;
-    if (!ctx_out) return sg::fail("ctx_out is NULL");
-    pl.ctx = ctx_out;
-    if (launch_sort(pl, nullptr, st)) return 1;
-    return launch_scan(pl, st);
+    if (ctx_out) pl.ctx = ctx_out;                 // else the contexts stay in the workspace
+    if (extra) { pl.scan_out[0] = extra->scan_out_fwd; pl.scan_out[1] = extra->scan_out_bwd; }
+    if (launch_sort(pl, extra ? extra->perm : nullptr, st)) return 1;
+    if (launch_scan(pl, st)) return 1;
+    if (extra && extra->x_sorted) return launch_x_sorted(pl, extra->x_sorted, st);
+    return 0;
 }
 
-int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const float* d_ctx,
-                         float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
+int sg2_bilevel_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, float* ctx_out,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+    if (!ctx_out && num_tensors > 0) return sg::fail("ctx_out is NULL");
+    return sg2_bilevel_forward_ex(dims, weights, num_tensors, tensors, ctx_out, nullptr, workspace, workspace_bytes, stream);
+}
+
+int sg2_bilevel_backward_ex(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const float* d_ctx,
+                            const float* d_scan_out_fwd, const float* d_scan_out_bwd, const float* row_dx, float* dx_out, float* grads_out,
+                            void* workspace, size_t workspace_bytes, void* stream) {
     using namespace sg2;
     hipStream_t st = (hipStream_t)stream;
     Plan pl;
     Layout L;
     const Sg2Scalars none = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
     if (!grads_out) return sg::fail("grads_out is NULL");
-    // same layout as the forward call: sorted keys / payloads / sharpness, the sharpness flags, coefficients and tile
-    // states are still in place
-    if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, true, st, &pl, &L)) return 1;
-    if (pl.total > 0 && !d_ctx) return sg::fail("d_ctx is NULL");
-    return launch_bilevel_backward(pl, d_ctx, grads_out, st);
+    BilevelRecord rec;
+    {
+        std::lock_guard<std::mutex> lock(g_bilevel_mutex);
+        const auto it = g_bilevel_records.find(workspace);
+        if (it == g_bilevel_records.end())
+            return sg::fail("sg2_bilevel_backward: no forward call has been made on this workspace");
+        rec = it->second;
+    }
+    // the layout of the forward call (its chunk length and window, whatever the settings are now): sorted keys /
+    // payloads / sharpness, the sharpness flags, coefficients and tile states are still in place
+    if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, true, st, &pl, &L, rec.chunk_len,
+                   rec.window))
+        return 1;
+    if (num_tensors != rec.P || pl.total != rec.total)
+        return sg::fail("sg2_bilevel_backward: %d tensors / %d elements, but the forward call on this workspace had %d / %d", num_tensors,
+                        pl.total, rec.P, rec.total);
+    if ((d_scan_out_fwd != nullptr) != (d_scan_out_bwd != nullptr)) return sg::fail("d_scan_out: both directions or neither");
+    if (pl.total > 0 && ((d_ctx != nullptr) == (d_scan_out_fwd != nullptr))) return sg::fail("exactly one of d_ctx and d_scan_out must be given");
+    if (dx_out != nullptr && row_dx == nullptr) return sg::fail("dx_out needs row_dx");
+    const float* const d_scan[2] = {d_scan_out_fwd, d_scan_out_bwd};
+    return launch_bilevel_backward(pl, d_ctx, d_scan, row_dx, dx_out, grads_out, st);
+}
+
+int sg2_bilevel_backward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const float* d_ctx,
+                         float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
+    if (num_tensors > 0 && !d_ctx) return sg::fail("d_ctx is NULL");
+    return sg2_bilevel_backward_ex(dims, weights, num_tensors, tensors, d_ctx, nullptr, nullptr, nullptr, nullptr, grads_out, workspace,
+                                   workspace_bytes, stream);
 }
 
 }  // extern "C"

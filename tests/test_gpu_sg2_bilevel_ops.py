@@ -1,0 +1,184 @@
+"""The reference's bilevel entry points through `_ops`
+(supergrok2_bilevel_fwd_save_batched / supergrok2_bilevel_backward_batched / supergrok2_bilevel_fwd_save, with the
+argument lists of csrc/ops.h:232-371 of the reference), driven the way the reference's own caller drives them
+(grokking_optimizers/supergrok2.py:646-1040 there): packed buffers allocated by the caller, out_proj / unsort / GRU /
+soft top-4 routing / experts in torch between the two calls, input_proj gradients from d_x_sorted afterwards.
+Checked against float64 autograd through the restatement of the whole differentiable forward
+(ref_fp64.forward_for_bilevel, pinned on the CPU by tests/test_oracle_sg2_pins.py): every one of the 42 parameter
+gradients within 2e-4 of its largest entry."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import ref_fp64
+
+pytestmark = pytest.mark.gpu
+
+
+def _meta_net(seed, dev):
+    from grokking_optimizers import Mamba3PEERMetaNet
+    torch.manual_seed(seed)
+    mn = Mamba3PEERMetaNet()
+    with torch.no_grad():       # the initial keys and experts are nearly silent: give every part a visible gradient
+        for p in mn.parameters():
+            if p.dim() > 0 and float(p.abs().max()) < 0.05:
+                p.add_(torch.randn_like(p) * 0.2)
+    return mn.to(dev)
+
+
+def _flat64(mn):
+    blk = lambda b: [b.in_proj.weight, b.dt_proj.weight, b.dt_proj.bias, b.B_proj.weight, b.C_proj.weight, b.A_log, b.D,
+                     b.rope_freq, b.out_proj.weight]
+    E = mn.num_experts
+    return ([mn.input_proj.weight, mn.input_proj.bias] + blk(mn.mamba_fwd) + blk(mn.mamba_bwd) +
+            [mn.gru.W_z.weight, mn.gru.W_z.bias, mn.gru.W_r.weight, mn.gru.W_r.bias, mn.gru.W_h.weight, mn.gru.W_h.bias] +
+            [torch.stack([q.weight for q in mn.peer_queries]), torch.stack(list(mn.product_keys_A)), torch.stack(list(mn.product_keys_B))] +
+            [mn.expert_W1.reshape(E, -1), mn.expert_b1, mn.expert_W2.reshape(E, -1), mn.expert_b2.reshape(-1)])
+
+
+MAMBA = ("in_proj", "dt_proj_W", "dt_proj_b", "B_proj", "C_proj", "A_log", "D", "rope_freq")
+
+
+def _mamba_args(w, tag, with_out):
+    names = MAMBA + (("out_proj",) if with_out else ())
+    return [w[f"mamba_{tag}_{n}"] for n in names]
+
+
+def test_reference_batched_bilevel_entry_points():
+    from grokking_optimizers import _bilevel, _ops
+    dev = torch.device("cuda:0")
+    mn = _meta_net(5, dev)
+    mn64 = copy.deepcopy(mn).double().cpu()
+    gen = torch.Generator().manual_seed(23)
+    Ns = [150, 99, 1300, 64]
+    data = [dict(g=torch.randn(n, generator=gen) * 0.5, s=torch.rand(n, generator=gen) * 0.3, h=torch.randn(n, 4, generator=gen) * 0.5,
+                 hf=torch.randn(16, 16, generator=gen) * 0.3, hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen))
+            for n in Ns]
+    # ---- float64 reference: gradient of sum_p <smart_p, R_p> with respect to all 42 parameters
+    dims = dict(d_model=8, num_heads=4, pk_dim=12)
+    for d in data:
+        smart, _, _, _ = ref_fp64.forward_for_bilevel(_flat64(mn64), d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(),
+                                                      d["hb"].double(), mn64.rescale, dims)
+        (smart * d["R"].double()).sum().backward()
+        d["smart64"] = smart.detach()
+    ref = {n: p.grad.clone() for n, p in mn64.named_parameters()}
+
+    # ---- the reference caller's sequence
+    w = mn.get_weights()
+    w = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in w.items()}
+    d_model, d_state, d_inner = 8, 16, 16
+    total, P = sum(Ns), len(Ns)
+    z = lambda *s: torch.zeros(*s, device=dev)
+    fwd_scan, bwd_scan = z(total, d_inner), z(total, d_inner)
+    saved = [z(total, d_inner, d_state)] + [z(total, d_inner) for _ in range(3)] + [z(total, d_inner, d_state)] + [z(total, d_inner) for _ in range(3)]
+    x_sorted, offsets_t = z(total, d_model), torch.zeros(P + 1, dtype=torch.int32, device=dev)
+    sort_idx = torch.zeros(total, dtype=torch.int32, device=dev)
+    init_f = torch.stack([d["hf"] for d in data]).to(dev)
+    init_b = torch.stack([d["hb"] for d in data]).to(dev)
+    init_f0, init_b0 = init_f.clone(), init_b.clone()
+    grads = [d["g"].to(dev) for d in data]
+    sharps = [d["s"].to(dev) for d in data]
+    print("fwd_save_batched", Ns, flush=True)
+    _ops.supergrok2_bilevel_fwd_save_batched(grads, sharps, w["input_proj_W"], w["input_proj_b"], *_mamba_args(w, "fwd", True),
+                                             *_mamba_args(w, "bwd", True), d_model, d_state, d_inner, fwd_scan, bwd_scan, *saved,
+                                             x_sorted, offsets_t, sort_idx, init_f, init_b, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(init_f, init_f0) and torch.equal(init_b, init_b0)         # the caller's states are not touched
+    offs = np.concatenate([[0], np.cumsum(Ns)])
+    assert np.array_equal(offsets_t.cpu().numpy(), offs)
+    for i, d in enumerate(data):                                                  # sort order and x_sorted
+        a, b = int(offs[i]), int(offs[i + 1])
+        want = torch.sort(d["g"].abs(), stable=True).indices
+        assert torch.equal(sort_idx[a:b].cpu().long(), want)
+        xs = torch.stack([d["g"][want], d["s"][want]], -1) @ w["input_proj_W"].cpu().T + w["input_proj_b"].cpu()
+        assert torch.allclose(x_sorted[a:b].cpu(), xs, rtol=1e-5, atol=1e-6)
+
+    # between the calls: out_proj, unsort, GRU, soft routing, experts in torch (fp32, autograd), as the caller does
+    for p in mn.parameters():
+        p.grad = None
+    fs = fwd_scan.clone().requires_grad_(True)
+    bs = bwd_scan.clone().requires_grad_(True)
+    loss = torch.zeros((), device=dev)
+    smarts = []
+    for i, d in enumerate(data):
+        a, b = int(offs[i]), int(offs[i + 1])
+        unsort = sort_idx[a:b].long().argsort()
+        ctx_f = (fs[a:b] @ mn.mamba_fwd.out_proj.weight.T)[unsort]
+        ctx_b = (bs[a:b] @ mn.mamba_bwd.out_proj.weight.T).flip(0)[unsort]
+        smart, _ = _bilevel.per_element(mn, grads[i], sharps[i], ctx_f, ctx_b, d["h"].to(dev))
+        loss = loss + (smart * d["R"].to(dev)).sum()
+        smarts.append(smart.detach())
+        err = (smart.detach().double().cpu() - d["smart64"]).abs()
+        assert bool((err <= 1e-4 * d["smart64"].abs() + 1e-6).all()), ("smart", i, float(err.max()))
+    loss.backward()
+
+    d_mamba = [torch.zeros_like(t) for t in _mamba_args(w, "fwd", False) + _mamba_args(w, "bwd", False)]
+    d_x_sorted = z(total, d_model)
+    print("backward_batched", flush=True)
+    _ops.supergrok2_bilevel_backward_batched(fs.grad.contiguous(), bs.grad.contiguous(), x_sorted, *saved, offsets_t,
+                                             *_mamba_args(w, "fwd", False), *_mamba_args(w, "bwd", False), *d_mamba, d_x_sorted,
+                                             init_f, init_b, d_model, d_state, d_inner, P, 1)
+    torch.cuda.synchronize()
+    # input_proj from d_x_sorted, as the caller does
+    dW, db = z(d_model, 2), z(d_model)
+    for i, d in enumerate(data):
+        a, b = int(offs[i]), int(offs[i + 1])
+        unsort = sort_idx[a:b].long().argsort()
+        dxu = d_x_sorted[a:b].index_select(0, unsort)
+        dW.addmm_(dxu.T, torch.stack([grads[i], sharps[i]], -1))
+        db.add_(dxu.sum(0))
+
+    got = {"input_proj.weight": dW, "input_proj.bias": db}
+    tags = {"in_proj": "in_proj.weight", "dt_proj_W": "dt_proj.weight", "dt_proj_b": "dt_proj.bias", "B_proj": "B_proj.weight",
+            "C_proj": "C_proj.weight", "A_log": "A_log", "D": "D", "rope_freq": "rope_freq"}
+    for k, tag in enumerate(("fwd", "bwd")):
+        for q, n in enumerate(MAMBA):
+            got[f"mamba_{tag}.{tags[n]}"] = d_mamba[k * 8 + q]
+    for n, p in mn.named_parameters():
+        if n not in got:
+            got[n] = p.grad if p.grad is not None else torch.zeros_like(p)
+    worst = {}
+    for n, r in ref.items():
+        g = got[n].double().cpu().reshape(r.shape)
+        scale = float(r.abs().max())
+        worst[n] = round(float((g - r).abs().max()) / (2e-4 * scale + 1e-12), 3)
+    print("worst gradient tolerance ratios", worst, flush=True)
+    assert max(worst.values()) <= 1.0, worst
+    # a second backward call on the same buffers has nothing to restart from
+    with pytest.raises(RuntimeError, match="fwd_save_batched"):
+        _ops.supergrok2_bilevel_backward_batched(fs.grad.contiguous(), bs.grad.contiguous(), x_sorted, *saved, offsets_t,
+                                                 *_mamba_args(w, "fwd", False), *_mamba_args(w, "bwd", False), *d_mamba, d_x_sorted,
+                                                 init_f, init_b, d_model, d_state, d_inner, P, 1)
+
+
+def test_reference_single_tensor_fwd_save_and_the_missing_backward():
+    from grokking_optimizers import _ops
+    dev = torch.device("cuda:0")
+    mn = _meta_net(9, dev)
+    w = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in mn.get_weights().items()}
+    gen = torch.Generator().manual_seed(3)
+    n = 700
+    g, s = (torch.randn(n, generator=gen) * 0.5).to(dev), (torch.rand(n, generator=gen) * 0.3).to(dev)
+    hf, hb = (torch.randn(16, 16, generator=gen) * 0.3).to(dev), (torch.randn(16, 16, generator=gen) * 0.3).to(dev)
+    z = lambda *sh: torch.zeros(*sh, device=dev)
+    fs, bs, ff, fb = z(n, 16), z(n, 16), z(16, 16), z(16, 16)
+    saved = [z(n, 16, 16)] + [z(n, 16) for _ in range(3)] + [z(n, 16, 16)] + [z(n, 16) for _ in range(3)]
+    xs, si = z(n, 8), torch.zeros(n, dtype=torch.int32, device=dev)
+    _ops.supergrok2_bilevel_fwd_save(g, s, w["input_proj_W"], w["input_proj_b"], *_mamba_args(w, "fwd", True), *_mamba_args(w, "bwd", True),
+                                     8, 16, 16, fs, bs, ff, fb, *saved, xs, si, hf, hb, 1)
+    torch.cuda.synchronize()
+    # against the float64 scan: gated outputs before out_proj, final states
+    perm = torch.sort(g.abs().cpu(), stable=True).indices
+    assert torch.equal(si.cpu().long(), perm)
+    W = [t.double().cpu() for t in mn.flat_weights()]
+    x = torch.stack([g.cpu().double()[perm], s.cpu().double()[perm]], -1) @ W[0].T + W[1]
+    eye = torch.eye(16, dtype=torch.float64)           # identity out_proj: scan_block then returns the gated output itself
+    fo, hF = ref_fp64.scan_block(x, W[2:10] + [eye], hf.double().cpu())
+    bo, hB = ref_fp64.scan_block(x.flip(0), W[11:19] + [eye], hb.double().cpu())
+    for name, got, want in (("fwd_scan_out", fs, fo), ("bwd_scan_out", bs, bo), ("fwd_final_state", ff, hF), ("bwd_final_state", fb, hB)):
+        err = (got.double().cpu() - want).abs()
+        assert bool((err <= 1e-4 * want.abs() + 1e-6).all()), (name, float(err.max()))
+    with pytest.raises(RuntimeError, match="supergrok2_bilevel_backward_batched"):
+        _ops.supergrok2_bilevel_backward(g, s)
