@@ -27,7 +27,7 @@ extern "C" {
 enum { SG_F32 = 0, SG_F16 = 1, SG_BF16 = 2 };
 
 /* meta-net dimensions, the trailing ints of
- * launch_mamba3_peer_batched_step (csrc/ops.h:342-370) */
+ * launch_mamba3_peer_batched_step (csrc/ops.h:196-229) */
 typedef struct SgDims {
     int32_t d_model, d_state, d_inner, gru_hidden, num_heads, pk_dim, expert_hidden, num_experts;
 } SgDims;
@@ -102,7 +102,7 @@ int sg2_get_scan_window(void);
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
 
 /* SuperGrok v2 full step over all tensors: replaces
- * launch_mamba3_peer_batched_step (csrc/ops.h:342-370,
+ * launch_mamba3_peer_batched_step (csrc/ops.h:196-229,
  * csrc/supergrok2_mamba_peer_kernels.cu:1754-2117) behind
  * supergrok2_mamba_peer_batched_step (csrc/ops.cpp:815-877).
  * `tensors` is a host array; tensors with numel == 0 are skipped.
