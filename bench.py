@@ -27,10 +27,13 @@ PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.625e9 + 1.612e9, "scan_summary": 0
                              "elementwise": 2.603e9 + 0.801e9}
 
 
-def build_workload(name, device, nonzero_sharpness=False, weights="bench"):
+LARGE_GEOMETRY = dict(d_model=16, d_state=32, d_inner=32)     # the second scan geometry the kernels are built for
+
+
+def build_workload(name, device, nonzero_sharpness=False, weights="bench", geometry="default"):
     import torch
     import workloads as wl
-    DIMS = wl.DEFAULT_DIMS
+    DIMS = dict(wl.DEFAULT_DIMS, **(LARGE_GEOMETRY if geometry == "large" else {}))
     shapes = {"scale50": wl.scale50_shapes, "shared14": wl.shared14_shapes}[name]()
     gh, di, ds = DIMS["gru_hidden"], DIMS["d_inner"], DIMS["d_state"]
     params = [p.reshape(-1).to(device) for p in wl.make_params(shapes, seed=0)]
@@ -52,8 +55,8 @@ def build_workload(name, device, nonzero_sharpness=False, weights="bench"):
         sharps = [(g.abs() * 0.5).contiguous() for g in grad_sets[1]]
     # "bench": N(0, 0.1) in every tensor (the configuration the metric is quoted on); "module": the optimizer's own
     # initial meta-net (A_log = log(1..16), default Linear weights)
-    weights = [w.to(device) for w in (wl.meta_weights(7) if weights == "bench" else wl.module_weights(0))]
-    return shapes, state, grad_sets, sharps, weights
+    weights = [w.to(device) for w in (wl.meta_weights(7, DIMS) if weights == "bench" else wl.module_weights(0))]
+    return shapes, state, grad_sets, sharps, weights, DIMS
 
 
 def cpu_baseline(sample_elems_target=4_000_000):
@@ -341,6 +344,8 @@ def main():
     ap.add_argument("--window", type=int, default=-1, help="scan summary window (-1: library default, 0: off)")
     ap.add_argument("--weights", default="bench", choices=["bench", "module"],
                     help="v2 workloads: meta-net weights N(0, 0.1) (default, the measured configuration) or the optimizer's own initialisation")
+    ap.add_argument("--geometry", default="default", choices=["default", "large"],
+                    help="v2 workloads: meta-net of d_model=8, d_state=16, d_inner=16 (the configuration the metric is quoted on) or 16, 32, 32")
     ap.add_argument("--boundary", default="ops", choices=["ops", "cabi"],
                     help="v2 workloads: time the torch-extension call _ops.supergrok2_mamba_peer_batched_step (default) or the bare C-ABI call")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -367,12 +372,13 @@ def main():
         return
     if _cabi.lib().sg2_set_chunk_len(args.chunk_len) or _cabi.lib().sg2_set_scan_window(args.window):
         raise SystemExit(_cabi.last_error())
-    shapes, st, grad_sets, sharps, weights = build_workload(args.workload, dev, args.sharpness, args.weights)
+    if args.geometry == "large" and args.weights != "bench":
+        raise SystemExit("--geometry large runs with --weights bench")
+    shapes, st, grad_sets, sharps, weights, D = build_workload(args.workload, dev, args.sharpness, args.weights, args.geometry)
     total = sum(p.numel() for p in st["params"])
-    D = _cabi.DEFAULT_DIMS
     if args.boundary == "cabi":
         step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
-                             st["counts"])
+                             st["counts"], dims=D)
     else:
         # the reference's own entry point: supergrok2_mamba_peer_batched_step of the torch extension, 51 arguments
         from grokking_optimizers import _ops
@@ -427,15 +433,16 @@ def main():
                                % (len(shapes), total, "50 log-uniform tensors" if args.workload == "scale50" else "2-layer transformer set"),
                    "chunk_len": _cabi.chunk_len_for([p.numel() for p in st["params"]]), "summary_window": _cabi.lib().sg2_get_scan_window(),
                    "timed_call": "_ops.supergrok2_mamba_peer_batched_step" if args.boundary == "ops" else "sg2_batched_step (C ABI)",
-                   "meta_weights": "N(0, 0.1), seed 7" if args.weights == "bench" else "Mamba3PEERMetaNet() initialisation, seed 0"},
+                   "meta_weights": "N(0, 0.1), seed 7" if args.weights == "bench" else "Mamba3PEERMetaNet() initialisation, seed 0",
+                   "meta_net": "d_model=%d d_state=%d d_inner=%d" % (D["d_model"], D["d_state"], D["d_inner"])},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if (args.workload, args.weights) == ("scale50", "bench") else None,
+                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if (args.workload, args.weights, args.geometry) == ("scale50", "bench", "default") else None,
                      "kernel_ms": stage_avg[dom]},
         "step_hbm_frac": BYTES_PER_ELEMENT * value / 1e9 / HBM_PEAK_GBS,
         "stage_ms": stage_avg,
     }
-    if not args.no_class_step:
+    if not args.no_class_step and args.geometry == "default":
         out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

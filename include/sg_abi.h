@@ -27,7 +27,11 @@ extern "C" {
 enum { SG_F32 = 0, SG_F16 = 1, SG_BF16 = 2 };
 
 /* meta-net dimensions, the trailing ints of
- * launch_mamba3_peer_batched_step (csrc/ops.h:196-229) */
+ * launch_mamba3_peer_batched_step (csrc/ops.h:196-229).  The step kernels
+ * are built for (d_model, d_state, d_inner) = (8, 16, 16) and (16, 32, 32),
+ * both with gru_hidden 4, num_heads 4, pk_dim 12, expert_hidden 16 and
+ * num_experts 144; anything else is refused with an error that says so.
+ * The bilevel entry points take the first set only. */
 typedef struct SgDims {
     int32_t d_model, d_state, d_inner, gru_hidden, num_heads, pk_dim, expert_hidden, num_experts;
 } SgDims;

@@ -22,9 +22,10 @@ namespace {
 constexpr int ELEM_THREADS = 256;
 constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[16] W2[16] + pad
 
-template <bool DBG>
+template <class G, bool DBG>
 __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
                                                        int32_t* __restrict__ dbg_eidx) {
+    constexpr int DM = G::DM, GRL = G::GRL, PIN = G::PIN;
     __shared__ float s_exp[NE * EXP_STRIDE];
     __shared__ float s_b2[NE];
     __shared__ int s_cnt[NE];
@@ -77,9 +78,12 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             {
                 const float4* pf = reinterpret_cast<const float4*>(pl.ctx + ((size_t)T.off + i) * DM);
                 const float4* pb = reinterpret_cast<const float4*>(pl.ctx + ((size_t)pl.total + T.off + i) * DM);
-                const float4 a0 = pf[0], a1 = pf[1], b0 = pb[0], b1 = pb[1];
-                cf[0] = a0.x; cf[1] = a0.y; cf[2] = a0.z; cf[3] = a0.w; cf[4] = a1.x; cf[5] = a1.y; cf[6] = a1.z; cf[7] = a1.w;
-                cb[0] = b0.x; cb[1] = b0.y; cb[2] = b0.z; cb[3] = b0.w; cb[4] = b1.x; cb[5] = b1.y; cb[6] = b1.z; cb[7] = b1.w;
+#pragma unroll
+                for (int q = 0; q < DM / 4; q++) {
+                    const float4 a = pf[q], b = pb[q];
+                    cf[4 * q] = a.x; cf[4 * q + 1] = a.y; cf[4 * q + 2] = a.z; cf[4 * q + 3] = a.w;
+                    cb[4 * q] = b.x; cb[4 * q + 1] = b.y; cb[4 * q + 2] = b.z; cb[4 * q + 3] = b.w;
+                }
                 const float4 h4 = reinterpret_cast<const float4*>(T.gru)[i];
                 hold[0] = h4.x; hold[1] = h4.y; hold[2] = h4.z; hold[3] = h4.w;
             }
@@ -199,10 +203,15 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st) {
     if (pl.total == 0) return 0;
     const int grid = pl.elem_tiles < 2048 ? pl.elem_tiles : 2048;
-    if (dbg_expert_idx)
-        hipLaunchKernelGGL(k_elem<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+    if (pl.geo == GEO_LARGE) {
+        if (dbg_expert_idx)
+            hipLaunchKernelGGL((k_elem<GeoLarge, true>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+        else
+            hipLaunchKernelGGL((k_elem<GeoLarge, false>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+    } else if (dbg_expert_idx)
+        hipLaunchKernelGGL((k_elem<GeoDefault, true>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
     else
-        hipLaunchKernelGGL(k_elem<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+        hipLaunchKernelGGL((k_elem<GeoDefault, false>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
     SG_LAUNCH_CHECK("k_elem");
     return 0;
 }

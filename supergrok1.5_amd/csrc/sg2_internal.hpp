@@ -5,25 +5,55 @@
 
 namespace sg2 {
 
-// Compile-time meta-net dimensions the kernels are specialised for (the
-// defaults of the optimizer class; csrc/supergrok2_mamba_peer_kernels.cu:36-42
-// of the reference only caps them).
-constexpr int DM = 8;      // d_model
-constexpr int DS = 16;     // d_state
-constexpr int DI = 16;     // d_inner
-constexpr int HP = DS / 2; // RoPE pairs
+// Compile-time meta-net geometries the step kernels are instantiated for: the
+// defaults of the optimizer class and the largest scan block the reference
+// admits (csrc/supergrok2_mamba_peer_kernels.cu:36-42 caps d_model at 16 and
+// d_state / d_inner at 32).  The GRU, routing and expert sizes are the same in both.
 constexpr int GH = 4;      // gru_hidden
 constexpr int NH = 4;      // PEER heads
 constexpr int PK = 12;     // sub-keys per half
 constexpr int EH = 16;     // expert hidden
 constexpr int NE = 144;    // experts
-constexpr int GRL = 2 + 2 * DM + GH;   // GRU row length (22)
-constexpr int PIN = GH + 2 * DM + 2;   // PEER query input length (22)
+template <int DM_, int DS_, int DI_>
+struct Geo {
+    static constexpr int DM = DM_;               // d_model
+    static constexpr int DS = DS_;               // d_state
+    static constexpr int DI = DI_;               // d_inner
+    static constexpr int HP = DS_ / 2;           // RoPE pairs
+    static constexpr int THREADS = DI_ * HP;     // scan workgroup: one lane per (column, RoPE pair)
+    static constexpr int PARTS = THREADS / 64;   // waves of that workgroup; each projects 1/PARTS of every output group
+    static constexpr int ROWS = DI_;             // rows per group of composed coefficients
+    static constexpr int GRL = 2 + 2 * DM_ + GH; // GRU row length
+    static constexpr int PIN = GH + 2 * DM_ + 2; // PEER query input length
+    static_assert(DI_ == DS_, "coefficient groups of equal height");
+    static_assert(HP == 8 || HP == 16, "a column's pairs are one half or one whole DPP row");
+    static_assert(THREADS % 64 == 0 && THREADS <= 1024 && DI_ % PARTS == 0 && DS_ % PARTS == 0 && DM_ % PARTS == 0 && DM_ % 4 == 0,
+                  "whole waves; every output group splits evenly over them");
+    static_assert(DM_ * DI_ == THREADS, "one out_proj entry per lane when it is staged");
+};
+using GeoDefault = Geo<8, 16, 16>;
+using GeoLarge = Geo<16, 32, 32>;
+enum { GEO_DEFAULT = 0, GEO_LARGE = 1, GEO_COUNT = 2 };
+// run-time view of a geometry for the host code that sizes the work arrays
+struct GeoInfo {
+    int dm, ds, di, threads, rows;
+};
+inline GeoInfo geo_info(int geo) {
+    return geo == GEO_LARGE ? GeoInfo{GeoLarge::DM, GeoLarge::DS, GeoLarge::DI, GeoLarge::THREADS, GeoLarge::ROWS}
+                            : GeoInfo{GeoDefault::DM, GeoDefault::DS, GeoDefault::DI, GeoDefault::THREADS, GeoDefault::ROWS};
+}
+// the bilevel kernels exist for the default geometry only and use its constants directly
+constexpr int DM = GeoDefault::DM;
+constexpr int DS = GeoDefault::DS;
+constexpr int DI = GeoDefault::DI;
+constexpr int HP = GeoDefault::HP;
+constexpr int GRL = GeoDefault::GRL;
+constexpr int PIN = GeoDefault::PIN;
 
 constexpr int ELEM_TILE = 1024;        // elements per tile of the elementwise kernels
 constexpr int SORT_TILE = 4096;        // keys per radix-sort tile (256 threads x 16)
 constexpr int SCAN_TT = 64;            // timesteps projected per LDS tile
-constexpr int SCAN_THREADS = DI * HP;  // one lane per (column, RoPE pair)
+constexpr int SCAN_THREADS = GeoDefault::THREADS;
 constexpr int SCAN_BLOCK_ITEMS = 2048; // entries per block of the spine scan
 
 // weight slots (argument order of supergrok2_mamba_peer_batched_step)
@@ -66,6 +96,7 @@ struct Plan {
     int P;
     int total;                     // sum of numel
     int elem_tiles, sort_tiles, chunks, wchunks;
+    int geo;                       // GEO_*: which instantiation of the scan / elementwise kernels runs
     int chunk_len;
     int window;                    // summary window (0: whole chunk), see k_scan<false>
     uint32_t* keys[2];
@@ -73,9 +104,9 @@ struct Plan {
     float* ssorted;                // [total] sharpness gathered into sorted order
     uint32_t* spine;               // [256 * sort_tiles] per-tile digit counts, layout [segment][digit][tile]
     uint32_t* blocksums;
-    float* summaries;              // [2][wchunks][6][128]
-    float* hstart;                 // [2][chunks][2][128]
-    float* comp;                   // [2][SG2_COMP_GROUPS][16][3] composed projection coefficients per direction
+    float* summaries;              // [2][wchunks][6][THREADS]
+    float* hstart;                 // [2][chunks][2][THREADS]
+    float* comp;                   // [2][SG2_COMP_GROUPS][ROWS][3] composed projection coefficients per direction
     float* htile;                  // bilevel: [2][htile_count][2][128] state entering every HT_STEP-th step, or NULL
     float* scan_out[2];            // bilevel, optional (NULL): per direction [total][DI] gated scan output of every step, in scan order
     float* adj_summ;               // bilevel: [2][chunks][128][6] adjoint transfer map of every chunk
@@ -83,7 +114,7 @@ struct Plan {
     float* adj_blk;                // bilevel: [2][SG2_BWD_STRIDE] sums of adj_part's rows
     float* adj_part;               // bilevel: [2][ADJ_GROUPS][SG2_BWD_STRIDE] per-workgroup gradient sums
     int* sharp_nonzero;            // [P] uploaded as 0; set by k_keys when some (finite) sharpness entry of the tensor is not 0
-    float* ctx;                    // [2][total][DM]
+    float* ctx;                    // [2][total][d_model]
     float decay, beta2, eps, rescale;
     Sg2Weights W;
 };
@@ -101,6 +132,9 @@ __host__ __device__ inline int htile_count(int total, int P) { return total / HT
 // floats per direction of the adjoint kernels' sums: composed coefficients [5][16][3], A_log [16][16], rope_freq [16][8], D [16], out_proj [8][16]
 constexpr int SG2_BWD_STRIDE = 768;
 constexpr int ADJ_GROUPS = 512;    // workgroups per direction of the adjoint replay (upper bound)
+// GEO_* of these dimensions, or -1 with the error set
+int geo_of(const SgDims* d);
+// 0 if the dimensions are the default geometry (what the bilevel kernels are built for), else 1 with the error set
 int check_dims(const SgDims* d);
 // exactly one of d_ctx (element order, after out_proj) / d_scan (scan order, before out_proj) is given; dx (with rx) is optional
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* const d_scan[2], const float* rx, float* dx, float* grads_out,

@@ -8,16 +8,16 @@
 //
 // The sorted sequence of a tensor is cut into chunks of chunk_len timesteps
 // (scan order: t ascending for the forward direction, descending for the
-// backward one).  One 128-lane workgroup owns one chunk; lane (j,p) owns
-// column j and RoPE pair p, i.e. the two states h[j][2p], h[j][2p+1].
+// backward one).  One workgroup of d_inner * d_state/2 lanes (128 for the default
+// geometry, 512 for the large one) owns one chunk; lane (j,p) owns column j and
+// RoPE pair p, i.e. the two states h[j][2p], h[j][2p+1].
 //   k_scan<false>  every chunk but the last of a tensor: 2x2 affine summary
 //                  (M,b) of the chunk, accumulated from the identity.  The
-//                  recurrence contracts (|A_bar| < 1), so the summary is first
-//                  taken over the last `window` steps only; if every |entry| of
-//                  that window's M, in all 128 lanes, is below 2^-100 the chunk
-//                  summary is (0, b_window) -- the state entering the window
-//                  is multiplied by less than 2^-100 -- otherwise the whole
-//                  chunk is accumulated.
+//                  recurrence contracts (|A_bar| < 1), so the chunk is walked
+//                  backwards in blocks of `window` steps and the walk stops as
+//                  soon as every |entry| of the running M, in all lanes, is
+//                  below 2^-100: the state entering that block is multiplied
+//                  by less than 2^-100, and the summary is (0, b).
 //   k_chunk_prefix start state of each chunk: summaries applied in order to
 //                  the carried state of the tensor.
 //   k_scan<true>   every chunk replayed from its start state: y = h.C, gate,
@@ -27,7 +27,7 @@
 //   k_compose      runs first: the input of a timestep is two numbers (g, s)
 //                  and every projection of the block is linear in their 8-float
 //                  input projection, so input_proj, in_proj, dt_proj, B_proj and
-//                  C_proj are folded into 5 x 16 coefficient triples per
+//                  C_proj are folded into 5 x d_inner coefficient triples per
 //                  direction (include/sg2_compose.h).
 // Per-timestep projections (x-branch, z, dt, B, C) are evaluated from those
 // triples in both passes for tiles of 64 timesteps and staged through LDS
@@ -66,12 +66,15 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int UB = SG2_SCAN_UB;           // timesteps per unrolled block of the recurrence
 static_assert(UB % 4 == 0 && SCAN_TT % UB == 0 && SCAN_TT == 64, "blocks are fetched 4 timesteps per LDS read; one ballot covers a tile");
 static_assert(HT_STEP % UB == 0 && SCAN_TT % HT_STEP == 0 && SCAN_TT / HT_STEP <= 2, "kept states fall on block borders: tile start and at most one more");
-// Three waves per SIMD (168 VGPRs) is where the kernels stop gaining from occupancy; keep the
-// register allocation from drifting just past that boundary.
+// Three waves per SIMD (168 VGPRs) is where the default geometry's kernels stop gaining from occupancy; keep the
+// register allocation from drifting just past that boundary.  The large geometry's workgroup is two waves per SIMD by itself,
+// and at 128 VGPRs (two workgroups per CU) the recurrence spills: one workgroup per CU, up to 256 VGPRs.
 #ifndef SG2_SCAN_WAVES
 #define SG2_SCAN_WAVES 3
 #endif
-#define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(SG2_SCAN_WAVES, SG2_SCAN_WAVES)))
+template <class G>
+constexpr int scan_waves() { return G::PARTS == 2 ? SG2_SCAN_WAVES : 2; }
+#define SG2_SCAN_ATTR __attribute__((amdgpu_waves_per_eu(scan_waves<G>(), scan_waves<G>())))
 
 __device__ __forceinline__ float dpp_quad_swap1(float v) {   // lane ^ 1
     return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0xB1, 0xF, 0xF, true));
@@ -82,21 +85,35 @@ __device__ __forceinline__ float dpp_quad_swap2(float v) {   // lane ^ 2
 __device__ __forceinline__ float dpp_half_mirror(float v) {  // lane -> 7 - lane within each group of 8
     return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0x141, 0xF, 0xF, true));
 }
-// sum over the 8 lanes of a (column) group, as the balanced tree ((0+1)+(2+3)) + ((4+5)+(6+7))
+__device__ __forceinline__ float dpp_row_mirror(float v) {   // lane -> 15 - lane within each group of 16
+    return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0x140, 0xF, 0xF, true));
+}
+// sum over the HP lanes of a (column) group, as the balanced tree ((0+1)+(2+3)) + ((4+5)+(6+7)) [+ the same over 8..15]
+template <int HP>
 __device__ __forceinline__ float pair_tree_sum(float y) {
     y = y + dpp_quad_swap1(y);
     y = y + dpp_quad_swap2(y);
-    return y + dpp_half_mirror(y);
+    y = y + dpp_half_mirror(y);
+    if (HP == 16) y = y + dpp_row_mirror(y);
+    return y;
+}
+template <int HP>
+__device__ __forceinline__ float pair_tree_max(float f) {
+    f = sg_max(f, dpp_quad_swap1(f));
+    f = sg_max(f, dpp_quad_swap2(f));
+    f = sg_max(f, dpp_half_mirror(f));
+    if (HP == 16) f = sg_max(f, dpp_row_mirror(f));
+    return f;
 }
 
 // Composed coefficient triples (see sg2_compose.h), one thread per (direction, group, row).
-__global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
-    static_assert(DI == 16 && DS == 16, "k_compose: 16 rows per group");
-    const int dir = threadIdx.x / (SG2_COMP_GROUPS * 16), r = threadIdx.x % (SG2_COMP_GROUPS * 16);
-    const int group = r / 16, row = r % 16;
+template <class G>
+__global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan pl) {
+    const int dir = threadIdx.x / (SG2_COMP_GROUPS * G::ROWS), r = threadIdx.x % (SG2_COMP_GROUPS * G::ROWS);
+    const int group = r / G::ROWS, row = r % G::ROWS;
     const int b = dir ? W_B_INPROJ : W_F_INPROJ;
     float out[3];
-    sg2_compose_one(group, row, DM, DI, pl.W.w[W_IN_W], pl.W.w[W_IN_B], pl.W.w[b], pl.W.w[b + 1], pl.W.w[b + 2], pl.W.w[b + 3],
+    sg2_compose_one(group, row, G::DM, G::DI, pl.W.w[W_IN_W], pl.W.w[W_IN_B], pl.W.w[b], pl.W.w[b + 1], pl.W.w[b + 2], pl.W.w[b + 3],
                     pl.W.w[b + 4], out);
     float* dst = pl.comp + (size_t)threadIdx.x * 3;
     dst[0] = out[0];
@@ -104,15 +121,15 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * 16) void k_compose(Plan pl) {
     dst[2] = out[2];
 }
 
-// Projections of one timestep from the element's (g, s).  Each half of the workgroup produces its
-// half of dt / dt*x-branch / B (/ D*x-branch / C / gate).  HALF is a template parameter so that every row
-// index is a compile-time constant.  The coefficient triple of an output row sits in the four padding floats of the
+// Projections of one timestep from the element's (g, s).  Each wave of the workgroup produces its
+// share (rows PART*n/PARTS ...) of dt / dt*x-branch / B (/ D*x-branch / C / gate).  PART is a template parameter so that every row
+// index is a compile-time constant; a caller with many waves passes PART = 0 and array pointers moved to its wave's first row.  The coefficient triple of an output row sits in the four padding floats of the
 // LDS row it produces (staged once per workgroup, see stage_coefficients): one 16-byte broadcast read per output,
 // no scalar loads in the loop (a scalar load can only be waited for with lgkmcnt(0), which also drains the LDS queue).
 // Returns bit 0: every rotation angle of this timestep, over this half's columns, is small enough for
 // sg_sincos_small; bit 1: small enough for sg_sincos_tiny (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
-template <bool OUT, int HALF, bool HAS_S>
+template <class G, bool OUT, int PART, bool HAS_S>
 __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_dt, float* s_ux, float* s_dx, float* s_B,
                                              float* s_C, float* s_gate, const float* s_fmax) {
     // HAS_S is false for a tensor whose sharpness is all zero: fma(c_s, 0, c_0) is c_0 itself, so the term is skipped
@@ -120,8 +137,8 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
     auto coef = [&](const float* arr, int row) { return *reinterpret_cast<const f32x4*>(arr + row * LDS_STRIDE + SCAN_TT); };
     bool small = true, tiny = true;
 #pragma unroll
-    for (int q = 0; q < DI / 2; q++) {
-        const int jj = HALF * (DI / 2) + q;
+    for (int q = 0; q < G::DI / G::PARTS; q++) {
+        const int jj = PART * (G::DI / G::PARTS) + q;
         const float dtv = sg_softplus(eval(coef(s_dt, jj)));
         const float amax = dtv * s_fmax[jj];
         small = small && (amax < SG_SINCOS_SMALL_LIMIT);
@@ -133,15 +150,15 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
         if (OUT) s_dx[jj * LDS_STRIDE + tu] = cx[3] * xbv;
     }
 #pragma unroll
-    for (int q = 0; q < DS / 2; q++) {
-        const int ss = HALF * (DS / 2) + q;
+    for (int q = 0; q < G::DS / G::PARTS; q++) {
+        const int ss = PART * (G::DS / G::PARTS) + q;
         s_B[ss * LDS_STRIDE + tu] = eval(coef(s_B, ss));
         if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(coef(s_C, ss));
     }
     if (OUT) {
 #pragma unroll
-        for (int q = 0; q < DI / 2; q++) {
-            const int jj = HALF * (DI / 2) + q;
+        for (int q = 0; q < G::DI / G::PARTS; q++) {
+            const int jj = PART * (G::DI / G::PARTS) + q;
             s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(coef(s_gate, jj)));
         }
     }
@@ -149,15 +166,15 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
 }
 
 // Once per workgroup: the composed coefficient triples of this direction (and D) into the padding of the LDS rows.
-template <bool OUT>
+template <class G, bool OUT>
 __device__ __forceinline__ void stage_coefficients(const float* __restrict__ comp, const float* __restrict__ Dw, int tid, float* s_dt,
                                                    float* s_ux, float* s_B, float* s_C, float* s_gate) {
-    static_assert(DI == 16 && DS == 16 && SG2_COMP_GROUPS * 16 <= SCAN_THREADS, "one thread per (group, row)");
-    if (tid < SG2_COMP_GROUPS * 16) {
-        const int group = tid / 16, row = tid % 16;
+    static_assert(SG2_COMP_GROUPS * G::ROWS <= G::THREADS, "one thread per (group, row)");
+    if (tid < SG2_COMP_GROUPS * G::ROWS) {
+        const int group = tid / G::ROWS, row = tid % G::ROWS;
         float* arr = group == SG2_COMP_XB ? s_ux : group == SG2_COMP_DT ? s_dt : group == SG2_COMP_B ? s_B : group == SG2_COMP_C ? s_C : s_gate;
         if (OUT || (group != SG2_COMP_C && group != SG2_COMP_Z)) {
-            const float* t = comp + (group * 16 + row) * 3;
+            const float* t = comp + (group * G::ROWS + row) * 3;
             *reinterpret_cast<f32x4*>(arr + row * LDS_STRIDE + SCAN_TT) = f32x4{t[0], t[1], t[2], group == SG2_COMP_XB ? Dw[row] : 0.0f};
         }
     }
@@ -189,7 +206,7 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
 // ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny (its own values).
-template <bool OUT, int ANGLE>
+template <int HP, bool OUT, int ANGLE>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, float (&y)[UB]) {
@@ -219,13 +236,15 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
     if (OUT) {
 #pragma unroll
-        for (int u = 0; u < UB; u++) y[u] = pair_tree_sum(y[u]);
+        for (int u = 0; u < UB; u++) y[u] = pair_tree_sum<HP>(y[u]);
     }
 }
 
 // KEEP (bilevel pass, OUT only): also store the state entering every HT_STEP-th step for the adjoint kernels.
-template <bool OUT, bool KEEP = false>
-__global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
+template <class G, bool OUT, bool KEEP = false>
+__global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
+    constexpr int DM = G::DM, DS = G::DS, DI = G::DI, HP = G::HP, SCAN_THREADS = G::THREADS, PARTS = G::PARTS;
+    static_assert(!KEEP || PARTS == 2, "the bilevel pass exists for the default geometry only");
     __shared__ __attribute__((aligned(16))) float s_dt[DI * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) float s_ux[DI * LDS_STRIDE];       // dt * x-branch
     __shared__ __attribute__((aligned(16))) float s_B[DS * LDS_STRIDE];
@@ -236,8 +255,8 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     float* const s_y = s_dt;
     __shared__ float s_fmax[DI];
     __shared__ __attribute__((aligned(16))) float s_wout[OUT ? DM * DI : 4];      // out_proj of this direction
-    __shared__ unsigned long long s_large[2];      // per projection half: bit t set = timestep t of the tile needs the full sin/cos
-    __shared__ unsigned long long s_nottiny[2];    // ... bit t set = timestep t is not eligible for sg_sincos_tiny
+    __shared__ unsigned long long s_large[PARTS];      // per wave's share of the columns: bit t set = timestep t of the tile needs the full sin/cos
+    __shared__ unsigned long long s_nottiny[PARTS];    // ... bit t set = timestep t is not eligible for sg_sincos_tiny
 
     const int per_dir = OUT ? pl.chunks : pl.wchunks;
     const int dir = (int)blockIdx.x >= per_dir ? 1 : 0;
@@ -256,21 +275,18 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
 
     const int tid = threadIdx.x;
     const int tu = tid & (SCAN_TT - 1);                                   // projection role: timestep of the tile
-    const int half = __builtin_amdgcn_readfirstlane(tid >> 6);           // projection role: which half of the outputs
-    const int j = tid >> 3, p = tid & 7;                                  // scan role
+    const int half = __builtin_amdgcn_readfirstlane(tid >> 6);           // projection role: which share of the outputs (the wave)
+    const int j = tid / HP, p = tid % HP;                                 // scan role
 
     // -A/2 with A = -exp(A_log): the two poles of this lane's pair
     const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
     const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
     const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
 
-    {   // largest |frequency| of each column's 8 pairs
-        float f = sg_abs(freq);
-        f = sg_max(f, dpp_quad_swap1(f));
-        f = sg_max(f, dpp_quad_swap2(f));
-        f = sg_max(f, dpp_half_mirror(f));
+    {   // largest |frequency| of each column's pairs
+        const float f = pair_tree_max<HP>(sg_abs(freq));
         if (p == 0) s_fmax[j] = f;
-        stage_coefficients<OUT>(pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3), pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_B, s_C, s_gate);
+        stage_coefficients<G, OUT>(pl.comp + dir * (SG2_COMP_GROUPS * G::ROWS * 3), pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_B, s_C, s_gate);
         static_assert(DM * DI == SCAN_THREADS, "one out_proj entry per thread");
         if (OUT) s_wout[tid] = pl.W.w[dir ? W_B_OUT : W_F_OUT][tid];
         __syncthreads();
@@ -320,18 +336,29 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
         const float sh = valid ? shv : 0.0f;
         int angle_t;
-        if (has_s) {
-            if (half == 0)
-                angle_t = project_tile<OUT, 0, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-            else
-                angle_t = project_tile<OUT, 1, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+        if (PARTS == 2) {
+            if (has_s) {
+                if (half == 0)
+                    angle_t = project_tile<G, OUT, 0, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                else
+                    angle_t = project_tile<G, OUT, 1, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+            } else {
+                if (half == 0)
+                    angle_t = project_tile<G, OUT, 0, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                else
+                    angle_t = project_tile<G, OUT, 1, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+            }
         } else {
-            if (half == 0)
-                angle_t = project_tile<OUT, 0, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+            // many waves: one copy of the code, the arrays moved to this wave's first row
+            const int rj = half * (DI / PARTS) * LDS_STRIDE, rs = half * (DS / PARTS) * LDS_STRIDE;
+            if (has_s)
+                angle_t = project_tile<G, OUT, 0, true>(g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0),
+                                                        s_gate + (OUT ? rj : 0), s_fmax + half * (DI / PARTS));
             else
-                angle_t = project_tile<OUT, 1, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
+                angle_t = project_tile<G, OUT, 0, false>(g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0),
+                                                         s_gate + (OUT ? rj : 0), s_fmax + half * (DI / PARTS));
         }
-        {   // half h projects the dt of columns 8h..8h+7, which are the columns wave h owns in the recurrence
+        {   // wave w projects the dt of columns w*64/HP .. (w+1)*64/HP-1, which are the columns it owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!(angle_t & 1));
             const unsigned long long nottiny = __builtin_amdgcn_ballot_w64(!(angle_t & 2));
             if (tu == 0) { s_large[half] = large; s_nottiny[half] = nottiny; }
@@ -370,11 +397,11 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             }
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
             if ((nottiny & blk) == 0)
-                block_steps<OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             else if ((large & blk) == 0)
-                block_steps<OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             else
-                block_steps<OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
             if (OUT && p == 0) {
 #pragma unroll
                 for (int q = 0; q < UB; q += 4)
@@ -389,7 +416,7 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             sg_sincos(dt * freq, &sn, &cs);
             step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             if (OUT) {
-                const float y = pair_tree_sum(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
+                const float y = pair_tree_sum<HP>(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
                 if (p == 0) s_y[j * LDS_STRIDE + k0] = y;
             }
         }
@@ -401,11 +428,12 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
 #pragma unroll
             for (int jj = 0; jj < DI; jj++)
                 o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], s_gate[jj * LDS_STRIDE + tu], s_dx[jj * LDS_STRIDE + tu]);
-            float cx[DM / 2];
+            constexpr int CPP = DM / PARTS;     // context entries this wave produces per timestep
+            float cx[CPP];
 #pragma unroll
-            for (int q = 0; q < DM / 2; q++) {
-                // row (DM/2) * half + q of out_proj: the same address for every lane of the wave (broadcast reads)
-                const float* wr = s_wout + (half * (DM / 2) + q) * DI;
+            for (int q = 0; q < CPP; q++) {
+                // row CPP * half + q of out_proj: the same address for every lane of the wave (broadcast reads)
+                const float* wr = s_wout + (half * CPP + q) * DI;
                 float a = 0.0f;
 #pragma unroll
                 for (int m = 0; m < DI; m += 4) {
@@ -418,13 +446,19 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                 cx[q] = a;
             }
             if (valid) {
-                float4* dst = reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM) + half;
-                *dst = make_float4(cx[0], cx[1], cx[2], cx[3]);
-                if (KEEP && pl.scan_out[dir] != nullptr) {
-                    // the gated scan output itself (before out_proj), at the step's position in scan order; this half's 8 columns
-                    float4* so = reinterpret_cast<float4*>(pl.scan_out[dir] + ((size_t)off + tile0 + tu) * DI) + 2 * half;
-                    so[0] = half ? make_float4(o[8], o[9], o[10], o[11]) : make_float4(o[0], o[1], o[2], o[3]);
-                    so[1] = half ? make_float4(o[12], o[13], o[14], o[15]) : make_float4(o[4], o[5], o[6], o[7]);
+                float* dst = pl.ctx + ((size_t)dir * pl.total + off + orig) * DM + half * CPP;
+                static_assert(CPP == 4 || CPP == 2, "one vector store per lane");
+                if constexpr (CPP == 4)
+                    *reinterpret_cast<float4*>(dst) = make_float4(cx[0], cx[1], cx[2], cx[3]);
+                else
+                    *reinterpret_cast<float2*>(dst) = make_float2(cx[0], cx[1]);
+                if constexpr (KEEP) {
+                    if (pl.scan_out[dir] != nullptr) {
+                        // the gated scan output itself (before out_proj), at the step's position in scan order; this half's 8 columns
+                        float4* so = reinterpret_cast<float4*>(pl.scan_out[dir] + ((size_t)off + tile0 + tu) * DI) + 2 * half;
+                        so[0] = half ? make_float4(o[8], o[9], o[10], o[11]) : make_float4(o[0], o[1], o[2], o[3]);
+                        so[1] = half ? make_float4(o[12], o[13], o[14], o[15]) : make_float4(o[4], o[5], o[6], o[7]);
+                    }
                 }
             }
             __syncthreads();
@@ -475,20 +509,23 @@ __global__ __launch_bounds__(SCAN_THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
 // Start state of every chunk: h_{c+1} = M_c h_c + b_c, applied in order from
 // the carried state of the tensor.  One workgroup per (tensor, direction).
 // The recurrence itself is a handful of fmas per chunk; what matters is the
-// latency of fetching 3 KB of summaries per chunk, so eight 128-lane groups
-// stream batches of 32 chunks into LDS (next batch prefetched into registers)
-// and group 0 applies them.
-constexpr int PREFIX_GROUPS = 8;
-constexpr int PREFIX_BATCH = 32;
-constexpr int PREFIX_PER_GROUP = PREFIX_BATCH / PREFIX_GROUPS;
+// latency of fetching 3 KB (12 KB for the large geometry) of summaries per chunk,
+// so the 1024 lanes of the workgroup, as groups of one chunk's lanes each, stream
+// batches of chunks into LDS (next batch prefetched into registers) and group 0
+// applies them.
+constexpr int PREFIX_PER_GROUP = 4;
 
-__global__ __launch_bounds__(PREFIX_GROUPS * SCAN_THREADS) void k_chunk_prefix(Plan pl) {
+template <class G>
+__global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
+    constexpr int DS = G::DS, HP = G::HP, SCAN_THREADS = G::THREADS;
+    constexpr int PREFIX_GROUPS = 1024 / SCAN_THREADS;             // 8 groups of 128 lanes, or 2 of 512
+    constexpr int PREFIX_BATCH = PREFIX_PER_GROUP * PREFIX_GROUPS;
     __shared__ float lds[PREFIX_BATCH * 6 * SCAN_THREADS];     // 96 KB
     const int ti = blockIdx.x % pl.P, dir = blockIdx.x / pl.P;
     const TensorDev& T = pl.tensors[ti];
     if (T.numel == 0) return;
     const int lane = threadIdx.x % SCAN_THREADS, grp = threadIdx.x / SCAN_THREADS;
-    const int j = lane >> 3, p = lane & 7;
+    const int j = lane / HP, p = lane % HP;
     float* __restrict__ hs = pl.hstart + ((size_t)(dir * pl.chunks + pl.chunk_prefix[ti]) * 2) * SCAN_THREADS;
     const float* __restrict__ sm = pl.summaries + (size_t)(dir * pl.wchunks + pl.wchunk_prefix[ti]) * 6 * SCAN_THREADS;
     const int ns = T.nchunks - 1;                               // summaries to apply
@@ -534,27 +571,38 @@ __global__ __launch_bounds__(PREFIX_GROUPS * SCAN_THREADS) void k_chunk_prefix(P
     }
 }
 
+template <class G>
+int launch_scan_geo(const Plan& pl, hipStream_t st) {
+    hipLaunchKernelGGL(k_compose<G>, dim3(1), dim3(2 * SG2_COMP_GROUPS * G::ROWS), 0, st, pl);
+    SG_LAUNCH_CHECK("k_compose");
+    if (pl.wchunks > 0) {
+        hipLaunchKernelGGL((k_scan<G, false, false>), dim3(2 * pl.wchunks), dim3(G::THREADS), 0, st, pl);
+        SG_LAUNCH_CHECK("k_scan<summary>");
+    }
+    prof_mark(2, st);
+    hipLaunchKernelGGL(k_chunk_prefix<G>, dim3(2 * pl.P), dim3(1024), 0, st, pl);
+    SG_LAUNCH_CHECK("k_chunk_prefix");
+    prof_mark(3, st);
+    if constexpr (G::PARTS == 2) {
+        if (pl.htile != nullptr) {
+            hipLaunchKernelGGL((k_scan<G, true, true>), dim3(2 * pl.chunks), dim3(G::THREADS), 0, st, pl);
+            SG_LAUNCH_CHECK("k_scan<out, keep>");
+            prof_mark(4, st);
+            return 0;
+        }
+    }
+    if (pl.htile != nullptr) return sg::fail("the bilevel pass is built for the default meta-net dimensions only");
+    hipLaunchKernelGGL((k_scan<G, true, false>), dim3(2 * pl.chunks), dim3(G::THREADS), 0, st, pl);
+    SG_LAUNCH_CHECK("k_scan<out>");
+    prof_mark(4, st);
+    return 0;
+}
+
 }  // namespace
 
 int launch_scan(const Plan& pl, hipStream_t st) {
     if (pl.total == 0) return 0;
-    hipLaunchKernelGGL(k_compose, dim3(1), dim3(2 * SG2_COMP_GROUPS * 16), 0, st, pl);
-    SG_LAUNCH_CHECK("k_compose");
-    if (pl.wchunks > 0) {
-        hipLaunchKernelGGL((k_scan<false, false>), dim3(2 * pl.wchunks), dim3(SCAN_THREADS), 0, st, pl);
-        SG_LAUNCH_CHECK("k_scan<summary>");
-    }
-    prof_mark(2, st);
-    hipLaunchKernelGGL(k_chunk_prefix, dim3(2 * pl.P), dim3(PREFIX_GROUPS * SCAN_THREADS), 0, st, pl);
-    SG_LAUNCH_CHECK("k_chunk_prefix");
-    prof_mark(3, st);
-    if (pl.htile != nullptr)
-        hipLaunchKernelGGL((k_scan<true, true>), dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
-    else
-        hipLaunchKernelGGL((k_scan<true, false>), dim3(2 * pl.chunks), dim3(SCAN_THREADS), 0, st, pl);
-    SG_LAUNCH_CHECK("k_scan<out>");
-    prof_mark(4, st);
-    return 0;
+    return pl.geo == GEO_LARGE ? launch_scan_geo<GeoLarge>(pl, st) : launch_scan_geo<GeoDefault>(pl, st);
 }
 
 }  // namespace sg2

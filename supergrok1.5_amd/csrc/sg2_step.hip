@@ -66,7 +66,8 @@ struct Layout {
     size_t tables_bytes;
 };
 
-int make_layout(int P, Numels numels, int chunk_len, Layout* L, bool bilevel = false) {
+int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bilevel = false) {
+    const GeoInfo gi = geo_info(geo);
     int64_t total = 0, et = 0, stl = 0, ch = 0, wch = 0;
     for (int i = 0; i < P; i++) {
         const int64_t n = numels[i];
@@ -92,11 +93,11 @@ int make_layout(int P, Numels numels, int chunk_len, Layout* L, bool bilevel = f
     L->off_ssorted = take(4 * (size_t)total);
     L->off_spine = take(4 * 256 * (size_t)stl);
     L->off_blocksums = take(4 * (size_t)(L->nb + 1));
-    L->off_summ = take(4 * 2 * (size_t)wch * 6 * SCAN_THREADS);
-    L->off_hstart = take(4 * 2 * (size_t)ch * 2 * SCAN_THREADS);
-    L->off_comp = take(4 * 2 * 5 * 16 * 3);
+    L->off_summ = take(4 * 2 * (size_t)wch * 6 * gi.threads);
+    L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
+    L->off_comp = take(4 * 2 * 5 * (size_t)gi.rows * 3);
     L->off_flags = take(4 * (size_t)P);        // apart from the tensor records: it is written while those are being read
-    L->off_ctx = take(4 * 2 * (size_t)total * DM);
+    L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions
     L->off_htile = take(bilevel ? 4 * 2 * (size_t)htile_count((int)total, P) * 2 * SCAN_THREADS : 0);
     L->off_adj_summ = take(bilevel ? 4 * 2 * (size_t)L->chunks * SCAN_THREADS * 6 : 0);
@@ -137,21 +138,32 @@ __global__ __launch_bounds__(256) void k_tables(TableChunk c) {
 
 }  // namespace
 
-int check_dims(const SgDims* d) {
-    if (!d) return sg::fail("dims is NULL");
+int geo_of(const SgDims* d) {
+    if (!d) return sg::fail("dims is NULL"), -1;
     // the limits the reference enforces (csrc/supergrok2_mamba_peer_kernels.cu:1796-1801)
-    if (d->d_state % 2) return sg::fail("d_state must be even for paired RoPE (got %d)", d->d_state);
-    if (d->d_state > 32) return sg::fail("d_state exceeds MAX_D_STATE (%d > 32)", d->d_state);
-    if (d->d_model > 16) return sg::fail("d_model exceeds MAX_D_MODEL (%d > 16)", d->d_model);
-    if (d->gru_hidden > 8) return sg::fail("gru_hidden exceeds MAX_GRU_HIDDEN (%d > 8)", d->gru_hidden);
-    if (d->d_inner > 32) return sg::fail("d_inner exceeds MAX_D_INNER (%d > 32)", d->d_inner);
-    if (d->d_inner % 4) return sg::fail("d_inner must be a multiple of 4 (got %d)", d->d_inner);
-    // the specialisation these kernels are compiled for
-    if (d->d_model != DM || d->d_state != DS || d->d_inner != DI || d->gru_hidden != GH || d->num_heads != NH ||
-        d->pk_dim != PK || d->expert_hidden != EH || d->num_experts != NE)
-        return sg::fail("unsupported meta-net dims: kernels are built for d_model=%d d_state=%d d_inner=%d "
-                        "gru_hidden=%d heads=%d pk_dim=%d expert_hidden=%d experts=%d",
-                        DM, DS, DI, GH, NH, PK, EH, NE);
+    if (d->d_state % 2) return sg::fail("d_state must be even for paired RoPE (got %d)", d->d_state), -1;
+    if (d->d_state > 32) return sg::fail("d_state exceeds MAX_D_STATE (%d > 32)", d->d_state), -1;
+    if (d->d_model > 16) return sg::fail("d_model exceeds MAX_D_MODEL (%d > 16)", d->d_model), -1;
+    if (d->gru_hidden > 8) return sg::fail("gru_hidden exceeds MAX_GRU_HIDDEN (%d > 8)", d->gru_hidden), -1;
+    if (d->d_inner > 32) return sg::fail("d_inner exceeds MAX_D_INNER (%d > 32)", d->d_inner), -1;
+    if (d->d_inner % 4) return sg::fail("d_inner must be a multiple of 4 (got %d)", d->d_inner), -1;
+    // the geometries these kernels are compiled for
+    if (d->gru_hidden == GH && d->num_heads == NH && d->pk_dim == PK && d->expert_hidden == EH && d->num_experts == NE)
+        for (int geo = 0; geo < GEO_COUNT; geo++) {
+            const GeoInfo gi = geo_info(geo);
+            if (d->d_model == gi.dm && d->d_state == gi.ds && d->d_inner == gi.di) return geo;
+        }
+    sg::fail("unsupported meta-net dims: kernels are built for (d_model, d_state, d_inner) = (%d, %d, %d) or (%d, %d, %d), with "
+             "gru_hidden=%d heads=%d pk_dim=%d expert_hidden=%d experts=%d",
+             GeoDefault::DM, GeoDefault::DS, GeoDefault::DI, GeoLarge::DM, GeoLarge::DS, GeoLarge::DI, GH, NH, PK, EH, NE);
+    return -1;
+}
+
+int check_dims(const SgDims* d) {
+    const int geo = geo_of(d);
+    if (geo < 0) return 1;
+    if (geo != GEO_DEFAULT)
+        return sg::fail("the bilevel pass is built for d_model=%d d_state=%d d_inner=%d only", GeoDefault::DM, GeoDefault::DS, GeoDefault::DI);
     return 0;
 }
 
@@ -218,9 +230,10 @@ int sg2_set_scan_window(int window) {
 int sg2_get_scan_window(void) { return sg2::g_window.load(); }
 
 size_t sg2_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
-    if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
+    const int geo = sg2::geo_of(dims);
+    if (geo < 0 || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;
-    if (sg2::make_layout(num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L)) return 0;
+    if (sg2::make_layout(geo, num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L)) return 0;
     return L.bytes;
 }
 
@@ -236,7 +249,9 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     Plan& pl = *plp;
     Layout& L = *Lp;
     pl.total = 0;
-    if (check_dims(dims)) return 1;
+    const int geo = geo_of(dims);
+    if (geo < 0 || (bilevel && check_dims(dims))) return 1;
+    pl.geo = geo;
     if (num_tensors == 0) return 0;
     if (num_tensors < 0 || !tensors || !weights || !scalars) return sg::fail("NULL argument");
     for (int k = 0; k < SG2_NUM_WEIGHTS; k++)
@@ -254,7 +269,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
         }
     }
     const int chunk_len = chunk_override > 0 ? chunk_override : effective_chunk_len(P, numels);
-    if (make_layout(P, numels, chunk_len, &L, bilevel)) return 1;
+    if (make_layout(geo, P, numels, chunk_len, &L, bilevel)) return 1;
     if (L.total == 0) return 0;
     if (!workspace || workspace_bytes < L.bytes)
         return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, workspace_bytes);
@@ -340,7 +355,7 @@ int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, con
     prof_mark(1, st);
     if (launch_scan(pl, st)) return 1;
     if (debug && debug->ctx)
-        SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * DM, hipMemcpyDeviceToDevice, st));
+        SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * geo_info(pl.geo).dm, hipMemcpyDeviceToDevice, st));
     if (launch_elem(pl, expert_counts, debug ? debug->expert_idx : nullptr, st)) return 1;
     prof_mark(5, st);
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;
@@ -384,11 +399,12 @@ size_t sg2_static_scratch_bytes(void) { return SG2_STATIC_SCRATCH_BYTES; }
 int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
                             const Sg2Scalars* scalars, int32_t* expert_counts, const Sg2Debug* debug, void* stream) {
     using namespace sg2;
-    if (check_dims(dims)) return 1;
+    const int geo = geo_of(dims);
+    if (geo < 0) return 1;
     if (num_tensors < 0 || (num_tensors > 0 && !tensors)) return sg::fail("NULL argument");
     Layout L;
     const Numels numels = {nullptr, tensors};
-    if (make_layout(num_tensors, numels, effective_chunk_len(num_tensors, numels), &L)) return 1;
+    if (make_layout(geo, num_tensors, numels, effective_chunk_len(num_tensors, numels), &L)) return 1;
     if (L.bytes > SG2_STATIC_SCRATCH_BYTES)
         return sg::fail("sg2_batched_step_static: these tensors need %zu bytes of scratch, the library's static buffer holds %zu "
                         "(about 700 000 elements per call); use sg2_batched_step with a caller-provided workspace",
@@ -402,7 +418,7 @@ int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int n
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;
-    if (sg2::make_layout(num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L, true)) return 0;
+    if (sg2::make_layout(sg2::GEO_DEFAULT, num_tensors, sg2::Numels{numels, nullptr}, sg2::effective_chunk_len(num_tensors, sg2::Numels{numels, nullptr}), &L, true)) return 0;
     return L.bytes;
 }
 

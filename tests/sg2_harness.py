@@ -24,14 +24,15 @@ class Sg2Case:
     """A list of parameter tensors with full optimizer state, mirrored on CPU
     (numpy, for the checker) and on the GPU (torch, for the C ABI)."""
 
-    def __init__(self, shapes, dtypes=None, seed=0, weights=None, random_state=False, device="cuda"):
+    def __init__(self, shapes, dtypes=None, seed=0, weights=None, random_state=False, device="cuda", dims=None):
         from grokking_optimizers import _cabi
         self.shapes = shapes
         self.P = len(shapes)
         self.dtypes = dtypes or [torch.float32] * self.P
-        self.W = weights if weights is not None else wl.meta_weights(7)
+        self.dims = dict(DIMS if dims is None else dims)
+        self.W = weights if weights is not None else wl.meta_weights(7, self.dims)
         params = wl.make_params(shapes, seed=seed)
-        gh, di, ds = DIMS["gru_hidden"], DIMS["d_inner"], DIMS["d_state"]
+        gh, di, ds = self.dims["gru_hidden"], self.dims["d_inner"], self.dims["d_state"]
         gen = torch.Generator().manual_seed(seed + 1000)
         self.cpu = []
         for p, dt in zip(params, self.dtypes):
@@ -49,15 +50,15 @@ class Sg2Case:
         keys = ("param", "exp_avg", "exp_avg_sq", "mu", "gru", "mamba_fwd", "mamba_bwd")
         self.gpu = [{k: st[k].to(device) for k in keys} for st in self.cpu]
         self.np = [dict({k: to_np(st[k]) for k in keys}, dtype=NAME_OF[dt]) for st, dt in zip(self.cpu, self.dtypes)]
-        self.counts_gpu = torch.zeros(DIMS["num_experts"], dtype=torch.int32, device=device)
-        self.counts_np = np.zeros(DIMS["num_experts"], np.int32)
+        self.counts_gpu = torch.zeros(self.dims["num_experts"], dtype=torch.int32, device=device)
+        self.counts_np = np.zeros(self.dims["num_experts"], np.int32)
         self.Wgpu = [w.to(device) for w in self.W]
         self.Wnp = [w.numpy() for w in self.W]
         g = self.gpu
         self.step_fn = _cabi.Sg2Step(self.Wgpu, [s["param"] for s in g], [s["exp_avg"] for s in g],
                                      [s["exp_avg_sq"] for s in g], [s["mu"] for s in g], [s["gru"] for s in g],
                                      [s["mamba_fwd"] for s in g], [s["mamba_bwd"] for s in g], self.counts_gpu,
-                                     debug=True)
+                                     dims=self.dims, debug=True)
         self.offsets = np.concatenate([[0], np.cumsum([wl.numel(s) for s in shapes])]).astype(np.int64)
 
     def gpu_step(self, grads, sharps, per_tensor, shared):
@@ -83,7 +84,7 @@ class Sg2Case:
             s = to_np(sharps[i].reshape(-1).to(self.dtypes[i]))
             if self.np[i]["exp_avg"].size == 0:
                 return
-            dbg[i] = orc.sg2_step(self.Wnp, self.np[i], g, s, sc, precision=precision, chunk_len=chunk_len, window=window,
+            dbg[i] = orc.sg2_step(self.Wnp, self.np[i], g, s, sc, dims=self.dims, precision=precision, chunk_len=chunk_len, window=window,
                                   expert_counts=counts[i], debug=True)
         with ThreadPoolExecutor(threads) as ex:
             list(ex.map(one, range(self.P)))
