@@ -285,8 +285,8 @@ def bench_probe(dev):
     ws = torch.empty(L.sg_probe_workspace_bytes(cus, 8), dtype=torch.uint8, device=dev)
     rows, best = [], 0.0
     for ncu in (cus,):
-        for op, name in enumerate(("fma", "mul", "add", "add_dpp")):
-            for w in (1, 2, 3, 4, 8):
+        for op, name in enumerate(("fma", "mul", "add", "add_dpp", "mfma_32x32x16_bf16", "mfma_32x32x16_bf16_random_operands")):
+            for w in ((1, 2) if op >= 4 else (1, 2, 3, 4, 8)):
                 ms, ticks, instr = C.c_float(), C.c_double(), C.c_double()
                 if L.sg_probe_valu(op, ncu, w, 2000, C.byref(ms), C.byref(ticks), C.byref(instr), ws.data_ptr(), ws.numel(),
                                    torch.cuda.current_stream().cuda_stream) != 0:
@@ -296,7 +296,9 @@ def bench_probe(dev):
                              "instr_per_ns_per_simd": round(rate, 4),
                              "clock_ticks_per_instr_per_simd": round(ticks.value / instr.value / w, 3),
                              "clock_ticks_per_ns": round(ticks.value / (ms.value * 1e6), 3)})
-                if ncu == cus:
+                if op >= 4:      # 32768 flop per instruction and SIMD
+                    rows[-1]["chip_tflops"] = round(rate * 32768 * 4 * ncu / 1e3, 1)
+                elif ncu == cus:
                     best = max(best, rate)
     return {"metric": "secondary: valu-probe", "value": best, "unit": "wave64 instructions/ns/SIMD (whole chip, best case)",
             "n_gpus": 1, "steps": 1, "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",

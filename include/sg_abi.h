@@ -148,7 +148,9 @@ int sg2_profile_read(float* ms, int* calls);
 /* Issue-rate probe of the fp32 vector ALU (measurement aid, no counterpart in
  * the reference): `iters` x 128 independent wave64 instructions of one kind
  * per wave (op 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_add_f32 with a DPP
- * operand; plain, not packed) on num_cus x waves_per_simd workgroups of four
+ * operand; plain, not packed; 4 v_mfma_f32_32x32x16_bf16 on constant register
+ * operands, 5 the same on pseudo-random operands: the matrix cores' own
+ * ceiling and what real data makes of it through the power limit) on num_cus x waves_per_simd workgroups of four
  * waves, i.e. waves_per_simd waves on every SIMD of num_cus compute units
  * when the dispatcher spreads them evenly.  Synchronises the stream.  Returns
  * the elapsed milliseconds of the launch, the shader-clock ticks a wave took

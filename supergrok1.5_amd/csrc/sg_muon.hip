@@ -9,19 +9,22 @@
 //     G = Y Y^T            H = b G + c G G            Y <- a Y + H Y
 // (for a tall parameter X this is X^T X and X (bG + cG^2): the reference's
 // X X^T form re-associated, 6 m^2 n instead of 6 n^2 m flops per iteration).
-// All three products are "NT" GEMMs (both operands K-contiguous) once the
-// transpose Y^T is kept next to Y; the apply step's epilogue writes the new Y
-// and, into the other of two Y^T buffers, its transpose (the current Y^T is
-// still being read as the B operand by other workgroups).  An LDS transpose
-// kernel is only needed once, after normalisation.  Work buffers are
-// zero-padded to multiples of
-// 256 so the GEMM needs no edge handling (zero rows/columns stay zero through
-// the iteration).
+// The Gram and polynomial products are "NT" GEMMs (both operands K-contiguous).
+// The apply step is an "NN" one: its B operand is Y itself, whose K axis is
+// the slow one.  Its tiles are staged in LDS as they lie in memory
+// ([k][n], n contiguous) and the MFMA operand (8 consecutive k per lane) is
+// fetched with gfx950's transposing LDS read (ds_read_b64_tr_b16), so no
+// transposed copy of Y is kept: an iteration reads Y twice and writes it once,
+// into the other of two buffers (the current one is still being read as the B
+// operand by other workgroups).  Only the last iteration of a tall parameter
+// also stores the transposed tile, which is the parameter's own orientation.
+// Work buffers are zero-padded to multiples of 256 so the GEMM needs no edge
+// handling (zero rows/columns stay zero through the iteration).
 //
 // GEMM: 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each
 // wave 128x128 = 4x4 MFMA 32x32x16 bf16 tiles (256 fp32 accumulators per
-// lane), K tiles of 64 staged through LDS with 144-byte row stride
-// (conflict-free 16-byte operand fetches, two stages), the tiles of the next
+// lane), K tiles of 64 staged through LDS with 144-byte row stride (576 bytes for
+// the [k][n] tiles; conflict-free operand fetches, two stages), the tiles of the next
 // K steps in flight in two register sets while the current one is multiplied,
 // memory instructions dealt between the MFMAs.  256x256x64 gives 128 flop per byte
 // fetched, which keeps the MFMA pipe ahead of the ~64 B/clk a CU can pull from
@@ -43,7 +46,9 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int BT = 256;            // GEMM tile (M and N)
 constexpr int BK = 64;             // GEMM K tile
-constexpr int LDS_ROW = BK + 8;    // bf16 elements per LDS row (144 bytes)
+constexpr int LDS_ROW = BK + 8;    // bf16 elements per LDS row (144 bytes) of a K-contiguous tile [BT][BK]
+constexpr int LDS_ROW_KN = BT + 32; // ... of a [BK][BT] tile (576 bytes: four rows start 16 banks apart)
+static_assert(BK * LDS_ROW_KN == BT * LDS_ROW, "both tile layouts fill the same LDS");
 constexpr int GEMM_LDS_BYTES = 2 * 2 * BT * LDS_ROW * 2;   // two stages of {A tile, B tile}: 147,456 bytes of the CU's 160 KB
 static_assert(BK == 64, "the K loop of k_gemm_nt is written for four 16-wide steps");
 constexpr int ETILE = 4096;        // elements per tile of the elementwise kernels
@@ -53,8 +58,8 @@ struct Mat {
     void* param;
     const void* grad;
     float* buf;
-    bf16_t *Y, *YT, *G, *H;       // [mp x np], [np x mp], [mp x mp], [mp x mp]
-    bf16_t* YT2;                   // second [np x mp] buffer: the apply step reads one transposed copy and writes the other
+    bf16_t *Y, *Y2, *G, *H;       // [mp x np] twice (an iteration reads one and writes the other), [mp x mp], [mp x mp]
+    bf16_t* YT;                    // [np x mp]: the final X of a tall parameter in its own orientation
     int rows, cols, dtype;
     int m, n, mp, np;              // min / max dim and their padded sizes
     int wide;                      // rows <= cols
@@ -160,11 +165,11 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
     if (threadIdx.x == 0) B.inv_norm[mi] = 1.0f / ((float)sqrt(tot) + 1e-7f);
 }
 
-// X = buf * inv_norm as bf16, written in both orientations at once: Y ([mp x np], the wide orientation) and its
-// transpose YT ([np x mp]).  One 64x64 tile of the parameter's own orientation per workgroup: rows are read and
-// written along the fast axis, the transposed copy goes through LDS.  The zero padding of both buffers is written
+// X = buf * inv_norm as bf16 into Y ([mp x np], the wide orientation); with `both` a tall matrix also gets YT
+// ([np x mp], its own orientation; needed when no iteration follows).  One 64x64 tile of the parameter's own orientation per workgroup: rows are read and
+// written along the fast axis, a transposed copy goes through LDS.  The zero padding of the buffers is written
 // here as well.
-__global__ __launch_bounds__(256) void k_normalize(Batch B) {
+__global__ __launch_bounds__(256) void k_normalize(Batch B, int both) {
     __shared__ bf16_t t[64][66];
     const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
@@ -174,6 +179,7 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
     const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
     const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
     const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
+    const bool w_own = M.wide || both, w_other = !M.wide;       // uniform over the workgroup (YT exists for tall matrices only)
     const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && (M.cols & 3) == 0 && (((uintptr_t)M.buf) & 15u) == 0;
     if (full) {
         // interior tile: a lane moves 16 consecutive elements of a row (four 16-byte loads, two 16-byte stores)
@@ -190,9 +196,12 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
             t[lr][c0 + 4 * q] = (bf16_t)b0; t[lr][c0 + 4 * q + 1] = (bf16_t)b1;
             t[lr][c0 + 4 * q + 2] = (bf16_t)b2; t[lr][c0 + 4 * q + 3] = (bf16_t)b3;
         }
-        uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
-        dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-        dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        if (w_own) {
+            uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        }
+        if (!w_other) return;
         __syncthreads();
         // transposed copy: output row lr (= own column), 16 consecutive output columns (= own rows)
 #pragma unroll
@@ -205,9 +214,10 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
     for (int k = threadIdx.x; k < 64 * 64; k += 256) {
         const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
         const bf16_t v = (r < M.rows && c < M.cols) ? sg::f_to_bf16_bits(M.buf[(size_t)r * M.cols + c] * inv) : (bf16_t)0;
-        own[(size_t)r * C + c] = v;
+        if (w_own) own[(size_t)r * C + c] = v;
         t[k >> 6][k & 63] = v;
     }
+    if (!w_other) return;
     __syncthreads();
     for (int k = threadIdx.x; k < 64 * 64; k += 256) {
         const int r = k >> 6, c = k & 63;     // output row r (= own column), column c (= own row)
@@ -215,7 +225,7 @@ __global__ __launch_bounds__(256) void k_normalize(Batch B) {
     }
 }
 
-// ---- NT GEMM  C[M x N] = A[M x K] * B[N x K]^T  with fused epilogues ---------------
+// ---- GEMM  C[M x N] = A[M x K] * B  with fused epilogues; B given as [N x K] (Gram, polynomial) or as [K x N] (apply)
 // 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
 // 32x32x16 tiles (256 fp32 accumulators per lane; one wave per SIMD, the whole register file).
 // Per 16-wide k step a wave fetches 4+4 16-byte operands from LDS for 16 MFMAs.  The next K tile
@@ -226,15 +236,41 @@ enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
 // explicit global address space: a generic (flat) load would count against the LDS wait counter as well
 typedef const __attribute__((address_space(1))) u32x4* gvec_p;
 
-__device__ __forceinline__ uint32_t bf16r(float v) {   // round to nearest even, NaN kept quiet; no branches
-    const uint32_t u = (uint32_t)sg_f2i(v);
-    const uint32_t rne = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-    const uint32_t nan = (u >> 16) | 0x40u;
-    return ((u & 0x7fffffffu) > 0x7f800000u) ? nan : rne;
+// two floats rounded to bf16 (nearest even, NaN stays NaN), packed lo | hi << 16: one v_cvt_pk_bf16_f32 on gfx950
+__device__ __forceinline__ uint32_t bf16r2(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
 }
 
+// the first eight MFMAs of a phase, each followed by one LDS read of the next k step (the [K x N] operand takes twelve
+// reads per k step: two after each of the first four)
+#define SG_MUON_SCHED_READS()                                                  \
+    do {                                                                       \
+        if (BKN) {                                                             \
+            _Pragma("unroll") for (int g_ = 0; g_ < 4; g_++) {                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
+                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);             \
+            }                                                                  \
+            _Pragma("unroll") for (int g_ = 0; g_ < 4; g_++) {                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             \
+            }                                                                  \
+        } else {                                                               \
+            _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                 \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             \
+            }                                                                  \
+        }                                                                      \
+    } while (0)
+
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4* lds_i16x4_p;
+
+// y_sel: which of the two Y buffers holds the current iterate
 template <int EPI>
-__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_iter) {
+__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int last_iter) {
+    constexpr bool BKN = EPI == EPI_APPLY;             // B operand stored [K x N]
     constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
     constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
     // LDS: two stages of {A tile, B tile}, each tile BT rows of LDS_ROW elements
@@ -257,8 +293,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
     bf16_t *C, *CT;         // CT: where the transposed tile goes (the symmetric products mirror into C itself)
     int K, lda, ldb, ldc, ldct, tm, tn;
     if (EPI == EPI_APPLY) {
-        A = Mt.H; B = yt_sel ? Mt.YT2 : Mt.YT; C = Mt.Y; K = Mt.mp; lda = ldb = Mt.mp; ldc = Mt.np;
-        CT = yt_sel ? Mt.YT : Mt.YT2; ldct = Mt.mp;
+        A = Mt.H; B = y_sel ? Mt.Y2 : Mt.Y; C = y_sel ? Mt.Y : Mt.Y2; K = Mt.mp; lda = Mt.mp; ldb = ldc = Mt.np;
+        CT = Mt.YT; ldct = Mt.mp;
         // bands of 8 tile columns: 32 tiles that run together span 4 x 8 tiles instead of 2 x 16,
         // which halves the panel bytes they pull into L2
         const int ntm = Mt.mp / BT, ntn = Mt.np / BT;
@@ -271,7 +307,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
             tn = tile % ntn;
         }
     } else {
-        if (EPI == EPI_GRAM) { A = Mt.Y; B = Mt.Y; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; }
+        if (EPI == EPI_GRAM) { A = y_sel ? Mt.Y2 : Mt.Y; B = A; C = Mt.G; K = Mt.np; lda = ldb = Mt.np; ldc = Mt.mp; }
         else { A = Mt.G; B = Mt.G; C = Mt.H; K = Mt.mp; lda = ldb = ldc = Mt.mp; }
         CT = C; ldct = ldc;
         const int nt = Mt.mp / BT;      // upper-triangular enumeration: row tm holds nt - tm tiles
@@ -280,7 +316,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
         tn = tm + tile;
     }
     A += (size_t)tm * BT * lda;
-    B += (size_t)tn * BT * ldb;
+    B += BKN ? (size_t)tn * BT : (size_t)tn * BT * ldb;
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -296,17 +332,19 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
     // A load has two K tiles of MFMA work (~4000 cycles) to arrive.  One barrier per K tile.
     u32x4 ra[2][CH], rb[2][CH];
     const uint32_t voff_a = (uint32_t)(((tid >> 3) * lda + (tid & 7) * 8) * 2);
-    const uint32_t voff_b = (uint32_t)(((tid >> 3) * ldb + (tid & 7) * 8) * 2);
+    // [N x K] tile: 8 lanes per 128-byte row, 32 rows per pass; [K x N] tile: 32 lanes per 512-byte row, 8 rows per pass
+    const uint32_t voff_b = BKN ? (uint32_t)(((tid >> 5) * ldb + (tid & 31) * 8) * 2) : (uint32_t)(((tid >> 3) * ldb + (tid & 7) * 8) * 2);
     const int soff = (tid >> 3) * LDS_ROW + (tid & 7) * 8;
+    const int soff_b = BKN ? (tid >> 5) * LDS_ROW_KN + (tid & 31) * 8 : soff;
     auto gload_a = [&](int set, int kt) {
         const char* pa = reinterpret_cast<const char*>(A + kt * BK);
 #pragma unroll
         for (int i = 0; i < CH; i++) ra[set][i] = *(gvec_p)(pa + (size_t)i * 32 * lda * 2 + voff_a);
     };
     auto gload_b = [&](int set, int kt) {
-        const char* pb = reinterpret_cast<const char*>(B + kt * BK);
+        const char* pb = reinterpret_cast<const char*>(BKN ? B + (size_t)kt * BK * ldb : B + kt * BK);
 #pragma unroll
-        for (int i = 0; i < CH; i++) rb[set][i] = *(gvec_p)(pb + (size_t)i * 32 * ldb * 2 + voff_b);
+        for (int i = 0; i < CH; i++) rb[set][i] = *(gvec_p)(pb + (size_t)i * (BKN ? 8 : 32) * ldb * 2 + voff_b);
     };
     auto sstore_a = [&](int set, bf16_t* stage) {
 #pragma unroll
@@ -314,10 +352,15 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
     };
     auto sstore_b = [&](int set, bf16_t* stage) {
 #pragma unroll
-        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[TILE_ELEMS + soff + i * 32 * LDS_ROW]) = rb[set][i];
+        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[TILE_ELEMS + soff_b + i * (BKN ? 8 * LDS_ROW_KN : 32 * LDS_ROW)]) = rb[set][i];
     };
     const int a_off = (wm * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
-    const int b_off = TILE_ELEMS + (wn * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
+    // [K x N] tile: the transposing read hands lane i of a 16-lane group, as element e, element i%4 of the 8 bytes
+    // that lane 4e + i/4 of the group addressed.  Lane s therefore points at row k0 + s/4, columns n0 + 4(s%4) .. +3
+    // of the group's 4(k) x 16(n) block, and lane i receives k0 .. k0+3 of column n0 + i.  Groups 0/1 of the wave
+    // cover columns 0-15 / 16-31 of the 32-column MFMA tile, groups 2/3 the same columns of the next 8 k.
+    const int b_off = BKN ? TILE_ELEMS + (8 * (lane >> 5) + ((lane & 15) >> 2)) * LDS_ROW_KN + wn * (BT / 2) + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)
+                          : TILE_ELEMS + (wn * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
     // MFMA operands are double-buffered in registers: the LDS reads of the next 16-wide k step are
     // in flight while the 16 MFMAs of the current one issue (one wave per SIMD, nothing else hides them)
     bf16x8 av[2][TM], bv[2][TN];
@@ -325,7 +368,18 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
 #pragma unroll
         for (int i = 0; i < TM; i++) av[s][i] = *reinterpret_cast<const bf16x8*>(stage + a_off + i * 32 * LDS_ROW + kk * 16);
 #pragma unroll
-        for (int j = 0; j < TN; j++) bv[s][j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+        for (int j = 0; j < TN; j++) {
+            if (BKN) {
+                const bf16_t* q = stage + b_off + j * 32 + kk * 16 * LDS_ROW_KN;
+                const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q));
+                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * LDS_ROW_KN));
+                typedef short i16x8 __attribute__((ext_vector_type(8)));
+                const i16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                bv[s][j] = __builtin_bit_cast(bf16x8, both);
+            } else {
+                bv[s][j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+            }
+        }
     };
     auto mma = [&](int s) {
 #pragma unroll
@@ -335,43 +389,56 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
     };
 
     const int nk = K / BK;      // a multiple of 4: K is a multiple of 256
+    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : (y_sel ? Mt.Y2 : Mt.Y);
+    const int gcol0 = tn * BT + wn * (BT / 2);
+    // the auxiliary operand of the epilogue (G for the polynomial, the current Y for the apply step):
+    // 8 x 16 bytes per lane and 32-row block of this wave's 128 x 128 tile.  The first two blocks are requested during
+    // the last K tile (whose register sets are free by then), each later one while the block two before it is
+    // being written, so that the epilogue does not wait for memory
+    u32x4 ax[2][8];
+    auto aux_load = [&](int i) {
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
+            ax[i & 1][c] = *(gvec_p)(aux + (size_t)(tm * BT + wm * (BT / 2) + i * 32 + row) * ldc + gcol0 + c8 * 8);
+        }
+    };
     gload_a(0, 0); gload_b(0, 0);
     sstore_a(0, smem); sstore_b(0, smem);
     gload_a(1, 1); gload_b(1, 1);
     gload_a(0, 2); gload_b(0, 2);
     __syncthreads();
+    lds_load(smem, 0, 0);
     // One wave per SIMD issues in order, so a burst of memory instructions leaves the MFMA pipe
-    // idle while it issues.  Each K tile is four phases of 16 MFMAs; the LDS reads of the next k
-    // step, the LDS writes of tile kt+1 and the global loads of tile kt+3 are dealt between the
-    // MFMAs of a phase with sched_group_barrier (masks: 0x008 MFMA, 0x020 VMEM read, 0x100 LDS
-    // read, 0x200 LDS write).  The steady-state body issues everything unconditionally (a static
-    // wait count has to be right on every path); the last four K tiles are peeled.
-    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : Mt.Y;
-    const int gcol0 = tn * BT + wn * (BT / 2);
-    auto ktile = [&](int kt, auto set_c, auto store_c, auto load_c) {
+    // idle while it issues, and an operand that is requested late stalls the whole SIMD.  Each K tile is four
+    // phases of 16 MFMAs.  The LDS reads of the next k step go between the first eight MFMAs of a phase (an
+    // operand then has at least eight MFMAs, 256 clocks, to arrive), the LDS writes of tile kt+1 and the global
+    // loads of tile kt+3 between the last eight, all placed with sched_group_barrier (masks: 0x008 MFMA,
+    // 0x020 VMEM read, 0x100 LDS read, 0x200 LDS write).  The workgroup barrier sits before the last phase:
+    // by then every wave has issued all its reads of the current stage and written its share of the next one,
+    // so the last phase's MFMAs cover the first operand reads of the next tile.  The steady-state body issues
+    // everything unconditionally (a static wait count has to be right on every path); the last four K tiles
+    // are peeled.
+    auto ktile = [&](int kt, auto set_c, auto store_c, auto load_c, auto last_c) {
         constexpr int S = decltype(set_c)::value;       // register set holding tile kt+1
-        constexpr bool LD = decltype(load_c)::value != 0, ST = decltype(store_c)::value != 0;
+        constexpr bool LD = decltype(load_c)::value != 0, ST = decltype(store_c)::value != 0, LAST = decltype(last_c)::value != 0;
         const bf16_t* cur = smem + (kt & 1) * 2 * TILE_ELEMS;
         bf16_t* nxt = smem + ((kt + 1) & 1) * 2 * TILE_ELEMS;
-        lds_load(cur, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         // phase 0: k step 0 | read k step 1
         lds_load(cur, 1, 1);
         mma(0);
-#pragma unroll
-        for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
+        SG_MUON_SCHED_READS();
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         __builtin_amdgcn_sched_barrier(0);
         // phase 1: k step 1 | read k step 2, write A of tile kt+1
         lds_load(cur, 2, 0);
         if (ST) sstore_a(S, nxt);
         mma(1);
+        SG_MUON_SCHED_READS();
 #pragma unroll
         for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -380,36 +447,48 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
         if (ST) sstore_b(S, nxt);
         if (LD) gload_a(S, kt + 3);
         mma(0);
+        SG_MUON_SCHED_READS();
 #pragma unroll
         for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
             if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // phase 3: k step 3 | load B of tile kt+3
+        __syncthreads();
+        // phase 3: k step 3 | read k step 0 of tile kt+1, load B of tile kt+3 (last tile: the epilogue's auxiliary operand)
+        if (!LAST) lds_load(nxt, 0, 0);
         if (LD) gload_b(S, kt + 3);
+        if (LAST && EPI != EPI_GRAM) { aux_load(0); aux_load(1); }
         mma(1);
+        if (!LAST) {
+            SG_MUON_SCHED_READS();
 #pragma unroll
-        for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            for (int g = 0; g < 8; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+        } else if (EPI != EPI_GRAM) {
+#pragma unroll
+            for (int g = 0; g < 16; g++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
     };
     using c0 = std::integral_constant<int, 0>;
     using c1 = std::integral_constant<int, 1>;
     int kt = 0;
     for (; kt + 4 < nk; kt += 2) {
-        ktile(kt, c1{}, c1{}, c1{});
-        ktile(kt + 1, c0{}, c1{}, c1{});
+        ktile(kt, c1{}, c1{}, c1{}, c0{});
+        ktile(kt + 1, c0{}, c1{}, c1{}, c0{});
     }
-    ktile(kt, c1{}, c1{}, c1{});        // kt = nk-4: loads the last tile
-    ktile(kt + 1, c0{}, c1{}, c0{});
-    ktile(kt + 2, c1{}, c1{}, c0{});
-    ktile(kt + 3, c0{}, c0{}, c0{});
+    ktile(kt, c1{}, c1{}, c1{}, c0{});        // kt = nk-4: loads the last tile
+    ktile(kt + 1, c0{}, c1{}, c0{}, c0{});
+    ktile(kt + 2, c1{}, c1{}, c0{}, c0{});
+    ktile(kt + 3, c0{}, c0{}, c0{}, c1{});
+    __syncthreads();        // the epilogue reuses the LDS stages: every wave is done reading them
 
     // ---- epilogue, staged through LDS (free after the last barrier) so that global memory sees
     // 16-byte accesses along rows.  Accumulator element e of MFMA tile (i,j) is
@@ -423,10 +502,9 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
     constexpr int EP_ROW = 128 + 4;     // floats per staged row
     static_assert(4 * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
     float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EP_ROW);
-    // uniform over the workgroup.  The apply step keeps the transposed copy of Y current for the
-    // next iteration's B operand; after the last iteration only tall matrices still need it (their
-    // parameter update reads the transposed orientation).
-    const bool mirror = (EPI == EPI_APPLY) ? (!last_iter || !Mt.wide) : (tm != tn);
+    // uniform over the workgroup.  The apply step stores the transposed tile only after the last iteration of a
+    // tall matrix (its parameter update reads that orientation).
+    const bool mirror = (EPI == EPI_APPLY) ? (last_iter && !Mt.wide) : (tm != tn);
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int grow0 = tm * BT + wm * (BT / 2) + i * 32;
@@ -435,16 +513,6 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
 #pragma unroll
             for (int e = 0; e < 16; e++)
                 ep[(8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * EP_ROW + 32 * j + (lane & 31)] = acc[i][j][e];
-        // the auxiliary operand (G for the polynomial, Y for the apply step, which updates Y in
-        // place): all of this block's chunks are fetched before its first store so the loads overlap
-        u32x4 ax[8];
-        if (EPI != EPI_GRAM) {
-#pragma unroll
-            for (int c = 0; c < 8; c++) {
-                const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
-                ax[c] = *(gvec_p)(aux + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8);
-            }
-        }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int c = 0; c < 8; c++) {
@@ -455,24 +523,23 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
             if (EPI != EPI_GRAM) {
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
-                    const uint32_t w = ax[c][k >> 1];
+                    const uint32_t w = ax[i & 1][c][k >> 1];
                     const float x = sg_i2f((int32_t)((k & 1) ? (w & 0xffff0000u) : (w << 16)));
                     v[k] = (EPI == EPI_POLY) ? sg_fma(NS_C, v[k], NS_B * x) : sg_fma(NS_A, x, v[k]);
                 }
             }
-            uint32_t o[8];
-#pragma unroll
-            for (int k = 0; k < 8; k++) o[k] = bf16r(v[k]);
             u32x4 out;
 #pragma unroll
-            for (int k = 0; k < 4; k++) out[k] = o[2 * k] | (o[2 * k + 1] << 16);
+            for (int k = 0; k < 4; k++) out[k] = bf16r2(v[2 * k], v[2 * k + 1]);
             *reinterpret_cast<u32x4*>(C + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8) = out;
             if (mirror) {   // rounded values (as bf16 bit patterns) back into the staged block
-                u32x4 b0 = {o[0], o[1], o[2], o[3]}, b1 = {o[4], o[5], o[6], o[7]};
+                u32x4 b0 = {out[0] & 0xffffu, out[0] >> 16, out[1] & 0xffffu, out[1] >> 16};
+                u32x4 b1 = {out[2] & 0xffffu, out[2] >> 16, out[3] & 0xffffu, out[3] >> 16};
                 reinterpret_cast<u32x4*>(src)[0] = b0;
                 reinterpret_cast<u32x4*>(src)[1] = b1;
             }
         }
+        if (EPI != EPI_GRAM && i + 2 < TM) aux_load(i + 2);
         __builtin_amdgcn_wave_barrier();
         if (mirror) {
             const uint32_t* epb = reinterpret_cast<const uint32_t*>(ep);
@@ -491,12 +558,12 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int yt_sel, int last_
 }
 
 // p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
-__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int yt_sel) {
+__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int y_sel) {
     const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
     const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
     const int cnt = min(ETILE, M.rows * M.cols - start);
-    const bf16_t* X = M.wide ? M.Y : (yt_sel ? M.YT2 : M.YT);
+    const bf16_t* X = M.wide ? (y_sel ? M.Y2 : M.Y) : M.YT;
     const int ld = M.wide ? M.np : M.mp;
     // the reference's scalar arithmetic (csrc/ops.cpp:729-734)
     const float max_dim = (float)max(M.rows, M.cols);
@@ -580,8 +647,8 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         Mat& M = L->mats[i];
         // offsets for now; turned into pointers once the workspace base is known
         M.Y = (bf16_t*)take(2 * (size_t)M.mp * M.np);
-        M.YT = (bf16_t*)take(2 * (size_t)M.mp * M.np);
-        M.YT2 = (bf16_t*)take(2 * (size_t)M.mp * M.np);
+        M.Y2 = (bf16_t*)take(2 * (size_t)M.mp * M.np);
+        M.YT = (bf16_t*)take(M.wide ? 0 : 2 * (size_t)M.mp * M.np);
         M.G = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
         M.H = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
     }
@@ -617,7 +684,7 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     const int P = L.P;
     for (auto& M : L.mats) {
-        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.YT = (bf16_t*)(ws + (size_t)M.YT); M.YT2 = (bf16_t*)(ws + (size_t)M.YT2);
+        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.Y2 = (bf16_t*)(ws + (size_t)M.Y2); M.YT = (bf16_t*)(ws + (size_t)M.YT);
         M.G = (bf16_t*)(ws + (size_t)M.G); M.H = (bf16_t*)(ws + (size_t)M.H);
     }
     SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, hipMemcpyHostToDevice, st));
@@ -662,7 +729,7 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
 
     hipLaunchKernelGGL(k_momentum, dim3(B.etiles), dim3(256), 0, st, B, momentum);
     hipLaunchKernelGGL(k_norm, dim3(P), dim3(256), 0, st, B);
-    hipLaunchKernelGGL(k_normalize, dim3(B.ttiles), dim3(256), 0, st, B);
+    hipLaunchKernelGGL(k_normalize, dim3(B.ttiles), dim3(256), 0, st, B, ns_steps == 0 ? 1 : 0);
     SG_LAUNCH_CHECK("muon prologue");
     for (int it = 0; it < ns_steps; it++) {
         const int sel = it & 1, last = it + 1 == ns_steps;

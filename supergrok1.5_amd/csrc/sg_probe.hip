@@ -2,6 +2,8 @@
 // SIMD for plain (non-packed) fma / mul / add / DPP-add streams, as a function of the waves resident per SIMD and
 // of the share of the chip that is busy.  It is the yardstick the arithmetic-bound kernels of this library
 // (the v2 scan and per-element kernels) are priced against; the reference has nothing comparable.
+// Op 4 is the same for the matrix cores: a stream of independent v_mfma_f32_32x32x16_bf16 on register operands
+// (no memory traffic at all), the ceiling the Muon GEMM's main loop is priced against.
 #include "sg_common.hpp"
 
 namespace {
@@ -35,6 +37,52 @@ __global__ __launch_bounds__(256) void k_probe(float* sink, long long* ticks, in
     if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
 }
 
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float probe_f32x16;
+constexpr int PROBE_MFMA_ACC = 4;  // independent accumulator tiles per wave
+
+// RANDOM: operands are pseudo-random bf16 values in (-1, 1), different in every lane and element, and four operand
+// pairs alternate: what the data of a real product costs in power (and therefore clock) against constant operands
+template <bool RANDOM>
+__global__ __launch_bounds__(256) void k_probe_mfma(float* sink, long long* ticks, int iters) {
+    probe_f32x16 acc[PROBE_MFMA_ACC];
+    probe_bf16x8 av[PROBE_MFMA_ACC], bv[PROBE_MFMA_ACC];
+#pragma unroll
+    for (int k = 0; k < PROBE_MFMA_ACC; k++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            if (RANDOM) {
+                uint32_t h = (threadIdx.x * 8u + e + 2048u * k + 8192u * blockIdx.x) * 2654435761u;
+                h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+                av[k][e] = (__bf16)(((int)(h & 0xffffu) - 32768) * (1.0f / 32768.0f));
+                bv[k][e] = (__bf16)(((int)(h >> 16) - 32768) * (1.0f / 32768.0f));
+            } else {
+                av[k][e] = (__bf16)(1.0f + 0.001f * (threadIdx.x & 7));
+                bv[k][e] = (__bf16)(0.5f);
+            }
+        }
+#pragma unroll
+    for (int k = 0; k < PROBE_MFMA_ACC; k++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[k][e] = 0.0f;
+    const long long t0 = clock64();
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int r = 0; r < PROBE_UNROLL * PROBE_ILP / PROBE_MFMA_ACC; r++) {
+#pragma unroll
+            for (int k = 0; k < PROBE_MFMA_ACC; k++) acc[k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[(k + r) % PROBE_MFMA_ACC], bv[k], acc[k], 0, 0, 0);
+        }
+    }
+    const long long t1 = clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PROBE_MFMA_ACC; k++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) s += acc[k][e];
+    if (s == 12345.678f) sink[0] = s;
+    if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -47,7 +95,7 @@ size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd) {
 int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
                   double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream) {
     hipStream_t st = (hipStream_t)stream;
-    if (op < 0 || op > 3) return sg::fail("op must be 0 (fma), 1 (mul), 2 (add) or 3 (add with a DPP operand)");
+    if (op < 0 || op > 5) return sg::fail("op must be 0 (fma), 1 (mul), 2 (add), 3 (add with a DPP operand), 4 (32x32x16 bf16 MFMA, constant operands) or 5 (the same, random operands)");
     if (num_cus <= 0 || num_cus > 1024 || waves_per_simd <= 0 || waves_per_simd > 8 || iters <= 0 || iters > 100000)
         return sg::fail("probe size out of range");
     if (!ms_out || !ticks_per_wave_out || !instr_per_wave_out) return sg::fail("NULL argument");
@@ -63,6 +111,8 @@ int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_
             case 0: hipLaunchKernelGGL(k_probe<0>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             case 1: hipLaunchKernelGGL(k_probe<1>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             case 2: hipLaunchKernelGGL(k_probe<2>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 4: hipLaunchKernelGGL(k_probe_mfma<false>, dim3(blocks), dim3(256), 0, st, sink, ticks, n); break;
+            case 5: hipLaunchKernelGGL(k_probe_mfma<true>, dim3(blocks), dim3(256), 0, st, sink, ticks, n); break;
             default: hipLaunchKernelGGL(k_probe<3>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
         }
     };
