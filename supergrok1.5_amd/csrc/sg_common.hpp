@@ -90,4 +90,34 @@ __device__ __forceinline__ int upper_seg(P prefix, int n, int x) {
 
 inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// ---- small host tables into device memory through kernel arguments -----------
+// A copy from pageable host memory blocks the calling thread until the stream has drained to it and cannot be
+// recorded into a graph; a few KB of per-call tables travel as kernel arguments instead, UPLOAD_WORDS 32-bit words
+// per launch.  dst 4-byte aligned, bytes a multiple of 4; the source is read before the call returns.
+constexpr int UPLOAD_WORDS = 896;            // 3584 bytes of payload: the argument block stays below 4 KB
+struct UploadChunk {
+    uint32_t w[UPLOAD_WORDS];
+    uint32_t* dst;
+    int n;
+};
+static __global__ __launch_bounds__(256) void k_upload(UploadChunk c) {
+    for (int i = threadIdx.x; i < c.n; i += 256) c.dst[i] = c.w[i];
+}
+inline int upload_words(void* dst, const void* src, size_t bytes, hipStream_t st) {
+    if ((bytes & 3u) != 0 || (reinterpret_cast<uintptr_t>(dst) & 3u) != 0) return fail("upload: size and destination must be multiples of 4");
+    const uint32_t* s = static_cast<const uint32_t*>(src);
+    uint32_t* d = static_cast<uint32_t*>(dst);
+    size_t left = bytes / 4;
+    while (left > 0) {
+        UploadChunk c;
+        c.n = (int)(left < (size_t)UPLOAD_WORDS ? left : (size_t)UPLOAD_WORDS);
+        for (int i = 0; i < c.n; i++) c.w[i] = s[i];
+        c.dst = d;
+        hipLaunchKernelGGL(k_upload, dim3(1), dim3(256), 0, st, c);
+        SG_LAUNCH_CHECK("k_upload");
+        s += c.n; d += c.n; left -= (size_t)c.n;
+    }
+    return 0;
+}
+
 }  // namespace sg

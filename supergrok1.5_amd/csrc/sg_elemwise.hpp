@@ -56,9 +56,10 @@ inline int make_layout(int n, const int64_t* numels, Layout* L) {
     L->tiles = (int)tiles;
     size_t o = 0;
     auto take = [&](size_t b) { size_t r = o; o = sg::align_up(o + b, 256); return r; };
-    L->off_recs = take(REC_BYTES * (size_t)n);
+    // records and tile prefix table back to back: one upload
+    L->off_recs = take(REC_BYTES * (size_t)n + sizeof(int) * (size_t)(n + 1));
+    L->off_prefix = L->off_recs + REC_BYTES * (size_t)n;
     L->off_nrecs = take(NREC_BYTES * (size_t)n);
-    L->off_prefix = take(sizeof(int) * (size_t)(n + 1));
     L->off_partials = take(sizeof(double) * 3 * (size_t)(tiles + 1));     // up to three sums per tile
     L->off_red = take(sizeof(Red));
     L->off_tred = take(sizeof(TRed) * (size_t)(n + 1));                   // per-tensor sums
@@ -89,11 +90,15 @@ int upload(const std::vector<Rec>& recs, void* workspace, size_t ws_bytes, hipSt
     if (make_layout(n, numels.data(), &L)) return 1;
     if (!workspace || ws_bytes < L.bytes) return sg::fail("workspace too small: need %zu bytes, got %zu", L.bytes, ws_bytes);
     if (((uintptr_t)workspace & 255u) != 0) return sg::fail("workspace must be 256-byte aligned");
-    std::vector<int> prefix(n + 1, 0);
+    // host image of [records (REC_BYTES apart is the layout's bound; they lie sizeof(Rec) apart) | prefix table]
+    std::vector<uint32_t> blob((REC_BYTES * (size_t)n + sizeof(int) * (size_t)(n + 1)) / 4, 0u);
+    static_assert(sizeof(Rec) % 4 == 0 && REC_BYTES % 4 == 0, "records are whole words");
+    const uint32_t* rw = reinterpret_cast<const uint32_t*>(recs.data());
+    for (size_t i = 0; i < sizeof(Rec) * (size_t)n / 4; i++) blob[i] = rw[i];
+    int* prefix = reinterpret_cast<int*>(blob.data() + REC_BYTES * (size_t)n / 4);
     for (int i = 0; i < n; i++) prefix[i + 1] = prefix[i] + (int)((numels[i] + L.tile - 1) / L.tile);
     unsigned char* ws = static_cast<unsigned char*>(workspace);
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_recs, recs.data(), sizeof(Rec) * (size_t)n, hipMemcpyHostToDevice, st));
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_prefix, prefix.data(), sizeof(int) * (size_t)(n + 1), hipMemcpyHostToDevice, st));
+    if (sg::upload_words(ws + L.off_recs, blob.data(), blob.size() * 4, st)) return 1;
     B->recs = reinterpret_cast<const Rec*>(ws + L.off_recs);
     B->prefix = reinterpret_cast<const int*>(ws + L.off_prefix);
     B->n = n;
@@ -178,7 +183,7 @@ int reduce_sumsq(const std::vector<Rec>& recs, const Batch<Rec>& B, float clip_n
     static_assert(sizeof(NormRec) == NREC_BYTES, "NormRec layout");
     std::vector<NormRec> nr(recs.size());
     for (size_t i = 0; i < recs.size(); i++) nr[i] = {recs[i].grad, recs[i].numel, recs[i].dtype};
-    SG_HIP_CHECK(hipMemcpyAsync(B.nrecs, nr.data(), sizeof(NormRec) * nr.size(), hipMemcpyHostToDevice, st));
+    if (sg::upload_words(B.nrecs, nr.data(), sizeof(NormRec) * nr.size(), st)) return 1;
     Batch<NormRec> NB;
     NB.recs = reinterpret_cast<const NormRec*>(B.nrecs);
     NB.prefix = B.prefix;

@@ -687,11 +687,12 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
         M.Y = (bf16_t*)(ws + (size_t)M.Y); M.Y2 = (bf16_t*)(ws + (size_t)M.Y2); M.YT = (bf16_t*)(ws + (size_t)M.YT);
         M.G = (bf16_t*)(ws + (size_t)M.G); M.H = (bf16_t*)(ws + (size_t)M.H);
     }
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, hipMemcpyHostToDevice, st));
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_e, L.pre_e.data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
+    // per-call tables: through kernel arguments (no host-to-device copy, nothing blocks the host)
+    if (sg::upload_words(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, st)) return 1;
+    if (sg::upload_words(ws + L.off_pre_e, L.pre_e.data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
     for (int k = 0; k < 3; k++)
-        SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_g[k], L.pre_g[k].data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
-    SG_HIP_CHECK(hipMemcpyAsync(ws + L.off_pre_t, L.pre_t.data(), sizeof(int) * (size_t)(P + 1), hipMemcpyHostToDevice, st));
+        if (sg::upload_words(ws + L.off_pre_g[k], L.pre_g[k].data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
+    if (sg::upload_words(ws + L.off_pre_t, L.pre_t.data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
     Batch B;
     B.mats = reinterpret_cast<const Mat*>(ws + L.off_mats);
     B.etile_prefix = reinterpret_cast<const int*>(ws + L.off_pre_e);

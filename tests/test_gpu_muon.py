@@ -56,11 +56,14 @@ def _run_case(shapes, dt, steps, seed, lr=0.02, wd=1.0, momentum=0.95, ns=5):
                 assert sv.min() > 0.5 and sv.max() < 1.3, (sv.min(), sv.max())
             else:
                 want = _bf16(new_p) if dt == torch.bfloat16 else new_p.astype(np.float16).astype(np.float32)
-                # one rounding step of the stored parameter + the bf16-vs-fp32 Newton-Schulz deviation of the
-                # update itself (elementwise bound: 10% of the largest update entry; Frobenius: 2e-2, above)
+                # one spacing of the stored 16-bit parameter + what keeping X, the Gram matrix and the polynomial in bf16
+                # between iterations costs against the checker's fp32 iteration: measured at most 2.2% of the largest
+                # update entry over these cases, gated at 3% (Frobenius norm of the whole update: 2e-2, above)
                 ulp = np.maximum(np.abs(want), np.abs(got)) * (2.0 ** -7 if dt == torch.bfloat16 else 2.0 ** -10)
-                tol = ulp + 0.1 * 0.2 * lr * np.abs(X).max() + 1e-12
+                tol = ulp + 0.03 * 0.2 * lr * np.abs(X).max() + 1e-12
                 nd = np.abs(got - want) / tol
+                need = (np.maximum(np.abs(got - want) - ulp, 0.0) / (0.2 * lr * np.abs(X).max())).max()
+                print("  bf16 NS deviation beyond one spacing, in units of the largest update entry: %.4f" % need, flush=True)
                 assert nd.max() <= 1.0, ("param tolerance", t, i, nd.max())
                 # keep the fp32 trajectory of the checker aligned with the 16-bit parameters of the device
                 new_p = got
