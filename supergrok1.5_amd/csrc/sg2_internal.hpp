@@ -51,7 +51,10 @@ constexpr int GRL = GeoDefault::GRL;
 constexpr int PIN = GeoDefault::PIN;
 
 constexpr int ELEM_TILE = 1024;        // elements per tile of the elementwise kernels
-constexpr int SORT_TILE = 4096;        // keys per radix-sort tile (256 threads x 16)
+#ifndef SG2_SORT_TILE
+#define SG2_SORT_TILE 8192
+#endif
+constexpr int SORT_TILE = SG2_SORT_TILE;   // keys per radix-sort tile (16 per thread)
 constexpr int SCAN_TT = 64;            // timesteps projected per LDS tile
 constexpr int SCAN_THREADS = GeoDefault::THREADS;
 constexpr int SCAN_BLOCK_ITEMS = 2048; // entries per block of the spine scan

@@ -6,8 +6,8 @@
 // cub::DeviceSegmentedRadixSort::SortPairs call (:1860-1879).  Non-negative
 // floats order like their bit patterns, so the keys are sorted as uint32.
 //
-// Four passes of 8 bits.  Per pass:
-//   hist     per-tile digit counts -> spine[segment][digit][tile]
+// Four passes of 8 bits over tiles of 8192 keys (512 lanes x 16).  Per pass:
+//   hist     per-tile digit counts -> spine[segment][digit][tile]  (first pass: counted while the keys are made)
 //   scan     exclusive prefix over the whole spine (3 small kernels).  Because
 //            the spine is laid out segment-major, the global prefix of entry
 //            (seg, d, tile) is exactly: keys in earlier segments + keys of this
@@ -21,36 +21,14 @@
 namespace sg2 {
 namespace {
 
-constexpr int SORT_THREADS = 256;
-constexpr int ITEMS = SORT_TILE / SORT_THREADS;      // 16 rounds per wave
+#ifndef SG2_SORT_THREADS
+#define SG2_SORT_THREADS 512
+#endif
+constexpr int SORT_THREADS = SG2_SORT_THREADS;
+constexpr int ITEMS = SORT_TILE / SORT_THREADS;      // rounds per wave
 constexpr int WAVES = SORT_THREADS / 64;
-constexpr int WAVE_ITEMS = SORT_TILE / WAVES;        // 1024 contiguous keys per wave
-
-// ---- key generation ----------------------------------------------------------
-__global__ __launch_bounds__(256) void k_keys(Plan pl) {
-    const int tile = blockIdx.x;
-    const int ti = sg::upper_seg(pl.elem_tile_prefix, pl.P, tile);
-    const TensorDev& T = pl.tensors[ti];
-    const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
-    const int cnt = min(ELEM_TILE, T.numel - start);
-    bool nz = false;
-    for (int k = threadIdx.x; k < cnt; k += 256) {
-        const int i = start + k;
-        const float g = sg::finite_or_zero(sg::load_elem(T.grad, T.dtype, i));
-        // key = |g| bits; the sign rides in bit 31 of the payload so that the sorted (key, payload)
-        // pair gives back g exactly and the scan never has to gather gradients from element order
-        pl.keys[0][T.off + i] = (uint32_t)sg_f2i(sg_abs(g));
-        pl.vals[0][T.off + i] = i | (sg_f2i(g) & (int32_t)0x80000000);
-        nz = nz || (sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, i)) != 0.0f);
-    }
-    // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
-    // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
-    // (plain store, and only while the flag still reads 0: every writer stores the same value)
-    if (__syncthreads_or(nz) && threadIdx.x == 0) {
-        volatile int* flag = pl.sharp_nonzero + ti;
-        if (*flag == 0) *flag = 1;
-    }
-}
+constexpr int WAVE_ITEMS = SORT_TILE / WAVES;        // contiguous keys per wave
+static_assert(SORT_THREADS >= 256 && SORT_THREADS % 64 == 0 && SORT_TILE % SORT_THREADS == 0, "one thread per digit at least");
 
 struct TileRef {
     int base;        // index of the tile's first key in the packed arrays
@@ -71,16 +49,72 @@ __device__ __forceinline__ TileRef tile_ref(const Plan& pl, int tile) {
     return r;
 }
 
+
+// ---- key generation + digit counts of the first pass -------------------------------
+// One sort tile per workgroup.  All of a lane's loads are issued before the first store (the tile length is a
+// compile-time bound, the tail is predicated).
+__global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
+    __shared__ uint32_t h[256];
+    const int seg = sg::upper_seg(pl.sort_tile_prefix, pl.P, (int)blockIdx.x);
+    const TileRef tr = tile_ref(pl, blockIdx.x);
+    const TensorDev& T = pl.tensors[seg];
+    const int start = tr.base - T.off;
+    if (threadIdx.x < 256) h[threadIdx.x] = 0;
+    __syncthreads();
+    float g[ITEMS];
+    bool nz = false;
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int k = r * SORT_THREADS + (int)threadIdx.x;
+        g[r] = (k < tr.cnt) ? sg::load_elem(T.grad, T.dtype, start + k) : 0.0f;
+    }
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int k = r * SORT_THREADS + (int)threadIdx.x;
+        if (k < tr.cnt) nz = nz || (sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, start + k)) != 0.0f);
+    }
+#pragma unroll
+    for (int r = 0; r < ITEMS; r++) {
+        const int k = r * SORT_THREADS + (int)threadIdx.x;
+        if (k < tr.cnt) {
+            const float gv = sg::finite_or_zero(g[r]);
+            // key = |g| bits; the sign rides in bit 31 of the payload so that the sorted (key, payload)
+            // pair gives back g exactly and the scan never has to gather gradients from element order
+            const uint32_t key = (uint32_t)sg_f2i(sg_abs(gv));
+            pl.keys[0][tr.base + k] = key;
+            pl.vals[0][tr.base + k] = (start + k) | (sg_f2i(gv) & (int32_t)0x80000000);
+            atomicAdd(&h[key & 255u], 1u);
+        }
+    }
+    // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
+    // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
+    // (plain store, and only while the flag still reads 0: every writer stores the same value)
+    if (__syncthreads_or(nz) && threadIdx.x == 0) {
+        volatile int* flag = pl.sharp_nonzero + seg;
+        if (*flag == 0) *flag = 1;
+    }
+    if (threadIdx.x < 256) pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
+}
+
 // ---- per-tile histogram ---------------------------------------------------------
 __global__ __launch_bounds__(SORT_THREADS) void k_hist(Plan pl, int src, int shift) {
     __shared__ uint32_t h[256];
     const TileRef tr = tile_ref(pl, blockIdx.x);
-    h[threadIdx.x] = 0;
+    if (threadIdx.x < 256) h[threadIdx.x] = 0;
     __syncthreads();
     const uint32_t* __restrict__ keys = pl.keys[src] + tr.base;
-    for (int k = threadIdx.x; k < tr.cnt; k += SORT_THREADS) atomicAdd(&h[(keys[k] >> shift) & 255u], 1u);
+    // 16 bytes per lane where the tile starts on a 16-byte boundary (tensor offsets are arbitrary); the ragged end by single keys
+    const int vec = ((tr.base & 3) == 0) ? (tr.cnt & ~3) : 0;
+    for (int k = threadIdx.x * 4; k < vec; k += SORT_THREADS * 4) {
+        const uint4 q = *reinterpret_cast<const uint4*>(keys + k);
+        atomicAdd(&h[(q.x >> shift) & 255u], 1u);
+        atomicAdd(&h[(q.y >> shift) & 255u], 1u);
+        atomicAdd(&h[(q.z >> shift) & 255u], 1u);
+        atomicAdd(&h[(q.w >> shift) & 255u], 1u);
+    }
+    for (int k = vec + threadIdx.x; k < tr.cnt; k += SORT_THREADS) atomicAdd(&h[(keys[k] >> shift) & 255u], 1u);
     __syncthreads();
-    pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
+    if (threadIdx.x < 256) pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
 }
 
 // ---- exclusive scan of the spine -------------------------------------------------
@@ -195,9 +229,10 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
     __syncthreads();
     // digit d = threadIdx.x: position of each wave's first key of digit d inside the tile's digit-sorted order
     // (cnt[k][d]), start of digit d in that order (lbase[d]) and its distance to the global destination (gdelta[d])
-    __shared__ uint32_t lbase[256], gdelta[256], wsum[WAVES];
+    __shared__ uint32_t lbase[256], gdelta[256], wsum[4];
     {
-        const int d = threadIdx.x;
+        const int d = threadIdx.x & 255;       // (threads beyond the 256 digits repeat the first ones' work and store nothing)
+        const bool own = threadIdx.x < 256;
         uint32_t tot = 0;
 #pragma unroll
         for (int k = 0; k < WAVES; k++) tot += cnt[k][d];
@@ -207,20 +242,22 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
             const uint32_t up = __shfl_up(inc, o, 64);
             if (lane >= o) inc += up;
         }
-        if (lane == 63) wsum[w] = inc;
+        if (lane == 63 && own) wsum[w] = inc;
         __syncthreads();
         uint32_t before = 0;
 #pragma unroll
-        for (int k = 0; k < WAVES; k++) before += (k < w) ? wsum[k] : 0u;
+        for (int k = 0; k < 4; k++) before += (k < (d >> 6)) ? wsum[k] : 0u;
         const uint32_t lb = before + inc - tot;
-        lbase[d] = lb;
-        gdelta[d] = pl.spine[tr.spine0 + d * tr.stride] - lb;     // global destination = gdelta[d] + local position (mod 2^32)
-        uint32_t run = lb;
+        if (own) {
+            lbase[d] = lb;
+            gdelta[d] = pl.spine[tr.spine0 + d * tr.stride] - lb;     // global destination = gdelta[d] + local position (mod 2^32)
+            uint32_t run = lb;
 #pragma unroll
-        for (int k = 0; k < WAVES; k++) {
-            const uint32_t c = cnt[k][d];
-            cnt[k][d] = run;
-            run += c;
+            for (int k = 0; k < WAVES; k++) {
+                const uint32_t c = cnt[k][d];
+                cnt[k][d] = run;
+                run += c;
+            }
         }
     }
     __syncthreads();
@@ -278,13 +315,13 @@ __global__ __launch_bounds__(256) void k_gather_sorted(Plan pl, int32_t* __restr
 
 int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st) {
     if (pl.total == 0) return 0;
-    hipLaunchKernelGGL(k_keys, dim3(pl.elem_tiles), dim3(256), 0, st, pl);
+    hipLaunchKernelGGL(k_keys, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_keys");
     const int n = 256 * pl.sort_tiles;
     const int nb = (n + SCAN_BLOCK_ITEMS - 1) / SCAN_BLOCK_ITEMS;
     for (int pass = 0; pass < 4; pass++) {
         const int src = pass & 1, shift = 8 * pass;
-        hipLaunchKernelGGL(k_hist, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
+        if (pass > 0) hipLaunchKernelGGL(k_hist, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);     // the first pass's counts come from k_keys
         hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
         hipLaunchKernelGGL(k_spine_top, dim3(1), dim3(256), 0, st, pl.blocksums, nb);
         hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
