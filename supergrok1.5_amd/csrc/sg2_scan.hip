@@ -364,7 +364,13 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             if (tu == 0) { s_large[half] = large; s_nottiny[half] = nottiny; }
         }
         __syncthreads();
-        const unsigned long long large = s_large[half], nottiny = s_nottiny[half];
+        // wave-uniform masks into scalar registers: the per-block tests below are then scalar instructions
+        auto uniform64 = [](unsigned long long v) {
+            const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v);
+            const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(v >> 32));
+            return ((unsigned long long)hi << 32) | lo;
+        };
+        const unsigned long long large = uniform64(s_large[half]), nottiny = uniform64(s_nottiny[half]);
 
         auto keep_state = [&](int u) {
             float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(off, ti, u)) * 2 * SCAN_THREADS;
