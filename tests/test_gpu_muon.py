@@ -52,8 +52,9 @@ def _run_case(shapes, dt, steps, seed, lr=0.02, wd=1.0, momentum=0.95, ns=5):
                 X_gpu = (got / decay - old) / (-0.2 * lr)
                 rel_f = np.linalg.norm(X_gpu - X) / np.linalg.norm(X)
                 assert rel_f < 2e-2, ("X frobenius", t, i, rel_f)
-                sv = np.linalg.svd(X_gpu.astype(np.float64), compute_uv=False)
-                assert sv.min() > 0.5 and sv.max() < 1.3, (sv.min(), sv.max())
+                if ns >= 5:     # orthogonalised: singular values near 1 (rank-deficient shapes aside)
+                    sv = np.linalg.svd(X_gpu.astype(np.float64), compute_uv=False)
+                    assert sv.min() > 0.5 and sv.max() < 1.3, (sv.min(), sv.max())
             else:
                 want = _bf16(new_p) if dt == torch.bfloat16 else new_p.astype(np.float16).astype(np.float32)
                 # one spacing of the stored 16-bit parameter + what keeping X, the Gram matrix and the polynomial in bf16
@@ -76,6 +77,16 @@ def test_small_shapes_all_dtypes():
     shapes = [(24, 40), (40, 24), (16, 16), (130, 70), (1, 5)]
     for dt in (torch.float32, torch.bfloat16, torch.float16):
         _run_case(shapes, dt, 2, seed=1)
+
+
+def test_iteration_counts_zero_to_three():
+    """ns_steps = 0 (the normalised momentum itself is the update: a tall matrix is then read back in its own
+    orientation without any iteration having transposed it), 1, 2 and 3 (the final iterate sits in either of the two
+    work buffers), wide, tall, square and padded shapes."""
+    shapes = [(24, 40), (40, 24), (16, 16), (300, 70), (70, 300)]
+    for ns in (0, 1, 2, 3):
+        _run_case(shapes, torch.float32, 1, seed=10 + ns, ns=ns)
+        _run_case(shapes, torch.bfloat16, 1, seed=20 + ns, ns=ns)
 
 
 def test_reference_golden_f32():
