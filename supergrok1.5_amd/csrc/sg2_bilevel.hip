@@ -165,15 +165,18 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, AdjIO io)
     fill_fmax(s_fmax, rope);
     float u1e, u1o, u2e, u2o, ve, vo;
     const int ntiles = (c.uend - c.ustart + SCAN_TT - 1) / SCAN_TT;
-    // The map contracts like the forward recurrence, so - as in the forward summary pass - it is first taken over the
-    // `window` steps at the start of the chunk only (the end of this reverse sweep).  If every entry of that matrix,
-    // in all 128 lanes, is below 2^-100, whatever arrives from later steps is multiplied by less than that: the
-    // chunk's map is (0, v_window).  Otherwise the whole chunk is swept.
-    const int wtiles = (pl.window > 0) ? pl.window / SCAN_TT : 0;
-    int first_tile = (wtiles > 0 && ntiles > wtiles) ? wtiles - 1 : ntiles - 1;
-    for (;;) {
+    // The map contracts like the forward recurrence, so - as in the forward summary pass - the chunk is walked in blocks
+    // of `window` steps, here from its start (the end of this reverse sweep): each block's map is taken from the identity
+    // and applied after the map of everything before it ((U, v) <- (U_early U_block, U_early v_block + v_early)).  As soon as
+    // every entry of the running matrix, in all 128 lanes, is below 2^-100, whatever arrives from later steps is multiplied
+    // by less than that: the chunk's map is (0, v) and the walk stops.
+    const int wtiles = (pl.window > 0 && pl.window < pl.chunk_len) ? max(1, pl.window / SCAN_TT) : ntiles;
+    float e1e = 1.0f, e1o = 0.0f, e2e = 0.0f, e2o = 1.0f, eve = 0.0f, evo = 0.0f;     // map of the blocks before the current one
+    bool have_early = false;
+    for (int blk_tile0 = 0; blk_tile0 < ntiles; blk_tile0 += wtiles) {
+      const int blk_last = min(ntiles, blk_tile0 + wtiles) - 1;
       u1e = 1.0f; u1o = 0.0f; u2e = 0.0f; u2o = 1.0f; ve = 0.0f; vo = 0.0f;
-      for (int tile = first_tile; tile >= 0; tile--) {
+      for (int tile = blk_last; tile >= blk_tile0; tile--) {
         const int u0 = c.ustart + tile * SCAN_TT, cnt = min(SCAN_TT, c.uend - u0);
         bool small = true;
         {
@@ -221,10 +224,17 @@ __global__ __launch_bounds__(SCAN_THREADS) void k_adj_summary(Plan pl, AdjIO io)
         }
         __syncthreads();
     }
-      if (first_tile == ntiles - 1) break;
+      if (have_early) {     // (U, v) of this block after (E, ev) of the earlier ones: E U, E v + ev
+          const float n1e = sg_fma(e1e, u1e, e2e * u1o), n1o = sg_fma(e1o, u1e, e2o * u1o);
+          const float n2e = sg_fma(e1e, u2e, e2e * u2o), n2o = sg_fma(e1o, u2e, e2o * u2o);
+          const float nve = sg_fma(e1e, ve, sg_fma(e2e, vo, eve)), nvo = sg_fma(e1o, ve, sg_fma(e2o, vo, evo));
+          u1e = n1e; u1o = n1o; u2e = n2e; u2o = n2o; ve = nve; vo = nvo;
+      }
+      if (blk_last == ntiles - 1) break;      // the whole chunk is covered
       const float big = sg_max(sg_max(sg_abs(u1e), sg_abs(u1o)), sg_max(sg_abs(u2e), sg_abs(u2o)));
       if (__syncthreads_and(big < 0x1p-100f)) { u1e = u1o = u2e = u2o = 0.0f; break; }
-      first_tile = ntiles - 1;
+      e1e = u1e; e1o = u1o; e2e = u2e; e2o = u2o; eve = ve; evo = vo;
+      have_early = true;
     }
     float* out = pl.adj_summ + (((size_t)dir * pl.chunks + chunk) * SCAN_THREADS + tid) * 6;
     out[0] = u1e; out[1] = u1o; out[2] = u2e; out[3] = u2o; out[4] = ve; out[5] = vo;

@@ -40,11 +40,13 @@ def _reference(W, grads, sharps, mf, mb, R):
     return ctx, [w.grad for w in Wd]
 
 
-def _case(shapes, seed, sharp, state_std, chunk_len=None, a_log=None):
+def _case(shapes, seed, sharp, state_std, chunk_len=None, a_log=None, window=None):
     from grokking_optimizers import _bilevel, _cabi
     dev = torch.device("cuda:0")
     if chunk_len is not None:
         assert _cabi.lib().sg2_set_chunk_len(chunk_len) == 0
+    if window is not None:
+        assert _cabi.lib().sg2_set_scan_window(window) == 0
     try:
         W = wl.meta_weights(seed)
         if a_log is not None:
@@ -87,6 +89,8 @@ def _case(shapes, seed, sharp, state_std, chunk_len=None, a_log=None):
     finally:
         if chunk_len is not None:
             _cabi.lib().sg2_set_chunk_len(0)
+        if window is not None:
+            _cabi.lib().sg2_set_scan_window(-1)
 
 
 def test_small_tensors_with_sharpness_and_carried_states():
@@ -109,10 +113,17 @@ def test_automatic_chunk_length_on_longer_tensors():
     _case([(5000,), (3000,)], seed=14, sharp=True, state_std=0.3)
 
 
-def test_barely_contracting_poles_fall_back_to_whole_chunk_summaries():
-    """A_log = -12: A_bar stays within 1e-5 of 1, so neither the forward nor the adjoint summary may be taken over a
-    window; both must redo the whole chunk (chunk length 512, window 256)."""
+def test_barely_contracting_poles_walk_the_whole_chunk():
+    """A_log = -12: A_bar stays within 1e-5 of 1, so neither the forward nor the adjoint summary contracts within a
+    block; both walk every block of the chunk (chunk length 512, window 256)."""
     _case([(3000,), (1500,)], seed=16, sharp=True, state_std=0.3, chunk_len=512, a_log=-12.0)
+
+
+def test_slow_poles_need_several_summary_blocks():
+    """A_log = -2 (A = -0.135, the slowest pole of the optimizer's own initialisation is -1): with blocks of 64 steps
+    the 2x2 part falls below 2^-100 only after several of them, so the block walk of both summary kernels composes
+    maps (chunk length 1024, window 64)."""
+    _case([(5000,), (2100,)], seed=17, sharp=True, state_std=0.3, chunk_len=1024, a_log=-2.0, window=64)
 
 
 def test_several_chunks():
