@@ -123,6 +123,9 @@ def build_step(workload, ops, dev, limit=None):
         bufs = [torch.zeros(s, device=dev) for s in shapes]
         W.update(step=lambda: ops.muon_fused_step(params, grads, bufs, 0.95, 0.02, 1.0, 5),
                  units=5 * sum(6 * min(s) ** 2 * max(s) for s in shapes), unit="FLOP/s",       # 6 min^2 max per NS iteration
+                 # what the kernels execute: the two symmetric products launch only the 256 x 256 tiles on or above the diagonal
+                 executed=5 * sum(2 * 256 * 256 * ((-(-min(s) // 256)) * (-(-min(s) // 256) + 1) // 2) * ((-(-max(s) // 256)) * 256 + (-(-min(s) // 256)) * 256)
+                                  + 2 * ((-(-min(s) // 256)) * 256) ** 2 * ((-(-max(s) // 256)) * 256) for s in shapes),
                  name="Muon step, %d x [1024,4096] + %d x [4096,1024], 5 Newton-Schulz iterations" % (len(shapes) // 2, len(shapes) // 2),
                  dtype="bf16", bound="mfma", peak=2500.0)
         return W
@@ -259,6 +262,9 @@ def bench_other(args, dev):
     if W["bound"] == "mfma":
         out["roofline"] = {"bound": "mfma", "achieved": units / el / 1e12, "peak": W["peak"], "unit": "TFLOP/s",
                            "frac": units / el / 1e12 / W["peak"], "traffic": None}
+        if "executed" in W:        # `achieved` counts the algorithm's FLOP; these count the FLOP the kernels execute
+            out["roofline"]["achieved_executed"] = W["executed"] / el / 1e12
+            out["roofline"]["frac_executed"] = W["executed"] / el / 1e12 / W["peak"]
     else:
         bpe = W["bytes_per_elem"]                      # algorithmic bytes per element of the step
         out["roofline"] = {"bound": "hbm", "achieved": bpe * units / el / 1e9, "peak": W["peak"], "unit": "GB/s",
