@@ -317,7 +317,7 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             const int t = dir ? (N - 1 - u) : u;
             nx_key = skey[t];
             nx_val = sval[t];
-            nx_sh = ssrt[t];
+            nx_sh = has_s ? ssrt[t] : 0.0f;      // an all-zero tensor has no sorted copy of its sharpness (uniform branch)
         }
     };
     for (;;) {

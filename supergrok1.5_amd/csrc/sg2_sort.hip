@@ -297,16 +297,13 @@ __global__ __launch_bounds__(256) void k_gather_sorted(Plan pl, int32_t* __restr
     const TensorDev& T = pl.tensors[ti];
     const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
     const int cnt = min(ELEM_TILE, T.numel - start);
-    const bool gather = pl.sharp_nonzero[ti] != 0;      // all-zero sharpness: nothing to gather, the sorted copy is 0 as well
-    if (!gather && !dbg_perm) {
-        for (int k = threadIdx.x; k < cnt; k += 256) pl.ssorted[T.off + start + k] = 0.0f;
-        return;
-    }
+    const bool gather = pl.sharp_nonzero[ti] != 0;      // all-zero sharpness: nothing to gather, no sorted copy is made
+    if (!gather && !dbg_perm) return;                   // every reader tests the same flag before it touches ssorted
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int t = T.off + start + k;
         int idx = pl.vals[0][t] & 0x7fffffff;
         idx = ((unsigned)idx < (unsigned)T.numel) ? idx : 0;       // never index outside the tensor
-        pl.ssorted[t] = gather ? sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, idx)) : 0.0f;
+        if (gather) pl.ssorted[t] = sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, idx));
         if (dbg_perm) dbg_perm[t] = idx;
     }
 }
