@@ -63,6 +63,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
         const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
         const int cnt = min(ELEM_TILE, T.numel - start);
         const int dtype = T.dtype;
+        const bool has_s = pl.sharp_nonzero[ti] != 0;       // set by the sort's key kernel: some sharpness entry of the tensor is not 0
         const float alpha = T.alpha, lamb = T.lamb, beta1 = T.beta1, bc2 = T.bc2, step_size = T.step_size;
         const float beta2 = pl.beta2, eps = pl.eps, rescale = pl.rescale, decay = pl.decay;
 
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             const sg::cfloat_p Wz = Wz0 + zo, bz = bz0 + zo, Wr = Wr0 + zo, br = br0 + zo, Wh = Wh0 + zo, bh = bh0 + zo;
             const sg::cfloat_p Wq = Wq0 + zo, KA = KA0 + zo, KB = KB0 + zo;
             const float g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, i));
-            const float s = sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i));
+            const float s = has_s ? sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i)) : 0.0f;
             float cf[DM], cb[DM], hold[GH];
             {
                 const float4* pf = reinterpret_cast<const float4*>(pl.ctx + ((size_t)T.off + i) * DM);
