@@ -1,4 +1,4 @@
-// Muon step: momentum, Frobenius normalisation, quintic Newton-Schulz
+// Muon step: momentum (which also leaves the bf16 work copy), Frobenius norm (folded into the first iteration), quintic Newton-Schulz
 // orthogonalisation as bf16 MFMA GEMMs with fp32 accumulation, parameter
 // update.  Replaces the body of muon_fused_step (csrc/ops.cpp:663-746 of the
 // reference: ATen norm + one host sync, three torch::mm per iteration,
@@ -73,7 +73,7 @@ struct Batch {
     const int* gtile_prefix[3];    // [P+1] GEMM output tiles for the three products
     const int* ttile_prefix;       // [P+1] 64x64 transpose tiles of Y
     int P, etiles, gtiles[3], ttiles;
-    double* partials;              // [etiles]
+    double* partials;              // [ttiles] sums of squares of the 64x64 tiles
     float* inv_norm;               // [P]
 };
 
@@ -124,33 +124,85 @@ __device__ __forceinline__ void store8(void* p, int dtype, size_t i, const float
     }
 }
 
-__global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum) {
+// buf = momentum * buf + grad, the sum of squares of the new buf, and the new buf as bf16 into Y ([mp x np], the wide
+// orientation) - NOT yet divided by its norm, which is only known once every tile of the matrix has been summed: the
+// first iteration's Gram and apply epilogues carry the factors 1/norm^2 and 1/norm instead (bf16 rounding is relative,
+// so rounding before or after the scaling costs the same), and no separate normalisation pass reads buf again.  With
+// `both` a tall matrix also gets YT ([np x mp], its own orientation; needed when no iteration follows).
+// One 64x64 tile of the parameter's own orientation per workgroup: rows are read and written along the fast axis, the
+// transposed copy goes through LDS.  The zero padding of the work buffers is written here as well.
+__global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum, int both) {
+    __shared__ bf16_t t[64][66];
     __shared__ double sm[4];
-    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
+    const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
-    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
-    const int cnt = min(ETILE, M.rows * M.cols - start);
+    bf16_t* own = M.wide ? M.Y : M.YT;            // [R x C] in the parameter's orientation, padded
+    bf16_t* other = M.wide ? M.YT : M.Y;          // [C x R]
+    const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
+    const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
+    const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
+    const bool w_own = M.wide || both, w_other = !M.wide;       // uniform over the workgroup (YT exists for tall matrices only)
+    const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && M.vec8;
     double acc = 0.0;
-    if (M.vec8) {
-        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
-            const size_t i = (size_t)start + k;
-            float g[8], b[8], part = 0.0f;
-            load8(M.grad, M.dtype, i, g);
-            load8(M.buf, SG_F32, i, b);
+    if (full) {
+        // interior tile: a lane moves 16 consecutive elements of a row
+        const int lr = threadIdx.x >> 2, c0 = (threadIdx.x & 3) * 16;
+        const size_t at = (size_t)(tr0 + lr) * M.cols + tc0 + c0;
+        float g[16], b[16], part = 0.0f;
+        load8(M.grad, M.dtype, at, g);
+        load8(M.grad, M.dtype, at + 8, g + 8);
+        load8(M.buf, SG_F32, at, b);
+        load8(M.buf, SG_F32, at + 8, b + 8);
 #pragma unroll
-            for (int e = 0; e < 8; e++) { b[e] = sg_fma(momentum, b[e], g[e]); part = sg_fma(b[e], b[e], part); }
-            store8(M.buf, SG_F32, i, b);
-            acc += (double)part;
+        for (int e = 0; e < 16; e++) { b[e] = sg_fma(momentum, b[e], g[e]); part = sg_fma(b[e], b[e], part); }
+        store8(M.buf, SG_F32, at, b);
+        store8(M.buf, SG_F32, at + 8, b + 8);
+        acc = (double)part;
+        uint32_t pk[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const uint32_t b0 = sg::f_to_bf16_bits(b[2 * q]), b1 = sg::f_to_bf16_bits(b[2 * q + 1]);
+            pk[q] = b0 | (b1 << 16);
+            t[lr][c0 + 2 * q] = (bf16_t)b0;
+            t[lr][c0 + 2 * q + 1] = (bf16_t)b1;
+        }
+        if (w_own) {
+            uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
+            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+        }
+        if (w_other) {
+            __syncthreads();
+            // transposed copy: output row lr (= own column), 16 consecutive output columns (= own rows)
+#pragma unroll
+            for (int q = 0; q < 8; q++) pk[q] = (uint32_t)t[c0 + 2 * q][lr] | ((uint32_t)t[c0 + 2 * q + 1][lr] << 16);
+            uint4* dt = reinterpret_cast<uint4*>(other + (size_t)(tc0 + lr) * R + tr0 + c0);
+            dt[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            dt[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
         }
     } else {
         float part = 0.0f;
-        for (int k = threadIdx.x; k < cnt; k += 256) {
-            const int i = start + k;
-            const float b = sg_fma(momentum, M.buf[i], sg::load_elem(M.grad, M.dtype, i));
-            M.buf[i] = b;
-            part = sg_fma(b, b, part);
+        for (int k = threadIdx.x; k < 64 * 64; k += 256) {
+            const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
+            bf16_t v = 0;
+            if (r < M.rows && c < M.cols) {
+                const size_t i = (size_t)r * M.cols + c;
+                const float bv = sg_fma(momentum, M.buf[i], sg::load_elem(M.grad, M.dtype, (int64_t)i));
+                M.buf[i] = bv;
+                part = sg_fma(bv, bv, part);
+                v = sg::f_to_bf16_bits(bv);
+            }
+            if (w_own) own[(size_t)r * C + c] = v;
+            t[k >> 6][k & 63] = v;
         }
         acc = (double)part;
+        if (w_other) {
+            __syncthreads();
+            for (int k = threadIdx.x; k < 64 * 64; k += 256) {
+                const int r = k >> 6, c = k & 63;     // output row r (= own column), column c (= own row)
+                other[(size_t)(tc0 + r) * R + tr0 + c] = t[c][r];
+            }
+        }
     }
     const double tot = block_sum(acc, sm);
     if (threadIdx.x == 0) B.partials[blockIdx.x] = tot;
@@ -160,69 +212,9 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
     __shared__ double sm[4];
     const int mi = blockIdx.x;
     double acc = 0.0;
-    for (int k = B.etile_prefix[mi] + (int)threadIdx.x; k < B.etile_prefix[mi + 1]; k += 256) acc += B.partials[k];
+    for (int k = B.ttile_prefix[mi] + (int)threadIdx.x; k < B.ttile_prefix[mi + 1]; k += 256) acc += B.partials[k];
     const double tot = block_sum(acc, sm);
     if (threadIdx.x == 0) B.inv_norm[mi] = 1.0f / ((float)sqrt(tot) + 1e-7f);
-}
-
-// X = buf * inv_norm as bf16 into Y ([mp x np], the wide orientation); with `both` a tall matrix also gets YT
-// ([np x mp], its own orientation; needed when no iteration follows).  One 64x64 tile of the parameter's own orientation per workgroup: rows are read and
-// written along the fast axis, a transposed copy goes through LDS.  The zero padding of the buffers is written
-// here as well.
-__global__ __launch_bounds__(256) void k_normalize(Batch B, int both) {
-    __shared__ bf16_t t[64][66];
-    const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
-    const Mat& M = B.mats[mi];
-    const float inv = B.inv_norm[mi];
-    bf16_t* own = M.wide ? M.Y : M.YT;            // [R x C] in the parameter's orientation, padded
-    bf16_t* other = M.wide ? M.YT : M.Y;          // [C x R]
-    const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
-    const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
-    const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
-    const bool w_own = M.wide || both, w_other = !M.wide;       // uniform over the workgroup (YT exists for tall matrices only)
-    const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && (M.cols & 3) == 0 && (((uintptr_t)M.buf) & 15u) == 0;
-    if (full) {
-        // interior tile: a lane moves 16 consecutive elements of a row (four 16-byte loads, two 16-byte stores)
-        const int lr = threadIdx.x >> 2, c0 = (threadIdx.x & 3) * 16;
-        const float4* src = reinterpret_cast<const float4*>(M.buf + (size_t)(tr0 + lr) * M.cols + tc0 + c0);
-        uint32_t pk[8];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const float4 v = src[q];
-            const uint32_t b0 = sg::f_to_bf16_bits(v.x * inv), b1 = sg::f_to_bf16_bits(v.y * inv);
-            const uint32_t b2 = sg::f_to_bf16_bits(v.z * inv), b3 = sg::f_to_bf16_bits(v.w * inv);
-            pk[2 * q] = b0 | (b1 << 16);
-            pk[2 * q + 1] = b2 | (b3 << 16);
-            t[lr][c0 + 4 * q] = (bf16_t)b0; t[lr][c0 + 4 * q + 1] = (bf16_t)b1;
-            t[lr][c0 + 4 * q + 2] = (bf16_t)b2; t[lr][c0 + 4 * q + 3] = (bf16_t)b3;
-        }
-        if (w_own) {
-            uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
-            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
-        }
-        if (!w_other) return;
-        __syncthreads();
-        // transposed copy: output row lr (= own column), 16 consecutive output columns (= own rows)
-#pragma unroll
-        for (int q = 0; q < 8; q++) pk[q] = (uint32_t)t[c0 + 2 * q][lr] | ((uint32_t)t[c0 + 2 * q + 1][lr] << 16);
-        uint4* dt = reinterpret_cast<uint4*>(other + (size_t)(tc0 + lr) * R + tr0 + c0);
-        dt[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-        dt[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
-        return;
-    }
-    for (int k = threadIdx.x; k < 64 * 64; k += 256) {
-        const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
-        const bf16_t v = (r < M.rows && c < M.cols) ? sg::f_to_bf16_bits(M.buf[(size_t)r * M.cols + c] * inv) : (bf16_t)0;
-        if (w_own) own[(size_t)r * C + c] = v;
-        t[k >> 6][k & 63] = v;
-    }
-    if (!w_other) return;
-    __syncthreads();
-    for (int k = threadIdx.x; k < 64 * 64; k += 256) {
-        const int r = k >> 6, c = k & 63;     // output row r (= own column), column c (= own row)
-        other[(size_t)(tc0 + r) * R + tr0 + c] = t[c][r];
-    }
 }
 
 // ---- GEMM  C[M x N] = A[M x K] * B  with fused epilogues; B given as [N x K] (Gram, polynomial) or as [K x N] (apply)
@@ -268,8 +260,10 @@ typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_p;
 
 // y_sel: which of the two Y buffers holds the current iterate
+// iter_flags: bit 0 = last iteration, bit 1 = first iteration (Y still carries the factor norm: see k_momentum)
 template <int EPI>
-__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int last_iter) {
+__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_flags) {
+    const int last_iter = iter_flags & 1;
     constexpr bool BKN = EPI == EPI_APPLY;             // B operand stored [K x N]
     constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
     constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
@@ -505,6 +499,9 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int last_i
     // uniform over the workgroup.  The apply step stores the transposed tile only after the last iteration of a
     // tall matrix (its parameter update reads that orientation).
     const bool mirror = (EPI == EPI_APPLY) ? (last_iter && !Mt.wide) : (tm != tn);
+    // first iteration: Y is the unnormalised momentum, so its Gram matrix carries 1/norm^2 and the applied Y 1/norm
+    const float inv = Bt.inv_norm[mi];
+    const float first_scale = (iter_flags & 2) ? (EPI == EPI_GRAM ? inv * inv : (EPI == EPI_APPLY ? inv : 1.0f)) : 1.0f;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int grow0 = tm * BT + wm * (BT / 2) + i * 32;
@@ -527,6 +524,10 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int last_i
                     const float x = sg_i2f((int32_t)((k & 1) ? (w & 0xffff0000u) : (w << 16)));
                     v[k] = (EPI == EPI_POLY) ? sg_fma(NS_C, v[k], NS_B * x) : sg_fma(NS_A, x, v[k]);
                 }
+            }
+            if (EPI != EPI_POLY) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) v[k] *= first_scale;        // 1 except in the first iteration
             }
             u32x4 out;
 #pragma unroll
@@ -558,7 +559,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int last_i
 }
 
 // p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
-__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int y_sel) {
+// scale_inv: no iteration ran, X is still the unnormalised momentum
+__global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int y_sel, int scale_inv) {
     const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
     const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
@@ -569,6 +571,7 @@ __global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, 
     const float max_dim = (float)max(M.rows, M.cols);
     const float scale_factor = 0.2f * sqrtf(max_dim);
     const float neg_lr_scale = -lr * scale_factor / sqrtf(max_dim);
+    const float xs = scale_inv ? B.inv_norm[mi] : 1.0f;
     if (M.vec8) {
         for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
             const int i = start + k, r = i / M.cols, c = i - r * M.cols;
@@ -577,6 +580,7 @@ __global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, 
             load8(M.param, M.dtype, (size_t)i, p);
 #pragma unroll
             for (int e = 0; e < 8; e++) {
+                o[e] *= xs;
                 if (M.dtype == SG_F16) o[e] = __half2float(__float2half_rn(o[e]));
                 p[e] = sg_fma(neg_lr_scale, o[e], p[e]) * decay;
             }
@@ -586,7 +590,7 @@ __global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, 
     }
     for (int k = threadIdx.x; k < cnt; k += 256) {
         const int i = start + k, r = i / M.cols, c = i - r * M.cols;
-        float o = sg::bf16_bits_to_f(X[(size_t)r * ld + c]);
+        float o = sg::bf16_bits_to_f(X[(size_t)r * ld + c]) * xs;
         if (M.dtype == SG_F16) o = __half2float(__float2half_rn(o));     // X.to(p.dtype)
         const float p = sg::load_elem(M.param, M.dtype, i);
         sg::store_elem(M.param, M.dtype, i, sg_fma(neg_lr_scale, o, p) * decay);
@@ -640,7 +644,9 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         L->pre_g[EPI_APPLY][i + 1] = L->pre_g[EPI_APPLY][i] + (M.mp / BT) * (M.np / BT);
         L->pre_t[i + 1] = L->pre_t[i] + (M.mp / 64) * (M.np / 64);
     }
-    L->off_partials = take(sizeof(double) * (size_t)(etiles + 1));
+    int64_t ttiles = 0;
+    for (int i = 0; i < P; i++) ttiles += (int64_t)(L->mats[i].mp / 64) * (L->mats[i].np / 64);
+    L->off_partials = take(sizeof(double) * (size_t)(ttiles + 1));
     L->off_inv = take(sizeof(float) * (size_t)P);
     L->off_buffers = o;
     for (int i = 0; i < P; i++) {
@@ -728,18 +734,17 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
                            reinterpret_cast<uint4*>(ws + L.off_buffers), n16);
     }
 
-    hipLaunchKernelGGL(k_momentum, dim3(B.etiles), dim3(256), 0, st, B, momentum);
+    hipLaunchKernelGGL(k_momentum, dim3(B.ttiles), dim3(256), 0, st, B, momentum, ns_steps == 0 ? 1 : 0);
     hipLaunchKernelGGL(k_norm, dim3(P), dim3(256), 0, st, B);
-    hipLaunchKernelGGL(k_normalize, dim3(B.ttiles), dim3(256), 0, st, B, ns_steps == 0 ? 1 : 0);
     SG_LAUNCH_CHECK("muon prologue");
     for (int it = 0; it < ns_steps; it++) {
-        const int sel = it & 1, last = it + 1 == ns_steps;
+        const int sel = it & 1, last = (it + 1 == ns_steps ? 1 : 0) | (it == 0 ? 2 : 0);     // iter_flags
         hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         SG_LAUNCH_CHECK("muon newton-schulz");
     }
-    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1);
+    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1, ns_steps == 0 ? 1 : 0);
     SG_LAUNCH_CHECK("k_update");
     return 0;
 }
