@@ -23,8 +23,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (read + written) on the 25M-element workload: constants copied from the rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE summary under profiles/ (scaled by what the same counters read for a 1 GiB device copy);
 # not measured by this script and valid for the default workload only
-PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.623e9 + 1.618e9, "scan_summary": 0.042e9 + 0.037e9,
-                             "elementwise": 2.603e9 + 0.801e9}
+PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.420e9 + 1.619e9, "scan_summary": 0.028e9 + 0.037e9,
+                             "elementwise": 2.503e9 + 0.801e9}
 
 
 LARGE_GEOMETRY = dict(d_model=16, d_state=32, d_inner=32)     # the second scan geometry the kernels are built for
