@@ -40,9 +40,16 @@ SgDims default_dims(int d_model, int d_state, int d_inner) { return SgDims{d_mod
 struct ScanWeights {
     torch::Tensor t[20];          // input_proj W, b; forward block (9); backward block (9)
     Sg2Weights W;
-    void fill(const char* fn) {
+    void fill(const char* fn, const SgDims& d) {
+        // element counts in argument order: input_proj W [d_model, 2], b [d_model]; per direction in_proj [2 d_inner, d_model],
+        // dt_W [d_inner, d_inner], dt_b [d_inner], B_proj / C_proj [d_state, d_inner], A_log [d_inner, d_state], D [d_inner],
+        // rope [d_inner, d_state/2], out_proj [d_model, d_inner]
+        const int64_t dm = d.d_model, ds = d.d_state, di = d.d_inner;
+        const int64_t block[9] = {2 * di * dm, di * di, di, ds * di, ds * di, di * ds, di, di * (ds / 2), dm * di};
         for (int k = 0; k < 20; k++) {
             require_f32_gpu(t[k], fn, "meta-net weight");
+            const int64_t want = k == 0 ? 2 * dm : (k == 1 ? dm : block[(k - 2) % 9]);
+            TORCH_CHECK(t[k].numel() == want, fn, ": meta-net weight ", k, " has ", t[k].numel(), " elements, expected ", want);
             W.w[k] = t[k].data_ptr<float>();
         }
         for (int k = 20; k < SG2_NUM_WEIGHTS; k++) W.w[k] = W.w[0];      // per-element weights: never read by sort and scan
@@ -132,7 +139,7 @@ void supergrok2_bilevel_fwd_save_batched(
                                  mamba_bwd_dt_W, mamba_bwd_dt_b, mamba_bwd_B_proj, mamba_bwd_C_proj, mamba_bwd_A_log, mamba_bwd_D,
                                  mamba_bwd_rope, mamba_bwd_out_proj};
     for (int k = 0; k < 20; k++) S.w.t[k] = w[k];
-    S.w.fill(fn);
+    S.w.fill(fn, dims);
     S.grads = grads;
     S.sharps = sharpness_list;
     const int64_t P = (int64_t)grads.size();
@@ -245,7 +252,7 @@ void supergrok2_bilevel_fwd_save(
                                  mamba_bwd_dt_W, mamba_bwd_dt_b, mamba_bwd_B_proj, mamba_bwd_C_proj, mamba_bwd_A_log, mamba_bwd_D,
                                  mamba_bwd_rope, mamba_bwd_out_proj};
     for (int k = 0; k < 20; k++) S.w.t[k] = w[k];
-    S.w.fill(fn);
+    S.w.fill(fn, dims);
     S.grads = {grad.contiguous()};
     S.sharps = {sharpness.contiguous()};
     S.mf = initial_states(fn, fwd_initial_state, 1, dims, input_proj_W);
