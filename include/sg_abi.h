@@ -139,7 +139,8 @@ int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int n
  * sg2_profile_enable(1) starts collecting (at most SG2_PROF_MAX_CALLS calls are
  * kept), sg2_profile_read waits for the recorded events, adds each stage's
  * elapsed milliseconds over the collected calls into ms[SG2_PROF_STAGES],
- * stores the number of calls and clears the collection. */
+ * stores the number of calls and clears the collection.  A measurement aid
+ * for one caller: while collecting, step calls must come from one thread. */
 #define SG2_PROF_STAGES 5
 #define SG2_PROF_MAX_CALLS 256
 int sg2_profile_enable(int on);
