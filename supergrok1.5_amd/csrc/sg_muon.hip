@@ -6,7 +6,10 @@
 //
 // Every matrix is worked on in its "wide" orientation Y [m x n] (m = min dim)
 // so the Gram matrix is always the small m x m one:
-//     G = Y Y^T            H = b G + c G G            Y <- a Y + H Y
+//     G = Y Y^T            H = a I + b G + c G G            Y <- H Y
+// (the a Y term rides on H's diagonal, so the apply step is one product with no third operand; the diagonal entry
+// is rounded to bf16 like every other entry of H: against the fp32 iteration this is no less accurate than adding
+// a Y in the epilogue, the error of either form is set by the rounding of G)
 // (for a tall parameter X this is X^T X and X (bG + cG^2): the reference's
 // X X^T form re-associated, 6 m^2 n instead of 6 n^2 m flops per iteration).
 // The Gram and polynomial products are "NT" GEMMs (both operands K-contiguous).
@@ -14,10 +17,11 @@
 // the slow one.  Its tiles are staged in LDS as they lie in memory
 // ([k][n], n contiguous) and the MFMA operand (8 consecutive k per lane) is
 // fetched with gfx950's transposing LDS read (ds_read_b64_tr_b16), so no
-// transposed copy of Y is kept: an iteration reads Y twice and writes it once,
+// transposed copy of Y is kept: an iteration reads Y as an operand of two products and writes it once,
 // into the other of two buffers (the current one is still being read as the B
-// operand by other workgroups).  Only the last iteration of a tall parameter
-// also stores the transposed tile, which is the parameter's own orientation.
+// operand by other workgroups).  A tall parameter enters and leaves the wide
+// orientation in the momentum and update kernels, which transpose 64x64 tiles
+// through LDS.
 // Work buffers are zero-padded to multiples of 256 so the GEMM needs no edge
 // handling (zero rows/columns stay zero through the iteration).
 //
@@ -51,7 +55,6 @@ constexpr int LDS_ROW_KN = BT + 32; // ... of a [BK][BT] tile (576 bytes: four r
 static_assert(BK * LDS_ROW_KN == BT * LDS_ROW, "both tile layouts fill the same LDS");
 constexpr int GEMM_LDS_BYTES = 2 * 2 * BT * LDS_ROW * 2;   // two stages of {A tile, B tile}: 147,456 bytes of the CU's 160 KB
 static_assert(BK == 64, "the K loop of k_gemm_nt is written for four 16-wide steps");
-constexpr int ETILE = 4096;        // elements per tile of the elementwise kernels
 constexpr float NS_A = 3.4445f, NS_B = -4.7750f, NS_C = 2.0315f;
 
 struct Mat {
@@ -59,20 +62,17 @@ struct Mat {
     const void* grad;
     float* buf;
     bf16_t *Y, *Y2, *G, *H;       // [mp x np] twice (an iteration reads one and writes the other), [mp x mp], [mp x mp]
-    bf16_t* YT;                    // [np x mp]: the final X of a tall parameter in its own orientation
     int rows, cols, dtype;
     int m, n, mp, np;              // min / max dim and their padded sizes
     int wide;                      // rows <= cols
-    int etile0;                    // first elementwise tile of this matrix
     int vec8;                      // cols % 8 == 0 and param/grad/buf 16-byte aligned: elementwise kernels move 8 elements per lane
 };
 
 struct Batch {
     const Mat* mats;
-    const int* etile_prefix;       // [P+1] elementwise tiles (rows*cols / ETILE)
     const int* gtile_prefix[3];    // [P+1] GEMM output tiles for the three products
-    const int* ttile_prefix;       // [P+1] 64x64 transpose tiles of Y
-    int P, etiles, gtiles[3], ttiles;
+    const int* ttile_prefix;       // [P+1] 64x64 tiles of Y (the elementwise kernels work on these)
+    int P, gtiles[3], ttiles;
     double* partials;              // [ttiles] sums of squares of the 64x64 tiles
     float* inv_norm;               // [P]
 };
@@ -127,21 +127,20 @@ __device__ __forceinline__ void store8(void* p, int dtype, size_t i, const float
 // buf = momentum * buf + grad, the sum of squares of the new buf, and the new buf as bf16 into Y ([mp x np], the wide
 // orientation) - NOT yet divided by its norm, which is only known once every tile of the matrix has been summed: the
 // first iteration's Gram and apply epilogues carry the factors 1/norm^2 and 1/norm instead (bf16 rounding is relative,
-// so rounding before or after the scaling costs the same), and no separate normalisation pass reads buf again.  With
-// `both` a tall matrix also gets YT ([np x mp], its own orientation; needed when no iteration follows).
-// One 64x64 tile of the parameter's own orientation per workgroup: rows are read and written along the fast axis, the
-// transposed copy goes through LDS.  The zero padding of the work buffers is written here as well.
-__global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum, int both) {
+// so rounding before or after the scaling costs the same), and no separate normalisation pass reads buf again.
+// One 64x64 tile of the parameter's own orientation per workgroup: rows are read and written along the fast axis, a
+// tall parameter's tile is transposed through LDS.
+__global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum) {
     __shared__ bf16_t t[64][66];
     __shared__ double sm[4];
     const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
-    bf16_t* own = M.wide ? M.Y : M.YT;            // [R x C] in the parameter's orientation, padded
-    bf16_t* other = M.wide ? M.YT : M.Y;          // [C x R]
+    bf16_t* own = M.Y;                            // wide: [R x C] in the parameter's orientation, padded
+    bf16_t* other = M.Y;                          // tall: [C x R]
     const int R = M.wide ? M.mp : M.np, C = M.wide ? M.np : M.mp;
     const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
     const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
-    const bool w_own = M.wide || both, w_other = !M.wide;       // uniform over the workgroup (YT exists for tall matrices only)
+    const bool w_own = M.wide, w_other = !M.wide;               // uniform over the workgroup
     const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && M.vec8;
     double acc = 0.0;
     if (full) {
@@ -260,10 +259,9 @@ typedef short i16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) i16x4* lds_i16x4_p;
 
 // y_sel: which of the two Y buffers holds the current iterate
-// iter_flags: bit 0 = last iteration, bit 1 = first iteration (Y still carries the factor norm: see k_momentum)
+// iter_flags: bit 1 = first iteration (Y still carries the factor norm: see k_momentum)
 template <int EPI>
 __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_flags) {
-    const int last_iter = iter_flags & 1;
     constexpr bool BKN = EPI == EPI_APPLY;             // B operand stored [K x N]
     constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
     constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
@@ -288,7 +286,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     int K, lda, ldb, ldc, ldct, tm, tn;
     if (EPI == EPI_APPLY) {
         A = Mt.H; B = y_sel ? Mt.Y2 : Mt.Y; C = y_sel ? Mt.Y : Mt.Y2; K = Mt.mp; lda = Mt.mp; ldb = ldc = Mt.np;
-        CT = Mt.YT; ldct = Mt.mp;
+        CT = C; ldct = ldc;      // unused: the apply step never mirrors
         // bands of 8 tile columns: 32 tiles that run together span 4 x 8 tiles instead of 2 x 16,
         // which halves the panel bytes they pull into L2
         const int ntm = Mt.mp / BT, ntn = Mt.np / BT;
@@ -383,9 +381,9 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     };
 
     const int nk = K / BK;      // a multiple of 4: K is a multiple of 256
-    const bf16_t* aux = (EPI == EPI_POLY) ? Mt.G : (y_sel ? Mt.Y2 : Mt.Y);
+    const bf16_t* aux = Mt.G;
     const int gcol0 = tn * BT + wn * (BT / 2);
-    // the auxiliary operand of the epilogue (G for the polynomial, the current Y for the apply step):
+    // the auxiliary operand of the polynomial's epilogue (G):
     // 8 x 16 bytes per lane and 32-row block of this wave's 128 x 128 tile.  The first two blocks are requested during
     // the last K tile (whose register sets are free by then), each later one while the block two before it is
     // being written, so that the epilogue does not wait for memory
@@ -450,10 +448,10 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
         }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
-        // phase 3: k step 3 | read k step 0 of tile kt+1, load B of tile kt+3 (last tile: the epilogue's auxiliary operand)
+        // phase 3: k step 3 | read k step 0 of tile kt+1, load B of tile kt+3 (last tile: the polynomial's auxiliary operand)
         if (!LAST) lds_load(nxt, 0, 0);
         if (LD) gload_b(S, kt + 3);
-        if (LAST && EPI != EPI_GRAM) { aux_load(0); aux_load(1); }
+        if (LAST && EPI == EPI_POLY) { aux_load(0); aux_load(1); }
         mma(1);
         if (!LAST) {
             SG_MUON_SCHED_READS();
@@ -462,7 +460,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
-        } else if (EPI != EPI_GRAM) {
+        } else if (EPI == EPI_POLY) {
 #pragma unroll
             for (int g = 0; g < 16; g++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -496,11 +494,11 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     constexpr int EP_ROW = 128 + 4;     // floats per staged row
     static_assert(4 * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
     float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EP_ROW);
-    // uniform over the workgroup.  The apply step stores the transposed tile only after the last iteration of a
-    // tall matrix (its parameter update reads that orientation).
-    const bool mirror = (EPI == EPI_APPLY) ? (last_iter && !Mt.wide) : (tm != tn);
+    // uniform over the workgroup
+    const bool mirror = EPI != EPI_APPLY && tm != tn;
     // first iteration: Y is the unnormalised momentum, so its Gram matrix carries 1/norm^2 and the applied Y 1/norm
     const float inv = Bt.inv_norm[mi];
+    const bool diag_wave = EPI == EPI_POLY && tm == tn && wm == wn;     // this wave's 128 x 128 block lies on the diagonal
     const float first_scale = (iter_flags & 2) ? (EPI == EPI_GRAM ? inv * inv : (EPI == EPI_APPLY ? inv : 1.0f)) : 1.0f;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
@@ -517,12 +515,17 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
             f32x4* src = reinterpret_cast<f32x4*>(&ep[row * EP_ROW + c8 * 8]);
             const f32x4 lo = src[0], hi = src[1];
             float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            if (EPI != EPI_GRAM) {
+            if (EPI == EPI_POLY) {
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
                     const uint32_t w = ax[i & 1][c][k >> 1];
                     const float x = sg_i2f((int32_t)((k & 1) ? (w & 0xffff0000u) : (w << 16)));
-                    v[k] = (EPI == EPI_POLY) ? sg_fma(NS_C, v[k], NS_B * x) : sg_fma(NS_A, x, v[k]);
+                    v[k] = sg_fma(NS_C, v[k], NS_B * x);
+                }
+                if (diag_wave) {        // H + a I: the apply step is then the single product (H + a I) Y
+                    const int dk = i * 32 + row - c8 * 8;
+#pragma unroll
+                    for (int k = 0; k < 8; k++) v[k] += (dk == k) ? NS_A : 0.0f;
                 }
             }
             if (EPI != EPI_POLY) {
@@ -540,7 +543,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
                 reinterpret_cast<u32x4*>(src)[1] = b1;
             }
         }
-        if (EPI != EPI_GRAM && i + 2 < TM) aux_load(i + 2);
+        if (EPI == EPI_POLY && i + 2 < TM) aux_load(i + 2);
         __builtin_amdgcn_wave_barrier();
         if (mirror) {
             const uint32_t* epb = reinterpret_cast<const uint32_t*>(ep);
@@ -558,40 +561,67 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     }
 }
 
-// p = (p - 0.2*lr*X) * (1 - lr*wd), X read in the parameter's own orientation
+// p = (p - 0.2*lr*X) * (1 - lr*wd).  X lies in the wide orientation; one 64x64 tile of the parameter's own
+// orientation per workgroup (the grid of k_momentum), a tall parameter's tile of X is transposed through LDS.
 // scale_inv: no iteration ran, X is still the unnormalised momentum
 __global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, int y_sel, int scale_inv) {
-    const int mi = sg::upper_seg(B.etile_prefix, B.P, blockIdx.x);
+    __shared__ bf16_t t[64][66];
+    const int mi = sg::upper_seg(B.ttile_prefix, B.P, blockIdx.x);
     const Mat& M = B.mats[mi];
-    const int start = ((int)blockIdx.x - B.etile_prefix[mi]) * ETILE;
-    const int cnt = min(ETILE, M.rows * M.cols - start);
-    const bf16_t* X = M.wide ? (y_sel ? M.Y2 : M.Y) : M.YT;
-    const int ld = M.wide ? M.np : M.mp;
+    const bf16_t* X = y_sel ? M.Y2 : M.Y;         // [mp x np]
+    const int C = M.wide ? M.np : M.mp;           // padded columns of the parameter's orientation
+    const int tile = (int)blockIdx.x - B.ttile_prefix[mi];
+    const int tc = C / 64, tr0 = (tile / tc) * 64, tc0 = (tile % tc) * 64;
+    if (tr0 >= M.rows || tc0 >= M.cols) return;   // padding only (uniform over the workgroup)
     // the reference's scalar arithmetic (csrc/ops.cpp:729-734)
     const float max_dim = (float)max(M.rows, M.cols);
     const float scale_factor = 0.2f * sqrtf(max_dim);
     const float neg_lr_scale = -lr * scale_factor / sqrtf(max_dim);
     const float xs = scale_inv ? B.inv_norm[mi] : 1.0f;
-    if (M.vec8) {
-        for (int k = threadIdx.x * 8; k < cnt; k += 256 * 8) {
-            const int i = start + k, r = i / M.cols, c = i - r * M.cols;
-            float o[8], p[8];
-            load8(X, SG_BF16, (size_t)r * ld + c, o);
-            load8(M.param, M.dtype, (size_t)i, p);
+    const bool full = tr0 + 64 <= M.rows && tc0 + 64 <= M.cols && M.vec8;
+    const int lr_ = threadIdx.x >> 2, c0 = (threadIdx.x & 3) * 16;
+    if (!M.wide) {
+        // X tile: rows = the parameter's columns tc0.., columns = its rows tr0.. (the padded buffer covers all of it)
+        const u32x4* src = reinterpret_cast<const u32x4*>(X + (size_t)(tc0 + lr_) * M.np + tr0 + c0);
+        const u32x4 w0 = src[0], w1 = src[1];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                o[e] *= xs;
-                if (M.dtype == SG_F16) o[e] = __half2float(__float2half_rn(o[e]));
-                p[e] = sg_fma(neg_lr_scale, o[e], p[e]) * decay;
-            }
-            store8(M.param, M.dtype, (size_t)i, p);
+        for (int q = 0; q < 4; q++) {
+            t[lr_][c0 + 2 * q] = (bf16_t)(w0[q] & 0xffffu);
+            t[lr_][c0 + 2 * q + 1] = (bf16_t)(w0[q] >> 16);
+            t[lr_][c0 + 8 + 2 * q] = (bf16_t)(w1[q] & 0xffffu);
+            t[lr_][c0 + 8 + 2 * q + 1] = (bf16_t)(w1[q] >> 16);
         }
+        __syncthreads();
+    }
+    if (full) {
+        // interior tile: a lane moves 16 consecutive elements of a row
+        const size_t at = (size_t)(tr0 + lr_) * M.cols + tc0 + c0;
+        float o[16], p[16];
+        if (M.wide) {
+            load8(X, SG_BF16, (size_t)(tr0 + lr_) * M.np + tc0 + c0, o);
+            load8(X, SG_BF16, (size_t)(tr0 + lr_) * M.np + tc0 + c0 + 8, o + 8);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; e++) o[e] = sg::bf16_bits_to_f(t[c0 + e][lr_]);
+        }
+        load8(M.param, M.dtype, at, p);
+        load8(M.param, M.dtype, at + 8, p + 8);
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            o[e] *= xs;
+            if (M.dtype == SG_F16) o[e] = __half2float(__float2half_rn(o[e]));     // X.to(p.dtype)
+            p[e] = sg_fma(neg_lr_scale, o[e], p[e]) * decay;
+        }
+        store8(M.param, M.dtype, at, p);
+        store8(M.param, M.dtype, at + 8, p + 8);
         return;
     }
-    for (int k = threadIdx.x; k < cnt; k += 256) {
-        const int i = start + k, r = i / M.cols, c = i - r * M.cols;
-        float o = sg::bf16_bits_to_f(X[(size_t)r * ld + c]) * xs;
-        if (M.dtype == SG_F16) o = __half2float(__float2half_rn(o));     // X.to(p.dtype)
+    for (int k = threadIdx.x; k < 64 * 64; k += 256) {
+        const int r = tr0 + (k >> 6), c = tc0 + (k & 63);
+        if (r >= M.rows || c >= M.cols) continue;
+        float o = sg::bf16_bits_to_f(M.wide ? X[(size_t)r * M.np + c] : t[k & 63][k >> 6]) * xs;
+        if (M.dtype == SG_F16) o = __half2float(__float2half_rn(o));
+        const int64_t i = (int64_t)r * M.cols + c;
         const float p = sg::load_elem(M.param, M.dtype, i);
         sg::store_elem(M.param, M.dtype, i, sg_fma(neg_lr_scale, o, p) * decay);
     }
@@ -606,23 +636,20 @@ inline int round_up(int x, int a) { return (x + a - 1) / a * a; }
 struct Layout {
     int P;
     std::vector<Mat> mats;
-    std::vector<int> pre_e, pre_g[3], pre_t;
-    size_t off_mats, off_pre_e, off_pre_g[3], off_pre_t, off_partials, off_inv, off_buffers, bytes;
+    std::vector<int> pre_g[3], pre_t;
+    size_t off_mats, off_pre_g[3], off_pre_t, off_partials, off_inv, off_buffers, bytes;
 };
 
 int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
     L->P = P;
     L->mats.resize(P);
-    L->pre_e.assign(P + 1, 0);
     for (int k = 0; k < 3; k++) L->pre_g[k].assign(P + 1, 0);
     L->pre_t.assign(P + 1, 0);
     size_t o = 0;
     auto take = [&](size_t b) { size_t r = o; o = sg::align_up(o + b, 256); return r; };
     L->off_mats = take(sizeof(Mat) * (size_t)P);
-    L->off_pre_e = take(sizeof(int) * (size_t)(P + 1));
     for (int k = 0; k < 3; k++) L->off_pre_g[k] = take(sizeof(int) * (size_t)(P + 1));
     L->off_pre_t = take(sizeof(int) * (size_t)(P + 1));
-    int64_t etiles = 0;
     for (int i = 0; i < P; i++) {
         const SgMuonMatrix& s = in[i];
         if (s.rows <= 0 || s.cols <= 0 || s.rows * s.cols > 0x7fffffff) return sg::fail("matrix %d: bad shape %lld x %lld", i, (long long)s.rows, (long long)s.cols);
@@ -634,10 +661,6 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         M.vec8 = (s.cols % 8 == 0) && ((((uintptr_t)s.param | (uintptr_t)s.grad | (uintptr_t)s.buf) & 15u) == 0);
         M.m = (int)std::min(s.rows, s.cols); M.n = (int)std::max(s.rows, s.cols);
         M.mp = round_up(M.m, BT); M.np = round_up(M.n, BT);
-        const int et = (int)((s.rows * s.cols + ETILE - 1) / ETILE);
-        M.etile0 = (int)etiles;
-        etiles += et;
-        L->pre_e[i + 1] = L->pre_e[i] + et;
         const int nt = M.mp / BT, tri = nt * (nt + 1) / 2;      // symmetric products: tiles on or above the diagonal
         L->pre_g[EPI_GRAM][i + 1] = L->pre_g[EPI_GRAM][i] + tri;
         L->pre_g[EPI_POLY][i + 1] = L->pre_g[EPI_POLY][i] + tri;
@@ -654,7 +677,6 @@ int make_layout(int P, const SgMuonMatrix* in, Layout* L) {
         // offsets for now; turned into pointers once the workspace base is known
         M.Y = (bf16_t*)take(2 * (size_t)M.mp * M.np);
         M.Y2 = (bf16_t*)take(2 * (size_t)M.mp * M.np);
-        M.YT = (bf16_t*)take(M.wide ? 0 : 2 * (size_t)M.mp * M.np);
         M.G = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
         M.H = (bf16_t*)take(2 * (size_t)M.mp * M.mp);
     }
@@ -690,22 +712,19 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
     unsigned char* ws = static_cast<unsigned char*>(workspace);
     const int P = L.P;
     for (auto& M : L.mats) {
-        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.Y2 = (bf16_t*)(ws + (size_t)M.Y2); M.YT = (bf16_t*)(ws + (size_t)M.YT);
+        M.Y = (bf16_t*)(ws + (size_t)M.Y); M.Y2 = (bf16_t*)(ws + (size_t)M.Y2);
         M.G = (bf16_t*)(ws + (size_t)M.G); M.H = (bf16_t*)(ws + (size_t)M.H);
     }
     // per-call tables: through kernel arguments (no host-to-device copy, nothing blocks the host)
     if (sg::upload_words(ws + L.off_mats, L.mats.data(), sizeof(Mat) * (size_t)P, st)) return 1;
-    if (sg::upload_words(ws + L.off_pre_e, L.pre_e.data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
     for (int k = 0; k < 3; k++)
         if (sg::upload_words(ws + L.off_pre_g[k], L.pre_g[k].data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
     if (sg::upload_words(ws + L.off_pre_t, L.pre_t.data(), sizeof(int) * (size_t)(P + 1), st)) return 1;
     Batch B;
     B.mats = reinterpret_cast<const Mat*>(ws + L.off_mats);
-    B.etile_prefix = reinterpret_cast<const int*>(ws + L.off_pre_e);
     for (int k = 0; k < 3; k++) B.gtile_prefix[k] = reinterpret_cast<const int*>(ws + L.off_pre_g[k]);
     B.ttile_prefix = reinterpret_cast<const int*>(ws + L.off_pre_t);
     B.P = P;
-    B.etiles = L.pre_e[P];
     for (int k = 0; k < 3; k++) B.gtiles[k] = L.pre_g[k][P];
     B.ttiles = L.pre_t[P];
     B.partials = reinterpret_cast<double*>(ws + L.off_partials);
@@ -734,17 +753,17 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
                            reinterpret_cast<uint4*>(ws + L.off_buffers), n16);
     }
 
-    hipLaunchKernelGGL(k_momentum, dim3(B.ttiles), dim3(256), 0, st, B, momentum, ns_steps == 0 ? 1 : 0);
+    hipLaunchKernelGGL(k_momentum, dim3(B.ttiles), dim3(256), 0, st, B, momentum);
     hipLaunchKernelGGL(k_norm, dim3(P), dim3(256), 0, st, B);
     SG_LAUNCH_CHECK("muon prologue");
     for (int it = 0; it < ns_steps; it++) {
-        const int sel = it & 1, last = (it + 1 == ns_steps ? 1 : 0) | (it == 0 ? 2 : 0);     // iter_flags
+        const int sel = it & 1, last = it == 0 ? 2 : 0;     // iter_flags
         hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
         SG_LAUNCH_CHECK("muon newton-schulz");
     }
-    hipLaunchKernelGGL(k_update, dim3(B.etiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1, ns_steps == 0 ? 1 : 0);
+    hipLaunchKernelGGL(k_update, dim3(B.ttiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1, ns_steps == 0 ? 1 : 0);
     SG_LAUNCH_CHECK("k_update");
     return 0;
 }
