@@ -226,6 +226,7 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
 enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
 // explicit global address space: a generic (flat) load would count against the LDS wait counter as well
 typedef const __attribute__((address_space(1))) u32x4* gvec_p;
+typedef __attribute__((address_space(1))) u32x4* gvec_w;
 
 // two floats rounded to bf16 (nearest even, NaN stays NaN), packed lo | hi << 16: one v_cvt_pk_bf16_f32 on gfx950
 __device__ __forceinline__ uint32_t bf16r2(float lo, float hi) {
@@ -499,7 +500,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     // first iteration: Y is the unnormalised momentum, so its Gram matrix carries 1/norm^2 and the applied Y 1/norm
     const float inv = Bt.inv_norm[mi];
     const bool diag_wave = EPI == EPI_POLY && tm == tn && wm == wn;     // this wave's 128 x 128 block lies on the diagonal
-    const float first_scale = (iter_flags & 2) ? (EPI == EPI_GRAM ? inv * inv : (EPI == EPI_APPLY ? inv : 1.0f)) : 1.0f;
+    const bool first = (iter_flags & 2) != 0;
+    const float first_scale = first ? (EPI == EPI_GRAM ? inv * inv : (EPI == EPI_APPLY ? inv : 1.0f)) : 1.0f;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int grow0 = tm * BT + wm * (BT / 2) + i * 32;
@@ -528,14 +530,14 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
                     for (int k = 0; k < 8; k++) v[k] += (dk == k) ? NS_A : 0.0f;
                 }
             }
-            if (EPI != EPI_POLY) {
+            if (EPI != EPI_POLY && first) {      // uniform over the grid
 #pragma unroll
-                for (int k = 0; k < 8; k++) v[k] *= first_scale;        // 1 except in the first iteration
+                for (int k = 0; k < 8; k++) v[k] *= first_scale;
             }
             u32x4 out;
 #pragma unroll
             for (int k = 0; k < 4; k++) out[k] = bf16r2(v[2 * k], v[2 * k + 1]);
-            *reinterpret_cast<u32x4*>(C + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8) = out;
+            *(gvec_w)(C + (size_t)(grow0 + row) * ldc + gcol0 + c8 * 8) = out;
             if (mirror) {   // rounded values (as bf16 bit patterns) back into the staged block
                 u32x4 b0 = {out[0] & 0xffffu, out[0] >> 16, out[1] & 0xffffu, out[1] >> 16};
                 u32x4 b1 = {out[2] & 0xffffu, out[2] >> 16, out[3] & 0xffffu, out[3] >> 16};
@@ -554,7 +556,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
 #pragma unroll
                 for (int k = 0; k < 4; k++)
                     t[k] = epb[(r8 * 8 + 2 * k) * EP_ROW + col] | (epb[(r8 * 8 + 2 * k + 1) * EP_ROW + col] << 16);
-                *reinterpret_cast<u32x4*>(CT + (size_t)(gcol0 + col) * ldct + grow0 + r8 * 8) = t;
+                *(gvec_w)(CT + (size_t)(gcol0 + col) * ldct + grow0 + r8 * 8) = t;
             }
             __builtin_amdgcn_wave_barrier();
         }
