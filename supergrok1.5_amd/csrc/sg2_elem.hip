@@ -21,6 +21,7 @@ namespace {
 
 constexpr int ELEM_THREADS = 256;
 constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[16] W2[16] + pad
+typedef float vf4 __attribute__((ext_vector_type(4)));
 
 template <class G, bool DBG>
 __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
@@ -77,17 +78,20 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             const float s = has_s ? sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i)) : 0.0f;
             float cf[DM], cb[DM], hold[GH];
             {
-                const float4* pf = reinterpret_cast<const float4*>(pl.ctx + ((size_t)T.off + i) * DM);
-                const float4* pb = reinterpret_cast<const float4*>(pl.ctx + ((size_t)pl.total + T.off + i) * DM);
+                const SG_GLOBAL vf4* pf = (const SG_GLOBAL vf4*)(pl.ctx + ((size_t)T.off + i) * DM);
+                const SG_GLOBAL vf4* pb = (const SG_GLOBAL vf4*)(pl.ctx + ((size_t)pl.total + T.off + i) * DM);
 #pragma unroll
                 for (int q = 0; q < DM / 4; q++) {
-                    const float4 a = pf[q], b = pb[q];
-                    cf[4 * q] = a.x; cf[4 * q + 1] = a.y; cf[4 * q + 2] = a.z; cf[4 * q + 3] = a.w;
-                    cb[4 * q] = b.x; cb[4 * q + 1] = b.y; cb[4 * q + 2] = b.z; cb[4 * q + 3] = b.w;
+                    const vf4 a = pf[q], b = pb[q];
+                    cf[4 * q] = a[0]; cf[4 * q + 1] = a[1]; cf[4 * q + 2] = a[2]; cf[4 * q + 3] = a[3];
+                    cb[4 * q] = b[0]; cb[4 * q + 1] = b[1]; cb[4 * q + 2] = b[2]; cb[4 * q + 3] = b[3];
                 }
-                const float4 h4 = reinterpret_cast<const float4*>(T.gru)[i];
-                hold[0] = h4.x; hold[1] = h4.y; hold[2] = h4.z; hold[3] = h4.w;
+                const vf4 h4 = ((const SG_GLOBAL vf4*)T.gru)[i];
+                hold[0] = h4[0]; hold[1] = h4[1]; hold[2] = h4[2]; hold[3] = h4[3];
             }
+            // the optimizer state is requested now, so that its latency passes under the meta-net's arithmetic
+            float mu = sg::gptr(T.mu)[i], ea = sg::gptr(T.ea)[i], easq = sg::gptr(T.easq)[i];
+            float pv = sg::load_elem(T.param, dtype, i);
 
             // ---- GRU: chain order = bias, g, s, fwd ctx, bwd ctx, h
             float zg[GH], rg[GH], hnew[GH];
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 const float ht = sg_tanh(v);
                 hnew[j] = sg_fma(zg[j], ht, (1.0f - zg[j]) * hold[j]);
             }
-            reinterpret_cast<float4*>(T.gru)[i] = make_float4(hnew[0], hnew[1], hnew[2], hnew[3]);
+            ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
 
             // ---- PEER routing + expert MLP
             float total = 0.0f;
@@ -178,17 +182,14 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             const float smart = g + (rescale * total) / (float)NH;
 
             // ---- mu EMA, Adam moments, decoupled weight decay
-            float mu = T.mu[i];
             mu = sg_fma(alpha, mu, (1.0f - alpha) * g);
-            T.mu[i] = mu;
+            sg::gptr(T.mu)[i] = mu;
             const float fg = sg_fma(lamb, mu, smart);
-            float ea = T.ea[i], easq = T.easq[i];
             ea = sg_fma(beta1, ea, (1.0f - beta1) * fg);
             easq = sg_fma(beta2, easq, ((1.0f - beta2) * fg) * fg);
-            T.ea[i] = ea;
-            T.easq[i] = easq;
+            sg::gptr(T.ea)[i] = ea;
+            sg::gptr(T.easq)[i] = easq;
             const float denom = __builtin_sqrtf(easq / bc2) + eps;
-            float pv = sg::load_elem(T.param, dtype, i);
             pv = sg_fma(pv, decay, -((step_size * ea) / denom));
             sg::store_elem(T.param, dtype, i, pv);
         }

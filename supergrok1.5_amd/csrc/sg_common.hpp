@@ -47,15 +47,20 @@ __device__ __forceinline__ uint16_t f_to_bf16_bits(float f) {
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
 }
+// Device buffers handed in by the caller are addressed in the global address space: a generic (flat) access also
+// counts against the wait counter of LDS, so a kernel that uses both would wait for memory whenever it waits for LDS.
+#define SG_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ SG_GLOBAL T* gptr(T* p) { return (SG_GLOBAL T*)p; }
 __device__ __forceinline__ float load_elem(const void* p, int dtype, int64_t i) {
-    if (dtype == SG_F32) return ((const float*)p)[i];
-    if (dtype == SG_F16) return __half2float(((const __half*)p)[i]);
-    return bf16_bits_to_f(((const uint16_t*)p)[i]);
+    if (dtype == SG_F32) return ((const SG_GLOBAL float*)p)[i];
+    if (dtype == SG_F16) return __half2float(__ushort_as_half(((const SG_GLOBAL uint16_t*)p)[i]));
+    return bf16_bits_to_f(((const SG_GLOBAL uint16_t*)p)[i]);
 }
 __device__ __forceinline__ void store_elem(void* p, int dtype, int64_t i, float v) {
-    if (dtype == SG_F32) ((float*)p)[i] = v;
-    else if (dtype == SG_F16) ((__half*)p)[i] = __float2half_rn(v);
-    else ((uint16_t*)p)[i] = f_to_bf16_bits(v);
+    if (dtype == SG_F32) ((SG_GLOBAL float*)p)[i] = v;
+    else if (dtype == SG_F16) ((SG_GLOBAL uint16_t*)p)[i] = __half_as_ushort(__float2half_rn(v));
+    else ((SG_GLOBAL uint16_t*)p)[i] = f_to_bf16_bits(v);
 }
 __device__ __forceinline__ float finite_or_zero(float v) { return sg_isfinite(v) ? v : 0.0f; }
 

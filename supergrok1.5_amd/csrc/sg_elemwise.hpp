@@ -147,7 +147,7 @@ __global__ __launch_bounds__(THREADS) void k_sumsq_partial(Batch<NormRec> B) {
         typedef float f32x4 __attribute__((ext_vector_type(4)));
         done = cnt & ~3;
         for (int k = threadIdx.x * 4; k < done; k += THREADS * 4) {
-            const f32x4 g = *reinterpret_cast<const f32x4*>(static_cast<const float*>(R.grad) + start + k);
+            const f32x4 g = *(const SG_GLOBAL f32x4*)(static_cast<const float*>(R.grad) + start + k);
             acc = sg_fma(g[0], g[0], acc);
             acc = sg_fma(g[1], g[1], acc);
             acc = sg_fma(g[2], g[2], acc);

@@ -31,8 +31,8 @@ struct FamRec {
 };
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ f32x4 ld4(const void* p, int i) { return *reinterpret_cast<const f32x4*>(static_cast<const float*>(p) + i); }
-__device__ __forceinline__ void st4(void* p, int i, f32x4 v) { *reinterpret_cast<f32x4*>(static_cast<float*>(p) + i) = v; }
+__device__ __forceinline__ f32x4 ld4(const void* p, int i) { return *(const SG_GLOBAL f32x4*)(static_cast<const float*>(p) + i); }
+__device__ __forceinline__ void st4(void* p, int i, f32x4 v) { *(SG_GLOBAL f32x4*)(static_cast<float*>(p) + i) = v; }
 
 // Runs body(i) for every element of the tile; when the tensor allows 16-byte accesses, body4(i) handles four
 // consecutive elements per lane and body(i) only the ragged end.

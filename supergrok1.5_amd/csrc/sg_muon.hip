@@ -94,12 +94,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // eight consecutive elements in the tensor's storage type; i a multiple of 8, base 16-byte aligned
 __device__ __forceinline__ void load8(const void* p, int dtype, size_t i, float v[8]) {
     if (dtype == SG_F32) {
-        const f32x4* q = reinterpret_cast<const f32x4*>(static_cast<const float*>(p) + i);
+        const SG_GLOBAL f32x4* q = (const SG_GLOBAL f32x4*)(static_cast<const float*>(p) + i);
         const f32x4 a = q[0], b = q[1];
 #pragma unroll
         for (int k = 0; k < 4; k++) { v[k] = a[k]; v[4 + k] = b[k]; }
     } else {
-        const u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(p) + i);
+        const u32x4 w = *(const SG_GLOBAL u32x4*)(static_cast<const uint16_t*>(p) + i);
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const uint16_t h = (uint16_t)((k & 1) ? (w[k >> 1] >> 16) : (w[k >> 1] & 0xffffu));
@@ -109,7 +109,7 @@ __device__ __forceinline__ void load8(const void* p, int dtype, size_t i, float 
 }
 __device__ __forceinline__ void store8(void* p, int dtype, size_t i, const float v[8]) {
     if (dtype == SG_F32) {
-        f32x4* q = reinterpret_cast<f32x4*>(static_cast<float*>(p) + i);
+        SG_GLOBAL f32x4* q = (SG_GLOBAL f32x4*)(static_cast<float*>(p) + i);
         q[0] = f32x4{v[0], v[1], v[2], v[3]};
         q[1] = f32x4{v[4], v[5], v[6], v[7]};
     } else {
@@ -120,7 +120,7 @@ __device__ __forceinline__ void store8(void* p, int dtype, size_t i, const float
             const uint32_t hi = (dtype == SG_F16) ? __half_as_ushort(__float2half_rn(v[2 * k + 1])) : sg::f_to_bf16_bits(v[2 * k + 1]);
             w[k] = lo | (hi << 16);
         }
-        *reinterpret_cast<u32x4*>(static_cast<uint16_t*>(p) + i) = w;
+        *(SG_GLOBAL u32x4*)(static_cast<uint16_t*>(p) + i) = w;
     }
 }
 
@@ -166,18 +166,18 @@ __global__ __launch_bounds__(256) void k_momentum(Batch B, float momentum) {
             t[lr][c0 + 2 * q + 1] = (bf16_t)b1;
         }
         if (w_own) {
-            uint4* dst = reinterpret_cast<uint4*>(own + (size_t)(tr0 + lr) * C + tc0 + c0);
-            dst[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-            dst[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+            SG_GLOBAL u32x4* dst = (SG_GLOBAL u32x4*)(own + (size_t)(tr0 + lr) * C + tc0 + c0);
+            dst[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+            dst[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
         }
         if (w_other) {
             __syncthreads();
             // transposed copy: output row lr (= own column), 16 consecutive output columns (= own rows)
 #pragma unroll
             for (int q = 0; q < 8; q++) pk[q] = (uint32_t)t[c0 + 2 * q][lr] | ((uint32_t)t[c0 + 2 * q + 1][lr] << 16);
-            uint4* dt = reinterpret_cast<uint4*>(other + (size_t)(tc0 + lr) * R + tr0 + c0);
-            dt[0] = make_uint4(pk[0], pk[1], pk[2], pk[3]);
-            dt[1] = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+            SG_GLOBAL u32x4* dt = (SG_GLOBAL u32x4*)(other + (size_t)(tc0 + lr) * R + tr0 + c0);
+            dt[0] = u32x4{pk[0], pk[1], pk[2], pk[3]};
+            dt[1] = u32x4{pk[4], pk[5], pk[6], pk[7]};
         }
     } else {
         float part = 0.0f;
@@ -584,7 +584,7 @@ __global__ __launch_bounds__(256) void k_update(Batch B, float lr, float decay, 
     const int lr_ = threadIdx.x >> 2, c0 = (threadIdx.x & 3) * 16;
     if (!M.wide) {
         // X tile: rows = the parameter's columns tc0.., columns = its rows tr0.. (the padded buffer covers all of it)
-        const u32x4* src = reinterpret_cast<const u32x4*>(X + (size_t)(tc0 + lr_) * M.np + tr0 + c0);
+        const SG_GLOBAL u32x4* src = (const SG_GLOBAL u32x4*)(X + (size_t)(tc0 + lr_) * M.np + tr0 + c0);
         const u32x4 w0 = src[0], w1 = src[1];
 #pragma unroll
         for (int q = 0; q < 4; q++) {
