@@ -94,11 +94,12 @@ int sg2_get_chunk_len(void);
 int sg2_chunk_len_for(int num_tensors, const int64_t* numels);
 
 /* Summary window of the scan (timesteps, a multiple of 64; 0 disables, a
- * negative value restores the default 256).  The recurrence contracts, so a
+ * negative value restores the default, SG2_DEFAULT_SCAN_WINDOW).  The recurrence contracts, so a
  * chunk summary is built backwards in blocks of `window` steps and the walk
  * stops as soon as every entry of the 2x2 part of the running summary is below
  * 2^-100 (the chunk summary is then (0, b)); a chunk that never contracts is
  * covered completely.  Takes effect when window < chunk_len. */
+#define SG2_DEFAULT_SCAN_WINDOW 64
 int sg2_set_scan_window(int window);
 int sg2_get_scan_window(void);
 

@@ -487,7 +487,7 @@ __global__ __launch_bounds__(256) void k_sum_partials(const float* __restrict__ 
 
 constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD);
 static_assert(2 * BE_LDS_BYTES <= 160 * 1024, "two workgroups of k_bilevel_elem per CU");
-constexpr int BE_MAX_GROUPS = 1024;
+constexpr int BE_MAX_GROUPS = 512;       // two resident workgroups on each of the 256 CUs: one round, every workgroup walks the same number of tiles (+-1)
 
 int elem_groups(int64_t total) {
     const int64_t tiles = (total + BE_THREADS - 1) / BE_THREADS;

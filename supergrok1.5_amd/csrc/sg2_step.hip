@@ -21,7 +21,7 @@ namespace {
 // process-wide settings (atomic: a call reads each once; changing them while other threads are inside a call only
 // affects calls that start later)
 std::atomic<int> g_chunk_len{0};      // 0: chosen per call from the amount of work, see auto_chunk_len
-std::atomic<int> g_window{256};
+std::atomic<int> g_window{SG2_DEFAULT_SCAN_WINDOW};
 
 // What the forward call of the bilevel pass laid out in a workspace, so that the backward call addresses it the same
 // way whatever the settings are by then.  Keyed by the workspace address.
@@ -222,7 +222,7 @@ int sg2_chunk_len_for(int num_tensors, const int64_t* numels) {
 }
 
 int sg2_set_scan_window(int window) {
-    if (window < 0) window = 256;
+    if (window < 0) window = SG2_DEFAULT_SCAN_WINDOW;
     if (window % sg2::SCAN_TT) return sg::fail("scan window must be a multiple of %d (0 disables it)", sg2::SCAN_TT);
     sg2::g_window = window;
     return 0;

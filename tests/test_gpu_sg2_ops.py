@@ -9,6 +9,7 @@ import workloads as wl
 from helpers import DIMS
 from sg2_harness import Sg2Case, per_tensor_scalars, shared_scalars, to_np
 from oracle import oracle as orc
+from grokking_optimizers import _cabi
 from helpers import rel_close
 
 pytestmark = pytest.mark.gpu
@@ -98,7 +99,7 @@ def test_supergrok2_class_against_checker_with_recycling():
             b1 = 0.9 * (0.9 ** i)
             sc = dict(alpha=f32(0.98), lamb_eff=f32(lamb_eff), beta1=f32(b1), bc1=f32(1.0 - b1 ** t), bc2=f32(1.0 - 0.999 ** t),
                       rescale=f32(0.1), beta2=f32(0.999), lr=f32(1e-3), wd_eff=f32(wd_eff), eps=f32(1e-8))
-            orc.sg2_step(W, ref[i], np.ascontiguousarray(gi, np.float32), np.zeros_like(gn), sc, chunk_len=1024, window=256,   # 745 elements: the automatic choice is 1024
+            orc.sg2_step(W, ref[i], np.ascontiguousarray(gi, np.float32), np.zeros_like(gn), sc, chunk_len=1024, window=_cabi.lib().sg2_get_scan_window(),   # 745 elements: the automatic choice is 1024
                         
                          expert_counts=step_counts)
         for i, p in enumerate(params):

@@ -32,7 +32,7 @@ def test_seeded_configuration(seed):
     shapes = [(int(SIZES[i]),) for i in r.choice(len(SIZES), size=P)]
     dtypes = [[torch.float32, torch.float32, torch.bfloat16, torch.float16][int(r.randint(4))] for _ in range(P)]
     chunk = [0, 64, 256, 1024][int(r.randint(4))]
-    window = [-1, 0, 64][int(r.randint(3))]
+    window = [-1, 0, 256][int(r.randint(3))]
     dims = LARGE if seed % 3 == 2 else None
     with_sharp = [bool(r.randint(2)) for _ in range(P)]
     print("sweep", seed, shapes, [str(d) for d in dtypes], "chunk", chunk, "window", window, "large" if dims else "default",
