@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (read + written) on the 25M-element workload: constants copied from the rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE summary under profiles/ (scaled by what the same counters read for a 1 GiB device copy);
 # not measured by this script and valid for the default workload only
-PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.420e9 + 1.619e9, "scan_summary": 0.028e9 + 0.037e9,
+PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.420e9 + 1.619e9, "scan_summary": 0.022e9 + 0.037e9,
                              "elementwise": 2.503e9 + 0.801e9}
 
 
