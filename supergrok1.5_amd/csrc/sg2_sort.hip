@@ -8,7 +8,7 @@
 //
 // Four passes of 8 bits over tiles of 8192 keys (512 lanes x 16).  Per pass:
 //   hist     per-tile digit counts -> spine[segment][digit][tile]  (first pass: counted while the keys are made)
-//   scan     exclusive prefix over the whole spine (3 small kernels).  Because
+//   scan     exclusive prefix over the whole spine (3 small kernels; one for small models).  Because
 //            the spine is laid out segment-major, the global prefix of entry
 //            (seg, d, tile) is exactly: keys in earlier segments + keys of this
 //            segment with a smaller digit + keys with digit d in earlier tiles
@@ -186,6 +186,35 @@ __global__ __launch_bounds__(256) void k_spine_down(uint32_t* spine, const uint3
     }
 }
 
+// The whole scan in one workgroup, for spines of at most SPINE_SINGLE_MAX entries (a model of up to a million
+// elements): three dependent launches of a few microseconds each cost more than the scan itself there.
+constexpr int SPINE_SINGLE_MAX = 32768;
+__global__ __launch_bounds__(1024) void k_spine_single(uint32_t* spine, int n /* a multiple of 256 */) {
+    __shared__ uint32_t sm[16];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    uint32_t carry = 0;
+    for (int base = 0; base < n; base += 4096) {
+        const int i = base + (int)threadIdx.x * 4;
+        uint4 v = make_uint4(0u, 0u, 0u, 0u);
+        if (i < n) v = *reinterpret_cast<const uint4*>(spine + i);
+        const uint32_t s = (v.x + v.y) + (v.z + v.w);
+        const uint32_t inc = wave_incl_scan(s);
+        if (lane == 63) sm[w] = inc;
+        __syncthreads();
+        uint32_t before = 0, tot = 0;
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const uint32_t t = sm[k];
+            if (k < w) before += t;
+            tot += t;
+        }
+        __syncthreads();
+        const uint32_t run = carry + before + inc - s;
+        if (i < n) *reinterpret_cast<uint4*>(spine + i) = make_uint4(run, run + v.x, run + v.x + v.y, run + v.x + v.y + v.z);
+        carry += tot;
+    }
+}
+
 // ---- stable scatter ---------------------------------------------------------------
 __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int shift) {
     __shared__ uint32_t cnt[WAVES][256];     // running digit counts of each wave; later: destinations
@@ -319,9 +348,13 @@ int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st) {
     for (int pass = 0; pass < 4; pass++) {
         const int src = pass & 1, shift = 8 * pass;
         if (pass > 0) hipLaunchKernelGGL(k_hist, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);     // the first pass's counts come from k_keys
-        hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
-        hipLaunchKernelGGL(k_spine_top, dim3(1), dim3(256), 0, st, pl.blocksums, nb);
-        hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
+        if (n <= SPINE_SINGLE_MAX) {
+            hipLaunchKernelGGL(k_spine_single, dim3(1), dim3(1024), 0, st, pl.spine, n);
+        } else {
+            hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
+            hipLaunchKernelGGL(k_spine_top, dim3(1), dim3(256), 0, st, pl.blocksums, nb);
+            hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
+        }
         hipLaunchKernelGGL(k_scatter, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
         SG_LAUNCH_CHECK("radix pass");
     }
