@@ -163,6 +163,32 @@ SG_HD float sg_rcp_pos(float d) {
     return r;
 }
 
+/* SiLU of n <= 8 values with ONE reciprocal (simultaneous inversion of the denominators 1 + exp(-z_k), all >= 1):
+ * out_k = z_k * (1/P_{n-1}) * (d_{k+1} ... d_{n-1}) * P_{k-1},  P_k = d_0 ... d_k.  Used only while the product of all
+ * denominators is below SG_SILU_BLOCK_LIMIT (a very negative z makes its denominator huge); sg_silu per value
+ * otherwise.  Differs from sg_silu in the last bits, so both sides of a parity comparison must group the values the
+ * same way. */
+#define SG_SILU_BLOCK_LIMIT 1e30f
+SG_HD void sg_silu_block(int n, const float* z, float* out) {
+    float d[8], P[8];
+    float acc = 1.0f;
+    for (int k = 0; k < n; k++) {
+        d[k] = 1.0f + sg_exp(-z[k]);
+        acc = (k == 0) ? d[k] : acc * d[k];
+        P[k] = acc;
+    }
+    if (acc < SG_SILU_BLOCK_LIMIT) {
+        float r = sg_rcp_pos(acc);
+        for (int k = n - 1; k >= 0; k--) {
+            const float inv = (k > 0) ? r * P[k - 1] : r;
+            if (k > 0) r = r * d[k];
+            out[k] = z[k] * inv;
+        }
+    } else {
+        for (int k = 0; k < n; k++) out[k] = z[k] / d[k];
+    }
+}
+
 /* sin and cos for |theta| < 0.3 with one polynomial term less each (least-squares fit on that
  * interval; ~1 ulp).  NOT bit-identical to sg_sincos: both sides of a parity comparison must take
  * this form for the same timesteps. */

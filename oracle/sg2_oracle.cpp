@@ -169,6 +169,10 @@ struct F32 {
     static R softplus(R x) { return sg_softplus(x); }
     static R sigmoid(R x) { return sg_sigmoid(x); }
     static R silu(R x) { return sg_silu(x); }
+    /* gates of n columns in groups of `group` consecutive ones, as the kernel's waves form them (sg_silu_block) */
+    static void silu_groups(const R* z, int n, int group, R* out) {
+        for (int j0 = 0; j0 < n; j0 += group) sg_silu_block(group, z + j0, out + j0);
+    }
     static R tanh(R x) { return sg_tanh(x); }
     static R sqrt(R x) { return __builtin_sqrtf(x); }
     static void sincos(R t, R* s, R* c) { sg_sincos(t, s, c); }
@@ -182,6 +186,9 @@ struct F64 {
     static R softplus(R x) { return (x > 20.0) ? x : std::log(1.0 + std::exp(x)); }
     static R sigmoid(R x) { return 1.0 / (1.0 + std::exp(-x)); }
     static R silu(R x) { return x / (1.0 + std::exp(-x)); }
+    static void silu_groups(const R* z, int n, int, R* out) {
+        for (int j = 0; j < n; j++) out[j] = silu(z[j]);
+    }
     static R tanh(R x) { return std::tanh(x); }
     static R sqrt(R x) { return std::sqrt(x); }
     static void sincos(R t, R* s, R* c) { *s = std::sin(t); *c = std::cos(t); }
@@ -449,6 +456,9 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
 
     /* pass 3: replay every chunk from its start state */
     std::vector<R> hc(di * ds), yp(hp), out(di);
+    R gate[32];
+    /* the kernel's waves each gate d_inner / (waves per chunk) consecutive columns with one shared reciprocal */
+    const int gate_group = di / std::max(1, di * hp / 64);
     for (int64_t c = 0; c < nchunks; c++) {
         std::copy(&hstart[(size_t)c * di * ds], &hstart[(size_t)c * di * ds] + di * ds, hc.begin());
         const int64_t u_end = std::min<int64_t>((c + 1) * chunk_len, N);
@@ -458,6 +468,7 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
             for (int k = 0; k < cnt; k++) {
                 const int64_t u = tile0 + k, t = reverse ? (N - 1 - u) : u;
                 const StepProj<O>& sp = tc.sp[k];
+                O::silu_groups(sp.z, di, gate_group, gate);
                 for (int j = 0; j < di; j++) {
                     const R dt = sp.dt[j], xb = sp.xb[j];
                     for (int p = 0; p < hp; p++) {
@@ -475,7 +486,7 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
                     /* balanced pairwise sum over the RoPE pairs (stride 1, 2, 4, ...) */
                     for (int st = 1; st < hp; st *= 2)
                         for (int p = 0; p + st < hp; p += 2 * st) yp[p] = yp[p] + yp[p + st];
-                    out[j] = O::fma(yp[0], O::silu(sp.z[j]), (R)w.D[j] * xb);
+                    out[j] = O::fma(yp[0], gate[j], (R)w.D[j] * xb);
                 }
                 for (int dd = 0; dd < dm; dd++) {
                     R a = 0;
@@ -694,6 +705,7 @@ float orc_sin_tiny(float x) { float s, c; sg_sincos_tiny(x, &s, &c); return s; }
 float orc_cos_tiny(float x) { float s, c; sg_sincos_tiny(x, &s, &c); return c; }
 float orc_sigmoid(float x) { return sg_sigmoid(x); }
 float orc_silu(float x) { return sg_silu(x); }
+void orc_silu_block(int n, const float* z, float* out) { sg_silu_block(n, z, out); }
 float orc_tanh(float x) { return sg_tanh(x); }
 float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }
 float orc_cos(float x) { float s, c; sg_sincos(x, &s, &c); return c; }

@@ -156,11 +156,15 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
         if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(coef(s_C, ss));
     }
     if (OUT) {
+        // the gates of this wave's columns share one reciprocal (sg_silu_block)
+        constexpr int NG = G::DI / G::PARTS;
+        static_assert(NG <= 8, "sg_silu_block takes at most 8 values");
+        float zv[NG], gv[NG];
 #pragma unroll
-        for (int q = 0; q < G::DI / G::PARTS; q++) {
-            const int jj = PART * (G::DI / G::PARTS) + q;
-            s_gate[jj * LDS_STRIDE + tu] = sg_silu(eval(coef(s_gate, jj)));
-        }
+        for (int q = 0; q < NG; q++) zv[q] = eval(coef(s_gate, PART * NG + q));
+        sg_silu_block(NG, zv, gv);
+#pragma unroll
+        for (int q = 0; q < NG; q++) s_gate[(PART * NG + q) * LDS_STRIDE + tu] = gv[q];
     }
     return (small ? 1 : 0) | (tiny ? 2 : 0);
 }

@@ -59,6 +59,34 @@ def test_sigmoid_silu_tanh():
     assert L.orc_tanh(0.0) == 0.0 and L.orc_tanh(30.0) == 1.0 and L.orc_tanh(-30.0) == -1.0
 
 
+def test_silu_block_shares_one_reciprocal():
+    """sg_silu_block (n values, one reciprocal) against x / (1 + exp(-x)) in double precision: groups of 4 and 8,
+    ordinary and mixed magnitudes, and a group whose denominators overflow the shared product (per-value fallback,
+    which must then equal sg_silu bit for bit)."""
+    import ctypes as C
+    def block(vals):
+        z = np.asarray(vals, np.float32)
+        out = np.zeros_like(z)
+        L.orc_silu_block(len(z), z.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data_as(C.POINTER(C.c_float)))
+        return z, out
+    worst = 0.0
+    for n in (4, 8):
+        for scale in (0.1, 1.0, 4.0):
+            for _ in range(2000):
+                z, out = block(RNG.randn(n) * scale)
+                ref = z.astype(np.float64) / (1.0 + np.exp(-z.astype(np.float64)))
+                worst = max(worst, float(np.max(np.abs(out - ref) / np.maximum(np.abs(ref), 1e-30))))
+    assert worst < 1.5e-6, worst          # a dozen roundings instead of the two of sg_silu
+    z, out = block([0.0, 1.0, -1.0, 30.0])
+    assert out[0] == 0.0 and abs(out[3] - 30.0) < 1e-5
+    # one very negative value makes the product of denominators overflow: every value takes the plain form
+    z, out = block([-80.0, -70.0, 0.5, -60.0, 2.0, -75.0, 1.0, -85.0])
+    assert all(out[k] == np.float32(L.orc_silu(float(z[k]))) for k in range(8))
+    # just below the limit the block form is used and agrees to rounding
+    z, out = block([-8.0] * 8)
+    assert np.all(np.abs(out - np.float32(-8.0 / (1 + math.exp(8.0)))) < 1e-9)
+
+
 def test_sincos():
     xs = np.concatenate([RNG.uniform(-100, 100, 30000), RNG.uniform(-1, 1, 5000),
                          [0.0, math.pi / 4, -math.pi / 4, math.pi / 2, math.pi, 3 * math.pi / 2]])
