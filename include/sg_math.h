@@ -267,6 +267,60 @@ SG_HD float sg_tanh(float x) {
     return y;
 }
 
+/* sigmoid of n <= 8 values and tanh of n <= 4 values with ONE reciprocal each (simultaneous inversion, as in
+ * sg_silu_block): the denominators 1 + exp(-x_k), resp. exp(2|x_k|) + 1, are all >= 1; the shared form is used only
+ * while their product stays below SG_SILU_BLOCK_LIMIT, the plain sg_sigmoid / sg_tanh per value otherwise (so a
+ * saturated gate keeps its exact value).  Last-bit differences from the plain forms: both sides of a parity
+ * comparison must group the values the same way. */
+SG_HD void sg_sigmoid_block(int n, const float* x, float* out) {
+    float d[8], P[8];
+    float acc = 1.0f;
+    for (int k = 0; k < n; k++) {
+        d[k] = 1.0f + sg_exp(-x[k]);
+        acc = (k == 0) ? d[k] : acc * d[k];
+        P[k] = acc;
+    }
+    if (acc < SG_SILU_BLOCK_LIMIT) {
+        float r = sg_rcp_pos(acc);
+        for (int k = n - 1; k >= 0; k--) {
+            out[k] = (k > 0) ? r * P[k - 1] : r;
+            if (k > 0) r = r * d[k];
+        }
+    } else {
+        for (int k = 0; k < n; k++) out[k] = 1.0f / d[k];
+    }
+}
+SG_HD void sg_tanh_block(int n, const float* x, float* out) {
+    float d[4], P[4];
+    float acc = 1.0f;
+    for (int k = 0; k < n; k++) {
+        const float ax = sg_abs(x[k]);
+        d[k] = sg_exp(ax + ax) + 1.0f;
+        acc = (k == 0) ? d[k] : acc * d[k];
+        P[k] = acc;
+    }
+    if (acc < SG_SILU_BLOCK_LIMIT) {
+        float r = sg_rcp_pos(acc);
+        for (int k = n - 1; k >= 0; k--) {
+            const float inv = (k > 0) ? r * P[k - 1] : r;
+            if (k > 0) r = r * d[k];
+            const float xk = x[k], ax = sg_abs(xk), z = xk * xk;
+            /* the two forms of sg_tanh, selected the same way */
+            float p = -5.70498872745e-3f;
+            p = sg_fma(p, z, 2.06390887954e-2f);
+            p = sg_fma(p, z, -5.37397155531e-2f);
+            p = sg_fma(p, z, 1.33314422036e-1f);
+            p = sg_fma(p, z, -3.33332819422e-1f);
+            const float small = sg_fma(p * z, xk, xk);
+            const float t = sg_fma(-2.0f, inv, 1.0f);
+            const float large = sg_i2f(sg_f2i(t) | (sg_f2i(xk) & (int32_t)0x80000000));
+            out[k] = (ax < 0.625f) ? small : large;
+        }
+    } else {
+        for (int k = 0; k < n; k++) out[k] = sg_tanh(x[k]);
+    }
+}
+
 /* erfc(x): Chebyshev fit with exponential prefactor (Numerical Recipes
  * "erfcc"), fractional error below 1.2e-7 for every x. */
 SG_HD float sg_erfc(float x) {

@@ -34,8 +34,9 @@ def load(path):
         f = getattr(L, "orc_" + n)
         f.restype = C.c_float
         f.argtypes = [C.c_float]
-    L.orc_silu_block.restype = None
-    L.orc_silu_block.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    for f in (L.orc_silu_block, L.orc_sigmoid_block, L.orc_tanh_block):
+        f.restype = None
+        f.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.orc_abar.restype = C.c_float
     L.orc_abar.argtypes = [C.c_float, C.c_float]
     L.orc_f_to_f16.restype = C.c_uint16

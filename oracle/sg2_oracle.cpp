@@ -173,6 +173,15 @@ struct F32 {
     static void silu_groups(const R* z, int n, int group, R* out) {
         for (int j0 = 0; j0 < n; j0 += group) sg_silu_block(group, z + j0, out + j0);
     }
+    /* the per-element kernel forms the 2 x 4 GRU gates, and the 4 candidates, with one reciprocal each */
+    static void sigmoid_group(int n, const R* x, R* out) {
+        if (n == 8) sg_sigmoid_block(n, x, out);
+        else for (int k = 0; k < n; k++) out[k] = sg_sigmoid(x[k]);
+    }
+    static void tanh_group(int n, const R* x, R* out) {
+        if (n == 4) sg_tanh_block(n, x, out);
+        else for (int k = 0; k < n; k++) out[k] = sg_tanh(x[k]);
+    }
     static R tanh(R x) { return sg_tanh(x); }
     static R sqrt(R x) { return __builtin_sqrtf(x); }
     static void sincos(R t, R* s, R* c) { sg_sincos(t, s, c); }
@@ -189,6 +198,8 @@ struct F64 {
     static void silu_groups(const R* z, int n, int, R* out) {
         for (int j = 0; j < n; j++) out[j] = silu(z[j]);
     }
+    static void sigmoid_group(int n, const R* x, R* out) { for (int k = 0; k < n; k++) out[k] = sigmoid(x[k]); }
+    static void tanh_group(int n, const R* x, R* out) { for (int k = 0; k < n; k++) out[k] = tanh(x[k]); }
     static R tanh(R x) { return std::tanh(x); }
     static R sqrt(R x) { return std::sqrt(x); }
     static void sincos(R t, R* s, R* c) { *s = std::sin(t); *c = std::cos(t); }
@@ -585,7 +596,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
         const R gv = g[i], sv = s[i];
         const R* f = &cf[(size_t)i * dm];
         const R* b = &cb[(size_t)i * dm];
-        R hold[8], zg[8], rg[8], hnew[8];
+        R hold[8], zg[8], rg[8], hnew[8], pre_g[16], gate[16], pre_c[8], cand[8];
         for (int k = 0; k < gh; k++) hold[k] = gru_io[i * gh + k];
         /* GRU gates: chain = bias, g, s, fwd ctx, bwd ctx, h */
         for (int j = 0; j < gh; j++) {
@@ -596,9 +607,11 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
             for (int k = 0; k < dm; k++) { vz = O::fma((R)wz[2 + k], f[k], vz); vr = O::fma((R)wr[2 + k], f[k], vr); }
             for (int k = 0; k < dm; k++) { vz = O::fma((R)wz[2 + dm + k], b[k], vz); vr = O::fma((R)wr[2 + dm + k], b[k], vr); }
             for (int k = 0; k < gh; k++) { vz = O::fma((R)wz[2 + 2 * dm + k], hold[k], vz); vr = O::fma((R)wr[2 + 2 * dm + k], hold[k], vr); }
-            zg[j] = O::sigmoid(vz);
-            rg[j] = O::sigmoid(vr);
+            pre_g[j] = vz;
+            pre_g[gh + j] = vr;
         }
+        O::sigmoid_group(2 * gh, pre_g, gate);
+        for (int j = 0; j < gh; j++) { zg[j] = gate[j]; rg[j] = gate[gh + j]; }
         for (int j = 0; j < gh; j++) {
             const float* wh = Wh + j * grl;
             R v = bh[j];
@@ -606,9 +619,10 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
             for (int k = 0; k < dm; k++) v = O::fma((R)wh[2 + k], f[k], v);
             for (int k = 0; k < dm; k++) v = O::fma((R)wh[2 + dm + k], b[k], v);
             for (int k = 0; k < gh; k++) v = O::fma((R)wh[2 + 2 * dm + k], rg[k] * hold[k], v);
-            const R ht = O::tanh(v);
-            hnew[j] = O::fma(zg[j], ht, ((R)1 - zg[j]) * hold[j]);
+            pre_c[j] = v;
         }
+        O::tanh_group(gh, pre_c, cand);
+        for (int j = 0; j < gh; j++) hnew[j] = O::fma(zg[j], cand[j], ((R)1 - zg[j]) * hold[j]);
         for (int k = 0; k < gh; k++) gru_io[i * gh + k] = (float)hnew[k];
 
         /* PEER: per head query -> two sub-key argmaxes -> expert MLP */
@@ -706,6 +720,8 @@ float orc_cos_tiny(float x) { float s, c; sg_sincos_tiny(x, &s, &c); return c; }
 float orc_sigmoid(float x) { return sg_sigmoid(x); }
 float orc_silu(float x) { return sg_silu(x); }
 void orc_silu_block(int n, const float* z, float* out) { sg_silu_block(n, z, out); }
+void orc_sigmoid_block(int n, const float* x, float* out) { sg_sigmoid_block(n, x, out); }
+void orc_tanh_block(int n, const float* x, float* out) { sg_tanh_block(n, x, out); }
 float orc_tanh(float x) { return sg_tanh(x); }
 float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }
 float orc_cos(float x) { float s, c; sg_sincos(x, &s, &c); return c; }

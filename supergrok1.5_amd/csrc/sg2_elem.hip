@@ -95,6 +95,7 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
 
             // ---- GRU: chain order = bias, g, s, fwd ctx, bwd ctx, h
             float zg[GH], rg[GH], hnew[GH];
+            float pre_g[2 * GH], gate[2 * GH], pre_c[GH], cand[GH];      // gates and candidates share one reciprocal each
 #pragma unroll
             for (int j = 0; j < GH; j++) {
                 const sg::cfloat_p wz = Wz + j * GRL;
@@ -108,9 +109,12 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 for (int q = 0; q < DM; q++) { vz = sg_fma(wz[2 + DM + q], cb[q], vz); vr = sg_fma(wr[2 + DM + q], cb[q], vr); }
 #pragma unroll
                 for (int q = 0; q < GH; q++) { vz = sg_fma(wz[2 + 2 * DM + q], hold[q], vz); vr = sg_fma(wr[2 + 2 * DM + q], hold[q], vr); }
-                zg[j] = sg_sigmoid(vz);
-                rg[j] = sg_sigmoid(vr);
+                pre_g[j] = vz;
+                pre_g[GH + j] = vr;
             }
+            sg_sigmoid_block(2 * GH, pre_g, gate);
+#pragma unroll
+            for (int j = 0; j < GH; j++) { zg[j] = gate[j]; rg[j] = gate[GH + j]; }
 #pragma unroll
             for (int j = 0; j < GH; j++) {
                 const sg::cfloat_p wh = Wh + j * GRL;
@@ -122,9 +126,11 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 for (int q = 0; q < DM; q++) v = sg_fma(wh[2 + DM + q], cb[q], v);
 #pragma unroll
                 for (int q = 0; q < GH; q++) v = sg_fma(wh[2 + 2 * DM + q], rg[q] * hold[q], v);
-                const float ht = sg_tanh(v);
-                hnew[j] = sg_fma(zg[j], ht, (1.0f - zg[j]) * hold[j]);
+                pre_c[j] = v;
             }
+            sg_tanh_block(GH, pre_c, cand);
+#pragma unroll
+            for (int j = 0; j < GH; j++) hnew[j] = sg_fma(zg[j], cand[j], (1.0f - zg[j]) * hold[j]);
             ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
 
             // ---- PEER routing + expert MLP

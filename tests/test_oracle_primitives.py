@@ -87,6 +87,33 @@ def test_silu_block_shares_one_reciprocal():
     assert np.all(np.abs(out - np.float32(-8.0 / (1 + math.exp(8.0)))) < 1e-9)
 
 
+def test_sigmoid_and_tanh_blocks():
+    """sg_sigmoid_block (8 values) and sg_tanh_block (4 values) against libm in double precision; saturated values
+    push the shared product over its limit and must then give exactly the plain forms."""
+    import ctypes as C
+    def call(fn, vals):
+        x = np.asarray(vals, np.float32)
+        out = np.zeros_like(x)
+        fn(len(x), x.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data_as(C.POINTER(C.c_float)))
+        return x, out
+    ws = wt = 0.0
+    for scale in (0.2, 1.0, 3.0):
+        for _ in range(3000):
+            x, out = call(L.orc_sigmoid_block, RNG.randn(8) * scale)
+            ref = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+            ws = max(ws, float(np.max(np.abs(out - ref) / ref)))
+            x, out = call(L.orc_tanh_block, RNG.randn(4) * scale)
+            ref = np.tanh(x.astype(np.float64))
+            wt = max(wt, float(np.max(np.abs(out - ref) / np.maximum(np.abs(ref), 1e-30))))
+    assert ws < 1.5e-6 and wt < 1.5e-6, (ws, wt)
+    x, out = call(L.orc_sigmoid_block, [-40.0, -41.0, 0.3, -39.0, 40.0, 1.0, -1.0, -45.0])
+    assert all(out[k] == np.float32(L.orc_sigmoid(float(x[k]))) for k in range(8)) and out[4] == 1.0
+    x, out = call(L.orc_tanh_block, [30.0, -25.0, 0.1, 20.0])
+    assert all(out[k] == np.float32(L.orc_tanh(float(x[k]))) for k in range(4)) and out[0] == 1.0 and out[1] == -1.0
+    x, out = call(L.orc_tanh_block, [0.0, 0.625, -0.625, 1e-6])
+    assert out[0] == 0.0 and abs(out[1] - math.tanh(0.625)) < 1e-7 and out[2] == -out[1]
+
+
 def test_sincos():
     xs = np.concatenate([RNG.uniform(-100, 100, 30000), RNG.uniform(-1, 1, 5000),
                          [0.0, math.pi / 4, -math.pi / 4, math.pi / 2, math.pi, 3 * math.pi / 2]])

@@ -125,8 +125,8 @@ def test_soft_top4_routing_closed_form():
 # ------------------------------------------------------------------------------- the pins notice injected mistakes
 MUTANTS = [
     # (name, text in sg2_oracle.cpp, replacement, the pin that has to fail)
-    ("gru_gates_exchanged", "hnew[j] = O::fma(zg[j], ht, ((R)1 - zg[j]) * hold[j]);",
-     "hnew[j] = O::fma((R)1 - zg[j], ht, zg[j] * hold[j]);", lambda run: pins.check_gru_update_gate_closed_keeps_state(run)),
+    ("gru_gates_exchanged", "hnew[j] = O::fma(zg[j], cand[j], ((R)1 - zg[j]) * hold[j]);",
+     "hnew[j] = O::fma((R)1 - zg[j], cand[j], zg[j] * hold[j]);", lambda run: pins.check_gru_update_gate_closed_keeps_state(run)),
     ("gru_reset_ignored", "v = O::fma((R)wh[2 + 2 * dm + k], rg[k] * hold[k], v);",
      "v = O::fma((R)wh[2 + 2 * dm + k], hold[k], v);", lambda run: pins.check_gru_candidate_with_reset_closed(run, 2e-5)),
     ("gru_ctx_order", "vz = O::fma((R)wz[2 + k], f[k], vz); vr = O::fma((R)wr[2 + k], f[k], vr);",
