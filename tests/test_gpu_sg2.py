@@ -110,6 +110,24 @@ def test_adaptive_window_needs_several_blocks():
     print("several blocks", _run_steps(case, 2, chunk_len=512, sharp=True, lamb_eff=2.0))
 
 
+def test_saturated_gates_take_the_plain_forms():
+    """The scan's output gates, the GRU gates and the GRU candidates are formed with one shared reciprocal per group
+    unless the product of the group's denominators is too large; then every value of the group takes the plain
+    form.  Weights that saturate some elements' gates and not others put both forms, and lanes of one wave on
+    different ones, through the device and the checker: any difference in the decision shows as a mismatch."""
+    shapes = [(2500,), (64, 33), (700,)]
+    W = wl.meta_weights(7)
+    for base in (2, 11):
+        W[base][16:, :] *= 1000.0             # z half of in_proj: gate pre-activations of order +-30
+    W[20][:, 0] = 60.0                        # W_z, W_r, W_h: the gradient itself drives the GRU gates
+    W[22][:, 0] = -45.0
+    W[24][:, 0] = 30.0
+    case = Sg2Case(shapes, seed=77, random_state=True, weights=W)
+    w = _run_steps(case, 2, chunk_len=None, sharp=True, lamb_eff=2.0, wd_eff=4.5, grad_std=1.0)
+    print("saturated gates: worst tolerance ratios", w)
+    assert all(v == 0.0 for v in w.values()), w        # identical arithmetic on both sides: not one bit differs
+
+
 def test_shared14_one_step_default_chunk():
     """The 14-tensor, 420 195-element transformer parameter set, default chunk length."""
     case = Sg2Case(wl.shared14_shapes(), seed=0)
