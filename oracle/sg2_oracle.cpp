@@ -324,8 +324,9 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
                 if (!tiny) continue;
                 for (int q = 0; q < ORC_BLOCK; q++)
                     for (int l = wave0; l < wave1; l++) {
-                        float sn, cs;
-                        sg_sincos_tiny((float)tc.sp[b0 + q].dt[l / hp] * w.rope[l], &sn, &cs);
+                        float sn, cs, coef[6];
+                        sg_sincos_tiny_coef(w.rope[l], coef);
+                        sg_sincos_tiny_dt((float)tc.sp[b0 + q].dt[l / hp], coef, &sn, &cs);
                         tc.sn[(size_t)(b0 + q) * lanes + l] = (R)sn;
                         tc.cs[(size_t)(b0 + q) * lanes + l] = (R)cs;
                     }

@@ -209,11 +209,11 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // UB consecutive timesteps (all valid): coefficients first, then the serial chain.  ux = dt * x-branch
 // (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
-// ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny (its own values).
+// ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values; tcoef = the lane's sg_sincos_tiny_coef).
 template <int HP, bool OUT, int ANGLE>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
-                                            float hAo, float freq, float (&y)[UB]) {
+                                            float hAo, float freq, const float (&tcoef)[6], float (&y)[UB]) {
     float ae[UB], ao[UB], sn[UB], cs[UB], be[UB], bo[UB];
     {
         float d_e[UB], d_o[UB], P[UB];
@@ -227,7 +227,7 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
-        if (ANGLE == 2) sg_sincos_tiny(dt[u] * freq, &sn[u], &cs[u]);
+        if (ANGLE == 2) sg_sincos_tiny_dt(dt[u], tcoef, &sn[u], &cs[u]);
         else if (ANGLE == 1) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
         else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
         be[u] = ux[u] * Be[u];
@@ -286,6 +286,8 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
     const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
     const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
+    float tcoef[6];             // tiny-angle sin/cos of this lane's pair as polynomials in dt
+    sg_sincos_tiny_coef(freq, tcoef);
 
     {   // largest |frequency| of each column's pairs
         const float f = pair_tree_max<HP>(sg_abs(freq));
@@ -407,11 +409,11 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             }
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
             if ((nottiny & blk) == 0)
-                block_steps<HP, OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
             else if ((large & blk) == 0)
-                block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
             else
-                block_steps<HP, OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, y);
+                block_steps<HP, OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
             if (OUT && p == 0) {
 #pragma unroll
                 for (int q = 0; q < UB; q += 4)
