@@ -73,8 +73,7 @@ SG_HD float sg_exp(float x) {
     p = sg_fma(p, r, 4.1665795894e-2f);
     p = sg_fma(p, r, 1.6666665459e-1f);
     p = sg_fma(p, r, 5.0000001201e-1f);
-    const float r2 = r * r;
-    p = sg_fma(p, r2, r) + 1.0f;
+    p = sg_fma(sg_fma(p, r, 1.0f), r, 1.0f);         /* 1 + r (1 + r p) */
     return sg_i2f((int32_t)((uint32_t)sg_f2i(p) + ((uint32_t)(int32_t)k << 23)));
 }
 
