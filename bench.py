@@ -27,6 +27,14 @@ PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.420e9 + 1.619e9, "scan_summary": 0
                              "elementwise": 2.503e9 + 0.801e9}
 
 
+# Vector-ALU instructions per launch (SQ_INSTS_VALU of the same profile, default workload only) and the rate the part
+# sustains on nothing but independent fp32 instructions (bench.py --workload valu-probe, profiles/valu_probe_mi355x.txt):
+# what actually bounds these kernels
+PMC_VALU_INSTS_SCALE50 = {"scan_output": 3.864e9, "scan_summary": 2.09e8, "elementwise": 8.66e8}
+VALU_SUSTAINED_PER_NS_SIMD = 0.59
+SIMDS = 1024
+
+
 LARGE_GEOMETRY = dict(d_model=16, d_state=32, d_inner=32)     # the second scan geometry the kernels are built for
 
 
@@ -450,6 +458,10 @@ def main():
         "step_hbm_frac": BYTES_PER_ELEMENT * value / 1e9 / HBM_PEAK_GBS,
         "stage_ms": stage_avg,
     }
+    if (args.workload, args.weights, args.geometry) == ("scale50", "bench", "default") and dom in PMC_VALU_INSTS_SCALE50:
+        rate = PMC_VALU_INSTS_SCALE50[dom] / (stage_avg[dom] * 1e6) / SIMDS       # wave instructions per ns and SIMD
+        out["valu"] = {"kernel": kernel_of[dom], "instructions": PMC_VALU_INSTS_SCALE50[dom], "per_ns_simd": rate,
+                       "sustained_per_ns_simd": VALU_SUSTAINED_PER_NS_SIMD, "frac": rate / VALU_SUSTAINED_PER_NS_SIMD}
     if not args.no_class_step and args.geometry == "default":
         out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if not args.no_cpu_baseline:
