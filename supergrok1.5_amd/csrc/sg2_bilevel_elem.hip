@@ -122,19 +122,19 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 
     // the lane's (expert, hidden unit) pairs: wave w owns the experts with first sub-key index 6w .. 6w+5; for first
     // index 6w + r, round c covers second indices 4c .. 4c+3 (one per 16 lanes) x 16 hidden units.  Per pair: the
-    // expert's W1, b1 entry and three sums over elements of t = (routing weight if the unit is active else 0):
-    // sum t, sum t*g, sum t*pre, from which d b1 = W2*sum t, d W1 = W2*sum t*g, d W2 = sum t*pre.
+    // expert's W1, b1 entry and two sums over elements of t = (routing weight if the unit is active else 0):
+    // sum t and sum t*g, from which d b1 = W2*sum t, d W1 = W2*sum t*g, d W2 = sum t*pre = W1*sum t*g + b1*sum t.
     constexpr int KA_PER_WAVE = PK / BE_WAVES, ROUNDS = PK / 4;
     static_assert(KA_PER_WAVE * ROUNDS == EXP_PER_LANE, "pairs per lane");
     const int ka0 = __builtin_amdgcn_readfirstlane(KA_PER_WAVE * (tid >> 6));
     const int kb_sub = (tid & 63) >> 4;
     float ew1[EXP_PER_LANE], eb1[EXP_PER_LANE];
-    float st0[EXP_PER_LANE], st1[EXP_PER_LANE], stp[EXP_PER_LANE], sdo[EXP_PER_LANE];
+    float st0[EXP_PER_LANE], st1[EXP_PER_LANE], sdo[EXP_PER_LANE];
 #pragma unroll
     for (int q = 0; q < EXP_PER_LANE; q++) {
         const int e = (ka0 + q / ROUNDS) * PK + 4 * (q % ROUNDS) + kb_sub, m = tid & (EH - 1);
         ew1[q] = s_exp[e * EXP_STRIDE + m]; eb1[q] = s_exp[e * EXP_STRIDE + EH + m];
-        st0[q] = st1[q] = stp[q] = sdo[q] = 0.0f;
+        st0[q] = st1[q] = sdo[q] = 0.0f;
     }
 
     const int tiles = (a.total + BE_THREADS - 1) / BE_THREADS;
@@ -353,7 +353,6 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                                 const float t = pre > 0.0f ? dout : 0.0f;
                                 st0[q] += t;
                                 st1[q] = sg_fma(t, v.g, st1[q]);
-                                stp[q] = sg_fma(t, pre, stp[q]);
                                 sdo[q] += dout;
                             }
                         }
@@ -464,7 +463,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         const float w2 = s_exp[e * EXP_STRIDE + 2 * EH + m];
         out[OFF_W1 + e * EH + m] = w2 * st1[q];
         out[OFF_B1 + e * EH + m] = w2 * st0[q];
-        out[OFF_W2 + e * EH + m] = stp[q];
+        out[OFF_W2 + e * EH + m] = sg_fma(ew1[q], st1[q], eb1[q] * st0[q]);      // sum t*pre with pre = W1 g + b1 wherever t != 0
         if (m == 0) out[OFF_B2 + e] = sdo[q];
     }
 }
