@@ -240,14 +240,20 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
     for (int r = 0; r < ITEMS; r++) {
         const int i = w * WAVE_ITEMS + r * 64 + lane;
         const bool ok = i < tr.cnt;
-        const uint32_t d = (key[r] >> shift) & 255u;
-        uint64_t m = __ballot(ok);
+        const uint32_t d = (key[r] >> shift) & 255u;       // 0 for a lane past the end (its key reads as 0)
+        // lanes of the wave with the same digit: for every bit, keep the lanes whose bit equals this lane's.  With
+        // rep = the lane's bit spread over a word, that is m & ~(ballot ^ rep): one three-input bit operation per
+        // half (truth table 0x90 = a & ~(b ^ c)).  Lanes past the end hold no set bit and are outside the initial mask.
+        const uint64_t m0 = __ballot(ok);
+        uint32_t mlo = (uint32_t)m0, mhi = (uint32_t)(m0 >> 32);
 #pragma unroll
         for (int b = 0; b < 8; b++) {
-            const bool bit = (d >> b) & 1u;
-            const uint64_t bal = __ballot(ok && bit);
-            m &= bit ? bal : ~bal;
+            const int32_t rep_b = __builtin_amdgcn_sbfe((int32_t)d, b, 1);
+            const uint64_t bal = __ballot(rep_b != 0);
+            mlo = __builtin_amdgcn_bitop3_b32(mlo, (uint32_t)bal, (uint32_t)rep_b, 0x90);
+            mhi = __builtin_amdgcn_bitop3_b32(mhi, (uint32_t)(bal >> 32), (uint32_t)rep_b, 0x90);
         }
+        const uint64_t m = ((uint64_t)mhi << 32) | mlo;
         if (ok) {
             const uint32_t before = __popcll(m & lt);
             const uint32_t prev = cnt[w][d];
