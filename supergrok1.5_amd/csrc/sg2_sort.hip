@@ -16,6 +16,8 @@
 //   scatter  stable rank inside the tile (each wave owns a contiguous quarter
 //            of the tile; match-any ballots give the rank among equal digits)
 //            and write to destination.
+#include <type_traits>
+
 #include "sg2_internal.hpp"
 
 namespace sg2 {
@@ -218,11 +220,17 @@ __global__ __launch_bounds__(1024) void k_spine_single(uint32_t* spine, int n /*
 // ---- stable scatter ---------------------------------------------------------------
 __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int shift) {
     __shared__ uint32_t cnt[WAVES][256];     // running digit counts of each wave; later: destinations
+    __shared__ uint32_t lbase[256], gdelta[256], wsum[4];
+    __shared__ uint32_t skey[SORT_TILE];
+    __shared__ int32_t sval[SORT_TILE];
     const TileRef tr = tile_ref(pl, blockIdx.x);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     for (int k = threadIdx.x; k < WAVES * 256; k += SORT_THREADS) (&cnt[0][0])[k] = 0;
     __syncthreads();
 
+    // a whole tile (all but the last tile of a tensor) needs no bounds tests: the body exists in both forms
+    auto body = [&](auto full_c) {
+    constexpr bool FULL = decltype(full_c)::value;
     const uint32_t* __restrict__ keys = pl.keys[src] + tr.base;
     const int32_t* __restrict__ vals = pl.vals[src] + tr.base;
     const uint64_t lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
@@ -232,14 +240,14 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int i = w * WAVE_ITEMS + r * 64 + lane;
-        const bool ok = i < tr.cnt;
+        const bool ok = FULL || i < tr.cnt;
         key[r] = ok ? keys[i] : 0u;
         val[r] = ok ? vals[i] : 0;
     }
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int i = w * WAVE_ITEMS + r * 64 + lane;
-        const bool ok = i < tr.cnt;
+        const bool ok = FULL || i < tr.cnt;
         const uint32_t d = (key[r] >> shift) & 255u;       // 0 for a lane past the end (its key reads as 0)
         // lanes of the wave with the same digit: for every bit, keep the lanes whose bit equals this lane's.  With
         // rep = the lane's bit spread over a word, that is m & ~(ballot ^ rep): one three-input bit operation per
@@ -264,7 +272,6 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
     __syncthreads();
     // digit d = threadIdx.x: position of each wave's first key of digit d inside the tile's digit-sorted order
     // (cnt[k][d]), start of digit d in that order (lbase[d]) and its distance to the global destination (gdelta[d])
-    __shared__ uint32_t lbase[256], gdelta[256], wsum[4];
     {
         const int d = threadIdx.x & 255;       // (threads beyond the 256 digits repeat the first ones' work and store nothing)
         const bool own = threadIdx.x < 256;
@@ -298,12 +305,10 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
     __syncthreads();
     // reorder through LDS so that global stores go out in digit-sorted order: consecutive lanes then write
     // consecutive addresses within each digit's run instead of 4-byte pieces all over the tile's 256 runs
-    __shared__ uint32_t skey[SORT_TILE];
-    __shared__ int32_t sval[SORT_TILE];
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int i = w * WAVE_ITEMS + r * 64 + lane;
-        if (i < tr.cnt) {
+        if (FULL || i < tr.cnt) {
             const uint32_t lp = cnt[w][(key[r] >> shift) & 255u] + rank[r];
             skey[lp] = key[r];
             sval[lp] = val[r];
@@ -315,13 +320,16 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int lp = r * SORT_THREADS + threadIdx.x;
-        if (lp < tr.cnt) {
+        if (FULL || lp < tr.cnt) {
             const uint32_t kk = skey[lp];
             const uint32_t dst = gdelta[(kk >> shift) & 255u] + (uint32_t)lp;
             kout[dst] = kk;
             vout[dst] = sval[lp];
         }
     }
+    };
+    if (tr.cnt == SORT_TILE) body(std::true_type{});
+    else body(std::false_type{});
 }
 
 // After the sort: sharpness gathered into sorted order (one random read per element, once, instead of
