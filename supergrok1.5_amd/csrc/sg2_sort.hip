@@ -100,9 +100,13 @@ __global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
 
 // ---- per-tile histogram ---------------------------------------------------------
 __global__ __launch_bounds__(SORT_THREADS) void k_hist(Plan pl, int src, int shift) {
-    __shared__ uint32_t h[256];
+    // HCOPY copies of the counters, chosen by lane: a pass whose digit takes few values (the exponent byte of the
+    // magnitudes) would otherwise queue most of a wave's lanes on a dozen counters.  Copies start 8 banks apart.
+    constexpr int HCOPY = 8, HSTRIDE = 256 + 8;
+    __shared__ uint32_t hc[HCOPY * HSTRIDE];
     const TileRef tr = tile_ref(pl, blockIdx.x);
-    if (threadIdx.x < 256) h[threadIdx.x] = 0;
+    for (int k = threadIdx.x; k < HCOPY * HSTRIDE; k += SORT_THREADS) hc[k] = 0;
+    uint32_t* const h = hc + (threadIdx.x & (HCOPY - 1)) * HSTRIDE;
     __syncthreads();
     const uint32_t* __restrict__ keys = pl.keys[src] + tr.base;
     // 16 bytes per lane where the tile starts on a 16-byte boundary (tensor offsets are arbitrary); the ragged end by single keys
@@ -116,7 +120,12 @@ __global__ __launch_bounds__(SORT_THREADS) void k_hist(Plan pl, int src, int shi
     }
     for (int k = vec + threadIdx.x; k < tr.cnt; k += SORT_THREADS) atomicAdd(&h[(keys[k] >> shift) & 255u], 1u);
     __syncthreads();
-    if (threadIdx.x < 256) pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
+    if (threadIdx.x < 256) {
+        uint32_t tot = 0;
+#pragma unroll
+        for (int c = 0; c < HCOPY; c++) tot += hc[c * HSTRIDE + threadIdx.x];
+        pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = tot;
+    }
 }
 
 // ---- exclusive scan of the spine -------------------------------------------------
