@@ -8,7 +8,7 @@
 //
 // Four passes of 8 bits over tiles of 8192 keys (512 lanes x 16).  Per pass:
 //   hist     per-tile digit counts -> spine[segment][digit][tile]  (first pass: counted while the keys are made)
-//   scan     exclusive prefix over the whole spine (3 small kernels; one for small models).  Because
+//   scan     exclusive prefix over the whole spine (2 small kernels; one for small models).  Because
 //            the spine is laid out segment-major, the global prefix of entry
 //            (seg, d, tile) is exactly: keys in earlier segments + keys of this
 //            segment with a smaller digit + keys with digit d in earlier tiles
@@ -166,21 +166,17 @@ __global__ __launch_bounds__(256) void k_spine_reduce(const uint32_t* __restrict
     block_excl_scan(s, sm, &tot);
     if (threadIdx.x == 0) blocksums[blockIdx.x] = tot;
 }
-__global__ __launch_bounds__(256) void k_spine_top(uint32_t* blocksums, int nb) {
-    __shared__ uint32_t sm[4];
-    uint32_t carry = 0;
-    for (int base = 0; base < nb; base += 256) {
-        const int i = base + threadIdx.x;
-        const uint32_t v = (i < nb) ? blocksums[i] : 0u;
-        uint32_t tot;
-        const uint32_t ex = block_excl_scan(v, sm, &tot);
-        if (i < nb) blocksums[i] = carry + ex;
-        carry += tot;
-    }
-}
+// Every workgroup adds up the block sums before its own by itself (a few hundred values for tens of millions of
+// elements; 16 K on average at the 2^31-element limit, still small beside that step): no launch for a scan of them.
 __global__ __launch_bounds__(256) void k_spine_down(uint32_t* spine, const uint32_t* __restrict__ blocksums, int n) {
     __shared__ uint32_t sm[4];
     constexpr int PER = SCAN_BLOCK_ITEMS / 256;
+    uint32_t before;
+    {
+        uint32_t part = 0;
+        for (int k = threadIdx.x; k < (int)blockIdx.x; k += 256) part += blocksums[k];
+        block_excl_scan(part, sm, &before);
+    }
     const int base = blockIdx.x * SCAN_BLOCK_ITEMS + threadIdx.x * PER;
     uint32_t v[PER], s = 0;
 #pragma unroll
@@ -189,7 +185,7 @@ __global__ __launch_bounds__(256) void k_spine_down(uint32_t* spine, const uint3
         s += v[k];
     }
     uint32_t tot;
-    uint32_t run = blocksums[blockIdx.x] + block_excl_scan(s, sm, &tot);
+    uint32_t run = before + block_excl_scan(s, sm, &tot);
 #pragma unroll
     for (int k = 0; k < PER; k++) {
         if (base + k < n) spine[base + k] = run;
@@ -198,7 +194,7 @@ __global__ __launch_bounds__(256) void k_spine_down(uint32_t* spine, const uint3
 }
 
 // The whole scan in one workgroup, for spines of at most SPINE_SINGLE_MAX entries (a model of up to a million
-// elements): three dependent launches of a few microseconds each cost more than the scan itself there.
+// elements): dependent launches of a few microseconds each cost more than the scan itself there.
 constexpr int SPINE_SINGLE_MAX = 32768;
 __global__ __launch_bounds__(1024) void k_spine_single(uint32_t* spine, int n /* a multiple of 256 */) {
     __shared__ uint32_t sm[16];
@@ -375,7 +371,6 @@ int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st) {
             hipLaunchKernelGGL(k_spine_single, dim3(1), dim3(1024), 0, st, pl.spine, n);
         } else {
             hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
-            hipLaunchKernelGGL(k_spine_top, dim3(1), dim3(256), 0, st, pl.blocksums, nb);
             hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
         }
         hipLaunchKernelGGL(k_scatter, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
