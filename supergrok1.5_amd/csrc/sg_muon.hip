@@ -27,12 +27,13 @@
 //
 // GEMM: 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each
 // wave 128x128 = 4x4 MFMA 32x32x16 bf16 tiles (256 fp32 accumulators per
-// lane), K tiles of 64 staged through LDS with 144-byte row stride (576 bytes for
-// the [k][n] tiles; conflict-free operand fetches, two stages), the tiles of the next
-// K steps in flight in two register sets while the current one is multiplied,
-// memory instructions dealt between the MFMAs.  256x256x64 gives 128 flop per byte
-// fetched, which keeps the MFMA pipe ahead of the ~64 B/clk a CU can pull from
-// L2; the symmetric products (G and G*G) compute only the tiles on or above
+// lane), K tiles of 32 in four LDS stages, filled by loads that go from global
+// memory straight into LDS (global_load_lds_dwordx4) three tiles ahead of their
+// use; no padding is possible in such a copy, so the tiles are swizzled by the
+// choice of the chunk each lane fetches (conflict-free operand fetches); memory
+// instructions are dealt between the MFMAs.  A 256x256 tile takes 128 flop per
+// byte fetched, which keeps the MFMA pipe ahead of the ~64 B/clk a CU can pull
+// from L2; the symmetric products (G and G*G) compute only the tiles on or above
 // the diagonal.  Tile index -> XCD-contiguous order so that the workgroups
 // sharing operand panels share an L2.
 #include <cmath>
@@ -49,12 +50,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int BT = 256;            // GEMM tile (M and N)
-constexpr int BK = 64;             // GEMM K tile
-constexpr int LDS_ROW = BK + 8;    // bf16 elements per LDS row (144 bytes) of a K-contiguous tile [BT][BK]
-constexpr int LDS_ROW_KN = BT + 32; // ... of a [BK][BT] tile (576 bytes: four rows start 16 banks apart)
-static_assert(BK * LDS_ROW_KN == BT * LDS_ROW, "both tile layouts fill the same LDS");
-constexpr int GEMM_LDS_BYTES = 2 * 2 * BT * LDS_ROW * 2;   // two stages of {A tile, B tile}: 147,456 bytes of the CU's 160 KB
-static_assert(BK == 64, "the K loop of k_gemm_nt is written for four 16-wide steps");
+constexpr int GEMM_LDS_BYTES = 4 * 2 * BT * 32 * 2;          // four stages of {A tile, B tile} of 32 k: 131,072 bytes of the CU's 160 KB
 constexpr float NS_A = 3.4445f, NS_B = -4.7750f, NS_C = 2.0315f;
 
 struct Mat {
@@ -219,8 +215,7 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
 // ---- GEMM  C[M x N] = A[M x K] * B  with fused epilogues; B given as [N x K] (Gram, polynomial) or as [K x N] (apply)
 // 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
 // 32x32x16 tiles (256 fp32 accumulators per lane; one wave per SIMD, the whole register file).
-// Per 16-wide k step a wave fetches 4+4 16-byte operands from LDS for 16 MFMAs.  The next K tile
-// is prefetched from global memory into registers while the current one is multiplied.
+// Per 16-wide k step a wave fetches 4+4 16-byte operands from LDS for 16 MFMAs.
 // The Gram and polynomial products are symmetric: only tiles on or above the diagonal are
 // computed, each off-diagonal tile is also stored transposed.
 enum { EPI_GRAM = 0, EPI_POLY = 1, EPI_APPLY = 2 };
@@ -265,10 +260,7 @@ template <int EPI>
 __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_flags) {
     constexpr bool BKN = EPI == EPI_APPLY;             // B operand stored [K x N]
     constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
-    constexpr int CH = BT * BK * 2 / 16 / 256;         // 16-byte chunks per thread and operand per K tile (8)
-    // LDS: two stages of {A tile, B tile}, each tile BT rows of LDS_ROW elements
     extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
-    constexpr int TILE_ELEMS = BT * LDS_ROW;
 
     // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs,
     // so that tiles that run together on an XCD share operand panels in its L2
@@ -319,58 +311,73 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // Global -> register -> LDS pipeline two K tiles deep: while tile kt is multiplied out of
-    // one LDS stage, tile kt+1 moves from its register set into the other stage and the loads of
-    // tile kt+3 are issued into the set just freed; tile kt+2 stays in flight in the other set.
-    // A load has two K tiles of MFMA work (~4000 cycles) to arrive.  One barrier per K tile.
-    u32x4 ra[2][CH], rb[2][CH];
-    const uint32_t voff_a = (uint32_t)(((tid >> 3) * lda + (tid & 7) * 8) * 2);
-    // [N x K] tile: 8 lanes per 128-byte row, 32 rows per pass; [K x N] tile: 32 lanes per 512-byte row, 8 rows per pass
-    const uint32_t voff_b = BKN ? (uint32_t)(((tid >> 5) * ldb + (tid & 31) * 8) * 2) : (uint32_t)(((tid >> 3) * ldb + (tid & 7) * 8) * 2);
-    const int soff = (tid >> 3) * LDS_ROW + (tid & 7) * 8;
-    const int soff_b = BKN ? (tid >> 5) * LDS_ROW_KN + (tid & 31) * 8 : soff;
-    auto gload_a = [&](int set, int kt) {
-        const char* pa = reinterpret_cast<const char*>(A + kt * BK);
-#pragma unroll
-        for (int i = 0; i < CH; i++) ra[set][i] = *(gvec_p)(pa + (size_t)i * 32 * lda * 2 + voff_a);
+    // Global memory -> LDS without passing through registers (global_load_lds_dwordx4: the 64 lanes' 16-byte chunks land
+    // contiguously, 1 KB per instruction, at the wave-uniform LDS address in M0).  K tiles of 32, four stages of
+    // {A tile, B tile} (16 KB each): the loads of a tile are issued three tiles ahead of its use and nothing of the
+    // copy occupies the wave's registers or its LDS-write slots.  A 1 KB block cannot carry padding, so the tiles are
+    // swizzled instead, by the choice of the chunk each lane fetches:
+    //   [256 rows x 32 k] tile (K-contiguous operand): block = 16 rows x 4 chunks, chunk c of row r at position
+    //                          c ^ ((r >> 2) & 3) of its row: 16 consecutive rows read one k chunk without a bank conflict
+    //   [32 k x 256 n] tile (the apply step's B): block = 2 k rows x 32 chunks, the 64-byte group g of row k at
+    //                          g ^ sw(k), sw(k) = (k & 3) | ((k >> 1) & 4): the 8 rows one transposing read touches
+    //                          (k0..k0+3 and k0+8..k0+11) fall on 8 different groups
+    constexpr int BKD = 32, STAGES = 4;
+    constexpr int OP_BYTES = BT * BKD * 2, STAGE_BYTES = 2 * OP_BYTES;
+    static_assert(STAGES * STAGE_BYTES <= GEMM_LDS_BYTES, "four stages fit the GEMM's LDS");
+    const unsigned char* const lds = reinterpret_cast<const unsigned char*>(smem);
+    const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;     // LDS byte address of smem
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    // address = wave-uniform 64-bit base (scalar registers, advanced by scalar adds) + this lane's constant 32-bit offset
+    auto dma16 = [](uint32_t lane_off, const void* base, uint32_t lds_addr) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n" : : "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
     };
-    auto gload_b = [&](int set, int kt) {
-        const char* pb = reinterpret_cast<const char*>(BKN ? B + (size_t)kt * BK * ldb : B + kt * BK);
-#pragma unroll
-        for (int i = 0; i < CH; i++) rb[set][i] = *(gvec_p)(pb + (size_t)i * (BKN ? 8 : 32) * ldb * 2 + voff_b);
+    // this lane's share of a block: row lane/4 of the block's 16 (block 4i + w of the tile), chunk (lane%4) ^ ((lane/16)%4)
+    const uint32_t lo_a = (uint32_t)((((lane >> 2) + 16 * wv) * lda + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2);
+    const uint32_t lo_b = (uint32_t)((((lane >> 2) + 16 * wv) * ldb + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2);
+    // [k][n] tile: wave w, instruction i loads k rows 8i + 2w + lane/32; sw of that row = (2(w&1) + lane/32) | ((i&1) << 2)
+    const int kn_row = 2 * wv + (lane >> 5);
+    const int kn_c0 = (lane & 31) ^ ((kn_row & 3) << 2);
+    const uint32_t lo_kn0 = (uint32_t)((kn_row * ldb + kn_c0 * 8) * 2);            // i even
+    const uint32_t lo_kn1 = (uint32_t)((kn_row * ldb + (kn_c0 ^ 16) * 8) * 2);     // i odd
+    // the q-th of a tile's eight loads (0-3: A, 4-7: B)
+    auto dma_one = [&](int kt, int q) {
+        const uint32_t st = lds0 + (uint32_t)(kt & (STAGES - 1)) * STAGE_BYTES;
+        const int i = q & 3, blk = 4 * i + wv;
+        if (q < 4) dma16(lo_a, reinterpret_cast<const char*>(A) + ((size_t)i * 64 * lda + (size_t)kt * BKD) * 2, st + blk * 1024);
+        else if (BKN) dma16((i & 1) ? lo_kn1 : lo_kn0, reinterpret_cast<const char*>(B) + (size_t)(kt * BKD + 8 * i) * ldb * 2, st + OP_BYTES + blk * 1024);
+        else dma16(lo_b, reinterpret_cast<const char*>(B) + ((size_t)i * 64 * ldb + (size_t)kt * BKD) * 2, st + OP_BYTES + blk * 1024);
     };
-    auto sstore_a = [&](int set, bf16_t* stage) {
+    auto dma_tile = [&](int kt) {
 #pragma unroll
-        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[soff + i * 32 * LDS_ROW]) = ra[set][i];
+        for (int q = 0; q < 8; q++) dma_one(kt, q);
     };
-    auto sstore_b = [&](int set, bf16_t* stage) {
-#pragma unroll
-        for (int i = 0; i < CH; i++) *reinterpret_cast<u32x4*>(&stage[TILE_ELEMS + soff_b + i * (BKN ? 8 * LDS_ROW_KN : 32 * LDS_ROW)]) = rb[set][i];
-    };
-    const int a_off = (wm * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
-    // [K x N] tile: the transposing read hands lane i of a 16-lane group, as element e, element i%4 of the 8 bytes
-    // that lane 4e + i/4 of the group addressed.  Lane s therefore points at row k0 + s/4, columns n0 + 4(s%4) .. +3
-    // of the group's 4(k) x 16(n) block, and lane i receives k0 .. k0+3 of column n0 + i.  Groups 0/1 of the wave
-    // cover columns 0-15 / 16-31 of the 32-column MFMA tile, groups 2/3 the same columns of the next 8 k.
-    const int b_off = BKN ? TILE_ELEMS + (8 * (lane >> 5) + ((lane & 15) >> 2)) * LDS_ROW_KN + wn * (BT / 2) + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)
-                          : TILE_ELEMS + (wn * (BT / 2) + (lane & 31)) * LDS_ROW + (lane >> 5) * 8;
-    // MFMA operands are double-buffered in registers: the LDS reads of the next 16-wide k step are
-    // in flight while the 16 MFMAs of the current one issue (one wave per SIMD, nothing else hides them)
+    // operand fetches.  K-contiguous tile: lane = row lane%32 of a 32-row MFMA block, k chunk 2kk + lane/32
+    const int ra0 = wm * (BT / 2) + (lane & 31), rb0 = wn * (BT / 2) + (lane & 31);
+    const int a_rd0 = (ra0 >> 4) * 1024 + (ra0 & 15) * 64 + (((lane >> 5) ^ ((ra0 >> 2) & 3)) * 16);                 // kk = 0; kk = 1 is this ^ 32
+    const int b_rd0 = OP_BYTES + (rb0 >> 4) * 1024 + (rb0 & 15) * 64 + (((lane >> 5) ^ ((rb0 >> 2) & 3)) * 16);
+    // [k][n] tile, transposing read (ds_read_b64_tr_b16: within a 16-lane group, lane i receives as element e element i%4 of
+    // the 8 bytes that lane 4e + i/4 addressed; groups 0/1 cover columns 0-15 / 16-31 of a 32-column MFMA block, groups 2/3
+    // the same columns of the next 8 k): lane -> k row 8(lane/32) + (lane%16)/4,
+    // columns 16((lane/16)%2) + 4(lane%4) of the 32-column MFMA block j of this wave; the block's 64-byte group is wn*4 + j
+    const int kn_q2 = (lane & 15) >> 2, kn_h = lane >> 5;
+    const int kn_rd0 = OP_BYTES + (8 * kn_h + kn_q2) * 512 + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+    const int kn_sw = kn_q2 | (kn_h << 2);
     bf16x8 av[2][TM], bv[2][TN];
-    auto lds_load = [&](const bf16_t* stage, int kk, int s) {
+    auto lds_load = [&](int stage, int kk, int s) {
+        const unsigned char* base = lds + stage * STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < TM; i++) av[s][i] = *reinterpret_cast<const bf16x8*>(stage + a_off + i * 32 * LDS_ROW + kk * 16);
+        for (int i = 0; i < TM; i++) av[s][i] = *reinterpret_cast<const bf16x8*>(base + ((a_rd0 ^ (kk * 32)) + i * 2048));
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             if (BKN) {
-                const bf16_t* q = stage + b_off + j * 32 + kk * 16 * LDS_ROW_KN;
+                const unsigned char* q = base + kn_rd0 + (((wn * 4 + j) ^ kn_sw) << 6) + kk * 16 * 512;
                 const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q));
-                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * LDS_ROW_KN));
+                const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * 512));
                 typedef short i16x8 __attribute__((ext_vector_type(8)));
                 const i16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 bv[s][j] = __builtin_bit_cast(bf16x8, both);
             } else {
-                bv[s][j] = *reinterpret_cast<const bf16x8*>(stage + b_off + j * 32 * LDS_ROW + kk * 16);
+                bv[s][j] = *reinterpret_cast<const bf16x8*>(base + ((b_rd0 ^ (kk * 32)) + j * 2048));
             }
         }
     };
@@ -381,12 +388,12 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
             for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[s][i], bv[s][j], acc[i][j], 0, 0, 0);
     };
 
-    const int nk = K / BK;      // a multiple of 4: K is a multiple of 256
+    const int nk = K / BKD;      // a multiple of 8: K is a multiple of 256
     const bf16_t* aux = Mt.G;
     const int gcol0 = tn * BT + wn * (BT / 2);
     // the auxiliary operand of the polynomial's epilogue (G):
     // 8 x 16 bytes per lane and 32-row block of this wave's 128 x 128 tile.  The first two blocks are requested during
-    // the last K tile (whose register sets are free by then), each later one while the block two before it is
+    // the last K tile, each later one while the block two before it is
     // being written, so that the epilogue does not wait for memory
     u32x4 ax[2][8];
     auto aux_load = [&](int i) {
@@ -396,91 +403,65 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
             ax[i & 1][c] = *(gvec_p)(aux + (size_t)(tm * BT + wm * (BT / 2) + i * 32 + row) * ldc + gcol0 + c8 * 8);
         }
     };
-    gload_a(0, 0); gload_b(0, 0);
-    sstore_a(0, smem); sstore_b(0, smem);
-    gload_a(1, 1); gload_b(1, 1);
-    gload_a(0, 2); gload_b(0, 2);
+    // wait until at most n of this wave's loads are outstanding (vmcnt only; the other counters unconstrained)
+#define SG_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
+    dma_tile(0); dma_tile(1); dma_tile(2); dma_tile(3);
+    SG_WAIT_VM(24);
     __syncthreads();
-    lds_load(smem, 0, 0);
-    // One wave per SIMD issues in order, so a burst of memory instructions leaves the MFMA pipe
-    // idle while it issues, and an operand that is requested late stalls the whole SIMD.  Each K tile is four
-    // phases of 16 MFMAs.  The LDS reads of the next k step go between the first eight MFMAs of a phase (an
-    // operand then has at least eight MFMAs, 256 clocks, to arrive), the LDS writes of tile kt+1 and the global
-    // loads of tile kt+3 between the last eight, all placed with sched_group_barrier (masks: 0x008 MFMA,
-    // 0x020 VMEM read, 0x100 LDS read, 0x200 LDS write).  The workgroup barrier sits before the last phase:
-    // by then every wave has issued all its reads of the current stage and written its share of the next one,
-    // so the last phase's MFMAs cover the first operand reads of the next tile.  The steady-state body issues
-    // everything unconditionally (a static wait count has to be right on every path); the last four K tiles
-    // are peeled.
-    auto ktile = [&](int kt, auto set_c, auto store_c, auto load_c, auto last_c) {
-        constexpr int S = decltype(set_c)::value;       // register set holding tile kt+1
-        constexpr bool LD = decltype(load_c)::value != 0, ST = decltype(store_c)::value != 0, LAST = decltype(last_c)::value != 0;
-        const bf16_t* cur = smem + (kt & 1) * 2 * TILE_ELEMS;
-        bf16_t* nxt = smem + ((kt + 1) & 1) * 2 * TILE_ELEMS;
+    lds_load(0, 0, 0);
+    // A K tile is two phases of 16 MFMAs.  Phase 0 multiplies k step 0 while the operands of k step 1 are read; then
+    // the wave makes sure the next tile has landed (its loads were issued three tiles ago: only the two tiles after it
+    // may still be in flight) and that its own reads of this stage are done, the workgroup meets, and the stage is
+    // handed to the loads of the tile four ahead; phase 1 multiplies k step 1 while the first operands of the next
+    // tile are read.
+    // Phase 1 is written out as eight pairs of MFMAs, each followed by one load of the tile four ahead and one operand
+    // read of the next tile: a burst of memory instructions would leave the matrix pipe idle while it issues.
+    auto ktile = [&](int kt, auto dma_c, auto wait_c, auto next_c) {
+        constexpr bool DMA = decltype(dma_c)::value != 0, NEXT = decltype(next_c)::value != 0;
+        constexpr int WAIT = decltype(wait_c)::value;      // loads that may stay in flight once the next tile has landed
+        const int stage = kt & (STAGES - 1), nstage = (kt + 1) & (STAGES - 1);
         __builtin_amdgcn_sched_barrier(0);
-        // phase 0: k step 0 | read k step 1
-        lds_load(cur, 1, 1);
+        lds_load(stage, 1, 1);
         mma(0);
         SG_MUON_SCHED_READS();
         __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // phase 1: k step 1 | read k step 2, write A of tile kt+1
-        lds_load(cur, 2, 0);
-        if (ST) sstore_a(S, nxt);
-        mma(1);
-        SG_MUON_SCHED_READS();
-#pragma unroll
-        for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // phase 2: k step 2 | read k step 3, write B of tile kt+1, load A of tile kt+3
-        lds_load(cur, 3, 1);
-        if (ST) sstore_b(S, nxt);
-        if (LD) gload_a(S, kt + 3);
-        mma(0);
-        SG_MUON_SCHED_READS();
-#pragma unroll
-        for (int g = 0; g < 8; g++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (ST) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        if (NEXT) SG_WAIT_VM(WAIT);
+        __builtin_amdgcn_s_waitcnt(0xC07F);     // lgkmcnt(0): this wave's reads of the stage have returned
         __syncthreads();
-        // phase 3: k step 3 | read k step 0 of tile kt+1, load B of tile kt+3 (last tile: the polynomial's auxiliary operand)
-        if (!LAST) lds_load(nxt, 0, 0);
-        if (LD) gload_b(S, kt + 3);
-        if (LAST && EPI == EPI_POLY) { aux_load(0); aux_load(1); }
-        mma(1);
-        if (!LAST) {
-            SG_MUON_SCHED_READS();
+        if (!NEXT && EPI == EPI_POLY) { aux_load(0); aux_load(1); }
+        const unsigned char* nbase = lds + nstage * STAGE_BYTES;
 #pragma unroll
-            for (int g = 0; g < 8; g++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (LD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        for (int g = 0; g < 8; g++) {
+            // operand reads of the next tile's k step 0: A block g/2 ... (K-contiguous B: one read per pair; [k][n] B: the
+            // two transposing reads of a block after pairs 4-7)
+            if (NEXT) {
+                if (g < TM) av[0][g] = *reinterpret_cast<const bf16x8*>(nbase + a_rd0 + g * 2048);
+                else if (!BKN) bv[0][g - TM] = *reinterpret_cast<const bf16x8*>(nbase + b_rd0 + (g - TM) * 2048);
+                else {
+                    const unsigned char* q = nbase + kn_rd0 + (((wn * 4 + (g - TM)) ^ kn_sw) << 6);
+                    const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q));
+                    const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * 512));
+                    bv[0][g - TM] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
             }
-        } else if (EPI == EPI_POLY) {
 #pragma unroll
-            for (int g = 0; g < 16; g++) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            }
+            for (int m = 2 * g; m < 2 * g + 2; m++)
+                acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][m >> 2], bv[1][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (DMA) dma_one(kt + 4, g);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
     };
     using c0 = std::integral_constant<int, 0>;
     using c1 = std::integral_constant<int, 1>;
     int kt = 0;
-    for (; kt + 4 < nk; kt += 2) {
-        ktile(kt, c1{}, c1{}, c1{}, c0{});
-        ktile(kt + 1, c0{}, c1{}, c1{}, c0{});
-    }
-    ktile(kt, c1{}, c1{}, c1{}, c0{});        // kt = nk-4: loads the last tile
-    ktile(kt + 1, c0{}, c1{}, c0{}, c0{});
-    ktile(kt + 2, c1{}, c1{}, c0{}, c0{});
-    ktile(kt + 3, c0{}, c0{}, c0{}, c1{});
+    for (; kt + 4 < nk; kt++) ktile(kt, c1{}, std::integral_constant<int, 16>{}, c1{});     // steady state
+    ktile(kt, c0{}, std::integral_constant<int, 16>{}, c1{});           // tiles nk-2 and nk-1 may still be in flight
+    ktile(kt + 1, c0{}, std::integral_constant<int, 8>{}, c1{});
+    ktile(kt + 2, c0{}, std::integral_constant<int, 0>{}, c1{});
+    ktile(kt + 3, c0{}, std::integral_constant<int, 0>{}, c0{});
+#undef SG_WAIT_VM
     __syncthreads();        // the epilogue reuses the LDS stages: every wave is done reading them
 
     // ---- epilogue, staged through LDS (free after the last barrier) so that global memory sees
