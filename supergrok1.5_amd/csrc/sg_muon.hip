@@ -25,9 +25,9 @@
 // Work buffers are zero-padded to multiples of 256 so the GEMM needs no edge
 // handling (zero rows/columns stay zero through the iteration).
 //
-// GEMM: 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each
-// wave 128x128 = 4x4 MFMA 32x32x16 bf16 tiles (256 fp32 accumulators per
-// lane), K tiles of 32 in four LDS stages, filled by loads that go from global
+// GEMM: 256x256 output tile per 512-thread workgroup, 8 waves as 2x4, each
+// wave 128x64 = 4x2 MFMA 32x32x16 bf16 tiles (128 fp32 accumulators per
+// lane, two waves per SIMD), K tiles of 32 in four LDS stages, filled by loads that go from global
 // memory straight into LDS (global_load_lds_dwordx4) three tiles ahead of their
 // use; no padding is possible in such a copy, so the tiles are swizzled by the
 // choice of the chunk each lane fetches (conflict-free operand fetches); memory
@@ -50,6 +50,12 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int BT = 256;            // GEMM tile (M and N)
+// Waves of a workgroup along N (2 along M).  Eight waves of 128 x 64 (two per SIMD, 128 accumulators each) measured
+// 3.5 % faster per step than four waves of 128 x 128: they fetch 1.5 x the operand bytes from LDS, but a second wave per
+// SIMD covers the fetch latencies that one wave cannot.
+constexpr int GWN = 4;
+constexpr int GWAVES = 2 * GWN, GTHREADS = 64 * GWAVES;
+constexpr int WCOLS = BT / GWN;      // columns of a wave's block
 constexpr int GEMM_LDS_BYTES = 4 * 2 * BT * 32 * 2;          // four stages of {A tile, B tile} of 32 k: 131,072 bytes of the CU's 160 KB
 constexpr float NS_A = 3.4445f, NS_B = -4.7750f, NS_C = 2.0315f;
 
@@ -213,8 +219,7 @@ __global__ __launch_bounds__(256) void k_norm(Batch B) {
 }
 
 // ---- GEMM  C[M x N] = A[M x K] * B  with fused epilogues; B given as [N x K] (Gram, polynomial) or as [K x N] (apply)
-// 256x256 output tile per 256-thread workgroup, 4 waves as 2x2, each wave 128x128 = 4x4 MFMA
-// 32x32x16 tiles (256 fp32 accumulators per lane; one wave per SIMD, the whole register file).
+// 256x256 output tile per workgroup of 2 x GWN waves, each wave 128 x (256/GWN) as MFMA 32x32x16 tiles.
 // Per 16-wide k step a wave fetches 4+4 16-byte operands from LDS for 16 MFMAs.
 // The Gram and polynomial products are symmetric: only tiles on or above the diagonal are
 // computed, each off-diagonal tile is also stored transposed.
@@ -230,25 +235,16 @@ __device__ __forceinline__ uint32_t bf16r2(float lo, float hi) {
     return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
 }
 
-// the first eight MFMAs of a phase, each followed by one LDS read of the next k step (the [K x N] operand takes twelve
-// reads per k step: two after each of the first four)
-#define SG_MUON_SCHED_READS()                                                  \
-    do {                                                                       \
-        if (BKN) {                                                             \
-            _Pragma("unroll") for (int g_ = 0; g_ < 4; g_++) {                 \
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
-                __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);             \
-            }                                                                  \
-            _Pragma("unroll") for (int g_ = 0; g_ < 4; g_++) {                 \
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             \
-            }                                                                  \
-        } else {                                                               \
-            _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                 \
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             \
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             \
-            }                                                                  \
-        }                                                                      \
+// The R operand reads of the next k step are dealt over the first eight of a phase's M MFMAs (R/8 after each, one more
+// after the first R%8), the other MFMAs follow on their own
+#define SG_MUON_SCHED_READS(R, M)                                                       \
+    do {                                                                               \
+        _Pragma("unroll") for (int g_ = 0; g_ < 8; g_++) {                              \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          \
+            if ((R) / 8 + (g_ < (R) % 8 ? 1 : 0) == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); \
+            else if ((R) / 8 + (g_ < (R) % 8 ? 1 : 0) == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); \
+        }                                                                              \
+        if ((M) > 8) __builtin_amdgcn_sched_group_barrier(0x008, (M) - 8, 0);           \
     } while (0)
 
 typedef short i16x4 __attribute__((ext_vector_type(4)));
@@ -257,9 +253,10 @@ typedef __attribute__((address_space(3))) i16x4* lds_i16x4_p;
 // y_sel: which of the two Y buffers holds the current iterate
 // iter_flags: bit 1 = first iteration (Y still carries the factor norm: see k_momentum)
 template <int EPI>
-__global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_flags) {
+__global__ __launch_bounds__(GTHREADS) void k_gemm_nt(Batch Bt, int y_sel, int iter_flags) {
     constexpr bool BKN = EPI == EPI_APPLY;             // B operand stored [K x N]
-    constexpr int TM = BT / 64, TN = BT / 64;          // MFMA tiles per wave in each direction (4 x 4)
+    constexpr int TM = BT / 64, TN = WCOLS / 32;       // MFMA tiles per wave in each direction (4 x 4 or 4 x 2)
+    constexpr int LPT = 16 / GWAVES;                  // loads per wave, tile and operand (a tile is 16 blocks of 1 KB)
     extern __shared__ __attribute__((aligned(16))) bf16_t smem[];
 
     // XCD-contiguous tile order: hardware deals consecutive workgroups round-robin over the 8 XCDs,
@@ -268,7 +265,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     int lb = blockIdx.x;
     if (nblk % 8 == 0) lb = (blockIdx.x % 8) * (nblk / 8) + blockIdx.x / 8;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / GWN, wn = wave % GWN;
     const sg::cint_p prefix = sg::as_const(Bt.gtile_prefix[EPI]);
     const int mi = sg::upper_seg(prefix, Bt.P, lb);
     const Mat& Mt = Bt.mats[mi];
@@ -332,27 +329,28 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n" : : "v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
     };
     // this lane's share of a block: row lane/4 of the block's 16 (block 4i + w of the tile), chunk (lane%4) ^ ((lane/16)%4)
+    // (block GWAVES*i + w of the tile for this wave's i-th load)
     const uint32_t lo_a = (uint32_t)((((lane >> 2) + 16 * wv) * lda + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2);
     const uint32_t lo_b = (uint32_t)((((lane >> 2) + 16 * wv) * ldb + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2);
-    // [k][n] tile: wave w, instruction i loads k rows 8i + 2w + lane/32; sw of that row = (2(w&1) + lane/32) | ((i&1) << 2)
+    // [k][n] tile: wave w's i-th load fetches k rows 2(GWAVES*i + w) + lane/32; sw of a row k is (k & 3) | ((k >> 1) & 4)
     const int kn_row = 2 * wv + (lane >> 5);
-    const int kn_c0 = (lane & 31) ^ ((kn_row & 3) << 2);
-    const uint32_t lo_kn0 = (uint32_t)((kn_row * ldb + kn_c0 * 8) * 2);            // i even
-    const uint32_t lo_kn1 = (uint32_t)((kn_row * ldb + (kn_c0 ^ 16) * 8) * 2);     // i odd
-    // the q-th of a tile's eight loads (0-3: A, 4-7: B)
+    const int kn_c0 = (lane & 31) ^ ((((kn_row & 3) | ((kn_row >> 1) & 4)) & 7) << 2);
+    const uint32_t lo_kn0 = (uint32_t)((kn_row * ldb + kn_c0 * 8) * 2);            // rows whose bit 3 is that of 2w + lane/32
+    const uint32_t lo_kn1 = (uint32_t)((kn_row * ldb + (kn_c0 ^ 16) * 8) * 2);     // ... the other value (four waves: odd i)
+    // the q-th of a tile's 2*LPT loads (first the A tile's, then the B tile's)
     auto dma_one = [&](int kt, int q) {
         const uint32_t st = lds0 + (uint32_t)(kt & (STAGES - 1)) * STAGE_BYTES;
-        const int i = q & 3, blk = 4 * i + wv;
-        if (q < 4) dma16(lo_a, reinterpret_cast<const char*>(A) + ((size_t)i * 64 * lda + (size_t)kt * BKD) * 2, st + blk * 1024);
-        else if (BKN) dma16((i & 1) ? lo_kn1 : lo_kn0, reinterpret_cast<const char*>(B) + (size_t)(kt * BKD + 8 * i) * ldb * 2, st + OP_BYTES + blk * 1024);
-        else dma16(lo_b, reinterpret_cast<const char*>(B) + ((size_t)i * 64 * ldb + (size_t)kt * BKD) * 2, st + OP_BYTES + blk * 1024);
+        const int i = q % LPT, blk = GWAVES * i + wv;
+        if (q < LPT) dma16(lo_a, reinterpret_cast<const char*>(A) + ((size_t)i * 16 * GWAVES * lda + (size_t)kt * BKD) * 2, st + blk * 1024);
+        else if (BKN) dma16(((2 * GWAVES * i) & 8) ? lo_kn1 : lo_kn0, reinterpret_cast<const char*>(B) + (size_t)(kt * BKD + 2 * GWAVES * i) * ldb * 2, st + OP_BYTES + blk * 1024);
+        else dma16(lo_b, reinterpret_cast<const char*>(B) + ((size_t)i * 16 * GWAVES * ldb + (size_t)kt * BKD) * 2, st + OP_BYTES + blk * 1024);
     };
     auto dma_tile = [&](int kt) {
 #pragma unroll
-        for (int q = 0; q < 8; q++) dma_one(kt, q);
+        for (int q = 0; q < 2 * LPT; q++) dma_one(kt, q);
     };
     // operand fetches.  K-contiguous tile: lane = row lane%32 of a 32-row MFMA block, k chunk 2kk + lane/32
-    const int ra0 = wm * (BT / 2) + (lane & 31), rb0 = wn * (BT / 2) + (lane & 31);
+    const int ra0 = wm * (BT / 2) + (lane & 31), rb0 = wn * WCOLS + (lane & 31);
     const int a_rd0 = (ra0 >> 4) * 1024 + (ra0 & 15) * 64 + (((lane >> 5) ^ ((ra0 >> 2) & 3)) * 16);                 // kk = 0; kk = 1 is this ^ 32
     const int b_rd0 = OP_BYTES + (rb0 >> 4) * 1024 + (rb0 & 15) * 64 + (((lane >> 5) ^ ((rb0 >> 2) & 3)) * 16);
     // [k][n] tile, transposing read (ds_read_b64_tr_b16: within a 16-lane group, lane i receives as element e element i%4 of
@@ -362,6 +360,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
     const int kn_q2 = (lane & 15) >> 2, kn_h = lane >> 5;
     const int kn_rd0 = OP_BYTES + (8 * kn_h + kn_q2) * 512 + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
     const int kn_sw = kn_q2 | (kn_h << 2);
+    constexpr int NREADS = TM + TN * (BKN ? 2 : 1);     // LDS reads of a k step's operands
     bf16x8 av[2][TM], bv[2][TN];
     auto lds_load = [&](int stage, int kk, int s) {
         const unsigned char* base = lds + stage * STAGE_BYTES;
@@ -370,7 +369,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             if (BKN) {
-                const unsigned char* q = base + kn_rd0 + (((wn * 4 + j) ^ kn_sw) << 6) + kk * 16 * 512;
+                const unsigned char* q = base + kn_rd0 + (((wn * TN + j) ^ kn_sw) << 6) + kk * 16 * 512;
                 const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q));
                 const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * 512));
                 typedef short i16x8 __attribute__((ext_vector_type(8)));
@@ -390,23 +389,23 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
 
     const int nk = K / BKD;      // a multiple of 8: K is a multiple of 256
     const bf16_t* aux = Mt.G;
-    const int gcol0 = tn * BT + wn * (BT / 2);
+    const int gcol0 = tn * BT + wn * WCOLS;
     // the auxiliary operand of the polynomial's epilogue (G):
-    // 8 x 16 bytes per lane and 32-row block of this wave's 128 x 128 tile.  The first two blocks are requested during
+    // 16 bytes per lane and 8-column chunk of a 32-row block of this wave's tile.  The first two blocks are requested during
     // the last K tile, each later one while the block two before it is
     // being written, so that the epilogue does not wait for memory
-    u32x4 ax[2][8];
+    u32x4 ax[2][WCOLS / 16];
     auto aux_load = [&](int i) {
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
+        for (int c = 0; c < WCOLS / 16; c++) {
+            const int id = lane + 64 * c, row = id / (WCOLS / 8), c8 = id % (WCOLS / 8);
             ax[i & 1][c] = *(gvec_p)(aux + (size_t)(tm * BT + wm * (BT / 2) + i * 32 + row) * ldc + gcol0 + c8 * 8);
         }
     };
     // wait until at most n of this wave's loads are outstanding (vmcnt only; the other counters unconstrained)
 #define SG_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(0x0F70 | ((n) & 15) | (((n) >> 4) << 14))
     dma_tile(0); dma_tile(1); dma_tile(2); dma_tile(3);
-    SG_WAIT_VM(24);
+    SG_WAIT_VM(6 * LPT);
     __syncthreads();
     lds_load(0, 0, 0);
     // A K tile is two phases of 16 MFMAs.  Phase 0 multiplies k step 0 while the operands of k step 1 are read; then
@@ -423,42 +422,42 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
         __builtin_amdgcn_sched_barrier(0);
         lds_load(stage, 1, 1);
         mma(0);
-        SG_MUON_SCHED_READS();
-        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        SG_MUON_SCHED_READS(NREADS, TM * TN);
         __builtin_amdgcn_sched_barrier(0);
         if (NEXT) SG_WAIT_VM(WAIT);
         __builtin_amdgcn_s_waitcnt(0xC07F);     // lgkmcnt(0): this wave's reads of the stage have returned
         __syncthreads();
         if (!NEXT && EPI == EPI_POLY) { aux_load(0); aux_load(1); }
         const unsigned char* nbase = lds + nstage * STAGE_BYTES;
+        constexpr int MPG = TM * TN / 8;        // MFMAs per group
 #pragma unroll
         for (int g = 0; g < 8; g++) {
-            // operand reads of the next tile's k step 0: A block g/2 ... (K-contiguous B: one read per pair; [k][n] B: the
-            // two transposing reads of a block after pairs 4-7)
+            // operand reads of the next tile's k step 0: one fragment per group
             if (NEXT) {
                 if (g < TM) av[0][g] = *reinterpret_cast<const bf16x8*>(nbase + a_rd0 + g * 2048);
+                else if (g - TM >= TN) {}
                 else if (!BKN) bv[0][g - TM] = *reinterpret_cast<const bf16x8*>(nbase + b_rd0 + (g - TM) * 2048);
                 else {
-                    const unsigned char* q = nbase + kn_rd0 + (((wn * 4 + (g - TM)) ^ kn_sw) << 6);
+                    const unsigned char* q = nbase + kn_rd0 + (((wn * TN + (g - TM)) ^ kn_sw) << 6);
                     const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q));
                     const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_i16x4_p)(q + 4 * 512));
                     bv[0][g - TM] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
                 }
             }
 #pragma unroll
-            for (int m = 2 * g; m < 2 * g + 2; m++)
-                acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][m >> 2], bv[1][m & 3], acc[m >> 2][m & 3], 0, 0, 0);
+            for (int m = MPG * g; m < MPG * (g + 1); m++)
+                acc[m / TN][m % TN] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1][m / TN], bv[1][m % TN], acc[m / TN][m % TN], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (DMA) dma_one(kt + 4, g);
+            if (DMA && g < 2 * LPT) dma_one(kt + 4, g);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
     using c0 = std::integral_constant<int, 0>;
     using c1 = std::integral_constant<int, 1>;
     int kt = 0;
-    for (; kt + 4 < nk; kt++) ktile(kt, c1{}, std::integral_constant<int, 16>{}, c1{});     // steady state
-    ktile(kt, c0{}, std::integral_constant<int, 16>{}, c1{});           // tiles nk-2 and nk-1 may still be in flight
-    ktile(kt + 1, c0{}, std::integral_constant<int, 8>{}, c1{});
+    for (; kt + 4 < nk; kt++) ktile(kt, c1{}, std::integral_constant<int, 4 * LPT>{}, c1{});     // steady state
+    ktile(kt, c0{}, std::integral_constant<int, 4 * LPT>{}, c1{});      // tiles nk-2 and nk-1 may still be in flight
+    ktile(kt + 1, c0{}, std::integral_constant<int, 2 * LPT>{}, c1{});
     ktile(kt + 2, c0{}, std::integral_constant<int, 0>{}, c1{});
     ktile(kt + 3, c0{}, std::integral_constant<int, 0>{}, c0{});
 #undef SG_WAIT_VM
@@ -466,21 +465,23 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
 
     // ---- epilogue, staged through LDS (free after the last barrier) so that global memory sees
     // 16-byte accesses along rows.  Accumulator element e of MFMA tile (i,j) is
-    // row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.  One 32-row block of the wave's 128x128
+    // row 8*(e/4) + 4*(lane/32) + e%4, column lane%32.  One 32-row block of the wave's
     // tile at a time: fp32 block -> LDS, read back as 8-column chunks, combine with the auxiliary
     // operand, round to bf16 and store.  Off-diagonal tiles of the symmetric products also store
     // the transposed block: the rounded values go back into the staged block and are read down
     // its columns.  Every wave stages in its own LDS region and LDS executes a wave's
     // instructions in order, so no workgroup barrier is needed, only the compiler kept from
     // reordering (wave_barrier).
-    constexpr int EP_ROW = 128 + 4;     // floats per staged row
-    static_assert(4 * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
+    constexpr int EP_ROW = WCOLS + 4;     // floats per staged row
+    constexpr int RCH = WCOLS / 8;        // 8-column chunks per row
+    constexpr int NC = 32 * RCH / 64;     // chunks per lane and 32-row block
+    static_assert(GWAVES * 32 * EP_ROW * 4 <= GEMM_LDS_BYTES, "epilogue staging exceeds the GEMM's LDS");
     float* ep = reinterpret_cast<float*>(smem) + wave * (32 * EP_ROW);
     // uniform over the workgroup
     const bool mirror = EPI != EPI_APPLY && tm != tn;
     // first iteration: Y is the unnormalised momentum, so its Gram matrix carries 1/norm^2 and the applied Y 1/norm
     const float inv = Bt.inv_norm[mi];
-    const bool diag_wave = EPI == EPI_POLY && tm == tn && wm == wn;     // this wave's 128 x 128 block lies on the diagonal
+    const bool diag_wave = EPI == EPI_POLY && tm == tn && wn / (GWN / 2) == wm;     // this wave's block meets the diagonal
     const bool first = (iter_flags & 2) != 0;
     const float first_scale = first ? (EPI == EPI_GRAM ? inv * inv : (EPI == EPI_APPLY ? inv : 1.0f)) : 1.0f;
 #pragma unroll
@@ -493,8 +494,8 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
                 ep[(8 * (e >> 2) + 4 * (lane >> 5) + (e & 3)) * EP_ROW + 32 * j + (lane & 31)] = acc[i][j][e];
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            const int id = lane + 64 * c, row = id >> 4, c8 = id & 15;
+        for (int c = 0; c < NC; c++) {
+            const int id = lane + 64 * c, row = id / RCH, c8 = id % RCH;
             f32x4* src = reinterpret_cast<f32x4*>(&ep[row * EP_ROW + c8 * 8]);
             const f32x4 lo = src[0], hi = src[1];
             float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -506,7 +507,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
                     v[k] = sg_fma(NS_C, v[k], NS_B * x);
                 }
                 if (diag_wave) {        // H + a I: the apply step is then the single product (H + a I) Y
-                    const int dk = i * 32 + row - c8 * 8;
+                    const int dk = (wm * (BT / 2) + i * 32 + row) - (wn * WCOLS + c8 * 8);
 #pragma unroll
                     for (int k = 0; k < 8; k++) v[k] += (dk == k) ? NS_A : 0.0f;
                 }
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(256) void k_gemm_nt(Batch Bt, int y_sel, int iter_f
         if (mirror) {
             const uint32_t* epb = reinterpret_cast<const uint32_t*>(ep);
 #pragma unroll
-            for (int c = 0; c < 8; c++) {
+            for (int c = 0; c < NC; c++) {
                 const int id = lane + 64 * c, col = id >> 2, r8 = id & 3;
                 u32x4 t;
 #pragma unroll
@@ -741,9 +742,9 @@ int sg_muon_step(int num_matrices, const SgMuonMatrix* mats, float momentum, flo
     SG_LAUNCH_CHECK("muon prologue");
     for (int it = 0; it < ns_steps; it++) {
         const int sel = it & 1, last = it == 0 ? 2 : 0;     // iter_flags
-        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
-        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(256), GEMM_LDS_BYTES, st, B, sel, last);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_GRAM>, dim3(B.gtiles[EPI_GRAM]), dim3(GTHREADS), GEMM_LDS_BYTES, st, B, sel, last);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_POLY>, dim3(B.gtiles[EPI_POLY]), dim3(GTHREADS), GEMM_LDS_BYTES, st, B, sel, last);
+        hipLaunchKernelGGL(k_gemm_nt<EPI_APPLY>, dim3(B.gtiles[EPI_APPLY]), dim3(GTHREADS), GEMM_LDS_BYTES, st, B, sel, last);
         SG_LAUNCH_CHECK("muon newton-schulz");
     }
     hipLaunchKernelGGL(k_update, dim3(B.ttiles), dim3(256), 0, st, B, lr, 1.0f - lr * wd, ns_steps & 1, ns_steps == 0 ? 1 : 0);
