@@ -354,7 +354,7 @@ SG_HD void sg_tanh_block(int n, const float* x, float* out) {
  * "erfcc"), fractional error below 1.2e-7 for every x. */
 SG_HD float sg_erfc(float x) {
     const float ax = sg_abs(x);
-    const float t = 1.0f / sg_fma(0.5f, ax, 1.0f);
+    const float t = sg_rcp_pos(sg_fma(0.5f, ax, 1.0f));      /* denominator >= 1: Newton reciprocal, no IEEE division sequence */
     float p = 0.17087277f;
     p = sg_fma(p, t, -0.82215223f);
     p = sg_fma(p, t, 1.48851587f);
