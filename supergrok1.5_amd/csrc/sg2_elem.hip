@@ -22,6 +22,7 @@ namespace {
 constexpr int ELEM_THREADS = 256;
 constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[16] W2[16] + pad
 typedef float vf4 __attribute__((ext_vector_type(4)));
+typedef float vf32 __attribute__((ext_vector_type(32)));
 
 template <class G, bool DBG>
 __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
@@ -54,7 +55,17 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
     const sg::cfloat_p br0 = sg::as_const(pl.W.w[W_GRU_BR]);
     const sg::cfloat_p Wh0 = sg::as_const(pl.W.w[W_GRU_WH]);
     const sg::cfloat_p bh0 = sg::as_const(pl.W.w[W_GRU_BH]);
-    const sg::cfloat_p Wq0 = sg::as_const(pl.W.w[W_PEER_Q]);
+    // The query projection runs on the matrix pipe: v_mfma_f32_32x32x1_2b is one fused multiply-add per output and
+    // step, so a chain of them is the fmaf chain of the scalar form, bit for bit, in the same order.  Lane l supplies
+    // row l % 32 of each 32-row slice of the query matrix (held in registers for the whole kernel) and its own
+    // element's inputs; the outputs come back split over lanes l and l ^ 32 and are exchanged below.
+    constexpr int NQM = NH * DM / 32;
+    static_assert(NH * DM % 32 == 0 && 32 % DM == 0, "query rows are handled in slices of 32");
+    float aq[NQM][PIN];
+#pragma unroll
+    for (int m = 0; m < NQM; m++)
+#pragma unroll
+        for (int q = 0; q < PIN; q++) aq[m][q] = pl.W.w[W_PEER_Q][(m * 32 + (threadIdx.x & 31)) * PIN + q];
     const sg::cfloat_p KA0 = sg::as_const(pl.W.w[W_KEYS_A]);
     const sg::cfloat_p KB0 = sg::as_const(pl.W.w[W_KEYS_B]);
 
@@ -68,12 +79,15 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
         const float alpha = T.alpha, lamb = T.lamb, beta1 = T.beta1, bc2 = T.bc2, step_size = T.step_size;
         const float beta2 = pl.beta2, eps = pl.eps, rescale = pl.rescale, decay = pl.decay;
 
-        for (int k = threadIdx.x; k < cnt; k += ELEM_THREADS) {
-            const int i = start + k;
+        // every lane runs every iteration (the matrix instructions ignore the execution mask); lanes past the end
+        // of the tile recompute its last element and store nothing
+        for (int k0 = 0; k0 < cnt; k0 += ELEM_THREADS) {
+            const bool live = k0 + (int)threadIdx.x < cnt;
+            const int i = start + min(k0 + (int)threadIdx.x, cnt - 1);
             // the weights are re-read (scalar loads, cache hits) for every element instead of being hoisted
             const int zo = sg::opaque_zero();
             const sg::cfloat_p Wz = Wz0 + zo, bz = bz0 + zo, Wr = Wr0 + zo, br = br0 + zo, Wh = Wh0 + zo, bh = bh0 + zo;
-            const sg::cfloat_p Wq = Wq0 + zo, KA = KA0 + zo, KB = KB0 + zo;
+            const sg::cfloat_p KA = KA0 + zo, KB = KB0 + zo;
             const float g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, i));
             const float s = has_s ? sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i)) : 0.0f;
             float cf[DM], cb[DM], hold[GH];
@@ -131,27 +145,37 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
             sg_tanh_block(GH, pre_c, cand);
 #pragma unroll
             for (int j = 0; j < GH; j++) hnew[j] = sg_fma(zg[j], cand[j], (1.0f - zg[j]) * hold[j]);
-            ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
+            if (live) ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
+
+            // ---- PEER queries: chain order = h, fwd ctx, bwd ctx, g, s
+            float qall[NH * DM];
+#pragma unroll
+            for (int m = 0; m < NQM; m++) {
+                vf32 acc = {};
+                int c = 0;
+#pragma unroll
+                for (int q = 0; q < GH; q++, c++) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(aq[m][c], hnew[q], acc, 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < DM; q++, c++) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(aq[m][c], cf[q], acc, 0, 0, 0);
+#pragma unroll
+                for (int q = 0; q < DM; q++, c++) acc = __builtin_amdgcn_mfma_f32_32x32x1f32(aq[m][c], cb[q], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x1f32(aq[m][c], g, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x1f32(aq[m][c + 1], s, acc, 0, 0, 0);
+                // register r of block b holds row 8 (r / 4) + 4 (lane / 32) + r % 4 of element 32 b + lane % 32:
+                // exchanging the upper half of block 0 with the lower half of block 1 gives each lane its own element
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const auto pr = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc[r]), __float_as_uint(acc[16 + r]), false, false);
+                    qall[m * 32 + 8 * (r / 4) + r % 4] = __uint_as_float(pr[0]);
+                    qall[m * 32 + 8 * (r / 4) + 4 + r % 4] = __uint_as_float(pr[1]);
+                }
+            }
 
             // ---- PEER routing + expert MLP
             float total = 0.0f;
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
-                float query[DM];
-#pragma unroll
-                for (int dd = 0; dd < DM; dd++) {
-                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
-                    float v = 0.0f;
-#pragma unroll
-                    for (int q = 0; q < GH; q++) v = sg_fma(qr[q], hnew[q], v);
-#pragma unroll
-                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + q], cf[q], v);
-#pragma unroll
-                    for (int q = 0; q < DM; q++) v = sg_fma(qr[GH + DM + q], cb[q], v);
-                    v = sg_fma(qr[GH + 2 * DM], g, v);
-                    v = sg_fma(qr[GH + 2 * DM + 1], s, v);
-                    query[dd] = v;
-                }
+                const float* query = qall + hh * DM;
                 int best[2];
 #pragma unroll
                 for (int hf = 0; hf < 2; hf++) {
@@ -169,8 +193,8 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
                 }
                 int e = best[0] * PK + best[1];
                 if (e >= NE) e = NE - 1;
-                atomicAdd(&s_cnt[e], 1);
-                if (DBG) dbg_eidx[((size_t)T.off + i) * NH + hh] = e;
+                if (live) atomicAdd(&s_cnt[e], 1);
+                if (DBG && live) dbg_eidx[((size_t)T.off + i) * NH + hh] = e;
 
                 const float4* rec = reinterpret_cast<const float4*>(s_exp + e * EXP_STRIDE);
                 float ho = s_b2[e];
@@ -189,15 +213,17 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restr
 
             // ---- mu EMA, Adam moments, decoupled weight decay
             mu = sg_fma(alpha, mu, (1.0f - alpha) * g);
-            sg::gptr(T.mu)[i] = mu;
+            if (live) sg::gptr(T.mu)[i] = mu;
             const float fg = sg_fma(lamb, mu, smart);
             ea = sg_fma(beta1, ea, (1.0f - beta1) * fg);
             easq = sg_fma(beta2, easq, ((1.0f - beta2) * fg) * fg);
-            sg::gptr(T.ea)[i] = ea;
-            sg::gptr(T.easq)[i] = easq;
+            if (live) {
+                sg::gptr(T.ea)[i] = ea;
+                sg::gptr(T.easq)[i] = easq;
+            }
             const float denom = __builtin_sqrtf(easq / bc2) + eps;
             pv = sg_fma(pv, decay, -((step_size * ea) / denom));
-            sg::store_elem(T.param, dtype, i, pv);
+            if (live) sg::store_elem(T.param, dtype, i, pv);
         }
     }
     __syncthreads();
