@@ -30,7 +30,8 @@ PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.420e9 + 1.619e9, "scan_summary": 0
 # Vector-ALU instructions per launch (SQ_INSTS_VALU of the same profile, default workload only) and the rate the part
 # sustains on nothing but independent fp32 instructions (bench.py --workload valu-probe, profiles/valu_probe_mi355x.txt):
 # what actually bounds these kernels
-PMC_VALU_INSTS_SCALE50 = {"scan_output": 3.864e9, "scan_summary": 2.09e8, "elementwise": 8.66e8}
+# (the per-element kernel's count holds 8.6e6 fp32 matrix instructions of 64 clocks each: 16 vector instructions' worth of time apiece)
+PMC_VALU_INSTS_SCALE50 = {"scan_output": 3.864e9, "scan_summary": 2.09e8, "elementwise": 6.19e8 + 15 * 8.6e6}
 VALU_SUSTAINED_PER_NS_SIMD = 0.59
 SIMDS = 1024
 
@@ -299,7 +300,8 @@ def bench_probe(dev):
     ws = torch.empty(L.sg_probe_workspace_bytes(cus, 8), dtype=torch.uint8, device=dev)
     rows, best = [], 0.0
     for ncu in (cus,):
-        for op, name in enumerate(("fma", "mul", "add", "add_dpp", "mfma_32x32x16_bf16", "mfma_32x32x16_bf16_random_operands")):
+        for op, name in enumerate(("fma", "mul", "add", "add_dpp", "mfma_32x32x16_bf16", "mfma_32x32x16_bf16_random_operands",
+                                   "mfma_32x32x1_f32", "mfma_32x32x1_f32_then_8_fma", "mfma_4x4x1_f32")):
             for w in ((1, 2) if op >= 4 else (1, 2, 3, 4, 8)):
                 ms, ticks, instr = C.c_float(), C.c_double(), C.c_double()
                 if L.sg_probe_valu(op, ncu, w, 2000, C.byref(ms), C.byref(ticks), C.byref(instr), ws.data_ptr(), ws.numel(),
@@ -310,8 +312,8 @@ def bench_probe(dev):
                              "instr_per_ns_per_simd": round(rate, 4),
                              "clock_ticks_per_instr_per_simd": round(ticks.value / instr.value / w, 3),
                              "clock_ticks_per_ns": round(ticks.value / (ms.value * 1e6), 3)})
-                if op >= 4:      # 32768 flop per instruction and SIMD
-                    rows[-1]["chip_tflops"] = round(rate * 32768 * 4 * ncu / 1e3, 1)
+                if op >= 4:      # flop per matrix instruction (the vector fma of the mixed stream are not counted)
+                    rows[-1]["chip_tflops"] = round(rate * (32768, 32768, 4096, 4096, 512)[op - 4] * 4 * ncu / 1e3, 1)
                 elif ncu == cus:
                     best = max(best, rate)
     return {"metric": "secondary: valu-probe", "value": best, "unit": "wave64 instructions/ns/SIMD (whole chip, best case)",

@@ -152,7 +152,11 @@ int sg2_profile_read(float* ms, int* calls);
  * per wave (op 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_add_f32 with a DPP
  * operand; plain, not packed; 4 v_mfma_f32_32x32x16_bf16 on constant register
  * operands, 5 the same on pseudo-random operands: the matrix cores' own
- * ceiling and what real data makes of it through the power limit) on num_cus x waves_per_simd workgroups of four
+ * ceiling and what real data makes of it through the power limit; 6
+ * v_mfma_f32_32x32x1_2b_f32, 7 the same with 8 v_fma_f32 after each in the
+ * same wave (the vector instructions are not counted), 8
+ * v_mfma_f32_4x4x1_16b_f32: the fp32 matrix forms that are one fused
+ * multiply-add per output) on num_cus x waves_per_simd workgroups of four
  * waves, i.e. waves_per_simd waves on every SIMD of num_cus compute units
  * when the dispatcher spreads them evenly.  Synchronises the stream.  Returns
  * the elapsed milliseconds of the launch, the shader-clock ticks a wave took

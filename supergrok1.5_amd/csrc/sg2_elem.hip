@@ -10,8 +10,9 @@
 // elements; the tile index is mapped to (tensor, offset) by a binary search
 // over a P+1 entry prefix table.  The 144 expert MLPs live in LDS (records of
 // 48 floats padded to 52 so that random per-lane experts spread over the
-// banks); GRU / query / key weights are wave-uniform and come in through
-// scalar loads (constant address space).  expert_counts is accumulated in an LDS histogram and flushed
+// banks); GRU and key weights are wave-uniform and come in through scalar
+// loads (constant address space); the query projection is a chain of fp32
+// matrix instructions.  expert_counts is accumulated in an LDS histogram and flushed
 // once per workgroup (the reference issues one global atomic per element and
 // head).
 #include "sg2_internal.hpp"

@@ -83,6 +83,50 @@ __global__ __launch_bounds__(256) void k_probe_mfma(float* sink, long long* tick
     if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
 }
 
+typedef __attribute__((ext_vector_type(32))) float probe_f32x32;
+typedef __attribute__((ext_vector_type(4))) float probe_f32x4;
+// fp32 matrix instructions with one fused multiply-add per output (k = 1), the forms whose chains equal fmaf chains
+// bit for bit.  KIND 0: v_mfma_f32_32x32x1_2b (2048 multiply-adds); 1: the same with 8 independent vector fma after
+// every matrix instruction, in the same wave (do the two pipes overlap?); 2: v_mfma_f32_4x4x1_16b (256 multiply-adds).
+template <int KIND>
+__global__ __launch_bounds__(256) void k_probe_mfma_f32(float* sink, long long* ticks, int iters, float a, float b) {
+    probe_f32x32 big[2];
+    probe_f32x4 small[PROBE_ILP];
+    float acc[PROBE_ILP];
+#pragma unroll
+    for (int k = 0; k < 2; k++)
+#pragma unroll
+        for (int e = 0; e < 32; e++) big[k][e] = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PROBE_ILP; k++) {
+        acc[k] = threadIdx.x * 1e-3f + k + 1.0f;
+        small[k] = probe_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const float av = a + 1e-3f * (threadIdx.x & 31), bv = b + 1e-3f * (threadIdx.x & 15);
+    const long long t0 = clock64();
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+        for (int r = 0; r < PROBE_UNROLL * PROBE_ILP; r++) {
+            if (KIND == 2) {
+                small[r % PROBE_ILP] = __builtin_amdgcn_mfma_f32_4x4x1f32(av, bv, small[r % PROBE_ILP], 0, 0, 0);
+            } else {
+                big[r & 1] = __builtin_amdgcn_mfma_f32_32x32x1f32(av, bv, big[r & 1], 0, 0, 0);
+                if (KIND == 1) {
+#pragma unroll
+                    for (int k = 0; k < PROBE_ILP; k++) acc[k] = __builtin_fmaf(acc[k], a, b);
+                }
+            }
+        }
+    }
+    const long long t1 = clock64();
+    float s = 0.0f;
+#pragma unroll
+    for (int k = 0; k < PROBE_ILP; k++) s += acc[k] + small[k][0] + small[k][3];
+    s += big[0][0] + big[0][31] + big[1][7];
+    if (s == 12345.678f) sink[0] = s;
+    if (threadIdx.x == 0) ticks[blockIdx.x] = t1 - t0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -95,7 +139,9 @@ size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd) {
 int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
                   double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream) {
     hipStream_t st = (hipStream_t)stream;
-    if (op < 0 || op > 5) return sg::fail("op must be 0 (fma), 1 (mul), 2 (add), 3 (add with a DPP operand), 4 (32x32x16 bf16 MFMA, constant operands) or 5 (the same, random operands)");
+    if (op < 0 || op > 8)
+        return sg::fail("op must be 0 (fma), 1 (mul), 2 (add), 3 (add with a DPP operand), 4 (32x32x16 bf16 MFMA, constant operands), 5 (the same, random "
+                        "operands), 6 (32x32x1 fp32 MFMA), 7 (the same with 8 vector fma after each) or 8 (4x4x1 fp32 MFMA)");
     if (num_cus <= 0 || num_cus > 1024 || waves_per_simd <= 0 || waves_per_simd > 8 || iters <= 0 || iters > 100000)
         return sg::fail("probe size out of range");
     if (!ms_out || !ticks_per_wave_out || !instr_per_wave_out) return sg::fail("NULL argument");
@@ -113,6 +159,9 @@ int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_
             case 2: hipLaunchKernelGGL(k_probe<2>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             case 4: hipLaunchKernelGGL(k_probe_mfma<false>, dim3(blocks), dim3(256), 0, st, sink, ticks, n); break;
             case 5: hipLaunchKernelGGL(k_probe_mfma<true>, dim3(blocks), dim3(256), 0, st, sink, ticks, n); break;
+            case 6: hipLaunchKernelGGL(k_probe_mfma_f32<0>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 7: hipLaunchKernelGGL(k_probe_mfma_f32<1>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 8: hipLaunchKernelGGL(k_probe_mfma_f32<2>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             default: hipLaunchKernelGGL(k_probe<3>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
         }
     };
