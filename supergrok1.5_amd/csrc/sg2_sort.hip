@@ -52,9 +52,14 @@ __device__ __forceinline__ TileRef tile_ref(const Plan& pl, int tile) {
 }
 
 
-// ---- key generation + digit counts of the first pass -------------------------------
-// One sort tile per workgroup.  All of a lane's loads are issued before the first store (the tile length is a
-// compile-time bound, the tail is predicated).
+// ---- digit counts of the first pass, straight from the gradients ----------------------
+// One sort tile per workgroup.  The keys themselves are never written in element order: the first scatter pass
+// forms them again from the gradients (key_of / payload_of) while it moves them.
+// key = |g| bits; the sign rides in bit 31 of the payload so that the sorted (key, payload) pair gives back g
+// exactly and the scan never has to gather gradients from element order
+__device__ __forceinline__ uint32_t key_of(float g) { return (uint32_t)sg_f2i(sg_abs(sg::finite_or_zero(g))); }
+__device__ __forceinline__ int32_t payload_of(float g, int index) { return index | (sg_f2i(sg::finite_or_zero(g)) & (int32_t)0x80000000); }
+
 __global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
     __shared__ uint32_t h[256];
     const int seg = sg::upper_seg(pl.sort_tile_prefix, pl.P, (int)blockIdx.x);
@@ -78,15 +83,7 @@ __global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
         const int k = r * SORT_THREADS + (int)threadIdx.x;
-        if (k < tr.cnt) {
-            const float gv = sg::finite_or_zero(g[r]);
-            // key = |g| bits; the sign rides in bit 31 of the payload so that the sorted (key, payload)
-            // pair gives back g exactly and the scan never has to gather gradients from element order
-            const uint32_t key = (uint32_t)sg_f2i(sg_abs(gv));
-            pl.keys[0][tr.base + k] = key;
-            pl.vals[0][tr.base + k] = (start + k) | (sg_f2i(gv) & (int32_t)0x80000000);
-            atomicAdd(&h[key & 255u], 1u);
-        }
+        if (k < tr.cnt) atomicAdd(&h[key_of(g[r]) & 255u], 1u);
     }
     // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
     // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
@@ -223,6 +220,9 @@ __global__ __launch_bounds__(1024) void k_spine_single(uint32_t* spine, int n /*
 }
 
 // ---- stable scatter ---------------------------------------------------------------
+// FIRST: the pass over digit 0 takes its keys and payloads from the tensor's gradients (element order) instead of
+// the key / payload arrays, which nothing has written yet.
+template <bool FIRST>
 __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int shift) {
     __shared__ uint32_t cnt[WAVES][256];     // running digit counts of each wave; later: destinations
     __shared__ uint32_t lbase[256], gdelta[256], wsum[4];
@@ -242,12 +242,30 @@ __global__ __launch_bounds__(SORT_THREADS) void k_scatter(Plan pl, int src, int 
 
     uint32_t key[ITEMS], rank[ITEMS];
     int32_t val[ITEMS];
+    if (FIRST) {
+        const TensorDev& T = pl.tensors[sg::upper_seg(pl.sort_tile_prefix, pl.P, (int)blockIdx.x)];
+        const int start = tr.base - T.off, dtype = T.dtype;
+        float g[ITEMS];
 #pragma unroll
-    for (int r = 0; r < ITEMS; r++) {
-        const int i = w * WAVE_ITEMS + r * 64 + lane;
-        const bool ok = FULL || i < tr.cnt;
-        key[r] = ok ? keys[i] : 0u;
-        val[r] = ok ? vals[i] : 0;
+        for (int r = 0; r < ITEMS; r++) {
+            const int i = w * WAVE_ITEMS + r * 64 + lane;
+            g[r] = (FULL || i < tr.cnt) ? sg::load_elem(T.grad, dtype, start + i) : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < ITEMS; r++) {
+            const int i = w * WAVE_ITEMS + r * 64 + lane;
+            const bool ok = FULL || i < tr.cnt;
+            key[r] = ok ? key_of(g[r]) : 0u;
+            val[r] = ok ? payload_of(g[r], start + i) : 0;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < ITEMS; r++) {
+            const int i = w * WAVE_ITEMS + r * 64 + lane;
+            const bool ok = FULL || i < tr.cnt;
+            key[r] = ok ? keys[i] : 0u;
+            val[r] = ok ? vals[i] : 0;
+        }
     }
 #pragma unroll
     for (int r = 0; r < ITEMS; r++) {
@@ -373,7 +391,8 @@ int launch_sort(const Plan& pl, int32_t* dbg_perm, hipStream_t st) {
             hipLaunchKernelGGL(k_spine_reduce, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
             hipLaunchKernelGGL(k_spine_down, dim3(nb), dim3(256), 0, st, pl.spine, pl.blocksums, n);
         }
-        hipLaunchKernelGGL(k_scatter, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
+        if (pass == 0) hipLaunchKernelGGL(k_scatter<true>, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
+        else hipLaunchKernelGGL(k_scatter<false>, dim3(pl.sort_tiles), dim3(SORT_THREADS), 0, st, pl, src, shift);
         SG_LAUNCH_CHECK("radix pass");
     }
     // result is back in keys[0] / vals[0]
