@@ -61,29 +61,52 @@ __device__ __forceinline__ uint32_t key_of(float g) { return (uint32_t)sg_f2i(sg
 __device__ __forceinline__ int32_t payload_of(float g, int index) { return index | (sg_f2i(sg::finite_or_zero(g)) & (int32_t)0x80000000); }
 
 __global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
-    __shared__ uint32_t h[256];
+    // lane-selected copies of the counters, as in k_hist: gradients that came from a 16-bit format have one value of digit 0
+    constexpr int HCOPY = 8, HSTRIDE = 256 + 8;
+    __shared__ uint32_t hc[HCOPY * HSTRIDE];
     const int seg = sg::upper_seg(pl.sort_tile_prefix, pl.P, (int)blockIdx.x);
     const TileRef tr = tile_ref(pl, blockIdx.x);
     const TensorDev& T = pl.tensors[seg];
     const int start = tr.base - T.off;
-    if (threadIdx.x < 256) h[threadIdx.x] = 0;
+    for (int k = threadIdx.x; k < HCOPY * HSTRIDE; k += SORT_THREADS) hc[k] = 0;
+    uint32_t* const h = hc + (threadIdx.x & (HCOPY - 1)) * HSTRIDE;
     __syncthreads();
-    float g[ITEMS];
     bool nz = false;
+    const float* gp = static_cast<const float*>(T.grad) + start;
+    const float* sp = static_cast<const float*>(T.sharp) + start;
+    if (T.dtype == SG_F32 && tr.cnt == SORT_TILE && ((((uintptr_t)gp) | ((uintptr_t)sp)) & 15u) == 0) {
+        // whole fp32 tile on a 16-byte boundary: 16 bytes per lane and load, everything requested before the first use
+        constexpr int VR = SORT_TILE / (4 * SORT_THREADS);
+        typedef float vf4 __attribute__((ext_vector_type(4)));
+        vf4 g[VR], sh[VR];
 #pragma unroll
-    for (int r = 0; r < ITEMS; r++) {
-        const int k = r * SORT_THREADS + (int)threadIdx.x;
-        g[r] = (k < tr.cnt) ? sg::load_elem(T.grad, T.dtype, start + k) : 0.0f;
-    }
+        for (int r = 0; r < VR; r++) g[r] = ((const SG_GLOBAL vf4*)gp)[r * SORT_THREADS + (int)threadIdx.x];
 #pragma unroll
-    for (int r = 0; r < ITEMS; r++) {
-        const int k = r * SORT_THREADS + (int)threadIdx.x;
-        if (k < tr.cnt) nz = nz || (sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, start + k)) != 0.0f);
-    }
+        for (int r = 0; r < VR; r++) sh[r] = ((const SG_GLOBAL vf4*)sp)[r * SORT_THREADS + (int)threadIdx.x];
 #pragma unroll
-    for (int r = 0; r < ITEMS; r++) {
-        const int k = r * SORT_THREADS + (int)threadIdx.x;
-        if (k < tr.cnt) atomicAdd(&h[key_of(g[r]) & 255u], 1u);
+        for (int r = 0; r < VR; r++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                atomicAdd(&h[key_of(g[r][e]) & 255u], 1u);
+                nz = nz || (sg::finite_or_zero(sh[r][e]) != 0.0f);
+            }
+    } else {
+        float g[ITEMS];
+#pragma unroll
+        for (int r = 0; r < ITEMS; r++) {
+            const int k = r * SORT_THREADS + (int)threadIdx.x;
+            g[r] = (k < tr.cnt) ? sg::load_elem(T.grad, T.dtype, start + k) : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < ITEMS; r++) {
+            const int k = r * SORT_THREADS + (int)threadIdx.x;
+            if (k < tr.cnt) nz = nz || (sg::finite_or_zero(sg::load_elem(T.sharp, T.dtype, start + k)) != 0.0f);
+        }
+#pragma unroll
+        for (int r = 0; r < ITEMS; r++) {
+            const int k = r * SORT_THREADS + (int)threadIdx.x;
+            if (k < tr.cnt) atomicAdd(&h[key_of(g[r]) & 255u], 1u);
+        }
     }
     // Without SAM the sharpness of every element is 0 (the optimizer's initial state): remember per tensor
     // whether anything else was seen, so that the gather into sorted order can be skipped for such tensors.
@@ -92,7 +115,12 @@ __global__ __launch_bounds__(SORT_THREADS) void k_keys(Plan pl) {
         volatile int* flag = pl.sharp_nonzero + seg;
         if (*flag == 0) *flag = 1;
     }
-    if (threadIdx.x < 256) pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = h[threadIdx.x];
+    if (threadIdx.x < 256) {
+        uint32_t tot = 0;
+#pragma unroll
+        for (int c = 0; c < HCOPY; c++) tot += hc[c * HSTRIDE + threadIdx.x];
+        pl.spine[tr.spine0 + (int)threadIdx.x * tr.stride] = tot;
+    }
 }
 
 // ---- per-tile histogram ---------------------------------------------------------
