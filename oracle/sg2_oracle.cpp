@@ -59,6 +59,9 @@
  * M_late b_early + b_late), and the test is repeated, until it passes or the
  * chunk start is reached (then the summary is the exact one, re-associated by
  * blocks).  window <= 0 accumulates the whole chunk in one block.
+ * A (j,p) whose M is exactly zero hands on b itself as the next start state
+ * (not 0 * h + b, which differs for a non-finite h): the kernels read no
+ * earlier state at all when every summary of a call is of that kind.
  *
  * Parity status: the reference's tests hold no golden vectors for this path
  * (tests/test_supergrok2.py checks finiteness and run-to-run determinism
@@ -461,8 +464,10 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
             for (int p = 0; p < hp; p++) {
                 const R* m = &sm[(j * hp + p) * 6];
                 const R he = h0[j * ds + 2 * p], ho = h0[j * ds + 2 * p + 1];
-                h1[j * ds + 2 * p] = O::fma(m[0], he, O::fma(m[2], ho, m[4]));
-                h1[j * ds + 2 * p + 1] = O::fma(m[1], he, O::fma(m[3], ho, m[5]));
+                /* an exactly zero 2x2 part hands on the offset itself (the kernels then never read the earlier state) */
+                const bool zero = m[0] == 0 && m[1] == 0 && m[2] == 0 && m[3] == 0;
+                h1[j * ds + 2 * p] = zero ? m[4] : O::fma(m[0], he, O::fma(m[2], ho, m[4]));
+                h1[j * ds + 2 * p + 1] = zero ? m[5] : O::fma(m[1], he, O::fma(m[3], ho, m[5]));
             }
     }
 

@@ -119,6 +119,7 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[0] = out[0];
     dst[1] = out[1];
     dst[2] = out[2];
+    if (threadIdx.x == 0) *pl.contracted = 1;      // until a summary kernel finds a chunk that has not contracted
 }
 
 // Projections of one timestep from the element's (g, s).  Each wave of the workgroup produces its
@@ -299,10 +300,19 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     }
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
+    bool fully_contracted = false;      // summary pass: the walk stopped because the 2x2 part had contracted
     if (OUT) {
-        const float* hs = pl.hstart + ((size_t)(dir * pl.chunks + cidx) * 2) * SCAN_THREADS;
-        S.he = hs[tid];
-        S.ho = hs[SCAN_THREADS + tid];
+        // When every summary of this call has an exactly zero 2x2 part, a chunk's start state is the offset of the
+        // summary before it, whatever came earlier: k_chunk_prefix has then only placed the carried states (chunk 0).
+        if (c > 0 && __builtin_amdgcn_readfirstlane(*pl.contracted) != 0) {
+            const float* sm = pl.summaries + (size_t)(dir * pl.wchunks + pl.wchunk_prefix[ti] + c - 1) * 6 * SCAN_THREADS;
+            S.he = sm[4 * SCAN_THREADS + tid];
+            S.ho = sm[5 * SCAN_THREADS + tid];
+        } else {
+            const float* hs = pl.hstart + ((size_t)(dir * pl.chunks + cidx) * 2) * SCAN_THREADS;
+            S.he = hs[tid];
+            S.ho = hs[SCAN_THREADS + tid];
+        }
     }
 
     // Summary pass: the chunk is walked backwards in blocks of `window` steps.  Each block is summarised from the
@@ -491,6 +501,7 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float mx = sg_max(sg_max(sg_abs(S.c0e), sg_abs(S.c0o)), sg_max(sg_abs(S.c1e), sg_abs(S.c1o)));
         if (!__syncthreads_or(!(mx < 7.888609052210118e-31f))) {
             S.c0e = S.c0o = S.c1e = S.c1o = 0.0f;
+            fully_contracted = true;
             break;
         }
     }
@@ -515,6 +526,7 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         sm[3 * SCAN_THREADS + tid] = S.c1o;
         sm[4 * SCAN_THREADS + tid] = S.he;
         sm[5 * SCAN_THREADS + tid] = S.ho;
+        if (!fully_contracted && tid == 0) *pl.contracted = 0;      // plain store: every writer stores the same value
     }
 }
 
@@ -549,6 +561,8 @@ __global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
         hs[lane] = he;
         hs[SCAN_THREADS + lane] = ho;
     }
+    // every summary has an exactly zero 2x2 part: the replay takes its start states from the summaries themselves
+    if (__builtin_amdgcn_readfirstlane(*pl.contracted) != 0) return;
     float r[PREFIX_PER_GROUP][6];
     auto prefetch = [&](int b) {
 #pragma unroll
@@ -570,10 +584,12 @@ __global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
             const int lim = min(PREFIX_BATCH, ns - b * PREFIX_BATCH);
             for (int cc = 0; cc < lim; cc++) {
                 const float* m = lds + cc * 6 * SCAN_THREADS + lane;
+                // a lane whose 2x2 part is exactly zero takes the offset itself (not 0 * h + b: the state may not be finite)
+                const bool zero = m[0] == 0.0f && m[SCAN_THREADS] == 0.0f && m[2 * SCAN_THREADS] == 0.0f && m[3 * SCAN_THREADS] == 0.0f;
                 const float ne = sg_fma(m[0], he, sg_fma(m[2 * SCAN_THREADS], ho, m[4 * SCAN_THREADS]));
                 const float no = sg_fma(m[SCAN_THREADS], he, sg_fma(m[3 * SCAN_THREADS], ho, m[5 * SCAN_THREADS]));
-                he = ne;
-                ho = no;
+                he = zero ? m[4 * SCAN_THREADS] : ne;
+                ho = zero ? m[5 * SCAN_THREADS] : no;
                 float* h1 = hs + (size_t)(b * PREFIX_BATCH + cc + 1) * 2 * SCAN_THREADS;
                 h1[lane] = he;
                 h1[SCAN_THREADS + lane] = ho;

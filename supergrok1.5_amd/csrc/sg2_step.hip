@@ -96,7 +96,7 @@ int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bi
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * gi.threads);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
     L->off_comp = take(4 * 2 * 5 * (size_t)gi.rows * 3);
-    L->off_flags = take(4 * (size_t)P);        // apart from the tensor records: it is written while those are being read
+    L->off_flags = take(4 * ((size_t)P + 1));        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions
     L->off_htile = take(bilevel ? 4 * 2 * (size_t)htile_count((int)total, P) * 2 * SCAN_THREADS : 0);
@@ -330,6 +330,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.hstart = reinterpret_cast<float*>(ws + L.off_hstart);
     pl.comp = reinterpret_cast<float*>(ws + L.off_comp);
     pl.sharp_nonzero = reinterpret_cast<int*>(ws + L.off_flags);
+    pl.contracted = pl.sharp_nonzero + P;
     pl.ctx = reinterpret_cast<float*>(ws + L.off_ctx);
     pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
