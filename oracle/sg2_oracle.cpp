@@ -500,9 +500,13 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
                         hc[j * ds + 2 * p + 1] = no;
                         yp[p] = O::fma(no, sp.C[2 * p + 1], ne * sp.C[2 * p]);
                     }
-                    /* balanced pairwise sum over the RoPE pairs (stride 1, 2, 4, ...) */
-                    for (int st = 1; st < hp; st *= 2)
-                        for (int p = 0; p + st < hp; p += 2 * st) yp[p] = yp[p] + yp[p + st];
+                    /* sum over the RoPE pairs in the kernels' order: the group is folded in halves, mirrored
+                     * (y_i + y_(n-1-i)), until four sums are left; those as (s0 + s1) + (s2 + s3) */
+                    int n = hp;
+                    for (; n > 4; n /= 2)
+                        for (int p = 0; p < n / 2; p++) yp[p] = yp[p] + yp[n - 1 - p];
+                    for (int st = 1; st < n; st *= 2)
+                        for (int p = 0; p + st < n; p += 2 * st) yp[p] = yp[p] + yp[p + st];
                     out[j] = O::fma(yp[0], gate[j], (R)w.D[j] * xb);
                 }
                 for (int dd = 0; dd < dm; dd++) {

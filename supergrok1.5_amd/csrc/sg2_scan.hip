@@ -88,14 +88,80 @@ __device__ __forceinline__ float dpp_half_mirror(float v) {  // lane -> 7 - lane
 __device__ __forceinline__ float dpp_row_mirror(float v) {   // lane -> 15 - lane within each group of 16
     return sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(v), 0x140, 0xF, 0xF, true));
 }
-// sum over the HP lanes of a (column) group, as the balanced tree ((0+1)+(2+3)) + ((4+5)+(6+7)) [+ the same over 8..15]
+// sum over the HP lanes of a (column) group.  The tree folds the group in halves, mirrored, until four sums are left:
+// HP = 8: s_i = y_i + y_(7-i), total = (s_0 + s_1) + (s_2 + s_3); HP = 16: r_i = y_i + y_(15-i) first, then the same on r.
+// (Mirrored folds first, because a fold across DPP banks can be written to some banks only: see block_pair_sums.)
 template <int HP>
 __device__ __forceinline__ float pair_tree_sum(float y) {
+    if (HP == 16) y = y + dpp_row_mirror(y);
+    y = y + dpp_half_mirror(y);
     y = y + dpp_quad_swap1(y);
     y = y + dpp_quad_swap2(y);
-    y = y + dpp_half_mirror(y);
-    if (HP == 16) y = y + dpp_row_mirror(y);
     return y;
+}
+// The same sums for the 8 steps of a block in 16 instructions instead of 24 (32 for HP = 16).  A DPP instruction can
+// be restricted to some banks (groups of four lanes) of every row of 16, leaving the destination's other lanes as
+// they were.  After a mirrored fold both halves of the folded group hold the same sums, so two steps' folds are
+// written into ONE register - step u into the first half's lanes, step u + 4 into the second half's - and the rest
+// of the tree runs on half as many registers.  Additions commute bit for bit, so every lane that ends up holding a
+// step's total holds pair_tree_sum's value.  On return, for HP = 8, y[k] (k < 4) is the total of step k + 4 (p >> 2)
+// in lane (j, p); for HP = 16, y[m] (m < 2) that of step m + 2 (p >> 2).
+// (Inline assembly: the compiler has no form for a bank-masked DPP addition that keeps the other lanes, and it does
+// not see a hazard between instructions inside the block - a DPP operand must not be read within two instructions of the
+// vector instruction that wrote it, hence the order of the instructions and the s_nop.)
+template <int HP>
+__device__ __forceinline__ void block_pair_sums(float (&y)[8]) {
+    float z0, z1, z2, z3;
+    if (HP == 8) {
+        asm volatile(
+            "s_nop 1\n\t"
+            "v_add_f32_dpp %0, %4, %4 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %0, %8, %8 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %1, %5, %5 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %1, %9, %9 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %2, %6, %6 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %2, %10, %10 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %3, %7, %7 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %3, %11, %11 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %2, %2, %2 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %3, %3, %3 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %2, %2, %2 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %3, %3, %3 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 1"
+            : "=&v"(z0), "=&v"(z1), "=&v"(z2), "=&v"(z3)
+            : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]));
+        y[0] = z0; y[1] = z1; y[2] = z2; y[3] = z3;
+    } else {
+        asm volatile(
+            "s_nop 1\n\t"
+            "v_add_f32_dpp %0, %4, %4 row_mirror row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %0, %8, %8 row_mirror row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %1, %5, %5 row_mirror row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %1, %9, %9 row_mirror row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %2, %6, %6 row_mirror row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %2, %10, %10 row_mirror row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %3, %7, %7 row_mirror row_mask:0xf bank_mask:0x3\n\t"
+            "v_add_f32_dpp %3, %11, %11 row_mirror row_mask:0xf bank_mask:0xc\n\t"
+            "v_add_f32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "v_add_f32_dpp %1, %1, %1 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+            "s_nop 0\n\t"
+            "v_add_f32_dpp %0, %2, %2 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "v_add_f32_dpp %1, %3, %3 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+            "s_nop 1\n\t"
+            "v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 1\n\t"
+            "v_add_f32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "v_add_f32_dpp %1, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "s_nop 1"
+            : "=&v"(z0), "=&v"(z1), "=&v"(z2), "=&v"(z3)
+            : "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]), "v"(y[4]), "v"(y[5]), "v"(y[6]), "v"(y[7]));
+        y[0] = z0; y[1] = z1;
+    }
 }
 template <int HP>
 __device__ __forceinline__ float pair_tree_max(float f) {
@@ -240,8 +306,8 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
         if (OUT) y[u] = sg_fma(S.ho, Co[u], S.he * Ce[u]);
     }
     if (OUT) {
-#pragma unroll
-        for (int u = 0; u < UB; u++) y[u] = pair_tree_sum<HP>(y[u]);
+        static_assert(UB == 8, "block_pair_sums folds blocks of 8 steps");
+        block_pair_sums<HP>(y);
     }
 }
 
@@ -424,10 +490,11 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                 block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
             else
                 block_steps<HP, OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
-            if (OUT && p == 0) {
-#pragma unroll
-                for (int q = 0; q < UB; q += 4)
-                    *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + q]) = f32x4{y[q], y[q + 1], y[q + 2], y[q + 3]};
+            if (OUT && (p & 3) == 0) {       // the first lane of every bank holds the totals of its bank's steps (block_pair_sums)
+                if constexpr (HP == 8)
+                    *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + 4 * (p >> 2)]) = f32x4{y[0], y[1], y[2], y[3]};
+                else
+                    *reinterpret_cast<float2*>(&s_y[j * LDS_STRIDE + k0 + 2 * (p >> 2)]) = make_float2(y[0], y[1]);
             }
         }
         if (KEEP && k0 == HT_STEP && cnt > HT_STEP) keep_state(tile0 + HT_STEP);      // the ragged end starts right there
