@@ -110,6 +110,38 @@ def test_adaptive_window_needs_several_blocks():
     print("several blocks", _run_steps(case, 2, chunk_len=512, sharp=True, lamb_eff=2.0))
 
 
+def test_contracted_summaries_forget_the_carried_state():
+    """With every chunk summary contracted to (0, b) the replay takes the start state of chunk c from summary c - 1 and
+    never reads what came before: the contexts of all later chunks and the new carried state are the same, bit for
+    bit, whether the tensor carried in a small state or an infinite one.  (The first chunk does see it.)"""
+    from grokking_optimizers import _cabi
+    shapes, cl = [(3000,), (700,), (256,)], 256
+    assert _cabi.lib().sg2_set_chunk_len(cl) == 0
+    ctx, fwd, perm = [], [], None
+    for poison in (False, True):
+        case = Sg2Case(shapes, seed=5, random_state=True)
+        if poison:
+            case.gpu[0]["mamba_fwd"].fill_(float("inf"))
+            case.gpu[1]["mamba_bwd"].fill_(-3.0e30)
+        grads = wl.make_grads(shapes, seed=77)
+        sharps = [torch.zeros_like(g) for g in grads]
+        print("carried state", "infinite" if poison else "small", flush=True)
+        case.gpu_step(grads, sharps, per_tensor_scalars(case.P, 1, 2.0), shared_scalars(4.5))
+        ctx.append(case.step_fn.ctx.cpu().numpy().copy())
+        fwd.append([case.gpu[i][k].cpu().numpy().copy() for i in range(case.P) for k in ("mamba_fwd", "mamba_bwd")])
+        perm = case.step_fn.perm.cpu().numpy()
+    n0, o1, n1 = 3000, 3000, 700
+    later0 = perm[:n0][cl:]                       # tensor 0, forward direction: scan steps >= one chunk
+    assert np.isfinite(ctx[1][0, later0]).all() and np.array_equal(ctx[0][0, later0], ctx[1][0, later0])
+    assert not np.isfinite(ctx[1][0, perm[:n0][:cl]]).all()
+    later1 = o1 + perm[o1:o1 + n1][:n1 - cl]      # tensor 1, backward direction
+    assert np.array_equal(ctx[0][1, later1], ctx[1][1, later1])
+    first1 = o1 + perm[o1:o1 + n1][n1 - cl:]
+    assert not np.array_equal(ctx[0][1, first1], ctx[1][1, first1])
+    for a, b in zip(fwd[0], fwd[1]):              # every new carried state comes from a last chunk (tensor 2 has one chunk
+        assert np.isfinite(b).all() and np.array_equal(a, b)      # only, and was not poisoned)
+
+
 def test_saturated_gates_take_the_plain_forms():
     """The scan's output gates, the GRU gates and the GRU candidates are formed with one shared reciprocal per group
     unless the product of the group's denominators is too large; then every value of the group takes the plain

@@ -158,6 +158,35 @@ def test_windowed_summaries_match_full_chunks():
     assert np.array_equal(dplain["ctx"], dwin["ctx"]) and np.array_equal(plain["mamba_fwd"], win["mamba_fwd"])
 
 
+def test_contracted_summary_forgets_what_came_before():
+    """A chunk summary whose 2x2 part has contracted to exactly zero hands on its offset b itself: every chunk after
+    the first is then independent of the state the tensor carried in -- bit for bit, and even for a carried state that
+    is not finite (0 * inf would poison the whole sequence; the kernels never read the earlier state in this case)."""
+    n, chunk = 1500, 256
+    W = weights_np()
+    g, s = _grad(n, 21), np.abs(_grad(n, 22))
+    sc = default_scalars()
+    st_a = random_state_np(n, 23)
+    st_b = copy_state(st_a)
+    st_b["mamba_fwd"][:] = np.inf
+    st_b["mamba_bwd"][:] = -3.0e30
+    a, da = _run_oracle(W, st_a, g, s, sc, 32, chunk, window=64)
+    b, db = _run_oracle(W, st_b, g, s, sc, 32, chunk, window=64)
+    perm = da["perm"]
+    assert np.array_equal(perm, db["perm"])
+    later_fwd, later_bwd = perm[chunk:], perm[:n - chunk]          # scan steps >= chunk of either direction
+    assert np.isfinite(db["ctx"][0][later_fwd]).all() and np.isfinite(db["ctx"][1][later_bwd]).all()
+    assert np.array_equal(da["ctx"][0][later_fwd], db["ctx"][0][later_fwd])
+    assert np.array_equal(da["ctx"][1][later_bwd], db["ctx"][1][later_bwd])
+    assert not np.isfinite(db["ctx"][0][perm[:chunk]]).all()       # the first chunk does see the carried state
+    assert not np.array_equal(da["ctx"][1][perm[n - chunk:]], db["ctx"][1][perm[n - chunk:]])
+    for k in ("mamba_fwd", "mamba_bwd"):                            # the new carried state comes from the last chunk
+        assert np.array_equal(a[k], b[k]) and np.isfinite(b[k]).all()
+    # without the window the exact summaries are applied (their 2x2 part is small, not zero): the carried state counts
+    c, dc = _run_oracle(W, st_b, g, s, sc, 32, chunk, window=0)
+    assert not np.isfinite(dc["ctx"][0][later_fwd]).all()
+
+
 # ------------------------------------------------- structural identities of the scan
 def test_reverse_scan_is_forward_scan_of_flipped_sequence():
     """With identical weights for both directions, the backward context of the
