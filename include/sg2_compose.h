@@ -59,6 +59,25 @@ SG_HD void sg2_compose_one(int group, int row, int d_model, int d_inner, const f
     }
 }
 
+/* Number of timesteps after which the 2x2 part of one RoPE pair's recurrence has shrunk below 2^-100 if every step
+ * had the step size dt0: rotations preserve length, so the part's norm shrinks by at most max(|A_bar_e|, |A_bar_o|)
+ * per step.  nhA = -A/2 of the pair's two poles (as sg_abar_pair takes them).  0 = not within a million steps.
+ * Kernel and checker size the first block of a chunk summary with it (sg2_first_block_steps). */
+SG_HD int sg2_contraction_steps(float dt0, float nhA_e, float nhA_o) {
+    float ae, ao;
+    sg_abar_pair(dt0, nhA_e, nhA_o, &ae, &ao);
+    const float m = sg_max(sg_abs(ae), sg_abs(ao));
+    if (!(m < 0.9999f)) return 0;
+    if (m < 1e-30f) return 1;
+    return (int)(69.3147202f / -sg_log(m)) + 1;       /* 100 ln 2 / -ln m */
+}
+/* The largest of those counts over all pairs of both directions (0 if one of them is 0), with an eighth and eight
+ * steps of margin, rounded up to whole blocks of eight steps. */
+SG_HD int sg2_first_block_steps(int largest, int any_zero) {
+    if (any_zero || largest <= 0) return 0;
+    return (largest + largest / 8 + 8 + 7) & ~7;
+}
+
 /* value of a composed output for one element */
 SG_HD float sg2_comp_eval(const float* c, float g, float s) { return sg_fma(c[0], g, sg_fma(c[1], s, c[2])); }
 

@@ -59,6 +59,11 @@
  * M_late b_early + b_late), and the test is repeated, until it passes or the
  * chunk start is reached (then the summary is the exact one, re-associated by
  * blocks).  window <= 0 accumulates the whole chunk in one block.
+ * Before that walk a windowed summary makes one cheaper attempt: a single block whose length comes from the weights
+ * alone (the steps the slowest RoPE pair needs to contract below 2^-100 at the step size of a zero input, plus a
+ * margin: sg2_first_block_steps in include/sg2_compose.h), walked with the state part only, while the 2x2 part is
+ * bounded by the running product of max(|A_bar_e|, |A_bar_o|) (rotations preserve length).  If the bound is below
+ * 2^-100 in every (j,p) the summary is (0, b) with that block's b; otherwise the walk above starts from scratch.
  * A (j,p) whose M is exactly zero hands on b itself as the next start state
  * (not 0 * h + b, which differs for a non-finite h): the kernels read no
  * earlier state at all when every summary of a call is of that kind.
@@ -378,7 +383,7 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
  * updated in place.  ctx: [N][d_model], written at sorted position t. */
 template <class O>
 void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const float* gs, int64_t N, bool reverse,
-              int64_t chunk_len, int64_t window, typename O::R* h, typename O::R* ctx) {
+              int64_t chunk_len, int64_t window, int64_t first_block, typename O::R* h, typename O::R* ctx) {
     typedef typename O::R R;
     const int dm = d.d_model, di = d.d_inner, ds = d.d_state, hp = ds / 2;
     if (N <= 0) return;
@@ -401,7 +406,45 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
         const int64_t u0 = c * chunk_len, u1 = (c + 1) * chunk_len;
         int64_t blk_end = u1, blk_first = (window > 0 && window < chunk_len) ? std::max(u0, u1 - window) : u0;
         bool have_late = false;
-        for (;;) {
+        /* first attempt (windowed summaries only): ONE block of first_block steps -- what the slowest pair needs to
+         * contract at the step size of a zero input, sg2_first_block_steps -- walked with the state part alone and,
+         * in place of the 2x2 part, the running product of max(|A_bar_e|, |A_bar_o|), which bounds its norm.  Below
+         * 2^-100 in every (j,p): the summary is (0, b).  Otherwise the general walk below starts from scratch. */
+        bool lite_done = false;
+        if (blk_first > u0 && first_block > 0 && u1 - first_block > u0) {
+            std::vector<R> bound(di * hp, (R)1);
+            for (int i = 0; i < di * hp; i++) {
+                R* m = &sm[i * 6];
+                m[0] = 0; m[1] = 0; m[2] = 0; m[3] = 0; m[4] = 0; m[5] = 0;
+            }
+            for (int64_t tile0 = u1 - first_block; tile0 < u1; tile0 += ORC_TILE) {
+                const int cnt = (int)std::min<int64_t>(ORC_TILE, u1 - tile0);
+                tile_coefficients<O>(d, w, A, x, gs, N, reverse, tile0, cnt, false, tc);
+                for (int k = 0; k < cnt; k++) {
+                    const StepProj<O>& sp = tc.sp[k];
+                    for (int j = 0; j < di; j++) {
+                        const R dt = sp.dt[j], xb = sp.xb[j];
+                        for (int p = 0; p < hp; p++) {
+                            const size_t li = (size_t)k * di * hp + j * hp + p;
+                            const R ae = tc.ae[li], ao = tc.ao[li], sn = tc.sn[li], cs = tc.cs[li];
+                            const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
+                            R* m = &sm[(j * hp + p) * 6];
+                            const R abs_e = ae < 0 ? -ae : ae, abs_o = ao < 0 ? -ao : ao;
+                            bound[j * hp + p] = bound[j * hp + p] * (abs_e > abs_o ? abs_e : abs_o);
+                            const R ve = m[4], vo = m[5];
+                            const R re = O::fma(ve, cs, -(vo * sn));
+                            const R ro = O::fma(vo, cs, ve * sn);
+                            m[4] = O::fma(ae, re, be);
+                            m[5] = O::fma(ao, ro, bo);
+                        }
+                    }
+                }
+            }
+            lite_done = true;
+            for (int i = 0; i < di * hp; i++)
+                if (!(bound[i] < (R)7.888609052210118e-31)) { lite_done = false; break; }
+        }
+        for (; !lite_done;) {
             for (int i = 0; i < di * hp; i++) {
                 R* m = &sm[i * 6];
                 m[0] = 1; m[1] = 0; m[2] = 0; m[3] = 1; m[4] = 0; m[5] = 0;   /* col0=(m0,m1) col1=(m2,m3) b=(m4,m5) */
@@ -554,6 +597,27 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
             x[t * dm + k] = O::fma((R)W[W_IN_W][2 * k + 1], sv, (R)W[W_IN_W][2 * k] * gv) + (R)W[W_IN_B][k];
     }
 
+    /* length of a summary's first block, from the weights alone (the kernels' k_compose does the same) */
+    int64_t first_block = 0;
+    {
+        int largest = 0, any_zero = 0;
+        for (int dir = 0; dir < 2; dir++) {
+            const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+            for (int j = 0; j < di; j++) {
+                float c[3];
+                sg2_compose_one(SG2_COMP_DT, j, dm, di, W[W_IN_W], W[W_IN_B], W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], c);
+                const float dt0 = sg_softplus(c[2]);
+                const float* alog = W[b + 5] + (size_t)j * ds;
+                for (int p = 0; p < ds / 2; p++) {
+                    const int n = sg2_contraction_steps(dt0, -0.5f * -sg_exp(alog[2 * p]), -0.5f * -sg_exp(alog[2 * p + 1]));
+                    if (n == 0) any_zero = 1;
+                    if (n > largest) largest = n;
+                }
+            }
+        }
+        first_block = sg2_first_block_steps(largest, any_zero);
+    }
+
     std::vector<R> ctx_sorted[2];
     std::vector<R> hst[2];
     for (int dir = 0; dir < 2; dir++) {
@@ -570,7 +634,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
         float* st = dir ? mbwd_io : mfwd_io;
         hst[dir].assign(st, st + di * ds);
         ctx_sorted[dir].resize((size_t)N * dm);
-        scan_dir<O>(d, w, x.data(), gs_sorted.data(), N, dir == 1, chunk_len, window, hst[dir].data(), ctx_sorted[dir].data());
+        scan_dir<O>(d, w, x.data(), gs_sorted.data(), N, dir == 1, chunk_len, window, first_block, hst[dir].data(), ctx_sorted[dir].data());
         for (int i = 0; i < di * ds; i++) st[i] = (float)hst[dir][i];
     }
     /* unsort: element perm[t] takes the context computed at sorted position t */

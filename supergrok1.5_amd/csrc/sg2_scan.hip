@@ -185,7 +185,25 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[0] = out[0];
     dst[1] = out[1];
     dst[2] = out[2];
-    if (threadIdx.x == 0) *pl.contracted = 1;      // until a summary kernel finds a chunk that has not contracted
+    // How many steps the first block of a chunk summary should cover: what the slowest pair of either direction needs
+    // to contract below 2^-100 at the step size a zero input gives (sg2_contraction_steps), plus a margin.
+    __shared__ int s_largest, s_zero;
+    if (threadIdx.x == 0) { s_largest = 0; s_zero = 0; }
+    __syncthreads();
+    if (group == SG2_COMP_DT) {
+        const float dt0 = sg_softplus(out[2]);
+        const float* alog = pl.W.w[dir ? W_B_ALOG : W_F_ALOG] + row * G::DS;
+        for (int p = 0; p < G::HP; p++) {
+            const int n = sg2_contraction_steps(dt0, -0.5f * -sg_exp(alog[2 * p]), -0.5f * -sg_exp(alog[2 * p + 1]));
+            if (n == 0) atomicOr(&s_zero, 1);
+            atomicMax(&s_largest, n);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        pl.contracted[0] = 1;      // until a summary kernel finds a chunk that has not contracted
+        pl.contracted[1] = sg2_first_block_steps(s_largest, s_zero);
+    }
 }
 
 // Projections of one timestep from the element's (g, s).  Each wave of the workgroup produces its
@@ -256,9 +274,12 @@ struct LaneState {
     float he, ho, c0e, c0o, c1e, c1o;
 };
 
-template <bool OUT>
+// LITE (summary pass only): the state part alone, and in c0e the running product of max(|A_bar_e|, |A_bar_o|), a bound
+// on the norm of the 2x2 part that is not formed
+template <bool OUT, bool LITE = false>
 __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, float sn, float cs, float be, float bo) {
-    if (!OUT) {
+    if (!OUT && LITE) S.c0e = S.c0e * sg_max(sg_abs(ae), sg_abs(ao));
+    if (!OUT && !LITE) {
         float re = sg_fma(S.c0e, cs, -(S.c0o * sn)), ro = sg_fma(S.c0o, cs, S.c0e * sn);
         S.c0e = ae * re;
         S.c0o = ao * ro;
@@ -277,7 +298,7 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
 // ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values; tcoef = the lane's sg_sincos_tiny_coef).
-template <int HP, bool OUT, int ANGLE>
+template <int HP, bool OUT, int ANGLE, bool LITE = false>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, const float (&tcoef)[6], float (&y)[UB]) {
@@ -302,7 +323,7 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
-        step_update<OUT>(S, ae[u], ao[u], sn[u], cs[u], be[u], bo[u]);
+        step_update<OUT, LITE>(S, ae[u], ao[u], sn[u], cs[u], be[u], bo[u]);
         if (OUT) y[u] = sg_fma(S.ho, Co[u], S.he * Ce[u]);
     }
     if (OUT) {
@@ -387,6 +408,17 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     int blk_end = u1;
     int blk_first = u0;
     if (!OUT && pl.window > 0 && pl.window < pl.chunk_len) blk_first = max(u0, u1 - pl.window);
+    // First attempt: ONE block of as many steps as k_compose expects the slowest pair to need, walked with the state
+    // part only (LITE) and a bound on the 2x2 part in its place.  If the bound is below 2^-100 in every lane the summary
+    // is (0, b) as below; if not, the walk starts over in its general form.
+    bool lite = false;
+    if (!OUT && blk_first > u0) {
+        const int first_block = __builtin_amdgcn_readfirstlane(pl.contracted[1]);
+        if (first_block > 0 && u1 - first_block > u0) {
+            lite = true;
+            blk_first = u1 - first_block;
+        }
+    }
     LaneState late = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     bool have_late = false;
     // inputs of one tile (sorted |g| bits, payload, sorted sharpness) for this lane's timestep; zero beyond the block
@@ -484,7 +516,14 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                 }
             }
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
-            if ((nottiny & blk) == 0)
+            if (!OUT && lite) {
+                if ((nottiny & blk) == 0)
+                    block_steps<HP, OUT, 2, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+                else if ((large & blk) == 0)
+                    block_steps<HP, OUT, 1, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+                else
+                    block_steps<HP, OUT, 0, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+            } else if ((nottiny & blk) == 0)
                 block_steps<HP, OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
             else if ((large & blk) == 0)
                 block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
@@ -503,7 +542,8 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             float ae, ao, sn, cs;
             sg_abar_pair(dt, hAe, hAo, &ae, &ao);
             sg_sincos(dt * freq, &sn, &cs);
-            step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
+            if (!OUT && lite) step_update<OUT, true>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
+            else step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             if (OUT) {
                 const float y = pair_tree_sum<HP>(sg_fma(S.ho, r_Co[k0], S.he * r_Ce[k0]));
                 if (p == 0) s_y[j * LDS_STRIDE + k0] = y;
@@ -554,6 +594,17 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         }
     }
     if (OUT) break;
+    if (lite) {          // c0e holds the bound (a NaN counts as "not contracted")
+        if (!__syncthreads_or(!(S.c0e < 7.888609052210118e-31f))) {
+            S.c0e = S.c0o = S.c1e = S.c1o = 0.0f;
+            fully_contracted = true;
+            break;
+        }
+        lite = false;    // the general walk, from the end of the chunk
+        blk_first = max(u0, u1 - pl.window);
+        S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
+        continue;
+    }
     if (have_late) {     // S covers [blk_first, blk_end), late covers [blk_end, u1): the summary of both is late o S
         const LaneState E = S;
         S.c0e = sg_fma(late.c0e, E.c0e, late.c1e * E.c0o);

@@ -96,7 +96,7 @@ int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bi
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * gi.threads);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
     L->off_comp = take(4 * 2 * 5 * (size_t)gi.rows * 3);
-    L->off_flags = take(4 * ((size_t)P + 1));        // apart from the tensor records: it is written while those are being read
+    L->off_flags = take(4 * ((size_t)P + 2));        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions
     L->off_htile = take(bilevel ? 4 * 2 * (size_t)htile_count((int)total, P) * 2 * SCAN_THREADS : 0);
