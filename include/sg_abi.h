@@ -98,7 +98,10 @@ int sg2_chunk_len_for(int num_tensors, const int64_t* numels);
  * chunk summary is built backwards in blocks of `window` steps and the walk
  * stops as soon as every entry of the 2x2 part of the running summary is below
  * 2^-100 (the chunk summary is then (0, b)); a chunk that never contracts is
- * covered completely.  Takes effect when window < chunk_len. */
+ * covered completely.  Before that walk one block whose length follows from
+ * the weights (the steps the slowest RoPE pair needs to contract at the step
+ * size of a zero input) is tried with a bound in place of the 2x2 part; the
+ * walk is the fallback.  Takes effect when window < chunk_len. */
 #define SG2_DEFAULT_SCAN_WINDOW 64
 int sg2_set_scan_window(int window);
 int sg2_get_scan_window(void);

@@ -17,7 +17,9 @@
 //                  backwards in blocks of `window` steps and the walk stops as
 //                  soon as every |entry| of the running M, in all lanes, is
 //                  below 2^-100: the state entering that block is multiplied
-//                  by less than 2^-100, and the summary is (0, b).
+//                  by less than 2^-100, and the summary is (0, b).  A first
+//                  attempt covers one block sized from the weights with the
+//                  state part only and a norm bound instead of M.
 //   k_chunk_prefix start state of each chunk: summaries applied in order to
 //                  the carried state of the tensor.
 //   k_scan<true>   every chunk replayed from its start state: y = h.C, gate,
