@@ -78,6 +78,37 @@ SG_HD int sg2_first_block_steps(int largest, int any_zero) {
     return (largest + largest / 8 + 8 + 7) & ~7;
 }
 
+/* Near-constant arguments.  The step size is softplus(c_0 + d) and the gate silu(c_0' + d') with d = c_g g + c_s s: for
+ * the small gradients of a trained model |d| is far below 1, and both functions are then their cubic Taylor
+ * polynomials around the constant to within a fraction of an fp32 ulp (remainder <= d^4/24 times the largest fourth
+ * derivative: 5e-9 for softplus, 2e-8 for silu at |d| = 2^-5).  The coefficients are formed once per call from the
+ * shared fp32 primitives (so kernel and checker hold the same bits); a tile of 64 timesteps uses the polynomials when
+ * cmax_g |g| + cmax_s |s| < SG2_TAYLOR_LIMIT for every timestep of the tile, cmax = the largest |c_g|, |c_s| over the dt
+ * and gate rows of the direction, and the functions themselves otherwise. */
+#define SG2_TAYLOR_LIMIT 0.03125f
+SG_HD void sg2_softplus_taylor(float c, float t[4]) {
+    const float s = sg_sigmoid(c), q = s * (1.0f - s);
+    t[0] = sg_softplus(c);
+    t[1] = s;
+    t[2] = 0.5f * q;
+    t[3] = (q * (1.0f - (s + s))) * 0.166666672f;
+}
+/* f = c s, f1 = s + c q, f2 = q (2 + c r), f3 = q (r (3 + c r) - 2 c q) with s = sigmoid(c), q = s (1 - s), r = 1 - 2 s */
+SG_HD void sg2_silu_taylor(float c, float t[4]) {
+    const float s = sg_sigmoid(c), q = s * (1.0f - s), r = 1.0f - (s + s);
+    const float cr = c * r;
+    t[0] = c * s;
+    t[1] = sg_fma(c, q, s);
+    t[2] = 0.5f * (q * (2.0f + cr));
+    t[3] = (q * sg_fma(r, 3.0f + cr, -((c + c) * q))) * 0.166666672f;
+}
+SG_HD float sg2_taylor_delta(const float* c, float g, float s) { return sg_fma(c[0], g, c[1] * s); }
+SG_HD float sg2_taylor_eval(const float* t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); }
+/* does this timestep qualify?  (every timestep of a tile must) */
+SG_HD int sg2_taylor_ok(float cmax_g, float cmax_s, float g, float s) {
+    return sg_fma(cmax_g, sg_abs(g), cmax_s * sg_abs(s)) < SG2_TAYLOR_LIMIT;
+}
+
 /* value of a composed output for one element */
 SG_HD float sg2_comp_eval(const float* c, float g, float s) { return sg_fma(c[0], g, sg_fma(c[1], s, c[2])); }
 

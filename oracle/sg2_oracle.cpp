@@ -235,27 +235,39 @@ struct DirW {
     /* fp32 policy: composed coefficient triples [group][row][3] (include/sg2_compose.h), as the device uses them */
     std::vector<float> comp;
     int comp_rows;
+    /* fp32 policy: cubic Taylor polynomials of the step size and of the gate around their zero-input arguments,
+     * [dt | gate][row][4], and the largest |c_g|, |c_s| of those rows (include/sg2_compose.h) */
+    std::vector<float> tay;
+    float cmax[2];
 };
 
 template <class O>
 struct StepProj {           /* per-timestep projections */
     typename O::R xb[32], z[32], dt[32], B[32], C[32];
+    bool taylor;            /* the tile uses the Taylor polynomials: gate[] holds the gates themselves */
+    typename O::R gate[32];
 };
 
 /* gs: the element's (gradient, sharpness); x: its input projection.  The fp32 policy evaluates the composed
  * affine maps from (g, s); the fp64 policy evaluates the reference's chain of projections from x literally. */
 template <class O>
-void project(const Dims& d, const DirW<O>& w, const typename O::R* x, const float* gs, bool need_zc, StepProj<O>& o) {
+void project(const Dims& d, const DirW<O>& w, const typename O::R* x, const float* gs, bool need_zc, bool taylor, StepProj<O>& o) {
     typedef typename O::R R;
     const int dm = d.d_model, di = d.d_inner, ds = d.d_state;
+    o.taylor = false;
     if (sizeof(R) == 4) {
         const float* c = w.comp.data();
         const int rows = w.comp_rows;
         auto eval = [&](int group, int row) { return (R)sg2_comp_eval(c + ((size_t)group * rows + row) * 3, gs[0], gs[1]); };
+        auto poly = [&](int kind, int group, int row) {
+            return (R)sg2_taylor_eval(&w.tay[((size_t)kind * rows + row) * 4], sg2_taylor_delta(c + ((size_t)group * rows + row) * 3, gs[0], gs[1]));
+        };
+        o.taylor = taylor;
         for (int j = 0; j < di; j++) {
             o.xb[j] = eval(SG2_COMP_XB, j);
             o.z[j] = need_zc ? eval(SG2_COMP_Z, j) : (R)0;
-            o.dt[j] = O::softplus(eval(SG2_COMP_DT, j));
+            o.dt[j] = taylor ? poly(0, SG2_COMP_DT, j) : O::softplus(eval(SG2_COMP_DT, j));
+            o.gate[j] = (taylor && need_zc) ? poly(1, SG2_COMP_Z, j) : (R)0;
         }
         for (int s = 0; s < ds; s++) {
             o.B[s] = eval(SG2_COMP_B, s);
@@ -308,9 +320,15 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
     tc.ao.resize((size_t)ORC_TILE * lanes);
     tc.sn.resize((size_t)ORC_TILE * lanes);
     tc.cs.resize((size_t)ORC_TILE * lanes);
+    /* the tile takes the Taylor polynomials if every one of its timesteps qualifies (the device decides per 64-step tile) */
+    bool taylor = sizeof(R) == 4;
+    for (int k = 0; k < cnt && taylor; k++) {
+        const int64_t u = u0 + k, t = reverse ? (N - 1 - u) : u;
+        taylor = sg2_taylor_ok(w.cmax[0], w.cmax[1], gs[2 * t], gs[2 * t + 1]) != 0;
+    }
     for (int k = 0; k < cnt; k++) {
         const int64_t u = u0 + k, t = reverse ? (N - 1 - u) : u;
-        project<O>(d, w, x + t * dm, gs + 2 * t, need_zc, tc.sp[k]);
+        project<O>(d, w, x + t * dm, gs + 2 * t, need_zc, taylor, tc.sp[k]);
         for (int j = 0; j < di; j++)
             for (int p = 0; p < hp; p++)
                 O::sincos(tc.sp[k].dt[j] * (R)w.rope[j * hp + p], &tc.sn[(size_t)k * lanes + j * hp + p],
@@ -528,7 +546,8 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
             for (int k = 0; k < cnt; k++) {
                 const int64_t u = tile0 + k, t = reverse ? (N - 1 - u) : u;
                 const StepProj<O>& sp = tc.sp[k];
-                O::silu_groups(sp.z, di, gate_group, gate);
+                if (sp.taylor) for (int j = 0; j < di; j++) gate[j] = sp.gate[j];
+                else O::silu_groups(sp.z, di, gate_group, gate);
                 for (int j = 0; j < di; j++) {
                     const R dt = sp.dt[j], xb = sp.xb[j];
                     for (int p = 0; p < hp; p++) {
@@ -622,7 +641,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
     std::vector<R> hst[2];
     for (int dir = 0; dir < 2; dir++) {
         const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0};
+        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0, {}, {0.0f, 0.0f}};
         if (sizeof(R) == 4) {
             w.comp_rows = std::max(di, ds);
             w.comp.assign((size_t)SG2_COMP_GROUPS * w.comp_rows * 3, 0.0f);
@@ -630,6 +649,15 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
                 for (int row = 0; row < ((grp == SG2_COMP_B || grp == SG2_COMP_C) ? ds : di); row++)
                     sg2_compose_one(grp, row, dm, di, W[W_IN_W], W[W_IN_B], W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4],
                                     &w.comp[((size_t)grp * w.comp_rows + row) * 3]);
+            w.tay.assign((size_t)2 * w.comp_rows * 4, 0.0f);
+            for (int j = 0; j < di; j++) {
+                const float* cd = &w.comp[((size_t)SG2_COMP_DT * w.comp_rows + j) * 3];
+                const float* cz = &w.comp[((size_t)SG2_COMP_Z * w.comp_rows + j) * 3];
+                sg2_softplus_taylor(cd[2], &w.tay[((size_t)0 * w.comp_rows + j) * 4]);
+                sg2_silu_taylor(cz[2], &w.tay[((size_t)1 * w.comp_rows + j) * 4]);
+                w.cmax[0] = sg_max(w.cmax[0], sg_max(sg_abs(cd[0]), sg_abs(cz[0])));
+                w.cmax[1] = sg_max(w.cmax[1], sg_max(sg_abs(cd[1]), sg_abs(cz[1])));
+            }
         }
         float* st = dir ? mbwd_io : mfwd_io;
         hst[dir].assign(st, st + di * ds);

@@ -53,6 +53,7 @@
 // and the CPU checker makes the same one).
 // For the bilevel pass k_scan<true, true> also stores the state entering every
 // 32nd step (Plan::htile), which the adjoint kernels restart from.
+#include <type_traits>
 #include "sg2_internal.hpp"
 #include "../../include/sg2_compose.h"
 
@@ -189,9 +190,20 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[2] = out[2];
     // How many steps the first block of a chunk summary should cover: what the slowest pair of either direction needs
     // to contract below 2^-100 at the step size a zero input gives (sg2_contraction_steps), plus a margin.
-    __shared__ int s_largest, s_zero;
-    if (threadIdx.x == 0) { s_largest = 0; s_zero = 0; }
+    __shared__ int s_largest, s_zero, s_cmax[2][2];
+    if (threadIdx.x == 0) { s_largest = 0; s_zero = 0; s_cmax[0][0] = s_cmax[0][1] = s_cmax[1][0] = s_cmax[1][1] = 0; }
     __syncthreads();
+    // Taylor polynomials of the step size and of the gate around their zero-input arguments (sg2_compose.h), and the
+    // largest |c_g|, |c_s| of those rows (bit patterns of non-negative floats order like integers)
+    if (group == SG2_COMP_DT || group == SG2_COMP_Z) {
+        float t[4];
+        if (group == SG2_COMP_DT) sg2_softplus_taylor(out[2], t);
+        else sg2_silu_taylor(out[2], t);
+        float* tay = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + ((dir * 2 + (group == SG2_COMP_Z ? 1 : 0)) * G::ROWS + row) * 4;
+        tay[0] = t[0]; tay[1] = t[1]; tay[2] = t[2]; tay[3] = t[3];
+        atomicMax(&s_cmax[dir][0], sg_f2i(sg_abs(out[0])));
+        atomicMax(&s_cmax[dir][1], sg_f2i(sg_abs(out[1])));
+    }
     if (group == SG2_COMP_DT) {
         const float dt0 = sg_softplus(out[2]);
         const float* alog = pl.W.w[dir ? W_B_ALOG : W_F_ALOG] + row * G::DS;
@@ -205,6 +217,9 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     if (threadIdx.x == 0) {
         pl.contracted[0] = 1;      // until a summary kernel finds a chunk that has not contracted
         pl.contracted[1] = sg2_first_block_steps(s_largest, s_zero);
+        float* cmax = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4;
+        cmax[0] = sg_i2f(s_cmax[0][0]); cmax[1] = sg_i2f(s_cmax[0][1]);
+        cmax[2] = sg_i2f(s_cmax[1][0]); cmax[3] = sg_i2f(s_cmax[1][1]);
     }
 }
 
@@ -216,17 +231,32 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
 // Returns bit 0: every rotation angle of this timestep, over this half's columns, is small enough for
 // sg_sincos_small; bit 1: small enough for sg_sincos_tiny (fmax: per column, the largest |rope frequency| of its 8 pairs; dt >= 0 and
 // rounding is monotone, so dt*fmax < limit is the same statement as |dt*freq| < limit for all pairs).
-template <class G, bool OUT, int PART, bool HAS_S>
+// TAYLOR: every timestep of the tile has passed sg2_taylor_ok: step size and gate come from their cubic Taylor
+// polynomials.  Those cost no LDS of their own in the output pass (the workgroup's LDS is what limits it to six per CU):
+// the step-size polynomial of column j sits in the padding of row j of s_dx, and the gate polynomial of column j
+// is spread over the fourth padding floats of rows j of s_dt, s_B, s_C and s_gate, which this wave reads anyway
+// (d_inner = d_state: the wave's columns and its rows of B and C carry the same indices).  The summary pass has
+// no s_dx and keeps the step-size polynomials in s_tay.
+template <class G, bool OUT, int PART, bool HAS_S, bool TAYLOR>
 __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_dt, float* s_ux, float* s_dx, float* s_B,
-                                             float* s_C, float* s_gate, const float* s_fmax) {
+                                             float* s_C, float* s_gate, const float* s_fmax, const float* s_tay) {
+    static_assert(G::DI == G::DS, "the gate polynomials ride on the rows of B and C");
+    auto delta = [&](const f32x4 t) { return HAS_S ? sg_fma(t[0], g, t[1] * s) : t[0] * g; };
+    auto poly = [&](const f32x4 t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); };
     // HAS_S is false for a tensor whose sharpness is all zero: fma(c_s, 0, c_0) is c_0 itself, so the term is skipped
     auto eval = [&](const f32x4 t) { return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]); };
     auto coef = [&](const float* arr, int row) { return *reinterpret_cast<const f32x4*>(arr + row * LDS_STRIDE + SCAN_TT); };
+    constexpr int NR = G::DI / G::PARTS;        // this wave's columns = its rows of B and C
+    float gp0[NR], gp1[NR], gp2[NR];            // first three coefficients of the gate polynomials, picked up on the way
     bool small = true, tiny = true;
 #pragma unroll
-    for (int q = 0; q < G::DI / G::PARTS; q++) {
-        const int jj = PART * (G::DI / G::PARTS) + q;
-        const float dtv = sg_softplus(eval(coef(s_dt, jj)));
+    for (int q = 0; q < NR; q++) {
+        const int jj = PART * NR + q;
+        const f32x4 cd = coef(s_dt, jj);
+        gp0[q] = cd[3];
+        float dtv;
+        if (TAYLOR) dtv = poly(OUT ? coef(s_dx, jj) : *reinterpret_cast<const f32x4*>(s_tay + jj * 4), delta(cd));
+        else dtv = sg_softplus(eval(cd));
         const float amax = dtv * s_fmax[jj];
         small = small && (amax < SG_SINCOS_SMALL_LIMIT);
         tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
@@ -237,36 +267,58 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
         if (OUT) s_dx[jj * LDS_STRIDE + tu] = cx[3] * xbv;
     }
 #pragma unroll
-    for (int q = 0; q < G::DS / G::PARTS; q++) {
-        const int ss = PART * (G::DS / G::PARTS) + q;
-        s_B[ss * LDS_STRIDE + tu] = eval(coef(s_B, ss));
-        if (OUT) s_C[ss * LDS_STRIDE + tu] = eval(coef(s_C, ss));
+    for (int q = 0; q < NR; q++) {
+        const int ss = PART * NR + q;
+        const f32x4 cb = coef(s_B, ss);
+        gp1[q] = cb[3];
+        s_B[ss * LDS_STRIDE + tu] = eval(cb);
+        if (OUT) {
+            const f32x4 cc = coef(s_C, ss);
+            gp2[q] = cc[3];
+            s_C[ss * LDS_STRIDE + tu] = eval(cc);
+        }
     }
     if (OUT) {
         // the gates of this wave's columns share one reciprocal (sg_silu_block)
-        constexpr int NG = G::DI / G::PARTS;
-        static_assert(NG <= 8, "sg_silu_block takes at most 8 values");
-        float zv[NG], gv[NG];
+        static_assert(NR <= 8, "sg_silu_block takes at most 8 values");
+        float zv[NR], gv[NR];
+        if (TAYLOR) {
 #pragma unroll
-        for (int q = 0; q < NG; q++) zv[q] = eval(coef(s_gate, PART * NG + q));
-        sg_silu_block(NG, zv, gv);
+            for (int q = 0; q < NR; q++) {
+                const f32x4 cz = coef(s_gate, PART * NR + q);
+                gv[q] = poly(f32x4{gp0[q], gp1[q], gp2[q], cz[3]}, delta(cz));
+            }
+        } else {
 #pragma unroll
-        for (int q = 0; q < NG; q++) s_gate[(PART * NG + q) * LDS_STRIDE + tu] = gv[q];
+            for (int q = 0; q < NR; q++) zv[q] = eval(coef(s_gate, PART * NR + q));
+            sg_silu_block(NR, zv, gv);
+        }
+#pragma unroll
+        for (int q = 0; q < NR; q++) s_gate[(PART * NR + q) * LDS_STRIDE + tu] = gv[q];
     }
     return (small ? 1 : 0) | (tiny ? 2 : 0);
 }
 
 // Once per workgroup: the composed coefficient triples of this direction (and D) into the padding of the LDS rows.
+// tay: this direction's Taylor polynomials, [step size | gate][row][4] (see project_tile for where they go).
 template <class G, bool OUT>
-__device__ __forceinline__ void stage_coefficients(const float* __restrict__ comp, const float* __restrict__ Dw, int tid, float* s_dt,
-                                                   float* s_ux, float* s_B, float* s_C, float* s_gate) {
-    static_assert(SG2_COMP_GROUPS * G::ROWS <= G::THREADS, "one thread per (group, row)");
+__device__ __forceinline__ void stage_coefficients(const float* __restrict__ comp, const float* __restrict__ tay, const float* __restrict__ Dw,
+                                                   int tid, float* s_dt, float* s_ux, float* s_dx, float* s_B, float* s_C, float* s_gate,
+                                                   float* s_tay) {
+    static_assert(SG2_COMP_GROUPS * G::ROWS <= G::THREADS && G::ROWS == G::DI, "one thread per (group, row)");
     if (tid < SG2_COMP_GROUPS * G::ROWS) {
         const int group = tid / G::ROWS, row = tid % G::ROWS;
         float* arr = group == SG2_COMP_XB ? s_ux : group == SG2_COMP_DT ? s_dt : group == SG2_COMP_B ? s_B : group == SG2_COMP_C ? s_C : s_gate;
         if (OUT || (group != SG2_COMP_C && group != SG2_COMP_Z)) {
             const float* t = comp + (group * G::ROWS + row) * 3;
-            *reinterpret_cast<f32x4*>(arr + row * LDS_STRIDE + SCAN_TT) = f32x4{t[0], t[1], t[2], group == SG2_COMP_XB ? Dw[row] : 0.0f};
+            // fourth float: D next to the x-branch triple; coefficient 0, 1, 2, 3 of the row's gate polynomial next to dt, B, C, z
+            const float* gp = tay + (G::ROWS + row) * 4;
+            const float w = group == SG2_COMP_XB ? Dw[row] : !OUT ? 0.0f : group == SG2_COMP_DT ? gp[0] : group == SG2_COMP_B ? gp[1] : group == SG2_COMP_C ? gp[2] : gp[3];
+            *reinterpret_cast<f32x4*>(arr + row * LDS_STRIDE + SCAN_TT) = f32x4{t[0], t[1], t[2], w};
+        }
+        if (group == SG2_COMP_DT) {
+            const float* dp = tay + row * 4;
+            *reinterpret_cast<f32x4*>(OUT ? s_dx + row * LDS_STRIDE + SCAN_TT : s_tay + row * 4) = f32x4{dp[0], dp[1], dp[2], dp[3]};
         }
     }
 }
@@ -348,6 +400,7 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     // y of column j goes where dt of column j was: both are touched only by the 8 lanes of column j, in program order
     float* const s_y = s_dt;
     __shared__ float s_fmax[DI];
+    __shared__ __attribute__((aligned(16))) float s_tay[OUT ? 4 : DI * 4];   // summary pass: Taylor polynomials of the step size (the output pass keeps its own in row padding)
     __shared__ __attribute__((aligned(16))) float s_wout[OUT ? DM * DI : 4];      // out_proj of this direction
     __shared__ unsigned long long s_large[PARTS];      // per wave's share of the columns: bit t set = timestep t of the tile needs the full sin/cos
     __shared__ unsigned long long s_nottiny[PARTS];    // ... bit t set = timestep t is not eligible for sg_sincos_tiny
@@ -382,11 +435,15 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     {   // largest |frequency| of each column's pairs
         const float f = pair_tree_max<HP>(sg_abs(freq));
         if (p == 0) s_fmax[j] = f;
-        stage_coefficients<G, OUT>(pl.comp + dir * (SG2_COMP_GROUPS * G::ROWS * 3), pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_B, s_C, s_gate);
+        stage_coefficients<G, OUT>(pl.comp + dir * (SG2_COMP_GROUPS * G::ROWS * 3), pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4,
+                                   pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_tay);
         static_assert(DM * DI == SCAN_THREADS, "one out_proj entry per thread");
         if (OUT) s_wout[tid] = pl.W.w[dir ? W_B_OUT : W_F_OUT][tid];
         __syncthreads();
     }
+    // largest |c_g|, |c_s| over this direction's step-size and gate rows: what decides whether a tile may use the polynomials
+    const float cmax_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir];
+    const float cmax_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir + 1];
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     bool fully_contracted = false;      // summary pass: the walk stopped because the 2x2 part had contracted
@@ -452,27 +509,23 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
         const float sh = valid ? shv : 0.0f;
         int angle_t;
-        if (PARTS == 2) {
-            if (has_s) {
-                if (half == 0)
-                    angle_t = project_tile<G, OUT, 0, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-                else
-                    angle_t = project_tile<G, OUT, 1, true>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-            } else {
-                if (half == 0)
-                    angle_t = project_tile<G, OUT, 0, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-                else
-                    angle_t = project_tile<G, OUT, 1, false>(g, sh, tu, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_fmax);
-            }
-        } else {
-            // many waves: one copy of the code, the arrays moved to this wave's first row
-            const int rj = half * (DI / PARTS) * LDS_STRIDE, rs = half * (DS / PARTS) * LDS_STRIDE;
-            if (has_s)
-                angle_t = project_tile<G, OUT, 0, true>(g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0),
-                                                        s_gate + (OUT ? rj : 0), s_fmax + half * (DI / PARTS));
-            else
-                angle_t = project_tile<G, OUT, 0, false>(g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0),
-                                                         s_gate + (OUT ? rj : 0), s_fmax + half * (DI / PARTS));
+        {
+            // the same 64 timesteps in every wave of the workgroup: the same decision without talking to one another
+            const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
+            // PARTS == 2: the wave's share is a template parameter; more waves: one copy of the code, the arrays moved to this wave's first row
+            const int rj = (PARTS == 2) ? 0 : half * (DI / PARTS) * LDS_STRIDE, rs = (PARTS == 2) ? 0 : half * (DS / PARTS) * LDS_STRIDE;
+            const int rt = (PARTS == 2 || OUT) ? 0 : half * (DI / PARTS) * 4;
+            auto run = [&](auto part_c, auto has_s_c, auto tay_c) {
+                return project_tile<G, OUT, decltype(part_c)::value, decltype(has_s_c)::value, decltype(tay_c)::value>(
+                    g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0), s_gate + (OUT ? rj : 0),
+                    s_fmax + ((PARTS == 2) ? 0 : half * (DI / PARTS)), s_tay + rt);
+            };
+            auto with_part = [&](auto has_s_c, auto tay_c) {
+                if (PARTS == 2 && half == 1) return run(std::integral_constant<int, (PARTS == 2) ? 1 : 0>{}, has_s_c, tay_c);
+                return run(std::integral_constant<int, 0>{}, has_s_c, tay_c);
+            };
+            if (tay) angle_t = has_s ? with_part(std::true_type{}, std::true_type{}) : with_part(std::false_type{}, std::true_type{});
+            else angle_t = has_s ? with_part(std::true_type{}, std::false_type{}) : with_part(std::false_type{}, std::false_type{});
         }
         {   // wave w projects the dt of columns w*64/HP .. (w+1)*64/HP-1, which are the columns it owns in the recurrence
             const unsigned long long large = __builtin_amdgcn_ballot_w64(!(angle_t & 1));
