@@ -39,6 +39,11 @@ def load(path):
         f.argtypes = [C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_float)]
     L.orc_abar.restype = C.c_float
     L.orc_abar.argtypes = [C.c_float, C.c_float]
+    for f in (L.orc_softplus_taylor, L.orc_silu_taylor):
+        f.restype = C.c_float
+        f.argtypes = [C.c_float, C.c_float]
+    L.orc_contraction_steps.restype = C.c_int
+    L.orc_contraction_steps.argtypes = [C.c_float, C.c_float, C.c_float]
     L.orc_f_to_f16.restype = C.c_uint16
     L.orc_f_to_f16.argtypes = [C.c_float]
     L.orc_f16_to_f.restype = C.c_float

@@ -64,6 +64,12 @@
  * margin: sg2_first_block_steps in include/sg2_compose.h), walked with the state part only, while the 2x2 part is
  * bounded by the running product of max(|A_bar_e|, |A_bar_o|) (rotations preserve length).  If the bound is below
  * 2^-100 in every (j,p) the summary is (0, b) with that block's b; otherwise the walk above starts from scratch.
+ * Step size and gate of a 64-step tile (fp32 policy, as the kernels): when every timestep of the tile has
+ * cmax_g |g| + cmax_s |s| < 2^-5 (cmax: the largest |c_g|, |c_s| of the composed dt and gate rows of the
+ * direction), softplus(c_0 + d) and silu(c_0' + d') are evaluated as their cubic Taylor polynomials in d around
+ * the zero-input arguments (sg2_softplus_taylor / sg2_silu_taylor in include/sg2_compose.h: within a fraction of an
+ * fp32 ulp of the functions, tests/test_oracle_primitives.py); other tiles take the functions themselves.  The
+ * float64 policy always takes the functions.
  * A (j,p) whose M is exactly zero hands on b itself as the next start state
  * (not 0 * h + b, which differs for a non-finite h): the kernels read no
  * earlier state at all when every summary of a call is of that kind.
@@ -824,6 +830,9 @@ float orc_silu(float x) { return sg_silu(x); }
 void orc_silu_block(int n, const float* z, float* out) { sg_silu_block(n, z, out); }
 void orc_sigmoid_block(int n, const float* x, float* out) { sg_sigmoid_block(n, x, out); }
 void orc_tanh_block(int n, const float* x, float* out) { sg_tanh_block(n, x, out); }
+float orc_softplus_taylor(float c, float d) { float t[4]; sg2_softplus_taylor(c, t); return sg2_taylor_eval(t, d); }
+float orc_silu_taylor(float c, float d) { float t[4]; sg2_silu_taylor(c, t); return sg2_taylor_eval(t, d); }
+int orc_contraction_steps(float dt0, float nhA_e, float nhA_o) { return sg2_contraction_steps(dt0, nhA_e, nhA_o); }
 float orc_tanh(float x) { return sg_tanh(x); }
 float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }
 float orc_cos(float x) { float s, c; sg_sincos(x, &s, &c); return c; }

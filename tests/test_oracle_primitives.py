@@ -192,3 +192,34 @@ def test_half_conversions_match_numpy():
     for x, hb, back in zip(t.numpy(), bits, b.float().numpy()):
         assert L.orc_f_to_bf16(float(x)) == int(hb)
         assert L.orc_bf16_to_f(int(hb)) == float(back)
+
+
+def test_taylor_polynomials_of_step_size_and_gate():
+    """softplus(c + d) and silu(c + d) from their cubic Taylor polynomials around c, for |d| below the limit a tile has
+    to meet (2^-5): within an fp32 rounding or two of the functions themselves (float64), over the whole range of c.
+    A wrong derivative (sign, factor) would be off by d^2 or d^3 times a derivative of order 0.1: 1e-4 .. 1e-6."""
+    r = np.random.RandomState(5)
+    cs = np.concatenate([r.uniform(-14, 14, 3000), r.uniform(-1, 1, 2000), [0.0, -30.0, 30.0, 88.0, -88.0]]).astype(np.float32)
+    ds = np.concatenate([r.uniform(-1, 1, cs.size - 4) * 2.0 ** -5, [2.0 ** -5, -2.0 ** -5, 0.0, 1e-8]]).astype(np.float32)
+    worst_sp = worst_si = 0.0
+    for c, d in zip(cs, ds):
+        x = float(c) + float(d)
+        sp = math.log1p(math.exp(-abs(x))) + max(x, 0.0)
+        si = x / (1.0 + math.exp(-x))
+        e_sp = abs(L.orc_softplus_taylor(float(c), float(d)) - sp) / (3e-7 * abs(sp) + 1e-8)
+        e_si = abs(L.orc_silu_taylor(float(c), float(d)) - si) / (3e-7 * abs(si) + 4e-8)
+        worst_sp, worst_si = max(worst_sp, e_sp), max(worst_si, e_si)
+    assert worst_sp <= 1.0 and worst_si <= 1.0, (worst_sp, worst_si)
+    # at d = 0 the polynomials are the functions' own values
+    for c in (-3.0, 0.25, 7.0):
+        assert L.orc_softplus_taylor(c, 0.0) == L.orc_softplus(c) and L.orc_silu_taylor(c, 0.0) == np.float32(c) * np.float32(L.orc_sigmoid(c))
+
+
+def test_contraction_steps_bound_the_decay():
+    """sg2_contraction_steps(dt, -A_e/2, -A_o/2): the slower pole's |A_bar| to that power is below 2^-100, and one step
+    fewer by more than a rounding's worth is not; poles that do not contract within a million steps give 0."""
+    for dt, Ae, Ao in ((0.7, -1.0, -0.75), (0.05, -3.0, -16.0), (1.7, -16.0, -1.0), (3.0, -0.01, -0.02)):
+        n = L.orc_contraction_steps(dt, -0.5 * Ae, -0.5 * Ao)
+        m = max(abs((1 + dt * A / 2) / (1 - dt * A / 2)) for A in (Ae, Ao))
+        assert n > 0 and m ** n < 2.0 ** -100 * 1.001 and m ** (n - 2) > 2.0 ** -100, (dt, Ae, Ao, n, m)
+    assert L.orc_contraction_steps(1e-6, -0.5 * -1e-3, -0.5 * -1e-3) == 0
