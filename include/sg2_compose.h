@@ -109,6 +109,33 @@ SG_HD int sg2_taylor_ok(float cmax_g, float cmax_s, float g, float s) {
     return sg_fma(cmax_g, sg_abs(g), cmax_s * sg_abs(s)) < SG2_TAYLOR_LIMIT;
 }
 
+/* Near-constant step sizes.  Where dt stays within a small d of the zero-input step size dt0 of its column, the
+ * coefficients of the recurrence are polynomials in d = dt - dt0 with per-pair constants: A_bar(dt) = 2/(1 + a dt) - 1
+ * (a = -A/2) as a cubic (remainder 2 (a d)^4), sin/cos(f dt) as quadratics (remainder (f d)^3 / 6).  A block of 8
+ * timesteps uses them when for each of its timesteps  kpoly_g |g| + kpoly_s |s| < 1,  with kpoly = max(128 a_max,
+ * 256 f_max) times the largest |c_g|, |c_s| of the direction's dt rows (|dt - dt0| <= |c_g g + c_s s|: softplus has
+ * slope <= 1): a d < 2^-7 and f d < 2^-8, remainders below 1e-8. */
+SG_HD void sg2_abar_poly(float dt0, float nhA, float p[4]) {
+    const float r = sg_rcp_pos(sg_fma(dt0, nhA, 1.0f));
+    const float ar = nhA * r;
+    p[0] = sg_fma(2.0f, r, -1.0f);
+    p[1] = -((ar + ar) * r);
+    p[2] = -(p[1] * ar);
+    p[3] = -(p[2] * ar);
+}
+SG_HD void sg2_sincos_poly(float dt0, float f, float qs[3], float qc[3]) {
+    float s0, c0;
+    sg_sincos(dt0 * f, &s0, &c0);
+    const float fs = f * s0, fc = f * c0;
+    qs[0] = s0; qs[1] = fc; qs[2] = -0.5f * (f * fs);
+    qc[0] = c0; qc[1] = -fs; qc[2] = -0.5f * (f * fc);
+}
+SG_HD float sg2_poly3(const float* p, float d) { return sg_fma(sg_fma(sg_fma(p[3], d, p[2]), d, p[1]), d, p[0]); }
+SG_HD float sg2_poly2(const float* q, float d) { return sg_fma(sg_fma(q[2], d, q[1]), d, q[0]); }
+SG_HD int sg2_poly_ok(float kpoly_g, float kpoly_s, float g, float s) {
+    return sg_fma(kpoly_g, sg_abs(g), kpoly_s * sg_abs(s)) < 1.0f;
+}
+
 /* value of a composed output for one element */
 SG_HD float sg2_comp_eval(const float* c, float g, float s) { return sg_fma(c[0], g, sg_fma(c[1], s, c[2])); }
 

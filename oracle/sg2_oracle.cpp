@@ -245,6 +245,10 @@ struct DirW {
      * [dt | gate][row][4], and the largest |c_g|, |c_s| of those rows (include/sg2_compose.h) */
     std::vector<float> tay;
     float cmax[2];
+    /* fp32 policy: every (column, pair) as polynomials in dt - dt0 (sg2_abar_poly, sg2_sincos_poly):
+     * [lane][pe 4 | po 4 | qs 3 | qc 3], and the two factors of sg2_poly_ok */
+    std::vector<float> lane_poly;
+    float kpoly[2];
 };
 
 template <class O>
@@ -340,6 +344,28 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
                 O::sincos(tc.sp[k].dt[j] * (R)w.rope[j * hp + p], &tc.sn[(size_t)k * lanes + j * hp + p],
                           &tc.cs[(size_t)k * lanes + j * hp + p]);
     }
+    /* blocks of 8 steps whose timesteps all pass sg2_poly_ok take A_bar, sin and cos from the lane polynomials */
+    std::vector<char> poly_block(ORC_TILE / ORC_BLOCK, 0);
+    if (sizeof(R) == 4) {
+        for (int b0 = 0; b0 + ORC_BLOCK <= cnt; b0 += ORC_BLOCK) {
+            bool ok = true;
+            for (int q = 0; q < ORC_BLOCK && ok; q++) {
+                const int64_t u = u0 + b0 + q, t = reverse ? (N - 1 - u) : u;
+                ok = sg2_poly_ok(w.kpoly[0], w.kpoly[1], gs[2 * t], gs[2 * t + 1]) != 0;
+            }
+            poly_block[b0 / ORC_BLOCK] = ok;
+            if (!ok) continue;
+            for (int q = 0; q < ORC_BLOCK; q++)
+                for (int l = 0; l < lanes; l++) {
+                    const float* lp = &w.lane_poly[(size_t)l * 14];
+                    const float dd = (float)tc.sp[b0 + q].dt[l / hp] - w.tay[((size_t)0 * w.comp_rows + l / hp) * 4];
+                    tc.ae[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly3(lp, dd);
+                    tc.ao[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly3(lp + 4, dd);
+                    tc.sn[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(lp + 8, dd);
+                    tc.cs[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(lp + 11, dd);
+                }
+        }
+    }
     if (sizeof(R) == 4) {
         /* blocks whose angles are all below SG_SINCOS_TINY_LIMIT, over the 8 steps and the columns of a wave, take
          * sg_sincos_tiny (the device decides with dt * max_p |rope[j,p]| per column) */
@@ -347,7 +373,7 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
         for (int j = 0; j < di; j++)
             for (int p = 0; p < hp; p++) fmax[j] = sg_max(fmax[j], sg_abs(w.rope[j * hp + p]));
         for (int b0 = 0; b0 + ORC_BLOCK <= cnt; b0 += ORC_BLOCK)
-            for (int wave0 = 0; wave0 < lanes; wave0 += ORC_WAVE) {
+            for (int wave0 = 0; wave0 < lanes && !poly_block[b0 / ORC_BLOCK]; wave0 += ORC_WAVE) {
                 const int wave1 = std::min(lanes, wave0 + ORC_WAVE);
                 bool tiny = true;
                 for (int q = 0; q < ORC_BLOCK && tiny; q++)
@@ -368,7 +394,7 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
     if (sizeof(R) == 4) {
         std::vector<float> de((size_t)lanes * ORC_BLOCK), dod((size_t)lanes * ORC_BLOCK), P((size_t)lanes * ORC_BLOCK);
         for (; k0 + ORC_BLOCK <= cnt; k0 += ORC_BLOCK) {
-            for (int wave0 = 0; wave0 < lanes; wave0 += ORC_WAVE) {
+            for (int wave0 = 0; wave0 < lanes && !poly_block[k0 / ORC_BLOCK]; wave0 += ORC_WAVE) {
                 const int wave1 = std::min(lanes, wave0 + ORC_WAVE);
                 bool block_ok = true;
                 for (int l = wave0; l < wave1; l++) {
@@ -647,7 +673,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
     std::vector<R> hst[2];
     for (int dir = 0; dir < 2; dir++) {
         const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0, {}, {0.0f, 0.0f}};
+        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0, {}, {0.0f, 0.0f}, {}, {0.0f, 0.0f}};
         if (sizeof(R) == 4) {
             w.comp_rows = std::max(di, ds);
             w.comp.assign((size_t)SG2_COMP_GROUPS * w.comp_rows * 3, 0.0f);
@@ -664,6 +690,29 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
                 w.cmax[0] = sg_max(w.cmax[0], sg_max(sg_abs(cd[0]), sg_abs(cz[0])));
                 w.cmax[1] = sg_max(w.cmax[1], sg_max(sg_abs(cd[1]), sg_abs(cz[1])));
             }
+            /* lane polynomials and the limit of their use */
+            const int hp = ds / 2;
+            float amax = 0.0f, fmax = 0.0f, cdt[2] = {0.0f, 0.0f};
+            w.lane_poly.assign((size_t)di * hp * 14, 0.0f);
+            for (int j = 0; j < di; j++) {
+                const float* cd = &w.comp[((size_t)SG2_COMP_DT * w.comp_rows + j) * 3];
+                cdt[0] = sg_max(cdt[0], sg_abs(cd[0]));
+                cdt[1] = sg_max(cdt[1], sg_abs(cd[1]));
+                const float dt0 = w.tay[((size_t)0 * w.comp_rows + j) * 4];
+                for (int p = 0; p < hp; p++) {
+                    const float a_e = -0.5f * -sg_exp(w.A_log[j * ds + 2 * p]), a_o = -0.5f * -sg_exp(w.A_log[j * ds + 2 * p + 1]);
+                    const float f = w.rope[j * hp + p];
+                    amax = sg_max(amax, sg_max(a_e, a_o));
+                    fmax = sg_max(fmax, sg_abs(f));
+                    float* lp = &w.lane_poly[((size_t)j * hp + p) * 14];
+                    sg2_abar_poly(dt0, a_e, lp);
+                    sg2_abar_poly(dt0, a_o, lp + 4);
+                    sg2_sincos_poly(dt0, f, lp + 8, lp + 11);
+                }
+            }
+            const float kp = sg_max(128.0f * amax, 256.0f * fmax);
+            w.kpoly[0] = kp * cdt[0];
+            w.kpoly[1] = kp * cdt[1];
         }
         float* st = dir ? mbwd_io : mfwd_io;
         hst[dir].assign(st, st + di * ds);

@@ -190,8 +190,11 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[2] = out[2];
     // How many steps the first block of a chunk summary should cover: what the slowest pair of either direction needs
     // to contract below 2^-100 at the step size a zero input gives (sg2_contraction_steps), plus a margin.
-    __shared__ int s_largest, s_zero, s_cmax[2][2];
-    if (threadIdx.x == 0) { s_largest = 0; s_zero = 0; s_cmax[0][0] = s_cmax[0][1] = s_cmax[1][0] = s_cmax[1][1] = 0; }
+    __shared__ int s_largest, s_zero, s_cmax[2][2], s_cdt[2][2], s_amax[2], s_fmax[2];
+    if (threadIdx.x == 0) {
+        s_largest = 0; s_zero = 0;
+        for (int k = 0; k < 2; k++) { s_cmax[k][0] = s_cmax[k][1] = s_cdt[k][0] = s_cdt[k][1] = s_amax[k] = s_fmax[k] = 0; }
+    }
     __syncthreads();
     // Taylor polynomials of the step size and of the gate around their zero-input arguments (sg2_compose.h), and the
     // largest |c_g|, |c_s| of those rows (bit patterns of non-negative floats order like integers)
@@ -203,14 +206,22 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
         tay[0] = t[0]; tay[1] = t[1]; tay[2] = t[2]; tay[3] = t[3];
         atomicMax(&s_cmax[dir][0], sg_f2i(sg_abs(out[0])));
         atomicMax(&s_cmax[dir][1], sg_f2i(sg_abs(out[1])));
+        if (group == SG2_COMP_DT) {
+            atomicMax(&s_cdt[dir][0], sg_f2i(sg_abs(out[0])));
+            atomicMax(&s_cdt[dir][1], sg_f2i(sg_abs(out[1])));
+        }
     }
     if (group == SG2_COMP_DT) {
         const float dt0 = sg_softplus(out[2]);
         const float* alog = pl.W.w[dir ? W_B_ALOG : W_F_ALOG] + row * G::DS;
         for (int p = 0; p < G::HP; p++) {
-            const int n = sg2_contraction_steps(dt0, -0.5f * -sg_exp(alog[2 * p]), -0.5f * -sg_exp(alog[2 * p + 1]));
+            const float a_e = -0.5f * -sg_exp(alog[2 * p]), a_o = -0.5f * -sg_exp(alog[2 * p + 1]);
+            const int n = sg2_contraction_steps(dt0, a_e, a_o);
             if (n == 0) atomicOr(&s_zero, 1);
             atomicMax(&s_largest, n);
+            // for sg2_poly_ok: the largest -A/2 and the largest |rotation frequency| of the direction
+            atomicMax(&s_amax[dir], sg_f2i(sg_max(a_e, a_o)));
+            atomicMax(&s_fmax[dir], sg_f2i(sg_abs(pl.W.w[dir ? W_B_ROPE : W_F_ROPE][row * G::HP + p])));
         }
     }
     __syncthreads();
@@ -220,6 +231,11 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
         float* cmax = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4;
         cmax[0] = sg_i2f(s_cmax[0][0]); cmax[1] = sg_i2f(s_cmax[0][1]);
         cmax[2] = sg_i2f(s_cmax[1][0]); cmax[3] = sg_i2f(s_cmax[1][1]);
+        for (int k = 0; k < 2; k++) {
+            const float kp = sg_max(128.0f * sg_i2f(s_amax[k]), 256.0f * sg_i2f(s_fmax[k]));
+            cmax[4 + 2 * k] = kp * sg_i2f(s_cdt[k][0]);
+            cmax[5 + 2 * k] = kp * sg_i2f(s_cdt[k][1]);
+        }
     }
 }
 
@@ -327,6 +343,10 @@ __device__ __forceinline__ void stage_coefficients(const float* __restrict__ com
 struct LaneState {
     float he, ho, c0e, c0o, c1e, c1o;
 };
+// the lane's pair as polynomials in dt - dt0 (sg2_abar_poly, sg2_sincos_poly): dt0 = step size of its column for a zero input
+struct LanePoly {
+    float dt0, pe[4], po[4], qs[3], qc[3];
+};
 
 // LITE (summary pass only): the state part alone, and in c0e the running product of max(|A_bar_e|, |A_bar_o|), a bound
 // on the norm of the 2x2 part that is not formed
@@ -351,13 +371,23 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // UB consecutive timesteps (all valid): coefficients first, then the serial chain.  ux = dt * x-branch
 // (formed once per timestep in phase A).  The A_bar of the block share one reciprocal per lane
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
-// ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values; tcoef = the lane's sg_sincos_tiny_coef).
+// ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values, polynomials in dt),
+// 3: every timestep of the block has passed sg2_poly_ok: A_bar, sin and cos from the lane's polynomials in dt - dt0.
 template <int HP, bool OUT, int ANGLE, bool LITE = false>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
-                                            float hAo, float freq, const float (&tcoef)[6], float (&y)[UB]) {
+                                            float hAo, float freq, const LanePoly& LP, float (&y)[UB]) {
     float ae[UB], ao[UB], sn[UB], cs[UB], be[UB], bo[UB];
-    {
+    if (ANGLE == 3) {
+#pragma unroll
+        for (int u = 0; u < UB; u++) {
+            const float d = dt[u] - LP.dt0;
+            ae[u] = sg2_poly3(LP.pe, d);
+            ao[u] = sg2_poly3(LP.po, d);
+            sn[u] = sg2_poly2(LP.qs, d);
+            cs[u] = sg2_poly2(LP.qc, d);
+        }
+    } else {
         float d_e[UB], d_o[UB], P[UB];
         const float last = sg_abar_block_prefix(UB, dt, hAe, hAo, d_e, d_o, P);
         if (__builtin_amdgcn_ballot_w64(!(last < SG_ABAR_BLOCK_LIMIT)) == 0) {
@@ -367,11 +397,13 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
             for (int u = 0; u < UB; u++) sg_abar_pair(dt[u], hAe, hAo, &ae[u], &ao[u]);
         }
     }
+    float tcoef[6];             // tiny-angle sin/cos of this lane's pair as polynomials in dt (formed here: a block that comes this way is the exception)
+    if (ANGLE == 2) sg_sincos_tiny_coef(freq, tcoef);
 #pragma unroll
     for (int u = 0; u < UB; u++) {
         if (ANGLE == 2) sg_sincos_tiny_dt(dt[u], tcoef, &sn[u], &cs[u]);
         else if (ANGLE == 1) sg_sincos_small(dt[u] * freq, &sn[u], &cs[u]);
-        else sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
+        else if (ANGLE == 0) sg_sincos(dt[u] * freq, &sn[u], &cs[u]);
         be[u] = ux[u] * Be[u];
         bo[u] = ux[u] * Bo[u];
     }
@@ -429,8 +461,12 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
     const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
     const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
-    float tcoef[6];             // tiny-angle sin/cos of this lane's pair as polynomials in dt
-    sg_sincos_tiny_coef(freq, tcoef);
+    // this lane's pair as polynomials in dt - dt0, dt0 = the step size of its column for a zero input
+    LanePoly LP;
+    LP.dt0 = pl.comp[2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4 + j * 4];
+    sg2_abar_poly(LP.dt0, hAe, LP.pe);
+    sg2_abar_poly(LP.dt0, hAo, LP.po);
+    sg2_sincos_poly(LP.dt0, freq, LP.qs, LP.qc);
 
     {   // largest |frequency| of each column's pairs
         const float f = pair_tree_max<HP>(sg_abs(freq));
@@ -444,6 +480,9 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     // largest |c_g|, |c_s| over this direction's step-size and gate rows: what decides whether a tile may use the polynomials
     const float cmax_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir];
     const float cmax_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir + 1];
+    // ... and whether a block of the recurrence may use the lane polynomials (sg2_poly_ok)
+    const float kpoly_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 4 + 2 * dir];
+    const float kpoly_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 4 + 2 * dir + 1];
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     bool fully_contracted = false;      // summary pass: the walk stopped because the 2x2 part had contracted
@@ -509,6 +548,8 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
         const float sh = valid ? shv : 0.0f;
         int angle_t;
+        // bit t set = timestep t of the tile may not use the lane polynomials (the same mask in every wave: the same 64 timesteps)
+        const unsigned long long notpoly = __builtin_amdgcn_ballot_w64(!sg2_poly_ok(kpoly_g, kpoly_s, g, sh));
         {
             // the same 64 timesteps in every wave of the workgroup: the same decision without talking to one another
             const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
@@ -571,19 +612,19 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
                 }
             }
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
-            if (!OUT && lite) {
-                if ((nottiny & blk) == 0)
-                    block_steps<HP, OUT, 2, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+            auto steps = [&](auto lite_c) {
+                constexpr bool LT = decltype(lite_c)::value;
+                if ((notpoly & blk) == 0)
+                    block_steps<HP, OUT, 3, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+                else if ((nottiny & blk) == 0)
+                    block_steps<HP, OUT, 2, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
                 else if ((large & blk) == 0)
-                    block_steps<HP, OUT, 1, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+                    block_steps<HP, OUT, 1, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
                 else
-                    block_steps<HP, OUT, 0, true>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
-            } else if ((nottiny & blk) == 0)
-                block_steps<HP, OUT, 2>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
-            else if ((large & blk) == 0)
-                block_steps<HP, OUT, 1>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
-            else
-                block_steps<HP, OUT, 0>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, tcoef, y);
+                    block_steps<HP, OUT, 0, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+            };
+            if (!OUT && lite) steps(std::true_type{});
+            else steps(std::false_type{});
             if (OUT && (p & 3) == 0) {       // the first lane of every bank holds the totals of its bank's steps (block_pair_sums)
                 if constexpr (HP == 8)
                     *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + 4 * (p >> 2)]) = f32x4{y[0], y[1], y[2], y[3]};
