@@ -70,6 +70,9 @@
  * the zero-input arguments (sg2_softplus_taylor / sg2_silu_taylor in include/sg2_compose.h: within a fraction of an
  * fp32 ulp of the functions, tests/test_oracle_primitives.py); other tiles take the functions themselves.  The
  * float64 policy always takes the functions.
+ * A block of 8 steps whose timesteps all pass sg2_poly_ok takes A_bar, sin and cos of every (j,p) from polynomials in
+ * dt - dt0 (dt0 = the column's step size for a zero input; sg2_abar_poly, sg2_sincos_poly), before the tiny-angle
+ * and shared-reciprocal forms are considered (fp32 policy only).
  * A (j,p) whose M is exactly zero hands on b itself as the next start state
  * (not 0 * h + b, which differs for a non-finite h): the kernels read no
  * earlier state at all when every summary of a call is of that kind.

@@ -51,6 +51,9 @@
 // the block is below 0.3 a shorter polynomial pair is used (sg_sincos_tiny,
 // not bit-identical to the general form: the choice depends on the angles only
 // and the CPU checker makes the same one).
+// Where the inputs are small (the usual case: sg2_taylor_ok, sg2_poly_ok in sg2_compose.h) the step size and the gate
+// of a tile come from cubic Taylor polynomials around their zero-input arguments, and A_bar, sin and cos of a block
+// from per-lane polynomials in dt - dt0; the forms above serve the remaining tiles and blocks.
 // For the bilevel pass k_scan<true, true> also stores the state entering every
 // 32nd step (Plan::htile), which the adjoint kernels restart from.
 #include <type_traits>
