@@ -42,6 +42,10 @@ def load(path):
     for f in (L.orc_softplus_taylor, L.orc_silu_taylor):
         f.restype = C.c_float
         f.argtypes = [C.c_float, C.c_float]
+    L.orc_abar_poly.restype = C.c_float
+    L.orc_abar_poly.argtypes = [C.c_float, C.c_float, C.c_float]
+    L.orc_sincos_poly.restype = C.c_float
+    L.orc_sincos_poly.argtypes = [C.c_float, C.c_float, C.c_float, C.c_int]
     L.orc_contraction_steps.restype = C.c_int
     L.orc_contraction_steps.argtypes = [C.c_float, C.c_float, C.c_float]
     L.orc_f_to_f16.restype = C.c_uint16

@@ -223,3 +223,24 @@ def test_contraction_steps_bound_the_decay():
         m = max(abs((1 + dt * A / 2) / (1 - dt * A / 2)) for A in (Ae, Ao))
         assert n > 0 and m ** n < 2.0 ** -100 * 1.001 and m ** (n - 2) > 2.0 ** -100, (dt, Ae, Ao, n, m)
     assert L.orc_contraction_steps(1e-6, -0.5 * -1e-3, -0.5 * -1e-3) == 0
+
+
+def test_recurrence_coefficients_as_polynomials_in_dt():
+    """A_bar(dt) = (1 - a dt)/(1 + a dt) as a cubic and sin/cos(f dt) as quadratics in d = dt - dt0, inside the limits a
+    block has to meet (a |d| < 2^-7, |f d| < 2^-8): within an fp32 rounding or two of the closed forms (float64).  A
+    coefficient with a wrong sign or factor is off by (a d)^k of order 1e-2 .. 1e-7 relative."""
+    r = np.random.RandomState(9)
+    worst = 0.0
+    for _ in range(4000):
+        dt0 = float(np.float32(r.uniform(0.01, 3.0)))
+        a = float(np.float32(np.exp(r.uniform(-4.0, 2.2))))          # -A/2 from 0.018 to 9
+        f = float(np.float32(r.uniform(-1.0, 1.0)))
+        lim = min(2.0 ** -7 / a, 2.0 ** -8 / max(abs(f), 1e-3), dt0)
+        d = float(np.float32(r.uniform(-1.0, 1.0) * lim))
+        dt = dt0 + d
+        exact = (1.0 - a * dt) / (1.0 + a * dt)
+        # (2 r - 1 cancels where a dt is close to 1, exactly as in sg_abar_pair: an absolute floor of one rounding of r)
+        worst = max(worst, abs(L.orc_abar_poly(dt0, a, d) - exact) / (4e-7 * abs(exact) + 1.5e-7))
+        worst = max(worst, abs(L.orc_sincos_poly(dt0, f, d, 0) - math.sin(f * dt)) / (4e-7 * abs(math.sin(f * dt)) + 3e-8))
+        worst = max(worst, abs(L.orc_sincos_poly(dt0, f, d, 1) - math.cos(f * dt)) / (4e-7 + 3e-8))
+    assert worst <= 1.0, worst
