@@ -461,18 +461,20 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const int j = tid / HP, p = tid % HP;                                 // scan role
 
     // -A/2 with A = -exp(A_log): the two poles of this lane's pair
-    const float hAe = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]);
-    const float hAo = -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]);
-    const float freq = pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p];
+    // (formed again from the weights wherever a block or a ragged end needs them: the usual blocks run on the lane
+    // polynomials below, and three registers held for the exceptions would spill)
+    auto pole_e = [&]() { return -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p]); };
+    auto pole_o = [&]() { return -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]); };
+    auto rope_f = [&]() { return pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p]; };
     // this lane's pair as polynomials in dt - dt0, dt0 = the step size of its column for a zero input
     LanePoly LP;
     LP.dt0 = pl.comp[2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4 + j * 4];
-    sg2_abar_poly(LP.dt0, hAe, LP.pe);
-    sg2_abar_poly(LP.dt0, hAo, LP.po);
-    sg2_sincos_poly(LP.dt0, freq, LP.qs, LP.qc);
+    sg2_abar_poly(LP.dt0, pole_e(), LP.pe);
+    sg2_abar_poly(LP.dt0, pole_o(), LP.po);
+    sg2_sincos_poly(LP.dt0, rope_f(), LP.qs, LP.qc);
 
     {   // largest |frequency| of each column's pairs
-        const float f = pair_tree_max<HP>(sg_abs(freq));
+        const float f = pair_tree_max<HP>(sg_abs(rope_f()));
         if (p == 0) s_fmax[j] = f;
         stage_coefficients<G, OUT>(pl.comp + dir * (SG2_COMP_GROUPS * G::ROWS * 3), pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4,
                                    pl.W.w[dir ? W_B_D : W_F_D], tid, s_dt, s_ux, s_dx, s_B, s_C, s_gate, s_tay);
@@ -618,13 +620,13 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             auto steps = [&](auto lite_c) {
                 constexpr bool LT = decltype(lite_c)::value;
                 if ((notpoly & blk) == 0)
-                    block_steps<HP, OUT, 3, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+                    block_steps<HP, OUT, 3, LT>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
                 else if ((nottiny & blk) == 0)
-                    block_steps<HP, OUT, 2, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+                    block_steps<HP, OUT, 2, LT>(S, dt, xv, Be, Bo, Ce, Co, pole_e(), pole_o(), rope_f(), LP, y);
                 else if ((large & blk) == 0)
-                    block_steps<HP, OUT, 1, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+                    block_steps<HP, OUT, 1, LT>(S, dt, xv, Be, Bo, Ce, Co, pole_e(), pole_o(), rope_f(), LP, y);
                 else
-                    block_steps<HP, OUT, 0, LT>(S, dt, xv, Be, Bo, Ce, Co, hAe, hAo, freq, LP, y);
+                    block_steps<HP, OUT, 0, LT>(S, dt, xv, Be, Bo, Ce, Co, pole_e(), pole_o(), rope_f(), LP, y);
             };
             if (!OUT && lite) steps(std::true_type{});
             else steps(std::false_type{});
@@ -639,8 +641,8 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
             const float dt = r_dt[k0], ux = r_ux[k0];
             float ae, ao, sn, cs;
-            sg_abar_pair(dt, hAe, hAo, &ae, &ao);
-            sg_sincos(dt * freq, &sn, &cs);
+            sg_abar_pair(dt, pole_e(), pole_o(), &ae, &ao);
+            sg_sincos(dt * rope_f(), &sn, &cs);
             if (!OUT && lite) step_update<OUT, true>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             else step_update<OUT>(S, ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
             if (OUT) {
