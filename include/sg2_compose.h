@@ -136,6 +136,31 @@ SG_HD int sg2_poly_ok(float kpoly_g, float kpoly_s, float g, float s) {
     return sg_fma(kpoly_g, sg_abs(g), kpoly_s * sg_abs(s)) < 1.0f;
 }
 
+/* The output pass goes one step further: its update h' = D R h + b needs only the four products of the pair,
+ * P1 = A_bar_e cos, N2 = -A_bar_e sin, P3 = A_bar_o cos, P4 = A_bar_o sin, and takes those as quadratics in d = dt - dt0
+ * (products of the series above, truncated): he' = P1 he + N2 ho + b_e, ho' = P3 ho + P4 he + b_o, four fma instead of
+ * two multiplications and four fma, and four quadratics instead of two cubics and two quadratics.  The truncated terms
+ * are bounded by ((2.3 a + |f|) d)^3 / 6; a block uses the products when kprod_g |g| + kprod_s |s| < 1 for each of its
+ * timesteps, kprod = (416 a_max + 184 f_max) times the largest |c_g|, |c_s| of the dt rows: (2.3 a + |f|) d < 2^-7.5,
+ * remainder below 3e-8. */
+SG_HD void sg2_prod_poly(const float a[3], const float c[3], float k[3]) {
+    k[0] = a[0] * c[0];
+    k[1] = sg_fma(a[0], c[1], a[1] * c[0]);
+    k[2] = sg_fma(a[0], c[2], sg_fma(a[1], c[1], a[2] * c[0]));
+}
+/* k: [P1 | N2 | P3 | P4][3] of the pair with poles nhA_e, nhA_o and rotation frequency f */
+SG_HD void sg2_pair_products(float dt0, float nhA_e, float nhA_o, float f, float k[12]) {
+    float pe[4], po[4], qs[3], qc[3], ns[3];
+    sg2_abar_poly(dt0, nhA_e, pe);
+    sg2_abar_poly(dt0, nhA_o, po);
+    sg2_sincos_poly(dt0, f, qs, qc);
+    ns[0] = -qs[0]; ns[1] = -qs[1]; ns[2] = -qs[2];
+    sg2_prod_poly(pe, qc, k);
+    sg2_prod_poly(pe, ns, k + 3);
+    sg2_prod_poly(po, qc, k + 6);
+    sg2_prod_poly(po, qs, k + 9);
+}
+
 /* value of a composed output for one element */
 SG_HD float sg2_comp_eval(const float* c, float g, float s) { return sg_fma(c[0], g, sg_fma(c[1], s, c[2])); }
 

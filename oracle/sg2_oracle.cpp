@@ -72,7 +72,8 @@
  * float64 policy always takes the functions.
  * A block of 8 steps whose timesteps all pass sg2_poly_ok takes A_bar, sin and cos of every (j,p) from polynomials in
  * dt - dt0 (dt0 = the column's step size for a zero input; sg2_abar_poly, sg2_sincos_poly), before the tiny-angle
- * and shared-reciprocal forms are considered (fp32 policy only).
+ * and shared-reciprocal forms are considered (fp32 policy only).  The replay uses, with a tighter limit, quadratics
+ * for the four products of its update instead (sg2_pair_products): he' = P1 he + N2 ho + b_e, ho' = P3 ho + P4 he + b_o.
  * A (j,p) whose M is exactly zero hands on b itself as the next start state
  * (not 0 * h + b, which differs for a non-finite h): the kernels read no
  * earlier state at all when every summary of a call is of that kind.
@@ -252,6 +253,10 @@ struct DirW {
      * [lane][pe 4 | po 4 | qs 3 | qc 3], and the two factors of sg2_poly_ok */
     std::vector<float> lane_poly;
     float kpoly[2];
+    /* the output pass: the four products of every (column, pair) as quadratics, [lane][P1 | N2 | P3 | P4][3]
+     * (sg2_pair_products), and the factors of their limit */
+    std::vector<float> lane_prod;
+    float kprod[2];
 };
 
 template <class O>
@@ -320,6 +325,8 @@ template <class O>
 struct TileCoef {
     std::vector<StepProj<O>> sp;
     std::vector<typename O::R> ae, ao, sn, cs;
+    /* output pass: blocks of 8 steps that hold the products instead (ae = P1, sn = N2, ao = P3, cs = P4) */
+    std::vector<char> prod_block;
 };
 enum { ORC_TILE = 64, ORC_BLOCK = 8, ORC_WAVE = 64 };
 
@@ -347,17 +354,33 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
                 O::sincos(tc.sp[k].dt[j] * (R)w.rope[j * hp + p], &tc.sn[(size_t)k * lanes + j * hp + p],
                           &tc.cs[(size_t)k * lanes + j * hp + p]);
     }
-    /* blocks of 8 steps whose timesteps all pass sg2_poly_ok take A_bar, sin and cos from the lane polynomials */
+    /* blocks of 8 steps whose timesteps all pass sg2_poly_ok take A_bar, sin and cos from the lane polynomials (summary
+     * pass) or, with the tighter limit of the output pass (need_zc), the four products of the update */
     std::vector<char> poly_block(ORC_TILE / ORC_BLOCK, 0);
+    tc.prod_block.assign(ORC_TILE / ORC_BLOCK, 0);
     if (sizeof(R) == 4) {
+        const float* lim = need_zc ? w.kprod : w.kpoly;
         for (int b0 = 0; b0 + ORC_BLOCK <= cnt; b0 += ORC_BLOCK) {
             bool ok = true;
             for (int q = 0; q < ORC_BLOCK && ok; q++) {
                 const int64_t u = u0 + b0 + q, t = reverse ? (N - 1 - u) : u;
-                ok = sg2_poly_ok(w.kpoly[0], w.kpoly[1], gs[2 * t], gs[2 * t + 1]) != 0;
+                ok = sg2_poly_ok(lim[0], lim[1], gs[2 * t], gs[2 * t + 1]) != 0;
             }
             poly_block[b0 / ORC_BLOCK] = ok;
             if (!ok) continue;
+            if (need_zc) {
+                tc.prod_block[b0 / ORC_BLOCK] = 1;
+                for (int q = 0; q < ORC_BLOCK; q++)
+                    for (int l = 0; l < lanes; l++) {
+                        const float* k = &w.lane_prod[(size_t)l * 12];
+                        const float dd = (float)tc.sp[b0 + q].dt[l / hp] - w.tay[((size_t)0 * w.comp_rows + l / hp) * 4];
+                        tc.ae[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k, dd);
+                        tc.sn[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 3, dd);
+                        tc.ao[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 6, dd);
+                        tc.cs[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 9, dd);
+                    }
+                continue;
+            }
             for (int q = 0; q < ORC_BLOCK; q++)
                 for (int l = 0; l < lanes; l++) {
                     const float* lp = &w.lane_poly[(size_t)l * 14];
@@ -590,9 +613,16 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
                         const R ae = tc.ae[li], ao = tc.ao[li], sn = tc.sn[li], cs = tc.cs[li];
                         const R ux = dt * xb, be = ux * sp.B[2 * p], bo = ux * sp.B[2 * p + 1];
                         const R he = hc[j * ds + 2 * p], ho = hc[j * ds + 2 * p + 1];
-                        const R re = O::fma(he, cs, -(ho * sn));
-                        const R ro = O::fma(ho, cs, he * sn);
-                        const R ne = O::fma(ae, re, be), no = O::fma(ao, ro, bo);
+                        R ne, no;
+                        if (tc.prod_block[k / ORC_BLOCK]) {      /* ae = P1, sn = N2, ao = P3, cs = P4 */
+                            ne = O::fma(ae, he, O::fma(sn, ho, be));
+                            no = O::fma(ao, ho, O::fma(cs, he, bo));
+                        } else {
+                            const R re = O::fma(he, cs, -(ho * sn));
+                            const R ro = O::fma(ho, cs, he * sn);
+                            ne = O::fma(ae, re, be);
+                            no = O::fma(ao, ro, bo);
+                        }
                         hc[j * ds + 2 * p] = ne;
                         hc[j * ds + 2 * p + 1] = no;
                         yp[p] = O::fma(no, sp.C[2 * p + 1], ne * sp.C[2 * p]);
@@ -676,7 +706,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
     std::vector<R> hst[2];
     for (int dir = 0; dir < 2; dir++) {
         const int b = dir ? W_B_INPROJ : W_F_INPROJ;
-        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0, {}, {0.0f, 0.0f}, {}, {0.0f, 0.0f}};
+        DirW<O> w = {W[b], W[b + 1], W[b + 2], W[b + 3], W[b + 4], W[b + 5], W[b + 6], W[b + 7], W[b + 8], {}, 0, {}, {0.0f, 0.0f}, {}, {0.0f, 0.0f}, {}, {0.0f, 0.0f}};
         if (sizeof(R) == 4) {
             w.comp_rows = std::max(di, ds);
             w.comp.assign((size_t)SG2_COMP_GROUPS * w.comp_rows * 3, 0.0f);
@@ -697,6 +727,7 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
             const int hp = ds / 2;
             float amax = 0.0f, fmax = 0.0f, cdt[2] = {0.0f, 0.0f};
             w.lane_poly.assign((size_t)di * hp * 14, 0.0f);
+            w.lane_prod.assign((size_t)di * hp * 12, 0.0f);
             for (int j = 0; j < di; j++) {
                 const float* cd = &w.comp[((size_t)SG2_COMP_DT * w.comp_rows + j) * 3];
                 cdt[0] = sg_max(cdt[0], sg_abs(cd[0]));
@@ -711,11 +742,15 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
                     sg2_abar_poly(dt0, a_e, lp);
                     sg2_abar_poly(dt0, a_o, lp + 4);
                     sg2_sincos_poly(dt0, f, lp + 8, lp + 11);
+                    sg2_pair_products(dt0, a_e, a_o, f, &w.lane_prod[((size_t)j * hp + p) * 12]);
                 }
             }
             const float kp = sg_max(128.0f * amax, 256.0f * fmax);
             w.kpoly[0] = kp * cdt[0];
             w.kpoly[1] = kp * cdt[1];
+            const float kq = sg_fma(416.0f, amax, 184.0f * fmax);
+            w.kprod[0] = kq * cdt[0];
+            w.kprod[1] = kq * cdt[1];
         }
         float* st = dir ? mbwd_io : mfwd_io;
         hst[dir].assign(st, st + di * ds);

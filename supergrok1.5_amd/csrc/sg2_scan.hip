@@ -238,6 +238,10 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
             const float kp = sg_max(128.0f * sg_i2f(s_amax[k]), 256.0f * sg_i2f(s_fmax[k]));
             cmax[4 + 2 * k] = kp * sg_i2f(s_cdt[k][0]);
             cmax[5 + 2 * k] = kp * sg_i2f(s_cdt[k][1]);
+            // ... and for the products of the output pass (sg2_pair_products)
+            const float kq = sg_fma(416.0f, sg_i2f(s_amax[k]), 184.0f * sg_i2f(s_fmax[k]));
+            cmax[8 + 2 * k] = kq * sg_i2f(s_cdt[k][0]);
+            cmax[9 + 2 * k] = kq * sg_i2f(s_cdt[k][1]);
         }
     }
 }
@@ -347,8 +351,14 @@ struct LaneState {
     float he, ho, c0e, c0o, c1e, c1o;
 };
 // the lane's pair as polynomials in dt - dt0 (sg2_abar_poly, sg2_sincos_poly): dt0 = step size of its column for a zero input
+// The summary pass keeps A_bar and sin/cos apart (its bound needs the A_bar); the output pass holds the four products.
+template <bool OUT>
 struct LanePoly {
     float dt0, pe[4], po[4], qs[3], qc[3];
+};
+template <>
+struct LanePoly<true> {
+    float dt0, k[12];
 };
 
 // LITE (summary pass only): the state part alone, and in c0e the running product of max(|A_bar_e|, |A_bar_o|), a bound
@@ -379,9 +389,19 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 template <int HP, bool OUT, int ANGLE, bool LITE = false>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
-                                            float hAo, float freq, const LanePoly& LP, float (&y)[UB]) {
+                                            float hAo, float freq, const LanePoly<OUT>& LP, float (&y)[UB]) {
     float ae[UB], ao[UB], sn[UB], cs[UB], be[UB], bo[UB];
-    if (ANGLE == 3) {
+    if constexpr (ANGLE == 3 && OUT) {
+        // the four products of the update as quadratics: ae = P1, sn = N2, ao = P3, cs = P4 (see the update below)
+#pragma unroll
+        for (int u = 0; u < UB; u++) {
+            const float d = dt[u] - LP.dt0;
+            ae[u] = sg2_poly2(LP.k, d);
+            sn[u] = sg2_poly2(LP.k + 3, d);
+            ao[u] = sg2_poly2(LP.k + 6, d);
+            cs[u] = sg2_poly2(LP.k + 9, d);
+        }
+    } else if constexpr (ANGLE == 3) {
 #pragma unroll
         for (int u = 0; u < UB; u++) {
             const float d = dt[u] - LP.dt0;
@@ -412,7 +432,13 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     }
 #pragma unroll
     for (int u = 0; u < UB; u++) {
-        step_update<OUT, LITE>(S, ae[u], ao[u], sn[u], cs[u], be[u], bo[u]);
+        if constexpr (ANGLE == 3 && OUT) {
+            const float he = sg_fma(ae[u], S.he, sg_fma(sn[u], S.ho, be[u]));      // P1 he + N2 ho + b_e
+            S.ho = sg_fma(ao[u], S.ho, sg_fma(cs[u], S.he, bo[u]));                // P3 ho + P4 he + b_o
+            S.he = he;
+        } else {
+            step_update<OUT, LITE>(S, ae[u], ao[u], sn[u], cs[u], be[u], bo[u]);
+        }
         if (OUT) y[u] = sg_fma(S.ho, Co[u], S.he * Ce[u]);
     }
     if (OUT) {
@@ -467,11 +493,15 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     auto pole_o = [&]() { return -0.5f * -sg_exp(pl.W.w[dir ? W_B_ALOG : W_F_ALOG][j * DS + 2 * p + 1]); };
     auto rope_f = [&]() { return pl.W.w[dir ? W_B_ROPE : W_F_ROPE][j * HP + p]; };
     // this lane's pair as polynomials in dt - dt0, dt0 = the step size of its column for a zero input
-    LanePoly LP;
+    LanePoly<OUT> LP;
     LP.dt0 = pl.comp[2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4 + j * 4];
-    sg2_abar_poly(LP.dt0, pole_e(), LP.pe);
-    sg2_abar_poly(LP.dt0, pole_o(), LP.po);
-    sg2_sincos_poly(LP.dt0, rope_f(), LP.qs, LP.qc);
+    if constexpr (OUT) {
+        sg2_pair_products(LP.dt0, pole_e(), pole_o(), rope_f(), LP.k);
+    } else {
+        sg2_abar_poly(LP.dt0, pole_e(), LP.pe);
+        sg2_abar_poly(LP.dt0, pole_o(), LP.po);
+        sg2_sincos_poly(LP.dt0, rope_f(), LP.qs, LP.qc);
+    }
 
     {   // largest |frequency| of each column's pairs
         const float f = pair_tree_max<HP>(sg_abs(rope_f()));
@@ -486,8 +516,9 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     const float cmax_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir];
     const float cmax_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 2 * dir + 1];
     // ... and whether a block of the recurrence may use the lane polynomials (sg2_poly_ok)
-    const float kpoly_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 4 + 2 * dir];
-    const float kpoly_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + 4 + 2 * dir + 1];
+    // (the output pass with the tighter limit of its products)
+    const float kpoly_g = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + (OUT ? 8 : 4) + 2 * dir];
+    const float kpoly_s = sg::as_const(pl.comp)[2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4 + (OUT ? 8 : 4) + 2 * dir + 1];
 
     LaneState S = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
     bool fully_contracted = false;      // summary pass: the walk stopped because the 2x2 part had contracted

@@ -95,7 +95,7 @@ int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bi
     L->off_blocksums = take(4 * (size_t)(L->nb + 1));
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * gi.threads);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
-    L->off_comp = take(4 * (2 * 5 * (size_t)gi.rows * 3 + 2 * 2 * (size_t)gi.rows * 4 + 8));      // composed triples, Taylor polynomials, coefficient maxima and polynomial limits
+    L->off_comp = take(4 * (2 * 5 * (size_t)gi.rows * 3 + 2 * 2 * (size_t)gi.rows * 4 + 12));      // composed triples, Taylor polynomials, coefficient maxima and polynomial limits
     L->off_flags = take(4 * ((size_t)P + 2));        // apart from the tensor records: it is written while those are being read
     L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions

@@ -145,8 +145,14 @@ MUTANTS = [
     ("clamp_wraps", "if (e >= E) e = E - 1;", "if (e >= E) e = e % E;", lambda run: pins.check_expert_index_clamp(run, 2e-5)),
     ("relu_dropped", "zv = zv > 0 ? zv : (R)0;", "zv = zv;", lambda run: pins.check_expert_mlp_by_hand(run, 2e-5)),
     ("expert_bias_dropped", "R ho = W[W_EXP_B2][e];", "R ho = 0;", lambda run: pins.check_expert_mlp_by_hand(run, 2e-5)),
-    ("rotation_reversed", "const R re = O::fma(he, cs, -(ho * sn));\n                        const R ro = O::fma(ho, cs, he * sn);",
-     "const R re = O::fma(he, cs, ho * sn);\n                        const R ro = O::fma(ho, cs, -(he * sn));",
+    # (both forms of the replay's update: the products of the polynomial blocks and the plain rotation)
+    ("rotation_reversed",
+     "ne = O::fma(ae, he, O::fma(sn, ho, be));\n                            no = O::fma(ao, ho, O::fma(cs, he, bo));\n"
+     "                        } else {\n                            const R re = O::fma(he, cs, -(ho * sn));\n"
+     "                            const R ro = O::fma(ho, cs, he * sn);",
+     "ne = O::fma(ae, he, O::fma(-sn, ho, be));\n                            no = O::fma(ao, ho, O::fma(-cs, he, bo));\n"
+     "                        } else {\n                            const R re = O::fma(he, cs, ho * sn);\n"
+     "                            const R ro = O::fma(ho, cs, -(he * sn));",
      lambda run: pins.check_rotation_sense(run, 4e-4)),
 ]
 
