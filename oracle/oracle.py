@@ -46,6 +46,8 @@ def load(path):
     L.orc_abar_poly.argtypes = [C.c_float, C.c_float, C.c_float]
     L.orc_sincos_poly.restype = C.c_float
     L.orc_sincos_poly.argtypes = [C.c_float, C.c_float, C.c_float, C.c_int]
+    L.orc_pair_product.restype = C.c_float
+    L.orc_pair_product.argtypes = [C.c_float] * 5 + [C.c_int]
     L.orc_contraction_steps.restype = C.c_int
     L.orc_contraction_steps.argtypes = [C.c_float, C.c_float, C.c_float]
     L.orc_f_to_f16.restype = C.c_uint16

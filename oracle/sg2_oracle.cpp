@@ -921,6 +921,11 @@ float orc_softplus_taylor(float c, float d) { float t[4]; sg2_softplus_taylor(c,
 float orc_silu_taylor(float c, float d) { float t[4]; sg2_silu_taylor(c, t); return sg2_taylor_eval(t, d); }
 float orc_abar_poly(float dt0, float nhA, float d) { float p[4]; sg2_abar_poly(dt0, nhA, p); return sg2_poly3(p, d); }
 float orc_sincos_poly(float dt0, float f, float d, int cosine) { float qs[3], qc[3]; sg2_sincos_poly(dt0, f, qs, qc); return sg2_poly2(cosine ? qc : qs, d); }
+float orc_pair_product(float dt0, float nhA_e, float nhA_o, float f, float d, int which) {
+    float k[12];
+    sg2_pair_products(dt0, nhA_e, nhA_o, f, k);
+    return sg2_poly2(k + 3 * which, d);
+}
 int orc_contraction_steps(float dt0, float nhA_e, float nhA_o) { return sg2_contraction_steps(dt0, nhA_e, nhA_o); }
 float orc_tanh(float x) { return sg_tanh(x); }
 float orc_sin(float x) { float s, c; sg_sincos(x, &s, &c); return s; }

@@ -244,3 +244,24 @@ def test_recurrence_coefficients_as_polynomials_in_dt():
         worst = max(worst, abs(L.orc_sincos_poly(dt0, f, d, 0) - math.sin(f * dt)) / (4e-7 * abs(math.sin(f * dt)) + 3e-8))
         worst = max(worst, abs(L.orc_sincos_poly(dt0, f, d, 1) - math.cos(f * dt)) / (4e-7 + 3e-8))
     assert worst <= 1.0, worst
+
+
+def test_update_products_as_quadratics_in_dt():
+    """The four products of the replay's update, A_bar_e cos, -A_bar_e sin, A_bar_o cos, A_bar_o sin (of f dt), as
+    quadratics in d = dt - dt0 inside the limit a block has to meet, (2.3 a + |f|) |d| < 2^-7.5: within an fp32 rounding
+    or two of the closed forms (float64).  A sign or a dropped cross term shows at first or second order in d."""
+    r = np.random.RandomState(10)
+    worst = 0.0
+    for _ in range(4000):
+        dt0 = float(np.float32(r.uniform(0.01, 3.0)))
+        ae, ao = (float(np.float32(np.exp(r.uniform(-4.0, 2.2)))) for _ in range(2))
+        f = float(np.float32(r.uniform(-1.0, 1.0)))
+        lim = min(2.0 ** -7.5 / (2.3 * max(ae, ao) + abs(f)), dt0)
+        d = float(np.float32(r.uniform(-1.0, 1.0) * lim))
+        dt = dt0 + d
+        A = [(1.0 - a * dt) / (1.0 + a * dt) for a in (ae, ao)]
+        want = (A[0] * math.cos(f * dt), -A[0] * math.sin(f * dt), A[1] * math.cos(f * dt), A[1] * math.sin(f * dt))
+        for which in range(4):
+            got = L.orc_pair_product(dt0, ae, ao, f, d, which)
+            worst = max(worst, abs(got - want[which]) / (4e-7 * abs(want[which]) + 2e-7))
+    assert worst <= 1.0, worst
