@@ -260,7 +260,10 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
 // is spread over the fourth padding floats of rows j of s_dt, s_B, s_C and s_gate, which this wave reads anyway
 // (d_inner = d_state: the wave's columns and its rows of B and C carry the same indices).  The summary pass has
 // no s_dx and keeps the step-size polynomials in s_tay.
-template <class G, bool OUT, int PART, bool HAS_S, bool TAYLOR>
+// DSTORE (with TAYLOR, whole tiles whose blocks all run on the lane polynomials): the step-size row receives dt - dt0,
+// which is all those blocks want to know (one subtraction per column here instead of one per pair in the recurrence),
+// and nobody asks for the angle flags.
+template <class G, bool OUT, int PART, bool HAS_S, bool TAYLOR, bool DSTORE = false>
 __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_dt, float* s_ux, float* s_dx, float* s_B,
                                              float* s_C, float* s_gate, const float* s_fmax, const float* s_tay) {
     static_assert(G::DI == G::DS, "the gate polynomials ride on the rows of B and C");
@@ -277,15 +280,22 @@ __device__ __forceinline__ int project_tile(float g, float s, int tu, float* s_d
         const int jj = PART * NR + q;
         const f32x4 cd = coef(s_dt, jj);
         gp0[q] = cd[3];
-        float dtv;
-        if (TAYLOR) dtv = poly(OUT ? coef(s_dx, jj) : *reinterpret_cast<const f32x4*>(s_tay + jj * 4), delta(cd));
-        else dtv = sg_softplus(eval(cd));
-        const float amax = dtv * s_fmax[jj];
-        small = small && (amax < SG_SINCOS_SMALL_LIMIT);
-        tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
+        float dtv, dt0 = 0.0f;
+        if (TAYLOR) {
+            const f32x4 tp = OUT ? coef(s_dx, jj) : *reinterpret_cast<const f32x4*>(s_tay + jj * 4);
+            dtv = poly(tp, delta(cd));
+            dt0 = tp[0];
+        } else {
+            dtv = sg_softplus(eval(cd));
+        }
+        if (!DSTORE) {
+            const float amax = dtv * s_fmax[jj];
+            small = small && (amax < SG_SINCOS_SMALL_LIMIT);
+            tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
+        }
         const f32x4 cx = coef(s_ux, jj);              // x-branch coefficients; [3] = D of this column
         const float xbv = eval(cx);
-        s_dt[jj * LDS_STRIDE + tu] = dtv;
+        s_dt[jj * LDS_STRIDE + tu] = DSTORE ? dtv - dt0 : dtv;
         s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
         if (OUT) s_dx[jj * LDS_STRIDE + tu] = cx[3] * xbv;
     }
@@ -386,7 +396,8 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
 // ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values, polynomials in dt),
 // 3: every timestep of the block has passed sg2_poly_ok: A_bar, sin and cos from the lane's polynomials in dt - dt0.
-template <int HP, bool OUT, int ANGLE, bool LITE = false>
+// DGIVEN (ANGLE 3 only): dt[] holds dt - dt0 already (project_tile's DSTORE).
+template <int HP, bool OUT, int ANGLE, bool LITE = false, bool DGIVEN = false>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, const LanePoly<OUT>& LP, float (&y)[UB]) {
@@ -395,7 +406,7 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
         // the four products of the update as quadratics: ae = P1, sn = N2, ao = P3, cs = P4 (see the update below)
 #pragma unroll
         for (int u = 0; u < UB; u++) {
-            const float d = dt[u] - LP.dt0;
+            const float d = DGIVEN ? dt[u] : dt[u] - LP.dt0;
             ae[u] = sg2_poly2(LP.k, d);
             sn[u] = sg2_poly2(LP.k + 3, d);
             ao[u] = sg2_poly2(LP.k + 6, d);
@@ -404,7 +415,7 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
     } else if constexpr (ANGLE == 3) {
 #pragma unroll
         for (int u = 0; u < UB; u++) {
-            const float d = dt[u] - LP.dt0;
+            const float d = DGIVEN ? dt[u] : dt[u] - LP.dt0;
             ae[u] = sg2_poly3(LP.pe, d);
             ao[u] = sg2_poly3(LP.po, d);
             sn[u] = sg2_poly2(LP.qs, d);
@@ -584,15 +595,21 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
         const float sh = valid ? shv : 0.0f;
         int angle_t;
+        bool dgiven = false;     // whole tile on the lane polynomials: phase A leaves dt - dt0 in place of dt
         // bit t set = timestep t of the tile may not use the lane polynomials (the same mask in every wave: the same 64 timesteps)
         const unsigned long long notpoly = __builtin_amdgcn_ballot_w64(!sg2_poly_ok(kpoly_g, kpoly_s, g, sh));
         {
             // the same 64 timesteps in every wave of the workgroup: the same decision without talking to one another
             const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
+            dgiven = tay && notpoly == 0 && cnt == SCAN_TT;
             // PARTS == 2: the wave's share is a template parameter; more waves: one copy of the code, the arrays moved to this wave's first row
             const int rj = (PARTS == 2) ? 0 : half * (DI / PARTS) * LDS_STRIDE, rs = (PARTS == 2) ? 0 : half * (DS / PARTS) * LDS_STRIDE;
             const int rt = (PARTS == 2 || OUT) ? 0 : half * (DI / PARTS) * 4;
             auto run = [&](auto part_c, auto has_s_c, auto tay_c) {
+                if (decltype(tay_c)::value && dgiven)
+                    return project_tile<G, OUT, decltype(part_c)::value, decltype(has_s_c)::value, true, true>(
+                        g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0), s_gate + (OUT ? rj : 0),
+                        s_fmax + ((PARTS == 2) ? 0 : half * (DI / PARTS)), s_tay + rt);
                 return project_tile<G, OUT, decltype(part_c)::value, decltype(has_s_c)::value, decltype(tay_c)::value>(
                     g, sh, tu, s_dt + rj, s_ux + rj, s_dx + (OUT ? rj : 0), s_B + rs, s_C + (OUT ? rs : 0), s_gate + (OUT ? rj : 0),
                     s_fmax + ((PARTS == 2) ? 0 : half * (DI / PARTS)), s_tay + rt);
@@ -650,7 +667,9 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
             auto steps = [&](auto lite_c) {
                 constexpr bool LT = decltype(lite_c)::value;
-                if ((notpoly & blk) == 0)
+                if (dgiven)
+                    block_steps<HP, OUT, 3, LT, true>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
+                else if ((notpoly & blk) == 0)
                     block_steps<HP, OUT, 3, LT>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
                 else if ((nottiny & blk) == 0)
                     block_steps<HP, OUT, 2, LT>(S, dt, xv, Be, Bo, Ce, Co, pole_e(), pole_o(), rope_f(), LP, y);
