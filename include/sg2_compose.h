@@ -143,6 +143,10 @@ SG_HD int sg2_poly_ok(float kpoly_g, float kpoly_s, float g, float s) {
  * are bounded by ((2.3 a + |f|) d)^3 / 6; a block uses the products when kprod_g |g| + kprod_s |s| < 1 for each of its
  * timesteps, kprod = (416 a_max + 184 f_max) times the largest |c_g|, |c_s| of the dt rows: (2.3 a + |f|) d < 2^-7.5,
  * remainder below 3e-8. */
+/* Where the inputs are smaller still, kprod times 24 below 1, i.e. (2.3 a + |f|) d < 2^-12, the linear part alone is
+ * within 3e-8 (remainder ((2.3 a + |f|) d)^2 / 2): SG2_PROD_LINEAR_FACTOR. */
+#define SG2_PROD_LINEAR_FACTOR 24.0f
+SG_HD float sg2_poly1(const float* k, float d) { return sg_fma(k[1], d, k[0]); }
 SG_HD void sg2_prod_poly(const float a[3], const float c[3], float k[3]) {
     k[0] = a[0] * c[0];
     k[1] = sg_fma(a[0], c[1], a[1] * c[0]);

@@ -360,6 +360,12 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
     tc.prod_block.assign(ORC_TILE / ORC_BLOCK, 0);
     if (sizeof(R) == 4) {
         const float* lim = need_zc ? w.kprod : w.kpoly;
+        /* (the device knows before its projections whether the whole 64-step tile qualifies) */
+        bool whole_tile_poly = taylor && cnt == ORC_TILE;
+        for (int k = 0; k < cnt && whole_tile_poly; k++) {
+            const int64_t u = u0 + k, t = reverse ? (N - 1 - u) : u;
+            whole_tile_poly = sg2_poly_ok(lim[0], lim[1], gs[2 * t], gs[2 * t + 1]) != 0;
+        }
         for (int b0 = 0; b0 + ORC_BLOCK <= cnt; b0 += ORC_BLOCK) {
             bool ok = true;
             for (int q = 0; q < ORC_BLOCK && ok; q++) {
@@ -370,14 +376,21 @@ void tile_coefficients(const Dims& d, const DirW<O>& w, const std::vector<typena
             if (!ok) continue;
             if (need_zc) {
                 tc.prod_block[b0 / ORC_BLOCK] = 1;
+                /* the linear parts alone: a whole tile on Taylor step sizes and products, and this block's inputs
+                 * SG2_PROD_LINEAR_FACTOR times further inside the limit */
+                bool linear = whole_tile_poly;
+                for (int q = 0; q < ORC_BLOCK && linear; q++) {
+                    const int64_t u = u0 + b0 + q, t = reverse ? (N - 1 - u) : u;
+                    linear = sg2_poly_ok(SG2_PROD_LINEAR_FACTOR * lim[0], SG2_PROD_LINEAR_FACTOR * lim[1], gs[2 * t], gs[2 * t + 1]) != 0;
+                }
                 for (int q = 0; q < ORC_BLOCK; q++)
                     for (int l = 0; l < lanes; l++) {
                         const float* k = &w.lane_prod[(size_t)l * 12];
                         const float dd = (float)tc.sp[b0 + q].dt[l / hp] - w.tay[((size_t)0 * w.comp_rows + l / hp) * 4];
-                        tc.ae[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k, dd);
-                        tc.sn[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 3, dd);
-                        tc.ao[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 6, dd);
-                        tc.cs[(size_t)(b0 + q) * lanes + l] = (R)sg2_poly2(k + 9, dd);
+                        tc.ae[(size_t)(b0 + q) * lanes + l] = (R)(linear ? sg2_poly1(k, dd) : sg2_poly2(k, dd));
+                        tc.sn[(size_t)(b0 + q) * lanes + l] = (R)(linear ? sg2_poly1(k + 3, dd) : sg2_poly2(k + 3, dd));
+                        tc.ao[(size_t)(b0 + q) * lanes + l] = (R)(linear ? sg2_poly1(k + 6, dd) : sg2_poly2(k + 6, dd));
+                        tc.cs[(size_t)(b0 + q) * lanes + l] = (R)(linear ? sg2_poly1(k + 9, dd) : sg2_poly2(k + 9, dd));
                     }
                 continue;
             }

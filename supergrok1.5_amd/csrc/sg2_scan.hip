@@ -396,8 +396,9 @@ __device__ __forceinline__ void step_update(LaneState& S, float ae, float ao, fl
 // (sg_abar_block_*) unless some lane of the wave has a product of denominators too large for it.
 // ANGLE: 0 full sin/cos, 1 sg_sincos_small (bit-identical to 0), 2 sg_sincos_tiny_dt (its own values, polynomials in dt),
 // 3: every timestep of the block has passed sg2_poly_ok: A_bar, sin and cos from the lane's polynomials in dt - dt0.
-// DGIVEN (ANGLE 3 only): dt[] holds dt - dt0 already (project_tile's DSTORE).
-template <int HP, bool OUT, int ANGLE, bool LITE = false, bool DGIVEN = false>
+// DGIVEN (ANGLE 3 only): dt[] holds dt - dt0 already (project_tile's DSTORE).  LINEAR (output pass, ANGLE 3): the
+// inputs are small enough for the linear parts of the products.
+template <int HP, bool OUT, int ANGLE, bool LITE = false, bool DGIVEN = false, bool LINEAR = false>
 __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB], const float (&ux)[UB], const float (&Be)[UB],
                                             const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], float hAe,
                                             float hAo, float freq, const LanePoly<OUT>& LP, float (&y)[UB]) {
@@ -407,10 +408,10 @@ __device__ __forceinline__ void block_steps(LaneState& S, const float (&dt)[UB],
 #pragma unroll
         for (int u = 0; u < UB; u++) {
             const float d = DGIVEN ? dt[u] : dt[u] - LP.dt0;
-            ae[u] = sg2_poly2(LP.k, d);
-            sn[u] = sg2_poly2(LP.k + 3, d);
-            ao[u] = sg2_poly2(LP.k + 6, d);
-            cs[u] = sg2_poly2(LP.k + 9, d);
+            ae[u] = LINEAR ? sg2_poly1(LP.k, d) : sg2_poly2(LP.k, d);
+            sn[u] = LINEAR ? sg2_poly1(LP.k + 3, d) : sg2_poly2(LP.k + 3, d);
+            ao[u] = LINEAR ? sg2_poly1(LP.k + 6, d) : sg2_poly2(LP.k + 6, d);
+            cs[u] = LINEAR ? sg2_poly1(LP.k + 9, d) : sg2_poly2(LP.k + 9, d);
         }
     } else if constexpr (ANGLE == 3) {
 #pragma unroll
@@ -598,6 +599,9 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
         bool dgiven = false;     // whole tile on the lane polynomials: phase A leaves dt - dt0 in place of dt
         // bit t set = timestep t of the tile may not use the lane polynomials (the same mask in every wave: the same 64 timesteps)
         const unsigned long long notpoly = __builtin_amdgcn_ballot_w64(!sg2_poly_ok(kpoly_g, kpoly_s, g, sh));
+        // ... may not use the linear parts alone (output pass)
+        const unsigned long long notlin =
+            OUT ? __builtin_amdgcn_ballot_w64(!sg2_poly_ok(SG2_PROD_LINEAR_FACTOR * kpoly_g, SG2_PROD_LINEAR_FACTOR * kpoly_s, g, sh)) : ~0ull;
         {
             // the same 64 timesteps in every wave of the workgroup: the same decision without talking to one another
             const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
@@ -667,7 +671,9 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
             const unsigned long long blk = ((1ull << UB) - 1) << k0;
             auto steps = [&](auto lite_c) {
                 constexpr bool LT = decltype(lite_c)::value;
-                if (dgiven)
+                if (OUT && dgiven && (notlin & blk) == 0)
+                    block_steps<HP, OUT, 3, LT, true, true>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
+                else if (dgiven)
                     block_steps<HP, OUT, 3, LT, true>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
                 else if ((notpoly & blk) == 0)
                     block_steps<HP, OUT, 3, LT>(S, dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP, y);
