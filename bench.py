@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch (read + written) on the 25M-element workload: constants copied from the rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE summary under profiles/ (scaled by what the same counters read for a 1 GiB device copy);
 # not measured by this script and valid for the default workload only
-PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.448e9 + 2.160e9, "scan_summary": 0.030e9 + 0.054e9,
+PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.513e9 + 2.501e9, "scan_summary": 0.028e9 + 0.049e9,
                              "elementwise": 2.503e9 + 0.801e9}
 
 
@@ -31,7 +31,7 @@ PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.448e9 + 2.160e9, "scan_summary": 0
 # sustains on nothing but independent fp32 instructions (bench.py --workload valu-probe, profiles/valu_probe_mi355x.txt):
 # what actually bounds these kernels
 # (the per-element kernel's count holds 8.6e6 fp32 matrix instructions of 64 clocks each: 16 vector instructions' worth of time apiece)
-PMC_VALU_INSTS_SCALE50 = {"scan_output": 2.848e9, "scan_summary": 1.21e8, "elementwise": 6.19e8 + 15 * 8.6e6}
+PMC_VALU_INSTS_SCALE50 = {"scan_output": 1.89e9, "scan_summary": 1.16e8, "elementwise": 6.19e8 + 15 * 8.6e6}
 VALU_SUSTAINED_PER_NS_SIMD = 0.59
 SIMDS = 1024
 
