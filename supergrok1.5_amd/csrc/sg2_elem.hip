@@ -25,8 +25,12 @@ constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[1
 typedef float vf4 __attribute__((ext_vector_type(4)));
 typedef float vf32 __attribute__((ext_vector_type(32)));
 
+// Four waves per SIMD for the default geometry: told so, the compiler keeps the matrix results in ordinary registers
+// (115 of them, no accumulation registers to copy out of) instead of settling for three waves at 112 + 32.
+template <class G>
+constexpr int elem_waves() { return G::DM == 8 ? 4 : 2; }
 template <class G, bool DBG>
-__global__ __launch_bounds__(ELEM_THREADS) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
+__global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(elem_waves<G>(), elem_waves<G>()))) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
                                                        int32_t* __restrict__ dbg_eidx) {
     constexpr int DM = G::DM, GRL = G::GRL, PIN = G::PIN;
     __shared__ float s_exp[NE * EXP_STRIDE];
