@@ -8,9 +8,40 @@ import torch
 
 import workloads as wl
 from helpers import DIMS
-from sg2_harness import per_tensor_scalars, shared_scalars
+from sg2_harness import Sg2Case, per_tensor_scalars, shared_scalars
 
 pytestmark = pytest.mark.gpu
+
+
+def test_benchmark_chunking_against_the_checker():
+    """The configuration the benchmark runs, compared value by value: the largest tensor of the 50-tensor set
+    (2048 x 2048: 1024 chunks of 4096 steps per direction, the multi-block spine of the radix sort) and two mid-size
+    ones, Student-t tailed gradients with the per-tensor clip applied (active for the large tensor), chunk length 4096
+    and summary window 64 as the library chooses them for the full set, a random carried state, two chained steps.
+    Sort permutation, expert indices and counts bit-exact; every float within rel 1e-4."""
+    from grokking_optimizers import _cabi
+    all_shapes = wl.scale50_shapes()
+    shapes = [all_shapes[49], all_shapes[40], all_shapes[33]]
+    assert wl.numel(shapes[0]) == 4194304
+    lib = _cabi.lib()
+    assert lib.sg2_set_chunk_len(4096) == 0 and lib.sg2_set_scan_window(64) == 0
+    try:
+        case = Sg2Case(shapes, seed=9, random_state=True)
+        for t in (1, 2):
+            raw = wl.make_grads(shapes, seed=40 + t, tail_frac=0.005, tail="student3")
+            grads = wl.clip_per_tensor(raw)
+            assert float(raw[0].norm()) > 1.0                       # the clip is active on the 4 M tensor
+            sharps = [torch.zeros_like(g) for g in grads]
+            pt, sh = per_tensor_scalars(len(shapes), t, lamb_eff=2.0), shared_scalars(wd_eff=4.5)
+            print("benchmark chunking: step", t, "GPU", flush=True)
+            case.gpu_step(grads, sharps, pt, sh)
+            print("benchmark chunking: step", t, "checker", flush=True)
+            dbg = case.oracle_step(grads, sharps, pt, sh, chunk_len=4096, window=64)
+            worst = case.compare(dbg, 1e-4, 1e-7)
+            print("benchmark chunking: step", t, "worst tolerance ratios", worst, flush=True)
+    finally:
+        lib.sg2_set_chunk_len(0)
+        lib.sg2_set_scan_window(-1)
 
 
 def _run(steps):
