@@ -508,7 +508,7 @@ int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t tota
                      float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace sg2;
     hipStream_t st = (hipStream_t)stream;
-    if (check_dims(dims)) return 1;
+    if (check_dims(dims, true)) return 1;
     if (!weights || !grads_out) return sg::fail("NULL argument");
     if (total < 0 || total > 0x7fffffffLL - BE_THREADS) return sg::fail("element count %lld out of range", (long long)total);
     for (int k = W_GRU_WZ; k < SG2_NUM_WEIGHTS; k++)

@@ -21,7 +21,10 @@ namespace sg2 {
 namespace {
 
 constexpr int ELEM_THREADS = 256;
-constexpr int EXP_STRIDE = 52;   // floats per expert record in LDS: W1[16] b1[16] W2[16] + pad
+// floats per expert record in LDS: W1[EH] b1[EH] W2[EH] (+ pad for the 16-wide experts so that random per-lane
+// experts spread over the banks)
+template <int EHW>
+constexpr int exp_stride() { return EHW == 16 ? 52 : 3 * EHW; }
 typedef float vf4 __attribute__((ext_vector_type(4)));
 typedef float vf32 __attribute__((ext_vector_type(32)));
 
@@ -29,10 +32,11 @@ typedef float vf32 __attribute__((ext_vector_type(32)));
 // (115 of them, no accumulation registers to copy out of) instead of settling for three waves at 112 + 32.
 template <class G>
 constexpr int elem_waves() { return G::DM == 8 ? 4 : 2; }
-template <class G, bool DBG>
+template <class G, int EH, bool DBG>
 __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(elem_waves<G>(), elem_waves<G>()))) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
                                                        int32_t* __restrict__ dbg_eidx) {
-    constexpr int DM = G::DM, GRL = G::GRL, PIN = G::PIN;
+    constexpr int DM = G::DM, GRL = G::GRL, PIN = G::PIN, EXP_STRIDE = exp_stride<EH>();
+    static_assert(EH % 4 == 0, "expert records are read 16 bytes at a time");
     __shared__ float s_exp[NE * EXP_STRIDE];
     __shared__ float s_b2[NE];
     __shared__ int s_cnt[NE];
@@ -237,6 +241,194 @@ __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(el
             if (s_cnt[i] != 0) atomicAdd(&expert_counts[i], s_cnt[i]);
 }
 
+
+// The same per-element step for any dimensions the reference admits (gru_hidden <= 8, d_model <= 16, any number of
+// heads, sub-keys, experts and expert width): every size is a run-time value, the loops over the bounded ones are
+// unrolled to their bounds and guarded so that the small arrays stay in registers, the expert tables are read from
+// global memory (per-lane gathers through the caches: 3 x E x expert_hidden floats need not fit the LDS), and the
+// counts go through an LDS histogram when it fits and global atomics otherwise.  The arithmetic is the specialised
+// kernel's, chain for chain (the query projection as plain fma chains: the fp32 matrix instructions compute the same
+// chains); the shared reciprocals of the gates apply when gru_hidden is 4, as in the checker.  ctx rows are
+// ctx_stride floats apart (d_model of the scan geometry the block was embedded in).
+constexpr int MAX_DM = 16, MAX_GH = 8, MAX_HD = 8, CNT_LDS = 4096;
+template <bool DBG>
+__global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stride, int32_t* __restrict__ expert_counts,
+                                                           int32_t* __restrict__ dbg_eidx) {
+    __shared__ int s_cnt[CNT_LDS];
+    const int dm = pl.dims.d_model, gh = pl.dims.gru_hidden, H = pl.dims.num_heads, pk = pl.dims.pk_dim;
+    const int eh = pl.dims.expert_hidden, E = pl.dims.num_experts, hd = dm / 2;
+    const int grl = 2 + 2 * dm + gh, pin = gh + 2 * dm + 2;
+    const bool lds_counts = E <= CNT_LDS;
+    if (lds_counts)
+        for (int i = threadIdx.x; i < E; i += ELEM_THREADS) s_cnt[i] = 0;
+    __syncthreads();
+    const sg::cfloat_p Wz = sg::as_const(pl.W.w[W_GRU_WZ]), bz = sg::as_const(pl.W.w[W_GRU_BZ]);
+    const sg::cfloat_p Wr = sg::as_const(pl.W.w[W_GRU_WR]), br = sg::as_const(pl.W.w[W_GRU_BR]);
+    const sg::cfloat_p Wh = sg::as_const(pl.W.w[W_GRU_WH]), bh = sg::as_const(pl.W.w[W_GRU_BH]);
+    const sg::cfloat_p Wq = sg::as_const(pl.W.w[W_PEER_Q]);
+    const sg::cfloat_p KA = sg::as_const(pl.W.w[W_KEYS_A]), KB = sg::as_const(pl.W.w[W_KEYS_B]);
+    const SG_GLOBAL float* W1 = sg::gptr(pl.W.w[W_EXP_W1]);
+    const SG_GLOBAL float* B1 = sg::gptr(pl.W.w[W_EXP_B1]);
+    const SG_GLOBAL float* W2 = sg::gptr(pl.W.w[W_EXP_W2]);
+    const SG_GLOBAL float* B2 = sg::gptr(pl.W.w[W_EXP_B2]);
+
+    for (int tile = blockIdx.x; tile < pl.elem_tiles; tile += gridDim.x) {
+        const int ti = sg::upper_seg(sg::as_const(pl.elem_tile_prefix), pl.P, tile);
+        const TensorDev& T = pl.tensors[ti];
+        const int start = (tile - pl.elem_tile_prefix[ti]) * ELEM_TILE;
+        const int cnt = min(ELEM_TILE, T.numel - start);
+        const int dtype = T.dtype;
+        const bool has_s = pl.sharp_nonzero[ti] != 0;
+        const float alpha = T.alpha, lamb = T.lamb, beta1 = T.beta1, bc2 = T.bc2, step_size = T.step_size;
+        const float beta2 = pl.beta2, eps = pl.eps, rescale = pl.rescale, decay = pl.decay;
+        for (int k0 = (int)threadIdx.x; k0 < cnt; k0 += ELEM_THREADS) {
+            const int i = start + k0;
+            const float g = sg::finite_or_zero(sg::load_elem(T.grad, dtype, i));
+            const float s = has_s ? sg::finite_or_zero(sg::load_elem(T.sharp, dtype, i)) : 0.0f;
+            float cf[MAX_DM], cb[MAX_DM], hold[MAX_GH];
+            {
+                const SG_GLOBAL float* pf = sg::gptr(pl.ctx) + ((size_t)T.off + i) * ctx_stride;
+                const SG_GLOBAL float* pb = sg::gptr(pl.ctx) + ((size_t)pl.total + T.off + i) * ctx_stride;
+#pragma unroll
+                for (int q = 0; q < MAX_DM; q++) { cf[q] = q < dm ? pf[q] : 0.0f; cb[q] = q < dm ? pb[q] : 0.0f; }
+#pragma unroll
+                for (int q = 0; q < MAX_GH; q++) hold[q] = q < gh ? sg::gptr(T.gru)[(size_t)i * gh + q] : 0.0f;
+            }
+            // ---- GRU: chain order = bias, g, s, fwd ctx, bwd ctx, h
+            float pre_g[2 * MAX_GH], gate[2 * MAX_GH], pre_c[MAX_GH], cand[MAX_GH], hnew[MAX_GH];
+#pragma unroll
+            for (int j = 0; j < MAX_GH; j++) {
+                pre_g[j] = pre_g[MAX_GH + j] = 0.0f;
+                if (j < gh) {
+                    const sg::cfloat_p wz = Wz + j * grl, wr = Wr + j * grl;
+                    float vz = bz[j], vr = br[j];
+                    vz = sg_fma(wz[0], g, vz); vz = sg_fma(wz[1], s, vz);
+                    vr = sg_fma(wr[0], g, vr); vr = sg_fma(wr[1], s, vr);
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) { vz = sg_fma(wz[2 + q], cf[q], vz); vr = sg_fma(wr[2 + q], cf[q], vr); }
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) { vz = sg_fma(wz[2 + dm + q], cb[q], vz); vr = sg_fma(wr[2 + dm + q], cb[q], vr); }
+#pragma unroll
+                    for (int q = 0; q < MAX_GH; q++) if (q < gh) { vz = sg_fma(wz[2 + 2 * dm + q], hold[q], vz); vr = sg_fma(wr[2 + 2 * dm + q], hold[q], vr); }
+                    pre_g[j] = vz;
+                    pre_g[MAX_GH + j] = vr;
+                }
+            }
+            if (gh == GH) {       // update and reset gates of the four units share one reciprocal
+                float in8[2 * GH], out8[2 * GH];
+#pragma unroll
+                for (int j = 0; j < GH; j++) { in8[j] = pre_g[j]; in8[GH + j] = pre_g[MAX_GH + j]; }
+                sg_sigmoid_block(2 * GH, in8, out8);
+#pragma unroll
+                for (int j = 0; j < MAX_GH; j++) { gate[j] = j < GH ? out8[j] : 0.0f; gate[MAX_GH + j] = j < GH ? out8[GH + j] : 0.0f; }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2 * MAX_GH; j++) gate[j] = sg_sigmoid(pre_g[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < MAX_GH; j++) {
+                pre_c[j] = 0.0f;
+                if (j < gh) {
+                    const sg::cfloat_p wh = Wh + j * grl;
+                    float v = bh[j];
+                    v = sg_fma(wh[0], g, v); v = sg_fma(wh[1], s, v);
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) v = sg_fma(wh[2 + q], cf[q], v);
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) v = sg_fma(wh[2 + dm + q], cb[q], v);
+#pragma unroll
+                    for (int q = 0; q < MAX_GH; q++) if (q < gh) v = sg_fma(wh[2 + 2 * dm + q], gate[MAX_GH + q] * hold[q], v);
+                    pre_c[j] = v;
+                }
+            }
+            if (gh == GH) {
+                float in4[GH], out4[GH];
+#pragma unroll
+                for (int j = 0; j < GH; j++) in4[j] = pre_c[j];
+                sg_tanh_block(GH, in4, out4);
+#pragma unroll
+                for (int j = 0; j < MAX_GH; j++) cand[j] = j < GH ? out4[j] : 0.0f;
+            } else {
+#pragma unroll
+                for (int j = 0; j < MAX_GH; j++) cand[j] = sg_tanh(pre_c[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < MAX_GH; j++) {
+                hnew[j] = sg_fma(gate[j], cand[j], (1.0f - gate[j]) * hold[j]);
+                if (j < gh) sg::gptr(T.gru)[(size_t)i * gh + j] = hnew[j];
+            }
+
+            // ---- PEER: per head the query (chain order = h, fwd ctx, bwd ctx, g, s), two sub-key arg-maxes, the expert
+            float total = 0.0f;
+            for (int hh = 0; hh < H; hh++) {
+                auto query_row = [&](int row) {
+                    const sg::cfloat_p qr = Wq + ((size_t)hh * dm + row) * pin;
+                    float v = 0.0f;
+#pragma unroll
+                    for (int q = 0; q < MAX_GH; q++) if (q < gh) v = sg_fma(qr[q], hnew[q], v);
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) v = sg_fma(qr[gh + q], cf[q], v);
+#pragma unroll
+                    for (int q = 0; q < MAX_DM; q++) if (q < dm) v = sg_fma(qr[gh + dm + q], cb[q], v);
+                    v = sg_fma(qr[gh + 2 * dm], g, v);
+                    v = sg_fma(qr[gh + 2 * dm + 1], s, v);
+                    return v;
+                };
+                float qa[MAX_HD], qb[MAX_HD];
+#pragma unroll
+                for (int dd = 0; dd < MAX_HD; dd++) {
+                    qa[dd] = qb[dd] = 0.0f;
+                    if (dd < hd) { qa[dd] = query_row(dd); qb[dd] = query_row(hd + dd); }
+                }
+                int best[2];
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++) {
+                    const sg::cfloat_p keys = (hf ? KB : KA) + (size_t)hh * pk * hd;
+                    int bi = 0;
+                    float bs = -1e30f;
+                    for (int q = 0; q < pk; q++) {
+                        float dot = 0.0f;
+#pragma unroll
+                        for (int dd = 0; dd < MAX_HD; dd++) if (dd < hd) dot = sg_fma(hf ? qb[dd] : qa[dd], keys[q * hd + dd], dot);
+                        if (dot > bs) { bs = dot; bi = q; }
+                    }
+                    best[hf] = bi;
+                }
+                int e = best[0] * pk + best[1];
+                if (e >= E) e = E - 1;
+                if (lds_counts) atomicAdd(&s_cnt[e], 1);
+                else if (expert_counts != nullptr) atomicAdd(&expert_counts[e], 1);
+                if (DBG) dbg_eidx[((size_t)T.off + i) * H + hh] = e;
+                float ho = B2[e];
+                for (int q = 0; q < eh; q++) {
+                    const float z = sg_max(sg_fma(W1[(size_t)e * eh + q], g, B1[(size_t)e * eh + q]), 0.0f);
+                    ho = sg_fma(W2[(size_t)e * eh + q], z, ho);
+                }
+                total = total + ho;
+            }
+            const float smart = g + (rescale * total) / (float)H;
+
+            // ---- mu EMA, Adam moments, decoupled weight decay
+            float mu = sg::gptr(T.mu)[i], ea = sg::gptr(T.ea)[i], easq = sg::gptr(T.easq)[i];
+            float pv = sg::load_elem(T.param, dtype, i);
+            mu = sg_fma(alpha, mu, (1.0f - alpha) * g);
+            sg::gptr(T.mu)[i] = mu;
+            const float fg = sg_fma(lamb, mu, smart);
+            ea = sg_fma(beta1, ea, (1.0f - beta1) * fg);
+            easq = sg_fma(beta2, easq, ((1.0f - beta2) * fg) * fg);
+            sg::gptr(T.ea)[i] = ea;
+            sg::gptr(T.easq)[i] = easq;
+            const float denom = __builtin_sqrtf(easq / bc2) + eps;
+            pv = sg_fma(pv, decay, -((step_size * ea) / denom));
+            sg::store_elem(T.param, dtype, i, pv);
+        }
+    }
+    __syncthreads();
+    if (lds_counts && expert_counts != nullptr)
+        for (int i = threadIdx.x; i < E; i += ELEM_THREADS)
+            if (s_cnt[i] != 0) atomicAdd(&expert_counts[i], s_cnt[i]);
+}
+
 }  // namespace
 
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st) {
@@ -244,15 +436,22 @@ int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx,
     // about five workgroups per resident slot (768 at three per CU): measured 1.38 / 1.35 / 1.33 / 1.33 / 1.37 ms with 768 / 2048 / 4096 /
     // 8192 / 16384 workgroups on 24 424 tiles (fewer leave the chip unevenly loaded at the end, more pay the LDS fill too often)
     const int grid = pl.elem_tiles < 4096 ? pl.elem_tiles : 4096;
-    if (pl.geo == GEO_LARGE) {
-        if (dbg_expert_idx)
-            hipLaunchKernelGGL((k_elem<GeoLarge, true>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
-        else
-            hipLaunchKernelGGL((k_elem<GeoLarge, false>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
-    } else if (dbg_expert_idx)
-        hipLaunchKernelGGL((k_elem<GeoDefault, true>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
-    else
-        hipLaunchKernelGGL((k_elem<GeoDefault, false>), dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx);
+    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx); };
+    if (pl.elem_kind == ELEM_ANY) {
+        const int stride = geo_info(pl.geo).dm;
+        if (dbg_expert_idx) hipLaunchKernelGGL(k_elem_any<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx);
+        else hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx);
+    } else if (pl.geo == GEO_LARGE) {
+        if (dbg_expert_idx) go(k_elem<GeoLarge, 16, true>);
+        else go(k_elem<GeoLarge, 16, false>);
+    } else if (pl.elem_kind == ELEM_FAST4) {
+        if (dbg_expert_idx) go(k_elem<GeoDefault, 4, true>);
+        else go(k_elem<GeoDefault, 4, false>);
+    } else if (dbg_expert_idx) {
+        go(k_elem<GeoDefault, 16, true>);
+    } else {
+        go(k_elem<GeoDefault, 16, false>);
+    }
     SG_LAUNCH_CHECK("k_elem");
     return 0;
 }

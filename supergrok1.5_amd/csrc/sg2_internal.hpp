@@ -8,12 +8,18 @@ namespace sg2 {
 // Compile-time meta-net geometries the step kernels are instantiated for: the
 // defaults of the optimizer class and the largest scan block the reference
 // admits (csrc/supergrok2_mamba_peer_kernels.cu:36-42 caps d_model at 16 and
-// d_state / d_inner at 32).  The GRU, routing and expert sizes are the same in both.
+// d_state / d_inner at 32).  Any smaller scan block runs on the smallest of the
+// two that holds it, with its weights embedded in that geometry (zero rows and
+// columns, see k_pad_weights in sg2_step.hip).  The specialised per-element
+// kernel is built for the GRU, routing and expert sizes below (expert width 16,
+// the class default, or 4, what the reference's training harness passes); every
+// other combination takes the run-time-dimension kernel (k_elem_any).
 constexpr int GH = 4;      // gru_hidden
 constexpr int NH = 4;      // PEER heads
 constexpr int PK = 12;     // sub-keys per half
-constexpr int EH = 16;     // expert hidden
+constexpr int EH = 16;     // expert hidden (class default)
 constexpr int NE = 144;    // experts
+enum { ELEM_FAST16 = 0, ELEM_FAST4 = 1, ELEM_ANY = 2 };    // Plan::elem_kind
 template <int DM_, int DS_, int DI_>
 struct Geo {
     static constexpr int DM = DM_;               // d_model
@@ -100,6 +106,10 @@ struct Plan {
     int total;                     // sum of numel
     int elem_tiles, sort_tiles, chunks, wchunks;
     int geo;                       // GEO_*: which instantiation of the scan / elementwise kernels runs
+    int elem_kind;                 // ELEM_*: which per-element kernel runs
+    int st_di, st_ds;              // the caller's carried Mamba states are [st_di][st_ds] (the true d_inner, d_state;
+                                   // entries of the kernel geometry beyond them read as 0 and are not stored)
+    SgDims dims;                   // the caller's dimensions (what k_elem_any indexes the per-element weights with)
     int chunk_len;
     int window;                    // summary window (0: whole chunk), see k_scan<false>
     uint32_t* keys[2];
@@ -136,10 +146,15 @@ __host__ __device__ inline int htile_count(int total, int P) { return total / HT
 // floats per direction of the adjoint kernels' sums: composed coefficients [5][16][3], A_log [16][16], rope_freq [16][8], D [16], out_proj [8][16]
 constexpr int SG2_BWD_STRIDE = 768;
 constexpr int ADJ_GROUPS = 512;    // workgroups per direction of the adjoint replay (upper bound)
-// GEO_* of these dimensions, or -1 with the error set
+// GEO_* of the smallest compiled geometry that holds these dimensions, or -1 with the error set
 int geo_of(const SgDims* d);
+// whether (d_model, d_state, d_inner) are exactly that geometry's (else the scan weights are embedded in it)
+bool scan_exact(const SgDims* d, int geo);
+// ELEM_* for these dimensions
+int elem_kind_of(const SgDims* d, int geo);
 // 0 if the dimensions are the default geometry (what the bilevel kernels are built for), else 1 with the error set
-int check_dims(const SgDims* d);
+// per_element: also the GRU / routing / expert sizes the bilevel per-element kernel is built for
+int check_dims(const SgDims* d, bool per_element = false);
 // exactly one of d_ctx (element order, after out_proj) / d_scan (scan order, before out_proj) is given; dx (with rx) is optional
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* const d_scan[2], const float* rx, float* dx, float* grads_out,
                             hipStream_t st);

@@ -790,8 +790,10 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     if (OUT) {
         if (u1 == N) {   // last chunk in scan order: new carried state of the tensor
             float* st = dir ? T.mbwd : T.mfwd;
-            st[j * DS + 2 * p] = S.he;
-            st[j * DS + 2 * p + 1] = S.ho;
+            if (j < pl.st_di && 2 * p < pl.st_ds) {
+                st[j * pl.st_ds + 2 * p] = S.he;
+                st[j * pl.st_ds + 2 * p + 1] = S.ho;
+            }
         }
     } else {
         float* sm = pl.summaries + (size_t)(dir * pl.wchunks + cidx) * 6 * SCAN_THREADS;
@@ -816,7 +818,7 @@ constexpr int PREFIX_PER_GROUP = 4;
 
 template <class G>
 __global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
-    constexpr int DS = G::DS, HP = G::HP, SCAN_THREADS = G::THREADS;
+    constexpr int HP = G::HP, SCAN_THREADS = G::THREADS;
     constexpr int PREFIX_GROUPS = 1024 / SCAN_THREADS;             // 8 groups of 128 lanes, or 2 of 512
     constexpr int PREFIX_BATCH = PREFIX_PER_GROUP * PREFIX_GROUPS;
     __shared__ float lds[PREFIX_BATCH * 6 * SCAN_THREADS];     // 96 KB
@@ -830,9 +832,12 @@ __global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
     const int ns = T.nchunks - 1;                               // summaries to apply
     float he = 0.0f, ho = 0.0f;
     if (grp == 0) {
+        // the caller's state is [st_di][st_ds] (its own d_inner, d_state); the rest of the kernel geometry starts at 0
         const float* st = dir ? T.mbwd : T.mfwd;
-        he = st[j * DS + 2 * p];
-        ho = st[j * DS + 2 * p + 1];
+        if (j < pl.st_di && 2 * p < pl.st_ds) {
+            he = st[j * pl.st_ds + 2 * p];
+            ho = st[j * pl.st_ds + 2 * p + 1];
+        }
         hs[lane] = he;
         hs[SCAN_THREADS + lane] = ho;
     }

@@ -62,9 +62,63 @@ struct Prof {
 
 struct Layout {
     int P, total, elem_tiles, sort_tiles, chunks, wchunks, nb;
-    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_ctx, off_htile, off_adj_summ, off_adj_lam, off_adj_part, off_adj_blk, bytes;
+    size_t off_tables, off_keys[2], off_vals[2], off_ssorted, off_spine, off_blocksums, off_summ, off_hstart, off_comp, off_flags, off_padw, off_ctx, off_htile, off_adj_summ, off_adj_lam, off_adj_part, off_adj_blk, bytes;
     size_t tables_bytes;
 };
+
+// Floats of the 20 scan weight tensors (input_proj W, b; 9 per direction) at a kernel geometry, each rounded up to
+// a multiple of 4 floats so that every tensor starts 16-byte aligned.
+inline size_t scan_weight_floats(const GeoInfo& gi, int k) {
+    const size_t dm = gi.dm, ds = gi.ds, di = gi.di;
+    const size_t block[9] = {2 * di * dm, di * di, di, ds * di, ds * di, di * ds, di, di * (ds / 2), dm * di};
+    const size_t n = k == 0 ? 2 * dm : (k == 1 ? dm : block[(k - 2) % 9]);
+    return (n + 3) / 4 * 4;
+}
+inline size_t padded_weight_floats(const GeoInfo& gi) {
+    size_t n = 0;
+    for (int k = 0; k < 20; k++) n += scan_weight_floats(gi, k);
+    return n;
+}
+
+// A scan block smaller than the kernel geometry, embedded in it so that it computes the same function:
+//   * rows / columns beyond the true d_model, d_inner, d_state of input_proj, in_proj, dt_W, B_proj, C_proj, D, rope
+//     and out_proj are zero: the extra columns see a zero x-branch and gate, the extra states receive no input and
+//     contribute nothing to y, the extra context entries are +0;
+//   * every fma chain only gains terms with a zero factor, so the real entries keep their bits;
+//   * the extra poles copy real ones (A_log[j][0] for extra states of a real column, column 0 for extra columns) and
+//     the extra columns take dt_b[0]: their (never used) states contract like real ones, so the decisions that look
+//     at all lanes (summary contraction, first-block length, polynomial limits) see nothing new.
+struct PadArgs {
+    const float* src[20];
+    float* dst[20];
+    int dm, ds, di;        // true dimensions
+    int DM, DS, DI;        // kernel geometry
+};
+__global__ __launch_bounds__(256) void k_pad_weights(PadArgs a) {
+    const int k = blockIdx.y;
+    const int dm = a.dm, ds = a.ds, di = a.di, hp = ds / 2, DM = a.DM, DS = a.DS, DI = a.DI, HP = DS / 2;
+    const int slot = k < 2 ? k : 2 + (k - 2) % 9;
+    const int count = k == 0 ? 2 * DM : k == 1 ? DM : slot == 2 ? 2 * DI * DM : slot == 3 ? DI * DI : (slot == 4 || slot == 8) ? DI
+                    : (slot == 5 || slot == 6) ? DS * DI : slot == 7 ? DI * DS : slot == 9 ? DI * HP : DM * DI;
+    const float* __restrict__ src = a.src[k];
+    float* __restrict__ dst = a.dst[k];
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < count; i += gridDim.x * 256) {
+        float v = 0.0f;
+        if (k == 0) { const int r = i / 2, c = i % 2; if (r < dm) v = src[r * 2 + c]; }                    // input_proj W [dm][2]
+        else if (k == 1) { if (i < dm) v = src[i]; }                                                          // input_proj b
+        else if (slot == 2) {                                                                                 // in_proj [2 di][dm]: x rows, then z rows
+            const int r = i / DM, c = i % DM, part = r / DI, j = r % DI;
+            if (j < di && c < dm) v = src[(part * di + j) * dm + c];
+        } else if (slot == 3) { const int r = i / DI, c = i % DI; if (r < di && c < di) v = src[r * di + c]; } // dt_W [di][di]
+        else if (slot == 4) v = src[i < di ? i : 0];                                                           // dt_b
+        else if (slot == 5 || slot == 6) { const int r = i / DI, c = i % DI; if (r < ds && c < di) v = src[r * di + c]; }   // B_proj, C_proj [ds][di]
+        else if (slot == 7) { const int j = i / DS, st = i % DS; v = src[(j < di ? j : 0) * ds + (st < ds ? st : 0)]; }     // A_log [di][ds]
+        else if (slot == 8) { if (i < di) v = src[i]; }                                                        // D
+        else if (slot == 9) { const int j = i / HP, q = i % HP; if (j < di && q < hp) v = src[j * hp + q]; }   // rope [di][ds/2]
+        else { const int r = i / DI, c = i % DI; if (r < dm && c < di) v = src[r * di + c]; }                  // out_proj [dm][di]
+        dst[i] = v;
+    }
+}
 
 int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bilevel = false) {
     const GeoInfo gi = geo_info(geo);
@@ -97,6 +151,7 @@ int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bi
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
     L->off_comp = take(4 * (2 * 5 * (size_t)gi.rows * 3 + 2 * 2 * (size_t)gi.rows * 4 + 12));      // composed triples, Taylor polynomials, coefficient maxima and polynomial limits
     L->off_flags = take(4 * ((size_t)P + 2));        // apart from the tensor records: it is written while those are being read
+    L->off_padw = take(4 * (size_t)padded_weight_floats(gi));   // scan weights embedded in the kernel geometry (used when the caller's block is smaller)
     L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions
     L->off_htile = take(bilevel ? 4 * 2 * (size_t)htile_count((int)total, P) * 2 * SCAN_THREADS : 0);
@@ -147,23 +202,47 @@ int geo_of(const SgDims* d) {
     if (d->gru_hidden > 8) return sg::fail("gru_hidden exceeds MAX_GRU_HIDDEN (%d > 8)", d->gru_hidden), -1;
     if (d->d_inner > 32) return sg::fail("d_inner exceeds MAX_D_INNER (%d > 32)", d->d_inner), -1;
     if (d->d_inner % 4) return sg::fail("d_inner must be a multiple of 4 (got %d)", d->d_inner), -1;
-    // the geometries these kernels are compiled for
-    if (d->gru_hidden == GH && d->num_heads == NH && d->pk_dim == PK && d->expert_hidden == EH && d->num_experts == NE)
-        for (int geo = 0; geo < GEO_COUNT; geo++) {
-            const GeoInfo gi = geo_info(geo);
-            if (d->d_model == gi.dm && d->d_state == gi.ds && d->d_inner == gi.di) return geo;
-        }
-    sg::fail("unsupported meta-net dims: kernels are built for (d_model, d_state, d_inner) = (%d, %d, %d) or (%d, %d, %d), with "
-             "gru_hidden=%d heads=%d pk_dim=%d expert_hidden=%d experts=%d",
-             GeoDefault::DM, GeoDefault::DS, GeoDefault::DI, GeoLarge::DM, GeoLarge::DS, GeoLarge::DI, GH, NH, PK, EH, NE);
-    return -1;
+    // what the reference takes for granted (its kernels index with these and would read out of bounds otherwise)
+    if (d->d_model < 1 || d->d_state < 2 || d->d_inner < 4 || d->gru_hidden < 1 || d->num_heads < 1 || d->pk_dim < 1 ||
+        d->expert_hidden < 1 || d->num_experts < 1)
+        return sg::fail("meta-net dimensions must be positive (d_model %d, d_state %d, d_inner %d, gru_hidden %d, num_heads %d, pk_dim %d, "
+                        "expert_hidden %d, num_experts %d)", d->d_model, d->d_state, d->d_inner, d->gru_hidden, d->num_heads, d->pk_dim,
+                        d->expert_hidden, d->num_experts), -1;
+    if (d->d_model % 2)
+        return sg::fail("d_model must be even (got %d): a query is split into two halves of d_model/2 entries, one per product-key table "
+                        "(grokking_optimizers/mamba3_peer_metanet.py:69,337-338)", d->d_model), -1;
+    if ((int64_t)d->num_experts > (int64_t)d->pk_dim * d->pk_dim)
+        return sg::fail("num_experts (%d) exceeds pk_dim^2 (%d): the product-key index a * pk_dim + b (csrc/supergrok2_mamba_peer_kernels.cu:1048) "
+                        "cannot reach every expert", d->num_experts, d->pk_dim * d->pk_dim), -1;
+    for (int geo = 0; geo < GEO_COUNT; geo++) {       // the smallest compiled geometry that holds the scan block
+        const GeoInfo gi = geo_info(geo);
+        if (d->d_model <= gi.dm && d->d_state <= gi.ds && d->d_inner <= gi.di) return geo;
+    }
+    return sg::fail("no scan geometry holds d_model %d, d_state %d, d_inner %d", d->d_model, d->d_state, d->d_inner), -1;
 }
 
-int check_dims(const SgDims* d) {
+bool scan_exact(const SgDims* d, int geo) {
+    const GeoInfo gi = geo_info(geo);
+    return d->d_model == gi.dm && d->d_state == gi.ds && d->d_inner == gi.di;
+}
+
+int elem_kind_of(const SgDims* d, int geo) {
+    if (!scan_exact(d, geo) || d->gru_hidden != GH || d->num_heads != NH || d->pk_dim != PK || d->num_experts != NE) return ELEM_ANY;
+    if (d->expert_hidden == EH) return ELEM_FAST16;
+    if (d->expert_hidden == 4 && geo == GEO_DEFAULT) return ELEM_FAST4;
+    return ELEM_ANY;
+}
+
+int check_dims(const SgDims* d, bool per_element) {
     const int geo = geo_of(d);
     if (geo < 0) return 1;
-    if (geo != GEO_DEFAULT)
-        return sg::fail("the bilevel pass is built for d_model=%d d_state=%d d_inner=%d only", GeoDefault::DM, GeoDefault::DS, GeoDefault::DI);
+    if (per_element && (d->gru_hidden != GH || d->num_heads != NH || d->pk_dim != PK || d->expert_hidden != EH || d->num_experts != NE))
+        return sg::fail("the per-element kernel of the bilevel pass is built for gru_hidden=%d num_heads=%d pk_dim=%d expert_hidden=%d "
+                        "num_experts=%d (got %d, %d, %d, %d, %d); experts narrower than %d run embedded in that width", GH, NH, PK, EH, NE,
+                        d->gru_hidden, d->num_heads, d->pk_dim, d->expert_hidden, d->num_experts, EH);
+    if (geo != GEO_DEFAULT || !scan_exact(d, geo))
+        return sg::fail("the bilevel pass is built for d_model=%d d_state=%d d_inner=%d only (got %d, %d, %d)", GeoDefault::DM, GeoDefault::DS,
+                        GeoDefault::DI, d->d_model, d->d_state, d->d_inner);
     return 0;
 }
 
@@ -252,6 +331,10 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     const int geo = geo_of(dims);
     if (geo < 0 || (bilevel && check_dims(dims))) return 1;
     pl.geo = geo;
+    pl.elem_kind = elem_kind_of(dims, geo);
+    pl.st_di = dims->d_inner;
+    pl.st_ds = dims->d_state;
+    pl.dims = *dims;
     if (num_tensors == 0) return 0;
     if (num_tensors < 0 || !tensors || !weights || !scalars) return sg::fail("NULL argument");
     for (int k = 0; k < SG2_NUM_WEIGHTS; k++)
@@ -335,6 +418,23 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
     pl.W = *weights;
+    if (!scan_exact(dims, geo)) {
+        // the caller's scan block is smaller than the kernel geometry: embed its 20 weight tensors (every call: the
+        // caller may have changed them) and let the sort / scan kernels read the embedded copies
+        const GeoInfo gi = geo_info(geo);
+        PadArgs a;
+        float* at = reinterpret_cast<float*>(ws + L.off_padw);
+        for (int k = 0; k < 20; k++) {
+            a.src[k] = weights->w[k];
+            a.dst[k] = at;
+            pl.W.w[k] = at;
+            at += scan_weight_floats(gi, k);
+        }
+        a.dm = dims->d_model; a.ds = dims->d_state; a.di = dims->d_inner;
+        a.DM = gi.dm; a.DS = gi.ds; a.DI = gi.di;
+        hipLaunchKernelGGL(k_pad_weights, dim3(4, 20), dim3(256), 0, st, a);
+        SG_LAUNCH_CHECK("k_pad_weights");
+    }
 
     pl.htile = bilevel ? reinterpret_cast<float*>(ws + L.off_htile) : nullptr;
     pl.scan_out[0] = pl.scan_out[1] = nullptr;
@@ -355,8 +455,9 @@ int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, con
     if (launch_sort(pl, debug ? debug->perm : nullptr, st)) return 1;
     prof_mark(1, st);
     if (launch_scan(pl, st)) return 1;
-    if (debug && debug->ctx)
-        SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * geo_info(pl.geo).dm, hipMemcpyDeviceToDevice, st));
+    if (debug && debug->ctx)      // [2][total][d_model] for the caller; the kernels' rows are d_model of the kernel geometry wide
+        SG_HIP_CHECK(hipMemcpy2DAsync(debug->ctx, 4 * (size_t)dims->d_model, pl.ctx, 4 * (size_t)geo_info(pl.geo).dm, 4 * (size_t)dims->d_model,
+                                      2 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
     if (launch_elem(pl, expert_counts, debug ? debug->expert_idx : nullptr, st)) return 1;
     prof_mark(5, st);
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;

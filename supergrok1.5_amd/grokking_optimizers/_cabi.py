@@ -241,11 +241,24 @@ class Sg2Bilevel:
 SG2_ELEM_GRAD_FLOATS = 8420
 
 
+BILEVEL_EXPERT_WIDTH = 16      # expert width sg2_bilevel_elem is compiled for
+
+
 def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, dims=None, want_smart=True):
     """sg2_bilevel_elem on flat fp32 GPU arrays: returns (smart [total] or None, d_ctx [2, total, d_model],
     weight-gradient block [SG2_ELEM_GRAD_FLOATS])."""
     d = make_dims(dims)
     ws_ = [w.detach().float().contiguous() for w in weights]
+    # The kernel is built for experts of width 16.  Narrower experts (the reference's training harness uses 4) run as
+    # 16-wide ones whose extra units have W1 = b1 = W2 = 0: relu(0) = 0 adds nothing to any output, every real entry
+    # keeps its bits, and the extra units' gradient entries (all zero) are dropped from the block below.
+    eh, E = d.expert_hidden, d.num_experts
+    if eh < BILEVEL_EXPERT_WIDTH:
+        for k in (29, 30, 31):
+            wide = torch.zeros(E, BILEVEL_EXPERT_WIDTH, dtype=torch.float32, device=ws_[k].device)
+            wide[:, :eh] = ws_[k].reshape(E, eh)
+            ws_[k] = wide
+        d.expert_hidden = BILEVEL_EXPERT_WIDTH
     W = Sg2Weights()
     for k, w in enumerate(ws_):
         W.w[k] = w.data_ptr()
@@ -264,4 +277,8 @@ def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, d
                                 work.numel(), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError("sg2_bilevel_elem: " + last_error())
+    if eh < BILEVEL_EXPERT_WIDTH:       # expert part of the block: W1, b1, W2 [E, 16] each, then b2 [E]
+        head = out.numel() - (3 * BILEVEL_EXPERT_WIDTH + 1) * E
+        ex = out[head:head + 3 * BILEVEL_EXPERT_WIDTH * E].view(3, E, BILEVEL_EXPERT_WIDTH)[:, :, :eh].reshape(-1)
+        out = torch.cat([out[:head], ex, out[-E:]])
     return smart, d_ctx, out

@@ -39,3 +39,27 @@ def test_host_side_validation_without_gpu():
     assert _cabi.chunk_len_for([1000, 5000]) == 1024 and _cabi.chunk_len_for([4 << 20] * 8) == 4096
     assert lib.sg2_set_scan_window(100) != 0 and lib.sg2_set_scan_window(128) == 0 and lib.sg2_get_scan_window() == 128
     assert lib.sg2_set_scan_window(-1) == 0 and lib.sg2_get_scan_window() == 64
+
+
+def test_refused_dims_name_the_reference_limit():
+    """Dimensions the library refuses are refused with the reference's own limit in the message
+    (csrc/supergrok2_mamba_peer_kernels.cu:1796-1801 and what its kernels take for granted); everything inside those
+    limits is accepted.  No GPU work: the size query only validates."""
+    import ctypes as C
+    from grokking_optimizers import _cabi
+    import workloads as wl
+    numels = (C.c_int64 * 2)(100, 200)
+
+    def query(**kw):
+        d = _cabi.make_dims(dict(wl.DEFAULT_DIMS, **kw))
+        return _cabi.lib().sg2_workspace_bytes(C.byref(d), 2, numels), _cabi.last_error()
+    for kw, text in ((dict(d_state=15), "d_state must be even"), (dict(d_state=34), "MAX_D_STATE"), (dict(d_model=18), "MAX_D_MODEL"),
+                     (dict(gru_hidden=9), "MAX_GRU_HIDDEN"), (dict(d_inner=36), "MAX_D_INNER"), (dict(d_inner=14), "multiple of 4"),
+                     (dict(d_model=7), "d_model must be even"), (dict(num_experts=200), "pk_dim^2"), (dict(num_heads=0), "positive")):
+        n, msg = query(**kw)
+        assert n == 0 and text in msg, (kw, msg)
+    for kw in (dict(), dict(expert_hidden=4), dict(d_model=4, d_state=8, d_inner=8), dict(d_model=16, d_state=32, d_inner=32),
+               dict(d_model=12, d_state=24, d_inner=24, gru_hidden=8, num_heads=3, pk_dim=6, expert_hidden=5, num_experts=36),
+               dict(num_heads=2, pk_dim=70, expert_hidden=2, num_experts=4900)):
+        n, msg = query(**kw)
+        assert n > 0, (kw, msg)

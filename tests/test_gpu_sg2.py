@@ -229,9 +229,10 @@ def test_rejects_unsupported_dims_and_small_workspace():
     d = dict(DIMS, d_state=15)
     with pytest.raises(RuntimeError, match="d_state must be even"):
         _cabi.workspace_bytes([10], d)
-    d = dict(DIMS, d_model=4)
-    with pytest.raises(RuntimeError, match="unsupported meta-net dims"):
+    d = dict(DIMS, d_model=18)
+    with pytest.raises(RuntimeError, match="MAX_D_MODEL"):
         _cabi.workspace_bytes([10], d)
+    assert _cabi.workspace_bytes([10], dict(DIMS, d_model=4, d_state=8, d_inner=8)) > 0      # runs embedded in (8, 16, 16)
     case = Sg2Case([(100,)], seed=1)
     case.step_fn.workspace = torch.empty(256, dtype=torch.uint8, device="cuda")
     g = [torch.zeros(100)]

@@ -150,10 +150,10 @@ def _ref_forward_for_bilevel(mn, grad, sharp, gru_state, hf, hb):
     return ref_fp64.forward_for_bilevel(W, grad, sharp, gru_state, hf, hb, mn.rescale, dims)
 
 
-def _meta_net(seed, dev):
+def _meta_net(seed, dev, **kw):
     from grokking_optimizers import Mamba3PEERMetaNet
     torch.manual_seed(seed)
-    mn = Mamba3PEERMetaNet()
+    mn = Mamba3PEERMetaNet(**kw)
     with torch.no_grad():       # the initial keys and experts are nearly silent: give every part a visible gradient
         for p in mn.parameters():
             if p.dim() > 0 and float(p.abs().max()) < 0.05:
@@ -217,6 +217,43 @@ def test_differentiable_forward_of_the_whole_meta_net():
     assert bool((err <= tol).all()), ("smart", float((err / tol).max()))
     w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_sum, 2e-4)
     print("all-HIP accumulation, worst gradient ratios", w, flush=True)
+    assert max(w.values()) <= 1.0, w
+
+
+def test_all_hip_accumulation_with_experts_of_width_4():
+    """The bilevel accumulation with expert_hidden = 4, the width the reference's training harness constructs the
+    optimizer with (grokking_race_v2.py:1583 -> :775): the per-element kernel runs the narrow experts embedded in its
+    own width.  Smart gradients and the gradients of every parameter against float64 autograd."""
+    import copy
+    from grokking_optimizers import _bilevel
+    dev = torch.device("cuda:0")
+    mn = _meta_net(8, dev, expert_hidden=4)
+    assert mn.expert_W1.shape[1] == 4
+    mn64 = copy.deepcopy(mn).double().cpu()
+    gen = torch.Generator().manual_seed(23)
+    data = []
+    for n in (200, 77, 1300):
+        data.append(dict(g=torch.randn(n, generator=gen) * 0.5, s=torch.rand(n, generator=gen) * 0.3,
+                         h=torch.randn(n, 4, generator=gen) * 0.5, hf=torch.randn(16, 16, generator=gen) * 0.3,
+                         hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
+    mn64.zero_grad()
+    ref_smart = []
+    for d in data:
+        rs, _, _, _ = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
+        (rs * d["R"].double()).sum().backward()
+        ref_smart.append(rs.detach())
+    ref_named = [(n, p.grad.clone()) for n, p in mn64.named_parameters()]
+    mn.zero_grad()
+    smart = _bilevel.accumulate_meta_gradients(mn, [d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data],
+                                               [d["h"].to(dev) for d in data], [d["hf"].to(dev) for d in data],
+                                               [d["hb"].to(dev) for d in data], [d["R"].to(dev) for d in data])
+    got, ref = smart.double().cpu(), torch.cat(ref_smart)
+    err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
+    assert bool((err <= tol).all()), ("smart", float((err / tol).max()))
+    for n, p in mn.named_parameters():
+        assert p.grad is not None and p.grad.shape == p.shape, n
+    w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_named, 2e-4)
+    print("expert width 4, worst gradient ratios", w, flush=True)
     assert max(w.values()) <= 1.0, w
 
 
