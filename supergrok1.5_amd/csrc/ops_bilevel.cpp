@@ -3,12 +3,18 @@
 // (csrc/ops.h:232-371, bound at csrc/ops.cpp:1072-1085 of the reference), with the reference's argument lists,
 // over sg2_bilevel_forward_ex / sg2_bilevel_backward_ex of libsg_hip.so.
 //
-// What is honoured: everything the reference's caller (grokking_optimizers/supergrok2.py:646-1040) reads between the
+// What is honoured: everything the reference's caller (grokking_optimizers/supergrok2.py:646-1330) reads between the
 // two calls and after them -- the gated scan outputs before out_proj in scan order, x_sorted, sort_indices, offsets,
-// the gradients of the 16 Mamba weight tensors (accumulated into the d_* arguments) and d_x_sorted.
-// What is not: the per-step `*_saved_*` buffers stay untouched.  The HIP adjoint recomputes the states of a 32-step
-// tile from the state entering it, which the forward call keeps in a workspace of its own; fwd_save_batched parks that
-// workspace under the address of `x_sorted_packed`, where backward_batched (which receives the same tensor) finds it.
+// the gradients of the Mamba weight tensors (accumulated into the d_* arguments) and d_x_sorted; for the one-tensor
+// pair also the gradients of every other weight of the meta-net.
+// What is not: the per-step `*_saved_x_branch / z / dt` buffers stay untouched and `*_saved_states` is not a table of
+// states.  The HIP adjoint recomputes the states of a 32-step tile from the state entering it, which the forward call
+// keeps in a workspace of its own.  That workspace (with the tensors it refers to) is parked in this process under a
+// fresh 64-bit ticket, and the ticket is written into the first four floats of the caller's `fwd_saved_states`
+// tensor -- which the backward call receives again: it reads the ticket back (one 16-byte device-to-host copy) and
+// claims exactly the forward call that filled its buffers.  Two optimizers, or interleaved forward / backward pairs,
+// therefore never see each other's state; a buffer no forward call has filled, or one whose ticket was already
+// claimed, is refused.  At most MAX_PARKED forward calls are kept; the oldest is dropped first.
 // checkpoint_interval is accepted and ignored.
 #include <torch/extension.h>
 
@@ -63,9 +69,47 @@ struct Saved {
     torch::Tensor mf, mb, workspace;
     std::vector<Sg2Tensor> tensors;
     int64_t total = 0;
+    const void* x_sorted_ptr = nullptr;
 };
 std::mutex g_mutex;
-std::map<const void*, Saved> g_saved;          // keyed by x_sorted_packed.data_ptr()
+std::map<uint64_t, Saved> g_saved;             // keyed by ticket; std::map iterates in ticket order = age
+uint64_t g_next_ticket = 1;
+constexpr size_t MAX_PARKED = 16;
+constexpr uint32_t TICKET_MAGIC = 0x5347324Bu;  // "SG2K"
+
+// Parks a forward call and writes its ticket into the caller's fwd_saved_states tensor: [magic, low, high, ~magic].
+void park(const char* fn, Saved&& S, torch::Tensor& tag) {
+    TORCH_CHECK(tag.defined() && tag.is_cuda() && tag.scalar_type() == torch::kFloat32 && tag.is_contiguous() && tag.numel() >= 4, fn,
+                ": fwd_saved_states must be a contiguous float32 GPU tensor of at least 4 elements (it carries the ticket of this call)");
+    uint64_t ticket;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        ticket = g_next_ticket++;
+        while (g_saved.size() >= MAX_PARKED) g_saved.erase(g_saved.begin());     // forward calls never followed by a backward call: oldest first
+        g_saved.emplace(ticket, std::move(S));
+    }
+    torch::Tensor words = torch::empty({4}, torch::kInt32);
+    int32_t* w = words.data_ptr<int32_t>();
+    w[0] = (int32_t)TICKET_MAGIC; w[1] = (int32_t)(uint32_t)ticket; w[2] = (int32_t)(uint32_t)(ticket >> 32); w[3] = (int32_t)~TICKET_MAGIC;
+    tag.view({-1}).narrow(0, 0, 4).view(torch::kInt32).copy_(words);
+}
+
+// Reads the ticket back and takes the parked call out of the table.
+Saved claim(const char* fn, const char* fwd_name, const torch::Tensor& tag) {
+    TORCH_CHECK(tag.defined() && tag.is_cuda() && tag.scalar_type() == torch::kFloat32 && tag.is_contiguous() && tag.numel() >= 4, fn,
+                ": fwd_saved_states must be the tensor the forward call received");
+    const torch::Tensor words = tag.view({-1}).narrow(0, 0, 4).view(torch::kInt32).cpu();
+    const int32_t* w = words.data_ptr<int32_t>();
+    const bool tagged = (uint32_t)w[0] == TICKET_MAGIC && (uint32_t)w[3] == ~TICKET_MAGIC;
+    const uint64_t ticket = (uint64_t)(uint32_t)w[1] | ((uint64_t)(uint32_t)w[2] << 32);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    const auto it = tagged ? g_saved.find(ticket) : g_saved.end();
+    TORCH_CHECK(it != g_saved.end(), fn, ": no ", fwd_name, " call has filled these buffers, or its backward pass has already run "
+                "(the backward pass restarts from what that call kept; one forward call, then one backward call)");
+    Saved S = std::move(it->second);
+    g_saved.erase(it);
+    return S;
+}
 
 void run_forward(const char* fn, Saved& S, const SgDims& dims, torch::Tensor fwd_scan_out, torch::Tensor bwd_scan_out, torch::Tensor x_sorted,
                  torch::Tensor sort_indices) {
@@ -94,6 +138,7 @@ void run_forward(const char* fn, Saved& S, const SgDims& dims, torch::Tensor fwd
     }
     require_f32_gpu(x_sorted, fn, "x_sorted");
     TORCH_CHECK(x_sorted.numel() == S.total * dims.d_model, fn, ": x_sorted must hold [sum N, d_model] floats");
+    S.x_sorted_ptr = x_sorted.data_ptr();
     TORCH_CHECK(sort_indices.is_cuda() && sort_indices.scalar_type() == torch::kInt32 && sort_indices.is_contiguous() &&
                     sort_indices.numel() == S.total, fn, ": sort_indices must be a contiguous int32 GPU tensor of sum N entries");
     const size_t bytes = sg2_bilevel_workspace_bytes(&dims, (int)P, numels.data());
@@ -151,9 +196,7 @@ void supergrok2_bilevel_fwd_save_batched(
     std::vector<int32_t> off(P + 1, 0);
     for (int64_t i = 0; i < P; i++) off[i + 1] = off[i] + (int32_t)grads[i].numel();
     offsets_t.copy_(torch::from_blob(off.data(), {P + 1}, torch::kInt32).clone());
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (g_saved.size() >= 4) g_saved.clear();          // forward calls that were never followed by a backward call
-    g_saved[x_sorted_packed.data_ptr()] = std::move(S);
+    park(fn, std::move(S), fwd_saved_states_packed);
 }
 
 void supergrok2_bilevel_backward_batched(
@@ -174,16 +217,9 @@ void supergrok2_bilevel_backward_batched(
     const char* fn = "supergrok2_bilevel_backward_batched";
     (void)checkpoint_interval;
     if (num_params == 0) return;
-    Saved S;
-    {
-        std::lock_guard<std::mutex> lock(g_mutex);
-        const auto it = g_saved.find(x_sorted_packed.data_ptr());
-        TORCH_CHECK(it != g_saved.end(), fn, ": no supergrok2_bilevel_fwd_save_batched call has filled this x_sorted_packed tensor "
-                    "(the backward pass restarts from what that call kept)");
-        S = std::move(it->second);
-        g_saved.erase(it);
-    }
+    Saved S = claim(fn, "supergrok2_bilevel_fwd_save_batched", fwd_saved_states_packed);
     TORCH_CHECK((int)S.grads.size() == num_params, fn, ": num_params differs from the forward call");
+    TORCH_CHECK(S.x_sorted_ptr == x_sorted_packed.data_ptr(), fn, ": x_sorted_packed is not the tensor the forward call filled");
     const torch::Tensor given[16] = {mamba_fwd_in_proj, mamba_fwd_dt_W, mamba_fwd_dt_b, mamba_fwd_B_proj, mamba_fwd_C_proj, mamba_fwd_A_log,
                                      mamba_fwd_D, mamba_fwd_rope, mamba_bwd_in_proj, mamba_bwd_dt_W, mamba_bwd_dt_b, mamba_bwd_B_proj,
                                      mamba_bwd_C_proj, mamba_bwd_A_log, mamba_bwd_D, mamba_bwd_rope};
@@ -262,4 +298,176 @@ void supergrok2_bilevel_fwd_save(
     require_f32_gpu(bwd_final_state, fn, "bwd_final_state");
     fwd_final_state.view({-1}).copy_(S.mf.view({-1}));
     bwd_final_state.view({-1}).copy_(S.mb.view({-1}));
+    park(fn, std::move(S), fwd_saved_states);
+}
+
+
+// One tensor, the whole meta-net (csrc/ops.h:256-299, launch_mamba3_peer_backward in
+// csrc/supergrok2_mamba_peer_backward_kernels.cu:2745-3098 of the reference).  The caller has run the per-element
+// part of the forward pass itself, in torch, and hands over what it saw there (gates, candidates, routing weights,
+// hidden activations of the picked experts ...), so the per-element backward is a chain of small dense products over
+// those saved values and is written with ATen calls here, step for step as the reference's launcher orders it
+// (experts and routing, GRU, context gradients, sort, out_proj); the scan's adjoint -- the expensive part -- is the
+// HIP pass of sg2_bilevel_backward_ex on the workspace the forward call parked, and the input projection is one
+// more product.  Every d_* argument is accumulated into.  (The reference overwrites d_B_proj / d_C_proj with the
+// current tensor's term, `torch::mm_out` at :2999-3000 and :3045-3046 there, so that after its loop over parameters
+// only the last one's contribution is left; this function adds like it does everywhere else.)
+void supergrok2_bilevel_backward(
+    torch::Tensor d_smart_grad, torch::Tensor grad, torch::Tensor sharpness, float rescale, torch::Tensor sort_indices, torch::Tensor x_sorted,
+    torch::Tensor fwd_scan_out, torch::Tensor bwd_scan_out, torch::Tensor fwd_saved_states, torch::Tensor fwd_saved_x_branch,
+    torch::Tensor fwd_saved_z, torch::Tensor fwd_saved_dt, torch::Tensor bwd_saved_states, torch::Tensor bwd_saved_x_branch,
+    torch::Tensor bwd_saved_z, torch::Tensor bwd_saved_dt, torch::Tensor gru_input, torch::Tensor gru_h_old, torch::Tensor gru_z_gate,
+    torch::Tensor gru_r_gate, torch::Tensor gru_h_tilde, torch::Tensor peer_input, torch::Tensor expert_indices, torch::Tensor routing_weights,
+    torch::Tensor saved_z_hidden, torch::Tensor saved_scores_a, torch::Tensor saved_scores_b, torch::Tensor saved_top_a_idx,
+    torch::Tensor saved_top_b_idx, torch::Tensor saved_soft_a, torch::Tensor saved_soft_b, torch::Tensor mamba_fwd_in_proj,
+    torch::Tensor mamba_fwd_dt_W, torch::Tensor mamba_fwd_dt_b, torch::Tensor mamba_fwd_B_proj, torch::Tensor mamba_fwd_C_proj,
+    torch::Tensor mamba_fwd_A_log, torch::Tensor mamba_fwd_D, torch::Tensor mamba_fwd_rope, torch::Tensor mamba_fwd_out_proj,
+    torch::Tensor mamba_bwd_in_proj, torch::Tensor mamba_bwd_dt_W, torch::Tensor mamba_bwd_dt_b, torch::Tensor mamba_bwd_B_proj,
+    torch::Tensor mamba_bwd_C_proj, torch::Tensor mamba_bwd_A_log, torch::Tensor mamba_bwd_D, torch::Tensor mamba_bwd_rope,
+    torch::Tensor mamba_bwd_out_proj, torch::Tensor gru_Wz, torch::Tensor gru_Wr, torch::Tensor gru_Wh, torch::Tensor peer_query_Ws,
+    torch::Tensor prod_keys_A, torch::Tensor prod_keys_B, torch::Tensor expert_W1, torch::Tensor expert_W2, torch::Tensor expert_b1_in,
+    torch::Tensor expert_b2_in, torch::Tensor input_proj_W, torch::Tensor mamba_fwd_init_state, torch::Tensor mamba_bwd_init_state,
+    torch::Tensor d_mamba_fwd_in_proj, torch::Tensor d_mamba_fwd_dt_W, torch::Tensor d_mamba_fwd_dt_b, torch::Tensor d_mamba_fwd_B_proj,
+    torch::Tensor d_mamba_fwd_C_proj, torch::Tensor d_mamba_fwd_A_log, torch::Tensor d_mamba_fwd_D, torch::Tensor d_mamba_fwd_rope,
+    torch::Tensor d_mamba_fwd_out_proj, torch::Tensor d_mamba_bwd_in_proj, torch::Tensor d_mamba_bwd_dt_W, torch::Tensor d_mamba_bwd_dt_b,
+    torch::Tensor d_mamba_bwd_B_proj, torch::Tensor d_mamba_bwd_C_proj, torch::Tensor d_mamba_bwd_A_log, torch::Tensor d_mamba_bwd_D,
+    torch::Tensor d_mamba_bwd_rope, torch::Tensor d_mamba_bwd_out_proj, torch::Tensor d_gru_Wz, torch::Tensor d_gru_bz, torch::Tensor d_gru_Wr,
+    torch::Tensor d_gru_br, torch::Tensor d_gru_Wh, torch::Tensor d_gru_bh, torch::Tensor d_peer_query_Ws, torch::Tensor d_prod_keys_A,
+    torch::Tensor d_prod_keys_B, torch::Tensor d_expert_W1, torch::Tensor d_expert_b1, torch::Tensor d_expert_W2, torch::Tensor d_expert_b2,
+    torch::Tensor d_input_proj_W, torch::Tensor d_input_proj_b, int d_model, int d_state, int d_inner, int gru_hidden, int gru_input_dim,
+    int num_heads, int topk, int pk_dim, int expert_hidden, int peer_input_dim, int num_experts, int checkpoint_interval) {
+    const char* fn = "supergrok2_bilevel_backward";
+    (void)checkpoint_interval; (void)fwd_saved_x_branch; (void)fwd_saved_z; (void)fwd_saved_dt; (void)bwd_saved_states;
+    (void)bwd_saved_x_branch; (void)bwd_saved_z; (void)bwd_saved_dt; (void)mamba_fwd_init_state; (void)mamba_bwd_init_state;
+    (void)input_proj_W; (void)expert_b1_in; (void)saved_scores_a; (void)saved_scores_b;
+    const int64_t N = d_smart_grad.numel();
+    if (N == 0) return;
+    if (!d_smart_grad.is_cuda()) throw std::runtime_error("supergrok2_bilevel_backward requires CUDA tensors.");
+    torch::NoGradGuard no_grad;
+    const SgDims dims = default_dims(d_model, d_state, d_inner);
+    Saved S = claim(fn, "supergrok2_bilevel_fwd_save", fwd_saved_states);
+    TORCH_CHECK(S.grads.size() == 1 && S.total == N, fn, ": the forward call on these buffers had ", S.total, " elements, this call has ", N);
+    TORCH_CHECK(S.x_sorted_ptr == x_sorted.data_ptr(), fn, ": x_sorted is not the tensor the forward call filled");
+    const int64_t H = num_heads, A = (int64_t)topk * topk, eh = expert_hidden, E = num_experts, hd = d_model / 2, gh = gru_hidden;
+    TORCH_CHECK(gru_input_dim == 2 + 2 * d_model && peer_input_dim == gh + 2 * d_model + 2, fn, ": gru_input_dim / peer_input_dim do not match d_model and gru_hidden");
+    auto f32 = [](const torch::Tensor& t) { return t.to(torch::kFloat32).contiguous(); };
+    const torch::Tensor g = f32(grad).reshape({N});
+    const torch::Tensor s = f32(sharpness).reshape({N});
+    const torch::Tensor pin = f32(peer_input).reshape({N, peer_input_dim});
+    // ---- 1: d(total expert output) = rescale * d_smart_grad; every head contributes 1/H of it
+    const torch::Tensor d_head = (f32(d_smart_grad).reshape({N}) * rescale / (double)H).unsqueeze(1);                  // [N,1]
+    // ---- 2: experts and soft top-k routing, head by head
+    const torch::Tensor eidx = expert_indices.reshape({N, H, A}).to(torch::kLong);
+    const torch::Tensor rw = f32(routing_weights).reshape({N, H, A});
+    const torch::Tensor zh = f32(saved_z_hidden).reshape({N, H, A, eh});
+    const torch::Tensor top_a = saved_top_a_idx.reshape({N, H, topk}).to(torch::kLong), top_b = saved_top_b_idx.reshape({N, H, topk}).to(torch::kLong);
+    const torch::Tensor soft_a = f32(saved_soft_a).reshape({N, H, topk}), soft_b = f32(saved_soft_b).reshape({N, H, topk});
+    const torch::Tensor W2 = f32(expert_W2).reshape({E, eh}), b2 = f32(expert_b2_in).reshape({E});
+    torch::Tensor d_pin = torch::zeros({N, peer_input_dim}, pin.options());
+    torch::Tensor dW1 = torch::zeros({E, eh}, pin.options()), db1 = torch::zeros({E, eh}, pin.options()), dW2 = torch::zeros({E, eh}, pin.options());
+    torch::Tensor db2 = torch::zeros({E}, pin.options());
+    const torch::Tensor Wq = f32(peer_query_Ws).reshape({H, d_model, peer_input_dim});
+    const torch::Tensor KA = f32(prod_keys_A).reshape({H, pk_dim, hd}), KB = f32(prod_keys_B).reshape({H, pk_dim, hd});
+    for (int64_t h = 0; h < H; h++) {
+        const torch::Tensor idx = eidx.select(1, h);                                   // [N,A]
+        const torch::Tensor z = zh.select(1, h);                                       // [N,A,eh]  relu(W1 g + b1) of the picked experts
+        const torch::Tensor w2 = W2.index_select(0, idx.reshape({-1})).reshape({N, A, eh});
+        const torch::Tensor out_k = (w2 * z).sum(-1) + b2.index_select(0, idx.reshape({-1})).reshape({N, A});
+        const torch::Tensor d_out = rw.select(1, h) * d_head;                          // [N,A]
+        const torch::Tensor d_rw = out_k * d_head;                                     // [N,A]
+        const torch::Tensor dz = d_out.unsqueeze(-1) * w2 * (z > 0).to(torch::kFloat32);    // through the ReLU
+        const torch::Tensor flat = idx.reshape({-1});
+        dW2.index_add_(0, flat, (d_out.unsqueeze(-1) * z).reshape({N * A, eh}));
+        db2.index_add_(0, flat, d_out.reshape({-1}));
+        dW1.index_add_(0, flat, (dz * g.reshape({N, 1, 1})).reshape({N * A, eh}));
+        db1.index_add_(0, flat, dz.reshape({N * A, eh}));
+        // routing weight of expert (i, j) is soft_a[i] * soft_b[j]
+        const torch::Tensor d_rw2 = d_rw.reshape({N, topk, topk});
+        const torch::Tensor sa = soft_a.select(1, h), sb = soft_b.select(1, h);
+        const torch::Tensor d_sa = (d_rw2 * sb.unsqueeze(1)).sum(2), d_sb = (d_rw2 * sa.unsqueeze(2)).sum(1);
+        // softmax of 10 x the k best scores
+        const torch::Tensor d_va = 10.0 * sa * (d_sa - (sa * d_sa).sum(-1, true)), d_vb = 10.0 * sb * (d_sb - (sb * d_sb).sum(-1, true));
+        torch::Tensor d_score_a = torch::zeros({N, pk_dim}, pin.options()), d_score_b = torch::zeros({N, pk_dim}, pin.options());
+        d_score_a.scatter_add_(1, top_a.select(1, h), d_va);
+        d_score_b.scatter_add_(1, top_b.select(1, h), d_vb);
+        const torch::Tensor q = torch::mm(pin, Wq[h].t());                             // [N,d_model]
+        d_prod_keys_A.view({H, pk_dim, hd})[h].addmm_(d_score_a.t(), q.narrow(1, 0, hd));
+        d_prod_keys_B.view({H, pk_dim, hd})[h].addmm_(d_score_b.t(), q.narrow(1, hd, hd));
+        const torch::Tensor d_q = torch::cat({torch::mm(d_score_a, KA[h]), torch::mm(d_score_b, KB[h])}, 1);      // [N,2 hd]
+        d_peer_query_Ws.view({H, d_model, peer_input_dim})[h].narrow(0, 0, 2 * hd).addmm_(d_q.t(), pin);
+        d_pin.addmm_(d_q, Wq[h].narrow(0, 0, 2 * hd));
+    }
+    d_expert_W1.view({E, eh}).add_(dW1);
+    d_expert_b1.view({E, eh}).add_(db1);
+    d_expert_W2.view({E, eh}).add_(dW2);
+    d_expert_b2.view({E}).add_(db2);
+    // ---- 3, 4: GRU.  h' = (1 - z) h + z h~, gates over [input, h], candidate over [input, r * h]
+    const torch::Tensor d_hn = d_pin.narrow(1, 0, gh);
+    const torch::Tensor inp = f32(gru_input).reshape({N, gru_input_dim}), h_old = f32(gru_h_old).reshape({N, gh});
+    const torch::Tensor zg = f32(gru_z_gate).reshape({N, gh}), rg = f32(gru_r_gate).reshape({N, gh}), ht = f32(gru_h_tilde).reshape({N, gh});
+    const torch::Tensor Wz = f32(gru_Wz).reshape({gh, gru_input_dim + gh}), Wr = f32(gru_Wr).reshape({gh, gru_input_dim + gh}), Wh = f32(gru_Wh).reshape({gh, gru_input_dim + gh});
+    const torch::Tensor d_pre_h = d_hn * zg * (1.0 - ht * ht);
+    const torch::Tensor d_pre_z = d_hn * (ht - h_old) * zg * (1.0 - zg);
+    const torch::Tensor xh = torch::cat({inp, h_old}, 1), xrh = torch::cat({inp, rg * h_old}, 1);
+    const torch::Tensor d_xrh = torch::mm(d_pre_h, Wh);
+    const torch::Tensor d_pre_r = d_xrh.narrow(1, gru_input_dim, gh) * h_old * rg * (1.0 - rg);
+    d_gru_Wh.view({gh, gru_input_dim + gh}).addmm_(d_pre_h.t(), xrh);
+    d_gru_bh.view({gh}).add_(d_pre_h.sum(0));
+    d_gru_Wz.view({gh, gru_input_dim + gh}).addmm_(d_pre_z.t(), xh);
+    d_gru_bz.view({gh}).add_(d_pre_z.sum(0));
+    d_gru_Wr.view({gh, gru_input_dim + gh}).addmm_(d_pre_r.t(), xh);
+    d_gru_br.view({gh}).add_(d_pre_r.sum(0));
+    const torch::Tensor d_inp = d_xrh.narrow(1, 0, gru_input_dim) + torch::mm(d_pre_z, Wz).narrow(1, 0, gru_input_dim) +
+                                torch::mm(d_pre_r, Wr).narrow(1, 0, gru_input_dim);
+    // ---- 5, 6: context gradients (GRU input [g, s, fwd, bwd]; query input [h', fwd, bwd, g, s]), into scan order
+    const torch::Tensor d_ctx_f = d_inp.narrow(1, 2, d_model) + d_pin.narrow(1, gh, d_model);
+    const torch::Tensor d_ctx_b = d_inp.narrow(1, 2 + d_model, d_model) + d_pin.narrow(1, gh + d_model, d_model);
+    const torch::Tensor order = sort_indices.reshape({N}).to(torch::kLong);
+    const torch::Tensor d_f_sorted = d_ctx_f.index_select(0, order), d_b_sorted = d_ctx_b.index_select(0, order).flip(0).contiguous();
+    // ---- 7: out_proj of both directions
+    const torch::Tensor fso = f32(fwd_scan_out).reshape({N, d_inner}), bso = f32(bwd_scan_out).reshape({N, d_inner});
+    d_mamba_fwd_out_proj.view({d_model, d_inner}).addmm_(d_f_sorted.t(), fso);
+    d_mamba_bwd_out_proj.view({d_model, d_inner}).addmm_(d_b_sorted.t(), bso);
+    const torch::Tensor d_fso = torch::mm(d_f_sorted, f32(mamba_fwd_out_proj).reshape({d_model, d_inner})).contiguous();
+    const torch::Tensor d_bso = torch::mm(d_b_sorted, f32(mamba_bwd_out_proj).reshape({d_model, d_inner})).contiguous();
+    // ---- 8: the scan's adjoint in HIP, on what the forward call kept
+    const torch::Tensor given[16] = {mamba_fwd_in_proj, mamba_fwd_dt_W, mamba_fwd_dt_b, mamba_fwd_B_proj, mamba_fwd_C_proj, mamba_fwd_A_log,
+                                     mamba_fwd_D, mamba_fwd_rope, mamba_bwd_in_proj, mamba_bwd_dt_W, mamba_bwd_dt_b, mamba_bwd_B_proj,
+                                     mamba_bwd_C_proj, mamba_bwd_A_log, mamba_bwd_D, mamba_bwd_rope};
+    for (int dir = 0; dir < 2; dir++)
+        for (int k = 0; k < 8; k++)
+            TORCH_CHECK(given[dir * 8 + k].data_ptr() == S.w.t[2 + dir * 9 + k].data_ptr(), fn, ": the Mamba weights must be the tensors the forward call received");
+    std::vector<torch::Tensor> rows;
+    for (int dir = 0; dir < 2; dir++) {
+        const torch::Tensor& in_proj = S.w.t[2 + dir * 9];
+        const torch::Tensor X = in_proj.view({2 * d_inner, d_model}).narrow(0, 0, d_inner), Z = in_proj.view({2 * d_inner, d_model}).narrow(0, d_inner, d_inner);
+        rows.push_back(torch::cat({X, Z, torch::mm(S.w.t[3 + dir * 9].view({d_inner, d_inner}), X), torch::mm(S.w.t[5 + dir * 9].view({d_state, d_inner}), X),
+                                   torch::mm(S.w.t[6 + dir * 9].view({d_state, d_inner}), X)}, 0));
+    }
+    const torch::Tensor row_dx = torch::stack(rows, 0).contiguous();
+    torch::Tensor dx = torch::empty({2, N, (int64_t)d_model}, pin.options()), block = torch::empty({SG2_SCAN_GRAD_FLOATS}, pin.options());
+    const int rc = sg2_bilevel_backward_ex(&dims, &S.w.W, 1, S.tensors.data(), nullptr, d_fso.data_ptr<float>(), d_bso.data_ptr<float>(),
+                                           row_dx.data_ptr<float>(), dx.data_ptr<float>(), block.data_ptr<float>(), S.workspace.data_ptr(),
+                                           (size_t)S.workspace.numel(), stream_of(block));
+    TORCH_CHECK(rc == 0, fn, ": ", sg_last_error());
+    torch::Tensor d_out[16] = {d_mamba_fwd_in_proj, d_mamba_fwd_dt_W, d_mamba_fwd_dt_b, d_mamba_fwd_B_proj, d_mamba_fwd_C_proj, d_mamba_fwd_A_log,
+                               d_mamba_fwd_D, d_mamba_fwd_rope, d_mamba_bwd_in_proj, d_mamba_bwd_dt_W, d_mamba_bwd_dt_b, d_mamba_bwd_B_proj,
+                               d_mamba_bwd_C_proj, d_mamba_bwd_A_log, d_mamba_bwd_D, d_mamba_bwd_rope};
+    int64_t at = 3 * d_model;
+    for (int dir = 0; dir < 2; dir++) {
+        for (int k = 0; k < 8; k++) {
+            torch::Tensor& d = d_out[dir * 8 + k];
+            require_f32_gpu(d, fn, "gradient accumulator");
+            TORCH_CHECK(d.numel() == S.w.t[2 + dir * 9 + k].numel(), fn, ": gradient accumulator ", dir * 8 + k, " has the wrong size");
+            d.view({-1}).add_(block.narrow(0, at, d.numel()));
+            at += d.numel();
+        }
+        at += (int64_t)d_model * d_inner;       // out_proj: formed above from the scan outputs
+    }
+    // ---- 9: input projection, x = W [g, s] + b in element order
+    const torch::Tensor d_x_sorted = dx[0] + dx[1];
+    const torch::Tensor unsort = torch::empty_like(order).scatter_(0, order, torch::arange(N, order.options()));
+    const torch::Tensor d_x = d_x_sorted.index_select(0, unsort);
+    d_input_proj_W.view({d_model, 2}).addmm_(d_x.t(), torch::stack({g, s}, 1));
+    d_input_proj_b.view({d_model}).add_(d_x.sum(0));
 }

@@ -648,6 +648,18 @@ void supergrok2_bilevel_fwd_save(
     torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int, int, int, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
     torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
     torch::Tensor, torch::Tensor, torch::Tensor, int);
+void supergrok2_bilevel_backward(
+    torch::Tensor, torch::Tensor, torch::Tensor, float, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor,
+    torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, int, int, int, int, int, int, int, int, int, int, int, int);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "Grokking optimizers: fused steps on MI355X (hand-written HIP behind the reference's _ops surface)";
@@ -731,11 +743,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("supergrok2_bilevel_fwd_save_batched", &supergrok2_bilevel_fwd_save_batched,
           "SuperGrok2 bilevel: batched forward scan with state saving");
     m.def("supergrok2_bilevel_backward_batched", &supergrok2_bilevel_backward_batched, "SuperGrok2 bilevel: batched backward through scan");
-    m.def("supergrok2_bilevel_backward", [](py::args, py::kwargs) {
-        throw std::runtime_error(
-            "supergrok2_bilevel_backward (one tensor, whole meta-net) is not provided: its argument list carries the saved gate values of "
-            "the GRU instead of the GRU biases, and the HIP per-element kernel recomputes the forward pass from the weights. Use "
-            "supergrok2_bilevel_fwd_save_batched / supergrok2_bilevel_backward_batched (which the reference's caller prefers whenever they "
-            "exist), or SuperGrok2.bilevel_step of this package.");
-    }, "SuperGrok2 bilevel: full backward through meta-net (raises: see the message)");
+    m.def("supergrok2_bilevel_backward", &supergrok2_bilevel_backward, "SuperGrok2 bilevel: full backward through meta-net");
 }

@@ -25,7 +25,9 @@ std::atomic<int> g_window{SG2_DEFAULT_SCAN_WINDOW};
 
 // What the forward call of the bilevel pass laid out in a workspace, so that the backward call addresses it the same
 // way whatever the settings are by then.  Keyed by the workspace address.
-struct BilevelRecord { int chunk_len, window, P, total; };
+struct BilevelRecord { int chunk_len, window, P, total; uint64_t seq; };
+uint64_t g_bilevel_seq = 0;
+constexpr size_t MAX_BILEVEL_RECORDS = 64;
 std::mutex g_bilevel_mutex;
 std::map<const void*, BilevelRecord> g_bilevel_records;
 
@@ -534,8 +536,15 @@ int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int nu
     if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, true, false, st, &pl, &L)) return 1;
     {
         std::lock_guard<std::mutex> lock(g_bilevel_mutex);
-        if (g_bilevel_records.size() > 64) g_bilevel_records.clear();       // forgotten workspaces: bounded memory
-        g_bilevel_records[workspace] = BilevelRecord{pl.total > 0 ? pl.chunk_len : 0, pl.total > 0 ? pl.window : 0, num_tensors, pl.total};
+        // bounded memory: a workspace whose forward call is the oldest on record is forgotten first (a live pair of
+        // forward and backward calls is only ever separated by the calls of other workspaces still in use)
+        while (g_bilevel_records.size() >= MAX_BILEVEL_RECORDS && g_bilevel_records.find(workspace) == g_bilevel_records.end()) {
+            auto oldest = g_bilevel_records.begin();
+            for (auto it = g_bilevel_records.begin(); it != g_bilevel_records.end(); ++it)
+                if (it->second.seq < oldest->second.seq) oldest = it;
+            g_bilevel_records.erase(oldest);
+        }
+        g_bilevel_records[workspace] = BilevelRecord{pl.total > 0 ? pl.chunk_len : 0, pl.total > 0 ? pl.window : 0, num_tensors, pl.total, ++g_bilevel_seq};
     }
     if (pl.total == 0) return 0;
     if (ctx_out) pl.ctx = ctx_out;                 // else the contexts stay in the workspace
