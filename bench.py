@@ -20,20 +20,46 @@ for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd")):
 
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch (read + written) on the 25M-element workload: constants copied from the rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE summary under profiles/ (scaled by what the same counters read for a 1 GiB device copy);
-# not measured by this script and valid for the default workload only
-PMC_TRAFFIC_BYTES_SCALE50 = {"scan_output": 0.513e9 + 2.501e9, "scan_summary": 0.028e9 + 0.049e9,
-                             "elementwise": 2.503e9 + 0.801e9}
-
-
-# Vector-ALU instructions per launch (SQ_INSTS_VALU of the same profile, default workload only) and the rate the part
-# sustains on nothing but independent fp32 instructions (bench.py --workload valu-probe, profiles/valu_probe_mi355x.txt):
-# what actually bounds these kernels
-# (the per-element kernel's count holds 8.6e6 fp32 matrix instructions of 64 clocks each: 16 vector instructions' worth of time apiece)
-PMC_VALU_INSTS_SCALE50 = {"scan_output": 1.89e9, "scan_summary": 1.16e8, "elementwise": 6.19e8 + 15 * 8.6e6}
-VALU_SUSTAINED_PER_NS_SIMD = 0.59
 SIMDS = 1024
+STAGE_KERNEL_PREFIX = {"scan_output": "k_scan<true, false>", "scan_summary": "k_scan<false, false>", "elementwise": "k_elem<"}
+
+
+def profile_figures():
+    """What the rocprofv3 counter runs committed under profiles/ say about the kernels of the default workload, per
+    stage: HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, scaled as that file describes), vector-ALU instructions per
+    launch, and the instruction rate the part sustains on nothing but independent fp32 instructions.  Read from the
+    text summaries at run time, so a figure can never drift from the file it is quoted from; None where a file or a
+    row is missing.  These are figures of the profiled build, not measurements of this run: the JSON names the files."""
+    out = {"traffic": {}, "valu": {}, "sustained": None, "source": {}}
+    pdir = os.path.join(ROOT, "profiles")
+
+    def rows(name):
+        try:
+            with open(os.path.join(pdir, name)) as f:
+                return f.read().splitlines()
+        except OSError:
+            return []
+    for stage, prefix in STAGE_KERNEL_PREFIX.items():
+        for line in rows("sg2_step_scale50_pmc_traffic.txt"):
+            if line.startswith(prefix):
+                cols = line.split()
+                out["traffic"][stage] = (float(cols[-2]) + float(cols[-1])) * 1e9        # read_GB + written_GB
+        for line in rows("sg2_step_scale50_pmc_sq.txt"):
+            if line.startswith(prefix):
+                cols = line[40:].split()                                                   # after the (truncated) kernel name
+                out["valu"][stage] = float(cols[1])                                        # us/launch, INSTS_VALU, ...
+    best = 0.0
+    for line in rows("valu_probe_mi355x.txt"):
+        cols = line.split()
+        if len(cols) >= 5 and cols[0] in ("fma", "mul", "add", "add_dpp"):
+            try:
+                best = max(best, float(cols[3]))
+            except ValueError:
+                pass
+    out["sustained"] = best or None
+    out["source"] = {"traffic": "profiles/sg2_step_scale50_pmc_traffic.txt", "valu": "profiles/sg2_step_scale50_pmc_sq.txt",
+                     "sustained": "profiles/valu_probe_mi355x.txt"}
+    return out
 
 
 LARGE_GEOMETRY = dict(d_model=16, d_state=32, d_inner=32)     # the second scan geometry the kernels are built for
@@ -323,6 +349,210 @@ def bench_probe(dev):
             "rows": rows}
 
 
+def make_v2_step(st, weights, D, boundary="ops"):
+    """step(grads, sharps, per_tensor, shared) over the tensors of `st`: the reference's own entry point of the torch
+    extension (51 arguments), or the bare C-ABI call."""
+    from grokking_optimizers import _cabi
+    if boundary == "cabi":
+        return _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"], st["counts"], dims=D)
+    from grokking_optimizers import _ops
+
+    def step(grads, sharps_, per_tensor, sh):
+        col = lambda k: [float(sc[k]) for sc in per_tensor]
+        _ops.supergrok2_mamba_peer_batched_step(
+            st["params"], grads, sharps_, st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"], *weights,
+            col("alpha"), col("lamb_eff"), col("beta1"), col("bc1"), col("bc2"), sh["rescale"], sh["beta2"], sh["lr"],
+            sh["wd_eff"], sh["eps"], D["d_model"], D["d_state"], D["d_inner"], D["gru_hidden"], D["num_heads"],
+            D["pk_dim"], D["expert_hidden"], D["num_experts"], st["counts"])
+    return step
+
+
+def time_v2(step, P, grad_sets, sharps, steps, warmup, t0_step=0):
+    """W untimed calls, then exactly `steps` calls between two device synchronisations; per-stage times from HIP events
+    recorded on the step's stream.  Returns (seconds of the timed region, average stage ms, step counter)."""
+    import torch
+    from grokking_optimizers import _cabi
+    from workloads import per_tensor_scalars, shared_scalars
+    shared = shared_scalars()
+    t = t0_step
+    for _ in range(warmup):
+        t += 1
+        step(grad_sets[t & 1], sharps, per_tensor_scalars(P, t), shared)
+    torch.cuda.synchronize()
+    scal = [per_tensor_scalars(P, t + k + 1) for k in range(steps)]
+    _cabi.profile_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        t += 1
+        step(grad_sets[t & 1], sharps, scal[k], shared)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    stage_ms, calls = _cabi.profile_read()
+    _cabi.profile_enable(False)
+    assert calls == min(steps, 256)
+    return elapsed, {k: v / calls for k, v in stage_ms.items()}, t
+
+
+def finite_state(st):
+    import torch
+    return all(bool(torch.isfinite(x).all()) for lst in (st["params"], st["eas"], st["grus"]) for x in lst)
+
+
+def v2_variants(shapes, st, grad_sets, D, dev, steps=8, warmup=2):
+    """The headline set again under the inputs the headline figure is friendliest to, so that its dependence on them is
+    measured in the same run: a populated sharpness cache; the optimizer's own initial meta-net; gradients large enough
+    that no tile of the scan qualifies for a polynomial form (the general recurrence); and routing spread over many
+    experts (per-lane gathers of the expert records in the per-element kernel instead of broadcasts)."""
+    import torch
+    import workloads as wl
+    P, total = len(shapes), sum(p.numel() for p in st["params"])
+    out = {}
+
+    def run(name, weights, grads, sharps, note, fresh_gru=None):
+        for lst in (st["eas"], st["easqs"], st["mus"], st["mf"], st["mb"]):
+            for x in lst:
+                x.zero_()
+        for x, p0 in zip(st["params"], fresh_params):
+            x.copy_(p0)
+        for i, x in enumerate(st["grus"]):
+            x.zero_() if fresh_gru is None else x.copy_(fresh_gru[i])
+        st["counts"].zero_()
+        el, stage, _ = time_v2(make_v2_step(st, weights, D), P, grads, sharps, steps, warmup)
+        assert finite_state(st), name
+        counts = st["counts"].cpu()
+        out[name] = {"ms_per_step": 1e3 * el / steps, "elements_per_s": total * steps / el, "stage_ms": stage,
+                     "experts_used": int((counts > 0).sum()), "steps": steps, "what": note}
+    fresh_params = [p.clone() for p in st["params"]]
+    zeros = [torch.zeros_like(p) for p in st["params"]]
+    bench_w = [w.to(dev) for w in wl.meta_weights(7, D)]
+    run("sharpness", bench_w, grad_sets, [(g.abs() * 0.5).contiguous() for g in grad_sets[1]],
+        "sharpness cache populated (|g|/2 of the other gradient set): gather into sorted order, sharpness terms in the projections")
+    run("module_weights", [w.to(dev) for w in wl.module_weights(0)], grad_sets, zeros,
+        "meta-net as Mamba3PEERMetaNet() initialises it (A_log = log(1..16)): slower contraction, fewer blocks on the product forms")
+    big = [[(torch.sign(g) * (g.abs() * 100.0 + 0.5)).contiguous() for g in gs] for gs in grad_sets]
+    run("general_path", bench_w, big, zeros,
+        "every |g| >= 0.5: no tile takes the Taylor / lane-polynomial / product forms, every block runs the general recurrence")
+    del big
+    # routing: queries driven by a random GRU state through amplified h columns of the query matrices
+    spread_w = [w.clone() for w in bench_w]
+    spread_w[26][:, :, :D["gru_hidden"]] *= 30.0
+    gen = torch.Generator().manual_seed(11)
+    gru0 = [torch.randn(p.numel(), D["gru_hidden"], generator=gen).to(dev) for p in st["params"]]
+    run("spread_routing", spread_w, grad_sets, zeros,
+        "query rows amplified x30 on a random GRU state: elements of a wave pick different experts", fresh_gru=gru0)
+    return out
+
+
+def muon_precision(dev):
+    """One wide and one tall matrix of the Muon workload: this library's step (bf16 Newton-Schulz on the Gram matrix of
+    the smaller side, fp32 accumulation) against the reference's arithmetic (fp32 iteration on X X^T, csrc/ops.cpp:704-727
+    of the reference) restated with torch fp32 products on the device.  Fraction of updated bf16 parameters that differ
+    from the fp32-iteration result rounded to bf16 by more than one bf16 spacing, the fraction that round differently at
+    all, and the largest deviation in bf16 spacings."""
+    import torch
+    from grokking_optimizers import _ops
+    gen = torch.Generator().manual_seed(0)
+    res = {}
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        for name, shape in (("wide_1024x4096", (1024, 4096)), ("tall_4096x1024", (4096, 1024))):
+            p = (torch.randn(*shape, generator=gen) * 0.02).to(torch.bfloat16).to(dev)
+            g = (torch.randn(*shape, generator=gen) * 1e-3).to(torch.bfloat16).to(dev)
+            buf = torch.zeros(shape, device=dev)
+            p_new = p.clone()
+            _ops.muon_fused_step([p_new], [g], [buf], 0.95, 0.02, 1.0, 5)
+            X = g.float()
+            X = X / (X.norm() + 1e-7)
+            if shape[0] > shape[1]:
+                X = X.T                       # X X^T of the tall form and X^T X of its transpose give the same iteration
+            for _ in range(5):
+                A = X @ X.T
+                AX = A @ X
+                X = 3.4445 * X + (-4.7750) * AX + 2.0315 * (A @ AX)
+            if shape[0] > shape[1]:
+                X = X.T
+            want = ((p.float() - 0.2 * 0.02 * X) * (1.0 - 0.02 * 1.0)).to(torch.bfloat16)
+            ulp = torch.maximum(want.float().abs(), torch.tensor(1e-30, device=dev)).log2().floor().exp2() * 2.0 ** -7
+            diff = (p_new.float() - want.float()).abs()
+            res[name] = {"frac_beyond_one_bf16_ulp": float((diff > ulp * 1.0001).float().mean()),
+                         "frac_rounded_differently": float((diff > 0).float().mean()),
+                         "largest_deviation_in_bf16_ulps": float((diff / ulp).max())}
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    return res
+
+
+def secondary_configs(dev, steps=20, warmup=3):
+    """The other measured configurations, each timed in this run: Grokfast and SuperGrok v1.5 on the 14-tensor set, the
+    SuperGrok v2 step on the 14-tensor set, Muon on its 24 bf16 matrices (algorithmic and executed MFMA fraction)."""
+    import torch
+    from grokking_optimizers import _ops
+    out = {}
+    for name, workload in (("config1_grokfast", "grokfast"), ("config2_supergrok15", "sg15"), ("config5_muon", "muon")):
+        W = build_step(workload, _ops, dev)
+        for _ in range(warmup):
+            W["step"]()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            W["step"]()
+        torch.cuda.synchronize()
+        el = (time.perf_counter() - t0) / steps
+        r = {"workload": W["name"], "ms_per_step": 1e3 * el, "value": W["units"] / el, "unit": W["unit"], "dtype": W["dtype"], "steps": steps}
+        if W["bound"] == "mfma":
+            r["roofline"] = {"bound": "mfma", "peak": W["peak"], "unit": "TFLOP/s", "achieved": W["units"] / el / 1e12,
+                             "frac": W["units"] / el / 1e12 / W["peak"], "achieved_executed": W["executed"] / el / 1e12,
+                             "frac_executed": W["executed"] / el / 1e12 / W["peak"]}
+            r["precision"] = muon_precision(dev)
+        else:
+            bpe = W["bytes_per_elem"]
+            r["roofline"] = {"bound": "hbm", "peak": W["peak"], "unit": "GB/s", "achieved": bpe * W["units"] / el / 1e9,
+                             "frac": bpe * W["units"] / el / 1e9 / W["peak"], "bytes_per_element": bpe}
+        out[name] = r
+        del W
+    shapes, st, grad_sets, sharps, weights, D = build_workload("shared14", dev)
+    total = sum(p.numel() for p in st["params"])
+    el, stage, _ = time_v2(make_v2_step(st, weights, D), len(shapes), grad_sets, sharps, steps, warmup)
+    out["config3_supergrok2_shared14"] = {
+        "workload": "SuperGrok v2 full step, 14 tensors, %d elements" % total, "ms_per_step": 1e3 * el / steps, "value": total * steps / el,
+        "unit": "elements/s", "dtype": "f32", "steps": steps, "stage_ms": stage,
+        "roofline": {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s", "achieved": BYTES_PER_ELEMENT * total * steps / el / 1e9,
+                     "frac": BYTES_PER_ELEMENT * total * steps / el / 1e9 / HBM_PEAK_GBS, "bytes_per_element": BYTES_PER_ELEMENT}}
+    return out
+
+
+def aten_loop_baseline(max_elems=16384, budget_s=10.0):
+    """The per-timestep ATen restatement of the reference's CPU path (oracle/aten_loop.py) on the smallest tensors of the
+    50-tensor set, as many as fit the time budget; elements per second with the thread count."""
+    import torch
+    import workloads as wl
+    from oracle import aten_loop
+    shapes = wl.scale50_shapes()
+    W = wl.meta_weights(7)
+    D = wl.DEFAULT_DIMS
+    done, t0 = 0, time.perf_counter()
+    used = []
+    for i, sh in enumerate(shapes):
+        n = wl.numel(sh)
+        if n > max_elems or (used and time.perf_counter() - t0 > budget_s):
+            break
+        g = wl.make_grads([sh], seed=1 + i)[0].reshape(-1)
+        st = dict(param=wl.make_params([sh], seed=i)[0].reshape(-1), exp_avg=torch.zeros(n), exp_avg_sq=torch.zeros(n), mu=torch.zeros(n),
+                  gru=torch.zeros(n, D["gru_hidden"]), mamba_fwd=torch.zeros(D["d_inner"], D["d_state"]), mamba_bwd=torch.zeros(D["d_inner"], D["d_state"]))
+        sc = dict(wl.per_tensor_scalars(i + 1, 1)[i], **wl.shared_scalars())
+        sc["lamb_eff"] = sc.get("lamb_eff", 0.0)
+        with torch.no_grad():
+            aten_loop.step(W, st, g, torch.zeros_like(g), sc, D)
+        done += n
+        used.append(i)
+    dt = time.perf_counter() - t0
+    return {"value": done / dt, "unit": "elements/s", "threads": torch.get_num_threads(), "host_cpus": os.cpu_count(),
+            "sample": "tensors %d..%d of the 50-tensor set (%d elements, each at most %d), 1 step, per-timestep ATen loop in fp32, %.1f s; "
+                      "the 25 M element set would take about %.1f hours at this rate" % (used[0], used[-1], done, max_elems, dt, 25010032 / (done / dt) / 3600)}
+
+
 def class_step_ms(shapes, grad_sets, dev, steps, warmup):
     """Wall time of SuperGrok2.step() itself (per-tensor clip on the device, scalar schedules, the 51-argument
     `_ops` call), same tensors and gradients, the module's own initial meta-weights, recycling off."""
@@ -367,6 +597,7 @@ def main():
     ap.add_argument("--boundary", default="ops", choices=["ops", "cabi"],
                     help="v2 workloads: time the torch-extension call _ops.supergrok2_mamba_peer_batched_step (default) or the bare C-ABI call")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="default workload: skip the variants / secondary configurations / ATen-loop baseline that ride on the same run")
     ap.add_argument("--no-class-step", action="store_true", help="skip the wall time of SuperGrok2.step() (keeps a kernel trace to the C-ABI steps)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain device copy of 1 GiB (a reference point for scaling the FETCH_SIZE / "
@@ -379,7 +610,6 @@ def main():
 
     import torch
     from grokking_optimizers import _cabi
-    from workloads import per_tensor_scalars, shared_scalars
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
     if args.workload == "valu-probe":
@@ -394,54 +624,24 @@ def main():
         raise SystemExit("--geometry large runs with --weights bench")
     shapes, st, grad_sets, sharps, weights, D = build_workload(args.workload, dev, args.sharpness, args.weights, args.geometry)
     total = sum(p.numel() for p in st["params"])
-    if args.boundary == "cabi":
-        step = _cabi.Sg2Step(weights, st["params"], st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"],
-                             st["counts"], dims=D)
-    else:
-        # the reference's own entry point: supergrok2_mamba_peer_batched_step of the torch extension, 51 arguments
-        from grokking_optimizers import _ops
-
-        def step(grads, sharps_, per_tensor, sh):
-            col = lambda k: [float(sc[k]) for sc in per_tensor]
-            _ops.supergrok2_mamba_peer_batched_step(
-                st["params"], grads, sharps_, st["eas"], st["easqs"], st["mus"], st["grus"], st["mf"], st["mb"], *weights,
-                col("alpha"), col("lamb_eff"), col("beta1"), col("bc1"), col("bc2"), sh["rescale"], sh["beta2"], sh["lr"],
-                sh["wd_eff"], sh["eps"], D["d_model"], D["d_state"], D["d_inner"], D["gru_hidden"], D["num_heads"],
-                D["pk_dim"], D["expert_hidden"], D["num_experts"], st["counts"])
-    shared = shared_scalars()
+    step = make_v2_step(st, weights, D, args.boundary)
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    t = 0
-    for _ in range(args.warmup):
-        t += 1
-        step(grad_sets[t & 1], sharps, per_tensor_scalars(len(shapes), t), shared)
-    torch.cuda.synchronize()
-    scal = [per_tensor_scalars(len(shapes), t + k + 1) for k in range(args.steps)]
-    _cabi.profile_enable(True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        t += 1
-        step(grad_sets[t & 1], sharps, scal[k], shared)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    stage_ms, calls = _cabi.profile_read()
-    _cabi.profile_enable(False)
-    assert calls == min(args.steps, 256)
-    for lst in (st["params"], st["eas"], st["grus"]):
-        assert all(bool(torch.isfinite(x).all()) for x in lst), "non-finite state after the timed steps"
+    elapsed, stage_avg, _ = time_v2(step, len(shapes), grad_sets, sharps, args.steps, args.warmup)
+    assert finite_state(st), "non-finite state after the timed steps"
 
     ms_per_step = 1e3 * elapsed / args.steps
     value = total * args.steps / elapsed
-    stage_avg = {k: v / calls for k, v in stage_ms.items()}
     dom = max(stage_avg, key=stage_avg.get)
     kernel_of = {"sort": "k_keys + 4 x (k_hist, k_spine_*, k_scatter)", "scan_summary": "k_scan<false>",
                  "chunk_prefix": "k_chunk_prefix", "scan_output": "k_scan<true>", "elementwise": "k_elem<false>"}
     achieved = BYTES_PER_ELEMENT * total / (stage_avg[dom] * 1e-3) / 1e9
+    default_workload = (args.workload, args.weights, args.geometry, args.sharpness) == ("scale50", "bench", "default", False)
+    prof = profile_figures() if default_workload else {"traffic": {}, "valu": {}, "sustained": None, "source": {}}
     out = {
         "metric": "param-elements/sec per optimizer step (SuperGrok v2); % HBM roofline",
         "value": value, "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -454,20 +654,30 @@ def main():
                    "meta_weights": "N(0, 0.1), seed 7" if args.weights == "bench" else "Mamba3PEERMetaNet() initialisation, seed 0",
                    "meta_net": "d_model=%d d_state=%d d_inner=%d" % (D["d_model"], D["d_state"], D["d_inner"])},
         "roofline": {"bound": "hbm", "kernel": kernel_of[dom], "achieved": achieved, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": PMC_TRAFFIC_BYTES_SCALE50.get(dom) if (args.workload, args.weights, args.geometry) == ("scale50", "bench", "default") else None,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": prof["traffic"].get(dom),
+                     "traffic_source": prof["source"].get("traffic") if prof["traffic"].get(dom) is not None else None,
                      "kernel_ms": stage_avg[dom]},
         "step_hbm_frac": BYTES_PER_ELEMENT * value / 1e9 / HBM_PEAK_GBS,
         "stage_ms": stage_avg,
     }
-    if (args.workload, args.weights, args.geometry) == ("scale50", "bench", "default") and dom in PMC_VALU_INSTS_SCALE50:
-        rate = PMC_VALU_INSTS_SCALE50[dom] / (stage_avg[dom] * 1e6) / SIMDS       # wave instructions per ns and SIMD
-        out["valu"] = {"kernel": kernel_of[dom], "instructions": PMC_VALU_INSTS_SCALE50[dom], "per_ns_simd": rate,
-                       "sustained_per_ns_simd": VALU_SUSTAINED_PER_NS_SIMD, "frac": rate / VALU_SUSTAINED_PER_NS_SIMD}
+    if prof["valu"].get(dom) is not None and prof["sustained"]:
+        # instructions per launch as counted in the profiled run (the file is named) over THIS run's kernel time
+        rate = prof["valu"][dom] / (stage_avg[dom] * 1e6) / SIMDS       # wave instructions per ns and SIMD
+        out["valu"] = {"kernel": kernel_of[dom], "instructions": prof["valu"][dom], "instructions_source": prof["source"]["valu"],
+                       "per_ns_simd": rate, "sustained_per_ns_simd": prof["sustained"], "sustained_source": prof["source"]["sustained"],
+                       "frac": rate / prof["sustained"]}
     if not args.no_class_step and args.geometry == "default":
         out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
+    if default_workload and not args.no_extras:
+        # everything below is timed in this same run, after the headline's timed region
+        out["variants"] = v2_variants(shapes, st, grad_sets, D, dev)
+        del st, grad_sets, sharps, step
+        torch.cuda.empty_cache()
+        out["secondary"] = secondary_configs(dev)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        if default_workload and not args.no_extras:
+            out["cpu_baseline"]["aten_loop"] = aten_loop_baseline()
     print(json.dumps(out))
 
 

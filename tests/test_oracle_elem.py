@@ -157,3 +157,26 @@ def test_sam_helpers_golden_are_the_plain_formulas():
         # (csrc/ops.cpp:201), so the caller's sharpness tensor is never written there;
         # only its GPU kernel stores |g_sam - g| in place (csrc/supergrok15_kernels.cu:182).
         assert not z[f"sharp_out_{i}"].any()
+
+
+def test_aten_loop_matches_checker():
+    """oracle/aten_loop.py (the per-timestep ATen restatement bench.py times as the CPU baseline) against the float64
+    policy of the C++ checker on one small tensor: same routing, states within fp32 rounding of a 300-step recurrence."""
+    import torch
+    import workloads as wl
+    from helpers import default_scalars, f32_scalars, random_state_np, weights_np
+    from oracle import aten_loop
+    from oracle import oracle as orc
+    n = 300
+    W = weights_np()
+    st = random_state_np(n, 4)
+    r = np.random.RandomState(5)
+    g, s = (r.randn(n) * 1e-2).astype(np.float32), np.abs(r.randn(n) * 1e-2).astype(np.float32)
+    sc = f32_scalars(default_scalars(i=1, step=3, lamb_eff=2.0, wd_eff=4.5))
+    ts = {k: torch.from_numpy(v.copy()) for k, v in st.items()}
+    eidx = aten_loop.step([torch.from_numpy(w) for w in W], ts, torch.from_numpy(g), torch.from_numpy(s), sc, wl.DEFAULT_DIMS)
+    dbg = orc.sg2_step(W, st, g, s, sc, precision=64, chunk_len=0, debug=True)
+    assert np.array_equal(eidx.numpy().astype(np.int32), dbg["expert_idx"])
+    for k in ("param", "exp_avg", "exp_avg_sq", "mu", "gru", "mamba_fwd", "mamba_bwd"):
+        a, b = ts[k].numpy().reshape(st[k].shape).astype(np.float64), st[k].astype(np.float64)
+        assert np.all(np.abs(a - b) <= 2e-5 * np.maximum(np.abs(a), np.abs(b)) + 1e-7), k
