@@ -807,6 +807,401 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     }
 }
 
+// Projections of one timestep for the one-wave replay: the lane computes every row of every group for its timestep
+// (what the two waves of k_scan each do half of through project_tile, with the same expressions in the same order).
+// Step size, dt * x-branch, B and C go to LDS for the recurrence; the skip terms D * x-branch stay in the lane's
+// registers, because in this kernel the lane that forms them is the one that uses them after the recurrence, and
+// for the same reason the gates are not formed here at all (gates_all, after the recurrence).
+// coef: [group][row] composed triple + one more float (D next to the x-branch triple); tay: [step size | gate][row][4].
+// angle[h]: bit 0 / 1 = every rotation angle of columns 8 h .. 8 h + 7 at this timestep is small / tiny.
+template <class G, bool HAS_S, bool TAYLOR, bool DSTORE>
+__device__ __forceinline__ void project_all(float g, float s, int tu, const float* s_coef, const float* s_tay, const float* s_fmax, float* s_dt,
+                                            float* s_ux, float* s_B, float* s_C, float (&dxv)[G::DI], int (&angle)[2]) {
+    constexpr int DI = G::DI, DS = G::DS;
+    auto delta = [&](const f32x4 t) { return HAS_S ? sg_fma(t[0], g, t[1] * s) : t[0] * g; };
+    auto poly = [&](const f32x4 t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); };
+    auto eval = [&](const f32x4 t) { return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]); };
+    auto coef = [&](int group, int row) { return *reinterpret_cast<const f32x4*>(s_coef + (group * DI + row) * 4); };
+    static_assert(DI == 16 && DS == 16, "two halves of eight columns");
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        bool small = true, tiny = true;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int jj = 8 * h + q;
+            const f32x4 cd = coef(SG2_COMP_DT, jj);
+            float dtv, dt0 = 0.0f;
+            if (TAYLOR) {
+                const f32x4 tp = *reinterpret_cast<const f32x4*>(s_tay + jj * 4);
+                dtv = poly(tp, delta(cd));
+                dt0 = tp[0];
+            } else {
+                dtv = sg_softplus(eval(cd));
+            }
+            if (!DSTORE) {
+                const float amax = dtv * s_fmax[jj];
+                small = small && (amax < SG_SINCOS_SMALL_LIMIT);
+                tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
+            }
+            const f32x4 cx = coef(SG2_COMP_XB, jj);       // x-branch coefficients; [3] = D of this column
+            const float xbv = eval(cx);
+            s_dt[jj * LDS_STRIDE + tu] = DSTORE ? dtv - dt0 : dtv;
+            s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
+            dxv[jj] = cx[3] * xbv;
+        }
+        angle[h] = (small ? 1 : 0) | (tiny ? 2 : 0);
+    }
+#pragma unroll
+    for (int ss = 0; ss < DS; ss++) {
+        s_B[ss * LDS_STRIDE + tu] = eval(coef(SG2_COMP_B, ss));
+        s_C[ss * LDS_STRIDE + tu] = eval(coef(SG2_COMP_C, ss));
+    }
+}
+// The 16 gates silu(z) of one timestep: Taylor polynomials for a tile that qualifies, else eight at a time on one shared
+// reciprocal (columns 0-7, 8-15: the groups the two-wave kernel and the checker form).
+template <class G, bool HAS_S, bool TAYLOR>
+__device__ __forceinline__ void gates_all(float g, float s, const float* s_coef, const float* s_tay, float (&gv)[G::DI]) {
+    constexpr int DI = G::DI;
+    auto delta = [&](const f32x4 t) { return HAS_S ? sg_fma(t[0], g, t[1] * s) : t[0] * g; };
+    auto poly = [&](const f32x4 t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); };
+    auto eval = [&](const f32x4 t) { return sg_fma(t[0], g, HAS_S ? sg_fma(t[1], s, t[2]) : t[2]); };
+    auto coef = [&](int row) { return *reinterpret_cast<const f32x4*>(s_coef + (SG2_COMP_Z * DI + row) * 4); };
+    if (TAYLOR) {
+#pragma unroll
+        for (int jj = 0; jj < DI; jj++) gv[jj] = poly(*reinterpret_cast<const f32x4*>(s_tay + (DI + jj) * 4), delta(coef(jj)));
+    } else {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float zv[8], out[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) zv[q] = eval(coef(8 * h + q));
+            sg_silu_block(8, zv, out);
+#pragma unroll
+            for (int q = 0; q < 8; q++) gv[8 * h + q] = out[q];
+        }
+    }
+}
+
+// UB steps of both columns of a lane on the lane polynomials, dt - dt0 given (what block_steps<HP, true, 3, false, true,
+// LINEAR> does for one column), written as one straight-line block so that the two independent recurrences interleave.
+template <int HP, bool LINEAR>
+__device__ __forceinline__ void block_steps_pair(LaneState (&S)[2], const float (&dt)[2][UB], const float (&ux)[2][UB], const float (&Be)[UB],
+                                                 const float (&Bo)[UB], const float (&Ce)[UB], const float (&Co)[UB], const LanePoly<true> (&LP)[2],
+                                                 float (&y)[2][UB]) {
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const float d = dt[h][u];
+            const float p1 = LINEAR ? sg2_poly1(LP[h].k, d) : sg2_poly2(LP[h].k, d);
+            const float n2 = LINEAR ? sg2_poly1(LP[h].k + 3, d) : sg2_poly2(LP[h].k + 3, d);
+            const float p3 = LINEAR ? sg2_poly1(LP[h].k + 6, d) : sg2_poly2(LP[h].k + 6, d);
+            const float p4 = LINEAR ? sg2_poly1(LP[h].k + 9, d) : sg2_poly2(LP[h].k + 9, d);
+            const float be = ux[h][u] * Be[u], bo = ux[h][u] * Bo[u];
+            const float he = sg_fma(p1, S[h].he, sg_fma(n2, S[h].ho, be));      // P1 he + N2 ho + b_e
+            S[h].ho = sg_fma(p3, S[h].ho, sg_fma(p4, S[h].he, bo));            // P3 ho + P4 he + b_o
+            S[h].he = he;
+            y[h][u] = sg_fma(S[h].ho, Co[u], S[h].he * Ce[u]);
+        }
+    }
+    block_pair_sums<HP>(y[0]);
+    block_pair_sums<HP>(y[1]);
+}
+
+// The replay of the default geometry (what k_scan<G, true> computes, value for value) as ONE wave per chunk: lane
+// (jl, p) owns RoPE pair p of the two columns jl and jl + 8.  The 16 lanes that need the same B / C entries of a
+// timestep are then 8, and each entry a lane fetches from LDS feeds two recurrences: a third less LDS traffic per
+// step -- the pass was bound by the LDS queue and the vector ALU together, and the B / C fetches alone were a fifth of
+// its time.  A single wave also needs no workgroup barrier between the phases of a tile (its LDS accesses execute in
+// program order), forms the 16 gated outputs of a timestep once instead of once per wave, and holds all eight context
+// entries of its timestep: the two 16-byte stores of an element are adjacent in one lane and leave as one 32-byte
+// write.  Column jl + 8 h plays the part of wave h of the two-wave kernel throughout (its half of the projections, its
+// angle masks, its ballots over the same 64 (column, pair) lanes), so every decision and every value is the one the
+// checker makes for the two-wave form.
+template <class G>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_replay(Plan pl) {
+    constexpr int DM = G::DM, DS = G::DS, DI = G::DI, HP = G::HP, LANES = G::THREADS;
+    static_assert(G::PARTS == 2 && LANES == 128 && HP == 8, "two columns per lane of one wave");
+    constexpr bool OUT = true;
+    __shared__ __attribute__((aligned(16))) float s_dt[DI * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_ux[DI * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_B[DS * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float s_C[DS * LDS_STRIDE];
+    float* const s_y = s_dt;      // y of column j goes where dt of column j was: both are touched by the same lanes, in program order
+    __shared__ float s_fmax[DI];
+    __shared__ __attribute__((aligned(16))) float s_coef[SG2_COMP_GROUPS * DI * 4];   // [group][row]: composed triple, D beside the x-branch's
+    __shared__ __attribute__((aligned(16))) float s_tay[2 * DI * 4];                  // [step size | gate][row]: cubic Taylor polynomials
+    __shared__ __attribute__((aligned(16))) float s_wout[DM * DI];
+    // four arrays of 16 x 68 floats and 2.4 KB of tables: 19.8 KB, eight workgroups (two waves per SIMD) share a compute unit
+
+    const int per_dir = pl.chunks;
+    const int dir = (int)blockIdx.x >= per_dir ? 1 : 0;
+    const int cidx = (int)blockIdx.x - dir * per_dir;
+    const sg::cint_p prefix = sg::as_const(pl.chunk_prefix);
+    const int ti = sg::upper_seg(prefix, pl.P, cidx);
+    const int c = cidx - prefix[ti];
+    const TensorDev& T = pl.tensors[ti];
+    const int N = T.numel, off = T.off;
+    const int u0 = c * pl.chunk_len;
+    const int u1 = min(u0 + pl.chunk_len, N);
+    const uint32_t* __restrict__ skey = pl.keys[0] + off;
+    const int32_t* __restrict__ sval = pl.vals[0] + off;
+    const float* __restrict__ ssrt = pl.ssorted + off;
+    const bool has_s = __builtin_amdgcn_readfirstlane(pl.sharp_nonzero[ti]) != 0;
+
+    const int tid = threadIdx.x;
+    const int tu = tid;                      // projection role: timestep of the tile
+    const int jl = tid >> 3, p = tid & 7;    // scan role: pair p of columns jl and jl + 8
+    const float* alog = pl.W.w[dir ? W_B_ALOG : W_F_ALOG];
+    const float* rope = pl.W.w[dir ? W_B_ROPE : W_F_ROPE];
+    auto pole_e = [&](int h) { return -0.5f * -sg_exp(alog[(jl + 8 * h) * DS + 2 * p]); };
+    auto pole_o = [&](int h) { return -0.5f * -sg_exp(alog[(jl + 8 * h) * DS + 2 * p + 1]); };
+    auto rope_f = [&](int h) { return rope[(jl + 8 * h) * HP + p]; };
+    LanePoly<true> LP[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        LP[h].dt0 = pl.comp[2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4 + (jl + 8 * h) * 4];
+        sg2_pair_products(LP[h].dt0, pole_e(h), pole_o(h), rope_f(h), LP[h].k);
+    }
+    {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const float f = pair_tree_max<HP>(sg_abs(rope_f(h)));
+            if (p == 0) s_fmax[jl + 8 * h] = f;
+        }
+        const float* comp = pl.comp + dir * (SG2_COMP_GROUPS * G::ROWS * 3);
+        const float* tay = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + dir * 2 * G::ROWS * 4;
+        const float* Dw = pl.W.w[dir ? W_B_D : W_F_D];
+        for (int i = tid; i < SG2_COMP_GROUPS * DI; i += 64) {
+            const float* t = comp + i * 3;
+            *reinterpret_cast<f32x4*>(s_coef + i * 4) = f32x4{t[0], t[1], t[2], i / DI == SG2_COMP_XB ? Dw[i % DI] : 0.0f};
+        }
+        for (int i = tid; i < 2 * DI * 4; i += 64) s_tay[i] = tay[i];
+        s_wout[tid] = pl.W.w[dir ? W_B_OUT : W_F_OUT][tid];
+        s_wout[tid + 64] = pl.W.w[dir ? W_B_OUT : W_F_OUT][tid + 64];
+        __syncthreads();
+    }
+    const sg::cfloat_p lim = sg::as_const(pl.comp) + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4;
+    const float cmax_g = lim[2 * dir], cmax_s = lim[2 * dir + 1];
+    const float kpoly_g = lim[8 + 2 * dir], kpoly_s = lim[8 + 2 * dir + 1];
+
+    LaneState S[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        S[h] = {0.0f, 0.0f, 1.0f, 0.0f, 0.0f, 1.0f};
+        const int lane = tid + 64 * h;       // (column jl + 8 h, pair p) in the order of the summaries and start states
+        if (c > 0 && __builtin_amdgcn_readfirstlane(*pl.contracted) != 0) {
+            const float* sm = pl.summaries + (size_t)(dir * pl.wchunks + pl.wchunk_prefix[ti] + c - 1) * 6 * LANES;
+            S[h].he = sm[4 * LANES + lane];
+            S[h].ho = sm[5 * LANES + lane];
+        } else {
+            const float* hs = pl.hstart + ((size_t)(dir * pl.chunks + cidx) * 2) * LANES;
+            S[h].he = hs[lane];
+            S[h].ho = hs[LANES + lane];
+        }
+    }
+
+    uint32_t nx_key = 0;
+    int32_t nx_val = 0;
+    float nx_sh = 0.0f;
+    auto load_inputs = [&](int tile0) {
+        const int u = tile0 + tu;
+        if (u < u1) {
+            const int t = dir ? (N - 1 - u) : u;
+            nx_key = skey[t];
+            nx_val = sval[t];
+            nx_sh = has_s ? ssrt[t] : 0.0f;
+        }
+    };
+    load_inputs(u0);
+    for (int tile0 = u0; tile0 < u1; tile0 += SCAN_TT) {
+        const int cnt = min(SCAN_TT, u1 - tile0);
+        // ---------------- phase A: projections of SCAN_TT timesteps -> LDS (both halves of every output group)
+        const uint32_t kbits = nx_key;
+        const int32_t v = nx_val;
+        const float shv = nx_sh;
+        const bool valid = tile0 + tu < u1;
+        if (tile0 + SCAN_TT < u1) load_inputs(tile0 + SCAN_TT);
+        int orig = v & 0x7fffffff;
+        orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
+        const float g = valid ? sg_i2f((int32_t)kbits | (v & (int32_t)0x80000000)) : 0.0f;
+        const float sh = valid ? shv : 0.0f;
+        const unsigned long long notpoly = __builtin_amdgcn_ballot_w64(!sg2_poly_ok(kpoly_g, kpoly_s, g, sh));
+        const unsigned long long notlin =
+            __builtin_amdgcn_ballot_w64(!sg2_poly_ok(SG2_PROD_LINEAR_FACTOR * kpoly_g, SG2_PROD_LINEAR_FACTOR * kpoly_s, g, sh));
+        const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
+        const bool dgiven = tay && notpoly == 0 && cnt == SCAN_TT;
+        unsigned long long large[2], nottiny[2];
+        float dxv[DI];           // D * x-branch of this lane's timestep, kept for phase C
+        {
+            int angle[2];
+            auto run = [&](auto has_s_c, auto tay_c) {
+                constexpr bool HS = decltype(has_s_c)::value, TY = decltype(tay_c)::value;
+                if (TY && dgiven) project_all<G, HS, true, true>(g, sh, tu, s_coef, s_tay, s_fmax, s_dt, s_ux, s_B, s_C, dxv, angle);
+                else project_all<G, HS, TY, false>(g, sh, tu, s_coef, s_tay, s_fmax, s_dt, s_ux, s_B, s_C, dxv, angle);
+            };
+            if (tay) { if (has_s) run(std::true_type{}, std::true_type{}); else run(std::false_type{}, std::true_type{}); }
+            else { if (has_s) run(std::true_type{}, std::false_type{}); else run(std::false_type{}, std::false_type{}); }
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                large[h] = __builtin_amdgcn_ballot_w64(!(angle[h] & 1));
+                nottiny[h] = __builtin_amdgcn_ballot_w64(!(angle[h] & 2));
+            }
+        }
+        __syncthreads();      // one wave: no s_barrier is issued, the LDS writes above are ordered before the reads below
+
+        // ---------------- phase B: the recurrences of this lane's two columns over the tile
+        const float* __restrict__ r_Be = s_B + (2 * p) * LDS_STRIDE;
+        const float* __restrict__ r_Bo = s_B + (2 * p + 1) * LDS_STRIDE;
+        const float* __restrict__ r_Ce = s_C + (2 * p) * LDS_STRIDE;
+        const float* __restrict__ r_Co = s_C + (2 * p + 1) * LDS_STRIDE;
+        int k0 = 0;
+        if (dgiven) {
+            // a whole tile on the lane polynomials (the usual case): both columns in one instruction stream, the
+            // operands of block b + 1 requested before block b is computed
+            float Be[UB], Bo[UB], Ce[UB], Co[UB], dt[2][UB], xv[2][UB];
+            auto fetch = [&](int kb, float (&tBe)[UB], float (&tBo)[UB], float (&tCe)[UB], float (&tCo)[UB], float (&tdt)[2][UB], float (&tux)[2][UB]) {
+#pragma unroll
+                for (int q = 0; q < UB; q += 4) {
+                    const f32x4 c4 = *reinterpret_cast<const f32x4*>(r_Be + kb + q), d4 = *reinterpret_cast<const f32x4*>(r_Bo + kb + q);
+                    const f32x4 f4 = *reinterpret_cast<const f32x4*>(r_Ce + kb + q), g4 = *reinterpret_cast<const f32x4*>(r_Co + kb + q);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { tBe[q + e] = c4[e]; tBo[q + e] = d4[e]; tCe[q + e] = f4[e]; tCo[q + e] = g4[e]; }
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const f32x4 a4 = *reinterpret_cast<const f32x4*>(s_dt + (jl + 8 * h) * LDS_STRIDE + kb + q);
+                        const f32x4 b4 = *reinterpret_cast<const f32x4*>(s_ux + (jl + 8 * h) * LDS_STRIDE + kb + q);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) { tdt[h][q + e] = a4[e]; tux[h][q + e] = b4[e]; }
+                    }
+                }
+            };
+#ifdef SG2_REPLAY_PREFETCH
+            float nBe[UB], nBo[UB], nCe[UB], nCo[UB], ndt[2][UB], nxv[2][UB];      // the other operand set: the two alternate
+#endif
+            auto compute = [&](int kb, const float (&tBe)[UB], const float (&tBo)[UB], const float (&tCe)[UB], const float (&tCo)[UB],
+                               const float (&tdt)[2][UB], const float (&tux)[2][UB]) {
+                float y[2][UB];
+                const unsigned long long blk = ((1ull << UB) - 1) << kb;
+                if ((notlin & blk) == 0) block_steps_pair<HP, true>(S, tdt, tux, tBe, tBo, tCe, tCo, LP, y);
+                else block_steps_pair<HP, false>(S, tdt, tux, tBe, tBo, tCe, tCo, LP, y);
+                if ((p & 3) == 0) {      // the first lane of every bank holds the totals of its bank's steps (block_pair_sums)
+                    *reinterpret_cast<f32x4*>(&s_y[jl * LDS_STRIDE + kb + 4 * (p >> 2)]) = f32x4{y[0][0], y[0][1], y[0][2], y[0][3]};
+                    *reinterpret_cast<f32x4*>(&s_y[(jl + 8) * LDS_STRIDE + kb + 4 * (p >> 2)]) = f32x4{y[1][0], y[1][1], y[1][2], y[1][3]};
+                }
+            };
+#ifdef SG2_REPLAY_PREFETCH
+            fetch(0, Be, Bo, Ce, Co, dt, xv);
+#pragma unroll 1
+            for (; k0 < SCAN_TT; k0 += 2 * UB) {
+                fetch(k0 + UB, nBe, nBo, nCe, nCo, ndt, nxv);
+                compute(k0, Be, Bo, Ce, Co, dt, xv);
+                if (k0 + 2 * UB < SCAN_TT) fetch(k0 + 2 * UB, Be, Bo, Ce, Co, dt, xv);
+                compute(k0 + UB, nBe, nBo, nCe, nCo, ndt, nxv);
+            }
+#else
+#pragma unroll 1
+            for (; k0 < SCAN_TT; k0 += UB) {
+                fetch(k0, Be, Bo, Ce, Co, dt, xv);
+                compute(k0, Be, Bo, Ce, Co, dt, xv);
+            }
+#endif
+        }
+        for (; k0 + UB <= cnt; k0 += UB) {
+            float Be[UB], Bo[UB], Ce[UB], Co[UB];
+#pragma unroll
+            for (int q = 0; q < UB; q += 4) {
+                const f32x4 c4 = *reinterpret_cast<const f32x4*>(r_Be + k0 + q), d4 = *reinterpret_cast<const f32x4*>(r_Bo + k0 + q);
+                const f32x4 f4 = *reinterpret_cast<const f32x4*>(r_Ce + k0 + q), g4 = *reinterpret_cast<const f32x4*>(r_Co + k0 + q);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { Be[q + e] = c4[e]; Bo[q + e] = d4[e]; Ce[q + e] = f4[e]; Co[q + e] = g4[e]; }
+            }
+            const unsigned long long blk = ((1ull << UB) - 1) << k0;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int j = jl + 8 * h;
+                float dt[UB], xv[UB], y[UB];
+#pragma unroll
+                for (int q = 0; q < UB; q += 4) {
+                    const f32x4 a4 = *reinterpret_cast<const f32x4*>(s_dt + j * LDS_STRIDE + k0 + q), b4 = *reinterpret_cast<const f32x4*>(s_ux + j * LDS_STRIDE + k0 + q);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { dt[q + e] = a4[e]; xv[q + e] = b4[e]; }
+                }
+                if (dgiven && (notlin & blk) == 0)
+                    block_steps<HP, OUT, 3, false, true, true>(S[h], dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP[h], y);
+                else if (dgiven)
+                    block_steps<HP, OUT, 3, false, true>(S[h], dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP[h], y);
+                else if ((notpoly & blk) == 0)
+                    block_steps<HP, OUT, 3, false>(S[h], dt, xv, Be, Bo, Ce, Co, 0.0f, 0.0f, 0.0f, LP[h], y);
+                else if ((nottiny[h] & blk) == 0)
+                    block_steps<HP, OUT, 2, false>(S[h], dt, xv, Be, Bo, Ce, Co, pole_e(h), pole_o(h), rope_f(h), LP[h], y);
+                else if ((large[h] & blk) == 0)
+                    block_steps<HP, OUT, 1, false>(S[h], dt, xv, Be, Bo, Ce, Co, pole_e(h), pole_o(h), rope_f(h), LP[h], y);
+                else
+                    block_steps<HP, OUT, 0, false>(S[h], dt, xv, Be, Bo, Ce, Co, pole_e(h), pole_o(h), rope_f(h), LP[h], y);
+                if ((p & 3) == 0)        // the first lane of every bank holds the totals of its bank's steps (block_pair_sums)
+                    *reinterpret_cast<f32x4*>(&s_y[j * LDS_STRIDE + k0 + 4 * (p >> 2)]) = f32x4{y[0], y[1], y[2], y[3]};
+            }
+        }
+        for (; k0 < cnt; k0++) {       // ragged end of the last tile of a tensor
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int j = jl + 8 * h;
+                const float dt = s_dt[j * LDS_STRIDE + k0], ux = s_ux[j * LDS_STRIDE + k0];
+                float ae, ao, sn, cs;
+                sg_abar_pair(dt, pole_e(h), pole_o(h), &ae, &ao);
+                sg_sincos(dt * rope_f(h), &sn, &cs);
+                step_update<OUT>(S[h], ae, ao, sn, cs, ux * r_Be[k0], ux * r_Bo[k0]);
+                const float y = pair_tree_sum<HP>(sg_fma(S[h].ho, r_Co[k0], S[h].he * r_Ce[k0]));
+                if (p == 0) s_y[j * LDS_STRIDE + k0] = y;
+            }
+        }
+        __syncthreads();
+
+        // ---------------- phase C: gate, D skip, out_proj, scatter to element order (one 32-byte row per lane)
+        {
+            float o[DI];
+            if (tay) { if (has_s) gates_all<G, true, true>(g, sh, s_coef, s_tay, o); else gates_all<G, false, true>(g, sh, s_coef, s_tay, o); }
+            else { if (has_s) gates_all<G, true, false>(g, sh, s_coef, s_tay, o); else gates_all<G, false, false>(g, sh, s_coef, s_tay, o); }
+#pragma unroll
+            for (int jj = 0; jj < DI; jj++) o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], o[jj], dxv[jj]);
+            float cx[DM];
+#pragma unroll
+            for (int q = 0; q < DM; q++) {
+                const float* wr = s_wout + q * DI;       // the same address for every lane (broadcast reads)
+                float a = 0.0f;
+#pragma unroll
+                for (int m = 0; m < DI; m += 4) {
+                    const f32x4 w4 = *reinterpret_cast<const f32x4*>(wr + m);
+                    a = sg_fma(w4[0], o[m], a);
+                    a = sg_fma(w4[1], o[m + 1], a);
+                    a = sg_fma(w4[2], o[m + 2], a);
+                    a = sg_fma(w4[3], o[m + 3], a);
+                }
+                cx[q] = a;
+            }
+            if (valid) {
+                static_assert(DM == 8, "two 16-byte stores per lane");
+                float4* dst = reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM);
+                dst[0] = make_float4(cx[0], cx[1], cx[2], cx[3]);
+                dst[1] = make_float4(cx[4], cx[5], cx[6], cx[7]);
+            }
+        }
+        __syncthreads();
+    }
+    if (u1 == N) {   // last chunk in scan order: new carried state of the tensor
+        float* st = dir ? T.mbwd : T.mfwd;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int j = jl + 8 * h;
+            if (j < pl.st_di && 2 * p < pl.st_ds) {
+                st[j * pl.st_ds + 2 * p] = S[h].he;
+                st[j * pl.st_ds + 2 * p + 1] = S[h].ho;
+            }
+        }
+    }
+}
+
 // Start state of every chunk: h_{c+1} = M_c h_c + b_c, applied in order from
 // the carried state of the tensor.  One workgroup per (tensor, direction).
 // The recurrence itself is a handful of fmas per chunk; what matters is the
@@ -900,6 +1295,14 @@ int launch_scan_geo(const Plan& pl, hipStream_t st) {
         }
     }
     if (pl.htile != nullptr) return sg::fail("the bilevel pass is built for the default meta-net dimensions only");
+#ifndef SG2_TWO_WAVE_REPLAY
+    if constexpr (G::PARTS == 2) {
+        hipLaunchKernelGGL(k_replay<G>, dim3(2 * pl.chunks), dim3(64), 0, st, pl);
+        SG_LAUNCH_CHECK("k_replay");
+        prof_mark(4, st);
+        return 0;
+    }
+#endif
     hipLaunchKernelGGL((k_scan<G, true, false>), dim3(2 * pl.chunks), dim3(G::THREADS), 0, st, pl);
     SG_LAUNCH_CHECK("k_scan<out>");
     prof_mark(4, st);
