@@ -75,8 +75,10 @@
  * and shared-reciprocal forms are considered (fp32 policy only).  The replay uses, with a tighter limit, quadratics
  * for the four products of its update instead (sg2_pair_products): he' = P1 he + N2 ho + b_e, ho' = P3 ho + P4 he + b_o.
  * A (j,p) whose M is exactly zero hands on b itself as the next start state
- * (not 0 * h + b, which differs for a non-finite h): the kernels read no
- * earlier state at all when every summary of a call is of that kind.
+ * when the state before it is finite (0 * h + b is then b): the kernels read no
+ * earlier state at all when every summary of a call is of that kind and every
+ * carried state is finite.  A non-finite state is multiplied through and keeps
+ * the rest of the tensor non-finite, as in the reference.
  *
  * Parity status: the reference's tests hold no golden vectors for this path
  * (tests/test_supergrok2.py checks finiteness and run-to-run determinism
@@ -596,8 +598,11 @@ void scan_dir(const Dims& d, const DirW<O>& w, const typename O::R* x, const flo
             for (int p = 0; p < hp; p++) {
                 const R* m = &sm[(j * hp + p) * 6];
                 const R he = h0[j * ds + 2 * p], ho = h0[j * ds + 2 * p + 1];
-                /* an exactly zero 2x2 part hands on the offset itself (the kernels then never read the earlier state) */
-                const bool zero = m[0] == 0 && m[1] == 0 && m[2] == 0 && m[3] == 0;
+                /* an exactly zero 2x2 part hands on the offset itself -- what 0 * h + b is for a finite h; the kernels then
+                 * never read the earlier state.  A state that is not finite goes through the product (0 * inf = NaN) and
+                 * stays non-finite to the end of the tensor, as in the reference (csrc/supergrok2_mamba_peer_kernels.cu:
+                 * 444-551 applies every chunk's summary to the state before it). */
+                const bool zero = m[0] == 0 && m[1] == 0 && m[2] == 0 && m[3] == 0 && std::isfinite((double)he) && std::isfinite((double)ho);
                 h1[j * ds + 2 * p] = zero ? m[4] : O::fma(m[0], he, O::fma(m[2], ho, m[4]));
                 h1[j * ds + 2 * p + 1] = zero ? m[5] : O::fma(m[1], he, O::fma(m[3], ho, m[5]));
             }

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        pl.contracted[0] = 1;      // until a summary kernel finds a chunk that has not contracted
+        pl.contracted[0] = pl.contracted[2] == 0 ? 1 : 0;      // until a summary kernel finds a chunk that has not contracted; never while a carried state is not finite
         pl.contracted[1] = sg2_first_block_steps(s_largest, s_zero);
         float* cmax = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4;
         cmax[0] = sg_i2f(s_cmax[0][0]); cmax[1] = sg_i2f(s_cmax[0][1]);
@@ -1259,8 +1259,10 @@ __global__ __launch_bounds__(1024) void k_chunk_prefix(Plan pl) {
             const int lim = min(PREFIX_BATCH, ns - b * PREFIX_BATCH);
             for (int cc = 0; cc < lim; cc++) {
                 const float* m = lds + cc * 6 * SCAN_THREADS + lane;
-                // a lane whose 2x2 part is exactly zero takes the offset itself (not 0 * h + b: the state may not be finite)
-                const bool zero = m[0] == 0.0f && m[SCAN_THREADS] == 0.0f && m[2 * SCAN_THREADS] == 0.0f && m[3 * SCAN_THREADS] == 0.0f;
+                // a lane whose 2x2 part is exactly zero takes the offset itself, which is what 0 * h + b is for every finite h;
+                // a state that is not finite goes through the product and stays non-finite to the end of the tensor
+                const bool zero = m[0] == 0.0f && m[SCAN_THREADS] == 0.0f && m[2 * SCAN_THREADS] == 0.0f && m[3 * SCAN_THREADS] == 0.0f &&
+                                  sg_isfinite(he) && sg_isfinite(ho);
                 const float ne = sg_fma(m[0], he, sg_fma(m[2 * SCAN_THREADS], ho, m[4 * SCAN_THREADS]));
                 const float no = sg_fma(m[SCAN_THREADS], he, sg_fma(m[3 * SCAN_THREADS], ho, m[5 * SCAN_THREADS]));
                 he = zero ? m[4 * SCAN_THREADS] : ne;

@@ -110,36 +110,55 @@ def test_adaptive_window_needs_several_blocks():
     print("several blocks", _run_steps(case, 2, chunk_len=512, sharp=True, lamb_eff=2.0))
 
 
-def test_contracted_summaries_forget_the_carried_state():
+def test_contracted_summaries_forget_a_finite_carried_state_only():
     """With every chunk summary contracted to (0, b) the replay takes the start state of chunk c from summary c - 1 and
     never reads what came before: the contexts of all later chunks and the new carried state are the same, bit for
-    bit, whether the tensor carried in a small state or an infinite one.  (The first chunk does see it.)"""
+    bit, whether the tensor carried in a small state or a huge finite one.  A carried state that is NOT finite switches
+    that shortcut off for the call and is multiplied through: every context of that tensor and direction comes out
+    non-finite, as in the reference, while the other tensors of the call keep their values bit for bit."""
     from grokking_optimizers import _cabi
     shapes, cl = [(3000,), (700,), (256,)], 256
     assert _cabi.lib().sg2_set_chunk_len(cl) == 0
     ctx, fwd, perm = [], [], None
-    for poison in (False, True):
+    for poison in ("none", "huge", "inf"):
         case = Sg2Case(shapes, seed=5, random_state=True)
-        if poison:
-            case.gpu[0]["mamba_fwd"].fill_(float("inf"))
+        if poison == "huge":
+            case.gpu[0]["mamba_fwd"].fill_(3.0e30)
             case.gpu[1]["mamba_bwd"].fill_(-3.0e30)
+        if poison == "inf":
+            case.gpu[0]["mamba_fwd"].fill_(float("inf"))
         grads = wl.make_grads(shapes, seed=77)
         sharps = [torch.zeros_like(g) for g in grads]
-        print("carried state", "infinite" if poison else "small", flush=True)
+        print("carried state:", poison, flush=True)
         case.gpu_step(grads, sharps, per_tensor_scalars(case.P, 1, 2.0), shared_scalars(4.5))
         ctx.append(case.step_fn.ctx.cpu().numpy().copy())
         fwd.append([case.gpu[i][k].cpu().numpy().copy() for i in range(case.P) for k in ("mamba_fwd", "mamba_bwd")])
         perm = case.step_fn.perm.cpu().numpy()
+        if poison == "inf":          # the checker makes the same statement, value for value where values are finite
+            for st in case.np[:1]:
+                st["mamba_fwd"][:] = np.inf
+            dbg = case.oracle_step(grads, sharps, per_tensor_scalars(case.P, 1, 2.0), shared_scalars(4.5), cl)
+            for i in range(case.P):
+                a, b = int(case.offsets[i]), int(case.offsets[i + 1])
+                for d in range(2):
+                    assert np.array_equal(np.isfinite(ctx[-1][d, a:b]), np.isfinite(dbg[i]["ctx"][d]))
+                    ok = np.isfinite(dbg[i]["ctx"][d])
+                    assert np.array_equal(ctx[-1][d, a:b][ok], dbg[i]["ctx"][d][ok])
     n0, o1, n1 = 3000, 3000, 700
     later0 = perm[:n0][cl:]                       # tensor 0, forward direction: scan steps >= one chunk
     assert np.isfinite(ctx[1][0, later0]).all() and np.array_equal(ctx[0][0, later0], ctx[1][0, later0])
-    assert not np.isfinite(ctx[1][0, perm[:n0][:cl]]).all()
+    assert not np.array_equal(ctx[0][0, perm[:n0][:cl]], ctx[1][0, perm[:n0][:cl]])
     later1 = o1 + perm[o1:o1 + n1][:n1 - cl]      # tensor 1, backward direction
     assert np.array_equal(ctx[0][1, later1], ctx[1][1, later1])
     first1 = o1 + perm[o1:o1 + n1][n1 - cl:]
     assert not np.array_equal(ctx[0][1, first1], ctx[1][1, first1])
-    for a, b in zip(fwd[0], fwd[1]):              # every new carried state comes from a last chunk (tensor 2 has one chunk
-        assert np.isfinite(b).all() and np.array_equal(a, b)      # only, and was not poisoned)
+    for a, b in zip(fwd[0], fwd[1]):              # every new carried state comes from a last chunk
+        assert np.isfinite(b).all() and np.array_equal(a, b)
+    # the infinite state: tensor 0's forward contexts all non-finite, its new forward state too; everything else as without it
+    assert (~np.isfinite(ctx[2][0, :n0]).all(axis=-1)).all() and not np.isfinite(fwd[2][0]).all()
+    assert np.array_equal(ctx[0][1], ctx[2][1]) and np.array_equal(ctx[0][0, n0:], ctx[2][0, n0:])
+    for k in range(1, len(fwd[0])):
+        assert np.array_equal(fwd[0][k], fwd[2][k])
 
 
 def test_saturated_gates_take_the_plain_forms():

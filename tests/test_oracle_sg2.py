@@ -158,17 +158,18 @@ def test_windowed_summaries_match_full_chunks():
     assert np.array_equal(dplain["ctx"], dwin["ctx"]) and np.array_equal(plain["mamba_fwd"], win["mamba_fwd"])
 
 
-def test_contracted_summary_forgets_what_came_before():
+def test_contracted_summary_forgets_a_finite_state_and_keeps_a_non_finite_one():
     """A chunk summary whose 2x2 part has contracted to exactly zero hands on its offset b itself: every chunk after
-    the first is then independent of the state the tensor carried in -- bit for bit, and even for a carried state that
-    is not finite (0 * inf would poison the whole sequence; the kernels never read the earlier state in this case)."""
+    the first is then independent of the (finite, however large) state the tensor carried in, bit for bit.  A carried
+    state that is not finite is multiplied through instead (0 * inf = NaN) and keeps every later context of that
+    direction non-finite, as the reference's chunked scan does: a diverged run stays visible."""
     n, chunk = 1500, 256
     W = weights_np()
     g, s = _grad(n, 21), np.abs(_grad(n, 22))
     sc = default_scalars()
     st_a = random_state_np(n, 23)
     st_b = copy_state(st_a)
-    st_b["mamba_fwd"][:] = np.inf
+    st_b["mamba_fwd"][:] = 3.0e30
     st_b["mamba_bwd"][:] = -3.0e30
     a, da = _run_oracle(W, st_a, g, s, sc, 32, chunk, window=64)
     b, db = _run_oracle(W, st_b, g, s, sc, 32, chunk, window=64)
@@ -178,13 +179,22 @@ def test_contracted_summary_forgets_what_came_before():
     assert np.isfinite(db["ctx"][0][later_fwd]).all() and np.isfinite(db["ctx"][1][later_bwd]).all()
     assert np.array_equal(da["ctx"][0][later_fwd], db["ctx"][0][later_fwd])
     assert np.array_equal(da["ctx"][1][later_bwd], db["ctx"][1][later_bwd])
-    assert not np.isfinite(db["ctx"][0][perm[:chunk]]).all()       # the first chunk does see the carried state
+    assert not np.array_equal(da["ctx"][0][perm[:chunk]], db["ctx"][0][perm[:chunk]])       # the first chunk does see the carried state
     assert not np.array_equal(da["ctx"][1][perm[n - chunk:]], db["ctx"][1][perm[n - chunk:]])
     for k in ("mamba_fwd", "mamba_bwd"):                            # the new carried state comes from the last chunk
         assert np.array_equal(a[k], b[k]) and np.isfinite(b[k]).all()
-    # without the window the exact summaries are applied (their 2x2 part is small, not zero): the carried state counts
-    c, dc = _run_oracle(W, st_b, g, s, sc, 32, chunk, window=0)
-    assert not np.isfinite(dc["ctx"][0][later_fwd]).all()
+    # a carried state that is not finite: every context of that direction is non-finite, and so is the new state;
+    # the other direction is untouched
+    st_c = copy_state(st_a)
+    st_c["mamba_fwd"][:] = np.inf
+    c, dc = _run_oracle(W, st_c, g, s, sc, 32, chunk, window=64)
+    assert not np.isfinite(dc["ctx"][0]).any(axis=-1).all() or not np.isfinite(dc["ctx"][0]).all()
+    assert (~np.isfinite(dc["ctx"][0]).all(axis=-1)).all()          # every element's forward context holds a non-finite entry
+    assert not np.isfinite(c["mamba_fwd"]).all()
+    assert np.array_equal(dc["ctx"][1], da["ctx"][1]) and np.array_equal(c["mamba_bwd"], a["mamba_bwd"])
+    # float64 policy, sequential recurrence: the same statement from the plain formulas
+    d, dd = _run_oracle(W, st_c, g, s, sc, 64, 0)
+    assert (~np.isfinite(dd["ctx"][0]).all(axis=-1)).all()
 
 
 # ------------------------------------------------- structural identities of the scan
