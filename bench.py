@@ -312,13 +312,17 @@ def bench_other(args, dev):
 
 
 def bench_probe(dev):
-    """Issue rate of plain fp32 vector instructions (sg_probe_valu): wave64 instructions per nanosecond and SIMD for
+    """Issue rate of plain fp32 vector instructions (sg_probe_valu of tests/probe/libsg_probe.so, a measurement aid built beside the
+    tests, not part of the product library): wave64 instructions per nanosecond and SIMD for
     fma / mul / add / DPP-add streams with every SIMD of the chip busy, by resident waves per SIMD; and the shader
     clock the part holds meanwhile (ticks of the in-kernel clock per nanosecond of the launch)."""
     import ctypes as C
     import torch
-    from grokking_optimizers import _cabi
-    L = _cabi.lib()
+    path = os.path.join(ROOT, "tests", "probe", "libsg_probe.so")
+    if not os.path.exists(path):
+        raise SystemExit("the probe library is not built (%s): make -C tests/probe, or __graft_entry__.build()" % path)
+    L = C.CDLL(path)
+    L.sg_probe_last_error.restype = C.c_char_p
     L.sg_probe_workspace_bytes.restype = C.c_size_t
     L.sg_probe_valu.argtypes = [C.c_int] * 4 + [C.POINTER(C.c_float), C.POINTER(C.c_double), C.POINTER(C.c_double),
                                                 C.c_void_p, C.c_size_t, C.c_void_p]
@@ -332,7 +336,7 @@ def bench_probe(dev):
                 ms, ticks, instr = C.c_float(), C.c_double(), C.c_double()
                 if L.sg_probe_valu(op, ncu, w, 2000, C.byref(ms), C.byref(ticks), C.byref(instr), ws.data_ptr(), ws.numel(),
                                    torch.cuda.current_stream().cuda_stream) != 0:
-                    raise RuntimeError(_cabi.last_error())
+                    raise RuntimeError(L.sg_probe_last_error().decode())
                 rate = instr.value * w / (ms.value * 1e6)            # per SIMD: w waves share one
                 rows.append({"op": name, "cus": ncu, "waves_per_simd": w, "ms": round(ms.value, 4),
                              "instr_per_ns_per_simd": round(rate, 4),

@@ -119,6 +119,23 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
                      const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
                      void* workspace, size_t workspace_bytes, const Sg2Debug* debug, void* stream);
 
+/* The same step with the scan's decomposition chosen by the caller for this
+ * call instead of by the process-wide settings above (no counterpart in the
+ * reference).  chunk_len: 0 = the automatic choice, else a positive multiple
+ * of 64; scan_window: negative = SG2_DEFAULT_SCAN_WINDOW, 0 = off, else a
+ * multiple of 64.  options == NULL means the process-wide settings, i.e.
+ * exactly sg2_workspace_bytes / sg2_batched_step.  The workspace must be sized
+ * with the same options. */
+typedef struct Sg2Options {
+    int32_t chunk_len;
+    int32_t scan_window;
+} Sg2Options;
+size_t sg2_workspace_bytes_opt(const SgDims* dims, int num_tensors, const int64_t* numels, const Sg2Options* options);
+int sg2_batched_step_opt(const SgDims* dims, const Sg2Weights* weights, int num_tensors,
+                         const Sg2Tensor* tensors, const Sg2Scalars* scalars, int32_t* expert_counts,
+                         void* workspace, size_t workspace_bytes, const Sg2Debug* debug,
+                         const Sg2Options* options, void* stream);
+
 /* sg2_batched_step without a workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.
@@ -129,7 +146,13 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
  * elements in total; sg2_workspace_bytes tells) are rejected with an error.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one
  * GPU (different streams or threads) race; calls on one stream are ordered.
- * Same kernels and results as sg2_batched_step. */
+ * Same kernels and results as sg2_batched_step.
+ * The first call on a device looks the array's device address up
+ * (hipGetDevice + hipGetSymbolAddress, no stream work): make one plain call per
+ * device before a stream capture starts, so that the captured calls only
+ * launch kernels.  The array is part of the library's device image: every
+ * process that loads libsg_hip.so holds SG2_STATIC_SCRATCH_BYTES (64 MiB) on each
+ * GPU it initialises, whether or not this entry point is ever called. */
 #define SG2_STATIC_SCRATCH_BYTES (64u << 20)
 size_t sg2_static_scratch_bytes(void);
 int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int num_tensors,
@@ -149,24 +172,6 @@ int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int n
 #define SG2_PROF_MAX_CALLS 256
 int sg2_profile_enable(int on);
 int sg2_profile_read(float* ms, int* calls);
-
-/* Issue-rate probe of the fp32 vector ALU (measurement aid, no counterpart in
- * the reference): `iters` x 128 independent wave64 instructions of one kind
- * per wave (op 0 v_fma_f32, 1 v_mul_f32, 2 v_add_f32, 3 v_add_f32 with a DPP
- * operand; plain, not packed; 4 v_mfma_f32_32x32x16_bf16 on constant register
- * operands, 5 the same on pseudo-random operands: the matrix cores' own
- * ceiling and what real data makes of it through the power limit; 6
- * v_mfma_f32_32x32x1_2b_f32, 7 the same with 8 v_fma_f32 after each in the
- * same wave (the vector instructions are not counted), 8
- * v_mfma_f32_4x4x1_16b_f32: the fp32 matrix forms that are one fused
- * multiply-add per output) on num_cus x waves_per_simd workgroups of four
- * waves, i.e. waves_per_simd waves on every SIMD of num_cus compute units
- * when the dispatcher spreads them evenly.  Synchronises the stream.  Returns
- * the elapsed milliseconds of the launch, the shader-clock ticks a wave took
- * on average and the instructions each wave issued. */
-size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd);
-int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
-                  double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ======================= Grokfast / SuperGrok v1.5 ======================== */
 

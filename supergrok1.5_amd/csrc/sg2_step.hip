@@ -463,11 +463,28 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     return 0;
 }
 
+// per-call options -> the override arguments of build_plan (0 / -1: the process-wide settings)
+int resolve_options(const Sg2Options* o, int P, Numels numels, int* chunk_len, int* window) {
+    *chunk_len = 0;
+    *window = -1;
+    if (!o) return 0;
+    if (o->chunk_len < 0 || o->chunk_len % SCAN_TT) return sg::fail("options: chunk_len must be 0 (automatic) or a positive multiple of %d", SCAN_TT);
+    if (o->scan_window > 0 && o->scan_window % SCAN_TT) return sg::fail("options: scan_window must be a multiple of %d (0 disables it, negative = default)", SCAN_TT);
+    *chunk_len = o->chunk_len > 0 ? o->chunk_len : auto_chunk_len(P, numels);
+    *window = o->scan_window < 0 ? SG2_DEFAULT_SCAN_WINDOW : o->scan_window;
+    return 0;
+}
+
 int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, const Sg2Scalars* scalars,
-             int32_t* expert_counts, void* workspace, size_t workspace_bytes, const Sg2Debug* debug, hipStream_t st) {
+             int32_t* expert_counts, void* workspace, size_t workspace_bytes, const Sg2Debug* debug, hipStream_t st,
+             const Sg2Options* options = nullptr) {
     Plan pl;
     Layout L;
-    if (build_plan(dims, weights, num_tensors, tensors, scalars, workspace, workspace_bytes, true, false, false, st, &pl, &L)) return 1;
+    int chunk_override = 0, window_override = -1;
+    if (options && num_tensors > 0 && tensors && resolve_options(options, num_tensors, Numels{nullptr, tensors}, &chunk_override, &window_override)) return 1;
+    if (build_plan(dims, weights, num_tensors, tensors, scalars, workspace, workspace_bytes, true, false, false, st, &pl, &L, chunk_override,
+                   window_override))
+        return 1;
     if (pl.total == 0) return 0;
     prof_mark(0, st);
     if (launch_sort(pl, debug ? debug->perm : nullptr, st)) return 1;
@@ -512,6 +529,24 @@ int sg2_batched_step(const SgDims* dims, const Sg2Weights* weights, int num_tens
                      const Sg2Debug* debug, void* stream) {
     return sg2::run_step(dims, weights, num_tensors, tensors, scalars, expert_counts, workspace, workspace_bytes, debug,
                          (hipStream_t)stream);
+}
+
+size_t sg2_workspace_bytes_opt(const SgDims* dims, int num_tensors, const int64_t* numels, const Sg2Options* options) {
+    if (!options) return sg2_workspace_bytes(dims, num_tensors, numels);
+    const int geo = sg2::geo_of(dims);
+    if (geo < 0 || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
+    int chunk_len = 0, window = -1;
+    if (sg2::resolve_options(options, num_tensors, sg2::Numels{numels, nullptr}, &chunk_len, &window)) return 0;
+    sg2::Layout L;
+    if (sg2::make_layout(geo, num_tensors, sg2::Numels{numels, nullptr}, chunk_len, &L)) return 0;
+    return L.bytes;
+}
+
+int sg2_batched_step_opt(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                         const Sg2Scalars* scalars, int32_t* expert_counts, void* workspace, size_t workspace_bytes,
+                         const Sg2Debug* debug, const Sg2Options* options, void* stream) {
+    return sg2::run_step(dims, weights, num_tensors, tensors, scalars, expert_counts, workspace, workspace_bytes, debug,
+                         (hipStream_t)stream, options);
 }
 
 size_t sg2_static_scratch_bytes(void) { return SG2_STATIC_SCRATCH_BYTES; }

@@ -43,6 +43,10 @@ class Sg2Scalars(C.Structure):
                 ("eps", C.c_float)]
 
 
+class Sg2Options(C.Structure):
+    _fields_ = [("chunk_len", C.c_int32), ("scan_window", C.c_int32)]
+
+
 class Sg2Debug(C.Structure):
     _fields_ = [("perm", C.c_void_p), ("expert_idx", C.c_void_p), ("ctx", C.c_void_p)]
 
@@ -69,6 +73,12 @@ def lib():
         L.sg2_batched_step.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
                                        C.POINTER(Sg2Scalars), C.c_void_p, C.c_void_p, C.c_size_t,
                                        C.POINTER(Sg2Debug), C.c_void_p]
+        L.sg2_workspace_bytes_opt.restype = C.c_size_t
+        L.sg2_workspace_bytes_opt.argtypes = [C.POINTER(SgDims), C.c_int, C.POINTER(C.c_int64), C.POINTER(Sg2Options)]
+        L.sg2_batched_step_opt.restype = C.c_int
+        L.sg2_batched_step_opt.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
+                                           C.POINTER(Sg2Scalars), C.c_void_p, C.c_void_p, C.c_size_t,
+                                           C.POINTER(Sg2Debug), C.POINTER(Sg2Options), C.c_void_p]
         L.sg2_static_scratch_bytes.restype = C.c_size_t
         L.sg2_batched_step_static.restype = C.c_int
         L.sg2_batched_step_static.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor),
@@ -119,10 +129,10 @@ def chunk_len_for(numels):
     return lib().sg2_chunk_len_for(len(numels), arr)
 
 
-def workspace_bytes(numels, dims=None):
+def workspace_bytes(numels, dims=None, options=None):
     arr = (C.c_int64 * len(numels))(*numels)
     d = make_dims(dims)
-    n = lib().sg2_workspace_bytes(C.byref(d), len(numels), arr)
+    n = lib().sg2_workspace_bytes_opt(C.byref(d), len(numels), arr, C.byref(options) if options is not None else None)
     if n == 0 and sum(numels) > 0:
         raise RuntimeError(last_error())
     return n
@@ -132,8 +142,13 @@ class Sg2Step:
     """Reusable call plan for sg2_batched_step on a fixed list of tensors."""
 
     def __init__(self, weights, params, exp_avgs, exp_avg_sqs, mus, gru_states, mamba_fwd, mamba_bwd,
-                 expert_counts, dims=None, debug=False):
+                 expert_counts, dims=None, debug=False, chunk_len=None, scan_window=None):
+        """chunk_len / scan_window: this plan's own scan decomposition (sg2_batched_step_opt); both None = the
+        process-wide settings (sg2_set_chunk_len / sg2_set_scan_window)."""
         self.dims = make_dims(dims)
+        self.options = None
+        if chunk_len is not None or scan_window is not None:
+            self.options = Sg2Options(0 if chunk_len is None else chunk_len, -1 if scan_window is None else scan_window)
         self.weights = [w.contiguous() for w in weights]
         assert len(self.weights) == 33 and all(w.dtype == torch.float32 and w.is_cuda for w in self.weights)
         self.W = Sg2Weights()
@@ -144,7 +159,7 @@ class Sg2Step:
         self.numels = [p.numel() for p in params]
         self.total = sum(self.numels)
         self.expert_counts = expert_counts
-        self.ws_bytes = workspace_bytes(self.numels, dims)
+        self.ws_bytes = workspace_bytes(self.numels, dims, self.options)
         dev = params[0].device
         self.workspace = torch.empty(max(self.ws_bytes, 256), dtype=torch.uint8, device=dev)
         self.tensors = (Sg2Tensor * self.P)()
@@ -171,10 +186,11 @@ class Sg2Step:
             t.alpha_mu, t.lamb_eff, t.beta1, t.bc1, t.bc2 = sc["alpha"], sc["lamb_eff"], sc["beta1"], sc["bc1"], sc["bc2"]
         S = Sg2Scalars(shared["rescale"], shared["beta2"], shared["lr"], shared["wd_eff"], shared["eps"])
         stream = torch.cuda.current_stream().cuda_stream
-        rc = lib().sg2_batched_step(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, C.byref(S),
-                                    self.expert_counts.data_ptr() if self.expert_counts is not None else None,
-                                    self.workspace.data_ptr(), self.workspace.numel(),
-                                    C.byref(self.debug) if self.debug is not None else None, stream)
+        rc = lib().sg2_batched_step_opt(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, C.byref(S),
+                                        self.expert_counts.data_ptr() if self.expert_counts is not None else None,
+                                        self.workspace.data_ptr(), self.workspace.numel(),
+                                        C.byref(self.debug) if self.debug is not None else None,
+                                        C.byref(self.options) if self.options is not None else None, stream)
         if rc != 0:
             raise RuntimeError("sg2_batched_step: " + last_error())
 

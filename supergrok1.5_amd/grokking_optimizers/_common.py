@@ -13,6 +13,13 @@ def check_hyper(lr=None, eps=None, betas=None):
                 raise ValueError(f"Invalid beta parameter at index {k}: {betas[k]}")
 
 
+def check_ranges(checks):
+    """checks: (name, value, lowest, upper bound or None); lowest <= value (< upper) or ValueError("Invalid <name>: <value>")."""
+    for name, value, low, high in checks:
+        if value < low or (high is not None and not value < high):
+            raise ValueError(f"Invalid {name}: {value}")
+
+
 def run_closure(closure):
     if closure is None:
         return None

@@ -9,6 +9,7 @@ from torch.optim import Optimizer
 
 from grokking_optimizers import _ops
 from grokking_optimizers._adamw_helper import adamw_step
+from grokking_optimizers._common import check_ranges
 
 
 class Muon(Optimizer):
@@ -20,18 +21,9 @@ class Muon(Optimizer):
     def __init__(self, params_2d: Iterable, params_1d: Optional[Iterable] = None, lr: float = 0.02,
                  momentum: float = 0.95, weight_decay: float = 1.0, adamw_lr: float = 1e-3,
                  adamw_betas: Tuple[float, float] = (0.9, 0.98), adamw_eps: float = 1e-8, ns_steps: int = 5) -> None:
-        if lr < 0.0:
-            raise ValueError(f"Invalid learning rate: {lr}")
-        if adamw_lr < 0.0:
-            raise ValueError(f"Invalid AdamW learning rate: {adamw_lr}")
-        if not 0.0 <= momentum < 1.0:
-            raise ValueError(f"Invalid momentum: {momentum}")
-        if not 0.0 <= adamw_betas[0] < 1.0:
-            raise ValueError(f"Invalid AdamW beta at index 0: {adamw_betas[0]}")
-        if not 0.0 <= adamw_betas[1] < 1.0:
-            raise ValueError(f"Invalid AdamW beta at index 1: {adamw_betas[1]}")
-        if ns_steps < 1:
-            raise ValueError(f"Invalid ns_steps: {ns_steps}")
+        check_ranges((("learning rate", lr, 0.0, None), ("AdamW learning rate", adamw_lr, 0.0, None), ("momentum", momentum, 0.0, 1.0),
+                      ("AdamW beta at index 0", adamw_betas[0], 0.0, 1.0), ("AdamW beta at index 1", adamw_betas[1], 0.0, 1.0),
+                      ("ns_steps", ns_steps, 1, None)))
         groups = [dict(params=list(params_2d), lr=lr, momentum=momentum, weight_decay=weight_decay,
                        ns_steps=ns_steps, group_type="muon")]
         one_d = list(params_1d) if params_1d is not None else []

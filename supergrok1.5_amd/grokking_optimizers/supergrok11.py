@@ -30,6 +30,7 @@ class SuperGrok11(MetaTraining, Optimizer):
                  alpha_update_freq: int = 50, meta_update_freq: int = 5, zero_loss_threshold: float = 1e-4,
                  zero_acc_threshold: float = 0.995, sam_rho: float = 0.05, sam_enable_threshold: float = 0.0):
         super().__init__(params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        self.gelu_mode = None      # None: the process-wide form of `_ops.supergrok15_set_gelu_mode`; "erf" / "sigmoid": this instance's own
         for k, v in dict(alpha_init=alpha_init, lamb=lamb, gamma=gamma, gamma_alpha=gamma_alpha, kappa=kappa,
                          warmup_steps=warmup_steps, warmup_ramp=max(1, warmup_ramp), gradient_clipping=gradient_clipping,
                          meta_hidden_dim=meta_hidden_dim, gate_temperature=gate_temperature, alpha_update_freq=alpha_update_freq,
@@ -91,6 +92,8 @@ class SuperGrok11(MetaTraining, Optimizer):
             self._weights_dirty = False
         W1, b1, W2, b2, rescale = self._cached_weights
         sharp = [s if (g.numel() == 0 or s.dtype == g.dtype) else s.to(g.dtype) for s, g in zip(self._flat_sharpness, grads)]
+        if self.gelu_mode is not None:        # this optimizer's own choice of the meta-net's GELU form, set right before its call
+            _ops.supergrok15_set_gelu_mode(self.gelu_mode)
         _ops.supergrok11_fused_step(
             self._flat_param_data, grads, self._flat_exp_avgs, self._flat_exp_avg_sqs, self._flat_mus, sharp, self._flat_steps,
             layer_alphas, self._flat_layer_beta1s, W1, b1, W2, b2, rescale, self.meta_hidden_dim, group["betas"][1], group["lr"],

@@ -57,6 +57,9 @@ class SuperGrok15(GrokSchedule, MetaTraining, ScheduledTraining, Optimizer):
                  wd_ramp: float = 4.0, wd_scale: float = 20.0, wd_thresh: float = 0.9,
                  sam_enable_threshold: float = 0.0):
         Optimizer.__init__(self, params, dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay))
+        # None: whatever `_ops.supergrok15_set_gelu_mode` last selected for the process ("erf" unless changed); "erf" / "sigmoid":
+        # this instance's own form (the reference's CPU path / its GPU kernel), whatever other instances use
+        self.gelu_mode = None
         for k, v in dict(alpha_init=alpha_init, lamb=lamb, gamma=gamma, gamma_alpha=gamma_alpha, kappa=kappa,
                          warmup_steps=warmup_steps, warmup_ramp=max(1, warmup_ramp),
                          gradient_clipping=gradient_clipping, alpha_update_freq=alpha_update_freq,
@@ -118,6 +121,8 @@ class SuperGrok15(GrokSchedule, MetaTraining, ScheduledTraining, Optimizer):
         # sharpness is kept in fp32; hand the kernel the gradient's element type
         sharp = [s if (g.numel() == 0 or s.dtype == g.dtype) else s.to(g.dtype)
                  for s, g in zip(self._flat_sharpness, grads)]
+        if self.gelu_mode is not None:        # this optimizer's own choice of the meta-net's GELU form, set right before its call
+            _ops.supergrok15_set_gelu_mode(self.gelu_mode)
         _ops.supergrok15_fused_step(
             self._flat_param_data, grads, self._flat_exp_avgs, self._flat_exp_avg_sqs, self._flat_mus, sharp,
             self._flat_steps, layer_alphas, self._flat_layer_beta1s, W1, b1, W2, b2, rescale, self.meta_hidden_dim,

@@ -4,7 +4,7 @@
 // (the v2 scan and per-element kernels) are priced against; the reference has nothing comparable.
 // Op 4 is the same for the matrix cores: a stream of independent v_mfma_f32_32x32x16_bf16 on register operands
 // (no memory traffic at all), the ceiling the Muon GEMM's main loop is priced against.
-#include "sg_common.hpp"
+#include "../../supergrok1.5_amd/csrc/sg_common.hpp"
 
 namespace {
 
@@ -130,6 +130,8 @@ __global__ __launch_bounds__(256) void k_probe_mfma_f32(float* sink, long long* 
 }  // namespace
 
 extern "C" {
+
+const char* sg_probe_last_error(void) { return sg::last_error().c_str(); }
 
 size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd) {
     if (num_cus <= 0 || waves_per_simd <= 0) return 0;

@@ -99,7 +99,8 @@ class Sg2Case:
     """A list of parameter tensors with full optimizer state, mirrored on CPU
     (numpy, for the checker) and on the GPU (torch, for the C ABI)."""
 
-    def __init__(self, shapes, dtypes=None, seed=0, weights=None, random_state=False, device="cuda", dims=None):
+    def __init__(self, shapes, dtypes=None, seed=0, weights=None, random_state=False, device="cuda", dims=None, chunk_len=None,
+                 scan_window=None):
         from grokking_optimizers import _cabi
         self.shapes = shapes
         self.P = len(shapes)
@@ -140,7 +141,7 @@ class Sg2Case:
         self.step_fn = _cabi.Sg2Step(self.Wgpu, [s["param"] for s in g], [s["exp_avg"] for s in g],
                                      [s["exp_avg_sq"] for s in g], [s["mu"] for s in g], [s["gru"] for s in g],
                                      [s["mamba_fwd"] for s in g], [s["mamba_bwd"] for s in g], self.counts_gpu,
-                                     dims=self.dims, debug=True)
+                                     dims=self.dims, debug=True, chunk_len=chunk_len, scan_window=scan_window)
         self.offsets = np.concatenate([[0], np.cumsum([wl.numel(s) for s in shapes])]).astype(np.int64)
 
     def gpu_step(self, grads, sharps, per_tensor, shared):

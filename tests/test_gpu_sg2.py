@@ -242,6 +242,27 @@ def test_heavy_ties_sort_is_stable():
         assert np.array_equal(perm[a:b], want)
 
 
+def test_per_call_scan_options_leave_the_process_settings_alone():
+    """Two call plans with their own chunk length and summary window (sg2_batched_step_opt), stepped alternately in one
+    process: each matches the checker run with ITS decomposition, and the process-wide settings stay at their defaults."""
+    from grokking_optimizers import _cabi
+    lib = _cabi.lib()
+    shapes = [(3000,), (64, 65), (700,)]
+    a = Sg2Case(shapes, seed=51, random_state=True, chunk_len=64, scan_window=0)
+    b = Sg2Case(shapes, seed=52, random_state=True, chunk_len=256, scan_window=64)
+    for t in (1, 2):
+        for case, cl, win in ((a, 64, 0), (b, 256, 64)):
+            grads = wl.make_grads(shapes, seed=60 + t)
+            sharps = [g.abs() * 0.5 for g in wl.make_grads(shapes, seed=560 + t)]
+            pt, sh = per_tensor_scalars(case.P, t, 2.0), shared_scalars(4.5)
+            case.gpu_step(grads, sharps, pt, sh)
+            dbg = case.oracle_step(grads, sharps, pt, sh, cl, window=win)
+            print("options", cl, win, "step", t, case.compare(dbg, REL, FLOOR), flush=True)
+    assert lib.sg2_get_chunk_len() == 0 and lib.sg2_get_scan_window() == 64
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        Sg2Case(shapes, seed=53, chunk_len=100)
+
+
 def test_rejects_unsupported_dims_and_small_workspace():
     from grokking_optimizers import _cabi
     import ctypes as C

@@ -97,6 +97,21 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     _run_both(small, 32, 2, W, dev)
     print("static-scratch step, third call (first shapes again)", flush=True)
     _run_both(big, 33, 3, W, dev)
+    # what the entry point exists for: a call allocates nothing, on the device or through torch's allocator
+    st = _state(small, 40, dev)
+    counts = torch.zeros(144, dtype=torch.int32, device=dev)
+    step = _StaticStep(W, st, counts)
+    grads = [g.reshape(-1).to(dev) for g in wl.make_grads(small, seed=41)]
+    sharps = [torch.zeros_like(g) for g in grads]
+    pt, sh = per_tensor_scalars(len(small), 1), shared_scalars()
+    assert step(grads, sharps, pt, sh) == 0
+    torch.cuda.synchronize()
+    free0, alloc0, reserved0 = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        assert step(grads, sharps, pt, sh) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "free device memory changed across static-scratch calls"
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit():
