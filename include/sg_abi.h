@@ -359,6 +359,22 @@ size_t sg2_bilevel_elem_workspace_bytes(int64_t total);
 int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
                      const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
                      float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
+/* ... and additionally the new GRU state of every element, gru_out [total][gru_hidden] (may be NULL): the second
+ * return value of forward_for_bilevel (mamba3_peer_metanet.py:436). */
+int sg2_bilevel_elem_ex(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
+                        const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
+                        float* gru_out, float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* The meta-net's own forward with the step's hard top-1 routing, for callers that use the net outside the fused
+ * step: Mamba3PEERMetaNet.forward (grokking_optimizers/mamba3_peer_metanet.py:275-370 of the reference).  Sort,
+ * scan and the per-element GRU / routing / experts as in sg2_batched_step, without the optimizer update: of every
+ * tensor record only grad, sharpness, gru_state (read), the two Mamba states (replaced by the new carried states),
+ * numel and dtype are used.  rescale: the net's output scale (smart = g + rescale * mean of the heads' expert
+ * outputs).  smart_out [total] and gru_out [total][gru_hidden] are packed in call order;
+ * expert_counts may be NULL.  Workspace as for sg2_batched_step (sg2_workspace_bytes). */
+int sg2_meta_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
+                     float rescale, float* smart_out, float* gru_out, int32_t* expert_counts, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 /* ================== the other fused steps of the reference ================== */
 

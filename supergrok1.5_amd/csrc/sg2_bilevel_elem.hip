@@ -64,7 +64,7 @@ __device__ __forceinline__ void query_entry(int o, int* dcol, int* xcol) {
 
 struct ElemArgs {
     const float *g, *s, *ctx, *gru, *cot;
-    float *smart, *d_ctx, *partials;
+    float *smart, *d_ctx, *partials, *gru_out;
     int total;
     float rescale;
     Sg2Weights W;
@@ -190,6 +190,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 cand[j] = sg_tanh(v);
                 hn[j] = sg_fma(zg[j], cand[j], (1.0f - zg[j]) * h[j]);
             }
+            if (valid && a.gru_out != nullptr) reinterpret_cast<float4*>(a.gru_out)[i] = make_float4(hn[0], hn[1], hn[2], hn[3]);
             xrow[X_G] = g; xrow[X_S] = s; xrow[X_ONE] = 1.0f;
 #pragma unroll
             for (int q = 0; q < DM; q++) { xrow[X_CF + q] = cf[q]; xrow[X_CB + q] = cb[q]; }
@@ -506,6 +507,13 @@ size_t sg2_bilevel_elem_workspace_bytes(int64_t total) {
 int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
                      const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
                      float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
+    return sg2_bilevel_elem_ex(dims, weights, total, grad, sharpness, ctx, gru_state, cotangent, rescale, smart_out, nullptr, d_ctx, grads_out,
+                               workspace, workspace_bytes, stream);
+}
+
+int sg2_bilevel_elem_ex(const SgDims* dims, const Sg2Weights* weights, int64_t total, const float* grad, const float* sharpness,
+                        const float* ctx, const float* gru_state, const float* cotangent, float rescale, float* smart_out,
+                        float* gru_out, float* d_ctx, float* grads_out, void* workspace, size_t workspace_bytes, void* stream) {
     using namespace sg2;
     hipStream_t st = (hipStream_t)stream;
     if (check_dims(dims, true)) return 1;
@@ -518,7 +526,8 @@ int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t tota
         return sg::fail("workspace too small: need %zu bytes, got %zu", sizeof(float) * (size_t)groups * N_GRADS, workspace_bytes);
     if (total > 0) {
         if (!grad || !sharpness || !ctx || !gru_state || !cotangent || !d_ctx) return sg::fail("NULL argument");
-        if ((((uintptr_t)ctx | (uintptr_t)gru_state | (uintptr_t)d_ctx) & 15u) != 0) return sg::fail("ctx, gru_state and d_ctx must be 16-byte aligned");
+        if ((((uintptr_t)ctx | (uintptr_t)gru_state | (uintptr_t)d_ctx | (uintptr_t)gru_out) & 15u) != 0)
+            return sg::fail("ctx, gru_state, gru_out and d_ctx must be 16-byte aligned");
     }
     {
         static bool raised[64] = {};
@@ -532,7 +541,7 @@ int sg2_bilevel_elem(const SgDims* dims, const Sg2Weights* weights, int64_t tota
     }
     ElemArgs a;
     a.g = grad; a.s = sharpness; a.ctx = ctx; a.gru = gru_state; a.cot = cotangent;
-    a.smart = smart_out; a.d_ctx = d_ctx; a.partials = static_cast<float*>(workspace);
+    a.smart = smart_out; a.d_ctx = d_ctx; a.partials = static_cast<float*>(workspace); a.gru_out = gru_out;
     a.total = (int)total; a.rescale = rescale; a.W = *weights;
     hipLaunchKernelGGL(k_bilevel_elem, dim3(groups), dim3(BE_THREADS), BE_LDS_BYTES, st, a);
     SG_LAUNCH_CHECK("k_bilevel_elem");

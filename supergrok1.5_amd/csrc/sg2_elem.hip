@@ -251,9 +251,12 @@ __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(el
 // chains); the shared reciprocals of the gates apply when gru_hidden is 4, as in the checker.  ctx rows are
 // ctx_stride floats apart (d_model of the scan geometry the block was embedded in).
 constexpr int MAX_DM = 16, MAX_GH = 8, MAX_HD = 8, CNT_LDS = 4096;
+// fwd_smart / fwd_gru (both or neither): the net's forward alone -- smart gradient and new GRU state of every element go
+// to these packed arrays, nothing of the optimizer state is read or written (sg2_meta_forward).
 template <bool DBG>
 __global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stride, int32_t* __restrict__ expert_counts,
-                                                           int32_t* __restrict__ dbg_eidx) {
+                                                           int32_t* __restrict__ dbg_eidx, float* __restrict__ fwd_smart,
+                                                           float* __restrict__ fwd_gru) {
     __shared__ int s_cnt[CNT_LDS];
     const int dm = pl.dims.d_model, gh = pl.dims.gru_hidden, H = pl.dims.num_heads, pk = pl.dims.pk_dim;
     const int eh = pl.dims.expert_hidden, E = pl.dims.num_experts, hd = dm / 2;
@@ -355,7 +358,10 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stri
 #pragma unroll
             for (int j = 0; j < MAX_GH; j++) {
                 hnew[j] = sg_fma(gate[j], cand[j], (1.0f - gate[j]) * hold[j]);
-                if (j < gh) sg::gptr(T.gru)[(size_t)i * gh + j] = hnew[j];
+                if (j < gh) {
+                    if (fwd_gru != nullptr) sg::gptr(fwd_gru)[((size_t)T.off + i) * gh + j] = hnew[j];
+                    else sg::gptr(T.gru)[(size_t)i * gh + j] = hnew[j];
+                }
             }
 
             // ---- PEER: per head the query (chain order = h, fwd ctx, bwd ctx, g, s), two sub-key arg-maxes, the expert
@@ -407,6 +413,10 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stri
                 total = total + ho;
             }
             const float smart = g + (rescale * total) / (float)H;
+            if (fwd_smart != nullptr) {
+                sg::gptr(fwd_smart)[(size_t)T.off + i] = smart;
+                continue;
+            }
 
             // ---- mu EMA, Adam moments, decoupled weight decay
             float mu = sg::gptr(T.mu)[i], ea = sg::gptr(T.ea)[i], easq = sg::gptr(T.easq)[i];
@@ -431,6 +441,14 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stri
 
 }  // namespace
 
+int launch_elem_forward(const Plan& pl, int32_t* expert_counts, float* smart_out, float* gru_out, hipStream_t st) {
+    if (pl.total == 0) return 0;
+    const int grid = pl.elem_tiles < 4096 ? pl.elem_tiles : 4096;
+    hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, geo_info(pl.geo).dm, expert_counts, nullptr, smart_out, gru_out);
+    SG_LAUNCH_CHECK("k_elem_any<forward>");
+    return 0;
+}
+
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st) {
     if (pl.total == 0) return 0;
     // about five workgroups per resident slot (768 at three per CU): measured 1.38 / 1.35 / 1.33 / 1.33 / 1.37 ms with 768 / 2048 / 4096 /
@@ -439,8 +457,9 @@ int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx,
     auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx); };
     if (pl.elem_kind == ELEM_ANY) {
         const int stride = geo_info(pl.geo).dm;
-        if (dbg_expert_idx) hipLaunchKernelGGL(k_elem_any<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx);
-        else hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx);
+        float* const none = nullptr;
+        if (dbg_expert_idx) hipLaunchKernelGGL(k_elem_any<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx, none, none);
+        else hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx, none, none);
     } else if (pl.geo == GEO_LARGE) {
         if (dbg_expert_idx) go(k_elem<GeoLarge, 16, true>);
         else go(k_elem<GeoLarge, 16, false>);

@@ -160,5 +160,7 @@ int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* con
                             hipStream_t st);
 int launch_x_sorted(const Plan& pl, float* x_out, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
+// the net's forward alone (run-time-dimension kernel): smart gradients [total] and new GRU states [total][gru_hidden], packed
+int launch_elem_forward(const Plan& pl, int32_t* expert_counts, float* smart_out, float* gru_out, hipStream_t st);
 
 }  // namespace sg2

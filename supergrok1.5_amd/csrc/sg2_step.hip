@@ -570,6 +570,24 @@ int sg2_batched_step_static(const SgDims* dims, const Sg2Weights* weights, int n
                     (hipStream_t)stream);
 }
 
+int sg2_meta_forward(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors, float rescale,
+                     float* smart_out, float* gru_out, int32_t* expert_counts, void* workspace, size_t workspace_bytes, void* stream) {
+    using namespace sg2;
+    hipStream_t st = (hipStream_t)stream;
+    Plan pl;
+    Layout L;
+    const Sg2Scalars none = {rescale, 0.0f, 0.0f, 0.0f, 0.0f};
+    if (num_tensors > 0 && tensors)
+        for (int i = 0; i < num_tensors; i++)
+            if (tensors[i].numel > 0 && !tensors[i].gru_state) return sg::fail("tensor %d: gru_state is NULL", i);
+    if (build_plan(dims, weights, num_tensors, tensors, &none, workspace, workspace_bytes, false, false, false, st, &pl, &L)) return 1;
+    if (pl.total == 0) return 0;
+    if (!smart_out || !gru_out) return sg::fail("smart_out / gru_out is NULL");
+    if (launch_sort(pl, nullptr, st)) return 1;
+    if (launch_scan(pl, st)) return 1;
+    return launch_elem_forward(pl, expert_counts, smart_out, gru_out, st);
+}
+
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels) {
     if (sg2::check_dims(dims) || num_tensors < 0 || (num_tensors > 0 && !numels)) return 0;
     sg2::Layout L;

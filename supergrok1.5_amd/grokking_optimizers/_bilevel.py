@@ -8,10 +8,13 @@ end: sort + bidirectional Mamba-3 scan (sg2_bilevel_forward), per-element GRU /
 soft top-4 PEER routing / expert MLPs forward and backward in one pass
 (sg2_bilevel_elem), then the exact adjoint of the scan down to the gradients
 of the scan's weights (sg2_bilevel_backward).
-`forward_for_bilevel` is the module-level differentiable forward of one tensor:
-the scan as an autograd Function over the same two entry points, the per-element
-part as torch ops (`per_element`), which is also what the tests check
-sg2_bilevel_elem against.
+`forward_for_bilevel` is the module-level differentiable forward of one tensor
+over the same kernels: the scan as one autograd Function (ScanContexts), the
+per-element part as another (SoftElements over sg2_bilevel_elem).  `forward`
+(hard top-1 routing, no gradients) is one call of sg2_meta_forward.  `per_element`
+restates the per-element part in torch ops: the tests check sg2_bilevel_elem
+against it, and it serves meta-nets whose GRU / routing / expert sizes the
+per-element bilevel kernel is not built for.
 """
 import torch
 
@@ -102,26 +105,67 @@ def per_element(mn, g, s, ctx_f, ctx_b, gru_state, topk=4):
     return g + mn.rescale * (total / mn.num_peer_heads), h_new
 
 
+class SoftElements(torch.autograd.Function):
+    """(smart_grad, new GRU state) of N elements from their two contexts, soft top-4 routing, through sg2_bilevel_elem
+    (forward and backward are the same fused kernel: the forward call runs it with a zero cotangent).  Gradients
+    reach the contexts and the 42 - 20 = 22 parameter tensors of the per-element part; the gradient, the sharpness
+    and the old GRU state are data, and the new GRU state is returned without a gradient path (nothing in the
+    reference differentiates through it)."""
+
+    @staticmethod
+    def forward(ctx, weights33, dims, rescale, g, s, h, contexts, *elem_params):
+        smart, _, _, h_new = _cabi.bilevel_elem(weights33, g, s, contexts, h, torch.zeros_like(g), rescale, dims, want_gru=True)
+        ctx.args = (weights33, dims, rescale)
+        ctx.save_for_backward(g, s, h, contexts, *elem_params)
+        ctx.mark_non_differentiable(h_new)
+        return smart, h_new
+
+    @staticmethod
+    def backward(ctx, d_smart, _d_h):
+        weights33, dims, rescale = ctx.args
+        g, s, h, contexts = ctx.saved_tensors[:4]
+        params = ctx.saved_tensors[4:]
+        _, d_ctx, blk = _cabi.bilevel_elem(weights33, g, s, contexts, h, d_smart.contiguous(), rescale, dims, want_smart=False)
+        return (None, None, None, None, None, None, d_ctx) + tuple(gr.to(p.dtype) for gr, p in zip(split_flat(blk, params), params))
+
+
+def elem_kernel_fits(mn):
+    """Whether sg2_bilevel_elem is built for this net's per-element sizes (experts narrower than its 16 run embedded)."""
+    d = meta_dims(mn)
+    return ((d["d_model"], d["d_state"], d["d_inner"], d["gru_hidden"], d["num_heads"], d["pk_dim"], d["num_experts"]) == (8, 16, 16, 4, 4, 12, 144)
+            and d["expert_hidden"] <= _cabi.BILEVEL_EXPERT_WIDTH)
+
+
 def forward(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
     """The step's own forward (hard top-1 routing) as a module call, for callers that use the meta-net outside the
-    fused step: same return values as the reference's Mamba3PEERMetaNet.forward."""
-    g = grad.reshape(-1).float()
-    s = sharpness.reshape(-1).float()
-    plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
-    ctx = ScanContexts.apply(plan, *scan_parameters(mn))
-    smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float(), topk=0)
-    return smart.reshape(grad.shape).to(grad.dtype), h_new, plan.mf[0], plan.mb[0]
+    fused step: same return values as the reference's Mamba3PEERMetaNet.forward, computed by one call of
+    sg2_meta_forward (sort, scan, GRU, routing, experts in HIP).  No gradient path: bilevel training differentiates
+    forward_for_bilevel."""
+    dev = grad.device
+    if dev.type != "cuda":
+        raise RuntimeError("the SuperGrok v2 meta-net needs GPU tensors: there is no CPU path")
+    g = grad.reshape(-1).float().contiguous()
+    s = sharpness.reshape(-1).float().contiguous()
+    shape = (mn.mamba_fwd.d_inner, mn.d_state)
+    state = lambda m: torch.zeros(*shape, dtype=torch.float32, device=dev) if m is None else m.detach().float().contiguous().clone()
+    mf, mb = state(mamba_fwd_state), state(mamba_bwd_state)
+    smart, h_new = _cabi.meta_forward(mn.flat_weights(), [g], [s], [gru_state], [mf], [mb], float(mn.rescale), meta_dims(mn))
+    return smart.reshape(grad.shape).to(grad.dtype), h_new, mf, mb
 
 
 def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
     """Differentiable forward of one tensor, the reference's return values: (smart_grad, new_gru, new_mamba_fwd_state,
-    new_mamba_bwd_state); gradients reach every parameter of `mn` (the two new states are plain tensors: nothing in
+    new_mamba_bwd_state); gradients reach every parameter of `mn` (the new states are plain tensors: nothing in
     the reference differentiates through them)."""
     g = grad.reshape(-1).float()
     s = sharpness.reshape(-1).float()
     plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
     ctx = ScanContexts.apply(plan, *scan_parameters(mn))
-    smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float())
+    if elem_kernel_fits(mn):
+        smart, h_new = SoftElements.apply(plan.weights, meta_dims(mn), float(mn.rescale), g.contiguous(), s.contiguous(),
+                                          gru_state.detach().float().contiguous(), ctx, *elem_parameters(mn))
+    else:
+        smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float())
     return smart.reshape(grad.shape).to(grad.dtype), h_new, plan.mf[0], plan.mb[0]
 
 

@@ -96,6 +96,12 @@ def lib():
         L.sg2_bilevel_elem.restype = C.c_int
         L.sg2_bilevel_elem.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int64] + [C.c_void_p] * 5 + [C.c_float] + \
                                       [C.c_void_p] * 4 + [C.c_size_t, C.c_void_p]
+        L.sg2_bilevel_elem_ex.restype = C.c_int
+        L.sg2_bilevel_elem_ex.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int64] + [C.c_void_p] * 5 + [C.c_float] + \
+                                         [C.c_void_p] * 5 + [C.c_size_t, C.c_void_p]
+        L.sg2_meta_forward.restype = C.c_int
+        L.sg2_meta_forward.argtypes = [C.POINTER(SgDims), C.POINTER(Sg2Weights), C.c_int, C.POINTER(Sg2Tensor), C.c_float, C.c_void_p,
+                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         _lib = L
     return _lib
 
@@ -260,9 +266,9 @@ SG2_ELEM_GRAD_FLOATS = 8420
 BILEVEL_EXPERT_WIDTH = 16      # expert width sg2_bilevel_elem is compiled for
 
 
-def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, dims=None, want_smart=True):
+def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, dims=None, want_smart=True, want_gru=False):
     """sg2_bilevel_elem on flat fp32 GPU arrays: returns (smart [total] or None, d_ctx [2, total, d_model],
-    weight-gradient block [SG2_ELEM_GRAD_FLOATS])."""
+    weight-gradient block [SG2_ELEM_GRAD_FLOATS]); with want_gru a fourth value, the new GRU state [total, gru_hidden]."""
     d = make_dims(dims)
     ws_ = [w.detach().float().contiguous() for w in weights]
     # The kernel is built for experts of width 16.  Narrower experts (the reference's training harness uses 4) run as
@@ -288,13 +294,51 @@ def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, d
     out = torch.empty(SG2_ELEM_GRAD_FLOATS, dtype=torch.float32, device=dev)
     nbytes = lib().sg2_bilevel_elem_workspace_bytes(total)
     work = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
-    rc = lib().sg2_bilevel_elem(C.byref(d), C.byref(W), total, *[t.data_ptr() for t in arrs], float(rescale),
-                                smart.data_ptr() if want_smart else None, d_ctx.data_ptr(), out.data_ptr(), work.data_ptr(),
-                                work.numel(), torch.cuda.current_stream().cuda_stream)
+    gru_out = torch.empty_like(arrs[3]) if want_gru else None
+    rc = lib().sg2_bilevel_elem_ex(C.byref(d), C.byref(W), total, *[t.data_ptr() for t in arrs], float(rescale),
+                                   smart.data_ptr() if want_smart else None, gru_out.data_ptr() if want_gru else None, d_ctx.data_ptr(),
+                                   out.data_ptr(), work.data_ptr(), work.numel(), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError("sg2_bilevel_elem: " + last_error())
     if eh < BILEVEL_EXPERT_WIDTH:       # expert part of the block: W1, b1, W2 [E, 16] each, then b2 [E]
         head = out.numel() - (3 * BILEVEL_EXPERT_WIDTH + 1) * E
         ex = out[head:head + 3 * BILEVEL_EXPERT_WIDTH * E].view(3, E, BILEVEL_EXPERT_WIDTH)[:, :, :eh].reshape(-1)
         out = torch.cat([out[:head], ex, out[-E:]])
+    if want_gru:
+        return smart, d_ctx, out, gru_out
     return smart, d_ctx, out
+
+
+def meta_forward(weights, grads, sharps, gru_states, mamba_fwd, mamba_bwd, rescale, dims=None, expert_counts=None):
+    """sg2_meta_forward: the meta-net's forward (hard top-1 routing) for a list of flat tensors.  mamba_fwd / mamba_bwd
+    are replaced by the new carried states.  Returns (smart [total], new GRU state [total, gru_hidden]), packed in call
+    order."""
+    d = make_dims(dims)
+    ws_ = [w.detach().float().contiguous() for w in weights]
+    W = Sg2Weights()
+    for k, w in enumerate(ws_):
+        W.w[k] = w.data_ptr()
+    P = len(grads)
+    dev = grads[0].device
+    numels = [g.numel() for g in grads]
+    total = sum(numels)
+    keep = []
+    tensors = (Sg2Tensor * P)()
+    for i in range(P):
+        g, s, h = grads[i].contiguous(), sharps[i].contiguous(), gru_states[i].detach().float().contiguous()
+        assert s.dtype == g.dtype and s.numel() == g.numel() and h.numel() == g.numel() * d.gru_hidden
+        assert mamba_fwd[i].dtype == torch.float32 and mamba_fwd[i].is_contiguous() and mamba_bwd[i].is_contiguous()
+        keep += [g, s, h]
+        t = tensors[i]
+        t.grad, t.sharpness, t.gru_state = g.data_ptr(), s.data_ptr(), h.data_ptr()
+        t.mamba_fwd_state, t.mamba_bwd_state = mamba_fwd[i].data_ptr(), mamba_bwd[i].data_ptr()
+        t.numel, t.dtype = g.numel(), SG_DTYPE[g.dtype]
+    smart = torch.empty(total, dtype=torch.float32, device=dev)
+    gru_out = torch.empty(total, d.gru_hidden, dtype=torch.float32, device=dev)
+    work = torch.empty(max(workspace_bytes(numels, dims), 256), dtype=torch.uint8, device=dev)
+    rc = lib().sg2_meta_forward(C.byref(d), C.byref(W), P, tensors, float(rescale), smart.data_ptr(), gru_out.data_ptr(),
+                                expert_counts.data_ptr() if expert_counts is not None else None, work.data_ptr(), work.numel(),
+                                torch.cuda.current_stream().cuda_stream)
+    if rc != 0:
+        raise RuntimeError("sg2_meta_forward: " + last_error())
+    return smart, gru_out

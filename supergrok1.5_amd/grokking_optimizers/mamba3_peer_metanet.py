@@ -9,8 +9,11 @@ is the host-side expert recycling.
 The arithmetic of the network runs inside the fused HIP step
 (`_ops.supergrok2_mamba_peer_batched_step`).  `forward` (:275-370 there) and
 `forward_for_bilevel` (:372-436 there, soft top-4 routing) are kept for callers
-that use the module outside the optimizer: sort and scan in HIP (forward and
-adjoint), the per-element part as torch ops; GPU tensors only.
+that use the module outside the optimizer and run on the same kernels:
+`forward` is one call of the library's forward-only entry point
+(sg2_meta_forward: sort, scan, GRU, routing, experts), `forward_for_bilevel`
+is differentiable through two autograd Functions over the bilevel kernels (scan
+forward / adjoint, per-element forward / backward).  GPU tensors only.
 """
 import math
 

@@ -314,24 +314,33 @@ def test_optimizer_bilevel_step_and_step_full():
     assert all(np.isfinite(losses)) and losses[-1] < losses[0]
 
 
-def test_module_forward_matches_the_float64_step():
-    """Mamba3PEERMetaNet.forward (hard top-1 routing, HIP scan + torch per-element part) against the float64
-    restatement of the step: smart gradient, new GRU state, both new Mamba states; expert choices may differ only at
-    near-ties, which the tolerance on smart (1e-4 of its scale) would expose."""
+@pytest.mark.parametrize("kw", [dict(), dict(expert_hidden=4), dict(d_model=4, d_state=8, gru_hidden=3, num_peer_heads=2, num_experts=25, expert_hidden=6)])
+def test_module_forward_matches_the_float64_step(kw):
+    """Mamba3PEERMetaNet.forward (hard top-1 routing; one call of sg2_meta_forward: sort, scan, GRU, routing and experts
+    in HIP, at the default sizes and at others) against the float64 restatement of the step: smart gradient, new GRU
+    state, both new Mamba states; expert choices may differ only at near-ties, which the tolerance on smart (1e-4 of
+    its scale) would expose.  The caller's states are not modified."""
     dev = torch.device("cuda:0")
-    mn = _meta_net(21, dev)
+    mn = _meta_net(21, dev, **kw)
     gen = torch.Generator().manual_seed(22)
     n = 333
+    di, ds, gh = mn.mamba_fwd.d_inner, mn.d_state, mn.gru_hidden
     g, s = torch.randn(n, generator=gen) * 0.5, torch.rand(n, generator=gen) * 0.3
-    h = torch.randn(n, 4, generator=gen) * 0.5
-    hf, hb = torch.randn(16, 16, generator=gen) * 0.3, torch.randn(16, 16, generator=gen) * 0.3
-    print("module forward, N", n, flush=True)
-    smart, hn, nf, nb = mn(g.to(dev), s.to(dev), h.to(dev), hf.to(dev), hb.to(dev))
-    dims = dict(d_model=8, gru_hidden=4, num_heads=4, pk_dim=12)
+    h = torch.randn(n, gh, generator=gen) * 0.5
+    hf, hb = torch.randn(di, ds, generator=gen) * 0.3, torch.randn(di, ds, generator=gen) * 0.3
+    print("module forward, N", n, kw, flush=True)
+    hf_dev, hb_dev, h_dev = hf.to(dev), hb.to(dev), h.to(dev)
+    smart, hn, nf, nb = mn(g.to(dev), s.to(dev), h_dev, hf_dev, hb_dev)
+    assert torch.equal(hf_dev.cpu(), hf) and torch.equal(hb_dev.cpu(), hb) and torch.equal(h_dev.cpu(), h)
+    dims = dict(d_model=mn.d_model, gru_hidden=gh, num_heads=mn.num_peer_heads, pk_dim=mn.pk_dim)
     sc = dict(rescale=mn.rescale, alpha=0.0, lamb_eff=0.0, beta1=0.9, beta2=0.999, bc1=1.0, bc2=1.0, eps=1e-8, lr=0.0, wd_eff=0.0)
     z = torch.zeros(n)
-    ref = ref_fp64.step([w.cpu() for w in mn.flat_weights()], z, g, s, z, z, z, h, hf, hb, sc, dims)
+    import workloads as wl
+    full = dict(d_model=mn.d_model, d_state=ds, d_inner=di, gru_hidden=gh, num_heads=mn.num_peer_heads, pk_dim=mn.pk_dim,
+                expert_hidden=mn.expert_hidden, num_experts=mn.num_experts)
+    W = [w.cpu().reshape(shape) for w, shape in zip(mn.flat_weights(), wl.meta_weight_shapes(full))]
+    ref = ref_fp64.step(W, z, g, s, z, z, z, h, hf, hb, sc, dims)
     for name, got, want in (("smart", smart, ref["smart"]), ("gru", hn, ref["gru"]), ("mamba_fwd", nf, ref["mamba_fwd"]),
                             ("mamba_bwd", nb, ref["mamba_bwd"])):
         got = got.detach().double().cpu()
-        assert float((got - want).abs().max()) <= 1e-4 * float(want.abs().max()) + 1e-7, name
+        assert float((got - want).abs().max()) <= 1e-4 * float(want.abs().max()) + 1e-7, (name, kw)
