@@ -21,7 +21,7 @@ for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd")):
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
 SIMDS = 1024
-STAGE_KERNEL_PREFIX = {"scan_output": "k_scan<true, false>", "scan_summary": "k_scan<false, false>", "elementwise": "k_elem<"}
+STAGE_KERNEL_PREFIX = {"scan_output": "k_replay<", "scan_summary": "k_scan<false, false>", "elementwise": "k_elem<"}
 
 
 def profile_figures():
@@ -642,7 +642,7 @@ def main():
     value = total * args.steps / elapsed
     dom = max(stage_avg, key=stage_avg.get)
     kernel_of = {"sort": "k_keys + 4 x (k_hist, k_spine_*, k_scatter)", "scan_summary": "k_scan<false>",
-                 "chunk_prefix": "k_chunk_prefix", "scan_output": "k_scan<true>", "elementwise": "k_elem<false>"}
+                 "chunk_prefix": "k_chunk_prefix", "scan_output": "k_replay", "elementwise": "k_elem<false>"}
     achieved = BYTES_PER_ELEMENT * total / (stage_avg[dom] * 1e-3) / 1e9
     default_workload = (args.workload, args.weights, args.geometry, args.sharpness) == ("scale50", "bench", "default", False)
     prof = profile_figures() if default_workload else {"traffic": {}, "valu": {}, "sustained": None, "source": {}}
