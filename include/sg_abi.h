@@ -85,8 +85,8 @@ typedef struct Sg2Debug {
 const char* sg_last_error(void);
 
 /* Length (timesteps) of the scan chunks a tensor's sorted sequence is cut
- * into; a multiple of 64.  0 (the default) lets each call choose 4096, 2048
- * or 1024 from the amount of work; sg2_chunk_len_for tells what a call with
+ * into; a multiple of 64.  0 (the default) lets each call choose 4096, 2048,
+ * 1024 or 512 from the amount of work; sg2_chunk_len_for tells what a call with
  * these tensor sizes will use.  Affects results only by re-association of the
  * chunk products. */
 int sg2_set_chunk_len(int chunk_len);

@@ -32,8 +32,10 @@ std::mutex g_bilevel_mutex;
 std::map<const void*, BilevelRecord> g_bilevel_records;
 
 // Longer chunks mean fewer summaries (less work in the first scan pass and the prefix), shorter chunks
-// mean more workgroups.  Take the longest of 4096 / 2048 / 1024 that still gives the replay pass about
-// four full waves of workgroups on 256 CUs.
+// mean more workgroups.  The replay runs one wave per chunk and direction, 2048 of them resident on 256 CUs:
+// take the longest of 4096 / 2048 / 1024 that still gives two full rounds of them, else 512 (on the 14-tensor set
+// of 0.42 M elements: 0.31 ms per step with 512, 0.36 with 1024, 0.33 with 256, whose summaries cost more than
+// the extra waves gain).
 // tensor sizes of a call, either as a plain array (the *_bytes queries) or read from the tensor records (no copy)
 struct Numels {
     const int64_t* plain;
@@ -42,12 +44,12 @@ struct Numels {
 };
 
 int auto_chunk_len(int P, Numels numels) {
-    for (int L = 4096; L > 1024; L >>= 1) {
+    for (int L = 4096; L > 512; L >>= 1) {
         int64_t wgs = 0;
         for (int i = 0; i < P; i++) wgs += 2 * ((numels[i] + L - 1) / L);
-        if (wgs >= 8192) return L;
+        if (wgs >= 4096) return L;
     }
-    return 1024;
+    return 512;
 }
 int effective_chunk_len(int P, Numels numels) {
     const int set = g_chunk_len.load();

@@ -36,7 +36,7 @@ def test_host_side_validation_without_gpu():
     assert lib.sg2_set_chunk_len(100) != 0 and b"multiple of 64" in lib.sg_last_error()
     assert lib.sg2_set_chunk_len(256) == 0 and lib.sg2_get_chunk_len() == 256
     assert lib.sg2_set_chunk_len(0) == 0 and lib.sg2_get_chunk_len() == 0
-    assert _cabi.chunk_len_for([1000, 5000]) == 1024 and _cabi.chunk_len_for([4 << 20] * 8) == 4096
+    assert _cabi.chunk_len_for([1000, 5000]) == 512 and _cabi.chunk_len_for([4 << 20] * 8) == 4096 and _cabi.chunk_len_for([1 << 20] * 3) == 1024
     assert lib.sg2_set_scan_window(100) != 0 and lib.sg2_set_scan_window(128) == 0 and lib.sg2_get_scan_window() == 128
     assert lib.sg2_set_scan_window(-1) == 0 and lib.sg2_get_scan_window() == 64
 

@@ -99,9 +99,8 @@ def test_supergrok2_class_against_checker_with_recycling():
             b1 = 0.9 * (0.9 ** i)
             sc = dict(alpha=f32(0.98), lamb_eff=f32(lamb_eff), beta1=f32(b1), bc1=f32(1.0 - b1 ** t), bc2=f32(1.0 - 0.999 ** t),
                       rescale=f32(0.1), beta2=f32(0.999), lr=f32(1e-3), wd_eff=f32(wd_eff), eps=f32(1e-8))
-            orc.sg2_step(W, ref[i], np.ascontiguousarray(gi, np.float32), np.zeros_like(gn), sc, chunk_len=1024, window=_cabi.lib().sg2_get_scan_window(),   # 745 elements: the automatic choice is 1024
-                        
-                         expert_counts=step_counts)
+            orc.sg2_step(W, ref[i], np.ascontiguousarray(gi, np.float32), np.zeros_like(gn), sc, chunk_len=_cabi.chunk_len_for([g_.numel() for g_ in grads]),
+                         window=_cabi.lib().sg2_get_scan_window(), expert_counts=step_counts)
         for i, p in enumerate(params):
             ok, r = rel_close(p.detach().cpu().numpy().reshape(-1), ref[i]["param"], 1e-4, 1e-7)
             assert ok, ("param", t, i, r)
