@@ -27,11 +27,17 @@ extern "C" {
 enum { SG_F32 = 0, SG_F16 = 1, SG_BF16 = 2 };
 
 /* meta-net dimensions, the trailing ints of
- * launch_mamba3_peer_batched_step (csrc/ops.h:196-229).  The step kernels
- * are built for (d_model, d_state, d_inner) = (8, 16, 16) and (16, 32, 32),
- * both with gru_hidden 4, num_heads 4, pk_dim 12, expert_hidden 16 and
- * num_experts 144; anything else is refused with an error that says so.
- * The bilevel entry points take the first set only. */
+ * launch_mamba3_peer_batched_step (csrc/ops.h:196-229).  The step takes every
+ * set that the reference's kernels admit
+ * (supergrok2_mamba_peer_kernels.cu:1796-1801: d_state even and <= 32,
+ * d_model <= 16, d_inner a multiple of 4 and <= 32, gru_hidden <= 8) with
+ * d_model even and num_experts <= pk_dim * pk_dim; anything else is refused
+ * with an error that names the limit.  Scan blocks other than the two
+ * compiled ones, (d_model, d_state, d_inner) = (8, 16, 16) and (16, 32, 32),
+ * run embedded in the smallest compiled block that holds them.  The bilevel
+ * entry points take (8, 16, 16) with gru_hidden 4, num_heads 4, pk_dim 12 and
+ * expert_hidden <= 16 (sg2_bilevel_elem: exactly 16; narrower experts are
+ * passed zero-padded). */
 typedef struct SgDims {
     int32_t d_model, d_state, d_inner, gru_hidden, num_heads, pk_dim, expert_hidden, num_experts;
 } SgDims;
