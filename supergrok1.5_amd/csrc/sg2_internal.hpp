@@ -126,7 +126,8 @@ struct Plan {
     float* adj_lam;                // bilevel: [2][chunks][128][2] adjoint state arriving at the end of every chunk
     float* adj_blk;                // bilevel: [2][SG2_BWD_STRIDE] sums of adj_part's rows
     float* adj_part;               // bilevel: [2][ADJ_GROUPS][SG2_BWD_STRIDE] per-workgroup gradient sums
-    int* contracted;               // [0] set by k_compose (1 while every carried state of the call is finite), cleared by any summary whose 2x2 part is not exactly zero; [1] steps of a summary's first block (k_compose); [2] set by k_tables: some carried state is not finite
+    int* contracted;               // [0] set by k_compose (1 while every carried state of the call is finite), cleared by any summary whose 2x2 part is not exactly zero; [1] steps of a summary's first block (k_compose); [2] k_compose: some carried state is not finite
+    int* state_bad;                // [P] set by k_tables: a carried Mamba state of the tensor holds a non-finite entry
     int* sharp_nonzero;            // [P] uploaded as 0; set by k_keys when some (finite) sharpness entry of the tensor is not 0
     float* ctx;                    // [2][total][d_model]
     float decay, beta2, eps, rescale;

@@ -193,9 +193,9 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[2] = out[2];
     // How many steps the first block of a chunk summary should cover: what the slowest pair of either direction needs
     // to contract below 2^-100 at the step size a zero input gives (sg2_contraction_steps), plus a margin.
-    __shared__ int s_largest, s_zero, s_cmax[2][2], s_cdt[2][2], s_amax[2], s_fmax[2];
+    __shared__ int s_largest, s_zero, s_bad, s_cmax[2][2], s_cdt[2][2], s_amax[2], s_fmax[2];
     if (threadIdx.x == 0) {
-        s_largest = 0; s_zero = 0;
+        s_largest = 0; s_zero = 0; s_bad = 0;
         for (int k = 0; k < 2; k++) { s_cmax[k][0] = s_cmax[k][1] = s_cdt[k][0] = s_cdt[k][1] = s_amax[k] = s_fmax[k] = 0; }
     }
     __syncthreads();
@@ -227,9 +227,12 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
             atomicMax(&s_fmax[dir], sg_f2i(sg_abs(pl.W.w[dir ? W_B_ROPE : W_F_ROPE][row * G::HP + p])));
         }
     }
+    for (int i = threadIdx.x; i < pl.P; i += blockDim.x)
+        if (pl.state_bad[i] != 0) s_bad = 1;       // plain store: every writer stores the same value
     __syncthreads();
     if (threadIdx.x == 0) {
-        pl.contracted[0] = pl.contracted[2] == 0 ? 1 : 0;      // until a summary kernel finds a chunk that has not contracted; never while a carried state is not finite
+        pl.contracted[0] = s_bad == 0 ? 1 : 0;      // until a summary kernel finds a chunk that has not contracted; never while a carried state is not finite
+        pl.contracted[2] = s_bad;
         pl.contracted[1] = sg2_first_block_steps(s_largest, s_zero);
         float* cmax = pl.comp + 2 * SG2_COMP_GROUPS * G::ROWS * 3 + 2 * 2 * G::ROWS * 4;
         cmax[0] = sg_i2f(s_cmax[0][0]); cmax[1] = sg_i2f(s_cmax[0][1]);

@@ -154,7 +154,7 @@ int make_layout(int geo, int P, Numels numels, int chunk_len, Layout* L, bool bi
     L->off_summ = take(4 * 2 * (size_t)wch * 6 * gi.threads);
     L->off_hstart = take(4 * 2 * (size_t)ch * 2 * gi.threads);
     L->off_comp = take(4 * (2 * 5 * (size_t)gi.rows * 3 + 2 * 2 * (size_t)gi.rows * 4 + 12));      // composed triples, Taylor polynomials, coefficient maxima and polynomial limits
-    L->off_flags = take(4 * ((size_t)P + 3));        // apart from the tensor records: it is written while those are being read
+    L->off_flags = take(4 * (2 * (size_t)P + 3));    // apart from the tensor records: it is written while those are being read
     L->off_padw = take(4 * (size_t)padded_weight_floats(gi));   // scan weights embedded in the kernel geometry (used when the caller's block is smaller)
     L->off_ctx = take(4 * 2 * (size_t)total * gi.dm);
     // bilevel only: state entering every HT_STEP-th step, both directions
@@ -177,12 +177,27 @@ struct TableChunk {
     TensorDev* dst_rec;
     int* dst_pre;                  // four tables of P+1 ints, back to back
     int* flags;                    // per-tensor "sharpness is not all zero" flags to clear, or NULL to keep them
-    int* nonfinite;                // with flags: set to 1 when a carried Mamba state of some tensor holds a non-finite entry
+    int* state_bad;                // with flags: per tensor, 1 when one of its carried Mamba states holds a non-finite entry
     int i0, cnt, P, state_floats;  // state_floats: d_inner * d_state of the caller's states
 };
 static_assert(sizeof(TableChunk) <= 3600, "kernel arguments stay well below 4 KB");
 
+// Workgroup 0 writes the records and tables; workgroup 1 + k looks at the carried states of tensor i0 + k.
 __global__ __launch_bounds__(256) void k_tables(TableChunk c) {
+    if (blockIdx.x > 0) {
+        // A tensor whose carried state is not finite (a diverged run) must come out non-finite as a whole, as it does in
+        // the reference, which multiplies every chunk's start state through: the scan only lets contracted summaries
+        // forget what came before them while every carried state of the call is finite (k_compose reads these flags).
+        const int k = blockIdx.x - 1;
+        const TensorDev& t = c.rec[k];
+        bool bad = false;
+        if (t.numel > 0)
+            for (int r = threadIdx.x; r < 2 * c.state_floats; r += 256)
+                bad = bad || !sg_isfinite((r < c.state_floats ? t.mfwd : t.mbwd)[r % c.state_floats]);
+        const int any = __syncthreads_or(bad ? 1 : 0);
+        if (threadIdx.x == 0) c.state_bad[c.i0 + k] = any ? 1 : 0;
+        return;
+    }
     constexpr int WORDS = sizeof(TensorDev) / 4;
     const int* src = reinterpret_cast<const int*>(c.rec);
     int* dst = reinterpret_cast<int*>(c.dst_rec + c.i0);
@@ -192,21 +207,8 @@ __global__ __launch_bounds__(256) void k_tables(TableChunk c) {
         c.dst_pre[q * (c.P + 1) + c.i0 + 1 + k] = c.pre[q][k];
     }
     if (c.i0 == 0 && threadIdx.x < 4) c.dst_pre[threadIdx.x * (c.P + 1)] = 0;
-    if (c.flags != nullptr) {
+    if (c.flags != nullptr)
         for (int k = threadIdx.x; k < c.cnt; k += 256) c.flags[c.i0 + k] = 0;
-        // A tensor whose carried state is not finite (a diverged run) must come out non-finite as a whole, as it does in
-        // the reference, which multiplies every chunk's start state through: the scan only lets contracted summaries
-        // forget what came before them while every carried state of the call is finite (k_compose reads this flag).
-        if (c.i0 == 0 && threadIdx.x == 0) *c.nonfinite = 0;
-        __syncthreads();
-        bool bad = false;
-        for (int w = threadIdx.x; w < c.cnt * 2 * c.state_floats; w += 256) {
-            const int k = w / (2 * c.state_floats), r = w % (2 * c.state_floats);
-            const TensorDev& t = c.rec[k];
-            if (t.numel > 0) bad = bad || !sg_isfinite((r < c.state_floats ? t.mfwd : t.mbwd)[r % c.state_floats]);
-        }
-        if (bad) *c.nonfinite = 1;       // plain store: every writer stores the same value
-    }
 }
 
 }  // namespace
@@ -387,7 +389,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
         for (int i0 = 0; i0 < P; i0 += UPLOAD_RECS) {
             TableChunk c;
             c.dst_rec = d_rec; c.dst_pre = d_pre; c.flags = d_flags;
-            c.nonfinite = reinterpret_cast<int*>(ws + L.off_flags) + P + 2;
+            c.state_bad = reinterpret_cast<int*>(ws + L.off_flags) + P + 3;
             c.state_floats = dims->d_inner * dims->d_state;
             c.i0 = i0; c.cnt = P - i0 < UPLOAD_RECS ? P - i0 : UPLOAD_RECS; c.P = P;
             for (int k = 0; k < c.cnt; k++) {
@@ -409,7 +411,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
                 run[3] += nc > 0 ? nc - 1 : 0;
                 for (int q = 0; q < 4; q++) c.pre[q][k] = run[q];
             }
-            hipLaunchKernelGGL(k_tables, dim3(1), dim3(256), 0, st, c);
+            hipLaunchKernelGGL(k_tables, dim3(d_flags ? 1 + c.cnt : 1), dim3(256), 0, st, c);
             SG_LAUNCH_CHECK("k_tables");
         }
     }
@@ -434,6 +436,7 @@ int build_plan(const SgDims* dims, const Sg2Weights* weights, int num_tensors, c
     pl.comp = reinterpret_cast<float*>(ws + L.off_comp);
     pl.sharp_nonzero = reinterpret_cast<int*>(ws + L.off_flags);
     pl.contracted = pl.sharp_nonzero + P;
+    pl.state_bad = pl.contracted + 3;
     pl.ctx = reinterpret_cast<float*>(ws + L.off_ctx);
     pl.decay = 1.0f - scalars->lr * scalars->wd_eff;
     pl.beta2 = scalars->beta2; pl.eps = scalars->eps; pl.rescale = scalars->rescale;
