@@ -301,7 +301,15 @@ int sg15_sharpness_restore(int num_tensors, const Sg15RestoreTensor* tensors, vo
  *   in_proj [32][8], dt_proj W [16][16], b [16], B_proj [16][16], C_proj
  *   [16][16], A_log [16][16], D [16], rope_freq [16][8], out_proj [8][16].
  * The adjoint is exact (no truncation window); sums over elements are formed in
- * a fixed order, so the result is reproducible run to run. */
+ * a fixed order, so the result is reproducible run to run.
+ *
+ * Scan blocks smaller than (d_model, d_state, d_inner) = (8, 16, 16) run
+ * embedded in that block (zero rows and columns, as in the step): ctx_out and
+ * d_ctx rows stay 8 floats wide (entries from d_model on are +0 / ignored),
+ * grads_out keeps the layout above with the block's gradients at the embedded
+ * positions (row r, column c of a smaller matrix at row r, column c of the
+ * listed one) and zeros elsewhere, and the two Mamba states keep the caller's
+ * own [d_inner][d_state] shape.  Larger blocks are refused. */
 #define SG2_SCAN_GRAD_FLOATS 3160
 size_t sg2_bilevel_workspace_bytes(const SgDims* dims, int num_tensors, const int64_t* numels);
 

@@ -1060,8 +1060,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const float* __restrict__ r_Co = s_C + (2 * p + 1) * LDS_STRIDE;
         int k0 = 0;
         if (dgiven) {
-            // a whole tile on the lane polynomials (the usual case): both columns in one instruction stream, the
-            // operands of block b + 1 requested before block b is computed
+            // a whole tile on the lane polynomials (the usual case): both columns in one instruction stream
             float Be[UB], Bo[UB], Ce[UB], Co[UB], dt[2][UB], xv[2][UB];
             auto fetch = [&](int kb, float (&tBe)[UB], float (&tBo)[UB], float (&tCe)[UB], float (&tCo)[UB], float (&tdt)[2][UB], float (&tux)[2][UB]) {
 #pragma unroll
@@ -1079,9 +1078,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                     }
                 }
             };
-#ifdef SG2_REPLAY_PREFETCH
-            float nBe[UB], nBo[UB], nCe[UB], nCo[UB], ndt[2][UB], nxv[2][UB];      // the other operand set: the two alternate
-#endif
             auto compute = [&](int kb, const float (&tBe)[UB], const float (&tBo)[UB], const float (&tCe)[UB], const float (&tCo)[UB],
                                const float (&tdt)[2][UB], const float (&tux)[2][UB]) {
                 float y[2][UB];
@@ -1093,22 +1089,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                     *reinterpret_cast<f32x4*>(&s_y[(jl + 8) * LDS_STRIDE + kb + 4 * (p >> 2)]) = f32x4{y[1][0], y[1][1], y[1][2], y[1][3]};
                 }
             };
-#ifdef SG2_REPLAY_PREFETCH
-            fetch(0, Be, Bo, Ce, Co, dt, xv);
-#pragma unroll 1
-            for (; k0 < SCAN_TT; k0 += 2 * UB) {
-                fetch(k0 + UB, nBe, nBo, nCe, nCo, ndt, nxv);
-                compute(k0, Be, Bo, Ce, Co, dt, xv);
-                if (k0 + 2 * UB < SCAN_TT) fetch(k0 + 2 * UB, Be, Bo, Ce, Co, dt, xv);
-                compute(k0 + UB, nBe, nBo, nCe, nCo, ndt, nxv);
-            }
-#else
 #pragma unroll 1
             for (; k0 < SCAN_TT; k0 += UB) {
                 fetch(k0, Be, Bo, Ce, Co, dt, xv);
                 compute(k0, Be, Bo, Ce, Co, dt, xv);
             }
-#endif
         }
         for (; k0 + UB <= cnt; k0 += UB) {
             float Be[UB], Bo[UB], Ce[UB], Co[UB];
@@ -1300,16 +1285,13 @@ int launch_scan_geo(const Plan& pl, hipStream_t st) {
         }
     }
     if (pl.htile != nullptr) return sg::fail("the bilevel pass is built for the default meta-net dimensions only");
-#ifndef SG2_TWO_WAVE_REPLAY
-    if constexpr (G::PARTS == 2) {
+    if constexpr (G::PARTS == 2) {          // one wave per chunk, two columns per lane
         hipLaunchKernelGGL(k_replay<G>, dim3(2 * pl.chunks), dim3(64), 0, st, pl);
         SG_LAUNCH_CHECK("k_replay");
-        prof_mark(4, st);
-        return 0;
+    } else {
+        hipLaunchKernelGGL((k_scan<G, true, false>), dim3(2 * pl.chunks), dim3(G::THREADS), 0, st, pl);
+        SG_LAUNCH_CHECK("k_scan<out>");
     }
-#endif
-    hipLaunchKernelGGL((k_scan<G, true, false>), dim3(2 * pl.chunks), dim3(G::THREADS), 0, st, pl);
-    SG_LAUNCH_CHECK("k_scan<out>");
     prof_mark(4, st);
     return 0;
 }

@@ -256,13 +256,15 @@ int elem_kind_of(const SgDims* d, int geo) {
 int check_dims(const SgDims* d, bool per_element) {
     const int geo = geo_of(d);
     if (geo < 0) return 1;
-    if (per_element && (d->gru_hidden != GH || d->num_heads != NH || d->pk_dim != PK || d->expert_hidden != EH || d->num_experts != NE))
-        return sg::fail("the per-element kernel of the bilevel pass is built for gru_hidden=%d num_heads=%d pk_dim=%d expert_hidden=%d "
-                        "num_experts=%d (got %d, %d, %d, %d, %d); experts narrower than %d run embedded in that width", GH, NH, PK, EH, NE,
-                        d->gru_hidden, d->num_heads, d->pk_dim, d->expert_hidden, d->num_experts, EH);
-    if (geo != GEO_DEFAULT || !scan_exact(d, geo))
-        return sg::fail("the bilevel pass is built for d_model=%d d_state=%d d_inner=%d only (got %d, %d, %d)", GeoDefault::DM, GeoDefault::DS,
-                        GeoDefault::DI, d->d_model, d->d_state, d->d_inner);
+    if (per_element && (d->gru_hidden != GH || d->num_heads != NH || d->pk_dim != PK || d->expert_hidden != EH || d->num_experts != NE ||
+                        d->d_model != GeoDefault::DM))
+        return sg::fail("the per-element kernel of the bilevel pass is built for d_model=%d gru_hidden=%d num_heads=%d pk_dim=%d expert_hidden=%d "
+                        "num_experts=%d (got %d, %d, %d, %d, %d, %d); smaller d_model, gru_hidden and expert_hidden run embedded in these "
+                        "(zero rows and columns)", GeoDefault::DM, GH, NH, PK, EH, NE, d->d_model, d->gru_hidden, d->num_heads, d->pk_dim,
+                        d->expert_hidden, d->num_experts);
+    if (geo != GEO_DEFAULT)
+        return sg::fail("the scan kernels of the bilevel pass are built for blocks up to d_model=%d d_state=%d d_inner=%d (got %d, %d, %d)",
+                        GeoDefault::DM, GeoDefault::DS, GeoDefault::DI, d->d_model, d->d_state, d->d_inner);
     return 0;
 }
 
@@ -621,6 +623,9 @@ int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int nu
         g_bilevel_records[workspace] = BilevelRecord{pl.total > 0 ? pl.chunk_len : 0, pl.total > 0 ? pl.window : 0, num_tensors, pl.total, ++g_bilevel_seq};
     }
     if (pl.total == 0) return 0;
+    if (extra && !scan_exact(dims, pl.geo))
+        return sg::fail("sg2_bilevel_forward_ex: the extra outputs are laid out for d_model=%d d_state=%d d_inner=%d only", GeoDefault::DM,
+                        GeoDefault::DS, GeoDefault::DI);
     if (ctx_out) pl.ctx = ctx_out;                 // else the contexts stay in the workspace
     if (extra) { pl.scan_out[0] = extra->scan_out_fwd; pl.scan_out[1] = extra->scan_out_bwd; }
     if (launch_sort(pl, extra ? extra->perm : nullptr, st)) return 1;
@@ -663,6 +668,9 @@ int sg2_bilevel_backward_ex(const SgDims* dims, const Sg2Weights* weights, int n
     if ((d_scan_out_fwd != nullptr) != (d_scan_out_bwd != nullptr)) return sg::fail("d_scan_out: both directions or neither");
     if (pl.total > 0 && ((d_ctx != nullptr) == (d_scan_out_fwd != nullptr))) return sg::fail("exactly one of d_ctx and d_scan_out must be given");
     if (dx_out != nullptr && row_dx == nullptr) return sg::fail("dx_out needs row_dx");
+    if ((d_scan_out_fwd != nullptr || row_dx != nullptr) && !scan_exact(dims, pl.geo))
+        return sg::fail("sg2_bilevel_backward_ex: d_scan_out / row_dx are laid out for d_model=%d d_state=%d d_inner=%d only", GeoDefault::DM,
+                        GeoDefault::DS, GeoDefault::DI);
     const float* const d_scan[2] = {d_scan_out_fwd, d_scan_out_bwd};
     return launch_bilevel_backward(pl, d_ctx, d_scan, row_dx, dx_out, grads_out, st);
 }

@@ -13,8 +13,9 @@ over the same kernels: the scan as one autograd Function (ScanContexts), the
 per-element part as another (SoftElements over sg2_bilevel_elem).  `forward`
 (hard top-1 routing, no gradients) is one call of sg2_meta_forward.  `per_element`
 restates the per-element part in torch ops: the tests check sg2_bilevel_elem
-against it, and it serves meta-nets whose GRU / routing / expert sizes the
-per-element bilevel kernel is not built for.
+against it, and it serves meta-nets whose routing sizes (heads, keys, experts)
+the per-element bilevel kernel is not built for.  Scan blocks up to the default
+(d_model 8, d_state 16, d_inner 16) run in HIP, smaller ones embedded.
 """
 import torch
 
@@ -130,10 +131,11 @@ class SoftElements(torch.autograd.Function):
 
 
 def elem_kernel_fits(mn):
-    """Whether sg2_bilevel_elem is built for this net's per-element sizes (experts narrower than its 16 run embedded)."""
+    """Whether sg2_bilevel_elem can run this net's per-element part: its routing sizes as built (4 heads, 12 x 12
+    keys, 144 experts); context width, GRU width and expert width up to its own (smaller ones run embedded)."""
     d = meta_dims(mn)
-    return ((d["d_model"], d["d_state"], d["d_inner"], d["gru_hidden"], d["num_heads"], d["pk_dim"], d["num_experts"]) == (8, 16, 16, 4, 4, 12, 144)
-            and d["expert_hidden"] <= _cabi.BILEVEL_EXPERT_WIDTH)
+    return ((d["num_heads"], d["pk_dim"], d["num_experts"]) == (4, 12, 144) and d["d_model"] <= _cabi.BILEVEL_SCAN_BLOCK[0]
+            and d["gru_hidden"] <= _cabi.BILEVEL_GRU_HIDDEN and d["expert_hidden"] <= _cabi.BILEVEL_EXPERT_WIDTH)
 
 
 def forward(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
@@ -191,11 +193,22 @@ def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bw
     .grad, for a list of tensors at once, all in HIP: scan forward (sg2_bilevel_forward), per-element forward and
     backward (sg2_bilevel_elem), scan adjoint (sg2_bilevel_backward).  Returns the smart gradients (flat, packed)."""
     plan = make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd)
-    ctx = plan.forward()
     g_all = torch.cat([g.reshape(-1).float() for g in grads])
     s_all = torch.cat([s.reshape(-1).float() for s in sharps])
     h_all = torch.cat([h.float() for h in gru_states])
     c_all = torch.cat([c.reshape(-1).float() for c in cotangents])
+    if not elem_kernel_fits(mn):
+        # routing sizes the per-element kernel is not built for: the scan and its adjoint in HIP, the per-element part
+        # and its derivative as torch operations on the GPU
+        with torch.enable_grad():
+            ctx = ScanContexts.apply(plan, *scan_parameters(mn))
+            smart, _ = per_element(mn, g_all, s_all, ctx[0], ctx[1], h_all)
+            params = [p for p in mn.parameters() if p.requires_grad]
+            for p, gr in zip(params, torch.autograd.grad((smart * c_all).sum(), params, allow_unused=True)):
+                if gr is not None:
+                    p.grad = gr if p.grad is None else p.grad + gr
+        return smart.detach()
+    ctx = plan.forward()
     smart, d_ctx, blk = _cabi.bilevel_elem(plan.weights, g_all, s_all, ctx, h_all, c_all, float(mn.rescale), meta_dims(mn))
     _add_grads(elem_parameters(mn), blk)
     _add_grads(scan_parameters(mn), plan.backward(d_ctx))

@@ -242,53 +242,127 @@ class Sg2Bilevel:
         self.device = dev
 
     def forward(self):
-        ctx = torch.empty(2, self.total, self.dims.d_model, dtype=torch.float32, device=self.device)
+        ctx = torch.empty(2, self.total, BILEVEL_SCAN_BLOCK[0], dtype=torch.float32, device=self.device)
         rc = lib().sg2_bilevel_forward(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, ctx.data_ptr(),
                                        self.workspace.data_ptr(), self.workspace.numel(), torch.cuda.current_stream().cuda_stream)
         if rc != 0:
             raise RuntimeError("sg2_bilevel_forward: " + last_error())
-        return ctx
+        # a smaller scan block runs embedded: its context entries are the first d_model of the kernel's rows
+        return ctx if self.dims.d_model == BILEVEL_SCAN_BLOCK[0] else ctx[..., :self.dims.d_model]
 
     def backward(self, d_ctx):
-        d_ctx = d_ctx.detach().float().contiguous()
+        d_ctx = d_ctx.detach().float()
         assert d_ctx.shape == (2, self.total, self.dims.d_model) and d_ctx.is_cuda
+        d_ctx = _widen_last(d_ctx, BILEVEL_SCAN_BLOCK[0])
         out = torch.empty(SG2_SCAN_GRAD_FLOATS, dtype=torch.float32, device=self.device)
         rc = lib().sg2_bilevel_backward(C.byref(self.dims), C.byref(self.W), self.P, self.tensors, d_ctx.data_ptr(), out.data_ptr(),
                                         self.workspace.data_ptr(), self.workspace.numel(), torch.cuda.current_stream().cuda_stream)
         if rc != 0:
             raise RuntimeError("sg2_bilevel_backward: " + last_error())
-        return out
+        return extract_scan_grads(out, self.dims)
+
+
+BILEVEL_SCAN_BLOCK = (8, 16, 16)   # (d_model, d_state, d_inner) the scan kernels of the bilevel pass are built for
+
+
+def _widen_last(t, width):
+    """`t` with its last dimension zero-padded to `width`, contiguous."""
+    if t.shape[-1] == width:
+        return t.contiguous()
+    wide = torch.zeros(*t.shape[:-1], width, dtype=t.dtype, device=t.device)
+    wide[..., :t.shape[-1]] = t
+    return wide
+
+
+def extract_scan_grads(flat, dims):
+    """The gradients of a scan block smaller than BILEVEL_SCAN_BLOCK out of sg2_bilevel_backward's block, which keeps
+    the kernel block's layout (include/sg_abi.h): flat again, in the caller's own shapes and the same order."""
+    DM, DS, DI = BILEVEL_SCAN_BLOCK
+    dm, ds, di = dims.d_model, dims.d_state, dims.d_inner
+    if (dm, ds, di) == (DM, DS, DI):
+        return flat
+    parts, o = [], 0
+
+    def take(*shape):
+        nonlocal o
+        n = 1
+        for k in shape:
+            n *= k
+        v = flat[o:o + n].view(*shape)
+        o += n
+        return v
+    parts += [take(DM, 2)[:dm], take(DM)[:dm]]
+    for _ in range(2):
+        parts += [take(2, DI, DM)[:, :di, :dm],          # in_proj: x rows, then z rows
+                  take(DI, DI)[:di, :di], take(DI)[:di], take(DS, DI)[:ds, :di], take(DS, DI)[:ds, :di],
+                  take(DI, DS)[:di, :ds], take(DI)[:di], take(DI, DS // 2)[:di, :ds // 2], take(DM, DI)[:dm, :di]]
+    assert o == flat.numel()
+    return torch.cat([v.reshape(-1) for v in parts])
 
 
 SG2_ELEM_GRAD_FLOATS = 8420
 
 
 BILEVEL_EXPERT_WIDTH = 16      # expert width sg2_bilevel_elem is compiled for
+BILEVEL_GRU_HIDDEN = 4         # its GRU width (d_model: BILEVEL_SCAN_BLOCK[0])
+
+
+def _elem_maps(dm, gh, dev):
+    """Where the entries of a smaller per-element net sit in the kernel's: columns of a GRU matrix
+    ([g, s, ctx_f, ctx_b, h]), columns of a query matrix ([h', ctx_f, ctx_b, g, s]) and its rows (two halves of
+    d_model/2 entries)."""
+    DM, GH = BILEVEL_SCAN_BLOCK[0], BILEVEL_GRU_HIDDEN
+    ix = lambda v: torch.tensor(v, dtype=torch.long, device=dev)
+    gru_cols = ix([0, 1] + [2 + c for c in range(dm)] + [2 + DM + c for c in range(dm)] + [2 + 2 * DM + k for k in range(gh)])
+    q_cols = ix(list(range(gh)) + [GH + c for c in range(dm)] + [GH + DM + c for c in range(dm)] + [GH + 2 * DM, GH + 2 * DM + 1])
+    q_rows = ix(list(range(dm // 2)) + [DM // 2 + r for r in range(dm // 2)])
+    return gru_cols, q_cols, q_rows
 
 
 def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, dims=None, want_smart=True, want_gru=False):
     """sg2_bilevel_elem on flat fp32 GPU arrays: returns (smart [total] or None, d_ctx [2, total, d_model],
-    weight-gradient block [SG2_ELEM_GRAD_FLOATS]); with want_gru a fourth value, the new GRU state [total, gru_hidden]."""
+    weight-gradient block, flat in the order of include/sg_abi.h at the caller's own sizes); with want_gru a fourth
+    value, the new GRU state [total, gru_hidden].
+
+    The kernel is built for d_model 8, gru_hidden 4 and experts of width 16.  A net that is smaller in any of these
+    runs embedded: the extra context entries, hidden units and expert units have zero weights (an extra hidden unit
+    starts at 0 and stays there: its candidate is tanh(0); an extra expert unit is relu(0)), every chain of products
+    only gains zero terms, so the real entries keep their bits, and the extra entries of the gradient block (all
+    zero) are dropped.  (The reference's training harness builds experts of width 4.)"""
     d = make_dims(dims)
+    DM, GH, EH = BILEVEL_SCAN_BLOCK[0], BILEVEL_GRU_HIDDEN, BILEVEL_EXPERT_WIDTH
+    dm, gh, eh, E, NH, PK = d.d_model, d.gru_hidden, d.expert_hidden, d.num_experts, d.num_heads, d.pk_dim
     ws_ = [w.detach().float().contiguous() for w in weights]
-    # The kernel is built for experts of width 16.  Narrower experts (the reference's training harness uses 4) run as
-    # 16-wide ones whose extra units have W1 = b1 = W2 = 0: relu(0) = 0 adds nothing to any output, every real entry
-    # keeps its bits, and the extra units' gradient entries (all zero) are dropped from the block below.
-    eh, E = d.expert_hidden, d.num_experts
-    if eh < BILEVEL_EXPERT_WIDTH:
-        for k in (29, 30, 31):
-            wide = torch.zeros(E, BILEVEL_EXPERT_WIDTH, dtype=torch.float32, device=ws_[k].device)
-            wide[:, :eh] = ws_[k].reshape(E, eh)
+    dev = ws_[20].device
+    embedded = dm < DM or gh < GH or eh < EH
+    if embedded:
+        if dm % 2 or dm < 2 or gh < 1 or eh < 1:
+            raise RuntimeError("sg2_bilevel_elem: d_model must be even and every size positive")
+        gru_cols, q_cols, q_rows = _elem_maps(dm, gh, dev)
+        zeros = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device=dev)
+        for k in (20, 22, 24):                                  # W_z, W_r, W_h [gh][2 + 2 dm + gh]
+            wide = zeros(GH, 2 + 2 * DM + GH)
+            wide[:gh, gru_cols] = ws_[k].reshape(gh, -1)
             ws_[k] = wide
-        d.expert_hidden = BILEVEL_EXPERT_WIDTH
+        for k in (21, 23, 25):                                  # their biases
+            ws_[k] = _widen_last(ws_[k].reshape(-1), GH)
+        q = zeros(NH, DM, GH + 2 * DM + 2)                      # queries [heads][d_model][gh + 2 dm + 2]
+        q[:, q_rows[:, None], q_cols[None, :]] = ws_[26].reshape(NH, dm, -1)
+        ws_[26] = q
+        for k in (27, 28):                                      # product keys [heads][pk][d_model / 2]
+            ws_[k] = _widen_last(ws_[k].reshape(NH, PK, dm // 2), DM // 2)
+        for k in (29, 30, 31):                                  # expert W1, b1, W2 [E][eh]
+            ws_[k] = _widen_last(ws_[k].reshape(E, eh), EH)
+        d.d_model, d.gru_hidden, d.expert_hidden = DM, GH, EH
     W = Sg2Weights()
     for k, w in enumerate(ws_):
         W.w[k] = w.data_ptr()
     arrs = [t.detach().float().contiguous() for t in (grad, sharpness, ctx, gru_state, cotangent)]
     total = arrs[0].numel()
-    dev = arrs[0].device
-    assert all(t.is_cuda for t in arrs) and arrs[2].shape == (2, total, d.d_model) and arrs[3].shape == (total, d.gru_hidden)
+    assert all(t.is_cuda for t in arrs) and arrs[2].shape == (2, total, dm) and arrs[3].shape == (total, gh)
     assert arrs[1].numel() == total and arrs[4].numel() == total
+    arrs[2] = _widen_last(arrs[2], DM)
+    arrs[3] = _widen_last(arrs[3], GH)
     smart = torch.empty(total, dtype=torch.float32, device=dev) if want_smart else None
     d_ctx = torch.empty_like(arrs[2])
     out = torch.empty(SG2_ELEM_GRAD_FLOATS, dtype=torch.float32, device=dev)
@@ -300,10 +374,26 @@ def bilevel_elem(weights, grad, sharpness, ctx, gru_state, cotangent, rescale, d
                                    out.data_ptr(), work.data_ptr(), work.numel(), torch.cuda.current_stream().cuda_stream)
     if rc != 0:
         raise RuntimeError("sg2_bilevel_elem: " + last_error())
-    if eh < BILEVEL_EXPERT_WIDTH:       # expert part of the block: W1, b1, W2 [E, 16] each, then b2 [E]
-        head = out.numel() - (3 * BILEVEL_EXPERT_WIDTH + 1) * E
-        ex = out[head:head + 3 * BILEVEL_EXPERT_WIDTH * E].view(3, E, BILEVEL_EXPERT_WIDTH)[:, :, :eh].reshape(-1)
-        out = torch.cat([out[:head], ex, out[-E:]])
+    if embedded:
+        parts, o = [], 0
+
+        def take(*shape):
+            nonlocal o
+            n = 1
+            for k in shape:
+                n *= k
+            v = out[o:o + n].view(*shape)
+            o += n
+            return v
+        for _ in range(3):                                      # (W, b) of the three gates
+            parts += [take(GH, 2 + 2 * DM + GH)[:gh][:, gru_cols], take(GH)[:gh]]
+        parts.append(take(NH, DM, GH + 2 * DM + 2)[:, q_rows[:, None], q_cols[None, :]])
+        parts += [take(NH, PK, DM // 2)[..., :dm // 2], take(NH, PK, DM // 2)[..., :dm // 2]]
+        parts += [take(E, EH)[:, :eh], take(E, EH)[:, :eh], take(E, EH)[:, :eh], take(E)]
+        assert o == out.numel()
+        out = torch.cat([v.reshape(-1) for v in parts])
+        d_ctx = d_ctx[..., :dm]
+        gru_out = gru_out[:, :gh].contiguous() if want_gru else None
     if want_gru:
         return smart, d_ctx, out, gru_out
     return smart, d_ctx, out

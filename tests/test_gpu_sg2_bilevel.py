@@ -220,22 +220,33 @@ def test_differentiable_forward_of_the_whole_meta_net():
     assert max(w.values()) <= 1.0, w
 
 
-def test_all_hip_accumulation_with_experts_of_width_4():
-    """The bilevel accumulation with expert_hidden = 4, the width the reference's training harness constructs the
-    optimizer with (grokking_race_v2.py:1583 -> :775): the per-element kernel runs the narrow experts embedded in its
-    own width.  Smart gradients and the gradients of every parameter against float64 autograd."""
+@pytest.mark.parametrize("kw", [dict(expert_hidden=4), dict(d_model=4, d_state=8, gru_hidden=2, expert_hidden=6),
+                                dict(d_model=6, d_state=10, gru_hidden=3, num_peer_heads=2, num_experts=25)],
+                         ids=["experts_of_width_4", "smaller_net_embedded", "other_routing_sizes"])
+def test_accumulation_at_other_meta_net_sizes(kw):
+    """The bilevel accumulation at sizes other than the defaults, smart gradients and the gradients of every
+    parameter against float64 autograd:
+    * expert_hidden = 4, the width the reference's training harness constructs the optimizer with
+      (grokking_race_v2.py:1583 -> :775): the per-element kernel runs the narrow experts embedded in its own width;
+    * a smaller scan block, GRU and expert width: scan kernels and per-element kernel both run the net embedded;
+    * other routing sizes (heads, keys, experts): the scan and its adjoint in HIP (embedded block), the per-element
+      part as torch operations.
+    Then one tensor through the module's forward_for_bilevel (the autograd form over the same kernels)."""
     import copy
     from grokking_optimizers import _bilevel
     dev = torch.device("cuda:0")
-    mn = _meta_net(8, dev, expert_hidden=4)
-    assert mn.expert_W1.shape[1] == 4
+    mn = _meta_net(8, dev, **kw)
+    assert mn.expert_W1.shape[1] == kw.get("expert_hidden", 16)
     mn64 = copy.deepcopy(mn).double().cpu()
+    gh, di, ds = mn.gru_hidden, mn.mamba_fwd.d_inner, mn.d_state
     gen = torch.Generator().manual_seed(23)
     data = []
     for n in (200, 77, 1300):
         data.append(dict(g=torch.randn(n, generator=gen) * 0.5, s=torch.rand(n, generator=gen) * 0.3,
-                         h=torch.randn(n, 4, generator=gen) * 0.5, hf=torch.randn(16, 16, generator=gen) * 0.3,
-                         hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
+                         h=torch.randn(n, gh, generator=gen) * 0.5, hf=torch.randn(di, ds, generator=gen) * 0.3,
+                         hb=torch.randn(di, ds, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
+    print("bilevel accumulation", kw, "per-element kernel:", _bilevel.elem_kernel_fits(mn), flush=True)
+    assert _bilevel.elem_kernel_fits(mn) == ("num_experts" not in kw)
     mn64.zero_grad()
     ref_smart = []
     for d in data:
@@ -253,7 +264,23 @@ def test_all_hip_accumulation_with_experts_of_width_4():
     for n, p in mn.named_parameters():
         assert p.grad is not None and p.grad.shape == p.shape, n
     w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_named, 2e-4)
-    print("expert width 4, worst gradient ratios", w, flush=True)
+    print(kw, "worst gradient ratios", w, flush=True)
+    assert max(w.values()) <= 1.0, w
+
+    d = data[0]
+    mn.zero_grad()
+    mn64.zero_grad()
+    smart, hn, nf, nb = mn.forward_for_bilevel(d["g"].to(dev), d["s"].to(dev), d["h"].to(dev), d["hf"].to(dev), d["hb"].to(dev))
+    (smart * d["R"].to(dev)).sum().backward()
+    rs, rh, rf, rb = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
+    (rs * d["R"].double()).sum().backward()
+    for name, got, ref in (("smart", smart, rs), ("gru", hn, rh), ("mamba_fwd", nf, rf), ("mamba_bwd", nb, rb)):
+        got, ref = got.detach().double().cpu(), ref.detach()
+        assert got.shape == ref.shape, (name, got.shape, ref.shape)
+        err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
+        assert bool((err <= tol).all()), (name, float((err / tol).max()))
+    w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], [(n, p.grad.clone()) for n, p in mn64.named_parameters()], 2e-4)
+    print(kw, "forward_for_bilevel, worst gradient ratios", w, flush=True)
     assert max(w.values()) <= 1.0, w
 
 
