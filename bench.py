@@ -524,8 +524,31 @@ def secondary_configs(dev, steps=20, warmup=3):
         "workload": "SuperGrok v2 full step, 14 tensors, %d elements" % total, "ms_per_step": 1e3 * el / steps, "value": total * steps / el,
         "unit": "elements/s", "dtype": "f32", "steps": steps, "stage_ms": stage,
         "roofline": {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s", "achieved": BYTES_PER_ELEMENT * total * steps / el / 1e9,
-                     "frac": BYTES_PER_ELEMENT * total * steps / el / 1e9 / HBM_PEAK_GBS, "bytes_per_element": BYTES_PER_ELEMENT}}
+                     "frac": BYTES_PER_ELEMENT * total * steps / el / 1e9 / HBM_PEAK_GBS, "bytes_per_element": BYTES_PER_ELEMENT},
+        "graph_replay_ms_per_step": graph_replay_ms(st, weights, D, grad_sets, sharps, steps)}
     return out
+
+
+def graph_replay_ms(st, weights, D, grad_sets, sharps, steps):
+    """The same step recorded once into a HIP graph (the call copies nothing from the host and blocks nowhere) and
+    replayed: what the ~30 launches of a step cost when the host does not issue them one by one.  A replay repeats
+    the recorded scalars; the state keeps evolving."""
+    import torch
+    from workloads import per_tensor_scalars, shared_scalars
+    step = make_v2_step(st, weights, D, boundary="cabi")
+    P = len(st["params"])
+    step(grad_sets[0], sharps, per_tensor_scalars(P, 1), shared_scalars())       # eager first
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(grad_sets[1], sharps, per_tensor_scalars(P, 2), shared_scalars())
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    return 1e3 * (time.perf_counter() - t0) / steps
 
 
 def aten_loop_baseline(max_elems=16384, budget_s=10.0):
