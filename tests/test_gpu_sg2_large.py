@@ -116,5 +116,5 @@ def test_bilevel_pass_refuses_the_large_geometry():
     from grokking_optimizers import _cabi
     g = [torch.zeros(100, device="cuda")]
     st = [torch.zeros(32, 32, device="cuda")]
-    with pytest.raises(RuntimeError, match="bilevel pass is built for"):
+    with pytest.raises(RuntimeError, match="bilevel pass are built for blocks up to"):
         _cabi.Sg2Bilevel([w.cuda() for w in wl.meta_weights(7, LARGE)], g, g, st, st, dims=LARGE)
