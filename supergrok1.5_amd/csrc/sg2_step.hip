@@ -497,9 +497,13 @@ int run_step(const SgDims* dims, const Sg2Weights* weights, int num_tensors, con
     if (launch_sort(pl, debug ? debug->perm : nullptr, st)) return 1;
     prof_mark(1, st);
     if (launch_scan(pl, st)) return 1;
-    if (debug && debug->ctx)      // [2][total][d_model] for the caller; the kernels' rows are d_model of the kernel geometry wide
-        SG_HIP_CHECK(hipMemcpy2DAsync(debug->ctx, 4 * (size_t)dims->d_model, pl.ctx, 4 * (size_t)geo_info(pl.geo).dm, 4 * (size_t)dims->d_model,
-                                      2 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
+    if (debug && debug->ctx) {    // [2][total][d_model] for the caller; the kernels' rows are d_model of the kernel geometry wide
+        if (dims->d_model == geo_info(pl.geo).dm)
+            SG_HIP_CHECK(hipMemcpyAsync(debug->ctx, pl.ctx, 4 * 2 * (size_t)L.total * dims->d_model, hipMemcpyDeviceToDevice, st));
+        else
+            SG_HIP_CHECK(hipMemcpy2DAsync(debug->ctx, 4 * (size_t)dims->d_model, pl.ctx, 4 * (size_t)geo_info(pl.geo).dm,
+                                          4 * (size_t)dims->d_model, 2 * (size_t)L.total, hipMemcpyDeviceToDevice, st));
+    }
     if (launch_elem(pl, expert_counts, debug ? debug->expert_idx : nullptr, st)) return 1;
     prof_mark(5, st);
     if (g_prof.on && g_prof.calls < SG2_PROF_MAX_CALLS) g_prof.calls++;

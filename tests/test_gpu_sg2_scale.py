@@ -150,3 +150,71 @@ def test_bilevel_pass_at_scale_linearity_and_chunking():
     for n in g1:
         scale = float(g1[n].abs().max())
         assert float((g1c[n].double() - g1[n].double()).abs().max()) <= 2e-4 * scale, (n, scale)
+
+
+def test_one_tensor_beyond_32_bit_byte_offsets():
+    """One tensor of 2^27 + 12345 elements (32 769 chunks of 4096 steps per direction, 16 386 sort tiles, context and
+    GRU arrays past 4 GiB, so every byte offset that could wrap a 32-bit integer is exercised), with a quarter of the
+    gradients quantised so that the sort meets long runs of equal keys.  Checked through what needs no CPU answer:
+    the permutation is a stable sort of |g|, expert_counts adds up, every state stays finite, a second run with a
+    different chunk length (another decomposition of the same scan) agrees within the step's tolerance, and a repeat
+    of the first run agrees bit for bit."""
+    from grokking_optimizers import _cabi
+    dev = "cuda"
+    n = (1 << 27) + 12345
+    gh, di, ds = DIMS["gru_hidden"], DIMS["d_inner"], DIMS["d_state"]
+    gen = torch.Generator(device=dev).manual_seed(5)
+    g = torch.randn(n, device=dev, generator=gen) * 1e-3
+    g[::4] = torch.round(g[::4] * 4096.0) / 4096.0            # multiples of 2^-12: mostly 0 and +-2.4e-4, huge tie groups
+    p0 = torch.randn(n, device=dev, generator=gen) * 0.02
+    W = [w.to(dev) for w in wl.meta_weights(7)]
+    lib = _cabi.lib()
+
+    def run(chunk_len, debug):
+        z = lambda *s: torch.zeros(*s, device=dev)
+        st = dict(p=[p0.clone()], ea=[z(n)], easq=[z(n)], mu=[z(n)], gru=[z(n, gh)], mf=[z(di, ds)], mb=[z(di, ds)])
+        counts = torch.zeros(144, dtype=torch.int32, device=dev)
+        step = _cabi.Sg2Step(W, st["p"], st["ea"], st["easq"], st["mu"], st["gru"], st["mf"], st["mb"], counts, debug=debug,
+                             chunk_len=chunk_len)
+        print("2^27 elements: chunk_len", chunk_len, flush=True)
+        step([g], [torch.zeros_like(g)], per_tensor_scalars(1, 1), shared_scalars())
+        torch.cuda.synchronize()
+        return st, counts, step
+
+    assert _cabi.chunk_len_for([n]) == 4096
+    st, counts, step = run(None, True)
+    assert int(counts.sum()) == 4 * n
+    perm = step.perm[:n].long()
+    seen = torch.zeros(n, dtype=torch.bool, device=dev)
+    seen[perm] = True
+    assert bool(seen.all())
+    keys = g.abs()[perm]
+    assert bool((keys[1:] >= keys[:-1]).all())
+    ties = keys[1:] == keys[:-1]
+    assert int(ties.sum()) > n // 8
+    assert bool((perm[1:][ties] > perm[:-1][ties]).all())
+    assert int(step.expert_idx.min()) >= 0 and int(step.expert_idx.max()) < 144
+    del perm, seen, keys, ties, step
+    for name, lst in st.items():
+        assert bool(torch.isfinite(lst[0]).all()), name
+    assert float((st["p"][0] - p0).abs().max()) > 0.0
+    torch.cuda.empty_cache()
+
+    other, counts_b, _ = run(1024, False)
+    worst = 0.0
+    for name in ("p", "ea", "easq", "mu", "gru", "mf", "mb"):
+        a, b = st[name][0], other[name][0]
+        floor = 1e-5 * float(a.abs().max()) + 1e-30
+        ratio = float(((a - b).abs() / (1e-4 * torch.maximum(a.abs(), b.abs()) + floor)).max())
+        worst = max(worst, ratio)
+        assert ratio <= 1.0, (name, ratio)
+    flips = int((counts - counts_b).abs().sum()) // 2
+    print("chunk 4096 against 1024: worst tolerance ratio", worst, "routing decisions that differ:", flips, flush=True)
+    assert flips <= n // 100000
+    del other
+    torch.cuda.empty_cache()
+
+    again, counts_c, _ = run(None, False)
+    for name in st:
+        assert torch.equal(st[name][0], again[name][0]), name
+    assert torch.equal(counts, counts_c)
