@@ -179,6 +179,25 @@ def test_saturated_gates_take_the_plain_forms():
     assert all(v == 0.0 for v in w.values()), w        # identical arithmetic on both sides: not one bit differs
 
 
+def test_routing_spread_over_most_experts():
+    """The query rows that read the GRU state amplified 30 times, on random GRU states (what the benchmark's
+    spread-routing variant times): the lanes of a wave pick different experts, so the expert records are gathered per
+    lane instead of broadcast.  Indices and counts bit for bit against the checker, with most of the 144 experts in
+    use."""
+    W = wl.meta_weights(7)
+    W[26][:, :, :4] *= 30.0
+    case = Sg2Case([(20000,), (64, 130), (3, 4096), (257,)], seed=31, weights=W, random_state=True)
+    for st_cpu, st_gpu, st_np in zip(case.cpu, case.gpu, case.np):       # GRU states of unit scale
+        st_cpu["gru"].mul_(1.0 / 0.3)
+        st_gpu["gru"].mul_(1.0 / 0.3)
+        st_np["gru"] *= np.float32(1.0 / 0.3)
+        assert np.array_equal(st_np["gru"], st_gpu["gru"].cpu().numpy())
+    w = _run_steps(case, 2, chunk_len=None, sharp=True, lamb_eff=2.0)
+    used = int((case.counts_gpu > 0).sum())
+    print("spread routing: experts in use", used, "worst tolerance ratios", w, flush=True)
+    assert used >= 100
+
+
 def test_shared14_one_step_default_chunk():
     """The 14-tensor, 420 195-element transformer parameter set, default chunk length."""
     case = Sg2Case(wl.shared14_shapes(), seed=0)
