@@ -95,3 +95,24 @@ def test_flip_rate_on_the_14_tensor_set():
     print("14-tensor set (420 195 elements, chunk 1024, window 64, populated sharpness): %d of %d routing decisions differ "
           "between fp32 and float64 (rate %.3g)" % (flips, total, flips / total), flush=True)
     assert flips <= 1e-3 * total
+
+
+def test_flip_rate_with_routing_spread_over_most_experts():
+    """The same comparison where routing decisions are close calls far more often: query rows that read the GRU state
+    amplified 30 times on GRU states of unit scale, so that the elements spread over most of the 144 experts and many
+    score pairs are near ties.  Every difference between the fp32 and the float64 routing must still sit at a
+    float64 margin below 1e-5; the rate is printed."""
+    n = 1 << 18
+    g = wl.make_grads([(n,)], seed=9, tail_frac=0.005, tail="student3")[0].reshape(-1).numpy()
+    s = np.abs(wl.make_grads([(n,)], seed=509)[0].reshape(-1).numpy()) * 0.5
+    W = weights_np()
+    W[26] = W[26].copy()
+    W[26][:, :, :4] *= 30.0
+    st = random_state_np(n, 78)
+    st["gru"] = (st["gru"] * np.float32(1.0 / 0.3)).astype(np.float32)
+    sc = f32_scalars(default_scalars(i=1, step=3, lamb_eff=2.0))
+    (a, da), (b, db) = _both_policies(W, st, g, s, sc, 1024, 64)
+    used = len(np.unique(db["expert_idx"]))
+    print("spread routing: %d experts in use" % used, flush=True)
+    assert used >= 100
+    _check(a, da, b, db, "262 144 elements, routing spread over %d experts" % used)
