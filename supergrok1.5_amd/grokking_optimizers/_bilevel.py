@@ -151,7 +151,8 @@ def forward(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_stat
     shape = (mn.mamba_fwd.d_inner, mn.d_state)
     state = lambda m: torch.zeros(*shape, dtype=torch.float32, device=dev) if m is None else m.detach().float().contiguous().clone()
     mf, mb = state(mamba_fwd_state), state(mamba_bwd_state)
-    smart, h_new = _cabi.meta_forward(mn.flat_weights(), [g], [s], [gru_state], [mf], [mb], float(mn.rescale), meta_dims(mn))
+    smart, h_new = _cabi.meta_forward(mn.flat_weights(), [g], [s], [gru_state], [mf], [mb], float(mn.rescale), meta_dims(mn),
+                                      expert_counts=mn.expert_counts if mn.training else None)
     return smart.reshape(grad.shape).to(grad.dtype), h_new, mf, mb
 
 

@@ -14,11 +14,14 @@ that use the module outside the optimizer and run on the same kernels:
 (sg2_meta_forward: sort, scan, GRU, routing, experts), `forward_for_bilevel`
 is differentiable through two autograd Functions over the bilevel kernels (scan
 forward / adjoint, per-element forward / backward).  GPU tensors only.
+The sub-modules' own forwards (Mamba3ScanBlock on an arbitrary sequence,
+MiniGRU) are plain torch operations for callers that use them on their own.
 """
 import math
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 
 class Mamba3ScanBlock(nn.Module):
@@ -41,6 +44,33 @@ class Mamba3ScanBlock(nn.Module):
         return [f(self.in_proj.weight), f(self.dt_proj.weight), f(self.dt_proj.bias), f(self.B_proj.weight),
                 f(self.C_proj.weight), f(self.A_log), f(self.D), f(self.rope_freq), f(self.out_proj.weight)]
 
+    def forward(self, x, initial_state=None):
+        """One scan block on an arbitrary input sequence x [N, d_model] (reference: mamba3_peer_metanet.py:90-160):
+        returns (output [N, d_model], final state [d_inner, d_state]).  A utility for callers that use the block on
+        its own, in torch operations on x's device and differentiable; the optimizer never comes here (its scan runs
+        in the fused kernels, where the input is the two-number feature (g, s) of an element).  Every coefficient of
+        the recurrence is formed for all steps at once; only the 2 x 2 state update itself walks the sequence, so
+        this is meant for sequences of thousands of steps, not millions."""
+        xb, z = self.in_proj(x).chunk(2, dim=-1)
+        dt = F.softplus(self.dt_proj(xb)).unsqueeze(-1)                       # [N, di, 1]
+        half = 0.5 * dt * -torch.exp(self.A_log)                               # dt A / 2
+        a_bar = (1.0 + half) / (1.0 - half + 1e-8)                             # [N, di, ds]
+        drive = dt * self.B_proj(xb).unsqueeze(1) * xb.unsqueeze(-1)           # dt B x
+        ang = dt * self.rope_freq                                              # [N, di, ds/2]
+        cs, sn = torch.cos(ang), torch.sin(ang)
+        h = (torch.zeros(self.d_inner, self.d_state, device=x.device, dtype=x.dtype) if initial_state is None
+             else initial_state.to(x.dtype))
+        states = []
+        for i in range(x.shape[0]):
+            he, ho = h[:, 0::2], h[:, 1::2]
+            rot = torch.stack([he * cs[i] - ho * sn[i], ho * cs[i] + he * sn[i]], dim=-1).reshape(self.d_inner, self.d_state)
+            h = a_bar[i] * rot + drive[i]
+            states.append(h)
+        if not states:
+            return x.new_zeros(0, self.d_model), h
+        y = (torch.stack(states) * self.C_proj(xb).unsqueeze(1)).sum(-1)
+        return self.out_proj(y * F.silu(z) + self.D * xb), h
+
 
 class MiniGRU(nn.Module):
     def __init__(self, input_dim: int, hidden_dim: int = 4):
@@ -49,6 +79,15 @@ class MiniGRU(nn.Module):
         self.W_z = nn.Linear(input_dim + hidden_dim, hidden_dim)
         self.W_r = nn.Linear(input_dim + hidden_dim, hidden_dim)
         self.W_h = nn.Linear(input_dim + hidden_dim, hidden_dim)
+
+    def forward(self, x, h):
+        """New hidden state [N, hidden] from inputs x [N, input_dim] and state h (reference:
+        mamba3_peer_metanet.py:178-192): update gate z, reset gate r, candidate from [x, r * h].  Torch operations,
+        for callers that use the cell on its own; the fused step evaluates the same cell per element in HIP."""
+        both = torch.cat([x, h], dim=-1)
+        z, r = torch.sigmoid(self.W_z(both)), torch.sigmoid(self.W_r(both))
+        cand = torch.tanh(self.W_h(torch.cat([x, r * h], dim=-1)))
+        return (1 - z) * h + z * cand
 
 
 class Mamba3PEERMetaNet(nn.Module):
@@ -99,8 +138,8 @@ class Mamba3PEERMetaNet(nn.Module):
         return w
 
     def forward(self, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
-        """(smart_grad, new_gru_state, new_mamba_fwd_state, new_mamba_bwd_state) with the step's hard top-1 routing.
-        Unlike the reference it does not update expert_counts: only the fused step does."""
+        """(smart_grad, new_gru_state, new_mamba_fwd_state, new_mamba_bwd_state) with the step's hard top-1 routing;
+        in training mode the winners are added to expert_counts, as in the reference (:342-348 there)."""
         from grokking_optimizers import _bilevel
         return _bilevel.forward(self, grad, sharpness, gru_state, mamba_fwd_state, mamba_bwd_state)
 
@@ -109,6 +148,17 @@ class Mamba3PEERMetaNet(nn.Module):
         every parameter of the module; GPU tensors only."""
         from grokking_optimizers import _bilevel
         return _bilevel.forward_for_bilevel(self, grad, sharpness, gru_state, mamba_fwd_state, mamba_bwd_state)
+
+    @property
+    def has_cuda_bilevel(self):
+        """Whether the device kernels of the bilevel pass can serve this module (reference: :493-496): they are part
+        of the library, so whenever the parameters live on the GPU."""
+        return next(self.parameters()).is_cuda
+
+    def forward_for_bilevel_cuda(self, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
+        """The reference's name for the bilevel forward with device kernels behind it (:498-513 there):
+        forward_for_bilevel already is that."""
+        return self.forward_for_bilevel(grad, sharpness, gru_state, mamba_fwd_state, mamba_bwd_state)
 
     def flat_weights(self):
         """The 33 tensors in the argument order of _ops.supergrok2_mamba_peer_batched_step."""

@@ -357,8 +357,16 @@ def test_module_forward_matches_the_float64_step(kw):
     hf, hb = torch.randn(di, ds, generator=gen) * 0.3, torch.randn(di, ds, generator=gen) * 0.3
     print("module forward, N", n, kw, flush=True)
     hf_dev, hb_dev, h_dev = hf.to(dev), hb.to(dev), h.to(dev)
+    assert mn.training and int(mn.expert_counts.sum()) == 0
     smart, hn, nf, nb = mn(g.to(dev), s.to(dev), h_dev, hf_dev, hb_dev)
     assert torch.equal(hf_dev.cpu(), hf) and torch.equal(hb_dev.cpu(), hb) and torch.equal(h_dev.cpu(), h)
+    # a module in training mode counts the winners (one per head and element), one in eval mode does not
+    assert int(mn.expert_counts.sum()) == n * mn.num_peer_heads
+    mn.eval()
+    again = mn(g.to(dev), s.to(dev), h_dev, hf_dev, hb_dev)
+    assert int(mn.expert_counts.sum()) == n * mn.num_peer_heads and torch.equal(again[0], smart)
+    mn.train()
+    assert mn.has_cuda_bilevel
     dims = dict(d_model=mn.d_model, gru_hidden=gh, num_heads=mn.num_peer_heads, pk_dim=mn.pk_dim)
     sc = dict(rescale=mn.rescale, alpha=0.0, lamb_eff=0.0, beta1=0.9, beta2=0.999, bc1=1.0, bc2=1.0, eps=1e-8, lr=0.0, wd_eff=0.0)
     z = torch.zeros(n)

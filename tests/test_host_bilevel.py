@@ -52,3 +52,45 @@ def test_bilevel_needs_gpu_tensors():
         assert "no CPU path" in str(e)
     else:
         raise AssertionError("a CPU call must fail loudly")
+
+
+def test_sub_module_forwards_match_the_float64_restatement():
+    """Mamba3ScanBlock.forward and MiniGRU.forward, the utilities of the reference's module for callers outside the
+    optimizer (mamba3_peer_metanet.py:90-160, 178-192): the block against tests/ref_fp64.scan_block, written from the
+    same lines with every step spelled out, in float64 with a carried state and with gradients reaching the weights;
+    the cell against its formula."""
+    import ref_fp64
+    from grokking_optimizers.mamba3_peer_metanet import Mamba3ScanBlock, MiniGRU
+    torch.manual_seed(3)
+    for kw in (dict(), dict(d_model=4, d_state=6, expand=3)):
+        blk = Mamba3ScanBlock(**kw).double()
+        with torch.no_grad():
+            blk.rope_freq.mul_(20.0)                  # visible rotations
+        x = torch.randn(37, blk.d_model, dtype=torch.float64)
+        h0 = torch.randn(blk.d_inner, blk.d_state, dtype=torch.float64) * 0.3
+        out, hN = blk(x, h0)
+        w9 = [t.detach() for t in (blk.in_proj.weight, blk.dt_proj.weight, blk.dt_proj.bias, blk.B_proj.weight, blk.C_proj.weight,
+                                   blk.A_log, blk.D, blk.rope_freq, blk.out_proj.weight)]
+        want, wantN = ref_fp64.scan_block(x, w9, h0)
+        assert out.shape == (37, blk.d_model) and hN.shape == h0.shape
+        assert torch.allclose(out, want, rtol=1e-10, atol=1e-12) and torch.allclose(hN, wantN, rtol=1e-10, atol=1e-12)
+        out.sum().backward()
+        assert all(p.grad is not None and bool(torch.isfinite(p.grad).all()) for p in blk.parameters())
+        empty, h_same = blk(x[:0], h0)
+        assert empty.shape == (0, blk.d_model) and torch.equal(h_same, h0)
+        zero_start, _ = blk(x)
+        want0, _ = ref_fp64.scan_block(x, w9, torch.zeros_like(h0))
+        assert torch.allclose(zero_start, want0, rtol=1e-10, atol=1e-12)
+    cell = MiniGRU(6, 3).double()
+    x, h = torch.randn(11, 6, dtype=torch.float64), torch.randn(11, 3, dtype=torch.float64)
+    xh = torch.cat([x, h], -1)
+    z = torch.sigmoid(xh @ cell.W_z.weight.T + cell.W_z.bias)
+    r = torch.sigmoid(xh @ cell.W_r.weight.T + cell.W_r.bias)
+    cand = torch.tanh(torch.cat([x, r * h], -1) @ cell.W_h.weight.T + cell.W_h.bias)
+    assert torch.allclose(cell(x, h), (1 - z) * h + z * cand, rtol=1e-12, atol=1e-14)
+
+
+def test_reference_names_for_the_device_bilevel_path():
+    mn = Mamba3PEERMetaNet()
+    assert mn.has_cuda_bilevel is False                # parameters on the CPU: no device kernels can serve it
+    assert callable(mn.forward_for_bilevel_cuda)
