@@ -17,7 +17,7 @@ from grokking_optimizers.grokfast import Grokfast
 from grokking_optimizers.muon import Muon
 from grokking_optimizers.supergrok15 import SuperGrok15, SharpnessMetaNet
 from grokking_optimizers.supergrok2 import SuperGrok2
-from grokking_optimizers.mamba3_peer_metanet import Mamba3PEERMetaNet
+from grokking_optimizers.mamba3_peer_metanet import Mamba3PEERMetaNet, Mamba3ScanBlock, MiniGRU
 from grokking_optimizers.supergrok11 import SuperGrok11
 from grokking_optimizers.grokadamw import GrokAdamW
 from grokking_optimizers.neuralgrok import NeuralGrok
@@ -25,5 +25,7 @@ from grokking_optimizers.prodigy import Prodigy
 from grokking_optimizers.lion import Lion
 from grokking_optimizers.looksam import LookSAM
 
-__all__ = ["Grokfast", "Muon", "SuperGrok15", "SharpnessMetaNet", "SuperGrok2", "Mamba3PEERMetaNet", "SuperGrok11", "GrokAdamW",
-           "NeuralGrok", "Prodigy", "Lion", "LookSAM"]
+__version__ = "2.0.0"      # the reference's (grokking_optimizers/__init__.py:11 there)
+
+__all__ = ["Grokfast", "Muon", "SuperGrok15", "SharpnessMetaNet", "SuperGrok2", "Mamba3PEERMetaNet", "Mamba3ScanBlock", "MiniGRU",
+           "SuperGrok11", "GrokAdamW", "NeuralGrok", "Prodigy", "Lion", "LookSAM"]
