@@ -15,7 +15,8 @@ per-element part as another (SoftElements over sg2_bilevel_elem).  `forward`
 restates the per-element part in torch ops: the tests check sg2_bilevel_elem
 against it, and it serves meta-nets whose routing sizes (heads, keys, experts)
 the per-element bilevel kernel is not built for.  Scan blocks up to the default
-(d_model 8, d_state 16, d_inner 16) run in HIP, smaller ones embedded.
+(d_model 8, d_state 16, d_inner 16) run in HIP, smaller ones embedded; larger ones
+take the scan blocks' own torch forward (chunked, on the GPU) under autograd.
 """
 import torch
 
@@ -138,6 +139,37 @@ def elem_kernel_fits(mn):
             and d["gru_hidden"] <= _cabi.BILEVEL_GRU_HIDDEN and d["expert_hidden"] <= _cabi.BILEVEL_EXPERT_WIDTH)
 
 
+def scan_kernels_fit(mn):
+    """Whether the scan kernels of the bilevel pass can run this net's scan block (up to d_model 8, d_state 16,
+    d_inner 16; smaller ones run embedded)."""
+    dm, ds, di = _cabi.BILEVEL_SCAN_BLOCK
+    return mn.d_model <= dm and mn.d_state <= ds and mn.mamba_fwd.d_inner <= di
+
+
+TORCH_SCAN_LIMIT = 1 << 30      # numel * d_inner * d_state of one tensor on the torch-operation scan (4 GiB per coefficient array)
+
+
+def torch_contexts(mn, g, s, mamba_fwd_state, mamba_bwd_state):
+    """The two contexts of one tensor ([2, N, d_model], element order) and the new Mamba states through the scan
+    blocks' own torch forward (Mamba3ScanBlock.forward, chunked), differentiable by autograd: the bilevel pass of
+    scan blocks larger than its kernels are built for.  Same sort as the kernels: stable, by |g| with non-finite
+    entries taken as 0."""
+    n = g.numel()
+    if n * mn.mamba_fwd.d_inner * mn.d_state > TORCH_SCAN_LIMIT:
+        raise RuntimeError("the bilevel pass of a scan block larger than d_model 8, d_state 16, d_inner 16 runs in torch operations and "
+                           "holds numel * d_inner * d_state floats per coefficient: %d elements exceed its limit of %d"
+                           % (n, TORCH_SCAN_LIMIT // (mn.mamba_fwd.d_inner * mn.d_state)))
+    g = torch.where(torch.isfinite(g), g, torch.zeros_like(g))
+    s = torch.where(torch.isfinite(s), s, torch.zeros_like(s))
+    perm = torch.sort(g.abs(), stable=True).indices
+    x = mn.input_proj(torch.stack([g[perm], s[perm]], dim=-1))
+    fwd, new_f = mn.mamba_fwd(x, mamba_fwd_state)
+    bwd, new_b = mn.mamba_bwd(x.flip(0), mamba_bwd_state)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(n, device=g.device)
+    return torch.stack([fwd[inv], bwd.flip(0)[inv]]), new_f.detach(), new_b.detach()
+
+
 def forward(mn, grad, sharpness, gru_state, mamba_fwd_state=None, mamba_bwd_state=None):
     """The step's own forward (hard top-1 routing) as a module call, for callers that use the meta-net outside the
     fused step: same return values as the reference's Mamba3PEERMetaNet.forward, computed by one call of
@@ -162,14 +194,21 @@ def forward_for_bilevel(mn, grad, sharpness, gru_state, mamba_fwd_state=None, ma
     the reference differentiates through them)."""
     g = grad.reshape(-1).float()
     s = sharpness.reshape(-1).float()
-    plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
-    ctx = ScanContexts.apply(plan, *scan_parameters(mn))
+    if g.device.type != "cuda":
+        raise RuntimeError("the bilevel path of SuperGrok v2 needs GPU tensors: there is no CPU path")
+    if scan_kernels_fit(mn):
+        plan = make_plan(mn, [g], [s], [mamba_fwd_state], [mamba_bwd_state])
+        ctx = ScanContexts.apply(plan, *scan_parameters(mn))
+        new_f, new_b, weights33 = plan.mf[0], plan.mb[0], plan.weights
+    else:
+        ctx, new_f, new_b = torch_contexts(mn, g, s, mamba_fwd_state, mamba_bwd_state)
+        weights33 = None
     if elem_kernel_fits(mn):
-        smart, h_new = SoftElements.apply(plan.weights, meta_dims(mn), float(mn.rescale), g.contiguous(), s.contiguous(),
-                                          gru_state.detach().float().contiguous(), ctx, *elem_parameters(mn))
+        smart, h_new = SoftElements.apply(mn.flat_weights() if weights33 is None else weights33, meta_dims(mn), float(mn.rescale),
+                                          g.contiguous(), s.contiguous(), gru_state.detach().float().contiguous(), ctx, *elem_parameters(mn))
     else:
         smart, h_new = per_element(mn, g, s, ctx[0], ctx[1], gru_state.float())
-    return smart.reshape(grad.shape).to(grad.dtype), h_new, plan.mf[0], plan.mb[0]
+    return smart.reshape(grad.shape).to(grad.dtype), h_new, new_f, new_b
 
 
 def elem_parameters(mn):
@@ -193,6 +232,19 @@ def accumulate_meta_gradients(mn, grads, sharps, gru_states, mamba_fwd, mamba_bw
     """Adds the gradient of  sum_p <smart_grad_p, cotangent_p>  with respect to every parameter of `mn` to its
     .grad, for a list of tensors at once, all in HIP: scan forward (sg2_bilevel_forward), per-element forward and
     backward (sg2_bilevel_elem), scan adjoint (sg2_bilevel_backward).  Returns the smart gradients (flat, packed)."""
+    if not scan_kernels_fit(mn):
+        # a scan block larger than the bilevel kernels are built for: tensor by tensor through the autograd form
+        params = [p for p in mn.parameters() if p.requires_grad]
+        smarts = []
+        for g, s, h, f, b, c in zip(grads, sharps, gru_states, mamba_fwd, mamba_bwd, cotangents):
+            with torch.enable_grad():
+                smart = forward_for_bilevel(mn, g.reshape(-1), s.reshape(-1), h, f, b)[0].float()
+                got = torch.autograd.grad((smart * c.reshape(-1).float()).sum(), params, allow_unused=True)
+            for p, gr in zip(params, got):
+                if gr is not None:
+                    p.grad = gr if p.grad is None else p.grad + gr
+            smarts.append(smart.detach())
+        return torch.cat(smarts)
     plan = make_plan(mn, grads, sharps, mamba_fwd, mamba_bwd)
     g_all = torch.cat([g.reshape(-1).float() for g in grads])
     s_all = torch.cat([s.reshape(-1).float() for s in sharps])

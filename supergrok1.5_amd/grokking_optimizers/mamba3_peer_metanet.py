@@ -46,11 +46,21 @@ class Mamba3ScanBlock(nn.Module):
 
     def forward(self, x, initial_state=None):
         """One scan block on an arbitrary input sequence x [N, d_model] (reference: mamba3_peer_metanet.py:90-160):
-        returns (output [N, d_model], final state [d_inner, d_state]).  A utility for callers that use the block on
-        its own, in torch operations on x's device and differentiable; the optimizer never comes here (its scan runs
-        in the fused kernels, where the input is the two-number feature (g, s) of an element).  Every coefficient of
-        the recurrence is formed for all steps at once; only the 2 x 2 state update itself walks the sequence, so
-        this is meant for sequences of thousands of steps, not millions."""
+        returns (output [N, d_model], final state [d_inner, d_state]).  Torch operations on x's device,
+        differentiable: a utility for callers that use the block on its own, and the scan of the bilevel pass for
+        blocks larger than its kernels are built for.  The optimizer's step never comes here (its scan runs in the
+        fused kernels, where the input is the two-number feature (g, s) of an element).
+
+        Every coefficient of the recurrence is formed for all steps at once; the 2 x 2 state update is then walked
+        in chunks, all chunks side by side: first every chunk's affine map state-in -> state-out (three walks from
+        (1, 0), (0, 1) and 0 + the drive, batched), then the chunk start states one after the other, then every
+        chunk from its start state.  About 2 sqrt(N) batched steps instead of N; memory grows with
+        N * d_inner * d_state."""
+        n = x.shape[0]
+        h0 = (torch.zeros(self.d_inner, self.d_state, device=x.device, dtype=x.dtype) if initial_state is None
+              else initial_state.to(x.dtype))
+        if n == 0:
+            return x.new_zeros(0, self.d_model), h0
         xb, z = self.in_proj(x).chunk(2, dim=-1)
         dt = F.softplus(self.dt_proj(xb)).unsqueeze(-1)                       # [N, di, 1]
         half = 0.5 * dt * -torch.exp(self.A_log)                               # dt A / 2
@@ -58,18 +68,47 @@ class Mamba3ScanBlock(nn.Module):
         drive = dt * self.B_proj(xb).unsqueeze(1) * xb.unsqueeze(-1)           # dt B x
         ang = dt * self.rope_freq                                              # [N, di, ds/2]
         cs, sn = torch.cos(ang), torch.sin(ang)
-        h = (torch.zeros(self.d_inner, self.d_state, device=x.device, dtype=x.dtype) if initial_state is None
-             else initial_state.to(x.dtype))
+
+        length = max(1, int(math.isqrt(n)))                                    # steps per chunk
+        chunks = (n + length - 1) // length
+        pad = chunks * length - n
+
+        def by_chunk(t, fill):                                                 # [N, ...] -> [length, chunks, ...]
+            if pad:
+                t = torch.cat([t, t.new_full((pad,) + tuple(t.shape[1:]), fill)])
+            return t.reshape(chunks, length, *t.shape[1:]).transpose(0, 1)
+        a_c, d_c, cs_c, sn_c = by_chunk(a_bar, 1.0), by_chunk(drive, 0.0), by_chunk(cs, 1.0), by_chunk(sn, 0.0)
+
+        def advance(h, k, driven):                                             # one step of all chunks: h [..., chunks, di, ds]
+            he, ho = h[..., 0::2], h[..., 1::2]
+            rot = torch.stack([he * cs_c[k] - ho * sn_c[k], ho * cs_c[k] + he * sn_c[k]], dim=-1).flatten(-2)
+            return a_c[k] * rot + driven
+
+        shape = (chunks, self.d_inner, self.d_state)
+        if chunks > 1:
+            # affine map of every chunk: the responses to an even unit state, an odd unit state, and the drive alone
+            basis = x.new_zeros(3, *shape)
+            basis[0, ..., 0::2] = 1.0
+            basis[1, ..., 1::2] = 1.0
+            only_third = x.new_zeros(3, 1, 1, 1)
+            only_third[2] = 1.0
+            for k in range(length):
+                basis = advance(basis, k, only_third * d_c[k])
+            starts = [h0]
+            for c in range(chunks - 1):
+                he = starts[-1][:, 0::2].repeat_interleave(2, dim=-1)          # each pair's even / odd entry, at both places
+                ho = starts[-1][:, 1::2].repeat_interleave(2, dim=-1)
+                starts.append(basis[0, c] * he + basis[1, c] * ho + basis[2, c])
+            h = torch.stack(starts)
+        else:
+            h = h0.unsqueeze(0)
         states = []
-        for i in range(x.shape[0]):
-            he, ho = h[:, 0::2], h[:, 1::2]
-            rot = torch.stack([he * cs[i] - ho * sn[i], ho * cs[i] + he * sn[i]], dim=-1).reshape(self.d_inner, self.d_state)
-            h = a_bar[i] * rot + drive[i]
+        for k in range(length):
+            h = advance(h, k, d_c[k])
             states.append(h)
-        if not states:
-            return x.new_zeros(0, self.d_model), h
-        y = (torch.stack(states) * self.C_proj(xb).unsqueeze(1)).sum(-1)
-        return self.out_proj(y * F.silu(z) + self.D * xb), h
+        states = torch.stack(states).transpose(0, 1).reshape(chunks * length, self.d_inner, self.d_state)[:n]
+        y = (states * self.C_proj(xb).unsqueeze(1)).sum(-1)
+        return self.out_proj(y * F.silu(z) + self.D * xb), states[n - 1]
 
 
 class MiniGRU(nn.Module):

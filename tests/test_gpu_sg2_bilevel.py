@@ -221,8 +221,9 @@ def test_differentiable_forward_of_the_whole_meta_net():
 
 
 @pytest.mark.parametrize("kw", [dict(expert_hidden=4), dict(d_model=4, d_state=8, gru_hidden=2, expert_hidden=6),
-                                dict(d_model=6, d_state=10, gru_hidden=3, num_peer_heads=2, num_experts=25)],
-                         ids=["experts_of_width_4", "smaller_net_embedded", "other_routing_sizes"])
+                                dict(d_model=6, d_state=10, gru_hidden=3, num_peer_heads=2, num_experts=25),
+                                dict(d_model=16, d_state=32)],
+                         ids=["experts_of_width_4", "smaller_net_embedded", "other_routing_sizes", "large_scan_block"])
 def test_accumulation_at_other_meta_net_sizes(kw):
     """The bilevel accumulation at sizes other than the defaults, smart gradients and the gradients of every
     parameter against float64 autograd:
@@ -230,7 +231,9 @@ def test_accumulation_at_other_meta_net_sizes(kw):
       (grokking_race_v2.py:1583 -> :775): the per-element kernel runs the narrow experts embedded in its own width;
     * a smaller scan block, GRU and expert width: scan kernels and per-element kernel both run the net embedded;
     * other routing sizes (heads, keys, experts): the scan and its adjoint in HIP (embedded block), the per-element
-      part as torch operations.
+      part as torch operations;
+    * the largest scan block the reference admits (d_model 16, d_state 32, d_inner 32), which the bilevel kernels are
+      not built for: the scan blocks' own chunked torch forward under autograd, on the GPU.
     Then one tensor through the module's forward_for_bilevel (the autograd form over the same kernels)."""
     import copy
     from grokking_optimizers import _bilevel
@@ -246,7 +249,8 @@ def test_accumulation_at_other_meta_net_sizes(kw):
                          h=torch.randn(n, gh, generator=gen) * 0.5, hf=torch.randn(di, ds, generator=gen) * 0.3,
                          hb=torch.randn(di, ds, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
     print("bilevel accumulation", kw, "per-element kernel:", _bilevel.elem_kernel_fits(mn), flush=True)
-    assert _bilevel.elem_kernel_fits(mn) == ("num_experts" not in kw)
+    assert _bilevel.elem_kernel_fits(mn) == ("num_experts" not in kw and kw.get("d_model", 8) <= 8)
+    assert _bilevel.scan_kernels_fit(mn) == (kw.get("d_model", 8) <= 8)
     mn64.zero_grad()
     ref_smart = []
     for d in data:
