@@ -340,6 +340,19 @@ typedef struct Sg2BilevelExtra {
     float* scan_out_bwd;
     float* x_sorted;
     int32_t* perm;
+    /* What launch_mamba3_peer_bilevel_fwd_save[_batched] leaves for its backward pass
+     * (csrc/supergrok2_mamba_peer_backward_kernels.cu:950-1008), per direction (0 forward, 1 backward), each may be
+     * NULL: the x-branch, the gate pre-activation z and the step size dt of every scan step
+     * ([sum numel][d_inner], rows in the order of the direction's own scan, like scan_out), and the scan state after
+     * a step ([rows][d_inner][d_state]).  checkpoint_interval <= 1: after every step, row = the tensor's offset +
+     * the step; otherwise after every checkpoint_interval-th step of the scan and after the last one, row = (sum
+     * over the earlier tensors of ceil(numel / checkpoint_interval)) + step / checkpoint_interval.  This library's
+     * own backward pass reads none of them. */
+    float* saved_x_branch[2];
+    float* saved_z[2];
+    float* saved_dt[2];
+    float* saved_states[2];
+    int32_t checkpoint_interval;
 } Sg2BilevelExtra;
 int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int num_tensors, const Sg2Tensor* tensors,
                            float* ctx_out, const Sg2BilevelExtra* extra, void* workspace, size_t workspace_bytes, void* stream);

@@ -7,15 +7,16 @@
 // two calls and after them -- the gated scan outputs before out_proj in scan order, x_sorted, sort_indices, offsets,
 // the gradients of the Mamba weight tensors (accumulated into the d_* arguments) and d_x_sorted; for the one-tensor
 // pair also the gradients of every other weight of the meta-net.
-// What is not: the per-step `*_saved_x_branch / z / dt` buffers stay untouched and `*_saved_states` is not a table of
-// states.  The HIP adjoint recomputes the states of a 32-step tile from the state entering it, which the forward call
-// keeps in a workspace of its own.  That workspace (with the tensors it refers to) is parked in this process under a
-// fresh 64-bit ticket, and the ticket is written into the first four floats of the caller's `fwd_saved_states`
-// tensor -- which the backward call receives again: it reads the ticket back (one 16-byte device-to-host copy) and
+// The per-step buffers of the interface are filled too, with the reference's layout (`*_saved_x_branch / z / dt` per
+// sorted position; `*_saved_states` after every step, or after every checkpoint_interval-th step of a scan and its
+// last one), although this library's backward pass reads none of them: its adjoint recomputes the states of a
+// 32-step tile from the state entering it, which the forward call keeps in a workspace of its own.  That workspace
+// (with the tensors it refers to) is parked in this process under a fresh 64-bit ticket, and the ticket is written
+// into the first four floats of the caller's `fwd_saved_states` tensor (which therefore do not hold state entries)
+// -- the tensor the backward call receives again: it reads the ticket back (one 16-byte device-to-host copy) and
 // claims exactly the forward call that filled its buffers.  Two optimizers, or interleaved forward / backward pairs,
 // therefore never see each other's state; a buffer no forward call has filled, or one whose ticket was already
 // claimed, is refused.  At most MAX_PARKED forward calls are kept; the oldest is dropped first.
-// checkpoint_interval is accepted and ignored.
 #include <torch/extension.h>
 
 #include <c10/hip/HIPStream.h>
@@ -111,8 +112,23 @@ Saved claim(const char* fn, const char* fwd_name, const torch::Tensor& tag) {
     return S;
 }
 
+// The per-step buffers of the reference's interface (saved x-branch, z, dt: [sum N, d_inner]; saved states:
+// [rows, d_inner, d_state], rows = sum N for checkpoint_interval <= 1, else sum of ceil(N_i / checkpoint_interval)).
+// A tensor of exactly that size is filled; a smaller one is taken as "not wanted" (fwd_saved_states still carries the
+// ticket of the call in its first four floats, which therefore do not hold state entries).
+struct SavedBuffers {
+    torch::Tensor states[2], xb[2], z[2], dt[2];
+    int checkpoint_interval = 1;
+};
+float* wanted(const char* fn, const torch::Tensor& t, int64_t numel, const char* what) {
+    if (!t.defined() || t.numel() < numel) return nullptr;
+    TORCH_CHECK(t.numel() == numel, fn, ": ", what, " holds ", t.numel(), " floats, more than the ", numel, " this call fills");
+    require_f32_gpu(t, fn, what);
+    return t.data_ptr<float>();
+}
+
 void run_forward(const char* fn, Saved& S, const SgDims& dims, torch::Tensor fwd_scan_out, torch::Tensor bwd_scan_out, torch::Tensor x_sorted,
-                 torch::Tensor sort_indices) {
+                 torch::Tensor sort_indices, const SavedBuffers& sv) {
     const size_t P = S.grads.size();
     std::vector<int64_t> numels(P);
     S.tensors.assign(P, Sg2Tensor{});
@@ -144,8 +160,20 @@ void run_forward(const char* fn, Saved& S, const SgDims& dims, torch::Tensor fwd
     const size_t bytes = sg2_bilevel_workspace_bytes(&dims, (int)P, numels.data());
     TORCH_CHECK(bytes > 0 || S.total == 0, fn, ": ", sg_last_error());
     S.workspace = torch::empty({(int64_t)std::max<size_t>(bytes, 256)}, torch::TensorOptions().device(S.w.t[0].device()).dtype(torch::kUInt8));
-    Sg2BilevelExtra extra = {fwd_scan_out.data_ptr<float>(), bwd_scan_out.data_ptr<float>(), x_sorted.data_ptr<float>(),
-                             sort_indices.data_ptr<int32_t>()};
+    Sg2BilevelExtra extra = {};
+    extra.scan_out_fwd = fwd_scan_out.data_ptr<float>();
+    extra.scan_out_bwd = bwd_scan_out.data_ptr<float>();
+    extra.x_sorted = x_sorted.data_ptr<float>();
+    extra.perm = sort_indices.data_ptr<int32_t>();
+    extra.checkpoint_interval = sv.checkpoint_interval;
+    int64_t rows = 0;
+    for (size_t i = 0; i < P; i++) rows += sv.checkpoint_interval <= 1 ? numels[i] : (numels[i] + sv.checkpoint_interval - 1) / sv.checkpoint_interval;
+    for (int d = 0; d < 2; d++) {
+        extra.saved_x_branch[d] = wanted(fn, sv.xb[d], S.total * dims.d_inner, "saved_x_branch");
+        extra.saved_z[d] = wanted(fn, sv.z[d], S.total * dims.d_inner, "saved_z");
+        extra.saved_dt[d] = wanted(fn, sv.dt[d], S.total * dims.d_inner, "saved_dt");
+        extra.saved_states[d] = wanted(fn, sv.states[d], rows * dims.d_inner * dims.d_state, "saved_states");
+    }
     const int rc = sg2_bilevel_forward_ex(&dims, &S.w.W, (int)P, S.tensors.data(), nullptr, &extra, S.workspace.data_ptr(),
                                           (size_t)S.workspace.numel(), stream_of(S.w.t[0]));
     TORCH_CHECK(rc == 0, fn, ": ", sg_last_error());
@@ -173,7 +201,6 @@ void supergrok2_bilevel_fwd_save_batched(
     torch::Tensor bwd_saved_dt_packed, torch::Tensor x_sorted_packed, torch::Tensor offsets_t, torch::Tensor sort_indices_packed,
     torch::Tensor fwd_initial_states, torch::Tensor bwd_initial_states, int checkpoint_interval) {
     const char* fn = "supergrok2_bilevel_fwd_save_batched";
-    (void)checkpoint_interval;
     if (grads.empty()) return;
     TORCH_CHECK(sharpness_list.size() == grads.size(), fn, ": one sharpness tensor per gradient");
     if (!grads[0].is_cuda()) throw std::runtime_error("supergrok2_bilevel_fwd_save_batched requires CUDA tensors.");
@@ -190,7 +217,11 @@ void supergrok2_bilevel_fwd_save_batched(
     const int64_t P = (int64_t)grads.size();
     S.mf = initial_states(fn, fwd_initial_states, P, dims, input_proj_W);
     S.mb = initial_states(fn, bwd_initial_states, P, dims, input_proj_W);
-    run_forward(fn, S, dims, fwd_scan_out_packed, bwd_scan_out_packed, x_sorted_packed, sort_indices_packed);
+    SavedBuffers sv;
+    sv.states[0] = fwd_saved_states_packed; sv.xb[0] = fwd_saved_xb_packed; sv.z[0] = fwd_saved_z_packed; sv.dt[0] = fwd_saved_dt_packed;
+    sv.states[1] = bwd_saved_states_packed; sv.xb[1] = bwd_saved_xb_packed; sv.z[1] = bwd_saved_z_packed; sv.dt[1] = bwd_saved_dt_packed;
+    sv.checkpoint_interval = checkpoint_interval;
+    run_forward(fn, S, dims, fwd_scan_out_packed, bwd_scan_out_packed, x_sorted_packed, sort_indices_packed, sv);
     // element offsets of the tensors in the packed arrays
     TORCH_CHECK(offsets_t.scalar_type() == torch::kInt32 && offsets_t.numel() == P + 1, fn, ": offsets_t must be int32[num_params + 1]");
     std::vector<int32_t> off(P + 1, 0);
@@ -215,7 +246,7 @@ void supergrok2_bilevel_backward_batched(
     torch::Tensor fwd_initial_states, torch::Tensor bwd_initial_states, int d_model, int d_state, int d_inner, int num_params,
     int checkpoint_interval) {
     const char* fn = "supergrok2_bilevel_backward_batched";
-    (void)checkpoint_interval;
+    (void)checkpoint_interval;      // the adjoint restarts from the tile states of the forward call's workspace
     if (num_params == 0) return;
     Saved S = claim(fn, "supergrok2_bilevel_fwd_save_batched", fwd_saved_states_packed);
     TORCH_CHECK((int)S.grads.size() == num_params, fn, ": num_params differs from the forward call");
@@ -278,7 +309,6 @@ void supergrok2_bilevel_fwd_save(
     torch::Tensor bwd_saved_z, torch::Tensor bwd_saved_dt, torch::Tensor x_sorted, torch::Tensor sort_indices,
     torch::Tensor fwd_initial_state, torch::Tensor bwd_initial_state, int checkpoint_interval) {
     const char* fn = "supergrok2_bilevel_fwd_save";
-    (void)checkpoint_interval;
     if (!grad.defined() || grad.numel() == 0) return;
     if (!grad.is_cuda()) throw std::runtime_error("supergrok2_bilevel_fwd_save requires CUDA tensors.");
     const SgDims dims = default_dims(d_model, d_state, d_inner);
@@ -293,7 +323,11 @@ void supergrok2_bilevel_fwd_save(
     S.sharps = {sharpness.contiguous()};
     S.mf = initial_states(fn, fwd_initial_state, 1, dims, input_proj_W);
     S.mb = initial_states(fn, bwd_initial_state, 1, dims, input_proj_W);
-    run_forward(fn, S, dims, fwd_scan_out, bwd_scan_out, x_sorted, sort_indices);
+    SavedBuffers sv;
+    sv.states[0] = fwd_saved_states; sv.xb[0] = fwd_saved_x_branch; sv.z[0] = fwd_saved_z; sv.dt[0] = fwd_saved_dt;
+    sv.states[1] = bwd_saved_states; sv.xb[1] = bwd_saved_x_branch; sv.z[1] = bwd_saved_z; sv.dt[1] = bwd_saved_dt;
+    sv.checkpoint_interval = checkpoint_interval;
+    run_forward(fn, S, dims, fwd_scan_out, bwd_scan_out, x_sorted, sort_indices, sv);
     require_f32_gpu(fwd_final_state, fn, "fwd_final_state");
     require_f32_gpu(bwd_final_state, fn, "bwd_final_state");
     fwd_final_state.view({-1}).copy_(S.mf.view({-1}));

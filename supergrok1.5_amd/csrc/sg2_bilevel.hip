@@ -728,7 +728,102 @@ __global__ __launch_bounds__(256) void k_x_sorted(Plan pl, float* __restrict__ x
     }
 }
 
+// The intermediates the reference's forward-save kernels leave behind (x-branch, z, dt of every scan step; the state
+// after a step, every step or every `interval`-th; rows in the order of each direction's own scan, like scan_out:
+// the reference runs its backward direction on a flipped copy of the input), rebuilt from what the forward pass kept: one workgroup per
+// (chunk, direction) restarts every 32-step tile from its kept entry state and walks it with the plain forms of the
+// recurrence (the forward pass may have taken a polynomial form for the same step: the values agree to rounding).
+struct SavedOut {
+    float* xb[2];
+    float* z[2];
+    float* dt[2];
+    float* states[2];
+    int interval;
+};
+__global__ __launch_bounds__(SCAN_THREADS) void k_saved_fill(Plan pl, SavedOut out) {
+    constexpr int ST = HT_STEP + 1;
+    __shared__ float s_dt[DI * ST], s_xb[DI * ST], s_B[DS * ST];
+    static_assert(SCAN_THREADS == 4 * HT_STEP && DI == 16 && DS == 16, "four row groups of four rows per step");
+    const int chunk = blockIdx.x, dir = blockIdx.y, tid = threadIdx.x;
+    const AdjIO none = {nullptr, {nullptr, nullptr}, nullptr, nullptr};
+    const ChunkRef c = chunk_ref(pl, chunk, dir, none);
+    const int b = dir ? W_B_INPROJ : W_F_INPROJ;
+    const float* __restrict__ Alog = pl.W.w[b + 5];
+    const float* __restrict__ rope = pl.W.w[b + 7];
+    const float* __restrict__ comp = pl.comp + dir * (SG2_COMP_GROUPS * 16 * 3);
+    const int tu = tid & (HT_STEP - 1), quarter = tid >> 5;
+    const int j = tid >> 3, p = tid & 7;
+    const float a_e = 0.5f * sg_exp(Alog[j * DS + 2 * p]), a_o = 0.5f * sg_exp(Alog[j * DS + 2 * p + 1]);
+    const float freq = rope[j * HP + p];
+    int row0 = c.off;                 // first row of this tensor in saved_states
+    if (out.interval > 1) {
+        row0 = 0;
+        for (int i = 0; i < c.ti; i++) row0 += (pl.tensors[i].numel + out.interval - 1) / out.interval;
+    }
+    for (int u0 = c.ustart; u0 < c.uend; u0 += HT_STEP) {
+        const int cnt = min(HT_STEP, c.uend - u0);
+        {
+            const bool valid = tu < cnt;
+            float g, s;
+            int orig;
+            load_step(c, dir, u0 + tu, valid, &g, &s, &orig);
+            float xv[4], zv[4], dv[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int r = quarter * 4 + q;
+                xv[q] = sg2_comp_eval(comp + (SG2_COMP_XB * 16 + r) * 3, g, s);
+                zv[q] = sg2_comp_eval(comp + (SG2_COMP_Z * 16 + r) * 3, g, s);
+                dv[q] = sg_softplus(sg2_comp_eval(comp + (SG2_COMP_DT * 16 + r) * 3, g, s));
+                s_dt[r * ST + tu] = valid ? dv[q] : 0.0f;
+                s_xb[r * ST + tu] = valid ? xv[q] : 0.0f;
+                s_B[r * ST + tu] = sg2_comp_eval(comp + (SG2_COMP_B * 16 + r) * 3, g, s);
+            }
+            if (valid) {
+                const size_t at = ((size_t)c.off + u0 + tu) * DI + quarter * 4;       // row = scan step, as for scan_out
+                if (out.xb[dir]) *reinterpret_cast<float4*>(out.xb[dir] + at) = make_float4(xv[0], xv[1], xv[2], xv[3]);
+                if (out.z[dir]) *reinterpret_cast<float4*>(out.z[dir] + at) = make_float4(zv[0], zv[1], zv[2], zv[3]);
+                if (out.dt[dir]) *reinterpret_cast<float4*>(out.dt[dir] + at) = make_float4(dv[0], dv[1], dv[2], dv[3]);
+            }
+        }
+        __syncthreads();
+        if (out.states[dir] != nullptr) {
+            const float* ht = pl.htile + ((size_t)dir * htile_count(pl.total, pl.P) + htile_index(c.off, c.ti, u0)) * 2 * SCAN_THREADS;
+            float he = ht[tid], ho = ht[SCAN_THREADS + tid];
+            for (int k = 0; k < cnt; k++) {
+                const float dt = s_dt[j * ST + k], ux = dt * s_xb[j * ST + k];
+                float ae, ao, sn, cs;
+                sg_abar_pair(dt, a_e, a_o, &ae, &ao);
+                sg_sincos(dt * freq, &sn, &cs);
+                const float re = sg_fma(he, cs, -(ho * sn)), ro = sg_fma(ho, cs, he * sn);
+                he = sg_fma(ae, re, ux * s_B[(2 * p) * ST + k]);
+                ho = sg_fma(ao, ro, ux * s_B[(2 * p + 1) * ST + k]);
+                const int u = u0 + k;
+                int row = -1;
+                if (out.interval <= 1) row = c.off + u;
+                else if ((u + 1) % out.interval == 0 || u == c.N - 1) row = row0 + u / out.interval;
+                if (row >= 0) *reinterpret_cast<float2*>(out.states[dir] + ((size_t)row * DI + j) * DS + 2 * p) = make_float2(he, ho);
+            }
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace
+
+int launch_saved_intermediates(const Plan& pl, const Sg2BilevelExtra& ex, hipStream_t st) {
+    if (pl.total == 0) return 0;
+    SavedOut out;
+    bool any = false;
+    for (int d = 0; d < 2; d++) {
+        out.xb[d] = ex.saved_x_branch[d]; out.z[d] = ex.saved_z[d]; out.dt[d] = ex.saved_dt[d]; out.states[d] = ex.saved_states[d];
+        any = any || out.xb[d] || out.z[d] || out.dt[d] || out.states[d];
+    }
+    if (!any) return 0;
+    out.interval = ex.checkpoint_interval;
+    hipLaunchKernelGGL(k_saved_fill, dim3(pl.chunks, 2), dim3(SCAN_THREADS), 0, st, pl, out);
+    SG_LAUNCH_CHECK("k_saved_fill");
+    return 0;
+}
 
 int launch_x_sorted(const Plan& pl, float* x_out, hipStream_t st) {
     static_assert(DM == 8, "k_x_sorted: two float4 per element");

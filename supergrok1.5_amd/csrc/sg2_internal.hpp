@@ -159,6 +159,7 @@ int check_dims(const SgDims* d, bool per_element = false);
 // exactly one of d_ctx (element order, after out_proj) / d_scan (scan order, before out_proj) is given; dx (with rx) is optional
 int launch_bilevel_backward(const Plan& pl, const float* d_ctx, const float* const d_scan[2], const float* rx, float* dx, float* grads_out,
                             hipStream_t st);
+int launch_saved_intermediates(const Plan& pl, const Sg2BilevelExtra& ex, hipStream_t st);
 int launch_x_sorted(const Plan& pl, float* x_out, hipStream_t st);
 int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx, hipStream_t st);
 // the net's forward alone (run-time-dimension kernel): smart gradients [total] and new GRU states [total][gru_hidden], packed

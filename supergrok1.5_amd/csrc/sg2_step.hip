@@ -634,6 +634,7 @@ int sg2_bilevel_forward_ex(const SgDims* dims, const Sg2Weights* weights, int nu
     if (extra) { pl.scan_out[0] = extra->scan_out_fwd; pl.scan_out[1] = extra->scan_out_bwd; }
     if (launch_sort(pl, extra ? extra->perm : nullptr, st)) return 1;
     if (launch_scan(pl, st)) return 1;
+    if (extra && launch_saved_intermediates(pl, *extra, st)) return 1;
     if (extra && extra->x_sorted) return launch_x_sorted(pl, extra->x_sorted, st);
     return 0;
 }

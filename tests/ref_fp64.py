@@ -42,6 +42,33 @@ def scan_block(x, w, h0):
     return y @ out_proj.T, h
 
 
+def scan_block_trace(x, w, h0):
+    """What the reference's forward-save kernels keep of a scan (csrc/supergrok2_mamba_peer_backward_kernels.cu:950-1008):
+    x-branch, z and dt of every step [N, di] and the state after every step [N, di, ds]."""
+    in_proj, dt_W, dt_b, Bp, _, A_log, _, rope, _ = [t.to(F) for t in w]
+    di = dt_W.shape[0]
+    xz = x @ in_proj.T
+    xb, z = xz[:, :di], xz[:, di:]
+    raw = xb @ dt_W.T + dt_b
+    dt = torch.where(raw > 20.0, raw, torch.log1p(torch.exp(torch.clamp(raw, max=20.0))))
+    B = xb @ Bp.T
+    A = -torch.exp(A_log)
+    h = h0.to(F).clone()
+    states = []
+    for i in range(x.shape[0]):
+        dti = dt[i].unsqueeze(-1)
+        A_bar = (1.0 + dti * A / 2.0) / (1.0 - dti * A / 2.0 + 1e-8)
+        ang = dti * rope
+        c, s = torch.cos(ang), torch.sin(ang)
+        he, ho = h[:, 0::2], h[:, 1::2]
+        hr = torch.zeros_like(h)
+        hr[:, 0::2] = he * c - ho * s
+        hr[:, 1::2] = ho * c + he * s
+        h = A_bar * hr + dti * B[i].unsqueeze(0) * xb[i].unsqueeze(-1)
+        states.append(h)
+    return xb, z, dt, torch.stack(states)
+
+
 def step(weights, param, grad, sharp, ea, easq, mu, gru, mfwd, mbwd, sc, dims):
     """Returns dict of new values (float64) + integer routing results."""
     W = [w.to(F) for w in weights]

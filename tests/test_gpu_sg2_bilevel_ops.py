@@ -327,3 +327,62 @@ def test_bilevel_pairs_do_not_see_each_other():
     fresh = dict(a, saved=[z(900, 16, 16)] + a["saved"][1:])
     with pytest.raises(RuntimeError, match="no supergrok2_bilevel_fwd_save_batched"):
         backward(fresh, 1)
+
+
+@pytest.mark.parametrize("interval", [1, 4])
+def test_forward_save_fills_the_per_step_buffers(interval):
+    """The buffers the reference's forward-save kernels leave for its own backward pass
+    (csrc/supergrok2_mamba_peer_backward_kernels.cu:950-1008; sizes as grokking_optimizers/supergrok2.py:667-681
+    allocates them): x-branch, z and dt of every scan step and the state after every step -- or, with a checkpoint
+    interval, after every interval-th step of a tensor's scan and after its last one, at that tensor's checkpoint
+    offset -- in the order of each direction's own scan, against the float64 recurrence.  The first four floats of
+    fwd_saved_states carry the call's ticket instead of state entries."""
+    from grokking_optimizers import _ops
+    dev = torch.device("cuda:0")
+    mn = _meta_net(9, dev)
+    mn64 = copy.deepcopy(mn).double().cpu()
+    gen = torch.Generator().manual_seed(41)
+    Ns = [150, 31, 1300, 64, 5]
+    data = [dict(g=torch.randn(n, generator=gen) * 0.5, s=torch.rand(n, generator=gen) * 0.3,
+                 hf=torch.randn(16, 16, generator=gen) * 0.3, hb=torch.randn(16, 16, generator=gen) * 0.3) for n in Ns]
+    w = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in mn.get_weights().items()}
+    d_model, d_state, d_inner = 8, 16, 16
+    total, P = sum(Ns), len(Ns)
+    ck = [n if interval <= 1 else (n + interval - 1) // interval for n in Ns]
+    z = lambda *s: torch.full(s, float("nan"), device=dev)          # whatever is not written stays NaN
+    fwd_scan, bwd_scan = z(total, d_inner), z(total, d_inner)
+    saved = [z(sum(ck), d_inner, d_state)] + [z(total, d_inner) for _ in range(3)] + [z(sum(ck), d_inner, d_state)] + [z(total, d_inner) for _ in range(3)]
+    x_sorted, offsets_t = z(total, d_model), torch.zeros(P + 1, dtype=torch.int32, device=dev)
+    sort_idx = torch.zeros(total, dtype=torch.int32, device=dev)
+    print("fwd_save_batched with checkpoint interval", interval, flush=True)
+    _ops.supergrok2_bilevel_fwd_save_batched([d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data], w["input_proj_W"],
+                                             w["input_proj_b"], *_mamba_args(w, "fwd", True), *_mamba_args(w, "bwd", True), d_model, d_state,
+                                             d_inner, fwd_scan, bwd_scan, *saved, x_sorted, offsets_t, sort_idx,
+                                             torch.stack([d["hf"] for d in data]).to(dev), torch.stack([d["hb"] for d in data]).to(dev), interval)
+    torch.cuda.synchronize()
+    got = [t.double().cpu() for t in saved]
+    W64 = _flat64(mn64)
+    offs, coffs = np.concatenate([[0], np.cumsum(Ns)]), np.concatenate([[0], np.cumsum(ck)])
+
+    def close(a, b, what):
+        assert bool(torch.isfinite(a).all()), what
+        err = (a - b).abs()
+        tol = 1e-4 * torch.maximum(a.abs(), b.abs()) + 1e-6
+        assert bool((err <= tol).all()), (what, float((err / tol).max()))
+    for i, d in enumerate(data):
+        a, b, ca, cb = int(offs[i]), int(offs[i + 1]), int(coffs[i]), int(coffs[i + 1])
+        perm = torch.sort(d["g"].abs(), stable=True).indices
+        x = torch.stack([d["g"][perm], d["s"][perm]], -1).double() @ W64[0].detach().T + W64[1].detach()
+        for k, (xs, w9, h0) in enumerate(((x, W64[2:11], d["hf"]), (x.flip(0), W64[11:20], d["hb"]))):
+            xb, zz, dt, states = ref_fp64.scan_block_trace(xs, [t.detach() for t in w9], h0.double())
+            close(got[4 * k + 1][a:b], xb, ("x_branch", i, k))
+            close(got[4 * k + 2][a:b], zz, ("z", i, k))
+            close(got[4 * k + 3][a:b], dt, ("dt", i, k))
+            n = Ns[i]
+            steps = list(range(n)) if interval <= 1 else [min((q + 1) * interval, n) - 1 for q in range(cb - ca)]
+            have, want = got[4 * k][ca:cb].clone(), states[steps]
+            if k == 0 and i == 0:
+                have.view(-1)[:4] = want.reshape(-1)[:4]          # the ticket of the call
+            close(have, want, ("states", i, k))
+    ticket = saved[0].view(-1)[:4].view(torch.int32).cpu()
+    assert int(ticket[0]) == 0x5347324B
