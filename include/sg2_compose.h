@@ -135,6 +135,16 @@ SG_HD float sg2_poly2(const float* q, float d) { return sg_fma(sg_fma(q[2], d, q
 SG_HD int sg2_poly_ok(float kpoly_g, float kpoly_s, float g, float s) {
     return sg_fma(kpoly_g, sg_abs(g), kpoly_s * sg_abs(s)) < 1.0f;
 }
+/* The factor in front of the dt rows' coefficients can be smaller than k: softplus is convex with derivative sigmoid, so
+ * |dt - dt0| <= sigmoid(c_0 + m) |c_g g + c_s s| for a row with constant term c_0 while |c_g g + c_s s| <= m.  A
+ * timestep that qualifies has |c_g g + c_s s| < 1 / (factor), so with m = 1/16 the largest sigmoid(c_0 + m) of the
+ * direction's dt rows may multiply k as long as the product stays at least 16; otherwise k stands. */
+#define SG2_SLOPE_MARGIN 0.0625f
+SG_HD float sg2_dt_slope(float c0) { return sg_sigmoid(c0 + SG2_SLOPE_MARGIN); }
+SG_HD float sg2_limit_factor(float k, float slope_max) {
+    const float ks = k * slope_max;
+    return ks >= 16.0f ? ks : k;
+}
 
 /* The output pass goes one step further: its update h' = D R h + b needs only the four products of the pair,
  * P1 = A_bar_e cos, N2 = -A_bar_e sin, P3 = A_bar_o cos, P4 = A_bar_o sin, and takes those as quadratics in d = dt - dt0

@@ -743,13 +743,14 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
             }
             /* lane polynomials and the limit of their use */
             const int hp = ds / 2;
-            float amax = 0.0f, fmax = 0.0f, cdt[2] = {0.0f, 0.0f};
+            float amax = 0.0f, fmax = 0.0f, cdt[2] = {0.0f, 0.0f}, slope = 0.0f;
             w.lane_poly.assign((size_t)di * hp * 14, 0.0f);
             w.lane_prod.assign((size_t)di * hp * 12, 0.0f);
             for (int j = 0; j < di; j++) {
                 const float* cd = &w.comp[((size_t)SG2_COMP_DT * w.comp_rows + j) * 3];
                 cdt[0] = sg_max(cdt[0], sg_abs(cd[0]));
                 cdt[1] = sg_max(cdt[1], sg_abs(cd[1]));
+                slope = sg_max(slope, sg2_dt_slope(cd[2]));
                 const float dt0 = w.tay[((size_t)0 * w.comp_rows + j) * 4];
                 for (int p = 0; p < hp; p++) {
                     const float a_e = -0.5f * -sg_exp(w.A_log[j * ds + 2 * p]), a_o = -0.5f * -sg_exp(w.A_log[j * ds + 2 * p + 1]);
@@ -763,10 +764,10 @@ int step_tensor(const Dims& d, const float* const* W, int64_t chunk_len, int64_t
                     sg2_pair_products(dt0, a_e, a_o, f, &w.lane_prod[((size_t)j * hp + p) * 12]);
                 }
             }
-            const float kp = sg_max(128.0f * amax, 256.0f * fmax);
+            const float kp = sg2_limit_factor(sg_max(128.0f * amax, 256.0f * fmax), slope);
             w.kpoly[0] = kp * cdt[0];
             w.kpoly[1] = kp * cdt[1];
-            const float kq = sg_fma(416.0f, amax, 184.0f * fmax);
+            const float kq = sg2_limit_factor(sg_fma(416.0f, amax, 184.0f * fmax), slope);
             w.kprod[0] = kq * cdt[0];
             w.kprod[1] = kq * cdt[1];
         }

@@ -193,10 +193,10 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
     dst[2] = out[2];
     // How many steps the first block of a chunk summary should cover: what the slowest pair of either direction needs
     // to contract below 2^-100 at the step size a zero input gives (sg2_contraction_steps), plus a margin.
-    __shared__ int s_largest, s_zero, s_bad, s_cmax[2][2], s_cdt[2][2], s_amax[2], s_fmax[2];
+    __shared__ int s_largest, s_zero, s_bad, s_cmax[2][2], s_cdt[2][2], s_amax[2], s_fmax[2], s_slope[2];
     if (threadIdx.x == 0) {
         s_largest = 0; s_zero = 0; s_bad = 0;
-        for (int k = 0; k < 2; k++) { s_cmax[k][0] = s_cmax[k][1] = s_cdt[k][0] = s_cdt[k][1] = s_amax[k] = s_fmax[k] = 0; }
+        for (int k = 0; k < 2; k++) { s_cmax[k][0] = s_cmax[k][1] = s_cdt[k][0] = s_cdt[k][1] = s_amax[k] = s_fmax[k] = s_slope[k] = 0; }
     }
     __syncthreads();
     // Taylor polynomials of the step size and of the gate around their zero-input arguments (sg2_compose.h), and the
@@ -212,6 +212,7 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
         if (group == SG2_COMP_DT) {
             atomicMax(&s_cdt[dir][0], sg_f2i(sg_abs(out[0])));
             atomicMax(&s_cdt[dir][1], sg_f2i(sg_abs(out[1])));
+            atomicMax(&s_slope[dir], sg_f2i(sg2_dt_slope(out[2])));       // positive: its bit pattern orders like the value
         }
     }
     if (group == SG2_COMP_DT) {
@@ -238,11 +239,12 @@ __global__ __launch_bounds__(2 * SG2_COMP_GROUPS * G::ROWS) void k_compose(Plan 
         cmax[0] = sg_i2f(s_cmax[0][0]); cmax[1] = sg_i2f(s_cmax[0][1]);
         cmax[2] = sg_i2f(s_cmax[1][0]); cmax[3] = sg_i2f(s_cmax[1][1]);
         for (int k = 0; k < 2; k++) {
-            const float kp = sg_max(128.0f * sg_i2f(s_amax[k]), 256.0f * sg_i2f(s_fmax[k]));
+            const float slope = sg_i2f(s_slope[k]);      // how much of a change of its argument the step size follows at most
+            const float kp = sg2_limit_factor(sg_max(128.0f * sg_i2f(s_amax[k]), 256.0f * sg_i2f(s_fmax[k])), slope);
             cmax[4 + 2 * k] = kp * sg_i2f(s_cdt[k][0]);
             cmax[5 + 2 * k] = kp * sg_i2f(s_cdt[k][1]);
             // ... and for the products of the output pass (sg2_pair_products)
-            const float kq = sg_fma(416.0f, sg_i2f(s_amax[k]), 184.0f * sg_i2f(s_fmax[k]));
+            const float kq = sg2_limit_factor(sg_fma(416.0f, sg_i2f(s_amax[k]), 184.0f * sg_i2f(s_fmax[k])), slope);
             cmax[8 + 2 * k] = kq * sg_i2f(s_cdt[k][0]);
             cmax[9 + 2 * k] = kq * sg_i2f(s_cdt[k][1]);
         }
