@@ -161,6 +161,38 @@ def test_contracted_summaries_forget_a_finite_carried_state_only():
         assert np.array_equal(fwd[0][k], fwd[2][k])
 
 
+def test_three_hundred_tensors_in_one_call():
+    """300 tensors of 0 .. 900 elements in one call (the per-call tables travel in 13 launches of 24 records each),
+    chunk length 256 so that the larger ones have several chunks; two steps against the checker.  Then the same call
+    with a carried state of tensor 211 made infinite: the flag that switches the contracted-summary shortcut off is
+    raised by a later table launch than the first, that tensor's forward contexts come out non-finite and every other
+    tensor's values stay what they were, bit for bit."""
+    from grokking_optimizers import _cabi
+    r = np.random.RandomState(4)
+    shapes = [(int(n),) for n in r.randint(0, 900, size=300)]
+    shapes[17] = (0,)
+    cl = 256
+    assert _cabi.lib().sg2_set_chunk_len(cl) == 0
+    case = Sg2Case(shapes, seed=12, random_state=True)
+    w = _run_steps(case, 2, chunk_len=cl, sharp=True, lamb_eff=2.0)
+    print("300 tensors: worst tolerance ratios", w, flush=True)
+    assert shapes[211][0] > cl
+    ctx = []
+    for poison in (False, True):
+        case = Sg2Case(shapes, seed=12, random_state=True)
+        if poison:
+            case.gpu[211]["mamba_fwd"][3, 5] = float("inf")
+        grads = wl.make_grads(shapes, seed=78)
+        case.gpu_step(grads, [torch.zeros_like(g) for g in grads], per_tensor_scalars(case.P, 1, 2.0), shared_scalars(4.5))
+        ctx.append(case.step_fn.ctx.cpu().numpy().copy())
+    a, b = int(case.offsets[211]), int(case.offsets[212])
+    assert not np.isfinite(ctx[1][0, a:b]).all(axis=-1).any()
+    assert np.isfinite(ctx[0]).all() and np.isfinite(ctx[1][1]).all()
+    keep = np.ones(ctx[0].shape[1], bool)
+    keep[a:b] = False
+    assert np.array_equal(ctx[0][:, keep], ctx[1][:, keep]) and np.array_equal(ctx[0][1], ctx[1][1])
+
+
 def test_saturated_gates_take_the_plain_forms():
     """The scan's output gates, the GRU gates and the GRU candidates are formed with one shared reciprocal per group
     unless the product of the group's denominators is too large; then every value of the group takes the plain
