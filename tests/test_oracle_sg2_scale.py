@@ -116,3 +116,21 @@ def test_flip_rate_with_routing_spread_over_most_experts():
     print("spread routing: %d experts in use" % used, flush=True)
     assert used >= 100
     _check(a, da, b, db, "262 144 elements, routing spread over %d experts" % used)
+
+
+def test_module_initialised_weights_around_the_polynomial_limits():
+    """The reference's own initial meta-net (A_log = log(1..16): poles down to -16, where the lane polynomials and
+    the product forms have their narrowest range of valid inputs), with gradients spread over three decades around
+    1e-3 so that the sorted sequence walks through every form the kernels have -- linear products, quadratic
+    products, lane polynomials with the plain update, the general recurrence -- and a populated sharpness.  The fp32
+    policy as the kernels chunk it against the float64 sequential recurrence: every state within 1e-4, every routing
+    difference at a float64 margin below 1e-5."""
+    n = 1 << 17
+    r = np.random.RandomState(31)
+    g = (r.randn(n) * np.exp(r.uniform(np.log(3e-5), np.log(3e-2), size=n))).astype(np.float32)
+    s = (np.abs(r.randn(n)) * 3e-4).astype(np.float32)
+    W = [w.numpy().copy() for w in wl.module_weights(3)]
+    st = random_state_np(n, 79)
+    sc = f32_scalars(default_scalars(i=2, step=5, lamb_eff=2.0))
+    (a, da), (b, db) = _both_policies(W, st, g, s, sc, 1024, 64)
+    _check(a, da, b, db, "131 072 elements, module-initialised weights, gradients 3e-5 .. 3e-2")
