@@ -491,11 +491,14 @@ def muon_precision(dev):
 
 def secondary_configs(dev, steps=20, warmup=3):
     """The other measured configurations, each timed in this run: Grokfast and SuperGrok v1.5 on the 14-tensor set, the
-    SuperGrok v2 step on the 14-tensor set, Muon on its 24 bf16 matrices (algorithmic and executed MFMA fraction)."""
+    SuperGrok v2 step on the 14-tensor set, Muon on its 24 bf16 matrices (algorithmic and executed MFMA fraction), the
+    bilevel meta-gradient pass of v2 on the 14-tensor set and the five other fused steps on the 25 M-element set."""
     import torch
     from grokking_optimizers import _ops
     out = {}
-    for name, workload in (("config1_grokfast", "grokfast"), ("config2_supergrok15", "sg15"), ("config5_muon", "muon")):
+    for name, workload in (("config1_grokfast", "grokfast"), ("config2_supergrok15", "sg15"), ("config5_muon", "muon"),
+                           ("bilevel_pass_shared14", "bilevel"), ("grokadamw_scale50", "grokadamw"), ("neuralgrok_scale50", "neuralgrok"),
+                           ("prodigy_scale50", "prodigy"), ("lion_scale50", "lion"), ("supergrok11_scale50", "sg11")):
         W = build_step(workload, _ops, dev)
         for _ in range(warmup):
             W["step"]()
