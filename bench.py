@@ -21,6 +21,7 @@ for p in (ROOT, os.path.join(ROOT, "supergrok1.5_amd")):
 BYTES_PER_ELEMENT = 72          # algorithmic HBM bytes per element per step (fp32): 40 read + 32 written
 HBM_PEAK_GBS = 8000.0
 SIMDS = 1024
+REPLAY_WAVES_PER_SIMD = 2        # k_replay: eight one-wave workgroups per compute unit (19.8 KB of LDS each)
 STAGE_KERNEL_PREFIX = {"scan_output": "k_replay<", "scan_summary": "k_scan<false, false>", "elementwise": "k_elem<"}
 
 
@@ -48,15 +49,17 @@ def profile_figures():
             if line.startswith(prefix):
                 cols = line[40:].split()                                                   # after the (truncated) kernel name
                 out["valu"][stage] = float(cols[1])                                        # us/launch, INSTS_VALU, ...
-    best = 0.0
+    best, by_waves = 0.0, {}
     for line in rows("valu_probe_mi355x.txt"):
         cols = line.split()
         if len(cols) >= 5 and cols[0] in ("fma", "mul", "add", "add_dpp"):
             try:
                 best = max(best, float(cols[3]))
+                by_waves.setdefault(int(cols[1]), {})[cols[0]] = float(cols[3])
             except ValueError:
                 pass
     out["sustained"] = best or None
+    out["sustained_by_waves"] = by_waves        # waves per SIMD -> {instruction kind: instructions per ns and SIMD}
     out["source"] = {"traffic": "profiles/sg2_step_scale50_pmc_traffic.txt", "valu": "profiles/sg2_step_scale50_pmc_sq.txt",
                      "sustained": "profiles/valu_probe_mi355x.txt"}
     return out
@@ -697,6 +700,11 @@ def main():
         out["valu"] = {"kernel": kernel_of[dom], "instructions": prof["valu"][dom], "instructions_source": prof["source"]["valu"],
                        "per_ns_simd": rate, "sustained_per_ns_simd": prof["sustained"], "sustained_source": prof["source"]["sustained"],
                        "frac": rate / prof["sustained"]}
+        # the yardstick that fits the kernel: it keeps REPLAY_WAVES_PER_SIMD waves on a SIMD and issues mostly fma
+        at = prof.get("sustained_by_waves", {}).get(REPLAY_WAVES_PER_SIMD)
+        if dom == "scan_output" and at and at.get("fma"):
+            out["valu"].update({"waves_per_simd": REPLAY_WAVES_PER_SIMD, "sustained_at_that_occupancy": at,
+                                "frac_of_fma_rate_at_that_occupancy": rate / at["fma"]})
     if not args.no_class_step and args.geometry == "default":
         out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if default_workload and not args.no_extras:
