@@ -52,7 +52,7 @@ def profile_figures():
     best, by_waves = 0.0, {}
     for line in rows("valu_probe_mi355x.txt"):
         cols = line.split()
-        if len(cols) >= 5 and cols[0] in ("fma", "mul", "add", "add_dpp"):
+        if len(cols) >= 5 and cols[0] in ("fma", "fmac", "fma_vector_operands", "fma_scalar_operand", "mul", "add", "add_dpp"):
             try:
                 best = max(best, float(cols[3]))
                 by_waves.setdefault(int(cols[1]), {})[cols[0]] = float(cols[3])
@@ -334,8 +334,10 @@ def bench_probe(dev):
     rows, best = [], 0.0
     for ncu in (cus,):
         for op, name in enumerate(("fma", "mul", "add", "add_dpp", "mfma_32x32x16_bf16", "mfma_32x32x16_bf16_random_operands",
-                                   "mfma_32x32x1_f32", "mfma_32x32x1_f32_then_8_fma", "mfma_4x4x1_f32")):
-            for w in ((1, 2) if op >= 4 else (1, 2, 3, 4, 8)):
+                                   "mfma_32x32x1_f32", "mfma_32x32x1_f32_then_8_fma", "mfma_4x4x1_f32", "fmac", "fma_vector_operands",
+                                   "fma_scalar_operand")):
+            matrix = 4 <= op <= 8
+            for w in ((1, 2) if matrix else (1, 2, 3, 4, 8)):
                 ms, ticks, instr = C.c_float(), C.c_double(), C.c_double()
                 if L.sg_probe_valu(op, ncu, w, 2000, C.byref(ms), C.byref(ticks), C.byref(instr), ws.data_ptr(), ws.numel(),
                                    torch.cuda.current_stream().cuda_stream) != 0:
@@ -345,7 +347,7 @@ def bench_probe(dev):
                              "instr_per_ns_per_simd": round(rate, 4),
                              "clock_ticks_per_instr_per_simd": round(ticks.value / instr.value / w, 3),
                              "clock_ticks_per_ns": round(ticks.value / (ms.value * 1e6), 3)})
-                if op >= 4:      # flop per matrix instruction (the vector fma of the mixed stream are not counted)
+                if matrix:       # flop per matrix instruction (the vector fma of the mixed stream are not counted)
                     rows[-1]["chip_tflops"] = round(rate * (32768, 32768, 4096, 4096, 512)[op - 4] * 4 * ncu / 1e3, 1)
                 elif ncu == cus:
                     best = max(best, rate)
@@ -702,9 +704,13 @@ def main():
                        "frac": rate / prof["sustained"]}
         # the yardstick that fits the kernel: it keeps REPLAY_WAVES_PER_SIMD waves on a SIMD and issues mostly fma
         at = prof.get("sustained_by_waves", {}).get(REPLAY_WAVES_PER_SIMD)
-        if dom == "scan_output" and at and at.get("fma"):
-            out["valu"].update({"waves_per_simd": REPLAY_WAVES_PER_SIMD, "sustained_at_that_occupancy": at,
-                                "frac_of_fma_rate_at_that_occupancy": rate / at["fma"]})
+        if dom == "scan_output" and at:
+            # fma_vector_operands: every operand in a vector register, as in the recurrence of the replay;
+            # fma / fma_scalar_operand: one operand in a scalar register, as where weights are wave-uniform
+            out["valu"].update({"waves_per_simd": REPLAY_WAVES_PER_SIMD, "sustained_at_that_occupancy": at})
+            for kind in ("fma_vector_operands", "fma_scalar_operand"):
+                if at.get(kind):
+                    out["valu"]["frac_of_%s_rate_at_that_occupancy" % kind] = rate / at[kind]
     if not args.no_class_step and args.geometry == "default":
         out["class_step_ms"] = class_step_ms(shapes, grad_sets, dev, args.steps, args.warmup)
     if default_workload and not args.no_extras:

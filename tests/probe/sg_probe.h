@@ -16,7 +16,11 @@ extern "C" {
  * v_mfma_f32_32x32x1_2b_f32, 7 the same with 8 v_fma_f32 after each in the
  * same wave (the vector instructions are not counted), 8
  * v_mfma_f32_4x4x1_16b_f32: the fp32 matrix forms that are one fused
- * multiply-add per output) on num_cus x waves_per_simd workgroups of four
+ * multiply-add per output; 9 v_fmac_f32, the accumulate form of the fma, on
+ * per-lane factors; 10 op 0 with its two other operands in per-lane vector
+ * registers; 11 v_fma_f32 with one scalar-register operand and three vector
+ * registers: an instruction that reads a scalar register issues more slowly
+ * once several waves share a SIMD) on num_cus x waves_per_simd workgroups of four
  * waves, i.e. waves_per_simd waves on every SIMD of num_cus compute units
  * when the dispatcher spreads them evenly.  Synchronises the stream.  Returns
  * the elapsed milliseconds of the launch, the shader-clock ticks a wave took

@@ -16,6 +16,12 @@ __global__ __launch_bounds__(256) void k_probe(float* sink, long long* ticks, in
     float acc[PROBE_ILP];
 #pragma unroll
     for (int k = 0; k < PROBE_ILP; k++) acc[k] = threadIdx.x * 1e-3f + k + 1.0f;
+    float xs[4], ys[4];        // per-lane factors of the accumulate form, of both signs so that the sums stay bounded
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        xs[k] = ((k & 1) ? -1.0f : 1.0f) * (a + 1e-3f * (threadIdx.x & 15) + 0.01f * k);
+        ys[k] = ((k & 2) ? -1.0f : 1.0f) * (b + 1e-3f * (threadIdx.x & 7));
+    }
     const long long t0 = clock64();
     for (int i = 0; i < iters; i++) {
 #pragma unroll
@@ -23,6 +29,9 @@ __global__ __launch_bounds__(256) void k_probe(float* sink, long long* ticks, in
 #pragma unroll
             for (int k = 0; k < PROBE_ILP; k++) {
                 if (OP == 0) acc[k] = __builtin_fmaf(acc[k], a, b);
+                else if (OP == 4) acc[k] = __builtin_fmaf(xs[(k + r) & 3], ys[k & 3], acc[k]);      // accumulate form: v_fmac_f32
+                else if (OP == 5) acc[k] = __builtin_fmaf(acc[k], xs[(k + r) & 3], ys[k & 3]);      // op 0 with per-lane register operands
+                else if (OP == 6) acc[k] = __builtin_fmaf(acc[k], a, acc[(k + 1) % PROBE_ILP]);     // three vector registers, one scalar
                 else if (OP == 1) acc[k] = acc[k] * a;
                 else if (OP == 2) acc[k] = acc[k] + a;
                 else acc[k] = acc[k] + sg_i2f(__builtin_amdgcn_update_dpp(0, sg_f2i(acc[k]), 0xB1, 0xF, 0xF, true));
@@ -141,9 +150,10 @@ size_t sg_probe_workspace_bytes(int num_cus, int waves_per_simd) {
 int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_out, double* ticks_per_wave_out,
                   double* instr_per_wave_out, void* workspace, size_t workspace_bytes, void* stream) {
     hipStream_t st = (hipStream_t)stream;
-    if (op < 0 || op > 8)
+    if (op < 0 || op > 11)
         return sg::fail("op must be 0 (fma), 1 (mul), 2 (add), 3 (add with a DPP operand), 4 (32x32x16 bf16 MFMA, constant operands), 5 (the same, random "
-                        "operands), 6 (32x32x1 fp32 MFMA), 7 (the same with 8 vector fma after each) or 8 (4x4x1 fp32 MFMA)");
+                        "operands), 6 (32x32x1 fp32 MFMA), 7 (the same with 8 vector fma after each), 8 (4x4x1 fp32 MFMA), 9 (fma in its accumulate "
+                        "form, per-lane factors), 10 (fma, vector-register operands only) or 11 (fma with one scalar-register operand)");
     if (num_cus <= 0 || num_cus > 1024 || waves_per_simd <= 0 || waves_per_simd > 8 || iters <= 0 || iters > 100000)
         return sg::fail("probe size out of range");
     if (!ms_out || !ticks_per_wave_out || !instr_per_wave_out) return sg::fail("NULL argument");
@@ -164,6 +174,9 @@ int sg_probe_valu(int op, int num_cus, int waves_per_simd, int iters, float* ms_
             case 6: hipLaunchKernelGGL(k_probe_mfma_f32<0>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             case 7: hipLaunchKernelGGL(k_probe_mfma_f32<1>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
             case 8: hipLaunchKernelGGL(k_probe_mfma_f32<2>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 9: hipLaunchKernelGGL(k_probe<4>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
+            case 10: hipLaunchKernelGGL(k_probe<5>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 0.9f, 0.5f); break;
+            case 11: hipLaunchKernelGGL(k_probe<6>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 0.4f, 0.5f); break;
             default: hipLaunchKernelGGL(k_probe<3>, dim3(blocks), dim3(256), 0, st, sink, ticks, n, 1.0001f, 0.5f); break;
         }
     };
