@@ -812,14 +812,15 @@ __global__ __launch_bounds__(G::THREADS) SG2_SCAN_ATTR void k_scan(Plan pl) {
     }
 }
 
-// Projections of one timestep for the one-wave replay: the lane computes every row of every group for its timestep
-// (what the two waves of k_scan each do half of through project_tile, with the same expressions in the same order).
-// Step size, dt * x-branch, B and C go to LDS for the recurrence; the skip terms D * x-branch stay in the lane's
-// registers, because in this kernel the lane that forms them is the one that uses them after the recurrence, and
-// for the same reason the gates are not formed here at all (gates_all, after the recurrence).
+// Projections of one timestep for the one-wave replay, for a tile that does not run on the polynomials throughout
+// (project_rows covers the usual tile): the lane computes every row of every group for its timestep (what the two
+// waves of k_scan each do half of through project_tile, with the same expressions in the same order).  Step size,
+// dt * x-branch, B and C go to LDS for the recurrence; the skip terms D * x-branch stay in the lane's registers,
+// because the lane that forms them is the one that uses them after the recurrence, and for the same reason the gates
+// are not formed here at all (gates_all, after the recurrence).
 // coef: [group][row] composed triple + one more float (D next to the x-branch triple); tay: [step size | gate][row][4].
 // angle[h]: bit 0 / 1 = every rotation angle of columns 8 h .. 8 h + 7 at this timestep is small / tiny.
-template <class G, bool HAS_S, bool TAYLOR, bool DSTORE>
+template <class G, bool HAS_S, bool TAYLOR>
 __device__ __forceinline__ void project_all(float g, float s, int tu, const float* s_coef, const float* s_tay, const float* s_fmax, float* s_dt,
                                             float* s_ux, float* s_B, float* s_C, float (&dxv)[G::DI], int (&angle)[2]) {
     constexpr int DI = G::DI, DS = G::DS;
@@ -835,22 +836,13 @@ __device__ __forceinline__ void project_all(float g, float s, int tu, const floa
         for (int q = 0; q < 8; q++) {
             const int jj = 8 * h + q;
             const f32x4 cd = coef(SG2_COMP_DT, jj);
-            float dtv, dt0 = 0.0f;
-            if (TAYLOR) {
-                const f32x4 tp = *reinterpret_cast<const f32x4*>(s_tay + jj * 4);
-                dtv = poly(tp, delta(cd));
-                dt0 = tp[0];
-            } else {
-                dtv = sg_softplus(eval(cd));
-            }
-            if (!DSTORE) {
-                const float amax = dtv * s_fmax[jj];
-                small = small && (amax < SG_SINCOS_SMALL_LIMIT);
-                tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
-            }
+            const float dtv = TAYLOR ? poly(*reinterpret_cast<const f32x4*>(s_tay + jj * 4), delta(cd)) : sg_softplus(eval(cd));
+            const float amax = dtv * s_fmax[jj];
+            small = small && (amax < SG_SINCOS_SMALL_LIMIT);
+            tiny = tiny && (amax < SG_SINCOS_TINY_LIMIT);
             const f32x4 cx = coef(SG2_COMP_XB, jj);       // x-branch coefficients; [3] = D of this column
             const float xbv = eval(cx);
-            s_dt[jj * LDS_STRIDE + tu] = DSTORE ? dtv - dt0 : dtv;
+            s_dt[jj * LDS_STRIDE + tu] = dtv;
             s_ux[jj * LDS_STRIDE + tu] = dtv * xbv;
             dxv[jj] = cx[3] * xbv;
         }
@@ -884,6 +876,92 @@ __device__ __forceinline__ void gates_all(float g, float s, const float* s_coef,
 #pragma unroll
             for (int q = 0; q < 8; q++) gv[8 * h + q] = out[q];
         }
+    }
+}
+
+// Projections of a whole tile that runs on the polynomials (every step size and gate inside its Taylor range, every
+// block of the recurrence on the lane polynomials), formed by lanes that own ROWS instead of timesteps: lane (column cj,
+// quarter cq) forms dt - dt0, dt * x-branch and D * x-branch of column cj for timesteps 16 cq .. 16 cq + 15, and lane
+// (row br, half bh) one row of B (br < 16) or C for timesteps 32 bh .. 32 bh + 31.  A row's coefficients are then four
+// 16-byte LDS reads per tile and lane instead of one per (timestep, row), the 64 (g, s) of the tile travel through the
+// four padding floats of the rows of s_B / s_C, and the results leave as 16-byte LDS writes: a third fewer vector
+// instructions and a fifth of the LDS instructions of the timestep-per-lane form.  Every value is formed by the
+// expressions of project_all (Taylor form) on the same operands, so it is the same float; the step-size row receives
+// dt - dt0, which is what the lane polynomials of the recurrence take.  dxk: this lane's 16 skips D * x-branch of (column cj, timestep 16 cq + k).
+template <class G, bool HAS_S>
+__device__ __forceinline__ void project_rows(float g, float s, int tid, const float* s_coef, const float* s_tay, float* s_dt, float* s_ux,
+                                             float* s_B, float* s_C, float (&dxk)[G::DI]) {
+    constexpr int DI = G::DI, DS = G::DS;
+    static_assert(DI == 16 && DS == 16 && SCAN_TT == 64 && LDS_STRIDE == SCAN_TT + 4, "64 lanes: 16 columns x 4 quarters, 32 rows x 2 halves");
+    auto delta = [&](const f32x4 t, float gg, float ss) { return HAS_S ? sg_fma(t[0], gg, t[1] * ss) : t[0] * gg; };
+    auto poly = [&](const f32x4 t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); };
+    auto eval = [&](const f32x4 t, float gg, float ss) { return sg_fma(t[0], gg, HAS_S ? sg_fma(t[1], ss, t[2]) : t[2]); };
+    auto coef = [&](int group, int row) { return *reinterpret_cast<const f32x4*>(s_coef + (group * DI + row) * 4); };
+    s_B[(tid >> 2) * LDS_STRIDE + SCAN_TT + (tid & 3)] = g;      // timestep t: padding float t % 4 of row t / 4
+    if (HAS_S) s_C[(tid >> 2) * LDS_STRIDE + SCAN_TT + (tid & 3)] = s;
+    __syncthreads();
+    auto inputs = [&](int t4, f32x4& g4, f32x4& s4) {            // (g, s) of timesteps 4 t4 .. 4 t4 + 3
+        g4 = *reinterpret_cast<const f32x4*>(s_B + t4 * LDS_STRIDE + SCAN_TT);
+        s4 = HAS_S ? *reinterpret_cast<const f32x4*>(s_C + t4 * LDS_STRIDE + SCAN_TT) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    };
+    {
+        const int cj = tid & 15, cq = tid >> 4;
+        const f32x4 cd = coef(SG2_COMP_DT, cj), cx = coef(SG2_COMP_XB, cj);
+        const f32x4 tp = *reinterpret_cast<const f32x4*>(s_tay + cj * 4);
+        float* const r_dt = s_dt + cj * LDS_STRIDE + 16 * cq;
+        float* const r_ux = s_ux + cj * LDS_STRIDE + 16 * cq;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f32x4 g4, s4, d4, u4;
+            inputs(4 * cq + i, g4, s4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float dtv = poly(tp, delta(cd, g4[e], s4[e]));
+                const float xbv = eval(cx, g4[e], s4[e]);
+                d4[e] = dtv - tp[0];
+                u4[e] = dtv * xbv;
+                dxk[4 * i + e] = cx[3] * xbv;
+            }
+            *reinterpret_cast<f32x4*>(r_dt + 4 * i) = d4;
+            *reinterpret_cast<f32x4*>(r_ux + 4 * i) = u4;
+        }
+    }
+    {
+        const int br = tid & 31, bh = tid >> 5;
+        const f32x4 cb = coef(br < DS ? SG2_COMP_B : SG2_COMP_C, br & (DS - 1));
+        float* const r_bc = (br < DS ? s_B : s_C) + (br & (DS - 1)) * LDS_STRIDE + 32 * bh;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            f32x4 g4, s4, v4;
+            inputs(8 * bh + i, g4, s4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v4[e] = eval(cb, g4[e], s4[e]);
+            *reinterpret_cast<f32x4*>(r_bc + 4 * i) = v4;
+        }
+    }
+}
+
+// The row owners' part after the recurrence: y of (column cj, timesteps 16 cq .. 16 cq + 15) becomes y * gate + D * x-branch
+// in place.  The gates are formed here, from the (g, s) that project_rows left in the padding floats, so that they do
+// not occupy 16 registers during the recurrence.
+template <class G, bool HAS_S>
+__device__ __forceinline__ void gate_rows(int tid, const float* s_coef, const float* s_tay, const float* s_B, const float* s_C, float* s_y,
+                                          const float (&dxk)[G::DI]) {
+    constexpr int DI = G::DI;
+    auto delta = [&](const f32x4 t, float gg, float ss) { return HAS_S ? sg_fma(t[0], gg, t[1] * ss) : t[0] * gg; };
+    auto poly = [&](const f32x4 t, float d) { return sg_fma(sg_fma(sg_fma(t[3], d, t[2]), d, t[1]), d, t[0]); };
+    const int cj = tid & 15, cq = tid >> 4;
+    const f32x4 cz = *reinterpret_cast<const f32x4*>(s_coef + (SG2_COMP_Z * DI + cj) * 4);
+    const f32x4 tz = *reinterpret_cast<const f32x4*>(s_tay + (DI + cj) * 4);
+    float* const r_y = s_y + cj * LDS_STRIDE + 16 * cq;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const f32x4 g4 = *reinterpret_cast<const f32x4*>(s_B + (4 * cq + i) * LDS_STRIDE + SCAN_TT);
+        const f32x4 s4 = HAS_S ? *reinterpret_cast<const f32x4*>(s_C + (4 * cq + i) * LDS_STRIDE + SCAN_TT) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        f32x4 y4 = *reinterpret_cast<const f32x4*>(r_y + 4 * i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) y4[e] = sg_fma(y4[e], poly(tz, delta(cz, g4[e], s4[e])), dxk[4 * i + e]);
+        *reinterpret_cast<f32x4*>(r_y + 4 * i) = y4;
     }
 }
 
@@ -923,6 +1001,11 @@ __device__ __forceinline__ void block_steps_pair(LaneState (&S)[2], const float 
 // write.  Column jl + 8 h plays the part of wave h of the two-wave kernel throughout (its half of the projections, its
 // angle masks, its ballots over the same 64 (column, pair) lanes), so every decision and every value is the one the
 // checker makes for the two-wave form.
+// A tile has three lane roles.  Recurrence (phase B): lane (jl, p) as above.  Timestep: lane t loads the inputs of
+// timestep t, votes on the form the tile takes, and at the end multiplies its 16 gated outputs by out_proj and stores
+// its element's row.  Row owner (the usual tile, on the polynomials throughout): lane (column, quarter of the tile)
+// forms that column's projections before the recurrence and gates its outputs after it (project_rows, gate_rows);
+// other tiles keep the timestep-per-lane projections (project_all, gates_all).
 template <class G>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void k_replay(Plan pl) {
     constexpr int DM = G::DM, DS = G::DS, DI = G::DI, HP = G::HP, LANES = G::THREADS;
@@ -1019,6 +1102,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         }
     };
     load_inputs(u0);
+    // The context row of a timestep leaves one tile late, after the next tile's inputs have arrived: the counter that
+    // tells a wave that its loads have landed also counts its stores, in order, so a store issued just before that
+    // wait would make every tile wait for a scattered write to be acknowledged.
+    static_assert(DM == 8, "two 16-byte stores per lane");
+    float4 held[2];
+    float4* held_dst = nullptr;
+    auto flush = [&]() {
+        if (held_dst != nullptr) {
+            held_dst[0] = held[0];
+            held_dst[1] = held[1];
+        }
+    };
     for (int tile0 = u0; tile0 < u1; tile0 += SCAN_TT) {
         const int cnt = min(SCAN_TT, u1 - tile0);
         // ---------------- phase A: projections of SCAN_TT timesteps -> LDS (both halves of every output group)
@@ -1026,6 +1121,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         const int32_t v = nx_val;
         const float shv = nx_sh;
         const bool valid = tile0 + tu < u1;
+        asm volatile("" : : "v"(kbits), "v"(v), "v"(shv) : "memory");      // the wait for this tile's inputs goes here, before the stores
+        flush();
         if (tile0 + SCAN_TT < u1) load_inputs(tile0 + SCAN_TT);
         int orig = v & 0x7fffffff;
         orig = ((unsigned)orig < (unsigned)N) ? orig : 0;   // never index outside the tensor
@@ -1036,14 +1133,16 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             __builtin_amdgcn_ballot_w64(!sg2_poly_ok(SG2_PROD_LINEAR_FACTOR * kpoly_g, SG2_PROD_LINEAR_FACTOR * kpoly_s, g, sh));
         const bool tay = __builtin_amdgcn_ballot_w64(!sg2_taylor_ok(cmax_g, cmax_s, g, sh)) == 0;
         const bool dgiven = tay && notpoly == 0 && cnt == SCAN_TT;
-        unsigned long long large[2], nottiny[2];
-        float dxv[DI];           // D * x-branch of this lane's timestep, kept for phase C
-        {
+        unsigned long long large[2] = {0, 0}, nottiny[2] = {0, 0};
+        float dxv[DI];           // D * x-branch, kept for phase C: of this lane's timestep, or (dgiven) of its column's 16 timesteps
+        if (dgiven) {
+            if (has_s) project_rows<G, true>(g, sh, tid, s_coef, s_tay, s_dt, s_ux, s_B, s_C, dxv);
+            else project_rows<G, false>(g, sh, tid, s_coef, s_tay, s_dt, s_ux, s_B, s_C, dxv);
+        } else {
             int angle[2];
             auto run = [&](auto has_s_c, auto tay_c) {
                 constexpr bool HS = decltype(has_s_c)::value, TY = decltype(tay_c)::value;
-                if (TY && dgiven) project_all<G, HS, true, true>(g, sh, tu, s_coef, s_tay, s_fmax, s_dt, s_ux, s_B, s_C, dxv, angle);
-                else project_all<G, HS, TY, false>(g, sh, tu, s_coef, s_tay, s_fmax, s_dt, s_ux, s_B, s_C, dxv, angle);
+                project_all<G, HS, TY>(g, sh, tu, s_coef, s_tay, s_fmax, s_dt, s_ux, s_B, s_C, dxv, angle);
             };
             if (tay) { if (has_s) run(std::true_type{}, std::true_type{}); else run(std::false_type{}, std::true_type{}); }
             else { if (has_s) run(std::true_type{}, std::false_type{}); else run(std::false_type{}, std::false_type{}); }
@@ -1151,10 +1250,18 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         // ---------------- phase C: gate, D skip, out_proj, scatter to element order (one 32-byte row per lane)
         {
             float o[DI];
-            if (tay) { if (has_s) gates_all<G, true, true>(g, sh, s_coef, s_tay, o); else gates_all<G, false, true>(g, sh, s_coef, s_tay, o); }
-            else { if (has_s) gates_all<G, true, false>(g, sh, s_coef, s_tay, o); else gates_all<G, false, false>(g, sh, s_coef, s_tay, o); }
+            if (dgiven) {        // the row owners gate their 16 outputs in place, then every timestep collects its 16 columns
+                if (has_s) gate_rows<G, true>(tid, s_coef, s_tay, s_B, s_C, s_y, dxv);
+                else gate_rows<G, false>(tid, s_coef, s_tay, s_B, s_C, s_y, dxv);
+                __syncthreads();
 #pragma unroll
-            for (int jj = 0; jj < DI; jj++) o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], o[jj], dxv[jj]);
+                for (int jj = 0; jj < DI; jj++) o[jj] = s_y[jj * LDS_STRIDE + tu];
+            } else {
+                if (tay) { if (has_s) gates_all<G, true, true>(g, sh, s_coef, s_tay, o); else gates_all<G, false, true>(g, sh, s_coef, s_tay, o); }
+                else { if (has_s) gates_all<G, true, false>(g, sh, s_coef, s_tay, o); else gates_all<G, false, false>(g, sh, s_coef, s_tay, o); }
+#pragma unroll
+                for (int jj = 0; jj < DI; jj++) o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], o[jj], dxv[jj]);
+            }
             float cx[DM];
 #pragma unroll
             for (int q = 0; q < DM; q++) {
@@ -1170,15 +1277,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 }
                 cx[q] = a;
             }
-            if (valid) {
-                static_assert(DM == 8, "two 16-byte stores per lane");
-                float4* dst = reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM);
-                dst[0] = make_float4(cx[0], cx[1], cx[2], cx[3]);
-                dst[1] = make_float4(cx[4], cx[5], cx[6], cx[7]);
-            }
+            held_dst = valid ? reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM) : nullptr;
+            held[0] = make_float4(cx[0], cx[1], cx[2], cx[3]);
+            held[1] = make_float4(cx[4], cx[5], cx[6], cx[7]);
         }
         __syncthreads();
     }
+    flush();
     if (u1 == N) {   // last chunk in scan order: new carried state of the tensor
         float* st = dir ? T.mbwd : T.mfwd;
 #pragma unroll
