@@ -884,8 +884,8 @@ __device__ __forceinline__ void gates_all(float g, float s, const float* s_coef,
 // quarter cq) forms dt - dt0, dt * x-branch and D * x-branch of column cj for timesteps 16 cq .. 16 cq + 15, and lane
 // (row br, half bh) one row of B (br < 16) or C for timesteps 32 bh .. 32 bh + 31.  A row's coefficients are then four
 // 16-byte LDS reads per tile and lane instead of one per (timestep, row), the 64 (g, s) of the tile travel through the
-// four padding floats of the rows of s_B / s_C, and the results leave as 16-byte LDS writes: a third fewer vector
-// instructions and a fifth of the LDS instructions of the timestep-per-lane form.  Every value is formed by the
+// four padding floats of the rows of s_B / s_C, and the results leave as 16-byte LDS writes: the same arithmetic as
+// the timestep-per-lane form with a fifth of its LDS instructions.  Every value is formed by the
 // expressions of project_all (Taylor form) on the same operands, so it is the same float; the step-size row receives
 // dt - dt0, which is what the lane polynomials of the recurrence take.  dxk: this lane's 16 skips D * x-branch of (column cj, timestep 16 cq + k).
 template <class G, bool HAS_S>
