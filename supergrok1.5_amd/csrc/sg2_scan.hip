@@ -1262,21 +1262,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
                 for (int jj = 0; jj < DI; jj++) o[jj] = sg_fma(s_y[jj * LDS_STRIDE + tu], o[jj], dxv[jj]);
             }
-            float cx[DM];
+            // out_proj on the matrix pipe: v_mfma_f32_4x4x1_16b is one fused multiply-add per output and step, so 16 of them
+            // in the order of the columns are the fmaf chain of the scalar form, bit for bit.  Block b of the instruction
+            // is timesteps 4 b .. 4 b + 3: the lane of a timestep supplies its gated output as the B operand and receives
+            // its own four outputs; the A operand of lane l is row l % 4 of out_proj (rows 4 .. 7 for the second chain).
+            static_assert(DM == 8 && DI % 4 == 0, "two chains of four output rows");
+            f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+            const float* wlo = s_wout + (tid & 3) * DI;
+            const float* whi = s_wout + (4 + (tid & 3)) * DI;
 #pragma unroll
-            for (int q = 0; q < DM; q++) {
-                const float* wr = s_wout + q * DI;       // the same address for every lane (broadcast reads)
-                float a = 0.0f;
+            for (int m = 0; m < DI; m += 4) {
+                const f32x4 wa = *reinterpret_cast<const f32x4*>(wlo + m), wb = *reinterpret_cast<const f32x4*>(whi + m);
 #pragma unroll
-                for (int m = 0; m < DI; m += 4) {
-                    const f32x4 w4 = *reinterpret_cast<const f32x4*>(wr + m);
-                    a = sg_fma(w4[0], o[m], a);
-                    a = sg_fma(w4[1], o[m + 1], a);
-                    a = sg_fma(w4[2], o[m + 2], a);
-                    a = sg_fma(w4[3], o[m + 3], a);
+                for (int e = 0; e < 4; e++) {
+                    lo = __builtin_amdgcn_mfma_f32_4x4x1f32(wa[e], o[m + e], lo, 0, 0, 0);
+                    hi = __builtin_amdgcn_mfma_f32_4x4x1f32(wb[e], o[m + e], hi, 0, 0, 0);
                 }
-                cx[q] = a;
             }
+            const float cx[DM] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             held_dst = valid ? reinterpret_cast<float4*>(pl.ctx + ((size_t)dir * pl.total + off + orig) * DM) : nullptr;
             held[0] = make_float4(cx[0], cx[1], cx[2], cx[3]);
             held[1] = make_float4(cx[4], cx[5], cx[6], cx[7]);
