@@ -885,9 +885,10 @@ __device__ __forceinline__ void gates_all(float g, float s, const float* s_coef,
 // (row br, half bh) one row of B (br < 16) or C for timesteps 32 bh .. 32 bh + 31.  A row's coefficients are then four
 // 16-byte LDS reads per tile and lane instead of one per (timestep, row), the 64 (g, s) of the tile travel through the
 // four padding floats of the rows of s_B / s_C, and the results leave as 16-byte LDS writes: the same arithmetic as
-// the timestep-per-lane form with a fifth of its LDS instructions.  Every value is formed by the
-// expressions of project_all (Taylor form) on the same operands, so it is the same float; the step-size row receives
-// dt - dt0, which is what the lane polynomials of the recurrence take.  dxk: this lane's 16 skips D * x-branch of (column cj, timestep 16 cq + k).
+// the timestep-per-lane form with a fifth of its LDS instructions.  Every value is formed by the expressions of
+// project_all (Taylor form) on the same operands, so it is the same float; the step-size row receives dt - dt0, which
+// is what the lane polynomials of the recurrence take.
+// dxk: this lane's 16 skips D * x-branch of (column cj, timestep 16 cq + k), kept for gate_rows.
 template <class G, bool HAS_S>
 __device__ __forceinline__ void project_rows(float g, float s, int tid, const float* s_coef, const float* s_tay, float* s_dt, float* s_ux,
                                              float* s_B, float* s_C, float (&dxk)[G::DI]) {
@@ -941,8 +942,8 @@ __device__ __forceinline__ void project_rows(float g, float s, int tid, const fl
     }
 }
 
-// The row owners' part after the recurrence: y of (column cj, timesteps 16 cq .. 16 cq + 15) becomes y * gate + D * x-branch
-// in place.  The gates are formed here, from the (g, s) that project_rows left in the padding floats, so that they do
+// The row owners' part after the recurrence: y of (column cj, timesteps 16 cq .. 16 cq + 15) becomes
+// y * gate + D * x-branch in place.  The gates are formed here, from the (g, s) that project_rows left in the padding floats, so that they do
 // not occupy 16 registers during the recurrence.
 template <class G, bool HAS_S>
 __device__ __forceinline__ void gate_rows(int tid, const float* s_coef, const float* s_tay, const float* s_B, const float* s_C, float* s_y,
