@@ -196,7 +196,7 @@ def build_step(workload, ops, dev, limit=None):
             ops.supergrok15_fused_step(params, grads, a, b, c, d, [0] * P, [0.98] * P, [0.9 * 0.9 ** i for i in range(P)],
                                        W1, b1, W2, b2, 0.1, H, 0.999, 1e-3, 1.0, 1e-8, 2.0, 1.0, 0.5, 1.0)
         what = "SuperGrok v1.5 full step (H=32, exact GELU, device-side clip)"
-    elif workload == "bilevel":
+    elif workload in ("bilevel", "bilevel50"):
         # gradient of sum <smart_grad, cotangent> with respect to every weight of the v2 meta-net, for all tensors
         # of the model at once: sort + scan forward, per-element forward/backward, scan adjoint, all in HIP
         from grokking_optimizers import Mamba3PEERMetaNet, _bilevel
@@ -497,23 +497,25 @@ def muon_precision(dev):
 def secondary_configs(dev, steps=20, warmup=3):
     """The other measured configurations, each timed in this run: Grokfast and SuperGrok v1.5 on the 14-tensor set, the
     SuperGrok v2 step on the 14-tensor set, Muon on its 24 bf16 matrices (algorithmic and executed MFMA fraction), the
-    bilevel meta-gradient pass of v2 on the 14-tensor set and the five other fused steps on the 25 M-element set."""
+    bilevel meta-gradient pass of v2 on the 14-tensor and on the 25 M-element set and the five other fused steps on the
+    25 M-element set."""
     import torch
     from grokking_optimizers import _ops
     out = {}
     for name, workload in (("config1_grokfast", "grokfast"), ("config2_supergrok15", "sg15"), ("config5_muon", "muon"),
-                           ("bilevel_pass_shared14", "bilevel"), ("grokadamw_scale50", "grokadamw"), ("neuralgrok_scale50", "neuralgrok"),
+                           ("bilevel_pass_shared14", "bilevel"), ("bilevel_pass_scale50", "bilevel50"), ("grokadamw_scale50", "grokadamw"), ("neuralgrok_scale50", "neuralgrok"),
                            ("prodigy_scale50", "prodigy"), ("lion_scale50", "lion"), ("supergrok11_scale50", "sg11")):
         W = build_step(workload, _ops, dev)
-        for _ in range(warmup):
+        n_steps, n_warm = (5, 1) if workload == "bilevel50" else (steps, warmup)       # 0.15 s a pass
+        for _ in range(n_warm):
             W["step"]()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
+        for _ in range(n_steps):
             W["step"]()
         torch.cuda.synchronize()
-        el = (time.perf_counter() - t0) / steps
-        r = {"workload": W["name"], "ms_per_step": 1e3 * el, "value": W["units"] / el, "unit": W["unit"], "dtype": W["dtype"], "steps": steps}
+        el = (time.perf_counter() - t0) / n_steps
+        r = {"workload": W["name"], "ms_per_step": 1e3 * el, "value": W["units"] / el, "unit": W["unit"], "dtype": W["dtype"], "steps": n_steps}
         if W["bound"] == "mfma":
             r["roofline"] = {"bound": "mfma", "peak": W["peak"], "unit": "TFLOP/s", "achieved": W["units"] / el / 1e12,
                              "frac": W["units"] / el / 1e12 / W["peak"], "achieved_executed": W["executed"] / el / 1e12,
@@ -621,7 +623,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--sharpness", action="store_true", help="v2 workloads: non-zero sharpness cache (as after a SAM probe)")
-    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11", "bilevel", "valu-probe"],
+    ap.add_argument("--workload", default="scale50", choices=["scale50", "shared14", "grokfast", "sg15", "muon", "grokadamw", "neuralgrok", "prodigy", "lion", "sg11", "bilevel", "bilevel50", "valu-probe"],
                     help="scale50 (default, the headline configuration) and shared14 time the SuperGrok v2 step; "
                          "grokfast / sg15 / muon time the other fused steps (14-tensor set; 24 bf16 matrices)")
     ap.add_argument("--chunk-len", type=int, default=0, help="scan chunk length (0: library default)")
