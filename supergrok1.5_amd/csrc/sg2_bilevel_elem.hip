@@ -8,31 +8,37 @@
 // grokking_optimizers/supergrok2.py:516-1330); the arithmetic is that of Mamba3PEERMetaNet.forward_for_bilevel
 // (grokking_optimizers/mamba3_peer_metanet.py:395-436) and its autograd derivative.
 //
-// One lane per element, persistent grid over tiles of 128 elements (two 128-lane workgroups share a CU, so one
-// workgroup's passes over its tile overlap the other's per-element arithmetic).  Nothing is kept between forward and backward:
-// a lane holds its element's activations in registers, and the routing of a head is differentiated before the
-// next head is evaluated.  Weight gradients are sums over elements:
-//   * experts (16 per element and head, chosen per element): gathered, not scattered.  Each lane owns 18
-//     (expert, hidden unit) pairs with their sums in registers and walks the tile's elements, whose routing
-//     weights of the head every lane has left in LDS as two 12-vectors (see the expert-gradient pass);
+// One lane per element, persistent grid over tiles of 256 elements, one 256-lane workgroup per CU.  Nothing is kept
+// between forward and backward: a lane holds its element's activations in registers, and the routing of a head is
+// differentiated before the next head is evaluated.  Weight gradients are sums over elements:
+//   * experts (16 per element and head, chosen per element).  An expert's hidden unit m is active where
+//     W1[m] g + b1[m] > 0, i.e. on one side of the threshold -b1[m] / W1[m], so between two neighbouring thresholds of
+//     its 16 units the expert is a straight line  out = A g + B.  Each workgroup sorts the thresholds of every expert
+//     once and tabulates (A, B) for the 17 intervals; an element then finds its interval with five LDS reads and
+//     evaluates the expert with one fma, instead of reading the expert's 49 weights.  The gradients of expert e need,
+//     per unit, S0 = sum w [unit active] and S1 = sum w g [unit active] over the elements routed to e (w: routing
+//     weight times d loss / d head): an element adds its (w, w g) to the bin of its interval (two LDS float atomics),
+//     and S0, S1 of a unit are the sums of the bins on the unit's active side, formed once when the workgroup is done.
+//     (An element exactly on a threshold counts the unit as inactive on both sides; forward value and gradient use
+//     the same interval, so they stay consistent.)
 //   * GRU and query matrices (dense outer products d (x) x): every lane leaves its x (31 values) and, per head
-//     and once more for the GRU, its d (8 / 12 values) in LDS; each lane of the workgroup owns up to two entries
-//     of the head's query matrix and three of the GRU matrices and sums their products over the tile's elements;
+//     and once more for the GRU, its d (8 / 12 values) in LDS; each lane of the workgroup owns one entry of the
+//     head's query matrix and up to two of the GRU matrices and sums their products over the tile's elements;
 //   * product keys (rows chosen per element): the same, with d score scattered into a 12-vector per sub-key.
 // Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
-// order.  No atomics anywhere: every sum is formed in a fixed order and the result repeats bit for bit.
+// order.  The dense and key sums are formed in a fixed order; the expert bins are filled by atomics of four waves, so
+// the last bits of the expert gradients can differ from run to run (as with the reference's atomicAdd).
 #include "sg2_internal.hpp"
 
 namespace sg2 {
 namespace {
 
-constexpr int BE_THREADS = 128;         // two waves; LDS is sized so that two workgroups share a CU
+constexpr int BE_THREADS = 256;         // four waves; the LDS tables leave room for one workgroup per CU
 constexpr int BE_WAVES = BE_THREADS / 64;
-constexpr int EXP_STRIDE = 52;          // floats per expert record in LDS: W1[16] b1[16] W2[16] b2 + pad
 constexpr int TOPK = 4;
 constexpr int RW = 2 * PK + 1;          // staged routing row of a head: first-index weights[12] (times d loss/d head), second-index weights[12], mask of first indices
-constexpr int EXP_PER_LANE = NE * EH / BE_THREADS;     // (expert, hidden unit) pairs a lane accumulates
-static_assert(NE * EH % BE_THREADS == 0 && PK % 4 == 0 && PK % BE_WAVES == 0, "expert pairs per lane");
+constexpr int NBIN = EH + 1;            // intervals between an expert's sorted unit thresholds
+static_assert(EH == 16, "the interval search takes steps of 8, 4, 2, 1 and one more");
 constexpr int XW = 31, DW = 13;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
 // x row: g, s, fwd ctx[8], bwd ctx[8], h_old[4], r*h_old[4], h_new[4], 1
 constexpr int X_G = 0, X_S = 1, X_CF = 2, X_CB = 10, X_H = 18, X_RH = 22, X_HN = 26, X_ONE = 30;
@@ -62,6 +68,12 @@ __device__ __forceinline__ void query_entry(int o, int* dcol, int* xcol) {
     *xcol = c < GH ? X_HN + c : (c < GH + 2 * DM ? X_CF + (c - GH) : (c == GH + 2 * DM ? X_G : X_S));
 }
 
+// Is the hidden unit (w1, b1), whose threshold is the rank-th lowest of its expert, active on interval k (the k lowest
+// thresholds lie below g)?  W1 > 0: above its threshold; W1 < 0: below it; W1 = 0: wherever b1 > 0.
+__device__ __forceinline__ bool unit_active(float w1, float b1, int rank, int k) {
+    return w1 > 0.0f ? rank < k : (w1 < 0.0f ? rank >= k : b1 > 0.0f);
+}
+
 struct ElemArgs {
     const float *g, *s, *ctx, *gru, *cot;
     float *smart, *d_ctx, *partials, *gru_out;
@@ -72,12 +84,15 @@ struct ElemArgs {
 
 __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    float* s_exp = lds;                                   // [NE][EXP_STRIDE] weights
-    float* s_gkey = s_exp + NE * EXP_STRIDE;              // [2][NH][PK][DM/2]
+    float* s_ths = lds;                                   // [NE][EH] unit thresholds of every expert, ascending
+    float* s_ab = s_ths + NE * EH;                        // [NE][NBIN][2] the expert as a line A g + B on each interval
+    float* s_bin = s_ab + NE * NBIN * 2;                  // [NE][NBIN][2] sums of w and w g over the elements of each interval
+    float* s_gkey = s_bin + NE * NBIN * 2;                // [2][NH][PK][DM/2]
     float* s_x = s_gkey + 2 * NH * PK * (DM / 2);         // [256][XW]
     float* s_d = s_x + BE_THREADS * XW;                   // [256][DW]
-    float* s_rt = s_d + BE_THREADS * DW;                  // [128][RW]
+    float* s_rt = s_d + BE_THREADS * DW;                  // [256][RW]
     float* s_gq = s_rt + BE_THREADS * RW;                 // [NH][8][22] query-matrix gradients of this workgroup
+    unsigned char* s_rank = reinterpret_cast<unsigned char*>(s_gq + NH * N_QHEAD);      // [NE][EH] position of a unit's threshold among its expert's
 
     const int tid = threadIdx.x;
     {
@@ -85,17 +100,37 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         const float* __restrict__ B1 = a.W.w[W_EXP_B1];
         const float* __restrict__ W2 = a.W.w[W_EXP_W2];
         const float* __restrict__ B2 = a.W.w[W_EXP_B2];
-        for (int i = tid; i < NE * EXP_STRIDE; i += BE_THREADS) s_exp[i] = 0.0f;
         for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) s_gkey[i] = 0.0f;
         for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) s_gq[i] = 0.0f;
-        __syncthreads();
-        for (int i = tid; i < NE * EH; i += BE_THREADS) {
-            const int e = i / EH, k = i % EH;
-            s_exp[e * EXP_STRIDE + k] = W1[i];
-            s_exp[e * EXP_STRIDE + EH + k] = B1[i];
-            s_exp[e * EXP_STRIDE + 2 * EH + k] = W2[i];
+        for (int i = tid; i < NE * NBIN * 2; i += BE_THREADS) s_bin[i] = 0.0f;
+        // one lane per expert: thresholds ranked by counting (ties by unit index), then the line of every interval.
+        // A unit with W1 = 0 has no threshold (+inf, never passed): it is active or not by the sign of b1 alone.
+        for (int e = tid; e < NE; e += BE_THREADS) {
+            const float* w1 = W1 + e * EH;
+            const float* b1 = B1 + e * EH;
+            const float* w2 = W2 + e * EH;
+            auto thr = [&](int m) { return w1[m] != 0.0f ? -b1[m] / w1[m] : __builtin_inff(); };
+            for (int m = 0; m < EH; m++) {
+                const float tm = thr(m);
+                int r = 0;
+                for (int j = 0; j < EH; j++) {
+                    const float tj = thr(j);
+                    r += (tj < tm || (tj == tm && j < m)) ? 1 : 0;
+                }
+                s_rank[e * EH + m] = (unsigned char)r;
+                s_ths[e * EH + r] = tm;
+            }
+            for (int k = 0; k < NBIN; k++) {        // interval k: the k lowest thresholds lie below g
+                float A = 0.0f, B = B2[e];
+                for (int m = 0; m < EH; m++) {
+                    if (!unit_active(w1[m], b1[m], (int)s_rank[e * EH + m], k)) continue;
+                    A = sg_fma(w2[m], w1[m], A);
+                    B = sg_fma(w2[m], b1[m], B);
+                }
+                s_ab[(e * NBIN + k) * 2] = A;
+                s_ab[(e * NBIN + k) * 2 + 1] = B;
+            }
         }
-        for (int i = tid; i < NE; i += BE_THREADS) s_exp[i * EXP_STRIDE + 3 * EH] = B2[i];
     }
     __syncthreads();
 
@@ -118,23 +153,6 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     for (int q = 0; q < Q_PER_LANE; q++) {
         qdcol[q] = 0; qxcol[q] = 0;
         if (tid + q * BE_THREADS < N_QHEAD) query_entry(tid + q * BE_THREADS, &qdcol[q], &qxcol[q]);
-    }
-
-    // the lane's (expert, hidden unit) pairs: wave w owns the experts with first sub-key index 6w .. 6w+5; for first
-    // index 6w + r, round c covers second indices 4c .. 4c+3 (one per 16 lanes) x 16 hidden units.  Per pair: the
-    // expert's W1, b1 entry and two sums over elements of t = (routing weight if the unit is active else 0):
-    // sum t and sum t*g, from which d b1 = W2*sum t, d W1 = W2*sum t*g, d W2 = sum t*pre = W1*sum t*g + b1*sum t.
-    constexpr int KA_PER_WAVE = PK / BE_WAVES, ROUNDS = PK / 4;
-    static_assert(KA_PER_WAVE * ROUNDS == EXP_PER_LANE, "pairs per lane");
-    const int ka0 = __builtin_amdgcn_readfirstlane(KA_PER_WAVE * (tid >> 6));
-    const int kb_sub = (tid & 63) >> 4;
-    float ew1[EXP_PER_LANE], eb1[EXP_PER_LANE];
-    float st0[EXP_PER_LANE], st1[EXP_PER_LANE], sdo[EXP_PER_LANE];
-#pragma unroll
-    for (int q = 0; q < EXP_PER_LANE; q++) {
-        const int e = (ka0 + q / ROUNDS) * PK + 4 * (q % ROUNDS) + kb_sub, m = tid & (EH - 1);
-        ew1[q] = s_exp[e * EXP_STRIDE + m]; eb1[q] = s_exp[e * EXP_STRIDE + EH + m];
-        st0[q] = st1[q] = sdo[q] = 0.0f;
     }
 
     const int tiles = (a.total + BE_THREADS - 1) / BE_THREADS;
@@ -256,39 +274,39 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 #pragma unroll
                     for (int k = 0; k < TOPK; k++) wgt[hf][k] *= inv;
                 }
-                // experts: outputs per lane; their weight gradients in the pass below, from the staged routing weights
-#pragma unroll
-                for (int k = 0; k < 2 * PK; k++) rtrow[k] = 0.0f;
-                {
-                    int mask = 0;
-#pragma unroll
-                    for (int k = 0; k < TOPK; k++) {
-                        rtrow[idx[0][k]] = kk * wgt[0][k];
-                        rtrow[PK + idx[1][k]] = wgt[1][k];
-                        mask |= 1 << idx[0][k];
-                    }
-                    rtrow[2 * PK] = __int_as_float(kk != 0.0f ? mask : 0);
-                }
+                // experts: outputs per lane; each expert's bin of this element's activation pattern takes (w, w g)
                 float ra[TOPK] = {0.f, 0.f, 0.f, 0.f}, rb[TOPK] = {0.f, 0.f, 0.f, 0.f};
                 float head_out = 0.0f;
 #pragma unroll 1
-                for (int c = 0; c < TOPK * TOPK; c++) {
-                    const int ia = c >> 2, ib = c & 3;
-                    // the unrolled selects keep idx/wgt in registers (a dynamic index would send them to scratch)
+                for (int ia = 0; ia < TOPK; ia++) {
+                    // the unrolled selects keep idx/wgt in registers (a dynamic index would send them to scratch); the four
+                    // second indices are unrolled, so that the record reads of four experts are in flight together
                     const int ea = ia == 0 ? idx[0][0] : ia == 1 ? idx[0][1] : ia == 2 ? idx[0][2] : idx[0][3];
-                    const int eb = ib == 0 ? idx[1][0] : ib == 1 ? idx[1][1] : ib == 2 ? idx[1][2] : idx[1][3];
                     const float wa = ia == 0 ? wgt[0][0] : ia == 1 ? wgt[0][1] : ia == 2 ? wgt[0][2] : wgt[0][3];
-                    const float wb = ib == 0 ? wgt[1][0] : ib == 1 ? wgt[1][1] : ib == 2 ? wgt[1][2] : wgt[1][3];
-                    int e = ea * PK + eb;
-                    if (e >= NE) e = NE - 1;
-                    const float* rec = s_exp + e * EXP_STRIDE;
-                    float out = rec[3 * EH];
+                    float ra_sum = 0.0f;
 #pragma unroll
-                    for (int m = 0; m < EH; m++) out = sg_fma(rec[2 * EH + m], sg_max(sg_fma(rec[m], g, rec[EH + m]), 0.0f), out);
-                    head_out = sg_fma(wa * wb, out, head_out);
-                    const float oa = wb * out, ob = wa * out;
-                    ra[0] += ia == 0 ? oa : 0.0f; ra[1] += ia == 1 ? oa : 0.0f; ra[2] += ia == 2 ? oa : 0.0f; ra[3] += ia == 3 ? oa : 0.0f;
-                    rb[0] += ib == 0 ? ob : 0.0f; rb[1] += ib == 1 ? ob : 0.0f; rb[2] += ib == 2 ? ob : 0.0f; rb[3] += ib == 3 ? ob : 0.0f;
+                    for (int ib = 0; ib < TOPK; ib++) {
+                        const float wb = wgt[1][ib];
+                        int e = ea * PK + idx[1][ib];
+                        if (e >= NE) e = NE - 1;
+                        const float* th = s_ths + e * EH;
+                        int k = th[7] < g ? 8 : 0;              // how many of the expert's thresholds lie below g
+                        k += th[k + 3] < g ? 4 : 0;
+                        k += th[k + 1] < g ? 2 : 0;
+                        k += th[k] < g ? 1 : 0;
+                        k += th[k] < g ? 1 : 0;
+                        const int bin = e * NBIN + k;
+                        const float out = sg_fma(s_ab[2 * bin], g, s_ab[2 * bin + 1]);
+                        {
+                            const float w = (kk * wa) * wb;
+                            atomicAdd(&s_bin[2 * bin], w);
+                            atomicAdd(&s_bin[2 * bin + 1], w * g);
+                        }
+                        head_out = sg_fma(wa * wb, out, head_out);
+                        ra_sum = sg_fma(wb, out, ra_sum);
+                        rb[ib] = sg_fma(wa, out, rb[ib]);
+                    }
+                    ra[0] += ia == 0 ? ra_sum : 0.0f; ra[1] += ia == 1 ? ra_sum : 0.0f; ra[2] += ia == 2 ? ra_sum : 0.0f; ra[3] += ia == 3 ? ra_sum : 0.0f;
                 }
                 total += head_out;
                 // routing backward: softmax, scores, query (the product keys' own gradients: see the end of the head)
@@ -321,59 +339,14 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 #pragma unroll
                     for (int q = 0; q < DM; q++) dcb[q] = sg_fma(qr[GH + DM + q], dq[dd], dcb[q]);
                 }
-                // Expert gradients.  The weight an element gives expert (ka, kb) of this head is the product
-                // (d loss/d head * wa)[ka] * wb[kb] of two 12-vectors with four non-zeros each, which every lane has
-                // just staged.  Scattering the 16 x 49 contributions of an element with LDS float atomics is far too
-                // slow (they retire about one lane per clock), and neighbours in element order share no routing, so
-                // the sums are gathered instead: a lane owns 18 fixed (expert, hidden unit) pairs, keeps their sums
-                // in registers, and walks the tile's 128 elements.  A wave's pairs belong to six first indices:
-                // those the element did not pick are skipped with a scalar branch on the element's staged mask.
                 __syncthreads();
-                {
-                    // an element's staged values are fetched one element ahead of their use (two register sets)
-                    struct Staged { float a[KA_PER_WAVE], b[ROUNDS], g, mask; };
-                    auto fetch = [&](int el, Staged& v) {
-                        const float* row = s_rt + el * RW;
-                        v.mask = row[2 * PK];
-                        v.g = s_x[el * XW + X_G];
-#pragma unroll
-                        for (int r = 0; r < KA_PER_WAVE; r++) v.a[r] = row[ka0 + r];
-#pragma unroll
-                        for (int c = 0; c < ROUNDS; c++) v.b[c] = row[PK + 4 * c + kb_sub];
-                    };
-                    auto add = [&](const Staged& v) {
-                        const int mask = __builtin_amdgcn_readfirstlane(__float_as_int(v.mask)) >> ka0;
-#pragma unroll
-                        for (int r = 0; r < KA_PER_WAVE; r++) {
-                            if (((mask >> r) & 1) == 0) continue;          // scalar: the element did not pick this first index
-#pragma unroll
-                            for (int c = 0; c < ROUNDS; c++) {
-                                const int q = r * ROUNDS + c;
-                                const float dout = v.a[r] * v.b[c];
-                                const float pre = sg_fma(ew1[q], v.g, eb1[q]);
-                                const float t = pre > 0.0f ? dout : 0.0f;
-                                st0[q] += t;
-                                st1[q] = sg_fma(t, v.g, st1[q]);
-                                sdo[q] += dout;
-                            }
-                        }
-                    };
-                    Staged v0, v1;
-                    fetch(0, v0);
-#pragma unroll 1
-                    for (int el = 0; el < BE_THREADS; el += 2) {
-                        fetch(el + 1, v1);
-                        add(v0);
-                        fetch(el + 2 < BE_THREADS ? el + 2 : el, v0);
-                        add(v1);
-                    }
-                }
                 // this head's query-matrix gradients: d query (x) query input over the tile's elements
                 {
                     float qs[Q_PER_LANE];
 #pragma unroll
                     for (int q = 0; q < Q_PER_LANE; q++) qs[q] = 0.0f;
-                    for (int e = 0; e < BE_THREADS; e++) {
+#pragma unroll 16
+                    for (int e = 0; e < BE_THREADS; e++) {      // (unrolled: the LDS reads of 16 elements are in flight together)
 #pragma unroll
                         for (int q = 0; q < Q_PER_LANE; q++) qs[q] = sg_fma(s_d[e * DW + qdcol[q]], s_x[e * XW + qxcol[q]], qs[q]);
                     }
@@ -397,6 +370,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 if (tid < 2 * PK * (DM / 2)) {
                     const int hf = tid / (PK * (DM / 2)), row = (tid / (DM / 2)) % PK, dd = tid % (DM / 2);
                     float acc = 0.0f;
+#pragma unroll 16
                     for (int e = 0; e < BE_THREADS; e++) acc = sg_fma(s_rt[e * RW + hf * PK + row], s_d[e * DW + hf * (DM / 2) + dd], acc);
                     s_gkey[(hf * NH + hh) * PK * (DM / 2) + row * (DM / 2) + dd] += acc;
                 }
@@ -441,6 +415,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         }
         __syncthreads();
         // ---- GRU gradients: each lane's entries, summed over the tile's elements
+#pragma unroll 16
         for (int e = 0; e < BE_THREADS; e++) {
 #pragma unroll
             for (int q = 0; q < GRU_PER_LANE; q++) gsum[q] = sg_fma(s_d[e * DW + gdcol[q]], s_x[e * XW + gxcol[q]], gsum[q]);
@@ -458,14 +433,25 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     __syncthreads();
     for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) out[N_GRU + i] = s_gq[i];
     for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) out[OFF_KA + i] = s_gkey[i];
-#pragma unroll
-    for (int q = 0; q < EXP_PER_LANE; q++) {
-        const int e = (ka0 + q / ROUNDS) * PK + 4 * (q % ROUNDS) + kb_sub, m = tid & (EH - 1);
-        const float w2 = s_exp[e * EXP_STRIDE + 2 * EH + m];
-        out[OFF_W1 + e * EH + m] = w2 * st1[q];
-        out[OFF_B1 + e * EH + m] = w2 * st0[q];
-        out[OFF_W2 + e * EH + m] = sg_fma(ew1[q], st1[q], eb1[q] * st0[q]);      // sum t*pre with pre = W1 g + b1 wherever t != 0
-        if (m == 0) out[OFF_B2 + e] = sdo[q];
+    // expert gradients from the bins: d b1 = W2 * S0, d W1 = W2 * S1, d W2 = sum w relu(pre) = W1 * S1 + b1 * S0, d b2 = sum w
+    for (int i = tid; i < NE * EH; i += BE_THREADS) {
+        const int e = i / EH;
+        const float w1 = a.W.w[W_EXP_W1][i], b1 = a.W.w[W_EXP_B1][i], w2 = a.W.w[W_EXP_W2][i];
+        const int rank = s_rank[i];
+        float S0 = 0.0f, S1 = 0.0f;
+        for (int k = 0; k < NBIN; k++) {
+            if (!unit_active(w1, b1, rank, k)) continue;
+            S0 += s_bin[2 * (e * NBIN + k)];
+            S1 += s_bin[2 * (e * NBIN + k) + 1];
+        }
+        out[OFF_W1 + i] = w2 * S1;
+        out[OFF_B1 + i] = w2 * S0;
+        out[OFF_W2 + i] = sg_fma(w1, S1, b1 * S0);
+    }
+    for (int e = tid; e < NE; e += BE_THREADS) {
+        float sd = 0.0f;
+        for (int k = 0; k < NBIN; k++) sd += s_bin[2 * (e * NBIN + k)];
+        out[OFF_B2 + e] = sd;
     }
 }
 
@@ -485,9 +471,9 @@ __global__ __launch_bounds__(256) void k_sum_partials(const float* __restrict__ 
     if (slice == 0 && o < N_GRADS) out[o] = ((s_part[0][col] + s_part[1][col]) + s_part[2][col]) + s_part[3][col];
 }
 
-constexpr int BE_LDS_BYTES = 4 * (NE * EXP_STRIDE + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD);
-static_assert(2 * BE_LDS_BYTES <= 160 * 1024, "two workgroups of k_bilevel_elem per CU");
-constexpr int BE_MAX_GROUPS = 512;       // two resident workgroups on each of the 256 CUs: one round, every workgroup walks the same number of tiles (+-1)
+constexpr int BE_LDS_BYTES = 4 * (NE * EH + NE * NBIN * 4 + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD) + NE * EH;
+static_assert(BE_LDS_BYTES <= 160 * 1024, "one workgroup of k_bilevel_elem per CU");
+constexpr int BE_MAX_GROUPS = 256;       // one resident workgroup on each of the 256 CUs: one round, every workgroup walks the same number of tiles (+-1)
 
 int elem_groups(int64_t total) {
     const int64_t tiles = (total + BE_THREADS - 1) / BE_THREADS;

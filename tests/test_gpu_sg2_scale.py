@@ -97,8 +97,9 @@ def test_scale50_properties_and_determinism():
 def test_bilevel_pass_at_scale_linearity_and_chunking():
     """The bilevel meta-gradient pass on the full 50-tensor set (25 M elements, up to 1024 chunks per tensor), through
     properties that do not need a CPU answer: the gradients are linear in the cotangent; a different chunk length
-    (another decomposition of the same sums) gives the same result; every gradient repeats bit for bit (no atomics
-    anywhere in the pass)."""
+    (another decomposition of the same sums) gives the same result; a repeat gives every gradient bit for bit, except
+    those of the expert MLPs, whose sums are filled by LDS atomics of four waves (order of addition varies): these
+    repeat to 2e-5 of their scale (fp32 sums of some 1e5 terms in another order)."""
     from grokking_optimizers import Mamba3PEERMetaNet, _bilevel, _cabi
     dev = torch.device("cuda:0")
     shapes = wl.scale50_shapes()
@@ -139,7 +140,11 @@ def test_bilevel_pass_at_scale_linearity_and_chunking():
     s1b, g1b = run(c1)
     assert torch.equal(s1, s1b)
     for n in g1:
-        assert torch.equal(g1[n], g1b[n]), n
+        if n.startswith("expert_"):
+            scale = float(g1[n].abs().max())
+            assert float((g1[n].double() - g1b[n].double()).abs().max()) <= 2e-5 * scale, (n, scale)
+        else:
+            assert torch.equal(g1[n], g1b[n]), n
     print("bilevel at scale: chunk length 1024", flush=True)
     assert _cabi.lib().sg2_set_chunk_len(1024) == 0
     try:
