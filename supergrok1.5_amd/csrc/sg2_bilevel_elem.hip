@@ -17,8 +17,13 @@
 //     once and tabulates (A, B) for the 17 intervals; an element then finds its interval with five LDS reads and
 //     evaluates the expert with one fma, instead of reading the expert's 49 weights.  The gradients of expert e need,
 //     per unit, S0 = sum w [unit active] and S1 = sum w g [unit active] over the elements routed to e (w: routing
-//     weight times d loss / d head): an element adds its (w, w g) to the bin of its interval (two LDS float atomics),
-//     and S0, S1 of a unit are the sums of the bins on the unit's active side, formed once when the workgroup is done.
+//     weight times d loss / d head), i.e. sums of (w, w g) per interval.  Small gradients lie in the interval next to
+//     g = 0 on their side of it for every expert; for those the sums over elements are outer products (first sub-key
+//     weights) (x) (second sub-key weights), which every wave accumulates for its 64 elements with fp32 matrix
+//     instructions in registers (16 x 16 x 4: four elements a step), separately for g > 0 and g <= 0.  An element in
+//     any other interval of one of its experts moves its (w, w g) there with LDS float atomics (about 3 clocks a lane,
+//     which is why they are kept for the exceptions).  S0, S1 of a unit are the sums of the bins on the unit's active
+//     side, formed once when the workgroup is done.
 //     (An element exactly on a threshold counts the unit as inactive on both sides; forward value and gradient use
 //     the same interval, so they stay consistent.)
 //   * GRU and query matrices (dense outer products d (x) x): every lane leaves its x (31 values) and, per head
@@ -26,8 +31,9 @@
 //     head's query matrix and up to two of the GRU matrices and sums their products over the tile's elements;
 //   * product keys (rows chosen per element): the same, with d score scattered into a 12-vector per sub-key.
 // Each workgroup writes its sums to its own row of a partials buffer; a second kernel adds the rows in a fixed
-// order.  The dense and key sums are formed in a fixed order; the expert bins are filled by atomics of four waves, so
-// the last bits of the expert gradients can differ from run to run (as with the reference's atomicAdd).
+// order.  The dense, key and near-zero expert sums are formed in a fixed order; the other expert bins are filled by
+// atomics of four waves, so where gradients reach beyond the intervals next to zero the last bits of the expert
+// gradients can differ from run to run (as with the reference's atomicAdd).
 #include "sg2_internal.hpp"
 
 namespace sg2 {
@@ -36,7 +42,10 @@ namespace {
 constexpr int BE_THREADS = 256;         // four waves; the LDS tables leave room for one workgroup per CU
 constexpr int BE_WAVES = BE_THREADS / 64;
 constexpr int TOPK = 4;
-constexpr int RW = 2 * PK + 1;          // staged routing row of a head: first-index weights[12] (times d loss/d head), second-index weights[12], mask of first indices
+constexpr int RH = 16;                  // a staged 12-vector is padded to 16 entries (zeros): one operand row of a 16 x 16 x 4 matrix instruction
+constexpr int RW = 2 * RH + 1;          // staged row of a head: first-index vector at 0, second-index vector at RH (odd stride: consecutive rows hit all banks)
+static_assert(PK <= RH, "a sub-key vector fits its padded half row");
+typedef float be_f32x4 __attribute__((ext_vector_type(4)));
 constexpr int NBIN = EH + 1;            // intervals between an expert's sorted unit thresholds
 static_assert(EH == 16, "the interval search takes steps of 8, 4, 2, 1 and one more");
 constexpr int XW = 31, DW = 13;         // row strides of the staged x and d vectors (odd: lane-consecutive rows hit all banks)
@@ -93,6 +102,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     float* s_rt = s_d + BE_THREADS * DW;                  // [256][RW]
     float* s_gq = s_rt + BE_THREADS * RW;                 // [NH][8][22] query-matrix gradients of this workgroup
     unsigned char* s_rank = reinterpret_cast<unsigned char*>(s_gq + NH * N_QHEAD);      // [NE][EH] position of a unit's threshold among its expert's
+    unsigned char* s_kz = s_rank + NE * EH;               // [NE][2] the interval just below / just above g = 0: thresholds < 0, thresholds <= 0
 
     const int tid = threadIdx.x;
     {
@@ -103,6 +113,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) s_gkey[i] = 0.0f;
         for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) s_gq[i] = 0.0f;
         for (int i = tid; i < NE * NBIN * 2; i += BE_THREADS) s_bin[i] = 0.0f;
+        for (int i = tid; i < BE_THREADS * RW; i += BE_THREADS) s_rt[i] = 0.0f;      // the padding entries stay zero
         // one lane per expert: thresholds ranked by counting (ties by unit index), then the line of every interval.
         // A unit with W1 = 0 has no threshold (+inf, never passed): it is active or not by the sign of b1 alone.
         for (int e = tid; e < NE; e += BE_THREADS) {
@@ -110,8 +121,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             const float* b1 = B1 + e * EH;
             const float* w2 = W2 + e * EH;
             auto thr = [&](int m) { return w1[m] != 0.0f ? -b1[m] / w1[m] : __builtin_inff(); };
+            int below = 0, upto = 0;
             for (int m = 0; m < EH; m++) {
                 const float tm = thr(m);
+                below += tm < 0.0f ? 1 : 0;
+                upto += tm <= 0.0f ? 1 : 0;
                 int r = 0;
                 for (int j = 0; j < EH; j++) {
                     const float tj = thr(j);
@@ -120,6 +134,8 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 s_rank[e * EH + m] = (unsigned char)r;
                 s_ths[e * EH + r] = tm;
             }
+            s_kz[2 * e] = (unsigned char)below;
+            s_kz[2 * e + 1] = (unsigned char)upto;
             for (int k = 0; k < NBIN; k++) {        // interval k: the k lowest thresholds lie below g
                 float A = 0.0f, B = B2[e];
                 for (int m = 0; m < EH; m++) {
@@ -155,6 +171,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
         if (tid + q * BE_THREADS < N_QHEAD) query_entry(tid + q * BE_THREADS, &qdcol[q], &qxcol[q]);
     }
 
+    // near-zero expert sums of this wave (the heads share the experts): sum of w for g > 0, for g <= 0, sum of w g for
+    // g > 0, for g <= 0, each a 16 x 16 (first index x second index) accumulator of the matrix instruction
+    be_f32x4 cen[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) cen[q] = be_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const int tiles = (a.total + BE_THREADS - 1) / BE_THREADS;
     const float kscale = a.rescale / (float)NH;
     for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
@@ -177,11 +198,14 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 const float4 h4 = reinterpret_cast<const float4*>(a.gru)[i];
                 h[0] = h4.x; h[1] = h4.y; h[2] = h4.z; h[3] = h4.w;
             }
+            // (a zero the compiler cannot see through where the wave-uniform weights are used keeps their scalar loads there;
+            //  held across the whole element they are spilled into vector-register lanes and read back, 3000 instructions)
+            const int zo_gf = sg::opaque_zero();
             // ---- GRU forward
             float zg[GH], rg[GH], cand[GH], hn[GH];
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const sg::cfloat_p wz = Wz + j * GRL, wr = Wr + j * GRL;
+                const sg::cfloat_p wz = Wz + j * GRL + zo_gf, wr = Wr + j * GRL + zo_gf;
                 float vz = bz[j], vr = br[j];
                 vz = sg_fma(wz[0], g, vz); vz = sg_fma(wz[1], s, vz);
                 vr = sg_fma(wr[0], g, vr); vr = sg_fma(wr[1], s, vr);
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             }
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const sg::cfloat_p wh = Wh + j * GRL;
+                const sg::cfloat_p wh = Wh + j * GRL + zo_gf;
                 float v = bh[j];
                 v = sg_fma(wh[0], g, v); v = sg_fma(wh[1], s, v);
 #pragma unroll
@@ -223,10 +247,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             const float kk = cot * kscale;                 // d loss / d head output
 #pragma unroll 1
             for (int hh = 0; hh < NH; hh++) {
+                const int zo_q = sg::opaque_zero();
                 float query[DM];
 #pragma unroll
                 for (int dd = 0; dd < DM; dd++) {
-                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN + zo_q;
                     float v = 0.0f;
 #pragma unroll
                     for (int q = 0; q < GH; q++) v = sg_fma(qr[q], hn[q], v);
@@ -242,7 +267,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 float wgt[2][TOPK];
 #pragma unroll
                 for (int hf = 0; hf < 2; hf++) {
-                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2) + zo_q;
                     float sc[PK];
 #pragma unroll
                     for (int q = 0; q < PK; q++) {
@@ -284,6 +309,8 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     const int ea = ia == 0 ? idx[0][0] : ia == 1 ? idx[0][1] : ia == 2 ? idx[0][2] : idx[0][3];
                     const float wa = ia == 0 ? wgt[0][0] : ia == 1 ? wgt[0][1] : ia == 2 ? wgt[0][2] : wgt[0][3];
                     float ra_sum = 0.0f;
+                    int xbin[TOPK], xcen[TOPK];         // a pick outside the interval next to zero: its bin and that interval's, else -1
+                    float xw[TOPK];
 #pragma unroll
                     for (int ib = 0; ib < TOPK; ib++) {
                         const float wb = wgt[1][ib];
@@ -297,23 +324,58 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                         k += th[k] < g ? 1 : 0;
                         const int bin = e * NBIN + k;
                         const float out = sg_fma(s_ab[2 * bin], g, s_ab[2 * bin + 1]);
-                        {
-                            const float w = (kk * wa) * wb;
-                            atomicAdd(&s_bin[2 * bin], w);
-                            atomicAdd(&s_bin[2 * bin + 1], w * g);
-                        }
+                        const int kc = g > 0.0f ? s_kz[2 * e + 1] : s_kz[2 * e];
+                        xbin[ib] = k != kc ? bin : -1;
+                        xcen[ib] = e * NBIN + kc;
+                        xw[ib] = (kk * wa) * wb;
                         head_out = sg_fma(wa * wb, out, head_out);
                         ra_sum = sg_fma(wb, out, ra_sum);
                         rb[ib] = sg_fma(wa, out, rb[ib]);
                     }
                     ra[0] += ia == 0 ? ra_sum : 0.0f; ra[1] += ia == 1 ? ra_sum : 0.0f; ra[2] += ia == 2 ? ra_sum : 0.0f; ra[3] += ia == 3 ? ra_sum : 0.0f;
+                    // picks outside the interval next to zero move their share from there to their own bin; the wave skips
+                    // this when none of its lanes has one (so the four interval searches above stay one straight block)
+                    if (__builtin_amdgcn_ballot_w64(((xbin[0] & xbin[1]) & (xbin[2] & xbin[3])) >= 0) != 0) {
+#pragma unroll
+                        for (int ib = 0; ib < TOPK; ib++) {
+                            if (xbin[ib] < 0) continue;
+                            atomicAdd(&s_bin[2 * xbin[ib]], xw[ib]);
+                            atomicAdd(&s_bin[2 * xbin[ib] + 1], xw[ib] * g);
+                            atomicAdd(&s_bin[2 * xcen[ib]], -xw[ib]);
+                            atomicAdd(&s_bin[2 * xcen[ib] + 1], -(xw[ib] * g));
+                        }
+                    }
+                }
+                // near-zero expert sums: this wave's 64 elements, four a step
+#pragma unroll
+                for (int k = 0; k < PK; k++) { rtrow[k] = 0.0f; rtrow[RH + k] = 0.0f; }
+#pragma unroll
+                for (int k = 0; k < TOPK; k++) {
+                    rtrow[idx[0][k]] = kk * wgt[0][k];
+                    rtrow[RH + idx[1][k]] = wgt[1][k];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                {
+                    const int li = tid & 15, el0 = (tid & ~63) + ((tid & 63) >> 4);
+#pragma unroll 4
+                    for (int t = 0; t < 16; t++) {
+                        const int el = el0 + 4 * t;
+                        const float av = s_rt[el * RW + li], bv = s_rt[el * RW + RH + li], gv = s_x[el * XW + X_G];
+                        const float ap = gv > 0.0f ? av : 0.0f, an = gv > 0.0f ? 0.0f : av;
+                        cen[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(ap, bv, cen[0], 0, 0, 0);
+                        cen[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(an, bv, cen[1], 0, 0, 0);
+                        cen[2] = __builtin_amdgcn_mfma_f32_16x16x4f32(ap * gv, bv, cen[2], 0, 0, 0);
+                        cen[3] = __builtin_amdgcn_mfma_f32_16x16x4f32(an * gv, bv, cen[3], 0, 0, 0);
+                    }
                 }
                 total += head_out;
+                const int zo_rb = sg::opaque_zero();
                 // routing backward: softmax, scores, query (the product keys' own gradients: see the end of the head)
                 float dq[DM], dv[2][TOPK];
 #pragma unroll
                 for (int hf = 0; hf < 2; hf++) {
-                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2);
+                    const sg::cfloat_p keys = (hf ? KB : KA) + hh * PK * (DM / 2) + zo_rb;
                     float mean = 0.0f;
 #pragma unroll
                     for (int k = 0; k < TOPK; k++) mean = sg_fma(wgt[hf][k], kk * (hf ? rb[k] : ra[k]), mean);
@@ -331,7 +393,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
 #pragma unroll
                 for (int dd = 0; dd < DM; dd++) {
                     drow[dd] = dq[dd];
-                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN;
+                    const sg::cfloat_p qr = Wq + (hh * DM + dd) * PIN + zo_rb;
 #pragma unroll
                     for (int q = 0; q < GH; q++) dhn[q] = sg_fma(qr[q], dq[dd], dhn[q]);
 #pragma unroll
@@ -358,11 +420,11 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                 // product-key gradients, d score (x) query half, the same way: the staged rows are free now, so each
                 // lane leaves d score as two 12-vectors (four non-zeros each) and its query; 96 lanes own one entry each
 #pragma unroll
-                for (int k = 0; k < 2 * PK; k++) rtrow[k] = 0.0f;
+                for (int k = 0; k < PK; k++) { rtrow[k] = 0.0f; rtrow[RH + k] = 0.0f; }
 #pragma unroll
                 for (int k = 0; k < TOPK; k++) {
                     rtrow[idx[0][k]] = dv[0][k];
-                    rtrow[PK + idx[1][k]] = dv[1][k];
+                    rtrow[RH + idx[1][k]] = dv[1][k];
                 }
 #pragma unroll
                 for (int dd = 0; dd < DM; dd++) drow[dd] = query[dd];
@@ -371,13 +433,14 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
                     const int hf = tid / (PK * (DM / 2)), row = (tid / (DM / 2)) % PK, dd = tid % (DM / 2);
                     float acc = 0.0f;
 #pragma unroll 16
-                    for (int e = 0; e < BE_THREADS; e++) acc = sg_fma(s_rt[e * RW + hf * PK + row], s_d[e * DW + hf * (DM / 2) + dd], acc);
+                    for (int e = 0; e < BE_THREADS; e++) acc = sg_fma(s_rt[e * RW + hf * RH + row], s_d[e * DW + hf * (DM / 2) + dd], acc);
                     s_gkey[(hf * NH + hh) * PK * (DM / 2) + row * (DM / 2) + dd] += acc;
                 }
                 __syncthreads();
             }
             if (valid && a.smart != nullptr) a.smart[i] = sg_fma(a.rescale, total / (float)NH, g);
 
+            const int zo_gb = sg::opaque_zero();
             // ---- GRU backward
             float dpz[GH], dpr[GH], dph[GH], drh[GH] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -387,7 +450,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             }
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const sg::cfloat_p wh = Wh + j * GRL;
+                const sg::cfloat_p wh = Wh + j * GRL + zo_gb;
 #pragma unroll
                 for (int q = 0; q < DM; q++) { dcf[q] = sg_fma(wh[2 + q], dph[j], dcf[q]); dcb[q] = sg_fma(wh[2 + DM + q], dph[j], dcb[q]); }
 #pragma unroll
@@ -397,7 +460,7 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
             for (int j = 0; j < GH; j++) dpr[j] = (drh[j] * h[j]) * (rg[j] * (1.0f - rg[j]));
 #pragma unroll
             for (int j = 0; j < GH; j++) {
-                const sg::cfloat_p wz = Wz + j * GRL, wr = Wr + j * GRL;
+                const sg::cfloat_p wz = Wz + j * GRL + zo_gb, wr = Wr + j * GRL + zo_gb;
 #pragma unroll
                 for (int q = 0; q < DM; q++) {
                     dcf[q] = sg_fma(wz[2 + q], dpz[j], dcf[q]); dcf[q] = sg_fma(wr[2 + q], dpr[j], dcf[q]);
@@ -433,6 +496,25 @@ __global__ __launch_bounds__(BE_THREADS) void k_bilevel_elem(ElemArgs a) {
     __syncthreads();
     for (int i = tid; i < NH * N_QHEAD; i += BE_THREADS) out[N_GRU + i] = s_gq[i];
     for (int i = tid; i < 2 * NH * PK * (DM / 2); i += BE_THREADS) out[OFF_KA + i] = s_gkey[i];
+    // the waves' near-zero sums into the bins of those intervals, one wave after the other (a fixed order).  Register v
+    // of an accumulator holds first index 4 (lane / 16) + v, second index lane % 16.
+    for (int w = 0; w < BE_WAVES; w++) {
+        __syncthreads();
+        if ((tid >> 6) != w) continue;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int ia = 4 * ((tid & 63) >> 4) + v, ib = tid & 15;
+            if (ia >= PK || ib >= PK) continue;
+            int e = ia * PK + ib;
+            if (e >= NE) e = NE - 1;
+            const int bp = e * NBIN + s_kz[2 * e + 1], bn = e * NBIN + s_kz[2 * e];
+            s_bin[2 * bp] += cen[0][v];
+            s_bin[2 * bn] += cen[1][v];
+            s_bin[2 * bp + 1] += cen[2][v];
+            s_bin[2 * bn + 1] += cen[3][v];
+        }
+    }
+    __syncthreads();
     // expert gradients from the bins: d b1 = W2 * S0, d W1 = W2 * S1, d W2 = sum w relu(pre) = W1 * S1 + b1 * S0, d b2 = sum w
     for (int i = tid; i < NE * EH; i += BE_THREADS) {
         const int e = i / EH;
@@ -471,7 +553,7 @@ __global__ __launch_bounds__(256) void k_sum_partials(const float* __restrict__ 
     if (slice == 0 && o < N_GRADS) out[o] = ((s_part[0][col] + s_part[1][col]) + s_part[2][col]) + s_part[3][col];
 }
 
-constexpr int BE_LDS_BYTES = 4 * (NE * EH + NE * NBIN * 4 + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD) + NE * EH;
+constexpr int BE_LDS_BYTES = 4 * (NE * EH + NE * NBIN * 4 + 2 * NH * PK * (DM / 2) + BE_THREADS * (XW + DW + RW) + NH * N_QHEAD) + NE * EH + NE * 2;
 static_assert(BE_LDS_BYTES <= 160 * 1024, "one workgroup of k_bilevel_elem per CU");
 constexpr int BE_MAX_GROUPS = 256;       // one resident workgroup on each of the 256 CUs: one round, every workgroup walks the same number of tiles (+-1)
 

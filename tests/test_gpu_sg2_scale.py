@@ -98,8 +98,9 @@ def test_bilevel_pass_at_scale_linearity_and_chunking():
     """The bilevel meta-gradient pass on the full 50-tensor set (25 M elements, up to 1024 chunks per tensor), through
     properties that do not need a CPU answer: the gradients are linear in the cotangent; a different chunk length
     (another decomposition of the same sums) gives the same result; a repeat gives every gradient bit for bit, except
-    those of the expert MLPs, whose sums are filled by LDS atomics of four waves (order of addition varies): these
-    repeat to 2e-5 of their scale (fp32 sums of some 1e5 terms in another order)."""
+    those of the expert MLPs: gradients as large as these (std 0.3) leave the intervals next to zero of their experts,
+    and such elements add to their bins with LDS atomics of four waves (order of addition varies), so these repeat to
+    2e-5 of their scale (fp32 sums of some 1e5 terms in another order)."""
     from grokking_optimizers import Mamba3PEERMetaNet, _bilevel, _cabi
     dev = torch.device("cuda:0")
     shapes = wl.scale50_shapes()
