@@ -220,6 +220,67 @@ def test_differentiable_forward_of_the_whole_meta_net():
     assert max(w.values()) <= 1.0, w
 
 
+@pytest.mark.parametrize("case", ["zero_biases_small_gradients", "thresholds_at_the_gradient_scale"])
+def test_expert_gradients_around_the_unit_thresholds(case):
+    """The expert part of the all-HIP accumulation works per interval between an expert's sorted unit thresholds
+    -b1 / W1: sums next to g = 0 through matrix instructions, the others through atomics.  Two corners against the
+    float64 statement.  (1) The module's own initial experts (b1 = 0, every threshold exactly 0, all tied) with
+    gradients of 1e-3: every element sits next to zero, on one side or the other.  (2) Thresholds spread over the
+    range of the gradients themselves, a few units with W1 = 0 (no threshold) and a few thresholds shared by several
+    units: most elements lie beyond the intervals next to zero of some of their experts."""
+    import copy
+    from grokking_optimizers import _bilevel
+    dev = torch.device("cuda:0")
+    mn = _meta_net(21, dev)
+    gen = torch.Generator().manual_seed(22)
+    gstd = 1e-3
+    with torch.no_grad():
+        E, EH = mn.num_experts, mn.expert_W1.shape[1]
+        w1 = (torch.randn(E, EH, 1, generator=gen) * 0.5)
+        if case == "zero_biases_small_gradients":
+            b1 = torch.zeros(E, EH)
+        else:
+            theta = torch.randn(E, EH, generator=gen) * 2.0 * gstd          # thresholds where the gradients are
+            theta[:, 3] = theta[:, 2]                                       # two units share a threshold
+            theta[:, 5] = 0.0
+            w1[:, 7, 0] = 0.0                                               # no threshold: active by the sign of b1 alone
+            w1[:, 8, 0] = 0.0
+            b1 = -theta * w1[:, :, 0]
+            b1[:, 7] = 0.3
+            b1[:, 8] = -0.3
+        mn.expert_W1.copy_(w1.to(dev))
+        mn.expert_b1.copy_(b1.to(dev))
+    mn64 = copy.deepcopy(mn).double().cpu()
+    shapes = [(700,), (33, 9), (130,)]
+    data = []
+    for shp in shapes:
+        n = int(np.prod(shp))
+        data.append(dict(g=torch.randn(n, generator=gen) * gstd, s=torch.rand(n, generator=gen) * gstd,
+                         h=torch.randn(n, 4, generator=gen) * 0.5, hf=torch.randn(16, 16, generator=gen) * 0.3,
+                         hb=torch.randn(16, 16, generator=gen) * 0.3, R=torch.randn(n, generator=gen)))
+    print("expert thresholds:", case, "shapes", shapes, flush=True)
+    ref_sum, ref_smart = None, []
+    for d in data:
+        mn64.zero_grad()
+        rs, _, _, _ = _ref_forward_for_bilevel(mn64, d["g"].double(), d["s"].double(), d["h"].double(), d["hf"].double(), d["hb"].double())
+        (rs * d["R"].double()).sum().backward()
+        ref_smart.append(rs.detach())
+        ref_named = [(n, p.grad.clone()) for n, p in mn64.named_parameters()]
+        ref_sum = ref_named if ref_sum is None else [(n, a + b) for (n, a), (_, b) in zip(ref_sum, ref_named)]
+    mn.zero_grad()
+    smart = _bilevel.accumulate_meta_gradients(mn, [d["g"].to(dev) for d in data], [d["s"].to(dev) for d in data],
+                                               [d["h"].to(dev) for d in data], [d["hf"].to(dev) for d in data],
+                                               [d["hb"].to(dev) for d in data], [d["R"].to(dev) for d in data])
+    got, ref = smart.double().cpu(), torch.cat(ref_smart)
+    err, tol = (got - ref).abs(), 1e-4 * torch.maximum(got.abs(), ref.abs()) + 1e-7
+    assert bool((err <= tol).all()), ("smart", float((err / tol).max()))
+    w = _grad_ratios([(n, p.grad) for n, p in mn.named_parameters()], ref_sum, 2e-4)
+    print("worst gradient ratios", w, flush=True)
+    assert max(w.values()) <= 1.0, w
+    for n in ("expert_W1", "expert_b1", "expert_W2", "expert_b2"):
+        assert float(dict(ref_sum)[n].abs().max()) > 0.0, n          # the comparison is not vacuous
+
+
 @pytest.mark.parametrize("kw", [dict(expert_hidden=4), dict(d_model=4, d_state=8, gru_hidden=2, expert_hidden=6),
                                 dict(d_model=6, d_state=10, gru_hidden=3, num_peer_heads=2, num_experts=25),
                                 dict(d_model=16, d_state=32)],
