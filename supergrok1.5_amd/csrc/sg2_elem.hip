@@ -32,9 +32,12 @@ typedef float vf32 __attribute__((ext_vector_type(32)));
 // (115 of them, no accumulation registers to copy out of) instead of settling for three waves at 112 + 32.
 template <class G>
 constexpr int elem_waves() { return G::DM == 8 ? 4 : 2; }
-template <class G, int EH, bool DBG>
+// FWD: the net's forward alone (sg2_meta_forward) -- smart gradient and new GRU state of every element go to the packed
+// arrays fwd_smart / fwd_gru, nothing of the optimizer state is read or written.
+template <class G, int EH, bool DBG, bool FWD = false>
 __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(elem_waves<G>(), elem_waves<G>()))) void k_elem(Plan pl, int32_t* __restrict__ expert_counts,
-                                                       int32_t* __restrict__ dbg_eidx) {
+                                                       int32_t* __restrict__ dbg_eidx, float* __restrict__ fwd_smart,
+                                                       float* __restrict__ fwd_gru) {
     constexpr int DM = G::DM, GRL = G::GRL, PIN = G::PIN, EXP_STRIDE = exp_stride<EH>();
     static_assert(EH % 4 == 0, "expert records are read 16 bytes at a time");
     __shared__ float s_exp[NE * EXP_STRIDE];
@@ -113,8 +116,11 @@ __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(el
                 hold[0] = h4[0]; hold[1] = h4[1]; hold[2] = h4[2]; hold[3] = h4[3];
             }
             // the optimizer state is requested now, so that its latency passes under the meta-net's arithmetic
-            float mu = sg::gptr(T.mu)[i], ea = sg::gptr(T.ea)[i], easq = sg::gptr(T.easq)[i];
-            float pv = sg::load_elem(T.param, dtype, i);
+            float mu = 0.0f, ea = 0.0f, easq = 0.0f, pv = 0.0f;
+            if (!FWD) {
+                mu = sg::gptr(T.mu)[i]; ea = sg::gptr(T.ea)[i]; easq = sg::gptr(T.easq)[i];
+                pv = sg::load_elem(T.param, dtype, i);
+            }
 
             // ---- GRU: chain order = bias, g, s, fwd ctx, bwd ctx, h
             float zg[GH], rg[GH], hnew[GH];
@@ -154,7 +160,10 @@ __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(el
             sg_tanh_block(GH, pre_c, cand);
 #pragma unroll
             for (int j = 0; j < GH; j++) hnew[j] = sg_fma(zg[j], cand[j], (1.0f - zg[j]) * hold[j]);
-            if (live) ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
+            if (live) {
+                if (FWD) ((SG_GLOBAL vf4*)fwd_gru)[(size_t)T.off + i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
+                else ((SG_GLOBAL vf4*)T.gru)[i] = vf4{hnew[0], hnew[1], hnew[2], hnew[3]};
+            }
 
             // ---- PEER queries: chain order = h, fwd ctx, bwd ctx, g, s
             float qall[NH * DM];
@@ -219,6 +228,10 @@ __global__ __launch_bounds__(ELEM_THREADS) __attribute__((amdgpu_waves_per_eu(el
                 total = total + ho;
             }
             const float smart = g + (rescale * total) / (float)NH;
+            if (FWD) {
+                if (live) sg::gptr(fwd_smart)[(size_t)T.off + i] = smart;
+                continue;
+            }
 
             // ---- mu EMA, Adam moments, decoupled weight decay
             mu = sg_fma(alpha, mu, (1.0f - alpha) * g);
@@ -444,8 +457,14 @@ __global__ __launch_bounds__(ELEM_THREADS) void k_elem_any(Plan pl, int ctx_stri
 int launch_elem_forward(const Plan& pl, int32_t* expert_counts, float* smart_out, float* gru_out, hipStream_t st) {
     if (pl.total == 0) return 0;
     const int grid = pl.elem_tiles < 4096 ? pl.elem_tiles : 4096;
-    hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, geo_info(pl.geo).dm, expert_counts, nullptr, smart_out, gru_out);
-    SG_LAUNCH_CHECK("k_elem_any<forward>");
+    int32_t* const no_dbg = nullptr;
+    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, no_dbg, smart_out, gru_out); };
+    if (pl.elem_kind == ELEM_ANY)
+        hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, geo_info(pl.geo).dm, expert_counts, no_dbg, smart_out, gru_out);
+    else if (pl.geo == GEO_LARGE) go(k_elem<GeoLarge, 16, false, true>);
+    else if (pl.elem_kind == ELEM_FAST4) go(k_elem<GeoDefault, 4, false, true>);
+    else go(k_elem<GeoDefault, 16, false, true>);
+    SG_LAUNCH_CHECK("k_elem<forward>");
     return 0;
 }
 
@@ -454,10 +473,10 @@ int launch_elem(const Plan& pl, int32_t* expert_counts, int32_t* dbg_expert_idx,
     // about five workgroups per resident slot (768 at three per CU): measured 1.38 / 1.35 / 1.33 / 1.33 / 1.37 ms with 768 / 2048 / 4096 /
     // 8192 / 16384 workgroups on 24 424 tiles (fewer leave the chip unevenly loaded at the end, more pay the LDS fill too often)
     const int grid = pl.elem_tiles < 4096 ? pl.elem_tiles : 4096;
-    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx); };
+    float* const none = nullptr;
+    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, expert_counts, dbg_expert_idx, none, none); };
     if (pl.elem_kind == ELEM_ANY) {
         const int stride = geo_info(pl.geo).dm;
-        float* const none = nullptr;
         if (dbg_expert_idx) hipLaunchKernelGGL(k_elem_any<true>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx, none, none);
         else hipLaunchKernelGGL(k_elem_any<false>, dim3(grid), dim3(ELEM_THREADS), 0, st, pl, stride, expert_counts, dbg_expert_idx, none, none);
     } else if (pl.geo == GEO_LARGE) {
